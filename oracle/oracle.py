@@ -1,0 +1,233 @@
+"""ctypes view of the CPU oracle (``xla_cpu_oracle.c``).
+
+Test infrastructure only: imported by ``tests/``, by ``__graft_entry__.smoke``
+and by the ``cpu_baseline`` leg of ``bench.py``; never by the ``xla_amd``
+package.  Arrays are numpy; bf16 travels as ``uint16`` bit patterns,
+f8e4m3fn as ``uint8`` codes, packed s4 as ``uint8`` bytes.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libxla_cpu_oracle.so")
+
+F32, BF16 = 0, 1
+EPI_NONE, EPI_RELU, EPI_GELU_TANH, EPI_SILU = 0, 1, 2, 3
+EPILOGUES = {"none": EPI_NONE, "relu": EPI_RELU, "gelu_tanh": EPI_GELU_TANH, "silu": EPI_SILU}
+TYPES = {"f32": F32, "bf16": BF16}
+
+
+def build(force=False):
+    """Compile the oracle with its Makefile (gcc, OpenMP)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        c = ctypes
+        vp, i64, i32, f32 = c.c_void_p, c.c_int64, c.c_int, c.c_float
+        L.xo_f32_to_bf16.restype = c.c_uint16
+        L.xo_f32_to_bf16.argtypes = [f32]
+        L.xo_bf16_to_f32.restype = f32
+        L.xo_bf16_to_f32.argtypes = [c.c_uint16]
+        L.xo_f32_to_f8e4m3fn.restype = c.c_uint8
+        L.xo_f32_to_f8e4m3fn.argtypes = [f32]
+        L.xo_f16_to_f8e4m3fn.restype = c.c_uint8
+        L.xo_f16_to_f8e4m3fn.argtypes = [c.c_uint16]
+        L.xo_f8e4m3fn_to_f16.restype = c.c_uint16
+        L.xo_f8e4m3fn_to_f16.argtypes = [c.c_uint8]
+        L.xo_f8e4m3fn_to_f32.restype = f32
+        L.xo_f8e4m3fn_to_f32.argtypes = [c.c_uint8]
+        L.xo_f16_to_f32.restype = f32
+        L.xo_f16_to_f32.argtypes = [c.c_uint16]
+        L.xo_f32_to_f16.restype = c.c_uint16
+        L.xo_f32_to_f16.argtypes = [f32]
+        L.xo_tanh_f32.restype = f32
+        L.xo_tanh_f32.argtypes = [f32]
+        L.xo_exp_f32.restype = f32
+        L.xo_exp_f32.argtypes = [f32]
+        for name in ("xo_pack_s4", "xo_unpack_s4", "xo_unpack_u4", "xo_f32_to_bf16_n",
+                     "xo_f32_to_f8e4m3fn_n", "xo_f8e4m3fn_to_f32_n", "xo_tanh_f32_n",
+                     "xo_exp_f32_n"):
+            fn = getattr(L, name)
+            fn.restype = None
+            fn.argtypes = [vp, c.c_size_t, vp]
+        L.xo_tree32_sum.restype = f32
+        L.xo_tree32_sum.argtypes = [vp, i64]
+        L.xo_epilogue_one.restype = c.c_uint16
+        L.xo_epilogue_one.argtypes = [f32, i32, i32, i32, f32, i32]
+        L.xo_dequant_dot.restype = i32
+        L.xo_dequant_dot.argtypes = [vp, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64, i64,
+                                     i64, i32, i32, i32, vp]
+        L.xo_fp8_scaled_dot.restype = i32
+        L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, f32, f32, i32, vp, i32, i64, i64, i64,
+                                        i32, i32, i32, vp]
+        L.xo_rmsnorm_quantize_fp8.restype = i32
+        L.xo_rmsnorm_quantize_fp8.argtypes = [vp, vp, f32, i64, i64, vp, vp]
+        L.xo_num_threads.restype = i32
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def num_threads():
+    return lib().xo_num_threads()
+
+
+# ---- array casts -----------------------------------------------------------
+
+def f32_to_bf16(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().xo_f32_to_bf16_n(_ptr(x), x.size, _ptr(out))
+    return out
+
+
+def bf16_to_f32(h):
+    h = _c(h, np.uint16)
+    return (h.astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_f8e4m3fn(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint8)
+    lib().xo_f32_to_f8e4m3fn_n(_ptr(x), x.size, _ptr(out))
+    return out
+
+
+def f8e4m3fn_to_f32(c):
+    c = _c(c, np.uint8)
+    out = np.empty(c.shape, np.float32)
+    lib().xo_f8e4m3fn_to_f32_n(_ptr(c), c.size, _ptr(out))
+    return out
+
+
+def pack_s4(v):
+    v = _c(v, np.int8).reshape(-1)
+    out = np.zeros((v.size + 1) // 2, np.uint8)
+    lib().xo_pack_s4(_ptr(v), v.size, _ptr(out))
+    return out
+
+
+def unpack_s4(b, n):
+    b = _c(b, np.uint8).reshape(-1)
+    out = np.empty(n, np.int8)
+    lib().xo_unpack_s4(_ptr(b), n, _ptr(out))
+    return out
+
+
+def unpack_u4(b, n):
+    b = _c(b, np.uint8).reshape(-1)
+    out = np.empty(n, np.uint8)
+    lib().xo_unpack_u4(_ptr(b), n, _ptr(out))
+    return out
+
+
+def tanh_f32(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().xo_tanh_f32_n(_ptr(x), x.size, _ptr(out))
+    return out
+
+
+def exp_f32(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().xo_exp_f32_n(_ptr(x), x.size, _ptr(out))
+    return out
+
+
+def tree32_sum(v):
+    v = _c(v, np.float32).reshape(-1)
+    return float(lib().xo_tree32_sum(_ptr(v), v.size))
+
+
+# ---- the three fused paths -------------------------------------------------
+
+def dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, bias=None, bias_ty="bf16",
+                group=None, dot_ty="f32", ep_ty="f32", epilogue="none"):
+    """a_bf16: uint16 [B,M,K] or [M,K]; w: int8 [..,K,N] (w_bits=8) or packed uint8 (w_bits=4,
+    with logical shape given by scale/N); scale: [..,K/group,N].  Returns uint16 bf16 [..,M,N]."""
+    a = _c(a_bf16, np.uint16)
+    batched = a.ndim == 3
+    if not batched:
+        a = a[None]
+    B, M, K = a.shape
+    scale = np.ascontiguousarray(scale)
+    s = scale if scale.ndim == 3 else scale.reshape(B, -1, scale.shape[-1])
+    G, N = s.shape[1], s.shape[2]
+    if group is None:
+        group = K // G
+    assert G * group == K
+    s = _c(s, np.uint16 if scale_ty == "bf16" else np.float32)
+    if w_bits == 8:
+        w = _c(w, np.int8)
+        assert w.size == B * K * N
+    else:
+        w = _c(w, np.uint8)
+        assert w.size == (B * K * N + 1) // 2
+    bp = None
+    if bias is not None:
+        bias = _c(bias, np.uint16 if bias_ty == "bf16" else np.float32)
+        assert bias.size == N
+        bp = _ptr(bias)
+    out = np.empty((B, M, N), np.uint16)
+    rc = lib().xo_dequant_dot(_ptr(a), _ptr(w), w_bits, _ptr(s), TYPES[scale_ty], TYPES[mul_ty],
+                              bp, TYPES[bias_ty], B, M, K, N, group, TYPES[dot_ty],
+                              TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
+    assert rc == 0
+    return out if batched else out[0]
+
+
+def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=None,
+                   bias_ty="bf16", dot_ty="f32", ep_ty="f32", epilogue="none"):
+    a8 = _c(a8, np.uint8)
+    b8 = _c(b8, np.uint8)
+    M, K = a8.shape
+    N = b8.shape[0] if b_is_nk else b8.shape[1]
+    assert (b8.shape[1] if b_is_nk else b8.shape[0]) == K
+    bp = None
+    if bias is not None:
+        bias = _c(bias, np.uint16 if bias_ty == "bf16" else np.float32)
+        assert bias.size == N
+        bp = _ptr(bias)
+    out = np.empty((M, N), np.uint16)
+    rc = lib().xo_fp8_scaled_dot(_ptr(a8), _ptr(b8), int(b_is_nk), float(a_scale), float(b_scale),
+                                 TYPES[mul_ty], bp, TYPES[bias_ty], M, K, N, TYPES[dot_ty],
+                                 TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
+    assert rc == 0
+    return out
+
+
+def rmsnorm_quantize_fp8(x_bf16, gamma_bf16, eps=1e-6):
+    x = _c(x_bf16, np.uint16)
+    g = _c(gamma_bf16, np.uint16)
+    rows, cols = x.shape
+    assert g.size == cols
+    q = np.empty((rows, cols), np.uint8)
+    s = np.empty(rows, np.float32)
+    rc = lib().xo_rmsnorm_quantize_fp8(_ptr(x), _ptr(g), float(np.float32(eps)), rows, cols,
+                                       _ptr(q), _ptr(s))
+    assert rc == 0
+    return q, s

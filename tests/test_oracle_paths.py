@@ -1,0 +1,237 @@
+"""Pins the fused functions of the CPU oracle with what the mathematics fixes:
+library routines, one-hot / power-of-two special cases with exact answers, brute
+force in float64 on tiny shapes, and order probes.  None of these re-types the
+oracle's own formulas.
+"""
+import numpy as np
+import pytest
+
+from xla_amd import dtypes
+
+
+def bf16(x):
+    return dtypes.f32_to_bf16(np.asarray(x, np.float32))
+
+
+def as_f32(h):
+    return dtypes.bf16_to_f32(h)
+
+
+# ---- tanh / exp against libm --------------------------------------------------
+
+def test_tanh_matches_libm(oracle):
+    x = np.concatenate([np.linspace(-25, 25, 200001), np.array([0.0, 1e-5, -3e-4, 4e-4, 7.99, 8.5, 19.9, 20.0, -20.0, 1e30])]).astype(np.float32)
+    got = oracle.tanh_f32(x).astype(np.float64)
+    want = np.tanh(x.astype(np.float64))
+    assert np.max(np.abs(got - want)) < 5e-7       # ~4 f32 ulp; a wrong coefficient is off by >1e-4
+    assert np.all(np.abs(got) <= 1.0)
+    assert np.array_equal(oracle.tanh_f32(-x), -oracle.tanh_f32(x))   # odd function, exactly
+    small = np.array([1e-5, -3.9e-4], np.float32)
+    assert np.array_equal(oracle.tanh_f32(small), small)             # |x| < 4e-4 -> x
+
+
+def test_exp_matches_libm(oracle):
+    x = np.linspace(-87, 88, 300001).astype(np.float32)
+    got = oracle.exp_f32(x).astype(np.float64)
+    want = np.exp(x.astype(np.float64))
+    assert np.max(np.abs(got / want - 1.0)) < 2.0 ** -21.5
+    assert oracle.exp_f32(np.array([0.0], np.float32))[0] == 1.0
+    assert oracle.exp_f32(np.array([-200.0], np.float32))[0] == 0.0   # clamps, then 2^-127 -> 0
+    assert np.isinf(oracle.exp_f32(np.array([89.0], np.float32))[0]) or \
+        oracle.exp_f32(np.array([89.0], np.float32))[0] > 3e38
+
+
+# ---- epilogue -----------------------------------------------------------------
+
+def _gelu64(x):
+    return 0.5 * x * (1 + np.tanh(np.sqrt(2 / np.pi) * (x + 0.044715 * x ** 3)))
+
+
+def _silu64(x):
+    return x / (1 + np.exp(-x))
+
+
+@pytest.mark.parametrize("epi,fn", [("gelu_tanh", _gelu64), ("silu", _silu64),
+                                    ("relu", lambda v: np.maximum(v, 0)), ("none", lambda v: v)])
+def test_epilogue_f32_close_to_float64(oracle, epi, fn):
+    L = oracle.lib()
+    xs = np.linspace(-12, 12, 4001).astype(np.float32)
+    bias = np.float32(0.375)
+    for has_bias in (0, 1):
+        got = np.array([L.xo_epilogue_one(float(v), 0, 0, has_bias, float(bias), oracle.EPILOGUES[epi])
+                        for v in xs], np.uint16)
+        want = fn(xs.astype(np.float64) + (float(bias) if has_bias else 0.0))
+        # single final rounding: within one bf16 step of the float64 value, plus the f32
+        # cancellation noise of x*(1+tanh) / x*sigmoid in the far negative tail
+        err = np.abs(as_f32(got).astype(np.float64) - want)
+        ulp = np.maximum(np.abs(want), 2.0 ** -126) * 2.0 ** -8
+        assert np.all(err <= ulp + 2e-6 * np.maximum(1.0, np.abs(xs))), epi
+
+
+def test_epilogue_bf16_rounds_every_op(oracle):
+    L = oracle.lib()
+    # bf16-typed dot: the accumulator 1 + 2^-9 is rounded to 1.0 before the bias add, and
+    # 1 + 2^-9 + 2^-12 rounds to 1.0; with f32 ops the single final rounding sees
+    # 1 + 2^-8 + 2^-12 and goes up to 1.0078125.
+    acc, b = 1.0 + 2.0 ** -9, 2.0 ** -9 + 2.0 ** -12
+    assert L.xo_epilogue_one(acc, 1, 1, 1, b, 0) == 0x3F80
+    assert L.xo_epilogue_one(acc, 0, 0, 1, b, 0) == 0x3F81
+    # bias itself is rounded to bf16 first when the add is bf16-typed
+    assert L.xo_epilogue_one(0.0, 1, 1, 1, 1.0 + 2.0 ** -9, 0) == 0x3F80
+
+
+# ---- dequant dot ----------------------------------------------------------------
+
+def _dot_case(rng, B, M, K, N, group, w_bits):
+    a = bf16(rng.standard_normal((B, M, K)))
+    lo, hi = (-127, 128) if w_bits == 8 else (-8, 8)
+    w = rng.integers(lo, hi, size=(B, K, N)).astype(np.int8)
+    G = K // group
+    return a, w, G
+
+
+@pytest.mark.parametrize("w_bits", [8, 4])
+def test_dequant_dot_one_hot_is_exact(oracle, w_bits):
+    """One-hot activations select single dequantised weights: out = bf16(round_mul(w*s))."""
+    rng = np.random.default_rng(11)
+    B, K, N, group = 2, 64, 48, 16
+    _, w, G = _dot_case(rng, B, K, K, N, group, w_bits)
+    a = np.zeros((B, K, K), np.float32)
+    a[:, np.arange(K), np.arange(K)] = 1.0
+    s32 = rng.uniform(1e-3, 2e-2, size=(B, G, N)).astype(np.float32)
+    wp = w if w_bits == 8 else dtypes.pack_s4(w)
+    for scale_ty, mul_ty in (("f32", "f32"), ("bf16", "bf16"), ("bf16", "f32"), ("f32", "bf16")):
+        s = bf16(s32) if scale_ty == "bf16" else s32
+        out = oracle.dequant_dot(bf16(a), wp, w_bits, s, scale_ty, mul_ty, group=group)
+        sv = as_f32(s) if scale_ty == "bf16" else s
+        if mul_ty == "bf16":
+            sv = as_f32(bf16(sv))
+        prod = w.astype(np.float64) * np.repeat(sv, group, axis=1).astype(np.float64)
+        prod32 = prod.astype(np.float32)                    # float64 product is exact; one rounding
+        if mul_ty == "bf16":
+            prod32 = as_f32(bf16(prod32))
+        assert np.array_equal(out, bf16(prod32)), (scale_ty, mul_ty)
+
+
+def test_dequant_dot_brute_force_float64(oracle):
+    rng = np.random.default_rng(5)
+    B, M, K, N, group = 2, 5, 96, 40, 32       # all different: a transposed operand cannot pass
+    a, w, G = _dot_case(rng, B, M, K, N, group, 4)
+    s = bf16(rng.uniform(1e-3, 2e-2, size=(B, G, N)))
+    bias = bf16(rng.standard_normal(N))
+    out = oracle.dequant_dot(a, dtypes.pack_s4(w), 4, s, "bf16", "bf16", bias=bias, group=group,
+                             epilogue="silu")
+    wd = as_f32(bf16((w.astype(np.float64) * np.repeat(as_f32(s), group, axis=1)).astype(np.float32)))
+    ref = np.einsum("bmk,bkn->bmn", as_f32(a).astype(np.float64), wd.astype(np.float64))
+    ref = _silu64(ref + as_f32(bias).astype(np.float64))
+    err = np.abs(as_f32(out).astype(np.float64) - ref)
+    assert np.all(err <= np.abs(ref) * 2.0 ** -8 + 1e-5)
+
+
+def test_dequant_dot_integer_data_is_exact(oracle):
+    """Small integers: every partial sum is exact in f32, so the result is order-free."""
+    rng = np.random.default_rng(2)
+    B, M, K, N = 1, 7, 128, 24
+    a = rng.integers(-4, 5, size=(B, M, K)).astype(np.float32)
+    w = rng.integers(-127, 128, size=(B, K, N)).astype(np.int8)
+    s = np.full((B, 1, N), 0.5, np.float32)
+    out = oracle.dequant_dot(bf16(a), w, 8, s, "f32", "f32")
+    ref = np.einsum("bmk,bkn->bmn", a.astype(np.int64), w.astype(np.int64)) * 0.5
+    assert np.array_equal(out, bf16(ref.astype(np.float32)))
+
+
+def test_dot_adds_in_increasing_k(oracle):
+    """Documents the (unpinned) order choice: 2^24 + 1 + 1 ... stays 2^24 left to right."""
+    K = 64
+    a = np.ones((1, K), np.float32)
+    w = np.ones((K, 1), np.int8)
+    a[0, 0] = 2.0 ** 12
+    s = np.ones((K, 1), np.float32)          # group 1: a scale per row
+    s[0, 0] = 2.0 ** 12
+    out = oracle.dequant_dot(bf16(a), w, 8, s, "f32", "f32", group=1)
+    assert as_f32(out)[0, 0] == 2.0 ** 24
+
+
+# ---- fp8 scaled dot -------------------------------------------------------------
+
+@pytest.mark.parametrize("b_is_nk", [False, True])
+def test_fp8_dot_brute_force(oracle, b_is_nk):
+    rng = np.random.default_rng(9)
+    M, K, N = 6, 80, 10
+    a8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 64, -448, 448))
+    b8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((K, N)) * 64, -448, 448))
+    bias = bf16(rng.standard_normal(N))
+    bmat = np.ascontiguousarray(b8.T) if b_is_nk else b8
+    out = oracle.fp8_scaled_dot(a8, bmat, 1 / 64, 1 / 64, b_is_nk=b_is_nk, bias=bias,
+                                epilogue="gelu_tanh")
+    ref = (dtypes.f8e4m3fn_to_f32(a8).astype(np.float64) / 64) @ (dtypes.f8e4m3fn_to_f32(b8).astype(np.float64) / 64)
+    ref = _gelu64(ref + as_f32(bias).astype(np.float64))
+    err = np.abs(as_f32(out).astype(np.float64) - ref)
+    assert np.all(err <= np.abs(ref) * 2.0 ** -8 + 1e-5)
+
+
+def test_fp8_dot_one_hot(oracle):
+    K, N = 32, 256
+    a = np.zeros((K, K), np.float32)
+    a[np.arange(K), np.arange(K)] = 1.0
+    a8 = dtypes.f32_to_f8e4m3fn(a)
+    b8 = np.tile(np.arange(256, dtype=np.uint8), (K, 1))
+    b8[(b8 & 0x7F) == 0x7F] = 0
+    out = oracle.fp8_scaled_dot(a8, b8, 1.0, 0.25)
+    want = bf16(dtypes.f8e4m3fn_to_f32(b8) * np.float32(0.25))
+    assert np.array_equal(as_f32(out), as_f32(want))       # value compare: -0 sums to +0
+
+
+# ---- RMSNorm + quantize -----------------------------------------------------------
+
+def test_tree32_sum_order(oracle):
+    v = np.arange(1, 1025, dtype=np.float32)
+    assert oracle.tree32_sum(v) == 1024 * 1025 / 2              # exact: order-free
+    # inside a window additions run left to right: 2^24 swallows 31 ones one at a time
+    w = np.ones(64, np.float32)
+    w[0] = 2.0 ** 24
+    assert oracle.tree32_sum(w) == 2.0 ** 24 + 32.0             # second window sums to 32 first
+    w2 = np.ones(64, np.float32)
+    w2[31] = 2.0 ** 24
+    assert oracle.tree32_sum(w2) == 2.0 ** 24 + 32.0 + 32.0     # 31 ones add up before the big one
+
+
+def test_quantize_power_of_two_rows_closed_form(oracle):
+    """x = +-2^k, eps = 0: x/sqrt(mean x^2) = +-1 exactly, so y = +-gamma, amax = max gamma."""
+    rng = np.random.default_rng(4)
+    rows, cols = 6, 160
+    sign = rng.choice([-1.0, 1.0], size=(rows, cols))
+    k = rng.integers(-3, 4, size=(rows, 1))
+    x = (sign * 2.0 ** k).astype(np.float32)
+    gamma = bf16(rng.uniform(0.5, 1.5, cols))
+    q, s = oracle.rmsnorm_quantize_fp8(bf16(x), gamma, eps=0.0)
+    g = as_f32(gamma)
+    amax = g.max()
+    assert np.all(s == np.float32(amax) / np.float32(448))
+    want = dtypes.f32_to_f8e4m3fn(((sign * g).astype(np.float32) / s[:, None]).astype(np.float32))
+    assert np.array_equal(q, want)
+    assert np.all((q & 0x7F).max(axis=1) == 0x7E)                # amax maps to +-448
+
+
+def test_quantize_invariants_and_float64(oracle):
+    rng = np.random.default_rng(8)
+    rows, cols = 16, 1000                                        # ragged: not a multiple of 32
+    x = rng.standard_normal((rows, cols))
+    x[rng.random((rows, cols)) < 0.01] *= 50
+    xb, gamma = bf16(x), bf16(rng.uniform(0.5, 1.5, cols))
+    q, s = oracle.rmsnorm_quantize_fp8(xb, gamma, eps=1e-6)
+    assert not np.any((q & 0x7F) == 0x7F)
+    assert np.all((q & 0x7F).max(axis=1) == 0x7E)
+    xf = as_f32(xb).astype(np.float64)
+    y = xf / np.sqrt((xf ** 2).mean(axis=1, keepdims=True) + 1e-6) * as_f32(gamma).astype(np.float64)
+    amax = np.abs(y).max(axis=1)
+    assert np.allclose(s, amax / 448, rtol=2.0 ** -7)             # y was rounded to bf16 first
+    deq = dtypes.f8e4m3fn_to_f32(q).astype(np.float64) * s[:, None]
+    # e4m3 has 3 mantissa bits: relative step 2^-3, half of it after rounding, plus bf16 noise
+    assert np.all(np.abs(deq - y) <= np.abs(y) * (2.0 ** -4 + 2.0 ** -7) + amax[:, None] * 2.0 ** -10)
+
+
+def test_quantize_zero_row_gives_nan_codes(oracle):
+    x = np.zeros((1, 64), np.float32)
+    q, s = oracle.rmsnorm_quantize_fp8(bf16(x), bf16(np.ones(64)), eps=1e-6)
+    assert s[0] == 0.0 and np.all((q & 0x7F) == 0x7F)
