@@ -1,0 +1,191 @@
+/*
+ * libxla_amd_quant.so -- hand-written CDNA4 (gfx950) kernels for XLA's GPU
+ * quantized-inference fusions, exposed as XLA typed-FFI custom calls.
+ *
+ * Two layers, both plain C ABI:
+ *   1. XLA FFI handlers: `XLA_FFI_Error* fn(XLA_FFI_CallFrame*)`
+ *      (XLA_FFI_Handler, xla/ffi/api/c_api.h:517).  These are what
+ *      XLA_FFI_REGISTER_HANDLER(GetXlaFfiApi(), "<target>", "ROCM", fn)
+ *      (xla/ffi/api/api.h:2881-2891) binds and what CustomCallThunk invokes
+ *      (xla/backends/gpu/runtime/custom_call_thunk.cc:394-422,546-575).
+ *   2. Launchers taking raw device pointers, sizes and a hipStream_t, for
+ *      callers that have no call frame.  The handlers are thin decoders over
+ *      these.
+ *
+ * Every entry point only enqueues work on the given stream and returns; none
+ * synchronises, allocates device memory or reads device data on the host, so
+ * all handlers advertise XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE.
+ */
+#ifndef XLA_AMD_QUANT_H_
+#define XLA_AMD_QUANT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "xla_ffi_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XLA_AMD_EXPORT __attribute__((visibility("default")))
+
+/* custom_call_target strings the rewrite pass emits */
+#define XLA_AMD_TARGET_DEQUANT_DOT "xla_amd.dequant_dot"
+#define XLA_AMD_TARGET_FP8_SCALED_DOT "xla_amd.fp8_scaled_dot"
+#define XLA_AMD_TARGET_QUANTIZE_FP8 "xla_amd.rowwise_quantize_fp8"
+
+/* ------------------------------------------------------------------------
+ * Layer 1: XLA FFI handlers (stage EXECUTE; they also answer the metadata
+ * query of xla/ffi/api/api.h:2305-2313 with api version 0.4).
+ * ------------------------------------------------------------------------ */
+
+/*
+ * Weight-only dequantize-dot.  Replaces the `__triton_gemm` fusion that
+ * GemmFusion builds for convert(s4|s8) -> [multiply by broadcast scale] -> dot
+ * (xla/backends/gpu/transforms/gemm_fusion.cc:1629-1702) together with the
+ * bias/activation epilogue that GemmRewriter folds into a library matmul
+ * (xla/backends/gpu/transforms/gemm_rewriter.cc:888-1007,1987-2304).
+ *   args: lhs     BF16 [M,K] or [B,M,K]
+ *         weights S8 or S4 [K,N] or [B,K,N]   (S4: two per byte, low nibble first over the
+ *                                              row-major index, ir_array.cc:588-603)
+ *         scales  F32 or BF16 [N] | [K/g,N] | [B,N] | [B,K/g,N]
+ *         bias    BF16 or F32 [N]             (only with a BIAS* epilogue)
+ *   rets: out     BF16 [M,N] or [B,M,N]
+ *   attrs (all optional, looked up by name):
+ *     epilogue      string: DEFAULT|BIAS|RELU|BIAS_RELU|GELU|BIAS_GELU|SILU|BIAS_SILU
+ *                   (GemmBackendConfig.Epilogue, xla/service/gpu/backend_configs.proto:105-119)
+ *     dequant_type  i32 XLA dtype of the multiply that applies the scale: 11 (F32, default)
+ *                   or 16 (BF16: each dequantised weight is rounded to bf16, as in
+ *                   fusion_emitter_int4_device_test.cc:93-104)
+ *     dot_type      i32: 11 (default) or 16 -- element type of the dot instruction
+ *     epilogue_type i32: 11 (default) or 16 -- element type of the bias add / activation ops
+ */
+XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame);
+
+/*
+ * f8e4m3fn scaled dot.  Replaces `__cublas$lt$matmul$f8`
+ * (xla/backends/gpu/transforms/gemm_rewriter.cc:1235-1591, executed by
+ * CublasLtMatmulThunk -> hipBLASLt, xla/stream_executor/rocm/hip_blas_lt.cc:468-484).
+ *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1);
+ *         a_scale F32 []; b_scale F32 []; bias BF16|F32 [N] (only with BIAS*)
+ *   rets: out BF16 [M,N]
+ *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
+ *          rhs_contracting_dim i64 (default 0)
+ */
+XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* call_frame);
+
+/*
+ * Row-wise dynamic quantisation to f8e4m3fn, optionally preceded by RMSNorm.
+ * Replaces the chain of reduction + elementwise fusions that PriorityFusion and
+ * the row-reduction emitter produce (xla/backends/gpu/codegen/emitters/reduction.cc:840-991).
+ *   args: x BF16 [R,C]; gamma BF16 [C] (only when rmsnorm is true)
+ *   rets: q F8E4M3FN [R,C]; scales F32 [R]
+ *   attrs: rmsnorm bool (default true); eps f32 (default 1e-6)
+ */
+XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_rowwise_quantize_fp8(XLA_FFI_CallFrame* call_frame);
+
+/*
+ * Registers the three handlers above for platform "ROCM" through the table's
+ * XLA_FFI_Handler_Register (xla/ffi/ffi_api.cc:280-315) -- the dynamic
+ * counterpart of XLA_FFI_REGISTER_HANDLER.  Returns NULL or the first error.
+ */
+XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_register_handlers(const XLA_FFI_Api* api);
+
+/* ------------------------------------------------------------------------
+ * Layer 2: launchers.  Return 0 on success, else an XLA_FFI_Error_Code; the
+ * message is available from xla_amd_last_error() on the calling thread.
+ * `stream` is a hipStream_t.  dtype / type fields hold XLA_FFI_DataType values.
+ * ------------------------------------------------------------------------ */
+
+enum {
+  XLA_AMD_EPI_DEFAULT = 0,
+  XLA_AMD_EPI_BIAS = 1,
+  XLA_AMD_EPI_RELU = 2,
+  XLA_AMD_EPI_BIAS_RELU = 3,
+  XLA_AMD_EPI_GELU = 4,
+  XLA_AMD_EPI_BIAS_GELU = 5,
+  XLA_AMD_EPI_SILU = 6,
+  XLA_AMD_EPI_BIAS_SILU = 7
+};
+
+typedef struct XlaAmdDequantDot {
+  const void* lhs;     /* bf16 [batch,M,K] */
+  const void* weights; /* s8 [batch,K,N] or packed s4 */
+  const void* scales;  /* [batch or 1, K/group, N] */
+  const void* bias;    /* [N] or NULL */
+  void* out;           /* bf16 [batch,M,N] */
+  void* workspace;     /* optional scratch, see xla_amd_dequant_dot_workspace_bytes */
+  size_t workspace_bytes;
+  int64_t batch, M, K, N;
+  int64_t group;           /* K for per-channel scales */
+  int64_t scale_batch;     /* 1 if the scales are shared by all batches, else batch */
+  int32_t weight_dtype;    /* S8 or S4 */
+  int32_t scale_dtype;     /* F32 or BF16 */
+  int32_t bias_dtype;      /* F32 or BF16 */
+  int32_t dequant_type, dot_type, epilogue_type; /* F32 or BF16 */
+  int32_t epilogue;        /* XLA_AMD_EPI_* */
+} XlaAmdDequantDot;
+
+XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);
+
+/* Scratch bytes with which the decode kernels may split K across workgroups (0 = never
+ * needed for this shape).  The rewrite pass sizes the custom call's second result with it,
+ * the way `__cublas$lt$matmul` carries its workspace (gemm_rewriter_fp8_test.cc:1167).
+ * A call without (enough) scratch still works; it just cannot split K. */
+XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K,
+                                                          int64_t N, int32_t weight_dtype);
+
+typedef struct XlaAmdFp8ScaledDot {
+  const void* a;       /* f8e4m3fn [M,K] */
+  const void* b;       /* f8e4m3fn [K,N] or [N,K] */
+  const float* a_scale; /* device scalars */
+  const float* b_scale;
+  const void* bias;
+  void* out;           /* bf16 [M,N] */
+  void* workspace;     /* optional scratch, see xla_amd_fp8_scaled_dot_workspace_bytes */
+  size_t workspace_bytes;
+  int64_t M, K, N;
+  int32_t rhs_contracting_dim; /* 0: b is [K,N]; 1: b is [N,K] */
+  int32_t bias_dtype;
+  int32_t dequant_type, dot_type, epilogue_type;
+  int32_t epilogue;
+} XlaAmdFp8ScaledDot;
+
+XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);
+
+/* K*N bytes when the rhs is [K,N] (it is re-laid out with K minor first, the transpose
+ * GemmRewriter inserts at gemm_rewriter.cc:1235-1591), else 0.  Without it a [K,N] rhs runs
+ * on the slow exact kernel. */
+XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
+                                                             int32_t rhs_contracting_dim);
+
+typedef struct XlaAmdRowwiseQuantize {
+  const void* x;     /* bf16 [rows, cols] */
+  const void* gamma; /* bf16 [cols] or NULL when rmsnorm == 0 */
+  void* q;           /* f8e4m3fn [rows, cols] */
+  float* scales;     /* f32 [rows] */
+  int64_t rows, cols;
+  float eps;
+  int32_t rmsnorm;
+} XlaAmdRowwiseQuantize;
+
+XLA_AMD_EXPORT int xla_amd_launch_rowwise_quantize_fp8(const XlaAmdRowwiseQuantize* p, void* stream);
+
+/* Message of the last failed launcher call on this thread ("" if none). */
+XLA_AMD_EXPORT const char* xla_amd_last_error(void);
+
+/* Name of the kernel variant the last successful launcher call on this thread selected
+ * (e.g. "dequant_dot_decode_s4_m16"); for profiling scripts and tests. */
+XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
+
+/* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
+ * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, 3 tiled),
+ * "dequant_dot_vec", "dequant_dot_slices", "fp8_dot_kernel" (1 exact, 2 tiled),
+ * "quantize_variant".  Returns 0, or -1 for an unknown key. */
+XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XLA_AMD_QUANT_H_ */

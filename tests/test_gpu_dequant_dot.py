@@ -1,0 +1,270 @@
+"""GPU parity of xla_amd.dequant_dot against the CPU oracle, through the FFI handler symbol.
+Dots accumulate in f32 in a different order than the oracle, so outputs are compared within
+2 bf16 ulp (with a cancellation floor derived from sum|a*w|); integer unpacking and the
+dequantised weights themselves are checked bit-exactly with one-hot activations."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_s8, dev_u8, dot_floor, host_bf16
+from xla_amd import dtypes, ffi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def run_dot(w, force_kernel=0, slices=0, vec=0):
+    lhs = dev_bf16(w["lhs"])
+    if w["weight_dtype"] == "s4":
+        wt = dev_u8(w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"]))
+    else:
+        wt = dev_s8(w["weights"])
+    sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
+    bias = None
+    if w.get("bias") is not None:
+        bias = dev_bf16(w["bias"]) if w["bias"].dtype == np.uint16 else dev_f32(w["bias"])
+    ffi.set_option("dequant_dot_kernel", force_kernel)
+    ffi.set_option("dequant_dot_slices", slices)
+    ffi.set_option("dequant_dot_vec", vec)
+    try:
+        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
+                              weight_shape=w["weight_shape"], epilogue=w["epilogue"],
+                              dequant_type=w["dequant_type"], dot_type=w.get("dot_type", "f32"),
+                              epilogue_type=w.get("epilogue_type", "f32"))
+        torch.cuda.synchronize()
+    finally:
+        for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec"):
+            ffi.set_option(k, 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+def oracle_dot(oracle, w):
+    scale_ty = "bf16" if w["scales"].dtype == np.uint16 else "f32"
+    wt = w["weights"]
+    bits = 8
+    if w["weight_dtype"] == "s4":
+        wt, bits = (w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"])), 4
+    epi = {"DEFAULT": "none", "BIAS": "none", "RELU": "relu", "BIAS_RELU": "relu", "GELU": "gelu_tanh",
+           "BIAS_GELU": "gelu_tanh", "SILU": "silu", "BIAS_SILU": "silu"}[w["epilogue"]]
+    bias = w.get("bias")
+    return oracle.dequant_dot(w["lhs"], wt, bits, w["scales"],
+                              scale_ty, w["dequant_type"], bias=bias,
+                              bias_ty="bf16" if (bias is not None and bias.dtype == np.uint16) else "f32",
+                              group=w["group"], dot_ty=w.get("dot_type", "f32"),
+                              ep_ty=w.get("epilogue_type", "f32"), epilogue=epi)
+
+
+def floor_for(w):
+    a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
+    s = w["scales"]
+    sv = (dtypes.bf16_to_f32(s) if s.dtype == np.uint16 else s).astype(np.float64)
+    wi = np.abs(w["weights"].astype(np.float64))
+    K = w["lhs"].shape[-1]
+    if w["lhs"].ndim == 3:
+        sv = sv.reshape(w["lhs"].shape[0], -1, sv.shape[-1])
+        wd = wi * np.repeat(sv, w["group"], axis=1)
+    else:
+        sv = sv.reshape(-1, sv.shape[-1])
+        wd = wi * np.repeat(sv, w["group"], axis=0)
+    return dot_floor(a, wd, K)
+
+
+def compare(oracle, w, got, what):
+    ref = oracle_dot(oracle, w)
+    n_floor = check_dot(got, ref, floor_for(w), what)
+    assert n_floor <= max(4, got.size // 200), "%s: %d outputs only passed through the floor" % (what, n_floor)
+
+
+# ---- decode kernels (M <= 64) --------------------------------------------------------------
+
+@pytest.mark.parametrize("M", [1, 8, 32, 64])
+def test_c2_shape_reduced_n(oracle, M):
+    """Configuration 2 with full K and group 128, N cut to 1024 so the oracle stays fast."""
+    say("dequant_dot C2 s4 M=%d K=8192 N=1024" % M)
+    w = workloads.c2_s4_group(M=M, K=8192, N=1024)
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s4"), kern
+    compare(oracle, w, got, "C2 M=%d %s" % (M, kern))
+
+
+@pytest.mark.parametrize("M,vec,slices", [(3, 4, 1), (3, 8, 2), (16, 16, 4), (16, 8, 1), (20, 4, 2),
+                                          (20, 8, 1), (64, 4, 2)])
+def test_s4_decode_variants(oracle, M, vec, slices):
+    say("dequant_dot s4 variants M=%d vec=%d slices=%d" % (M, vec, slices))
+    w = workloads.c2_s4_group(M=M, K=2048, N=768, group=64)
+    got, kern = run_dot(w, force_kernel=2, slices=slices, vec=vec)
+    assert "_v%d_" % vec in kern, kern
+    compare(oracle, w, got, "s4 %s slices=%d" % (kern, slices))
+
+
+def test_s4_unpack_and_dequant_bit_exact(oracle):
+    """One-hot activations: every output is one dequantised weight, so nibble order, sign
+    extension, the scale lookup and the bf16 rounding are checked exactly."""
+    say("dequant_dot s4 one-hot")
+    K, N, group = 256, 512, 32
+    rng = np.random.default_rng(3)
+    wv = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    wv[:16, :16] = np.arange(-8, 8, dtype=np.int8)[:, None]
+    sc = dtypes.f32_to_bf16(rng.uniform(1e-3, 2e-2, size=(K // group, N)).astype(np.float32))
+    for m0 in range(0, K, 64):
+        a = np.zeros((64, K), np.float32)
+        a[np.arange(64), m0 + np.arange(64)] = 1.0
+        w = dict(lhs=dtypes.f32_to_bf16(a), weights=wv, weights_packed=dtypes.pack_s4(wv), scales=sc,
+                 bias=None, weight_dtype="s4", weight_shape=(K, N), group=group, dequant_type="bf16",
+                 epilogue="DEFAULT")
+        got, kern = run_dot(w, force_kernel=2)
+        prod = wv[m0:m0 + 64].astype(np.float32) * np.repeat(dtypes.bf16_to_f32(sc), group, axis=0)[m0:m0 + 64]
+        want = dtypes.f32_to_bf16(prod)
+        assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want)), kern
+
+
+def test_c1_full_size(oracle):
+    say("dequant_dot C1 s8 per-channel full size")
+    w = workloads.c1_s8_channel()
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s8"), kern
+    compare(oracle, w, got, "C1 " + kern)
+
+
+@pytest.mark.parametrize("M,vec,slices,deq", [(5, 16, 2, "f32"), (16, 8, 1, "f32"), (24, 8, 2, "f32"),
+                                              (64, 4, 1, "f32"), (7, 16, 1, "bf16"), (40, 4, 2, "bf16")])
+def test_s8_decode_variants(oracle, M, vec, slices, deq):
+    say("dequant_dot s8 variants M=%d vec=%d slices=%d deq=%s" % (M, vec, slices, deq))
+    w = workloads.c1_s8_channel(M=M, K=1024, N=640)
+    if deq == "bf16":
+        w["scales"] = dtypes.f32_to_bf16(w["scales"])
+        w["dequant_type"] = "bf16"
+    w["bias"] = dtypes.f32_to_bf16(np.random.default_rng(9).standard_normal(640).astype(np.float32))
+    w["epilogue"] = "BIAS_GELU"
+    got, kern = run_dot(w, force_kernel=2, slices=slices, vec=vec)
+    compare(oracle, w, got, "s8 %s" % kern)
+
+
+def test_s8_one_hot_integer_exact(oracle):
+    say("dequant_dot s8 one-hot")
+    K, N = 256, 384
+    wv = np.random.default_rng(4).integers(-128, 128, size=(K, N)).astype(np.int8)
+    sc = np.full((N,), 0.5, np.float32)
+    a = np.zeros((64, K), np.float32)
+    a[np.arange(64), np.arange(64) * 4] = 1.0
+    w = dict(lhs=dtypes.f32_to_bf16(a), weights=wv, scales=sc, bias=None, weight_dtype="s8",
+             weight_shape=(K, N), group=K, dequant_type="f32", epilogue="DEFAULT")
+    got, kern = run_dot(w, force_kernel=2)
+    want = dtypes.f32_to_bf16(wv[np.arange(64) * 4].astype(np.float32) * 0.5)
+    assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want)), kern
+
+
+@pytest.mark.parametrize("epilogue,ep_ty,dot_ty", [("BIAS_SILU", "f32", "f32"), ("BIAS_GELU", "bf16", "bf16"),
+                                                   ("RELU", "bf16", "f32"), ("BIAS", "f32", "bf16"),
+                                                   ("GELU", "f32", "f32"), ("SILU", "bf16", "bf16")])
+def test_epilogues_and_rounding_points(oracle, epilogue, ep_ty, dot_ty):
+    say("dequant_dot epilogue %s ops=%s dot=%s" % (epilogue, ep_ty, dot_ty))
+    w = workloads.c2_s4_group(M=8, K=512, N=512)
+    w["epilogue"] = epilogue
+    if "BIAS" not in epilogue:
+        w["bias"] = None
+    w["epilogue_type"] = ep_ty
+    w["dot_type"] = dot_ty
+    got, kern = run_dot(w)
+    ref = oracle_dot(oracle, w)
+    # per-op bf16 rounding amplifies a last-bit difference of the accumulator into up to one ulp per
+    # rounded op downstream; allow the floor of the plain dot times the op count
+    fl = floor_for(w) * (12 if ep_ty == "bf16" else 1.2)
+    tol_ulp_fail = check_dot(got, ref, fl + (np.abs(dtypes.bf16_to_f32(ref)) * 2.0 ** -6 if ep_ty == "bf16" or dot_ty == "bf16" else 0), kern)
+    assert tol_ulp_fail <= got.size // 20
+
+
+# ---- generic fallback ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,K,N,group,bits", [(3, 40, 37, 8, 8), (2, 96, 50, 32, 4), (5, 33, 7, 33, 8),
+                                              (70, 128, 130, 128, 4)])
+def test_generic_kernel_odd_shapes(oracle, M, K, N, group, bits):
+    say("dequant_dot generic M=%d K=%d N=%d group=%d bits=%d" % (M, K, N, group, bits))
+    rng = np.random.default_rng(M * 7 + N)
+    lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+    wv = rng.integers(lo, hi, size=(K, N)).astype(np.int8)
+    w = dict(lhs=dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)), weights=wv,
+             scales=rng.uniform(1e-3, 1e-2, size=(K // group, N)).astype(np.float32),
+             bias=rng.standard_normal(N).astype(np.float32), weight_dtype="s4" if bits == 4 else "s8",
+             weight_shape=(K, N), group=group, dequant_type="f32", epilogue="BIAS_RELU")
+    if bits == 4:
+        w["weights_packed"] = dtypes.pack_s4(wv)
+    got, kern = run_dot(w)
+    assert kern == "dequant_dot_generic", kern
+    compare(oracle, w, got, "generic")
+
+
+# ---- tiled MFMA kernel (M > 64) and batches -------------------------------------------------
+
+@pytest.mark.parametrize("B,M,K,N", [(2, 256, 512, 512), (1, 200, 264, 388), (3, 128, 128, 1024)])
+def test_c5_shape_reduced(oracle, B, M, K, N):
+    say("dequant_dot C5 batched s8 B=%d M=%d K=%d N=%d" % (B, M, K, N))
+    w = workloads.c5_s8_batched(B=B, M=M, K=K, N=N)
+    got, kern = run_dot(w)
+    assert kern == "dequant_dot_tiled_s8_factored", kern
+    compare(oracle, w, got, "C5 reduced")
+
+
+def test_batched_decode(oracle):
+    say("dequant_dot batched decode B=4 M=8")
+    w = workloads.c5_s8_batched(B=4, M=8, K=512, N=512)
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s8"), kern
+    compare(oracle, w, got, "batched decode")
+
+
+def test_c5_full_size_sampled_blocks(oracle):
+    """Configuration 5 at full size; the oracle evaluates random (expert, row block, column block)
+    sub-problems of the same inputs."""
+    say("dequant_dot C5 full size")
+    w = workloads.c5_s8_batched()
+    got, kern = run_dot(w)
+    assert kern == "dequant_dot_tiled_s8_factored", kern
+    rng = np.random.default_rng(0)
+    for _ in range(6):
+        b = int(rng.integers(0, 8)); m0 = int(rng.integers(0, 512 - 32)); n0 = int(rng.integers(0, 14336 - 64))
+        sub = dict(w, lhs=np.ascontiguousarray(w["lhs"][b, m0:m0 + 32]),
+                   weights=np.ascontiguousarray(w["weights"][b][:, n0:n0 + 64]),
+                   scales=np.ascontiguousarray(w["scales"][b, n0:n0 + 64]), weight_shape=(4096, 64))
+        compare(oracle, sub, got[b, m0:m0 + 32, n0:n0 + 64], "C5 block b=%d m0=%d n0=%d" % (b, m0, n0))
+
+
+@pytest.mark.parametrize("M", [1, 8, 32, 64])
+def test_c2_full_size_sampled_columns(oracle, M):
+    """Configuration 2 at full size; the oracle evaluates column blocks of the same inputs."""
+    say("dequant_dot C2 full size M=%d" % M)
+    w = workloads.c2_s4_group(M=M)
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s4"), kern
+    rng = np.random.default_rng(M)
+    for n0 in [0, 28672 - 256] + [int(v) * 2 for v in rng.integers(0, (28672 - 256) // 2, size=3)]:
+        wv = np.ascontiguousarray(w["weights"][:, n0:n0 + 256])
+        sub = dict(w, weights=wv, weights_packed=dtypes.pack_s4(wv),
+                   scales=np.ascontiguousarray(w["scales"][:, n0:n0 + 256]),
+                   bias=np.ascontiguousarray(w["bias"][n0:n0 + 256]), weight_shape=(8192, 256))
+        compare(oracle, sub, got[:, n0:n0 + 256], "C2 full M=%d n0=%d" % (M, n0))
+
+
+# ---- errors ---------------------------------------------------------------------------------
+
+def test_dequant_dot_error_paths():
+    say("dequant_dot error paths")
+    lhs = torch.zeros((4, 64), dtype=torch.bfloat16, device="cuda")
+    wt = torch.zeros((64, 32), dtype=torch.int8, device="cuda")
+    sc = torch.ones((32,), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffi.FfiError, match="contracting dimensions differ"):
+        ops.dequant_dot(lhs, torch.zeros((48, 32), dtype=torch.int8, device="cuda"), sc)
+    with pytest.raises(ffi.FfiError, match="BIAS"):
+        ops.dequant_dot(lhs, wt, sc, epilogue="BIAS")
+    with pytest.raises(ffi.FfiError, match="bf16-typed dequantise multiply needs bf16 scales"):
+        ops.dequant_dot(lhs, wt, sc, dequant_type="bf16")
+    with pytest.raises(ffi.FfiError, match="number of scale groups must divide K"):
+        ops.dequant_dot(lhs, wt, torch.ones((5, 32), dtype=torch.float32, device="cuda"))
+    out = ops.dequant_dot(torch.zeros((0, 64), dtype=torch.bfloat16, device="cuda"), wt, sc)
+    assert out.shape == (0, 32)

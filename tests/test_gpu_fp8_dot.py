@@ -1,0 +1,138 @@
+"""GPU parity of xla_amd.fp8_scaled_dot against the CPU oracle, through the FFI handler symbol."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_u8, dot_floor, host_bf16
+from xla_amd import dtypes, ffi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+EPI = {"DEFAULT": "none", "BIAS": "none", "RELU": "relu", "BIAS_RELU": "relu", "GELU": "gelu_tanh",
+       "BIAS_GELU": "gelu_tanh", "SILU": "silu", "BIAS_SILU": "silu"}
+
+
+def run(w, nk=False, force=0, scratch="auto", **types):
+    a = dev_u8(w["a"])
+    b = dev_u8(np.ascontiguousarray(w["b"].T) if nk else w["b"])
+    sa = dev_f32(np.array(w["a_scale"], np.float32))
+    sb = dev_f32(np.array(w["b_scale"], np.float32))
+    bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
+    ffi.set_option("fp8_dot_kernel", force)
+    try:
+        out = ops.fp8_scaled_dot(a, b, sa, sb, bias, rhs_contracting_dim=1 if nk else 0,
+                                 epilogue=w["epilogue"], scratch=scratch, **types)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+def reference(oracle, w, **types):
+    return oracle.fp8_scaled_dot(w["a"], w["b"], w["a_scale"], w["b_scale"], b_is_nk=False,
+                                 mul_ty=types.get("dequant_type", "f32"), bias=w.get("bias"),
+                                 dot_ty=types.get("dot_type", "f32"), ep_ty=types.get("epilogue_type", "f32"),
+                                 epilogue=EPI[w["epilogue"]])
+
+
+def floor_for(w):
+    a = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * float(w["a_scale"])
+    b = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * float(w["b_scale"])
+    return dot_floor(a, b, w["a"].shape[1])
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("M,K,N", [(256, 512, 384), (128, 1024, 128), (130, 272, 200), (16, 32, 16)])
+def test_c3_shape_reduced(oracle, M, K, N, nk):
+    say("fp8_scaled_dot M=%d K=%d N=%d nk=%s" % (M, K, N, nk))
+    w = workloads.c3_fp8(M, K, N)
+    got, kern = run(w, nk=nk)
+    assert kern.startswith("fp8_scaled_dot_tiled"), kern
+    n_floor = check_dot(got, reference(oracle, w), floor_for(w), kern)
+    assert n_floor <= got.size // 100
+
+
+def test_fp8_one_hot_exact(oracle):
+    """A = selector rows of 1.0: outputs are single B values times the scales, exactly."""
+    say("fp8_scaled_dot one-hot")
+    K, N = 256, 256
+    a = np.zeros((128, K), np.float32)
+    a[np.arange(128), np.arange(128) * 2] = 1.0
+    b8 = np.tile(np.arange(256, dtype=np.uint8), (K, 1))
+    b8 = np.roll(b8, 3, axis=1)
+    b8[(b8 & 0x7F) == 0x7F] = 0x3A
+    w = dict(a=dtypes.f32_to_f8e4m3fn(a), b=b8, a_scale=np.float32(0.5), b_scale=np.float32(0.25),
+             bias=None, epilogue="DEFAULT")
+    for nk in (False, True):
+        got, kern = run(w, nk=nk)
+        want = dtypes.f32_to_bf16(dtypes.f8e4m3fn_to_f32(b8[np.arange(128) * 2]) * np.float32(0.125))
+        assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want)), kern
+
+
+def test_reference_pattern_bf16_typed_ops(oracle):
+    """The reference's own test pattern (gemm_rewriter_fp8_test.cc:1110-1141): every op bf16-typed."""
+    say("fp8_scaled_dot bf16-typed pattern")
+    w = workloads.c3_fp8(128, 256, 128)
+    types = dict(dequant_type="bf16", dot_type="bf16", epilogue_type="bf16")
+    got, kern = run(w, **types)
+    ref = reference(oracle, w, **types)
+    fl = floor_for(w) * 12 + np.abs(dtypes.bf16_to_f32(ref)) * 2.0 ** -6
+    check_dot(got, ref, fl, kern)
+
+
+def test_non_power_of_two_scales_take_exact_kernel(oracle):
+    say("fp8_scaled_dot bf16-typed multiply with scale 0.3")
+    w = workloads.c3_fp8(64, 128, 64)
+    w["a_scale"] = np.float32(0.3)
+    w["b_scale"] = np.float32(1 / 64)
+    types = dict(dequant_type="bf16")
+    got, kern = run(w, **types)
+    n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w), kern)
+    assert n_floor <= got.size // 100
+
+
+def test_exact_kernel_and_missing_scratch(oracle):
+    say("fp8_scaled_dot exact kernel / no scratch")
+    w = workloads.c3_fp8(48, 80, 40)
+    got, kern = run(w, scratch=None)
+    assert kern == "fp8_scaled_dot_exact", kern
+    check_dot(got, reference(oracle, w), floor_for(w), kern)
+    with pytest.raises(ffi.FfiError, match="tiled kernel needs"):
+        run(w, force=2, scratch=None)
+
+
+def test_c3_full_size_sampled_blocks(oracle):
+    """Configuration 3 at full size; the oracle evaluates random row/column blocks of the same
+    inputs."""
+    say("fp8_scaled_dot C3 full size")
+    w = workloads.c3_fp8()
+    got, kern = run(w)
+    assert kern.startswith("fp8_scaled_dot_tiled"), kern
+    rng = np.random.default_rng(1)
+    for _ in range(6):
+        m0 = int(rng.integers(0, 8192 - 32)); n0 = int(rng.integers(0, 8192 - 64))
+        sub = dict(w, a=np.ascontiguousarray(w["a"][m0:m0 + 32]), b=np.ascontiguousarray(w["b"][:, n0:n0 + 64]),
+                   bias=np.ascontiguousarray(w["bias"][n0:n0 + 64]))
+        n_floor = check_dot(got[m0:m0 + 32, n0:n0 + 64], reference(oracle, sub), floor_for(sub),
+                            "C3 block m0=%d n0=%d" % (m0, n0))
+        assert n_floor <= 32
+
+
+def test_fp8_error_paths():
+    say("fp8_scaled_dot error paths")
+    a = torch.zeros((16, 32), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((48, 16), dtype=torch.uint8, device="cuda")
+    one = torch.ones((), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffi.FfiError, match="contracting dimensions differ"):
+        ops.fp8_scaled_dot(a, b, one, one)
+    with pytest.raises(ffi.FfiError, match="rhs_contracting_dim"):
+        ops.fp8_scaled_dot(a, torch.zeros((32, 16), dtype=torch.uint8, device="cuda"), one, one,
+                           rhs_contracting_dim=2)

@@ -1,0 +1,102 @@
+// C ABI of the launcher layer (include/xla_amd_quant.h, "Layer 2") and the
+// per-thread state behind xla_amd_last_error / xla_amd_last_kernel.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <atomic>
+
+#include "launch.h"
+
+namespace xla_amd {
+namespace {
+thread_local char g_error[512] = "";
+thread_local char g_kernel[128] = "";
+
+struct Option {
+  const char* key;
+  std::atomic<int> value;
+};
+Option g_options[] = {{"dequant_dot_kernel", {0}}, {"dequant_dot_vec", {0}},
+                      {"dequant_dot_slices", {0}}, {"fp8_dot_kernel", {0}},
+                      {"quantize_variant", {0}}};
+}  // namespace
+
+int Fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void SetLastKernel(const char* name) {
+  strncpy(g_kernel, name, sizeof(g_kernel) - 1);
+  g_kernel[sizeof(g_kernel) - 1] = 0;
+}
+
+int CheckLaunch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+}
+
+int GetOption(const char* key) {
+  for (auto& o : g_options)
+    if (strcmp(o.key, key) == 0) return o.value.load(std::memory_order_relaxed);
+  return 0;
+}
+
+size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices);
+size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim);
+
+}  // namespace xla_amd
+
+extern "C" {
+
+int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream) {
+  if (!p) return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: null params");
+  return xla_amd::LaunchDequantDot(*p, (hipStream_t)stream);
+}
+
+int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream) {
+  if (!p) return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: null params");
+  return xla_amd::LaunchFp8ScaledDot(*p, (hipStream_t)stream);
+}
+
+int xla_amd_launch_rowwise_quantize_fp8(const XlaAmdRowwiseQuantize* p, void* stream) {
+  if (!p) return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "rowwise_quantize_fp8: null params");
+  return xla_amd::LaunchRowwiseQuantize(*p, (hipStream_t)stream, xla_amd::GetOption("quantize_variant"));
+}
+
+size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, int64_t N,
+                                           int32_t weight_dtype) {
+  (void)K;
+  (void)weight_dtype;
+  if (M > 64 || M <= 0) return 0;
+  // the decode kernels never use more than 64/M slices (capped at 16)
+  int slices = (int)(64 / M);
+  if (slices > 16) slices = 16;
+  return xla_amd::DequantDotWorkspaceBytes(batch, M, N, slices);
+}
+
+size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
+                                              int32_t rhs_contracting_dim) {
+  (void)M;
+  return xla_amd::Fp8ScaledDotWorkspaceBytes(K, N, rhs_contracting_dim);
+}
+
+const char* xla_amd_last_error(void) { return xla_amd::g_error; }
+const char* xla_amd_last_kernel(void) { return xla_amd::g_kernel; }
+
+int xla_amd_debug_set_option(const char* key, int value) {
+  for (auto& o : xla_amd::g_options)
+    if (strcmp(o.key, key) == 0) {
+      o.value.store(value, std::memory_order_relaxed);
+      return 0;
+    }
+  return -1;
+}
+
+}  // extern "C"

@@ -1,0 +1,451 @@
+// Weight-streaming dequantize-dot for decode shapes (M <= 64):
+//   out[b,m,n] = epilogue( sum_k lhs[b,m,k] * W'[b,k,n] ),  W' = dequant(w, scale)
+// lhs bf16 [M,K]; w s4 (two per byte, low nibble first) or s8, [K,N] with N
+// minor; scales per output channel or per group of rows.
+//
+// The packed weights are the only large operand, so the kernel is a stream
+// over W with everything else fused around it: each lane pulls VEC bytes of 8
+// consecutive rows straight into registers, dequantises them there, and feeds
+// them to v_mfma_f32_16x16x32_bf16 as the 16x32 operand whose 16 rows are 16
+// *output channels*; the activations are the 32x16 operand, so one
+// instruction produces a [16 channels x 16 tokens] tile.  A lane owns NV
+// adjacent channels (the NV values of its VEC-byte chunk), hence NV
+// instructions and NV*4 accumulator registers per 16 tokens.  The waves of a
+// workgroup split the K range and add their tiles through LDS; an optional
+// split of K across workgroups goes through an f32 workspace and a finalize
+// kernel, in a fixed order, so results do not depend on scheduling.
+//
+// Bound: HBM.  Algorithmic bytes: K*N*bits/8 (weights) + scale, bias, lhs and
+// out once each.
+//
+// Two dequantisation modes, following where the matched HLO rounds:
+//  * kRounded : multiply(convert(w), broadcast(scale)) is bf16-typed, so every
+//    dequantised weight is one RNE rounding of the exact product
+//    (fusion_emitter_int4_device_test.cc:93-104 pattern; FloatNormalization,
+//    xla/service/cpu/cpu_compiler.cc:804-817).  Done per weight, in registers.
+//  * kFactored: the multiply is f32-typed and the scale is constant along K
+//    (per output channel).  Integers go through the MFMA exactly and the scale
+//    multiplies the f32 sum once.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_numerics.h"
+#include "launch.h"
+
+namespace xla_amd {
+namespace {
+
+enum : int { kRounded = 0, kFactored = 1 };
+
+struct DecodeParams {
+  const uint16_t* lhs;   // [batch, M, K]
+  const uint8_t* w;      // [batch, K, N] packed
+  const void* scales;    // [scale_batch, K/group, N]
+  const void* bias;      // [N] or null
+  uint16_t* out;         // [batch, M, N]
+  float* workspace;      // [batch, slices, M, N] when slices > 1
+  int M, K, N, group;
+  int scale_is_bf16, bias_is_bf16, scale_batched;
+  int bf16_dot, bf16_ops, epilogue;
+  int strips, slices, rows_per_slice;  // rows_per_slice: multiple of 32 * WAVES
+};
+
+__device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
+  return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];
+}
+
+// s4 nibble (two's complement, in the low 4 bits of `v`) -> f32 value/16, one instruction
+__device__ __forceinline__ float s4_to_f32_div16(uint32_t v) {
+  return __builtin_amdgcn_cvt_off_f32_i4((int)v);
+}
+
+// WBITS: 4 or 8.  VEC: bytes a lane reads per row (4, 8, 16).  MT: 16-token
+// tiles.  WAVES: waves per workgroup, splitting the workgroup's rows.
+template <int WBITS, int VEC, int MT, int WAVES, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodeParams p) {
+  constexpr int NV = VEC * 8 / WBITS;   // channels per lane
+  constexpr int WORDS = VEC / 4;        // dwords per lane per row
+  constexpr int NPW = 32 / WBITS;       // channels per dword
+  constexpr int R = NV * 4 * MT;        // accumulator registers per lane
+  constexpr int TN = 16 * NV;           // channels per wave tile
+  extern __shared__ float lds[];        // [WAVES][R][64]
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, kb = lane >> 4;
+  // Consecutive workgroup ids land on different XCDs (round robin over 8); give each XCD a
+  // contiguous range of strips so neighbouring strips, which share cache lines, share an L2.
+  int bid = blockIdx.x;
+  {
+    const int total = gridDim.x;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
+  }
+  const int slice = bid % p.slices;
+  const int strip = bid / p.slices;
+  const int batch = blockIdx.y;
+
+  const int n_lane = strip * TN + li * NV;
+  const bool n_ok = n_lane < p.N;  // N % NV == 0: a chunk is all in or all out
+  const size_t wbase = (size_t)batch * p.K * p.N;
+  const uint16_t* lhs = p.lhs + (size_t)batch * p.M * p.K;
+
+  floatx4 acc[NV][MT];
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int rows_per_wave = p.rows_per_slice / WAVES;  // multiple of 32
+  const int k_begin = slice * p.rows_per_slice + wave * rows_per_wave;
+  const int k_end = min(k_begin + rows_per_wave, p.K);
+
+  float sc[NV];       // kRounded: scale (x16 for s4) of each owned channel, for the current group
+  int g_cur = -1;
+
+  uint32_t wq[2][8][WORDS];
+  auto load_rows = [&](int buf, int k0) {
+    const int krow = k0 + 8 * kb;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const bool ok = n_ok && (krow + r) < k_end;
+      const size_t e = wbase + (size_t)(krow + r) * p.N + n_lane;  // element index
+      const uint8_t* src = p.w + (e * WBITS >> 3);
+      if (WORDS == 4) {
+        uintx4 v = ok ? *reinterpret_cast<const uintx4*>(src) : uintx4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) wq[buf][r][q] = v[q];
+      } else if (WORDS == 2) {
+        uintx2 v = ok ? *reinterpret_cast<const uintx2*>(src) : uintx2{0u, 0u};
+        wq[buf][r][0] = v[0];
+        wq[buf][r][WORDS - 1] = v[1];
+      } else {
+        wq[buf][r][0] = ok ? *reinterpret_cast<const uint32_t*>(src) : 0u;
+      }
+    }
+  };
+
+  auto compute = [&](int buf, int k0) {
+    const int krow = k0 + 8 * kb;
+    // activations: 8 consecutive k of token (16*mt + li)
+    bf16x8 bop[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + li;
+      uintx4 v = {0u, 0u, 0u, 0u};
+      if (m < p.M && krow < k_end) v = *reinterpret_cast<const uintx4*>(lhs + (size_t)m * p.K + krow);
+      bop[mt] = __builtin_bit_cast(bf16x8, v);
+    }
+    if (MODE == kRounded) {
+      const int g = krow / p.group;
+      if (g != g_cur && krow < k_end) {
+        g_cur = g;
+        const size_t sb = ((size_t)(p.scale_batched ? batch : 0) * (p.K / p.group) + g) * p.N + n_lane;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+          float s = n_ok ? load_scale(p.scales, sb + j, p.scale_is_bf16) : 0.0f;
+          sc[j] = WBITS == 4 ? s * 16.0f : s;  // the s4 convert yields value/16
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < WORDS; ++q) {
+#pragma unroll
+      for (int e = 0; e < NPW; ++e) {
+        const int j = q * NPW + e;
+        float f[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const uint32_t word = wq[buf][r][q];
+          if (WBITS == 4) {
+            f[r] = s4_to_f32_div16(word >> (4 * e));
+          } else {
+            f[r] = (float)(int8_t)((word >> (8 * e)) & 0xffu);
+          }
+          if (MODE == kRounded) f[r] = f[r] * sc[j];
+        }
+        uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                    pack_bf16x2(f[6], f[7])};
+        const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+      }
+    }
+  };
+
+  if (k_begin < k_end) {
+    load_rows(0, k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+      load_rows(1, k0 + 32);
+      compute(0, k0);
+      load_rows(0, k0 + 64);
+      compute(1, k0 + 32);
+    }
+  }
+
+  // ---- add the waves' tiles through LDS; wave w finishes registers [w*R/WAVES, (w+1)*R/WAVES)
+  // Register index r = (mt*4 + t)*NV + j; in the accumulator tile, lane (li, kb) register t of
+  // instruction j is channel strip*TN + (4*kb + t)*NV + j, token 16*mt + li.
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float v = acc[j][mt][t];
+        if (MODE == kFactored && WBITS == 4) v *= 16.0f;  // undo value/16 (exact)
+        lds[(wave * R + (mt * 4 + t) * NV + j) * 64 + lane] = v;
+      }
+  __syncthreads();
+
+  constexpr int RPW = R / WAVES;  // registers finished per wave; divides NV or is a multiple of it
+  static_assert(R % WAVES == 0, "accumulators must split evenly over the waves");
+  static_assert(RPW >= NV ? RPW % NV == 0 : NV % RPW == 0, "finish chunks must align to channel runs");
+  constexpr int RUN = RPW < NV ? RPW : NV;  // consecutive channels finished together
+#pragma unroll
+  for (int c = 0; c < RPW / RUN; ++c) {
+    const int r0 = wave * RPW + c * RUN;
+    const int mt_t = r0 / NV, j0 = r0 % NV;
+    const int mt = mt_t / 4, t = mt_t % 4;
+    const int m = mt * 16 + li;
+    const int n0 = strip * TN + (4 * kb + t) * NV + j0;
+    float sum[RUN];
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) {
+      float s = 0.0f;
+#pragma unroll
+      for (int w2 = 0; w2 < WAVES; ++w2) s = s + lds[(w2 * R + r0 + u) * 64 + lane];
+      sum[u] = s;
+    }
+    if (m >= p.M || n0 >= p.N) continue;
+    if (p.slices > 1) {
+      float* dst = p.workspace + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
+#pragma unroll
+      for (int u = 0; u < RUN; ++u) dst[u] = sum[u];
+    } else {
+      uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n0;
+#pragma unroll
+      for (int u = 0; u < RUN; ++u) {
+        float v = sum[u];
+        if (MODE == kFactored)
+          v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n0 + u,
+                             p.scale_is_bf16);
+        const float b = p.bias ? load_scale(p.bias, n0 + u, p.bias_is_bf16) : 0.0f;
+        dst[u] = f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+      }
+    }
+  }
+}
+
+// Sums the K-slices of the workspace in slice order and applies scale/bias/activation.
+__global__ __launch_bounds__(256) void dequant_dot_finalize_kernel(DecodeParams p, int mode) {
+  const size_t total = (size_t)p.M * p.N;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int batch = blockIdx.y;
+  if (idx >= total) return;
+  const int n = (int)(idx % p.N);
+  const float* ws = p.workspace + (size_t)batch * p.slices * total + idx;
+  float v = 0.0f;
+  for (int s = 0; s < p.slices; ++s) v = v + ws[(size_t)s * total];
+  if (mode == kFactored)
+    v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n, p.scale_is_bf16);
+  const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  p.out[(size_t)batch * total + idx] =
+      f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+}
+
+// Any shape, any alignment: one thread per output, k in increasing order.  Correct for every
+// case the handlers accept; used when the streaming kernels' divisibility rules do not hold
+// and for grouped scales with an f32-typed multiply.
+__global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p, int wbits, int mode) {
+  const size_t total = (size_t)p.M * p.N;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int batch = blockIdx.y;
+  if (idx >= total) return;
+  const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+  const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
+  const size_t wbase = (size_t)batch * p.K * p.N;
+  const size_t sbase = (size_t)(p.scale_batched ? batch : 0) * (p.K / p.group) * p.N;
+  float acc = 0.0f;
+  for (int k = 0; k < p.K; ++k) {
+    const size_t e = wbase + (size_t)k * p.N + n;
+    int wi;
+    if (wbits == 8) {
+      wi = (int8_t)p.w[e];
+    } else {
+      const uint32_t nib = (p.w[e >> 1] >> (4 * (e & 1))) & 0xfu;
+      wi = (int)(nib ^ 8u) - 8;
+    }
+    float s = load_scale(p.scales, sbase + (size_t)(k / p.group) * p.N + n, p.scale_is_bf16);
+    float wv = (float)wi * s;
+    if (mode == kRounded) wv = round_bf16(wv);
+    acc = acc + bf16_to_f32(a[k]) * wv;
+  }
+  const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  p.out[(size_t)batch * total + idx] =
+      f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+}
+
+template <int WBITS, int VEC, int MT, int WAVES, int MODE>
+int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
+  constexpr int NV = VEC * 8 / WBITS;
+  constexpr int R = NV * 4 * MT;
+  const size_t lds_bytes = (size_t)WAVES * R * 64 * sizeof(float);
+  auto kern = dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE>;
+  if (lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes);
+    if (e != hipSuccess)
+      return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot: cannot reserve %zu bytes of LDS: %s",
+                  lds_bytes, hipGetErrorString(e));
+  }
+  dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
+  hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds_bytes, stream, dp);
+  int rc = CheckLaunch(name);
+  if (rc) return rc;
+  if (dp.slices > 1) {
+    dim3 fgrid((unsigned)(((size_t)dp.M * dp.N + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(dequant_dot_finalize_kernel, fgrid, dim3(256), 0, stream, dp, MODE);
+    rc = CheckLaunch("dequant_dot_finalize");
+  }
+  SetLastKernel(name);
+  return rc;
+}
+
+}  // namespace
+
+int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream);  // dequant_dot_mfma.hip
+
+// Rows of K each workgroup takes so that `slices` workgroups cover K; multiple of 32*waves.
+static int RowsPerSlice(int K, int slices, int waves) {
+  const int unit = 32 * waves;
+  const int per = (K + slices - 1) / slices;
+  return (per + unit - 1) / unit * unit;
+}
+
+size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices) {
+  return slices > 1 ? (size_t)batch * slices * M * N * sizeof(float) : 0;
+}
+
+int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
+  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4;
+  if (!s4 && p.weight_dtype != XLA_FFI_DataType_S8)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: weights must be S4 or S8");
+  if (!IsF32OrBf16(p.scale_dtype) || !IsF32OrBf16(p.dequant_type) || !IsF32OrBf16(p.dot_type) ||
+      !IsF32OrBf16(p.epilogue_type) || (p.bias && !IsF32OrBf16(p.bias_dtype)))
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: types must be F32 or BF16");
+  if (p.batch < 0 || p.M < 0 || p.K < 0 || p.N < 0 || p.M > 0x7fffffff || p.K > 0x7fffffff ||
+      p.N > 0x7fffffff || p.batch > 65535)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: bad shape");
+  if (p.K > 0 && (p.group <= 0 || p.K % p.group != 0))
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT,
+                "dequant_dot: group size %lld does not divide K=%lld", (long long)p.group,
+                (long long)p.K);
+  if (p.epilogue < 0 || p.epilogue > XLA_AMD_EPI_BIAS_SILU)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: unknown epilogue %d", p.epilogue);
+  if ((p.epilogue & 1) && !p.bias)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: BIAS epilogue without a bias");
+  if (p.scale_batch != 1 && p.scale_batch != p.batch)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: scale batch must be 1 or batch");
+  if (p.dequant_type == XLA_FFI_DataType_BF16 && p.scale_dtype != XLA_FFI_DataType_BF16)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT,
+                "dequant_dot: a bf16-typed dequantise multiply needs bf16 scales");
+  if (p.batch == 0 || p.M == 0 || p.N == 0) {
+    SetLastKernel("dequant_dot:empty");
+    return 0;
+  }
+  if (!p.lhs || !p.weights || !p.scales || !p.out)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: null buffer");
+
+  DecodeParams dp;
+  dp.lhs = (const uint16_t*)p.lhs;
+  dp.w = (const uint8_t*)p.weights;
+  dp.scales = p.scales;
+  dp.bias = (p.epilogue & 1) ? p.bias : nullptr;
+  dp.out = (uint16_t*)p.out;
+  dp.workspace = (float*)p.workspace;
+  dp.M = (int)p.M; dp.K = (int)p.K; dp.N = (int)p.N;
+  dp.group = p.K > 0 ? (int)p.group : 1;
+  dp.scale_is_bf16 = p.scale_dtype == XLA_FFI_DataType_BF16;
+  dp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
+  dp.scale_batched = p.scale_batch == p.batch && p.batch > 1;
+  dp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
+  dp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
+  dp.epilogue = p.epilogue;
+  dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
+  const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
+  const bool per_channel = p.group == p.K;
+
+  const int force = GetOption("dequant_dot_kernel");  // 0 auto, 1 generic, 2 decode, 3 prefill
+  const bool aligned = p.K % 8 == 0 && p.group % 8 == 0 && ((uintptr_t)p.lhs % 16 == 0) &&
+                       ((uintptr_t)p.weights % 16 == 0);
+  const bool mode_ok = mode == kRounded || per_channel;
+
+  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64) {
+    int rc = LaunchDequantDotPrefill(p, stream);
+    if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
+  }
+
+  if (force != 1 && force != 3 && aligned && mode_ok && p.M <= 64 && p.K >= 32) {
+    // VEC bytes per lane per row -> NV channels per lane; needs N % NV == 0 and 16-byte rows
+    const int mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+    int vec = mt == 1 ? (s4 ? 8 : 16) : mt == 2 ? (s4 ? 4 : 8) : 4;
+    if (int v = GetOption("dequant_dot_vec")) vec = v;
+    const int nv = vec * (s4 ? 2 : 1);
+    const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
+    const bool shape_ok = p.N % nv == 0 && row_bytes % vec == 0 && nv * mt <= 32 &&
+                          (vec == 4 || vec == 8 || vec == 16) && (s4 || nv * mt <= 16 || true);
+    if (shape_ok) {
+      const int waves = 8;
+      dp.strips = (int)((p.N + 16 * nv - 1) / (16 * nv));
+      // enough workgroups for ~2 per CU, but never slices that leave a wave without rows
+      int slices = 1;
+      if (int s = GetOption("dequant_dot_slices")) {
+        slices = s;
+      } else {
+        while (dp.strips * slices * p.batch < 384 && p.K / (slices * 2) >= 32 * waves &&
+               slices * 2 * p.M <= 64)
+          slices *= 2;
+      }
+      if (slices > 1 && (!p.workspace ||
+                         p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, slices)))
+        slices = 1;
+      dp.slices = slices;
+      dp.rows_per_slice = RowsPerSlice(dp.K, slices, waves);
+#define XLA_AMD_DECODE(WB, V, MT_, MODE_, NAME)                                       \
+  if ((s4 ? 4 : 8) == WB && vec == V && mt == MT_ && mode == MODE_)                   \
+    return launch_decode<WB, V, MT_, 8, MODE_>(dp, (int)p.batch, stream, NAME);
+      XLA_AMD_DECODE(4, 16, 1, kRounded, "dequant_dot_decode_s4_v16_m16_rounded")
+      XLA_AMD_DECODE(4, 8, 1, kRounded, "dequant_dot_decode_s4_v8_m16_rounded")
+      XLA_AMD_DECODE(4, 4, 1, kRounded, "dequant_dot_decode_s4_v4_m16_rounded")
+      XLA_AMD_DECODE(4, 8, 2, kRounded, "dequant_dot_decode_s4_v8_m32_rounded")
+      XLA_AMD_DECODE(4, 4, 2, kRounded, "dequant_dot_decode_s4_v4_m32_rounded")
+      XLA_AMD_DECODE(4, 4, 4, kRounded, "dequant_dot_decode_s4_v4_m64_rounded")
+      XLA_AMD_DECODE(4, 8, 1, kFactored, "dequant_dot_decode_s4_v8_m16_factored")
+      XLA_AMD_DECODE(4, 4, 2, kFactored, "dequant_dot_decode_s4_v4_m32_factored")
+      XLA_AMD_DECODE(4, 4, 4, kFactored, "dequant_dot_decode_s4_v4_m64_factored")
+      XLA_AMD_DECODE(8, 16, 1, kRounded, "dequant_dot_decode_s8_v16_m16_rounded")
+      XLA_AMD_DECODE(8, 8, 1, kRounded, "dequant_dot_decode_s8_v8_m16_rounded")
+      XLA_AMD_DECODE(8, 8, 2, kRounded, "dequant_dot_decode_s8_v8_m32_rounded")
+      XLA_AMD_DECODE(8, 4, 4, kRounded, "dequant_dot_decode_s8_v4_m64_rounded")
+      XLA_AMD_DECODE(8, 16, 1, kFactored, "dequant_dot_decode_s8_v16_m16_factored")
+      XLA_AMD_DECODE(8, 8, 1, kFactored, "dequant_dot_decode_s8_v8_m16_factored")
+      XLA_AMD_DECODE(8, 8, 2, kFactored, "dequant_dot_decode_s8_v8_m32_factored")
+      XLA_AMD_DECODE(8, 4, 4, kFactored, "dequant_dot_decode_s8_v4_m64_factored")
+#undef XLA_AMD_DECODE
+      dp.strips = 1; dp.slices = 1;
+    }
+  }
+  if (force == 2 || force == 3)
+    return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
+                "dequant_dot: the requested kernel does not cover this shape");
+  // fallback: any shape
+  {
+    dp.slices = 1;
+    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)p.batch);
+    hipLaunchKernelGGL(dequant_dot_generic_kernel, grid, dim3(256), 0, stream, dp, s4 ? 4 : 8, mode);
+    SetLastKernel("dequant_dot_generic");
+    return CheckLaunch("dequant_dot_generic");
+  }
+}
+
+}  // namespace xla_amd

@@ -1,0 +1,174 @@
+// Device-side element-type helpers shared by the gfx950 kernels.
+//
+// The library is compiled with -ffp-contract=off: every `a * b + c` written
+// below is two roundings, and a fused multiply-add appears only where
+// __builtin_fmaf is spelled out.  Casts follow the XLA CPU backend's
+// definitions: f32 -> bf16 is round-to-nearest-even with quiet NaNs
+// (xla/codegen/intrinsic/fptrunc.cc:64-114), f32 -> f8e4m3fn is
+// round-to-nearest-even with overflow to NaN (fptrunc.cc:275-511).
+#ifndef XLA_AMD_CSRC_DEVICE_NUMERICS_H_
+#define XLA_AMD_CSRC_DEVICE_NUMERICS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xla_amd {
+
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// bf16 pair packed in one dword -> two f32 (exact)
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return bits_to_f32(w << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) { return bits_to_f32(w & 0xffff0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return bits_to_f32((uint32_t)h << 16); }
+
+// two f32 -> packed bf16 pair, RNE, NaN -> quiet NaN with the sign kept: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  floatx2 v = {lo, hi};
+  bf16x2 b = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, b);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) { return (uint16_t)(pack_bf16x2(x, 0.0f) & 0xffffu); }
+// value of an f32 after a bf16-typed HLO op re-rounds it
+__device__ __forceinline__ float round_bf16(float x) { return bf16lo_to_f32(pack_bf16x2(x, 0.0f)); }
+
+// f8e4m3fn code -> f32 (exact; 0x7F/0xFF -> NaN), pure integer/f32 arithmetic
+__device__ __forceinline__ float f8e4m3fn_to_f32(uint32_t c) {
+  uint32_t mag = c & 0x7fu;
+  // normal codes: move exponent+mantissa to the f32 fields and re-bias by 127-7;
+  // subnormal codes (mag < 8) are mag * 2^-9.
+  float v = mag < 8u ? (float)mag * 0x1p-9f : bits_to_f32((mag << 20) + (120u << 23));
+  if (mag == 0x7fu) v = bits_to_f32(0x7fc00000u);
+  return bits_to_f32(f32_to_bits(v) | ((c & 0x80u) << 24));
+}
+
+// Software f32 -> f8e4m3fn, all inputs (slow path; the hot loops use the
+// hardware convert on values already clamped to +-448).
+__device__ __forceinline__ uint32_t f32_to_f8e4m3fn_any(float x) {
+  uint32_t u = f32_to_bits(x), a = u & 0x7fffffffu, sign = (u >> 24) & 0x80u;
+  uint32_t code;
+  if (a > 0x43e80000u) {  // |x| > 464 (0x43e80000), inf, NaN
+    code = 0x7fu;
+  } else if (a < 0x3c800000u) {  // below 2^-6: subnormal grid of 2^-9, ties to even
+    code = (uint32_t)__builtin_rintf(bits_to_f32(a) * 512.0f);
+  } else {
+    uint32_t r = a + 0x7ffffu + ((a >> 20) & 1u);  // RNE at 3 mantissa bits
+    code = (r >> 20) - (120u << 3);
+  }
+  return code | sign;
+}
+
+// 4 f32 (clamped to +-448, not NaN) -> 4 f8e4m3fn codes in one dword; gfx950's
+// v_cvt_pk_fp8_f32 is OCP e4m3fn with round-to-nearest-even.
+__device__ __forceinline__ uint32_t pack_f8x4(float a, float b, float c, float d) {
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  return (uint32_t)r;
+}
+
+// xla/codegen/intrinsic/tanh.cc:48-108 rational, then the |x| >= 20 -> +-1 rule of :33-46.
+__device__ __forceinline__ float tanh_xla(float x) {
+  const float kClamp = 7.99881172180175781f;
+  float ax = __builtin_fabsf(x);
+  float xc = __builtin_fminf(__builtin_fmaxf(x, -kClamp), kClamp);
+  float x2 = xc * xc;
+  float p = -2.76076847742355e-16f;
+  p = x2 * p + 2.00018790482477e-13f;
+  p = x2 * p + -8.60467152213735e-11f;
+  p = x2 * p + 5.12229709037114e-08f;
+  p = x2 * p + 1.48572235717979e-05f;
+  p = x2 * p + 6.37261928875436e-04f;
+  p = x2 * p + 4.89352455891786e-03f;
+  p = xc * p;
+  float q = 1.19825839466702e-06f;
+  q = x2 * q + 1.18534705686654e-04f;
+  q = x2 * q + 2.26843463243900e-03f;
+  q = x2 * q + 4.89352518554385e-03f;
+  float r = ax < 0.0004f ? x : p / q;
+  return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
+}
+
+// xla/backends/cpu/codegen/polynomial_approximations.cc:173-296 (Cephes expf)
+__device__ __forceinline__ float exp_xla(float x) {
+  float in = __builtin_fminf(__builtin_fmaxf(x, -87.8f), 88.8f);
+  float n = __builtin_floorf(in * 1.44269504088896341f + 0.5f);
+  n = __builtin_fminf(__builtin_fmaxf(n, -127.0f), 127.0f);
+  float r = in - 0.693359375f * n;
+  r = r - -2.12194440e-4f * n;
+  float z = r * 1.9875691500E-4f + 1.3981999507E-3f;
+  z = z * r + 8.3334519073E-3f;
+  z = z * r + 4.1665795894E-2f;
+  z = z * r + 1.6666665459E-1f;
+  z = z * r + 5.0000001201E-1f;
+  z = z * (r * r) + r;
+  z = 1.0f + z;
+  float p2 = bits_to_f32((uint32_t)((int)n + 0x7f) << 23);
+  float res = z * p2;
+  return x != x ? x : res;
+}
+
+enum : int { kEpiDefault = 0, kEpiBias = 1, kEpiRelu = 2, kEpiBiasRelu = 3, kEpiGelu = 4,
+             kEpiBiasGelu = 5, kEpiSilu = 6, kEpiBiasSilu = 7 };
+
+// What follows the dot in the matched HLO, op by op.  BF16_DOT: the dot
+// instruction is bf16-typed (accumulator rounded first).  BF16_OPS: bias add
+// and activation ops are bf16-typed, each result re-rounded (what
+// FloatNormalization makes of them, xla/service/cpu/cpu_compiler.cc:804-817);
+// otherwise they run in f32 and only the final convert rounds.  GELU op order:
+// gemm_rewriter_fp8_test.cc:1123-1141; SiLU: gemm_rewriter.cc:995-1002.
+template <bool BF16_DOT, bool BF16_OPS>
+__device__ __forceinline__ float epilogue_value(float acc, float bias, int epi) {
+  auto R = [](float v) { return BF16_OPS ? round_bf16(v) : v; };
+  float x = BF16_DOT ? round_bf16(acc) : acc;
+  x = R(x);
+  if (epi & 1) x = R(x + R(bias));
+  switch (epi & ~1) {
+    case kEpiRelu:
+      x = x > 0.0f ? x : (x != x ? x : 0.0f);
+      break;
+    case kEpiGelu: {
+      float m0 = R(x * x);
+      float m1 = R(x * m0);
+      float m2 = R(m1 * R(0.044715f));
+      float a0 = R(x + m2);
+      float m3 = R(a0 * R(0.797884583f));
+      float th = R(tanh_xla(m3));
+      float a2 = R(th + 1.0f);
+      float m4 = R(a2 * 0.5f);
+      x = R(x * m4);
+      break;
+    }
+    case kEpiSilu: {
+      float ex = R(exp_xla(-x));
+      float dn = R(1.0f + ex);
+      float sg = R(1.0f / dn);
+      x = R(x * sg);
+      break;
+    }
+    default:
+      break;
+  }
+  return x;
+}
+
+__device__ __forceinline__ float epilogue_dispatch(float acc, float bias, int epi, bool bf16_dot,
+                                                   bool bf16_ops) {
+  if (bf16_ops) {
+    return bf16_dot ? epilogue_value<true, true>(acc, bias, epi)
+                    : epilogue_value<false, true>(acc, bias, epi);
+  }
+  return bf16_dot ? epilogue_value<true, false>(acc, bias, epi)
+                  : epilogue_value<false, false>(acc, bias, epi);
+}
+
+}  // namespace xla_amd
+#endif  // XLA_AMD_CSRC_DEVICE_NUMERICS_H_

@@ -1,0 +1,32 @@
+// Host-side plumbing shared by the launchers: per-thread error text, the name
+// of the kernel variant last selected, and the internal launch entry points
+// the C ABI in include/xla_amd_quant.h forwards to.
+#ifndef XLA_AMD_CSRC_LAUNCH_H_
+#define XLA_AMD_CSRC_LAUNCH_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "xla_amd_quant.h"
+
+namespace xla_amd {
+
+// Records `msg` as this thread's last error and returns `code`.
+int Fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void SetLastKernel(const char* name);
+// hipGetLastError() after a launch -> 0 or XLA_FFI_Error_Code_INTERNAL with the HIP message.
+int CheckLaunch(const char* what);
+
+// Tuning knobs set through xla_amd_debug_set_option (0 = default choice).
+int GetOption(const char* key);
+
+int LaunchRowwiseQuantize(const XlaAmdRowwiseQuantize& p, hipStream_t stream, int variant);
+int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream);
+int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
+
+inline bool IsF32OrBf16(int32_t t) {
+  return t == XLA_FFI_DataType_F32 || t == XLA_FFI_DataType_BF16;
+}
+
+}  // namespace xla_amd
+#endif  // XLA_AMD_CSRC_LAUNCH_H_

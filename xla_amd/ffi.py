@@ -1,0 +1,340 @@
+"""A small XLA-FFI host in Python: builds ``XLA_FFI_CallFrame`` structs with ctypes and calls
+the library's handlers the way ``CustomCallThunk`` does
+(xla/backends/gpu/runtime/custom_call_thunk.cc:110-157,394-422), including the function
+table (``XLA_FFI_Api``) a handler calls back into for errors and for the stream.
+
+Struct layouts restate xla/ffi/api/c_api.h (same field order as include/xla_ffi_abi.h).
+Device memory and streams come from the caller (torch tensors' ``data_ptr()`` and
+``torch.cuda.current_stream().cuda_stream``); nothing here touches the GPU itself.
+"""
+import ctypes as C
+import os
+
+from . import dtypes
+
+_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+LIB_PATH = os.path.join(_LIB_DIR, "libxla_amd_quant.so")
+
+HANDLER_SYMBOLS = {
+    "xla_amd.dequant_dot": "xla_amd_dequant_dot",
+    "xla_amd.fp8_scaled_dot": "xla_amd_fp8_scaled_dot",
+    "xla_amd.rowwise_quantize_fp8": "xla_amd_rowwise_quantize_fp8",
+}
+EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
+    "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_fp8_scaled_dot",
+    "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
+    "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
+    "xla_amd_debug_set_option"]
+
+STAGE_INSTANTIATE, STAGE_PREPARE, STAGE_INITIALIZE, STAGE_EXECUTE, STAGE_RECORD = range(5)
+ATTR_ARRAY, ATTR_DICTIONARY, ATTR_SCALAR, ATTR_STRING = 1, 2, 3, 4
+ERROR_CODES = {0: "OK", 3: "INVALID_ARGUMENT", 9: "FAILED_PRECONDITION", 12: "UNIMPLEMENTED",
+               13: "INTERNAL"}
+TRAIT_COMMAND_BUFFER_COMPATIBLE = 1
+
+
+class Extension(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("type", C.c_int), ("next", C.c_void_p)]
+
+
+class ApiVersion(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p),
+                ("major_version", C.c_int), ("minor_version", C.c_int)]
+
+
+class ErrorCreateArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p),
+                ("message", C.c_char_p), ("errc", C.c_int)]
+
+
+class Buffer(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("dtype", C.c_int),
+                ("data", C.c_void_p), ("rank", C.c_int64), ("dims", C.POINTER(C.c_int64))]
+
+
+class ByteSpan(C.Structure):
+    _fields_ = [("ptr", C.c_char_p), ("len", C.c_size_t)]
+
+
+class Scalar(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("value", C.c_void_p)]
+
+
+class Array(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("size", C.c_size_t), ("data", C.c_void_p)]
+
+
+class Args(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("size", C.c_int64),
+                ("types", C.POINTER(C.c_int)), ("args", C.POINTER(C.c_void_p))]
+
+
+class Attrs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("size", C.c_int64),
+                ("types", C.POINTER(C.c_int)), ("names", C.POINTER(C.POINTER(ByteSpan))),
+                ("attrs", C.POINTER(C.c_void_p))]
+
+
+class CallFrame(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("api", C.c_void_p),
+                ("ctx", C.c_void_p), ("stage", C.c_int), ("args", Args), ("rets", Args),
+                ("attrs", Attrs), ("future", C.c_void_p)]
+
+
+CALL_FRAME_STRUCT_SIZE = CallFrame.attrs.offset + C.sizeof(Attrs)
+
+
+class StreamGetArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("ctx", C.c_void_p),
+                ("stream", C.c_void_p)]
+
+
+class RegisterArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("name", ByteSpan),
+                ("platform", ByteSpan), ("instantiate", C.c_void_p), ("prepare", C.c_void_p),
+                ("initialize", C.c_void_p), ("execute", C.c_void_p), ("record", C.c_void_p),
+                ("traits", C.c_uint32)]
+
+
+class Metadata(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("api_version", ApiVersion), ("traits", C.c_uint32),
+                ("state_type_id", C.c_int64)]
+
+
+class MetadataExtension(C.Structure):
+    _fields_ = [("base", Extension), ("metadata", C.POINTER(Metadata))]
+
+
+_FN = C.CFUNCTYPE(C.c_void_p, C.c_void_p)
+_API_SLOTS = ["Error_Create", "Error_GetDetails", "Error_Destroy", "Handler_Register", "Stream_Get",
+              "Type_Register", "InvokeContext_Get", "State_Set", "State_Get",
+              "DeviceMemory_Allocate", "DeviceMemory_Free", "ThreadPool_Schedule",
+              "ThreadPool_NumThreads", "Future_Create", "Future_SetAvailable", "Future_SetError",
+              "RunId_Get", "DeviceOrdinal_Get", "InvokeContext_FindExtension"]
+
+
+class Api(C.Structure):
+    _fields_ = ([("struct_size", C.c_size_t), ("extension_start", C.c_void_p),
+                 ("api_version", ApiVersion), ("internal_api", C.c_void_p)] +
+                [(n, _FN) for n in _API_SLOTS])
+
+
+class FfiError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("%s: %s" % (ERROR_CODES.get(code, code), message))
+        self.code = code
+        self.message = message
+
+
+class Host:
+    """Owns the function table; one per process is enough.  ``stream`` is the hipStream_t
+    (an int) handed to handlers through XLA_FFI_Stream_Get."""
+
+    def __init__(self, stream=0, fail_stream_get=False):
+        self.stream = stream
+        self.fail_stream_get = fail_stream_get
+        self.errors = {}
+        self.registry = {}
+        self._next_error = 1
+        self._keep = []
+        api = Api()
+        api.struct_size = Api.InvokeContext_FindExtension.offset + C.sizeof(_FN)
+        api.api_version = ApiVersion(C.sizeof(ApiVersion), None, 0, 4)
+
+        def error_create(p):
+            a = C.cast(p, C.POINTER(ErrorCreateArgs)).contents
+            h = self._next_error
+            self._next_error += 1
+            self.errors[h] = (a.errc, a.message.decode())
+            return h
+
+        def stream_get(p):
+            a = C.cast(p, C.POINTER(StreamGetArgs)).contents
+            if self.fail_stream_get:
+                h = self._next_error
+                self._next_error += 1
+                self.errors[h] = (3, "XLA FFI GPU context is not available")
+                return h
+            a.stream = self.stream
+            return None
+
+        def handler_register(p):
+            a = C.cast(p, C.POINTER(RegisterArgs)).contents
+            name = C.string_at(a.name.ptr, a.name.len).decode()
+            platform = C.string_at(a.platform.ptr, a.platform.len).decode()
+            self.registry[(name, platform.lower())] = (a.execute, a.traits)
+            return None
+
+        def unimplemented(p):
+            h = self._next_error
+            self._next_error += 1
+            self.errors[h] = (12, "not implemented by this host")
+            return h
+
+        table = {"Error_Create": error_create, "Stream_Get": stream_get,
+                 "Handler_Register": handler_register}
+        for n in _API_SLOTS:
+            cb = _FN(table.get(n, unimplemented))
+            self._keep.append(cb)
+            setattr(api, n, cb)
+        self.api = api
+
+    def take_error(self, handle):
+        return self.errors.pop(handle)
+
+
+_lib = None
+
+
+def library():
+    """The HIP library, loaded once.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m xla_amd.build` (hipcc, gfx950); "
+                               "this package has no CPU fallback" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for sym in HANDLER_SYMBOLS.values():
+            fn = getattr(L, sym)
+            fn.restype = C.c_void_p
+            fn.argtypes = [C.c_void_p]
+        L.xla_amd_register_handlers.restype = C.c_void_p
+        L.xla_amd_register_handlers.argtypes = [C.c_void_p]
+        L.xla_amd_last_error.restype = C.c_char_p
+        L.xla_amd_last_kernel.restype = C.c_char_p
+        L.xla_amd_debug_set_option.argtypes = [C.c_char_p, C.c_int]
+        L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
+        L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
+        L.xla_amd_fp8_scaled_dot_workspace_bytes.restype = C.c_size_t
+        L.xla_amd_fp8_scaled_dot_workspace_bytes.argtypes = [C.c_int64] * 3 + [C.c_int32]
+        _lib = L
+    return _lib
+
+
+def _buffer(dtype, data_ptr, dims):
+    dims = list(dims)
+    arr = (C.c_int64 * max(len(dims), 1))(*dims)
+    b = Buffer(C.sizeof(Buffer), None, dtype, data_ptr, len(dims), C.cast(arr, C.POINTER(C.c_int64)))
+    return b, arr
+
+
+_SCALAR_CTYPES = {dtypes.PRED: C.c_bool, dtypes.S8: C.c_int8, dtypes.S16: C.c_int16,
+                  dtypes.S32: C.c_int32, dtypes.S64: C.c_int64, dtypes.U8: C.c_uint8,
+                  dtypes.U32: C.c_uint32, dtypes.U64: C.c_uint64, dtypes.F32: C.c_float,
+                  dtypes.F64: C.c_double}
+
+
+class Attr:
+    """Typed attribute value: Attr.i32(3), Attr.i64(0), Attr.f32(1e-6), Attr.pred(True), Attr.str("BIAS")."""
+
+    def __init__(self, kind, dtype, value):
+        self.kind, self.dtype, self.value = kind, dtype, value
+
+    i32 = staticmethod(lambda v: Attr(ATTR_SCALAR, dtypes.S32, int(v)))
+    i64 = staticmethod(lambda v: Attr(ATTR_SCALAR, dtypes.S64, int(v)))
+    f32 = staticmethod(lambda v: Attr(ATTR_SCALAR, dtypes.F32, float(v)))
+    f64 = staticmethod(lambda v: Attr(ATTR_SCALAR, dtypes.F64, float(v)))
+    pred = staticmethod(lambda v: Attr(ATTR_SCALAR, dtypes.PRED, bool(v)))
+    str = staticmethod(lambda v: Attr(ATTR_STRING, 0, v))
+    i64_array = staticmethod(lambda v: Attr(ATTR_ARRAY, dtypes.S64, list(v)))
+
+
+class Frame:
+    """One call frame plus everything it points at (kept alive as attributes)."""
+
+    def __init__(self, host, args, rets, attrs=None, stage=STAGE_EXECUTE):
+        """args/rets: lists of (dtype, data_ptr, dims); attrs: dict name -> Attr."""
+        self.host = host
+        keep = self._keep = []
+        f = self.frame = CallFrame()
+        f.struct_size = CALL_FRAME_STRUCT_SIZE
+        f.api = C.addressof(host.api)
+        f.ctx = 0xC0FFEE
+        f.stage = stage
+
+        def fill(side, items):
+            n = len(items)
+            types = (C.c_int * max(n, 1))(*([1] * n))
+            ptrs = (C.c_void_p * max(n, 1))()
+            for i, (dt, ptr, dims) in enumerate(items):
+                b, arr = _buffer(dt, ptr, dims)
+                keep.extend([b, arr])
+                ptrs[i] = C.addressof(b)
+            side.struct_size = C.sizeof(Args)
+            side.size = n
+            side.types = C.cast(types, C.POINTER(C.c_int))
+            side.args = C.cast(ptrs, C.POINTER(C.c_void_p))
+            keep.extend([types, ptrs])
+
+        fill(f.args, args)
+        fill(f.rets, rets)
+        attrs = attrs or {}
+        names = sorted(attrs)                     # XLA passes attributes sorted by name
+        n = len(names)
+        types = (C.c_int * max(n, 1))()
+        nptrs = (C.POINTER(ByteSpan) * max(n, 1))()
+        vptrs = (C.c_void_p * max(n, 1))()
+        for i, name in enumerate(names):
+            a = attrs[name]
+            raw = name.encode()
+            span = ByteSpan(raw, len(raw))
+            keep.extend([raw, span])
+            nptrs[i] = C.pointer(span)
+            types[i] = a.kind
+            if a.kind == ATTR_SCALAR:
+                val = _SCALAR_CTYPES[a.dtype](a.value)
+                sc = Scalar(a.dtype, C.cast(C.pointer(val), C.c_void_p))
+                keep.extend([val, sc])
+                vptrs[i] = C.addressof(sc)
+            elif a.kind == ATTR_STRING:
+                sraw = a.value.encode()
+                sspan = ByteSpan(sraw, len(sraw))
+                keep.extend([sraw, sspan])
+                vptrs[i] = C.addressof(sspan)
+            else:
+                data = (_SCALAR_CTYPES[a.dtype] * max(len(a.value), 1))(*a.value)
+                arr = Array(a.dtype, len(a.value), C.cast(data, C.c_void_p))
+                keep.extend([data, arr])
+                vptrs[i] = C.addressof(arr)
+        f.attrs.struct_size = C.sizeof(Attrs)
+        f.attrs.size = n
+        f.attrs.types = C.cast(types, C.POINTER(C.c_int))
+        f.attrs.names = C.cast(nptrs, C.POINTER(C.POINTER(ByteSpan)))
+        f.attrs.attrs = C.cast(vptrs, C.POINTER(C.c_void_p))
+        keep.extend([types, nptrs, vptrs])
+
+    def address(self):
+        return C.addressof(self.frame)
+
+
+def invoke(target, frame):
+    """Calls the handler registered for ``target``; raises FfiError on a non-null result."""
+    fn = getattr(library(), HANDLER_SYMBOLS[target])
+    err = fn(frame.address())
+    if err:
+        code, msg = frame.host.take_error(err)
+        raise FfiError(code, msg)
+
+
+def query_metadata(target, host):
+    """The registration-time handshake (xla/ffi/invoke.cc:218-233): returns (major, minor, traits)."""
+    md = Metadata()
+    md.struct_size = Metadata.traits.offset + C.sizeof(C.c_uint32)
+    ext = MetadataExtension()
+    ext.base.struct_size = C.sizeof(MetadataExtension)
+    ext.base.type = 1
+    ext.metadata = C.pointer(md)
+    fr = Frame(host, [], [])
+    fr.frame.extension_start = C.addressof(ext)
+    invoke(target, fr)
+    return md.api_version.major_version, md.api_version.minor_version, md.traits
+
+
+def last_kernel():
+    return library().xla_amd_last_kernel().decode()
+
+
+def set_option(key, value):
+    rc = library().xla_amd_debug_set_option(key.encode(), int(value))
+    if rc != 0:
+        raise KeyError(key)

@@ -1,0 +1,119 @@
+"""The three custom calls as Python callables over device tensors.
+
+Every function builds an XLA FFI call frame and goes through the library's exported
+handler symbol -- the same entry XLA's CustomCallThunk would call -- on torch's current
+HIP stream.  torch only supplies device memory and the stream.  bf16 operands are
+``torch.bfloat16`` tensors, f8e4m3fn operands ``torch.float8_e4m3fn`` (or ``uint8`` codes),
+s8 weights ``int8``, s4 weights ``uint8`` holding two values per byte (low nibble first)
+with the logical shape passed separately.
+"""
+import torch
+
+from . import dtypes, ffi
+
+_host = None
+
+
+def host():
+    global _host
+    if _host is None:
+        _host = ffi.Host()
+    return _host
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("operands must live on the GPU; this package has no CPU path")
+
+
+_FLOAT = {torch.float32: dtypes.F32, torch.bfloat16: dtypes.BF16}
+_NAMES = {dtypes.F32: "f32", dtypes.BF16: "bf16"}
+_TYPE_ATTR = {"f32": dtypes.F32, "bf16": dtypes.BF16}
+
+
+def _scratch(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device) if nbytes else None
+
+
+def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
+                epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
+                out=None, scratch="auto"):
+    """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K]."""
+    _check_cuda(lhs, weights, scales, bias)
+    wdt = dtypes.S4 if weight_dtype == "s4" else dtypes.S8
+    wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
+    n = wshape[-1]
+    oshape = list(lhs.shape[:-1]) + [n]
+    if out is None:
+        out = torch.empty(oshape, dtype=torch.bfloat16, device=lhs.device)
+    batch = lhs.shape[0] if lhs.dim() == 3 else 1
+    args = [(dtypes.BF16, lhs.data_ptr(), lhs.shape), (wdt, weights.data_ptr(), wshape),
+            (_FLOAT[scales.dtype], scales.data_ptr(), scales.shape)]
+    if bias is not None:
+        args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
+    rets = [(dtypes.BF16, out.data_ptr(), oshape)]
+    if scratch == "auto":
+        nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(batch, lhs.shape[-2], lhs.shape[-1], n, wdt)
+        scratch = _scratch(nbytes, lhs.device)
+    if scratch is not None:
+        rets.append((dtypes.U8, scratch.data_ptr(), [scratch.numel()]))
+    attrs = {"epilogue": ffi.Attr.str(epilogue), "dequant_type": ffi.Attr.i32(_TYPE_ATTR[dequant_type]),
+             "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
+             "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type])}
+    h = host()
+    h.stream = _stream()
+    ffi.invoke("xla_amd.dequant_dot", ffi.Frame(h, args, rets, attrs))
+    return out
+
+
+def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, epilogue="DEFAULT",
+                   dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto"):
+    """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K]; scales f32 []."""
+    _check_cuda(a, b, a_scale, b_scale, bias)
+    m, k = a.shape
+    n = b.shape[1 - rhs_contracting_dim]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    args = [(dtypes.F8E4M3FN, a.data_ptr(), a.shape), (dtypes.F8E4M3FN, b.data_ptr(), b.shape),
+            (dtypes.F32, a_scale.data_ptr(), []), (dtypes.F32, b_scale.data_ptr(), [])]
+    if bias is not None:
+        args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
+    rets = [(dtypes.BF16, out.data_ptr(), [m, n])]
+    if scratch == "auto":
+        nbytes = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(m, k, n, rhs_contracting_dim)
+        scratch = _scratch(nbytes, a.device)
+    if scratch is not None:
+        rets.append((dtypes.U8, scratch.data_ptr(), [scratch.numel()]))
+    attrs = {"epilogue": ffi.Attr.str(epilogue), "dequant_type": ffi.Attr.i32(_TYPE_ATTR[dequant_type]),
+             "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
+             "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type]),
+             "rhs_contracting_dim": ffi.Attr.i64(rhs_contracting_dim)}
+    h = host()
+    h.stream = _stream()
+    ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(h, args, rets, attrs))
+    return out
+
+
+def rowwise_quantize_fp8(x, gamma=None, *, eps=1e-6, q=None, scales=None):
+    """(q, scales) = per-row dynamic f8e4m3fn quantisation of x (bf16 [R,C]), after RMSNorm with
+    ``gamma`` when given.  q is returned as uint8 codes."""
+    _check_cuda(x, gamma)
+    r, c = x.shape
+    if q is None:
+        q = torch.empty((r, c), dtype=torch.uint8, device=x.device)
+    if scales is None:
+        scales = torch.empty((r,), dtype=torch.float32, device=x.device)
+    args = [(dtypes.BF16, x.data_ptr(), [r, c])]
+    if gamma is not None:
+        args.append((dtypes.BF16, gamma.data_ptr(), [c]))
+    rets = [(dtypes.F8E4M3FN, q.data_ptr(), [r, c]), (dtypes.F32, scales.data_ptr(), [r])]
+    attrs = {"rmsnorm": ffi.Attr.pred(gamma is not None), "eps": ffi.Attr.f32(eps)}
+    h = host()
+    h.stream = _stream()
+    ffi.invoke("xla_amd.rowwise_quantize_fp8", ffi.Frame(h, args, rets, attrs))
+    return q, scales
