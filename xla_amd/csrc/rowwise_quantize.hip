@@ -49,7 +49,9 @@ __device__ __forceinline__ float wave_max(float v) {
 __device__ __forceinline__ float div_by_row_scale(float y, float s, float rs) {
   float q0 = y * rs;
   float r = __builtin_fmaf(-q0, s, y);
-  return __builtin_fmaf(r, rs, q0);
+  // s > 0 here, so the quotient carries the sign of y even when it is zero (-0/s = -0, which the
+  // correction step would turn into +0)
+  return __builtin_copysignf(__builtin_fmaf(r, rs, q0), y);
 }
 
 // CH: consecutive 8-element chunks owned by a lane inside one group;

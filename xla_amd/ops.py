@@ -110,7 +110,7 @@ def rowwise_quantize_fp8(x, gamma=None, *, eps=1e-6, q=None, scales=None):
         scales = torch.empty((r,), dtype=torch.float32, device=x.device)
     args = [(dtypes.BF16, x.data_ptr(), [r, c])]
     if gamma is not None:
-        args.append((dtypes.BF16, gamma.data_ptr(), [c]))
+        args.append((dtypes.BF16, gamma.data_ptr(), gamma.shape))
     rets = [(dtypes.F8E4M3FN, q.data_ptr(), [r, c]), (dtypes.F32, scales.data_ptr(), [r])]
     attrs = {"rmsnorm": ffi.Attr.pred(gamma is not None), "eps": ffi.Attr.f32(eps)}
     h = host()
