@@ -78,7 +78,8 @@ def floor_for(w):
 def compare(oracle, w, got, what):
     ref = oracle_dot(oracle, w)
     n_floor = check_dot(got, ref, floor_for(w), what)
-    assert n_floor <= max(4, got.size // 200), "%s: %d outputs only passed through the floor" % (what, n_floor)
+    # near-zero outputs (cancellation, or the flat tail of GELU/SiLU) are judged by the floor
+    assert n_floor <= max(4, got.size // 50), "%s: %d outputs only passed through the floor" % (what, n_floor)
 
 
 # ---- decode kernels (M <= 64) --------------------------------------------------------------

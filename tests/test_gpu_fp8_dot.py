@@ -43,10 +43,20 @@ def reference(oracle, w, **types):
                                  epilogue=EPI[w["epilogue"]])
 
 
-def floor_for(w):
+def floor_for(w, exact_kernel=False):
+    """Absolute floor under the 2-ulp rule.  The exact kernel adds in f32, so only summation order
+    differs from the oracle.  v_mfma_f32_16x16x128_f8f6f4 does not: inside one instruction the
+    products of a group of 8 consecutive k are aligned to the group's largest exponent and bits
+    more than ~13 below it are dropped (measured: 2 products of 448*448 swallow their 6
+    neighbours of 4.0, but not of 16.0).  Each product therefore carries an error of up to
+    2^-13 of its group's maximum; summed as a random walk that is 2^-13 * sqrt(sum (a*b)^2),
+    taken with a factor 2 of slack and 1.2 for the slope of GELU/SiLU."""
     a = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * float(w["a_scale"])
     b = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * float(w["b_scale"])
-    return dot_floor(a, b, w["a"].shape[1])
+    f32_order = dot_floor(a, b, w["a"].shape[1])
+    if exact_kernel:
+        return f32_order
+    return f32_order + 1.2 * 2.0 ** -12 * np.sqrt((a * a) @ (b * b))
 
 
 @pytest.mark.parametrize("nk", [False, True])
@@ -84,7 +94,11 @@ def test_reference_pattern_bf16_typed_ops(oracle):
     types = dict(dequant_type="bf16", dot_type="bf16", epilogue_type="bf16")
     got, kern = run(w, **types)
     ref = reference(oracle, w, **types)
-    fl = floor_for(w) * 12 + np.abs(dtypes.bf16_to_f32(ref)) * 2.0 ** -6
+    # the dot itself is rounded to bf16 here, so an accumulator difference far below one ulp can
+    # flip that rounding; the flip then passes through bias add and nine more bf16-rounded ops.
+    # Allow 6 ulp of the result (the reference's own ErrorSpec for this pattern is 1e-2,
+    # gemm_rewriter_fp8_test.cc:110).
+    fl = floor_for(w) * 12 + np.abs(dtypes.bf16_to_f32(ref)) * 6 * 2.0 ** -8
     check_dot(got, ref, fl, kern)
 
 
@@ -104,7 +118,7 @@ def test_exact_kernel_and_missing_scratch(oracle):
     w = workloads.c3_fp8(48, 80, 40)
     got, kern = run(w, scratch=None)
     assert kern == "fp8_scaled_dot_exact", kern
-    check_dot(got, reference(oracle, w), floor_for(w), kern)
+    check_dot(got, reference(oracle, w), floor_for(w, exact_kernel=True), kern)
     with pytest.raises(ffi.FfiError, match="tiled kernel needs"):
         run(w, force=2, scratch=None)
 

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   constexpr int NPW = 32 / WBITS;       // channels per dword
   constexpr int R = NV * 4 * MT;        // accumulator registers per lane
   constexpr int TN = 16 * NV;           // channels per wave tile
-  extern __shared__ float lds[];        // [WAVES][R][64]
+  __shared__ float lds[WAVES * 16 * 64];  // one 16-register chunk of every wave's tile
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, kb = lane >> 4;
@@ -182,49 +182,46 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     }
   }
 
-  // ---- add the waves' tiles through LDS; wave w finishes registers [w*R/WAVES, (w+1)*R/WAVES)
-  // Register index r = (mt*4 + t)*NV + j; in the accumulator tile, lane (li, kb) register t of
-  // instruction j is channel strip*TN + (4*kb + t)*NV + j, token 16*mt + li.
+  // ---- add the waves' tiles through LDS, kChunk accumulator registers per pass; in each pass
+  // wave w finishes registers [w*RPW, (w+1)*RPW) of the chunk.  Register index
+  // r = (mt*4 + t)*NV + j; in the accumulator tile, lane (li, kb) register t of instruction j
+  // is channel strip*TN + (4*kb + t)*NV + j, token 16*mt + li.
+  constexpr int kChunk = 16;
+  constexpr int RPW = kChunk / WAVES;
+  static_assert(R % kChunk == 0 && kChunk % WAVES == 0 && NV % RPW == 0, "reduction split");
 #pragma unroll
-  for (int j = 0; j < NV; ++j)
+  for (int pass = 0; pass < R / kChunk; ++pass) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        float v = acc[j][mt][t];
-        if (MODE == kFactored && WBITS == 4) v *= 16.0f;  // undo value/16 (exact)
-        lds[(wave * R + (mt * 4 + t) * NV + j) * 64 + lane] = v;
-      }
-  __syncthreads();
-
-  constexpr int RPW = R / WAVES;  // registers finished per wave; divides NV or is a multiple of it
-  static_assert(R % WAVES == 0, "accumulators must split evenly over the waves");
-  static_assert(RPW >= NV ? RPW % NV == 0 : NV % RPW == 0, "finish chunks must align to channel runs");
-  constexpr int RUN = RPW < NV ? RPW : NV;  // consecutive channels finished together
-#pragma unroll
-  for (int c = 0; c < RPW / RUN; ++c) {
-    const int r0 = wave * RPW + c * RUN;
-    const int mt_t = r0 / NV, j0 = r0 % NV;
-    const int mt = mt_t / 4, t = mt_t % 4;
+    for (int c = 0; c < kChunk; ++c) {
+      const int r = pass * kChunk + c;
+      const int j = r % NV, mt = (r / NV) / 4, t = (r / NV) % 4;
+      float v = acc[j][mt][t];
+      if (MODE == kFactored && WBITS == 4) v *= 16.0f;  // undo value/16 (exact)
+      lds[(wave * kChunk + c) * 64 + lane] = v;
+    }
+    __syncthreads();
+    const int r0 = pass * kChunk + wave * RPW;  // first register this wave finishes
+    const int j0 = r0 % NV, mt = (r0 / NV) / 4, t = (r0 / NV) % 4;
     const int m = mt * 16 + li;
     const int n0 = strip * TN + (4 * kb + t) * NV + j0;
-    float sum[RUN];
+    float sum[RPW];
 #pragma unroll
-    for (int u = 0; u < RUN; ++u) {
+    for (int u = 0; u < RPW; ++u) {
       float s = 0.0f;
 #pragma unroll
-      for (int w2 = 0; w2 < WAVES; ++w2) s = s + lds[(w2 * R + r0 + u) * 64 + lane];
+      for (int w2 = 0; w2 < WAVES; ++w2) s = s + lds[(w2 * kChunk + wave * RPW + u) * 64 + lane];
       sum[u] = s;
     }
+    __syncthreads();
     if (m >= p.M || n0 >= p.N) continue;
     if (p.slices > 1) {
       float* dst = p.workspace + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
 #pragma unroll
-      for (int u = 0; u < RUN; ++u) dst[u] = sum[u];
+      for (int u = 0; u < RPW; ++u) dst[u] = sum[u];
     } else {
       uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n0;
 #pragma unroll
-      for (int u = 0; u < RUN; ++u) {
+      for (int u = 0; u < RPW; ++u) {
         float v = sum[u];
         if (MODE == kFactored)
           v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n0 + u,
@@ -287,19 +284,9 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
 
 template <int WBITS, int VEC, int MT, int WAVES, int MODE>
 int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
-  constexpr int NV = VEC * 8 / WBITS;
-  constexpr int R = NV * 4 * MT;
-  const size_t lds_bytes = (size_t)WAVES * R * 64 * sizeof(float);
   auto kern = dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE>;
-  if (lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes);
-    if (e != hipSuccess)
-      return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot: cannot reserve %zu bytes of LDS: %s",
-                  lds_bytes, hipGetErrorString(e));
-  }
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
-  hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds_bytes, stream, dp);
+  hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
   if (rc) return rc;
   if (dp.slices > 1) {
