@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference custom calls on one MI355X.
+
+A *step* is one pass of the decode hot path over the configuration-2 workload: the weight-only
+s4 group-128 dequantize-dot [M,8192] x [8192,28672] (+bias, SiLU) for M = 1, 8, 32 and 64, one
+custom call each, all through the library's XLA FFI handler symbols.  Inputs are synthetic, of
+the benchmark's shapes and distributions, and resident in HBM before the timed region.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-other] [--skip-cpu]
+
+Prints ONE JSON line: `value` = algorithmic bytes of a step / wall time per step (GB/s);
+`roofline` = the step's slowest kernel against the 8 TB/s HBM peak, timed with events on the
+launch stream; `cpu_baseline` = the CPU oracle on a column slice of the same workload;
+`kernels` / `other_configs` = every kernel of the step and the four other configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+HBM_PEAK_XLA_GBS = 6810.0      # what XLA's own device file assumes (mi350.txtpb:28)
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}
+K2, N2, GROUP2 = 8192, 28672, 128
+MS2 = (1, 8, 32, 64)
+
+
+def c2_bytes(m):
+    return K2 * N2 // 2 + (K2 // GROUP2) * N2 * 2 + N2 * 2 + m * K2 * 2 + m * N2 * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-other", action="store_true", help="only the headline workload")
+    ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
+    ap.add_argument("--reps", type=int, default=20, help="launches per event-timed batch")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (the path shards by output channels with no "
+                 "exchange step; see DESIGN.md); --gpus %d is not supported" % args.gpus)
+
+    import torch
+    from xla_amd import ffi, ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the kernels have no CPU fallback")
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+
+    def ev_time(fn, reps):
+        """Average device time of fn() over `reps` back-to-back launches, events on the stream."""
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = None
+        for _ in range(3):
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            e1.synchronize()
+            t = e0.elapsed_time(e1) / reps
+            best = t if best is None else min(best, t)
+        return best  # ms
+
+    # ---- configuration 2 on the device -------------------------------------------------------
+    w_packed = torch.randint(0, 256, (K2 * N2 // 2,), dtype=torch.uint8, device=dev)   # nibbles ~U{-8..7}
+    scales = torch.empty((K2 // GROUP2, N2), device=dev).uniform_(1e-3, 2e-2).to(torch.bfloat16)
+    bias = torch.randn((N2,), device=dev).to(torch.bfloat16)
+    calls = []
+    for m in MS2:
+        lhs = torch.randn((m, K2), device=dev).to(torch.bfloat16)
+        calls.append(ops.dequant_dot(lhs, w_packed, scales, bias, weight_dtype="s4", weight_shape=(K2, N2),
+                                     epilogue="BIAS_SILU", dequant_type="bf16", build_only=True))
+    for c in calls:
+        c.frame.host.stream = torch.cuda.current_stream().cuda_stream
+    step = ffi.Replay([(c.target, c.frame) for c in calls])
+
+    step.run(max(args.warmup, 1))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    step.run(args.steps)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    step_bytes = sum(c2_bytes(m) for m in MS2)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    kernels = []
+    for m, c in zip(MS2, calls):
+        one = ffi.Replay([(c.target, c.frame)])
+        ms = ev_time(lambda: one.run(1), args.reps)
+        c.run()
+        gbs = c2_bytes(m) / (ms * 1e-3) / 1e9
+        kernels.append({"workload": "C2 M=%d" % m, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
+                        "bytes": c2_bytes(m), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                        "TFLOP/s": round(2 * m * K2 * N2 / (ms * 1e-3) / 1e12, 2)})
+    dom = max(kernels, key=lambda k: k["ms"])
+    roofline = {"bound": "hbm", "kernel": dom["kernel"], "workload": dom["workload"],
+                "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
+                "frac_of_xla_device_file_peak": round(dom["GB/s"] / HBM_PEAK_XLA_GBS, 4),
+                "traffic": None, "launch_ms": dom["ms"], "algorithmic_bytes": dom["bytes"]}
+
+    # ---- the other four configurations (informational) -----------------------------------------
+    other = []
+    if not args.skip_other:
+        def entry(name, call, bytes_, flops, bound, dtype=None):
+            ms = ev_time(lambda: call.run(), max(3, args.reps // 4))
+            e = {"workload": name, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
+                 "GB/s": round(bytes_ / (ms * 1e-3) / 1e9, 1)}
+            e["frac_hbm"] = round(e["GB/s"] / HBM_PEAK_GBS, 4)
+            if flops:
+                e["TFLOP/s"] = round(flops / (ms * 1e-3) / 1e12, 2)
+                if dtype:
+                    e["frac_mfma"] = round(e["TFLOP/s"] / MFMA_PEAK_TFLOPS[dtype], 4)
+            e["bound"] = bound
+            other.append(e)
+
+        # C1: s8 per-channel decode
+        a = torch.randn((16, 4096), device=dev).to(torch.bfloat16)
+        w8 = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
+        sc = torch.empty((4096,), device=dev).uniform_(1e-3, 1e-2)
+        entry("C1 s8 [16,4096]x[4096,4096]", ops.dequant_dot(a, w8, sc, build_only=True),
+              4096 * 4096 + 2 * 16 * 4096 * 2 + 4096 * 4, 2 * 16 * 4096 * 4096, "hbm")
+        # C4: RMSNorm + rowwise fp8 quantize
+        x = torch.randn((16384, 8192), device=dev)
+        x = torch.where(torch.rand_like(x) < 0.01, x * 50, x).to(torch.bfloat16)
+        g = torch.empty((8192,), device=dev).uniform_(0.5, 1.5).to(torch.bfloat16)
+        entry("C4 rmsnorm+quantize [16384,8192]", ops.rowwise_quantize_fp8(x, g, build_only=True),
+              16384 * 8192 * 3 + 16384 * 4 + 8192 * 2, 0, "hbm")
+        del x
+        # C3: fp8 scaled dot + bias + GELU
+        a8 = (torch.randn((8192, 8192), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+        b8 = (torch.randn((8192, 8192), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+        s64 = torch.full((), 1 / 64, device=dev)
+        b3 = torch.randn((8192,), device=dev).to(torch.bfloat16)
+        entry("C3 fp8 [8192,8192]x[8192,8192] (rhs [K,N])",
+              ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", build_only=True),
+              2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+        entry("C3 fp8, rhs given as [N,K]",
+              ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", rhs_contracting_dim=1,
+                                 build_only=True),
+              2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+        del a8, b8
+        # C5: batched s8 per-channel prefill
+        a5 = torch.randn((8, 512, 4096), device=dev).to(torch.bfloat16)
+        w5 = torch.randint(-127, 128, (8, 4096, 14336), dtype=torch.int8, device=dev)
+        s5 = torch.empty((8, 14336), device=dev).uniform_(1e-3, 1e-2)
+        entry("C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, build_only=True),
+              8 * (4096 * 14336 + 512 * 4096 * 2 + 14336 * 4 + 512 * 14336 * 2),
+              2 * 8 * 512 * 4096 * 14336, "mfma", "bf16")
+        del a5, w5
+
+    # ---- CPU baseline: the oracle on a column slice of the same workload -------------------------
+    cpu = None
+    if not args.skip_cpu:
+        import numpy as np
+        from oracle import oracle
+        from xla_amd import workloads
+        ncols = 2048
+        t_cpu, b_cpu = 0.0, 0
+        for m in MS2:
+            wl = workloads.c2_s4_group(M=m, K=K2, N=ncols)
+            t1 = time.perf_counter()
+            oracle.dequant_dot(wl["lhs"], wl["weights_packed"], 4, wl["scales"], "bf16", "bf16",
+                               bias=wl["bias"], group=GROUP2, epilogue="silu")
+            t_cpu += time.perf_counter() - t1
+            b_cpu += wl["algorithmic_bytes"]
+        cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(),
+               "kind": "port",
+               "sample": "C2 at M=1,8,32,64 on the first %d of %d output channels (full K), %.2f s of "
+                         "CPU time; scalar restatement of the XLA CPU backend's op-by-op semantics, "
+                         "OpenMP over output channels" % (ncols, N2, t_cpu)}
+
+    out = {
+        "metric": "quant-dot HBM GB/s on the s4 group-128 decode dequantize-dot (% of MI355X roofline) "
+                  "next to the XLA-CPU-semantics oracle",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C2: bf16 [M,8192] x s4 [8192,28672] group-128 bf16 scales + bias + SiLU, "
+                               "M in {1,8,32,64}, one custom call per M per step",
+                   "boundary": "XLA FFI handler xla_amd_dequant_dot via native call-frame replay"},
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "other_configs": other,
+        "frac_of_hbm_peak_whole_step": round(value / HBM_PEAK_GBS, 4),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

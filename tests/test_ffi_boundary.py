@@ -182,3 +182,19 @@ def test_restated_abi_matches_xla_header(tmp_path):
     mine = _probe(tmp_path, os.path.join(ROOT, "include", "xla_ffi_abi.h"), "mine")
     theirs = _probe(tmp_path, "/root/reference/xla/ffi/api/c_api.h", "theirs")
     assert mine == theirs
+
+
+def test_native_host_registry_and_errors():
+    """The C++ function table: registration by (target, platform), lookup, error ownership."""
+    host = ffi.NativeHost()
+    host.register()
+    for target, sym in ffi.HANDLER_SYMBOLS.items():
+        fn = host.find_handler(target, "rocm")
+        assert fn == C.cast(getattr(ffi.library(), sym), C.c_void_p).value
+        assert host.find_handler(target, "cuda") is None
+    fr = quant_frame(host, g_dims=(8, 8))
+    with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 1 but got 2"):
+        ffi.invoke("xla_amd.rowwise_quantize_fp8", fr)
+    rp = ffi.Replay([("xla_amd.rowwise_quantize_fp8", quant_frame(host, n_rets=1))])
+    with pytest.raises(ffi.FfiError, match="call 0: .*Wrong number of results"):
+        rp.run(3)

@@ -182,6 +182,51 @@ class Host:
     def take_error(self, handle):
         return self.errors.pop(handle)
 
+    def api_address(self):
+        return C.addressof(self.api)
+
+    def ctx(self):
+        return 0xC0FFEE
+
+
+class NativeHost:
+    """The same services implemented in C++ (libxla_amd_host.so): no Python runs between a
+    handler and its function table, so replays are not slowed down by callbacks."""
+
+    def __init__(self, stream=0):
+        L = host_library()
+        self._h = L.xla_amd_host_create()
+        self.stream = stream
+
+    @property
+    def stream(self):
+        return self._stream
+
+    @stream.setter
+    def stream(self, value):
+        self._stream = value
+        host_library().xla_amd_host_set_stream(self._h, value)
+
+    def api_address(self):
+        return host_library().xla_amd_host_api(self._h)
+
+    def ctx(self):
+        return self._h
+
+    def take_error(self, handle):
+        buf = C.create_string_buffer(4096)
+        code = host_library().xla_amd_host_take_error(handle, buf, len(buf))
+        return code, buf.value.decode()
+
+    def register(self, register_symbol="xla_amd_register_handlers"):
+        fn = C.cast(getattr(library(), register_symbol), C.c_void_p)
+        err = host_library().xla_amd_host_register(self._h, fn)
+        if err:
+            raise FfiError(*self.take_error(err))
+
+    def find_handler(self, target, platform="rocm"):
+        return host_library().xla_amd_host_find_handler(self._h, target.encode(), platform.encode())
+
 
 _lib = None
 
@@ -248,8 +293,8 @@ class Frame:
         keep = self._keep = []
         f = self.frame = CallFrame()
         f.struct_size = CALL_FRAME_STRUCT_SIZE
-        f.api = C.addressof(host.api)
-        f.ctx = 0xC0FFEE
+        f.api = host.api_address()
+        f.ctx = host.ctx()
         f.stage = stage
 
         def fill(side, items):
@@ -314,6 +359,56 @@ def invoke(target, frame):
     if err:
         code, msg = frame.host.take_error(err)
         raise FfiError(code, msg)
+
+
+HOST_LIB_PATH = os.path.join(_LIB_DIR, "libxla_amd_host.so")
+_host_lib = None
+
+
+def host_library():
+    """The host-only helper library (frame replay, HLO rewrite pass); no GPU code inside."""
+    global _host_lib
+    if _host_lib is None:
+        if not os.path.exists(HOST_LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m xla_amd.build host`" % HOST_LIB_PATH)
+        L = C.CDLL(HOST_LIB_PATH)
+        L.xla_amd_host_replay.restype = C.c_void_p
+        L.xla_amd_host_replay.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                          C.POINTER(C.c_int64)]
+        L.xla_amd_host_create.restype = C.c_void_p
+        L.xla_amd_host_destroy.argtypes = [C.c_void_p]
+        L.xla_amd_host_api.restype = C.c_void_p
+        L.xla_amd_host_api.argtypes = [C.c_void_p]
+        L.xla_amd_host_set_stream.argtypes = [C.c_void_p, C.c_void_p]
+        L.xla_amd_host_take_error.restype = C.c_int
+        L.xla_amd_host_take_error.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
+        L.xla_amd_host_register.restype = C.c_void_p
+        L.xla_amd_host_register.argtypes = [C.c_void_p, C.c_void_p]
+        L.xla_amd_host_find_handler.restype = C.c_void_p
+        L.xla_amd_host_find_handler.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
+        _host_lib = L
+    return _host_lib
+
+
+class Replay:
+    """A fixed sequence of (target, Frame) pairs that is re-invoked from native code, like the
+    custom-call thunks of a compiled executable being run step after step."""
+
+    def __init__(self, calls):
+        self.calls = list(calls)
+        n = len(self.calls)
+        lib = library()
+        self._handlers = (C.c_void_p * n)(*[C.cast(getattr(lib, HANDLER_SYMBOLS[t]), C.c_void_p).value
+                                            for t, _ in self.calls])
+        self._frames = (C.c_void_p * n)(*[f.address() for _, f in self.calls])
+
+    def run(self, rounds=1):
+        failed = C.c_int64(-1)
+        err = host_library().xla_amd_host_replay(self._handlers, self._frames, len(self.calls), rounds,
+                                                 C.byref(failed))
+        if err:
+            code, msg = self.calls[0][1].host.take_error(err)
+            raise FfiError(code, "call %d: %s" % (failed.value, msg))
 
 
 def query_metadata(target, host):

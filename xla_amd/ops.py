@@ -15,9 +15,10 @@ _host = None
 
 
 def host():
+    """The process-wide FFI host (function table in C++)."""
     global _host
     if _host is None:
-        _host = ffi.Host()
+        _host = ffi.NativeHost()
     return _host
 
 
@@ -36,13 +37,27 @@ _NAMES = {dtypes.F32: "f32", dtypes.BF16: "bf16"}
 _TYPE_ATTR = {"f32": dtypes.F32, "bf16": dtypes.BF16}
 
 
+class Call:
+    """A prepared custom call: the call frame, its result tensors, and references that keep every
+    operand alive.  ``run()`` invokes it on torch's current stream; ``build_only=True`` on the
+    functions below returns the Call so that ffi.Replay can re-invoke it natively."""
+
+    def __init__(self, target, frame, result, keep=()):
+        self.target, self.frame, self.result, self._keep = target, frame, result, keep
+
+    def run(self):
+        self.frame.host.stream = _stream()
+        ffi.invoke(self.target, self.frame)
+        return self.result
+
+
 def _scratch(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device) if nbytes else None
 
 
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
-                out=None, scratch="auto"):
+                out=None, scratch="auto", build_only=False):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K]."""
     _check_cuda(lhs, weights, scales, bias)
     wdt = dtypes.S4 if weight_dtype == "s4" else dtypes.S8
@@ -65,14 +80,14 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     attrs = {"epilogue": ffi.Attr.str(epilogue), "dequant_type": ffi.Attr.i32(_TYPE_ATTR[dequant_type]),
              "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
              "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type])}
-    h = host()
-    h.stream = _stream()
-    ffi.invoke("xla_amd.dequant_dot", ffi.Frame(h, args, rets, attrs))
-    return out
+    call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
+                keep=(lhs, weights, scales, bias, scratch))
+    return call if build_only else call.run()
 
 
 def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, epilogue="DEFAULT",
-                   dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto"):
+                   dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto",
+                   build_only=False):
     """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K]; scales f32 []."""
     _check_cuda(a, b, a_scale, b_scale, bias)
     m, k = a.shape
@@ -93,13 +108,12 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
              "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
              "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type]),
              "rhs_contracting_dim": ffi.Attr.i64(rhs_contracting_dim)}
-    h = host()
-    h.stream = _stream()
-    ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(h, args, rets, attrs))
-    return out
+    call = Call("xla_amd.fp8_scaled_dot", ffi.Frame(host(), args, rets, attrs), out,
+                keep=(a, b, a_scale, b_scale, bias, scratch))
+    return call if build_only else call.run()
 
 
-def rowwise_quantize_fp8(x, gamma=None, *, eps=1e-6, q=None, scales=None):
+def rowwise_quantize_fp8(x, gamma=None, *, eps=1e-6, q=None, scales=None, build_only=False):
     """(q, scales) = per-row dynamic f8e4m3fn quantisation of x (bf16 [R,C]), after RMSNorm with
     ``gamma`` when given.  q is returned as uint8 codes."""
     _check_cuda(x, gamma)
@@ -113,7 +127,6 @@ def rowwise_quantize_fp8(x, gamma=None, *, eps=1e-6, q=None, scales=None):
         args.append((dtypes.BF16, gamma.data_ptr(), gamma.shape))
     rets = [(dtypes.F8E4M3FN, q.data_ptr(), [r, c]), (dtypes.F32, scales.data_ptr(), [r])]
     attrs = {"rmsnorm": ffi.Attr.pred(gamma is not None), "eps": ffi.Attr.f32(eps)}
-    h = host()
-    h.stream = _stream()
-    ffi.invoke("xla_amd.rowwise_quantize_fp8", ffi.Frame(h, args, rets, attrs))
-    return q, scales
+    call = Call("xla_amd.rowwise_quantize_fp8", ffi.Frame(host(), args, rets, attrs), (q, scales),
+                keep=(x, gamma))
+    return call if build_only else call.run()
