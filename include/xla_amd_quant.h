@@ -181,7 +181,7 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
 
 /* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
  * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, 3 tiled),
- * "dequant_dot_vec", "dequant_dot_slices", "fp8_dot_kernel" (1 exact, 2 tiled),
+ * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "fp8_dot_kernel" (1 exact, 2 tiled),
  * "quantize_variant".  Returns 0, or -1 for an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
 

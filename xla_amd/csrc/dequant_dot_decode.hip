@@ -59,18 +59,49 @@ __device__ __forceinline__ float s4_to_f32_div16(uint32_t v) {
   return __builtin_amdgcn_cvt_off_f32_i4((int)v);
 }
 
-// WBITS: 4 or 8.  VEC: bytes a lane reads per row (4, 8, 16).  MT: 16-token
-// tiles.  WAVES: waves per workgroup, splitting the workgroup's rows.
-template <int WBITS, int VEC, int MT, int WAVES, int MODE>
+// Buffer descriptor over [base, base+bytes): loads through it return 0 past the end, which is
+// how rows beyond K and tokens beyond M drop out of the main loop without any branch.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// N32 consecutive dwords (1, 2 or a multiple of 4) at voff + soff (soff wave-uniform).
+template <int N32>
+__device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff,
+                                                  uint32_t* dst) {
+  if constexpr (N32 >= 4) {
+#pragma unroll
+    for (int q = 0; q < N32 / 4; ++q) {
+      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff + 16 * q, soff, 0);
+      dst[4 * q] = v[0]; dst[4 * q + 1] = v[1]; dst[4 * q + 2] = v[2]; dst[4 * q + 3] = v[3];
+    }
+  } else if constexpr (N32 == 2) {
+    uintx2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    dst[0] = v[0]; dst[1] = v[1];
+  } else {
+    dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+  }
+}
+
+// WBITS: 4 or 8.  VEC: bytes a lane reads per row (4, 8, 16).  MT: 16-token tiles.  WAVES: waves
+// per workgroup, splitting the workgroup's rows.  SCALE_BF16: element type of the scales.
+// GROUP32: the scale group size is a multiple of 32, so the 32 rows of a step share one group
+// and the scales are reloaded only when a step starts a new group.
+//
+// The main loop has no per-lane control flow and no per-lane address arithmetic: every load is
+// a buffer load whose lane offset is fixed for the whole kernel and whose row offset is a scalar.
+template <int WBITS, int VEC, int MT, int WAVES, int MODE, bool SCALE_BF16, bool GROUP32>
 __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodeParams p) {
   constexpr int NV = VEC * 8 / WBITS;   // channels per lane
   constexpr int WORDS = VEC / 4;        // dwords per lane per row
   constexpr int NPW = 32 / WBITS;       // channels per dword
   constexpr int R = NV * 4 * MT;        // accumulator registers per lane
   constexpr int TN = 16 * NV;           // channels per wave tile
+  constexpr int SSZ = SCALE_BF16 ? 2 : 4;
   __shared__ float lds[WAVES * 16 * 64];  // one 16-register chunk of every wave's tile
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, in an SGPR
   const int li = lane & 15, kb = lane >> 4;
   // Consecutive workgroup ids land on different XCDs (round robin over 8); give each XCD a
   // contiguous range of strips so neighbouring strips, which share cache lines, share an L2.
@@ -83,10 +114,19 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   const int strip = bid / p.slices;
   const int batch = blockIdx.y;
 
-  const int n_lane = strip * TN + li * NV;
-  const bool n_ok = n_lane < p.N;  // N % NV == 0: a chunk is all in or all out
-  const size_t wbase = (size_t)batch * p.K * p.N;
-  const uint16_t* lhs = p.lhs + (size_t)batch * p.M * p.K;
+  const int n_lane = strip * TN + li * NV;   // first channel of this lane (may be >= N: discarded)
+  const uint32_t pitch = (uint32_t)(((size_t)p.N * WBITS) >> 3);  // bytes per row of W
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.w + (size_t)batch * p.K * pitch, (uint32_t)p.K * pitch);
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.lhs + (size_t)batch * p.M * p.K, (uint32_t)p.M * p.K * 2u);
+  const int groups = p.K / p.group;
+  const __amdgpu_buffer_rsrc_t rs =
+      make_rsrc((const char*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N * SSZ,
+                (uint32_t)groups * p.N * SSZ);
+  const uint32_t voff_w = (uint32_t)(8 * kb) * pitch + (uint32_t)((n_lane * WBITS) >> 3);
+  uint32_t voff_a[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) voff_a[mt] = ((uint32_t)(mt * 16 + li) * p.K + 8 * kb) * 2u;
+  const uint32_t voff_s = (uint32_t)n_lane * SSZ;
 
   floatx4 acc[NV][MT];
 #pragma unroll
@@ -94,71 +134,75 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int rows_per_wave = p.rows_per_slice / WAVES;  // multiple of 32
+  const int rows_per_wave = p.rows_per_slice / WAVES;  // multiple of 64
   const int k_begin = slice * p.rows_per_slice + wave * rows_per_wave;
-  const int k_end = min(k_begin + rows_per_wave, p.K);
+  const int k_stop = k_begin + rows_per_wave;           // may run past K: those rows load zeros
 
-  float sc[NV];       // kRounded: scale (x16 for s4) of each owned channel, for the current group
-  int g_cur = -1;
-
-  uint32_t wq[2][8][WORDS];
-  auto load_rows = [&](int buf, int k0) {
-    const int krow = k0 + 8 * kb;
+  float sc[NV];  // kRounded: scale (x16 for s4) of each owned channel, for the current group
+  auto load_scales = [&](int k0) {
+    uint32_t raw[NV * SSZ / 4];
+    if (GROUP32) {
+      const uint32_t g = (uint32_t)min(k0, p.K - 1) / (uint32_t)p.group;  // scalar
+      buffer_load_words<NV * SSZ / 4>(rs, voff_s, g * (uint32_t)p.N * SSZ, raw);
+    } else {
+      const uint32_t g = (uint32_t)min(k0 + 8 * kb, p.K - 1) / (uint32_t)p.group;  // per lane
+      buffer_load_words<NV * SSZ / 4>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, raw);
+    }
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const bool ok = n_ok && (krow + r) < k_end;
-      const size_t e = wbase + (size_t)(krow + r) * p.N + n_lane;  // element index
-      const uint8_t* src = p.w + (e * WBITS >> 3);
-      if (WORDS == 4) {
-        uintx4 v = ok ? *reinterpret_cast<const uintx4*>(src) : uintx4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) wq[buf][r][q] = v[q];
-      } else if (WORDS == 2) {
-        uintx2 v = ok ? *reinterpret_cast<const uintx2*>(src) : uintx2{0u, 0u};
-        wq[buf][r][0] = v[0];
-        wq[buf][r][WORDS - 1] = v[1];
-      } else {
-        wq[buf][r][0] = ok ? *reinterpret_cast<const uint32_t*>(src) : 0u;
-      }
+    for (int j = 0; j < NV; ++j) {
+      float v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
+                           : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
+      sc[j] = WBITS == 4 ? v * 16.0f : v;  // the s4 convert yields value/16
     }
   };
 
+  uint32_t wq[2][8][WORDS];
+  auto load_rows = [&](int buf, int k0) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      buffer_load_words<WORDS>(rw, voff_w, (uint32_t)(k0 + r) * pitch, wq[buf][r]);
+  };
+
   auto compute = [&](int buf, int k0) {
-    const int krow = k0 + 8 * kb;
-    // activations: 8 consecutive k of token (16*mt + li)
+    // activations: 8 consecutive k of token (16*mt + li); tokens >= M read past the buffer -> 0
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const int m = mt * 16 + li;
-      uintx4 v = {0u, 0u, 0u, 0u};
-      if (m < p.M && krow < k_end) v = *reinterpret_cast<const uintx4*>(lhs + (size_t)m * p.K + krow);
+      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt], (uint32_t)k0 * 2u, 0);
+      if (k0 + 32 > p.K) {  // scalar condition: only a step that crosses the end of K
+        const bool ok = k0 + 8 * kb < p.K;
+        v = uintx4{ok ? v[0] : 0u, ok ? v[1] : 0u, ok ? v[2] : 0u, ok ? v[3] : 0u};
+      }
       bop[mt] = __builtin_bit_cast(bf16x8, v);
     }
     if (MODE == kRounded) {
-      const int g = krow / p.group;
-      if (g != g_cur && krow < k_end) {
-        g_cur = g;
-        const size_t sb = ((size_t)(p.scale_batched ? batch : 0) * (p.K / p.group) + g) * p.N + n_lane;
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-          float s = n_ok ? load_scale(p.scales, sb + j, p.scale_is_bf16) : 0.0f;
-          sc[j] = WBITS == 4 ? s * 16.0f : s;  // the s4 convert yields value/16
-        }
+      if (GROUP32) {
+        if (k0 % p.group == 0 || k0 == k_begin) load_scales(k0);  // scalar condition
+      } else {
+        load_scales(k0);
       }
     }
 #pragma unroll
     for (int q = 0; q < WORDS; ++q) {
+      // s4: one shift exposes the odd nibbles; byte selects then come for free with the convert
+      uint32_t lo[8], hi[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        lo[r] = wq[buf][r][q];
+        hi[r] = lo[r] >> 4;
+        if (WBITS == 4) asm volatile("" : "+v"(hi[r]));  // keep it one shift, not one per nibble
+      }
 #pragma unroll
       for (int e = 0; e < NPW; ++e) {
         const int j = q * NPW + e;
         float f[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-          const uint32_t word = wq[buf][r][q];
           if (WBITS == 4) {
-            f[r] = s4_to_f32_div16(word >> (4 * e));
+            const uint32_t src = (e & 1) ? hi[r] : lo[r];
+            f[r] = s4_to_f32_div16((src >> (8 * (e >> 1))) & 0xffu);
           } else {
-            f[r] = (float)(int8_t)((word >> (8 * e)) & 0xffu);
+            f[r] = (float)(int8_t)((lo[r] >> (8 * e)) & 0xffu);
           }
           if (MODE == kRounded) f[r] = f[r] * sc[j];
         }
@@ -172,9 +216,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     }
   };
 
-  if (k_begin < k_end) {
+  if (k_begin < p.K) {
     load_rows(0, k_begin);
-    for (int k0 = k_begin; k0 < k_end; k0 += 64) {
+    for (int k0 = k_begin; k0 < k_stop; k0 += 64) {
       load_rows(1, k0 + 32);
       compute(0, k0);
       load_rows(0, k0 + 64);
@@ -284,7 +328,16 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
 
 template <int WBITS, int VEC, int MT, int WAVES, int MODE>
 int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
-  auto kern = dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE>;
+  void (*kern)(DecodeParams) = nullptr;
+  const bool g32 = dp.group % 32 == 0;
+  if constexpr (MODE == kFactored)  // the main loop never touches the scales
+    kern = dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, true>;
+  else if (dp.scale_is_bf16)
+    kern = g32 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, true>
+               : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, false>;
+  else
+    kern = g32 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, true>
+               : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, false>;
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
   hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
@@ -302,9 +355,9 @@ int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const c
 
 int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream);  // dequant_dot_mfma.hip
 
-// Rows of K each workgroup takes so that `slices` workgroups cover K; multiple of 32*waves.
+// Rows of K each workgroup takes so that `slices` workgroups cover K; multiple of 64*waves.
 static int RowsPerSlice(int K, int slices, int waves) {
-  const int unit = 32 * waves;
+  const int unit = 64 * waves;
   const int per = (K + slices - 1) / slices;
   return (per + unit - 1) / unit * unit;
 }
@@ -375,22 +428,31 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
   if (force != 1 && force != 3 && aligned && mode_ok && p.M <= 64 && p.K >= 32) {
     // VEC bytes per lane per row -> NV channels per lane; needs N % NV == 0 and 16-byte rows
     const int mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
-    int vec = mt == 1 ? (s4 ? 8 : 16) : mt == 2 ? (s4 ? 4 : 8) : 4;
+    // Narrow strips (4 bytes of s4 = 8 channels, 8 bytes of s8 per lane) measured fastest on
+    // MI355X: the loop is bound by the dequantising VALU work, not by load width, and narrow
+    // strips give more workgroups to spread over the 256 CUs.
+    int vec = s4 ? 4 : (mt == 4 ? 4 : 8);
     if (int v = GetOption("dequant_dot_vec")) vec = v;
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
+    // buffer offsets are 32-bit: keep every operand (plus one loop overrun) below 2 GiB
+    const bool fits32 = (double)p.K * row_bytes + 128.0 * row_bytes < 2147483648.0 &&
+                        (double)p.M * p.K * 2 < 2147483648.0 &&
+                        (double)(p.K / p.group) * p.N * 4 < 2147483648.0;
     const bool shape_ok = p.N % nv == 0 && row_bytes % vec == 0 && nv * mt <= 32 &&
-                          (vec == 4 || vec == 8 || vec == 16) && (s4 || nv * mt <= 16 || true);
+                          (vec == 4 || vec == 8 || vec == 16) && fits32;
     if (shape_ok) {
-      const int waves = 8;
+      int waves = 8;
+      if (int wv = GetOption("dequant_dot_waves")) waves = wv == 4 ? 4 : 8;
       dp.strips = (int)((p.N + 16 * nv - 1) / (16 * nv));
       // enough workgroups for ~2 per CU, but never slices that leave a wave without rows
       int slices = 1;
       if (int s = GetOption("dequant_dot_slices")) {
         slices = s;
       } else {
-        while (dp.strips * slices * p.batch < 384 && p.K / (slices * 2) >= 32 * waves &&
-               slices * 2 * p.M <= 64)
+        const int want = p.M <= 8 ? 768 : 384;  // workgroups; partial sums cost slices*M*N*4 bytes
+        while (dp.strips * slices * p.batch < want && p.K / (slices * 2) >= 64 * waves &&
+               slices * 2 * p.M <= 32)
           slices *= 2;
       }
       if (slices > 1 && (!p.workspace ||
@@ -400,7 +462,8 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
       dp.rows_per_slice = RowsPerSlice(dp.K, slices, waves);
 #define XLA_AMD_DECODE(WB, V, MT_, MODE_, NAME)                                       \
   if ((s4 ? 4 : 8) == WB && vec == V && mt == MT_ && mode == MODE_)                   \
-    return launch_decode<WB, V, MT_, 8, MODE_>(dp, (int)p.batch, stream, NAME);
+    return waves == 4 ? launch_decode<WB, V, MT_, 4, MODE_>(dp, (int)p.batch, stream, NAME) \
+                      : launch_decode<WB, V, MT_, 8, MODE_>(dp, (int)p.batch, stream, NAME);
       XLA_AMD_DECODE(4, 16, 1, kRounded, "dequant_dot_decode_s4_v16_m16_rounded")
       XLA_AMD_DECODE(4, 8, 1, kRounded, "dequant_dot_decode_s4_v8_m16_rounded")
       XLA_AMD_DECODE(4, 4, 1, kRounded, "dequant_dot_decode_s4_v4_m16_rounded")
