@@ -1,0 +1,102 @@
+"""End to end on the GPU: the benchmark HLO modules go through the rewrite pass, the rewritten
+module runs through the FFI registry (xla_amd/hlo_runner.py), and the result is compared with
+the op-by-op CPU evaluation of the *original* module -- what run_hlo_module does with
+--reference_platform (xla/tools/run_hlo_module.cc:211-390)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hlo_eval
+from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_s8, dev_u8, dot_floor, host_bf16
+from xla_amd import dtypes, hlo, hlo_modules as hm, hlo_runner, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def reference(text, args):
+    return hlo_eval.evaluate(hlo.to_json(text), args)
+
+
+def test_c1_module():
+    say("module C1")
+    M, K, N = 16, 512, 256
+    w = workloads.c1_s8_channel(M, K, N)
+    text = hm.c1_s8_channel(M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_s8(w["weights"]), dev_f32(w["scales"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8]"]
+    ref = reference(text, [w["lhs"], w["weights"], w["scales"]])
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)),
+                   np.abs(w["weights"].astype(np.float64)) * w["scales"].astype(np.float64)[None, :], K)
+    check_dot(host_bf16(out), ref, fl, "C1 module")
+
+
+def test_c2_module():
+    say("module C2")
+    M, K, N = 8, 1024, 512
+    w = workloads.c2_s4_group(M, K, N)
+    text = hm.c2_s4_group(M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_u8(w["weights_packed"]),
+                                                   dev_bf16(w["scales"]), dev_bf16(w["bias"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"]
+    ref = reference(text, [w["lhs"], w["weights"], w["scales"], w["bias"]])
+    wd = np.abs(w["weights"].astype(np.float64)) * np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=0)
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+    check_dot(host_bf16(out), ref, fl, "C2 module")
+
+
+def test_c3_module():
+    say("module C3")
+    M, K, N = 128, 256, 128
+    w = workloads.c3_fp8(M, K, N)
+    text = hm.c3_fp8(M, K, N)
+    s = np.array(1 / 64, np.float32)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(w["a"]), dev_u8(w["b"]), dev_f32(s), dev_f32(s), dev_bf16(w["bias"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"]
+    ref = reference(text, [w["a"], w["b"], s, s, w["bias"]])
+    fa = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) / 64
+    fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) / 64
+    check_dot(host_bf16(out), ref, dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "C3 module")
+
+
+@pytest.mark.parametrize("rmsnorm", [True, False])
+def test_c4_module_bit_exact(rmsnorm):
+    say("module C4 rmsnorm=%s" % rmsnorm)
+    rows, cols = 24, 2048
+    w = workloads.c4_quantize(rows, cols)
+    text = hm.c4_quantize(rows, cols, rmsnorm=rmsnorm)
+    args_dev = [dev_bf16(w["x"])] + ([dev_bf16(w["gamma"])] if rmsnorm else [])
+    (q, s), rw, _ = hlo_runner.compile_and_run(text, args_dev)
+    torch.cuda.synchronize()
+    assert len(rw) == 1 and "rowwise_quantize_fp8" in rw[0]
+    q_ref, s_ref = reference(text, [w["x"]] + ([w["gamma"]] if rmsnorm else []))
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def test_c5_module():
+    say("module C5")
+    B, M, K, N = 2, 128, 256, 256
+    w = workloads.c5_s8_batched(B, M, K, N)
+    text = hm.c5_s8_batched(B, M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_s8(w["weights"]), dev_f32(w["scales"])])
+    torch.cuda.synchronize()
+    ref = reference(text, [w["lhs"], w["weights"], w["scales"]])
+    wd = np.abs(w["weights"].astype(np.float64)) * w["scales"].astype(np.float64)[:, None, :]
+    check_dot(host_bf16(out), ref, dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K), "C5 module")
+
+
+def test_unrewritten_module_does_not_run():
+    say("module with nothing to rewrite")
+    text = "HloModule m\nENTRY e {\n  a = f32[4] parameter(0)\n  ROOT b = f32[4] add(a, a)\n}\n"
+    with pytest.raises(NotImplementedError, match="was not rewritten into a custom call"):
+        hlo_runner.compile_and_run(text, [torch.zeros(4, device="cuda")])

@@ -1,0 +1,56 @@
+"""The fused C oracle functions against an op-by-op evaluation of the benchmark HLO modules
+(oracle/hlo_eval.py: one numpy op per HLO instruction, re-rounded to the instruction's type).
+Both add in the same order, so the comparison is bit for bit: it shows the fused restatement
+computes exactly what the un-fused module means under the CPU backend's rounding rules."""
+import numpy as np
+import pytest
+
+from oracle import hlo_eval
+from xla_amd import dtypes, hlo, hlo_modules as hm, workloads
+
+
+def run_module(text, args):
+    return hlo_eval.evaluate(hlo.to_json(text), args)
+
+
+def test_c1(oracle):
+    w = workloads.c1_s8_channel(M=5, K=96, N=40)
+    got = run_module(hm.c1_s8_channel(5, 96, 40), [w["lhs"], w["weights"], w["scales"]])
+    ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("M", [1, 3])
+def test_c2(oracle, M):
+    w = workloads.c2_s4_group(M=M, K=256, N=48, group=64)
+    got = run_module(hm.c2_s4_group(M, 256, 48, 64), [w["lhs"], w["weights"], w["scales"], w["bias"]])
+    ref = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", bias=w["bias"],
+                             group=64, epilogue="silu")
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("typed", ["f32", "bf16"])
+def test_c3(oracle, typed):
+    w = workloads.c3_fp8(12, 64, 20)
+    sa = np.float32(1 / 64)
+    scal = dtypes.f32_to_bf16(np.array([sa])) if typed == "bf16" else np.array([sa], np.float32)
+    got = run_module(hm.c3_fp8(12, 64, 20, typed=typed), [w["a"], w["b"], scal[0:1].reshape(()), scal[0:1].reshape(()), w["bias"]])
+    ref = oracle.fp8_scaled_dot(w["a"], w["b"], sa, sa, mul_ty=typed, bias=w["bias"], dot_ty=typed, ep_ty=typed,
+                                epilogue="gelu_tanh")
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 256), (3, 1000), (2, 33)])
+def test_c4(oracle, rows, cols):
+    w = workloads.c4_quantize(rows, cols)
+    q, s = run_module(hm.c4_quantize(rows, cols), [w["x"], w["gamma"]])
+    q_ref, s_ref = oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6)
+    assert np.array_equal(s.view(np.uint32), s_ref.view(np.uint32))
+    assert np.array_equal(q, q_ref)
+
+
+def test_c5(oracle):
+    w = workloads.c5_s8_batched(B=2, M=4, K=64, N=24)
+    got = run_module(hm.c5_s8_batched(2, 4, 64, 24), [w["lhs"], w["weights"], w["scales"]])
+    ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
+    assert np.array_equal(got, ref)

@@ -1,0 +1,285 @@
+"""QuantFusionRewriter on HLO text, without a device: FileCheck-style checks on the printed
+module, in the manner of the reference's pass tests (gemm_rewriter_fp8_test.cc:137-158).
+Patterns are the five benchmark modules plus the shapes of the reference's own test HLO
+(gemm_rewriter_fp8_test.cc:469-519,1106-1203,1301+; fusion_emitter_int4_device_test.cc:85-449,
+698-716)."""
+import re
+
+import pytest
+
+from xla_amd import ffi, hlo, hlo_modules as hm
+
+
+def check(text, *patterns):
+    """Each pattern (regex) must match somewhere after the previous one -- FileCheck's CHECK."""
+    pos = 0
+    for p in patterns:
+        m = re.compile(p).search(text, pos)
+        assert m, "CHECK failed: %s\n--- module ---\n%s" % (p, text)
+        pos = m.end()
+
+
+def opcodes(text):
+    entry = next(c for c in hlo.to_json(text)["computations"] if c["entry"])
+    return [i["opcode"] for i in entry["instructions"]]
+
+
+def test_parser_round_trip_is_stable():
+    for text in (hm.c1_s8_channel(4, 32, 16), hm.c2_s4_group(2, 256, 64), hm.c3_fp8(16, 32, 16),
+                 hm.c4_quantize(4, 64), hm.c5_s8_batched(2, 8, 32, 16)):
+        once = hlo.print_module(text)
+        assert hlo.print_module(once) == once
+        j = hlo.to_json(text)
+        assert sum(c["entry"] for c in j["computations"]) == 1
+
+
+def test_parser_accepts_xla_printed_form():
+    text = """HloModule m, entry_computation_layout={(bf16[4,8]{1,0})->bf16[4,8]{1,0}}
+
+ENTRY %main.3 (p0: bf16[4,8]) -> bf16[4,8] {
+  %p0 = bf16[4,8]{1,0} parameter(0), metadata={op_name="x" source_file="a,b.py"}
+  %c = bf16[] constant(1) // trailing comment
+  %b = bf16[4,8]{1,0} broadcast(bf16[] %c), dimensions={}
+  ROOT %add.1 = bf16[4,8]{1,0} add(bf16[4,8]{1,0} %p0, bf16[4,8]{1,0} %b)
+}
+"""
+    j = hlo.to_json(text)
+    ins = j["computations"][0]["instructions"]
+    assert [i["name"] for i in ins] == ["p0", "c", "b", "add.1"]
+    assert ins[3]["operands"] == ["p0", "b"] and ins[3]["root"]
+    assert ins[0]["attrs"]["metadata"].startswith("{op_name=")
+    assert ins[0]["shape"] == {"dtype": "bf16", "dims": [4, 8], "layout": "1,0"}
+
+
+@pytest.mark.parametrize("bad,msg", [
+    ("HloModule m\nENTRY e {\n  a = f32[2] add(b, b)\n}\n", "not defined before its use"),
+    ("HloModule m\nENTRY e {\n  a = f32[2 parameter(0)\n}\n", "line 3"),
+    ("HloModule m\nENTRY e {\n  a = f32[2] parameter(0)\n  a = f32[2] parameter(1)\n}\n", "duplicate"),
+    ("HloModule m\n", "no computation"),
+])
+def test_parser_errors(bad, msg):
+    with pytest.raises(hlo.HloError, match=msg):
+        hlo.rewrite(bad)
+
+
+def test_c1_per_channel_s8():
+    new, rw, rf = hlo.rewrite(hm.c1_s8_channel())
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8]"] and rf == []
+    check(new, r"%lhs = bf16\[16,4096\] parameter\(0\)", r"%w = s8\[4096,4096\] parameter\(1\)",
+          r"\(bf16\[16,4096\]\{1,0\}, s8\[\d+\]\{0\}\) custom-call\(%lhs, %w, %scale\), "
+          r'custom_call_target="xla_amd.dequant_dot", api_version=API_VERSION_TYPED_FFI',
+          r'epilogue = \\"DEFAULT\\", dequant_type = 11 : i32, dot_type = 11 : i32, epilogue_type = 11 : i32',
+          r"ROOT %\S+ = bf16\[16,4096\]\{1,0\} get-tuple-element\(%\S+\), index=0")
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+
+
+def test_c2_grouped_s4_with_bias_silu():
+    new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=8))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
+    want_ws = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 28672, 21)
+    check(new, r"custom-call\(%lhs, %w, %scales, %bias\)",
+          r'epilogue = \\"BIAS_SILU\\", dequant_type = 16 : i32, dot_type = 11 : i32, epilogue_type = 11 : i32')
+    assert "s8[%d]{0})" % want_ws in new
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+    # x * logistic(x) is the same activation before LogisticExpander has run
+    text = hm.c2_s4_group(M=8)
+    text = re.sub(r"  %neg = .*\n  %exp = .*\n  %one = .*\n  %one_b = .*\n  %den = .*\n  %sig = f32(\[\d+,\d+\]) divide.*\n",
+                  r"  %sig = f32\1 logistic(%z)\n", text)
+    assert "logistic" in text
+    assert hlo.rewrite(text)[1] == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"]
+
+
+@pytest.mark.parametrize("typed,code", [("f32", 11), ("bf16", 16)])
+def test_c3_fp8_bias_gelu(typed, code):
+    new, rw, rf = hlo.rewrite(hm.c3_fp8(typed=typed))
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"] and rf == []
+    check(new, r"custom-call\(%a, %b, %a_scale\S*, %b_scale\S*, %bias\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
+          r'epilogue = \\"BIAS_GELU\\", dequant_type = %d : i32, dot_type = %d : i32, epilogue_type = %d : i32, '
+          r'rhs_contracting_dim = 0 : i64' % (code, code, code))
+    assert "s8[67108864]{0}" in new            # K*N bytes to re-lay the [K,N] rhs out with K minor
+    if typed == "bf16":                        # bf16 scalars are widened, as GemmRewriter does
+        check(new, r"%a_scale.f32 = f32\[\] convert\(%a_scale\)", r"%b_scale.f32 = f32\[\] convert\(%b_scale\)")
+
+
+def test_c4_quantize_rmsnorm_and_plain():
+    new, rw, rf = hlo.rewrite(hm.c4_quantize())
+    assert rw == ["q -> xla_amd.rowwise_quantize_fp8 [rmsnorm]"] and rf == []
+    check(new, r"\(f8e4m3fn\[16384,8192\]\{1,0\}, f32\[16384\]\{0\}\) custom-call\(%x, %gamma\)",
+          r'backend_config="\{rmsnorm = true, eps = 1e-06 : f32\}"',
+          r"ROOT %result = .* tuple\(%q.codes, %scale.scales\)")
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter", "tuple"]
+    new, rw, rf = hlo.rewrite(hm.c4_quantize(rmsnorm=False))
+    assert rw == ["q -> xla_amd.rowwise_quantize_fp8 [plain]"]
+    check(new, r"custom-call\(%x\)", r"rmsnorm = false")
+    # reduce-max seeded with 0 instead of -inf is the same amax of absolute values
+    assert hlo.rewrite(hm.c4_quantize(rmsnorm=False).replace("constant(-inf)", "constant(0)"))[1]
+
+
+def test_c5_batched_s8():
+    new, rw, rf = hlo.rewrite(hm.c5_s8_batched())
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8]"] and rf == []
+    check(new, r"bf16\[8,512,14336\]\{2,1,0\}", r"custom-call\(%lhs, %w, %scale\)")
+
+
+def test_rewrite_without_scratch_callbacks_has_single_result():
+    new, rw, _ = hlo.rewrite(hm.c1_s8_channel(), with_scratch=False)
+    check(new, r"ROOT %\S+ = bf16\[16,4096\]\{1,0\} custom-call\(%lhs, %w, %scale\)")
+
+
+FP8_HEAD = """HloModule test
+ENTRY test {
+  x = f8e4m3fn[16,32] parameter(0)
+  y = f8e4m3fn[32,16] parameter(1)
+  x_scale = f32[] parameter(2)
+  y_scale = f32[] parameter(3)
+"""
+
+
+def test_fp8_scaled_ab_relu_bf16_out():
+    text = FP8_HEAD + """  x_f32 = f32[16,32] convert(x)
+  y_f32 = f32[32,16] convert(y)
+  x_scale_bcast = f32[16,32] broadcast(x_scale), dimensions={}
+  y_scale_bcast = f32[32,16] broadcast(y_scale), dimensions={}
+  x_unscaled = f32[16,32] multiply(x_f32, x_scale_bcast)
+  y_unscaled = f32[32,16] multiply(y_f32, y_scale_bcast)
+  dot_a = f32[16,16] dot(x_unscaled, y_unscaled), lhs_contracting_dims={1}, rhs_contracting_dims={0}
+  c = f32[] constant(0)
+  c_bcast = f32[16,16] broadcast(c), dimensions={}
+  relu = f32[16,16] maximum(dot_a, c_bcast)
+  ROOT out = bf16[16,16] convert(relu)
+}
+"""
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot_a -> xla_amd.fp8_scaled_dot [RELU]"], (rw, rf)
+    check(new, r"custom-call\(%x, %y, %x_scale, %y_scale\)", r'epilogue = \\"RELU\\"')
+
+
+def test_fp8_f32_result_is_refused_with_reason():
+    """ScaledABUnscaledDF8 (gemm_rewriter_fp8_test.cc:469-519) leaves an f32 dot; the kernels
+    produce bf16, so the pass says so and leaves the module alone."""
+    text = FP8_HEAD + """  x_f32 = f32[16,32] convert(x)
+  y_f32 = f32[32,16] convert(y)
+  x_scale_bcast = f32[16,32] broadcast(x_scale), dimensions={}
+  y_scale_bcast = f32[32,16] broadcast(y_scale), dimensions={}
+  x_unscaled = f32[16,32] multiply(x_f32, x_scale_bcast)
+  y_unscaled = f32[32,16] multiply(y_f32, y_scale_bcast)
+  ROOT out = f32[16,16] dot(x_unscaled, y_unscaled), lhs_contracting_dims={1}, rhs_contracting_dims={0}
+}
+"""
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == [] and "custom-call" not in new
+    assert len(rf) == 1 and "is f32, the kernels produce bf16" in rf[0]
+
+
+def test_fp8_divide_by_scale_and_rhs_contracting_minor():
+    text = FP8_HEAD.replace("y = f8e4m3fn[32,16]", "y = f8e4m3fn[16,32]") + """  x_bf16 = bf16[16,32] convert(x)
+  y_bf16 = bf16[16,32] convert(y)
+  xs = bf16[] convert(x_scale)
+  ys = bf16[] convert(y_scale)
+  x_scale_bcast = bf16[16,32] broadcast(xs), dimensions={}
+  y_scale_bcast = bf16[16,32] broadcast(ys), dimensions={}
+  x_unscaled = bf16[16,32] divide(x_bf16, x_scale_bcast)
+  y_unscaled = bf16[16,32] multiply(y_scale_bcast, y_bf16)
+  ROOT out = bf16[16,16] dot(x_unscaled, y_unscaled), lhs_contracting_dims={1}, rhs_contracting_dims={1}
+}
+"""
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["out -> xla_amd.fp8_scaled_dot [DEFAULT]"], (rw, rf)
+    check(new, r"%\S+ = f32\[\] divide\(%one\S*, %\S+\)", r"rhs_contracting_dim = 1 : i64")
+    assert "s8[" not in new                      # K-minor rhs needs no scratch
+
+
+def test_unscaled_fp8_dot_gets_unit_scales():
+    text = """HloModule t
+ENTRY e {
+  x = f8e4m3fn[16,32] parameter(0)
+  y = f8e4m3fn[32,16] parameter(1)
+  xb = bf16[16,32] convert(x)
+  yb = bf16[32,16] convert(y)
+  ROOT d = bf16[16,16] dot(xb, yb), lhs_contracting_dims={1}, rhs_contracting_dims={0}
+}
+"""
+    new, rw, _ = hlo.rewrite(text)
+    assert rw == ["d -> xla_amd.fp8_scaled_dot [DEFAULT]"]
+    check(new, r"%one\S* = f32\[\]\S* constant\(1\)", r"custom-call\(%x, %y, %one\S*, %one\S*\)")
+
+
+def test_int4_channel_dequant_with_bias_from_reference_shape():
+    """Channel dequantisation of fusion_emitter_int4_device_test.cc:217-247, with the weights
+    as the dot's rhs [B,K,N]."""
+    text = """HloModule FuseChannelDequantization
+ENTRY main {
+  w.s4 = s4[32,128,256] parameter(0)
+  w.s8 = s8[32,128,256] convert(w.s4)
+  w.bf16 = bf16[32,128,256] convert(w.s8)
+  s = bf16[32,256] parameter(1)
+  s.broadcast.2 = bf16[32,128,256] broadcast(s), dimensions={0,2}
+  w.scaled = bf16[32,128,256] multiply(w.bf16, s.broadcast.2)
+  a = bf16[32,2,128] parameter(2)
+  ROOT dot = bf16[32,2,256] dot(a, w.scaled), lhs_batch_dims={0}, lhs_contracting_dims={2}, rhs_batch_dims={0}, rhs_contracting_dims={1}
+}
+"""
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s4]"], (rw, rf)
+    check(new, r"custom-call\(%a, %w.s4, %s\)", r"dequant_type = 16 : i32, dot_type = 16 : i32")
+
+
+def test_weights_on_the_lhs_and_minor_batch_dim_are_left_alone():
+    # weights as lhs (fusion_emitter_int4_device_test.cc:93-104 orientation): not this kernel's layout
+    text = """HloModule t
+ENTRY main {
+  w = s4[128,256] parameter(0)
+  w8 = s8[128,256] convert(w)
+  wb = bf16[128,256] convert(w8)
+  s = bf16[256] parameter(1)
+  sb = bf16[128,256] broadcast(s), dimensions={1}
+  ws = bf16[128,256] multiply(wb, sb)
+  a = bf16[128,4] parameter(2)
+  ROOT dot = bf16[256,4] dot(ws, a), lhs_contracting_dims={0}, rhs_contracting_dims={0}
+}
+"""
+    new, rw, _ = hlo.rewrite(text)
+    assert rw == [] and "custom-call" not in new
+    # RejectTritonFusionForWithMinorBatchDim (fusion_emitter_int4_device_test.cc:698-716)
+    text = """HloModule t
+ENTRY main {
+  lhs = s4[32,64,2] parameter(0)
+  lhs_converted = bf16[32,64,2] convert(lhs)
+  rhs = bf16[2,64,16] parameter(1)
+  ROOT dot = bf16[2,32,16] dot(lhs_converted, rhs), lhs_batch_dims={2}, lhs_contracting_dims={1}, rhs_batch_dims={0}, rhs_contracting_dims={1}
+}
+"""
+    assert hlo.rewrite(text)[1] == []
+    # weights as rhs but contracting their minor dimension: refused with the reason
+    text = """HloModule t
+ENTRY main {
+  a = bf16[4,128] parameter(0)
+  w = s8[256,128] parameter(1)
+  wf = bf16[256,128] convert(w)
+  s = bf16[256] parameter(2)
+  sb = bf16[256,128] broadcast(s), dimensions={0}
+  ws = bf16[256,128] multiply(wf, sb)
+  ROOT dot = bf16[4,256] dot(a, ws), lhs_contracting_dims={1}, rhs_contracting_dims={1}
+}
+"""
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == [] and "custom-call" not in new
+
+
+def test_dot_with_second_user_keeps_epilogue_outside():
+    text = hm.c1_s8_channel(4, 64, 32).replace("ROOT %out = bf16[4,32] convert(%dot)",
+                                               "%out = bf16[4,32] convert(%dot)\n  ROOT %t = (bf16[4,32], f32[4,32]) tuple(%out, %dot)")
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == [] and any("is f32" in r for r in rf)
+
+
+def test_quantize_near_misses_are_refused_with_reasons():
+    base = hm.c4_quantize(8, 64)
+    _, rw, rf = hlo.rewrite(base.replace("constant(448)", "constant(240)"))
+    assert rw == [] and rf == []                       # not even the clamp bounds match
+    _, rw, rf = hlo.rewrite(base.replace("%scale = f32[8] divide(%amax, %c448_b)", "%scale = f32[8] multiply(%amax, %c448_b)"))
+    assert rw == [] and "scale is not amax / 448" in rf[0]
+    rs = base.replace("%rt = f32[8] sqrt(%ms_eps)", "%rt = f32[8] rsqrt(%ms_eps)").replace(
+        "%rinv = f32[8] divide(%one_b, %rt)", "%rinv = f32[8] multiply(%one_b, %rt)")
+    _, rw, rf = hlo.rewrite(rs)
+    assert rw == [] and "not the RMSNorm form" in rf[0]

@@ -1,0 +1,598 @@
+// QuantFusionRewriter: matches the quantized-inference patterns in an HLO module and replaces
+// each with one typed-FFI custom call to this library's kernels, in the place where XLA's
+// GemmFusion / GemmRewriter run (xla/service/gpu/gpu_compiler.cc:2113-2129):
+//
+//   convert(f8e4m3fn) [* or / broadcast(scalar)] -> dot [-> +bias] [-> relu|gelu|silu]
+//       => xla_amd.fp8_scaled_dot          (what gemm_rewriter.cc:190-336,1235-1591 turns into
+//                                           __cublas$lt$matmul$f8, epilogues :888-1007,1987-2304)
+//   convert(s8|s4) * broadcast(scale) -> dot [-> +bias] [-> activation]
+//       => xla_amd.dequant_dot             (what gemm_fusion.cc:1629-1702 wraps into __triton_gemm;
+//                                           pattern zoo: fusion_emitter_int4_device_test.cc:85-449)
+//   [RMSNorm ->] reduce-max(abs) -> /448 -> divide -> clamp -> convert(f8e4m3fn)
+//       => xla_amd.rowwise_quantize_fp8    (today: several reduction/loop fusions,
+//                                           codegen/emitters/reduction.cc:840-991)
+//
+// Every refusal is recorded with a reason (the reference logs them with VLOG(1),
+// gemm_rewriter.cc:295,316,1248).  The kernels produce bf16 (f8 for the quantizer), so a
+// pattern is only taken when the value leaving it has that type.
+#include "quant_fusion_rewriter.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <algorithm>
+#include <functional>
+#include <set>
+
+namespace xla_amd {
+namespace hlo {
+namespace {
+
+bool IsFloatTy(const std::string& t) { return t == "f32" || t == "bf16"; }
+int DTypeCode(const std::string& t) { return t == "bf16" ? 16 : 11; }  // XLA PrimitiveType values
+
+std::unique_ptr<Instr> Make(const std::string& name, const std::string& opcode, Shape shape,
+                            std::vector<Instr*> operands) {
+  auto i = std::make_unique<Instr>();
+  i->name = name;
+  i->opcode = opcode;
+  i->shape = std::move(shape);
+  i->operands = std::move(operands);
+  return i;
+}
+
+// Scalar constant value, looking through broadcast and convert.
+bool ConstScalar(const Instr* i, double* v) {
+  while (i->Is("broadcast") || i->Is("convert") || i->Is("reshape") || i->Is("bitcast")) i = i->operands[0];
+  if (!i->Is("constant") || i->shape.num_elements() != 1) return false;
+  std::string lit = i->literal;
+  lit.erase(std::remove_if(lit.begin(), lit.end(), [](char c) { return c == '{' || c == '}' || c == ' '; }),
+            lit.end());
+  if (lit == "inf") { *v = INFINITY; return true; }
+  if (lit == "-inf") { *v = -INFINITY; return true; }
+  char* end = nullptr;
+  *v = strtod(lit.c_str(), &end);
+  return end && *end == 0 && !lit.empty();
+}
+
+bool IsConst(const Instr* i, double want, double rel_tol = 0) {
+  double v;
+  if (!ConstScalar(i, &v)) return false;
+  if (rel_tol == 0) return v == want;
+  return fabs(v - want) <= rel_tol * fabs(want);
+}
+
+// broadcast of a rank-0 value (dimensions={})
+bool ScalarBroadcast(const Instr* i, Instr** scalar) {
+  if (!i->Is("broadcast") || i->operands[0]->shape.rank() != 0) return false;
+  *scalar = i->operands[0];
+  return true;
+}
+
+// broadcast(src), dimensions=dims
+bool BroadcastAlong(const Instr* i, const std::vector<int64_t>& dims, Instr** src) {
+  if (!i->Is("broadcast") || i->DimsAttr("dimensions") != dims) return false;
+  *src = i->operands[0];
+  return true;
+}
+
+bool Binary(const Instr* i, const char* op, Instr** a, Instr** b) {
+  if (!i->Is(op) || i->operands.size() != 2) return false;
+  *a = i->operands[0];
+  *b = i->operands[1];
+  return true;
+}
+
+// Commutative binary op with one side satisfying `pred`; *other receives the other side.
+bool BinaryWith(const Instr* i, const char* op, const std::function<bool(Instr*)>& pred, Instr** other) {
+  Instr *a, *b;
+  if (!Binary(i, op, &a, &b)) return false;
+  if (pred(b)) { *other = a; return true; }
+  if (pred(a)) { *other = b; return true; }
+  return false;
+}
+
+// convert whose operand has element type `from`
+bool ConvertFrom(const Instr* i, const std::string& from, Instr** src) {
+  if (!i->Is("convert") || i->operands[0]->shape.dtype != from) return false;
+  *src = i->operands[0];
+  return true;
+}
+
+std::string I32(int v) { return std::to_string(v) + " : i32"; }
+
+struct Epilogue {
+  Instr* tail = nullptr;     // last instruction absorbed (its value is what the custom call returns)
+  Instr* bias = nullptr;     // [N] operand, bf16 or f32 (null if none)
+  std::string act = "";      // "", RELU, GELU, SILU
+  std::string ops_type;      // element type of the bias add / activation ops
+  std::string Name() const {
+    std::string a = act.empty() ? "" : act;
+    if (bias) return a.empty() ? "BIAS" : "BIAS_" + a;
+    return a.empty() ? "DEFAULT" : a;
+  }
+};
+
+Instr* SoleUser(Instr* i) { return i->users.size() == 1 ? i->users[0] : nullptr; }
+
+// tanh-GELU rooted at `out` = x * cdf, with the op structure of gemm_rewriter.cc:923-973:
+//   cdf = 0.5 * (1 + tanh(c1 * (x + c0 * (x*x*x))))
+bool MatchGelu(Instr* out, Instr* x) {
+  Instr* cdf;
+  if (!BinaryWith(out, "multiply", [&](Instr* s) { return s == x; }, &cdf)) return false;
+  Instr* onep;
+  if (!BinaryWith(cdf, "multiply", [](Instr* s) { return IsConst(s, 0.5); }, &onep)) return false;
+  Instr* th;
+  if (!BinaryWith(onep, "add", [](Instr* s) { return IsConst(s, 1.0); }, &th)) return false;
+  if (!th->Is("tanh")) return false;
+  Instr* inner;
+  if (!BinaryWith(th->operands[0], "multiply", [](Instr* s) { return IsConst(s, 0.7978845608, 1e-2); }, &inner))
+    return false;
+  Instr* cube_term;
+  if (!BinaryWith(inner, "add", [&](Instr* s) { return s == x; }, &cube_term)) return false;
+  Instr* cube;
+  if (!BinaryWith(cube_term, "multiply", [](Instr* s) { return IsConst(s, 0.044715, 1e-2); }, &cube)) return false;
+  Instr* sq;
+  if (!BinaryWith(cube, "multiply", [&](Instr* s) { return s == x; }, &sq)) return false;
+  Instr *a, *b;
+  return Binary(sq, "multiply", &a, &b) && a == x && b == x;
+}
+
+// x * (1 / (1 + exp(-x)))  (gemm_rewriter.cc:995-1002) or x * logistic(x)
+bool MatchSilu(Instr* out, Instr* x) {
+  Instr* sg;
+  if (!BinaryWith(out, "multiply", [&](Instr* s) { return s == x; }, &sg)) return false;
+  if (sg->Is("logistic")) return sg->operands[0] == x;
+  Instr *one, *den;
+  if (!Binary(sg, "divide", &one, &den) || !IsConst(one, 1.0)) return false;
+  Instr* ex;
+  if (!BinaryWith(den, "add", [](Instr* s) { return IsConst(s, 1.0); }, &ex)) return false;
+  return ex->Is("exponential") && ex->operands[0]->Is("negate") && ex->operands[0]->operands[0] == x;
+}
+
+// Walks forward from the dot: optional convert, optional + broadcast(bias) along the minor
+// dimension, optional activation, optional final convert to bf16.  Returns false when what
+// leaves the chain is not bf16.
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why) {
+  Instr* cur = dot;
+  const int64_t rank = dot->shape.rank();
+  ep->ops_type = dot->shape.dtype;
+  auto step_convert = [&]() {
+    Instr* u = SoleUser(cur);
+    if (u && u->Is("convert") && IsFloatTy(u->shape.dtype) && u->shape.dtype != cur->shape.dtype) {
+      cur = u;
+      return true;
+    }
+    return false;
+  };
+  Instr* after_dot = cur;
+  if (step_convert()) ep->ops_type = cur->shape.dtype;
+  // bias: add(cur, broadcast(bias[N]), dimensions={rank-1})
+  if (Instr* u = SoleUser(cur)) {
+    Instr* bsrc = nullptr;
+    Instr* bb = nullptr;
+    if (BinaryWith(u, "add", [&](Instr* s) { return BroadcastAlong(s, {rank - 1}, &bsrc) && s != cur; }, &bb) &&
+        bb == cur && bsrc->shape.rank() == 1) {
+      Instr* raw = bsrc;
+      Instr* inner;
+      if (bsrc->Is("convert") && ConvertFrom(bsrc, "bf16", &inner) && bsrc->shape.dtype == "f32") raw = inner;
+      if (IsFloatTy(raw->shape.dtype)) {
+        ep->bias = raw;
+        cur = u;
+      }
+    }
+  }
+  // activation on cur
+  {
+    // the activation's result is the unique multiply/maximum that consumes cur last; find it
+    // among cur's (transitive) users by trying each candidate root.
+    std::vector<Instr*> frontier = cur->users;
+    std::set<Instr*> seen;
+    Instr* found = nullptr;
+    std::string act;
+    while (!frontier.empty() && !found) {
+      Instr* c = frontier.back();
+      frontier.pop_back();
+      if (!seen.insert(c).second) continue;
+      Instr* other;
+      if (c->Is("maximum") && BinaryWith(c, "maximum", [](Instr* s) { return IsConst(s, 0.0); }, &other) &&
+          other == cur) {
+        found = c;
+        act = "RELU";
+      } else if (c->Is("multiply") && MatchGelu(c, cur)) {
+        found = c;
+        act = "GELU";
+      } else if (c->Is("multiply") && MatchSilu(c, cur)) {
+        found = c;
+        act = "SILU";
+      } else if (seen.size() < 24) {
+        for (Instr* u : c->users) frontier.push_back(u);
+      }
+    }
+    if (found) {
+      // every value between cur and found must stay inside the pattern
+      std::set<Instr*> inside;
+      std::function<void(Instr*)> collect = [&](Instr* n) {
+        if (n == cur || !inside.insert(n).second) return;
+        for (Instr* op : n->operands)
+          if (!op->Is("constant") && !op->Is("broadcast")) collect(op);
+      };
+      collect(found);
+      bool closed = true;
+      for (Instr* n : inside)
+        if (n != found)
+          for (Instr* u : n->users) closed &= inside.count(u) > 0;
+      for (Instr* u : cur->users) closed &= inside.count(u) > 0;
+      if (closed) {
+        ep->act = act;
+        cur = found;
+      }
+    }
+  }
+  if (cur != after_dot && cur != dot) ep->ops_type = cur->shape.dtype;
+  if (!ep->bias && ep->act.empty()) ep->ops_type = dot->shape.dtype;  // nothing between dot and result
+  step_convert();
+  if (cur->shape.dtype != "bf16") {
+    *why = "the value leaving the dot pattern is " + cur->shape.dtype + ", the kernels produce bf16";
+    return false;
+  }
+  ep->tail = cur;
+  return true;
+}
+
+std::string CommonConfig(const Epilogue& ep, const std::string& dequant_ty, const std::string& dot_ty) {
+  return "epilogue = \\\"" + ep.Name() + "\\\", dequant_type = " + I32(DTypeCode(dequant_ty)) +
+         ", dot_type = " + I32(DTypeCode(dot_ty)) + ", epilogue_type = " + I32(DTypeCode(ep.ops_type));
+}
+
+// Emits `(result, scratch) custom-call(...)` + get-tuple-element 0 before `before`, and moves
+// the uses of `tail` to it.
+Instr* EmitCall(Computation* comp, Instr* tail, const std::string& target, std::vector<Instr*> operands,
+                std::vector<Shape> results, const std::string& config) {
+  Shape shape = results.size() == 1 ? results[0] : Shape::Tuple(results);
+  auto cc = Make(comp->UniqueName(tail->name + ".call"), "custom-call", shape, std::move(operands));
+  cc->attrs.emplace_back("custom_call_target", "\"" + target + "\"");
+  cc->attrs.emplace_back("api_version", "API_VERSION_TYPED_FFI");
+  cc->attrs.emplace_back("backend_config", "\"{" + config + "}\"");
+  return comp->Insert(std::move(cc), tail);
+}
+
+Instr* EmitGte(Computation* comp, Instr* call, int index, const Instr* before, const std::string& name) {
+  auto g = Make(comp->UniqueName(name), "get-tuple-element", call->shape.elements[index], {call});
+  g->attrs.emplace_back("index", std::to_string(index));
+  return comp->Insert(std::move(g), before);
+}
+
+Instr* AsF32Scalar(Computation* comp, Instr* s, const Instr* before) {
+  if (s->shape.dtype == "f32") return s;
+  return comp->Insert(Make(comp->UniqueName(s->name + ".f32"), "convert", Shape::Array("f32", {}), {s}), before);
+}
+
+// ---------------------------------------------------------------- f8 scaled dot
+struct F8Operand {
+  Instr* value = nullptr;   // the f8e4m3fn tensor
+  Instr* scale = nullptr;   // scalar, null = 1
+  bool divide = false;
+  std::string type;         // element type of the convert / multiply
+};
+
+bool MatchF8Operand(Instr* op, F8Operand* out) {
+  Instr* src;
+  if (ConvertFrom(op, "f8e4m3fn", &src)) {
+    *out = {src, nullptr, false, op->shape.dtype};
+    return IsFloatTy(op->shape.dtype);
+  }
+  Instr *cv = nullptr, *sc = nullptr;
+  if (op->Is("multiply")) {
+    if (!BinaryWith(op, "multiply", [&](Instr* s) { return ScalarBroadcast(s, &sc); }, &cv)) return false;
+  } else if (op->Is("divide")) {
+    Instr* b;
+    if (!Binary(op, "divide", &cv, &b) || !ScalarBroadcast(b, &sc)) return false;
+    out->divide = true;
+  } else {
+    return false;
+  }
+  if (!ConvertFrom(cv, "f8e4m3fn", &src) || cv->shape.dtype != op->shape.dtype || !IsFloatTy(op->shape.dtype))
+    return false;
+  if (sc->shape.dtype != op->shape.dtype && !(sc->Is("convert") || IsFloatTy(sc->shape.dtype))) return false;
+  out->value = src;
+  out->scale = sc;
+  out->type = op->shape.dtype;
+  return true;
+}
+
+bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
+  F8Operand a, b;
+  if (!MatchF8Operand(dot->operands[0], &a) || !MatchF8Operand(dot->operands[1], &b)) return false;
+  auto refuse = [&](const std::string& why) {
+    log->refusals.push_back(dot->name + ": f8 operands found but not rewritten: " + why);
+    return false;
+  };
+  if (a.type != b.type) return refuse("operands are dequantised in different types");
+  if (dot->shape.rank() != 2 || a.value->shape.rank() != 2 || b.value->shape.rank() != 2)
+    return refuse("only rank-2 dots are supported");
+  if (!dot->DimsAttr("lhs_batch_dims").empty()) return refuse("batch dimensions are not supported");
+  auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
+  if (lc.size() != 1 || rc.size() != 1 || lc[0] != 1) return refuse("lhs must contract its minor dimension");
+  if (!IsFloatTy(dot->shape.dtype)) return refuse("dot result type " + dot->shape.dtype);
+  Epilogue ep;
+  std::string why;
+  if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
+
+  const int64_t M = a.value->shape.dims[0], K = a.value->shape.dims[1], N = b.value->shape.dims[1 - rc[0]];
+  auto scale_of = [&](const F8Operand& o) -> Instr* {
+    Instr* s = o.scale;
+    if (!s) {
+      auto one = Make(comp->UniqueName("one"), "constant", Shape::Array("f32", {}), {});
+      one->literal = "1";
+      return comp->Insert(std::move(one), ep.tail);
+    }
+    s = AsF32Scalar(comp, s, ep.tail);
+    if (o.divide) {
+      auto one = Make(comp->UniqueName("one"), "constant", Shape::Array("f32", {}), {});
+      one->literal = "1";
+      Instr* o1 = comp->Insert(std::move(one), ep.tail);
+      s = comp->Insert(Make(comp->UniqueName(s->name + ".rcp"), "divide", Shape::Array("f32", {}), {o1, s}), ep.tail);
+    }
+    return s;
+  };
+  std::vector<Instr*> ops = {a.value, b.value, scale_of(a), scale_of(b)};
+  if (ep.bias) ops.push_back(ep.bias);
+  std::vector<Shape> results = {Shape::Array("bf16", {M, N})};
+  size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0]) : 0;
+  if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
+  std::string cfg = CommonConfig(ep, a.type, dot->shape.dtype) + ", rhs_contracting_dim = " +
+                    std::to_string(rc[0]) + " : i64";
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, results, cfg);
+  Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
+  comp->ReplaceAllUses(ep.tail, value);
+  log->rewrites.push_back(dot->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + "]");
+  return true;
+}
+
+// ---------------------------------------------------------------- weight-only dequantize dot
+struct QWeights {
+  Instr* w = nullptr;       // s8 or s4 tensor [B,]K,N
+  Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N], bf16 or f32
+  std::string type;         // element type of the multiply
+};
+
+// integer tensor behind convert(s4->s8)? -> convert(->float)
+bool IntSource(Instr* cv, const std::string& float_ty, Instr** w) {
+  if (!cv->Is("convert") || cv->shape.dtype != float_ty) return false;
+  Instr* s = cv->operands[0];
+  if (s->shape.dtype == "s8" && s->Is("convert") && s->operands[0]->shape.dtype == "s4") s = s->operands[0];
+  if (s->shape.dtype != "s8" && s->shape.dtype != "s4") return false;
+  *w = s;
+  return true;
+}
+
+Instr* LookThroughWidening(Instr* s, const std::string& to) {
+  // convert(bf16 -> f32) of a scale is exact: hand the kernel the narrow original
+  if (s->Is("convert") && to == "f32" && s->operands[0]->shape.dtype == "bf16") return s->operands[0];
+  return s;
+}
+
+bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
+  const std::string ty = op->shape.dtype;
+  if (!IsFloatTy(ty)) return false;
+  const int64_t rank = op->shape.rank();
+  // grouped: reshape([G,g,N] product) -> [K,N]
+  if (op->Is("reshape") && rank == 2 && op->operands[0]->shape.rank() == 3 && op->operands[0]->Is("multiply")) {
+    Instr* mul = op->operands[0];
+    const auto& d3 = mul->shape.dims;  // G, g, N
+    if (d3[0] * d3[1] != op->shape.dims[0] || d3[2] != op->shape.dims[1]) return false;
+    Instr *sc = nullptr, *cv = nullptr;
+    if (!BinaryWith(mul, "multiply", [&](Instr* s) { return BroadcastAlong(s, {0, 2}, &sc); }, &cv)) return false;
+    // the convert may sit before or after the reshape to [G,g,N]
+    Instr* w = nullptr;
+    if (cv->Is("convert") && cv->operands[0]->Is("reshape")) {
+      Instr* rs = cv->operands[0];
+      Instr* src = rs->operands[0];
+      if (src->shape.dtype == "s8" && src->Is("convert") && src->operands[0]->shape.dtype == "s4") src = src->operands[0];
+      if ((src->shape.dtype == "s8" || src->shape.dtype == "s4") && src->shape.rank() == 2) w = src;
+    } else if (cv->Is("reshape")) {
+      IntSource(cv->operands[0], ty, &w);
+    }
+    if (!w || w->shape.dims != op->shape.dims) {
+      *why = "grouped dequantise: could not find the integer weights behind the reshape";
+      return false;
+    }
+    sc = LookThroughWidening(sc, ty);
+    if (sc->shape.rank() != 2 || sc->shape.dims[0] != d3[0] || sc->shape.dims[1] != d3[2]) return false;
+    *out = {w, sc, ty};
+    return true;
+  }
+  if (!op->Is("multiply")) return false;
+  Instr *sc = nullptr, *cv = nullptr;
+  const std::vector<int64_t> bdims = rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2};
+  if (!BinaryWith(op, "multiply", [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
+  Instr* w;
+  if (!IntSource(cv, ty, &w) || w->shape.dims != op->shape.dims) return false;
+  sc = LookThroughWidening(sc, ty);
+  *out = {w, sc, ty};
+  return true;
+}
+
+bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
+  QWeights q;
+  std::string why;
+  if (!MatchQWeights(dot->operands[1], &q, &why)) {
+    if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
+    return false;
+  }
+  auto refuse = [&](const std::string& w) {
+    log->refusals.push_back(dot->name + ": quantized weights found but not rewritten: " + w);
+    return false;
+  };
+  Instr* lhs = dot->operands[0];
+  Instr* inner;
+  if (lhs->Is("convert") && ConvertFrom(lhs, "bf16", &inner) && lhs->shape.dtype == "f32") lhs = inner;
+  if (lhs->shape.dtype != "bf16") return refuse("the activation must be bf16 (or its convert to f32)");
+  const int64_t rank = dot->shape.rank();
+  if (rank != 2 && rank != 3) return refuse("rank " + std::to_string(rank));
+  auto lb = dot->DimsAttr("lhs_batch_dims"), rb = dot->DimsAttr("rhs_batch_dims");
+  auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
+  if (rank == 3 && (lb != std::vector<int64_t>{0} || rb != std::vector<int64_t>{0}))
+    return refuse("the batch dimension must be dimension 0 of both operands");
+  if (rank == 2 && !lb.empty()) return refuse("unexpected batch dimensions");
+  if (lc != std::vector<int64_t>{rank - 1} || rc != std::vector<int64_t>{rank - 2})
+    return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] contracting K (N minor); s4 with a "
+                  "minor contracting or batch dimension is rejected as in gemm_fusion.cc:1572-1590");
+  if (q.w->shape.dtype == "s4" && q.w->shape.dims.back() % 2 != 0)
+    return refuse("s4 rows must hold an even number of values");
+  if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
+  Epilogue ep;
+  if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
+
+  const int64_t B = rank == 3 ? lhs->shape.dims[0] : 1;
+  const int64_t M = lhs->shape.dims[rank - 2], K = lhs->shape.dims[rank - 1], N = q.w->shape.dims[rank - 1];
+  std::vector<Instr*> ops = {lhs, q.w, q.scale};
+  if (ep.bias) ops.push_back(ep.bias);
+  std::vector<Shape> results = {Shape::Array("bf16", dot->shape.dims)};
+  size_t ws = opt.dequant_workspace_bytes
+                  ? opt.dequant_workspace_bytes(B, M, K, N, q.w->shape.dtype == "s4" ? 21 : 2)
+                  : 0;
+  if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results, CommonConfig(ep, q.type, dot->shape.dtype));
+  Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
+  comp->ReplaceAllUses(ep.tail, value);
+  log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype + "]");
+  return true;
+}
+
+// ---------------------------------------------------------------- row-wise fp8 quantize
+bool IsReduceOver(const Instr* r, const Module& m, const char* body_op, int64_t dim, Instr** src, Instr** init) {
+  if (!r->Is("reduce") || r->operands.size() != 2 || r->DimsAttr("dimensions") != std::vector<int64_t>{dim}) return false;
+  const std::string* to = r->Attr("to_apply");
+  if (!to) return false;
+  std::string name = *to;
+  if (!name.empty() && name[0] == '%') name = name.substr(1);
+  const Computation* c = m.FindComputation(name);
+  if (!c || !c->root() || !c->root()->Is(body_op)) return false;
+  *src = r->operands[0];
+  *init = r->operands[1];
+  return true;
+}
+
+bool RewriteQuantize(const Module& mod, Computation* comp, Instr* q, RewriteLog* log) {
+  // q = convert(clamp(-448, yf / broadcast(s), 448)) -> f8e4m3fn [R,C]
+  if (!q->Is("convert") || q->shape.dtype != "f8e4m3fn" || q->shape.rank() != 2) return false;
+  Instr* cl = q->operands[0];
+  if (!cl->Is("clamp") || cl->operands.size() != 3 || !IsConst(cl->operands[0], -448.0) || !IsConst(cl->operands[2], 448.0))
+    return false;
+  auto refuse = [&](const std::string& w) {
+    log->refusals.push_back(q->name + ": clamp/convert to f8e4m3fn found but not rewritten: " + w);
+    return false;
+  };
+  Instr *yf, *sb, *s;
+  if (!Binary(cl->operands[1], "divide", &yf, &sb) || !BroadcastAlong(sb, {0}, &s))
+    return refuse("the clamped value is not y / broadcast(scale[rows])");
+  Instr *amax, *c448;
+  if (!Binary(s, "divide", &amax, &c448) || !IsConst(c448, 448.0)) return refuse("scale is not amax / 448");
+  Instr *absy, *init;
+  if (!IsReduceOver(amax, mod, "maximum", 1, &absy, &init) || !absy->Is("abs") || absy->operands[0] != yf)
+    return refuse("amax is not reduce-max(abs(y)) over the columns");
+  double iv;
+  if (!ConstScalar(init, &iv) || !(iv == 0.0 || iv == -INFINITY)) return refuse("reduce-max init must be 0 or -inf");
+  Instr* y;
+  if (!ConvertFrom(yf, "bf16", &y) || yf->shape.dtype != "f32") return refuse("y must be a bf16 value converted to f32");
+  // users of yf: abs and the divide; of s: its broadcast (and possibly the module result)
+  for (Instr* u : yf->users)
+    if (u != absy && u != cl->operands[1]) return refuse("f32(y) has other users");
+
+  Instr *x = y, *gamma = nullptr;
+  double eps = 1e-6;
+  bool rms = false;
+  // y = convert((xf * broadcast(rinv)) * broadcast(f32(gamma))) -> bf16
+  if (y->Is("convert") && y->operands[0]->shape.dtype == "f32" && y->operands[0]->Is("multiply")) {
+    Instr *gsrc = nullptr, *t = nullptr;
+    if (BinaryWith(y->operands[0], "multiply", [&](Instr* b) { return BroadcastAlong(b, {1}, &gsrc); }, &t)) {
+      Instr *rinv = nullptr, *xf = nullptr, *g = nullptr, *xin = nullptr;
+      if (ConvertFrom(gsrc, "bf16", &g) &&
+          BinaryWith(t, "multiply", [&](Instr* b) { return BroadcastAlong(b, {0}, &rinv); }, &xf) &&
+          ConvertFrom(xf, "bf16", &xin)) {
+        // rinv = 1 / sqrt(sum(xf*xf)/C + eps)
+        Instr *one, *rt;
+        if (Binary(rinv, "divide", &one, &rt) && IsConst(one, 1.0) && rt->Is("sqrt")) {
+          Instr* ms = nullptr;
+          Instr* me = rt->operands[0];
+          if (BinaryWith(me, "add", [&](Instr* b) { return ConstScalar(b, &eps); }, &ms)) {
+            Instr *ssum = nullptr, *cnt = nullptr;
+            double cv = 0;
+            bool mean_ok = false;
+            if (Binary(ms, "divide", &ssum, &cnt) && ConstScalar(cnt, &cv) && cv == (double)q->shape.dims[1]) mean_ok = true;
+            Instr *sq, *zero;
+            if (mean_ok && IsReduceOver(ssum, mod, "add", 1, &sq, &zero) && IsConst(zero, 0.0)) {
+              Instr *a, *b;
+              if (Binary(sq, "multiply", &a, &b) && a == xf && b == xf) {
+                rms = true;
+                x = xin;
+                gamma = g;
+              }
+            }
+          }
+        }
+      }
+    }
+    if (!rms) return refuse("y is computed from a multiply that is not the RMSNorm form x * (1/sqrt(mean(x^2)+eps)) * gamma");
+  }
+  if (x->shape.dtype != "bf16") return refuse("input must be bf16");
+
+  const int64_t R = q->shape.dims[0], C = q->shape.dims[1];
+  std::vector<Instr*> ops = {x};
+  if (rms) ops.push_back(gamma);
+  char epsbuf[64];
+  snprintf(epsbuf, sizeof(epsbuf), "%.9g", eps);
+  std::string cfg = std::string("rmsnorm = ") + (rms ? "true" : "false") + ", eps = " + epsbuf + " : f32";
+  // place the call where the scale is computed: it precedes every user of q and of s
+  Instr* call = EmitCall(comp, s, "xla_amd.rowwise_quantize_fp8", ops,
+                         {Shape::Array("f8e4m3fn", {R, C}), Shape::Array("f32", {R})}, cfg);
+  Instr* s_new = EmitGte(comp, call, 1, s, s->name + ".scales");
+  Instr* q_new = EmitGte(comp, call, 0, s, q->name + ".codes");
+  // every user of the scale other than the pattern's own broadcast keeps working on s_new
+  for (auto& i : comp->instrs)
+    if (i.get() != sb)
+      for (Instr*& op : i->operands)
+        if (op == s) op = s_new;
+  if (s->is_root) { s->is_root = false; s_new->is_root = true; }
+  comp->ReplaceAllUses(q, q_new);
+  log->rewrites.push_back(q->name + " -> xla_amd.rowwise_quantize_fp8 [" + (rms ? "rmsnorm" : "plain") + "]");
+  return true;
+}
+
+}  // namespace
+
+int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* log) {
+  int changed = 0;
+  for (auto& comp : mod->computations) {
+    bool again = true;
+    while (again) {
+      again = false;
+      comp->RecomputeUsers();
+      for (auto& up : comp->instrs) {
+        Instr* i = up.get();
+        bool did = false;
+        if (i->Is("dot") && i->operands.size() == 2) {
+          did = RewriteF8Dot(comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
+        } else if (i->Is("convert") && i->shape.dtype == "f8e4m3fn") {
+          did = RewriteQuantize(*mod, comp.get(), i, log);
+        }
+        if (did) {
+          ++changed;
+          comp->RemoveDead();
+          again = true;
+          break;  // the instruction list changed under the loop
+        }
+      }
+    }
+  }
+  // refusals are re-recorded on every sweep; keep each once
+  std::sort(log->refusals.begin(), log->refusals.end());
+  log->refusals.erase(std::unique(log->refusals.begin(), log->refusals.end()), log->refusals.end());
+  return changed;
+}
+
+}  // namespace hlo
+}  // namespace xla_amd

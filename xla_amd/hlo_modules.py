@@ -1,0 +1,189 @@
+"""HLO text of the five benchmark configurations, parameterised by shape.
+
+These are the modules a framework would hand to XLA: plain convert / multiply / dot /
+reduce ops with no custom calls.  The CPU backend runs them as they are; the rewrite pass
+turns each into one custom call of this library.
+"""
+
+REDUCERS = """
+%add_f32 {
+  %a = f32[] parameter(0)
+  %b = f32[] parameter(1)
+  ROOT %s = f32[] add(%a, %b)
+}
+
+%max_f32 {
+  %a = f32[] parameter(0)
+  %b = f32[] parameter(1)
+  ROOT %m = f32[] maximum(%a, %b)
+}
+"""
+
+
+def c1_s8_channel(M=16, K=4096, N=4096):
+    """bf16 [M,K] . (convert(s8 [K,N]) * f32 scale[N]) -> bf16; f32 multiply, one final rounding."""
+    return f"""HloModule c1_s8_channel_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s8[{K},{N}] parameter(1)
+  %scale = f32[{N}] parameter(2)
+  %lhs_f32 = f32[{M},{K}] convert(%lhs)
+  %w_f32 = f32[{K},{N}] convert(%w)
+  %scale_b = f32[{K},{N}] broadcast(%scale), dimensions={{1}}
+  %w_deq = f32[{K},{N}] multiply(%w_f32, %scale_b)
+  %dot = f32[{M},{N}] dot(%lhs_f32, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
+  ROOT %out = bf16[{M},{N}] convert(%dot)
+}}
+"""
+
+
+def c2_s4_group(M=1, K=8192, N=28672, group=128):
+    """bf16 [M,K] . bf16(convert(s4 [K,N]) * bf16 scale[K/g,N]) + bias, SiLU in f32 -> bf16.
+    The dequantise multiply is bf16-typed, as in XLA's int4 tests."""
+    G = K // group
+    return f"""HloModule c2_s4_group_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s4[{K},{N}] parameter(1)
+  %scales = bf16[{G},{N}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %w_s8 = s8[{K},{N}] convert(%w)
+  %w_g = s8[{G},{group},{N}] reshape(%w_s8)
+  %w_bf16 = bf16[{G},{group},{N}] convert(%w_g)
+  %scales_b = bf16[{G},{group},{N}] broadcast(%scales), dimensions={{0,2}}
+  %w_deq_g = bf16[{G},{group},{N}] multiply(%w_bf16, %scales_b)
+  %w_deq = bf16[{K},{N}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] dot(%lhs, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  %neg = f32[{M},{N}] negate(%z)
+  %exp = f32[{M},{N}] exponential(%neg)
+  %one = f32[] constant(1)
+  %one_b = f32[{M},{N}] broadcast(%one), dimensions={{}}
+  %den = f32[{M},{N}] add(%one_b, %exp)
+  %sig = f32[{M},{N}] divide(%one_b, %den)
+  %silu = f32[{M},{N}] multiply(%z, %sig)
+  ROOT %out = bf16[{M},{N}] convert(%silu)
+}}
+"""
+
+
+def c3_fp8(M=8192, K=8192, N=8192, typed="f32"):
+    """f8 [M,K] . f8 [K,N] with per-tensor scales, + bias, GELU(tanh) -> bf16.  typed="f32":
+    f32 ops and one final rounding; typed="bf16": every op bf16-typed (the shape of
+    gemm_rewriter_fp8_test.cc:1110-1141)."""
+    t = typed
+    scale_decl = (f"  %a_scale = {t}[] parameter(2)\n  %b_scale = {t}[] parameter(3)\n")
+    tail = (f"  ROOT %out = bf16[{M},{N}] convert(%gelu)\n" if t == "f32" else "")
+    root = "" if t == "f32" else "ROOT "
+    bias_line = (f"  %bias_t = f32[{N}] convert(%bias)\n" if t == "f32" else "")
+    bias_name = "%bias_t" if t == "f32" else "%bias"
+    return f"""HloModule c3_fp8_scaled_dot
+
+ENTRY %main {{
+  %a = f8e4m3fn[{M},{K}] parameter(0)
+  %b = f8e4m3fn[{K},{N}] parameter(1)
+{scale_decl}  %bias = bf16[{N}] parameter(4)
+  %a_t = {t}[{M},{K}] convert(%a)
+  %b_t = {t}[{K},{N}] convert(%b)
+  %a_scale_b = {t}[{M},{K}] broadcast(%a_scale), dimensions={{}}
+  %b_scale_b = {t}[{K},{N}] broadcast(%b_scale), dimensions={{}}
+  %a_deq = {t}[{M},{K}] multiply(%a_t, %a_scale_b)
+  %b_deq = {t}[{K},{N}] multiply(%b_t, %b_scale_b)
+  %dot = {t}[{M},{N}] dot(%a_deq, %b_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
+{bias_line}  %bias_b = {t}[{M},{N}] broadcast({bias_name}), dimensions={{1}}
+  %z = {t}[{M},{N}] add(%dot, %bias_b)
+  %z2 = {t}[{M},{N}] multiply(%z, %z)
+  %z3 = {t}[{M},{N}] multiply(%z, %z2)
+  %c0 = {t}[] constant(0.044715)
+  %c0_b = {t}[{M},{N}] broadcast(%c0), dimensions={{}}
+  %z3c = {t}[{M},{N}] multiply(%z3, %c0_b)
+  %inner = {t}[{M},{N}] add(%z, %z3c)
+  %c1 = {t}[] constant(0.797884583)
+  %c1_b = {t}[{M},{N}] broadcast(%c1), dimensions={{}}
+  %arg = {t}[{M},{N}] multiply(%inner, %c1_b)
+  %tanh = {t}[{M},{N}] tanh(%arg)
+  %one = {t}[] constant(1)
+  %one_b = {t}[{M},{N}] broadcast(%one), dimensions={{}}
+  %onep = {t}[{M},{N}] add(%tanh, %one_b)
+  %half = {t}[] constant(0.5)
+  %half_b = {t}[{M},{N}] broadcast(%half), dimensions={{}}
+  %cdf = {t}[{M},{N}] multiply(%onep, %half_b)
+  {root}%gelu = {t}[{M},{N}] multiply(%z, %cdf)
+{tail}}}
+"""
+
+
+def c4_quantize(rows=16384, cols=8192, rmsnorm=True, eps=1e-6):
+    """RMSNorm (f32 math, bf16 result) -> per-row amax -> scale = amax/448 -> clamp -> f8e4m3fn."""
+    R, C = rows, cols
+    if rmsnorm:
+        norm = f"""  %gamma = bf16[{C}] parameter(1)
+  %x_f32 = f32[{R},{C}] convert(%x)
+  %sq = f32[{R},{C}] multiply(%x_f32, %x_f32)
+  %zero = f32[] constant(0)
+  %ssum = f32[{R}] reduce(%sq, %zero), dimensions={{1}}, to_apply=%add_f32
+  %count = f32[] constant({C})
+  %count_b = f32[{R}] broadcast(%count), dimensions={{}}
+  %ms = f32[{R}] divide(%ssum, %count_b)
+  %eps = f32[] constant({eps!r})
+  %eps_b = f32[{R}] broadcast(%eps), dimensions={{}}
+  %ms_eps = f32[{R}] add(%ms, %eps_b)
+  %rt = f32[{R}] sqrt(%ms_eps)
+  %one = f32[] constant(1)
+  %one_b = f32[{R}] broadcast(%one), dimensions={{}}
+  %rinv = f32[{R}] divide(%one_b, %rt)
+  %rinv_b = f32[{R},{C}] broadcast(%rinv), dimensions={{0}}
+  %xn = f32[{R},{C}] multiply(%x_f32, %rinv_b)
+  %gamma_f32 = f32[{C}] convert(%gamma)
+  %gamma_b = f32[{R},{C}] broadcast(%gamma_f32), dimensions={{1}}
+  %y_f32 = f32[{R},{C}] multiply(%xn, %gamma_b)
+  %y = bf16[{R},{C}] convert(%y_f32)
+"""
+        ysrc = "%y"
+    else:
+        norm = ""
+        ysrc = "%x"
+    return f"""HloModule c4_rowwise_quantize_fp8
+{REDUCERS}
+ENTRY %main {{
+  %x = bf16[{R},{C}] parameter(0)
+{norm}  %yf = f32[{R},{C}] convert({ysrc})
+  %absy = f32[{R},{C}] abs(%yf)
+  %ninf = f32[] constant(-inf)
+  %amax = f32[{R}] reduce(%absy, %ninf), dimensions={{1}}, to_apply=%max_f32
+  %c448 = f32[] constant(448)
+  %c448_b = f32[{R}] broadcast(%c448), dimensions={{}}
+  %scale = f32[{R}] divide(%amax, %c448_b)
+  %scale_b = f32[{R},{C}] broadcast(%scale), dimensions={{0}}
+  %scaled = f32[{R},{C}] divide(%yf, %scale_b)
+  %lo = f32[] constant(-448)
+  %lo_b = f32[{R},{C}] broadcast(%lo), dimensions={{}}
+  %hi = f32[] constant(448)
+  %hi_b = f32[{R},{C}] broadcast(%hi), dimensions={{}}
+  %clamped = f32[{R},{C}] clamp(%lo_b, %scaled, %hi_b)
+  %q = f8e4m3fn[{R},{C}] convert(%clamped)
+  ROOT %result = (f8e4m3fn[{R},{C}], f32[{R}]) tuple(%q, %scale)
+}}
+"""
+
+
+def c5_s8_batched(B=8, M=512, K=4096, N=14336):
+    """bf16 [B,M,K] . (convert(s8 [B,K,N]) * f32 scale[B,N]), batch dimension 0 -> bf16 [B,M,N]."""
+    return f"""HloModule c5_s8_batched_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{B},{M},{K}] parameter(0)
+  %w = s8[{B},{K},{N}] parameter(1)
+  %scale = f32[{B},{N}] parameter(2)
+  %lhs_f32 = f32[{B},{M},{K}] convert(%lhs)
+  %w_f32 = f32[{B},{K},{N}] convert(%w)
+  %scale_b = f32[{B},{K},{N}] broadcast(%scale), dimensions={{0,2}}
+  %w_deq = f32[{B},{K},{N}] multiply(%w_f32, %scale_b)
+  %dot = f32[{B},{M},{N}] dot(%lhs_f32, %w_deq), lhs_batch_dims={{0}}, lhs_contracting_dims={{2}}, rhs_batch_dims={{0}}, rhs_contracting_dims={{1}}
+  ROOT %out = bf16[{B},{M},{N}] convert(%dot)
+}}
+"""
