@@ -65,7 +65,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
-// N32 consecutive dwords (1, 2 or a multiple of 4) at voff + soff (soff wave-uniform).
+// N32 consecutive dwords (1, 2 or a multiple of 4) at voff + soff.  The hardware range-checks
+// the per-lane offset only, so soff must be 0 wherever running past the end is possible.
 template <int N32>
 __device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff,
                                                   uint32_t* dst) {
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   auto load_rows = [&](int buf, int k0) {
 #pragma unroll
     for (int r = 0; r < 8; ++r)
-      buffer_load_words<WORDS>(rw, voff_w, (uint32_t)(k0 + r) * pitch, wq[buf][r]);
+      buffer_load_words<WORDS>(rw, voff_w + (uint32_t)(k0 + r) * pitch, 0, wq[buf][r]);
   };
 
   auto compute = [&](int buf, int k0) {
@@ -168,7 +169,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt], (uint32_t)k0 * 2u, 0);
+      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt] + (uint32_t)k0 * 2u, 0, 0);
       if (k0 + 32 > p.K) {  // scalar condition: only a step that crosses the end of K
         const bool ok = k0 + 8 * kb < p.K;
         v = uintx4{ok ? v[0] : 0u, ok ? v[1] : 0u, ok ? v[2] : 0u, ok ? v[3] : 0u};

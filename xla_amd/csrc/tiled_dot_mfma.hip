@@ -3,21 +3,24 @@
 //   kFp8 : out[m,n] = epi( a_scale*b_scale * sum_k A8[m,k] * B8[n,k] )   f8e4m3fn x f8e4m3fn
 //   kS8  : out[b,m,n] = epi( scale[b,n] * sum_k A[b,m,k] * W[b,k,n] )    bf16 x s8 (per channel)
 //
-// A workgroup of 4 waves owns a 128x128 output tile and walks K in stages of
-// 128 bytes of the activation row (128 fp8 or 64 bf16 values).  Both operand
-// tiles of a stage sit in LDS with the contracting dimension contiguous, so a
-// lane fetches its MFMA fragment with 128-bit reads; the next stage's global
-// loads are issued before the current stage's MFMAs and written to the other
-// LDS buffer afterwards.  The s8 weights are [K,N] with N minor: a lane reads
-// 4 channels of 8 consecutive rows, converts (exactly) to bf16 and writes each
-// channel's 8 values as one 16-byte LDS row piece -- the transposition costs
-// nothing beyond the convert.
+// A workgroup of 4 waves (2x2) owns a 256x256 output tile, each wave a 128x128 quarter held
+// in 256 accumulator registers, and walks K in stages of 128 bytes per activation row (128
+// fp8 or 64 bf16 values).  Both operand tiles of a stage sit in LDS with the contracting
+// dimension contiguous (128-byte rows, 16-byte chunks XOR-swizzled by row so that the
+// 128-bit fragment reads of 8 consecutive rows hit 8 different bank groups).  The
+// activation tile -- and the fp8 weight tile, stored [N,K] -- go from global memory
+// straight into LDS (buffer_load ... lds: no staging registers, out-of-range rows arrive as
+// zeros); the swizzle is applied by permuting which global chunk each lane fetches.  The s8
+// weights are [K,N] with N minor: a lane reads 4 channels of 8 consecutive rows, converts
+// (exactly) to bf16 and writes each channel's 8 values as one swizzled 16-byte chunk, so
+// the transposition costs nothing beyond the convert.  Stage s+1 is in flight while stage
+// s feeds the matrix cores.
 //
-// The MFMA's 16-row operand is fed with *output channels* and the 16-column
-// operand with tokens, so a lane ends up with 4 consecutive channels of one
-// token and stores them as one 8-byte piece of the bf16 output row.
+// The 32-row MFMA operand is fed with *output channels* and the 32-column operand with
+// tokens, so a lane ends up with runs of 4 consecutive channels of one token and stores
+// each as one 8-byte piece of the bf16 output row.
 //
-// Bound: MFMA (fp8: v_mfma_f32_16x16x128_f8f6f4, bf16: v_mfma_f32_16x16x32_bf16).
+// Bound: MFMA (fp8: v_mfma_f32_32x32x64_f8f6f4, bf16: v_mfma_f32_32x32x16_bf16).
 // Algorithmic flops: 2*M*N*K per batch.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -30,9 +33,8 @@ namespace {
 
 enum : int { kFp8 = 0, kS8 = 1 };
 
-constexpr int kTM = 128, kTN = 128;  // output tile (tokens x channels)
-constexpr int kStageBytes = 128;     // bytes of K per LDS row per stage
-constexpr int kPitch = kStageBytes + 16;  // padded LDS row pitch: 128-bit reads stay conflict-free
+constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
+constexpr int kRow = 128;            // bytes of K per LDS row per stage
 
 struct TiledParams {
   const uint8_t* a;     // kFp8: f8 [M,K]; kS8: bf16 [batch,M,K]
@@ -56,174 +58,260 @@ __device__ __forceinline__ bool is_pow2_f32(float s) {
   return (u & 0x807fffffu) == 0u && e > 24u && e < 230u;
 }
 
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// 64 lanes x 16 bytes from the buffer into 1 KiB of LDS starting at `dst` (lane l lands at
+// dst + 16*l); out-of-range lanes deposit zeros.
+// Everything goes into the per-lane offset: that is the part the hardware range-checks.
+constexpr uint32_t kOutOfRange = 0x80000000u;  // every buffer here is smaller than 2 GiB
+__device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t r, uint8_t* dst, uint32_t voff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(uintptr_t)dst, 16, voff, 0, 0, 0);
+}
+
+// Writes one wave's 128x128 quarter.  Register v of tile (nt, mt) in lane (l32, kb) is
+//   token   m_base + mt*32 + l32,   channel n_base + nt*32 + (v/4)*8 + kb*4 + v%4.
+// ACT >= 0: f32-typed ops with that activation (bias folded in as an add of 0 when absent);
+// ACT < 0: any typing, through epilogue_dispatch.
+template <int KIND, int ACT>
+__device__ __forceinline__ void store_tile(const TiledParams& p, const floatx16 (&acc)[4][4], float alpha,
+                                           int batch, int m_base, int n_base, int l32, int kb) {
+  const bool n_vec = (p.N & 3) == 0;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+    for (int vq = 0; vq < 4; ++vq) {
+      const int n = n_base + nt * 32 + vq * 8 + kb * 4;
+      float sc[4], bs[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const bool ok = n + t < p.N;
+        sc[t] = alpha;
+        if (KIND == kS8) {
+          const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
+          sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
+        }
+        bs[t] = 0.0f;
+        if (p.bias) {
+          const int bi = ok ? n + t : 0;
+          bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        const int m = m_base + mt * 32 + l32;
+        float v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const float x = acc[nt][mt][vq * 4 + t] * sc[t];
+          if (ACT >= 0) v[t] = epilogue_value<false, false>(x, bs[t], ACT | 1);
+          else v[t] = epilogue_dispatch(x, bs[t], p.epilogue, p.bf16_dot, p.bf16_ops);
+        }
+        if (m < p.M && n < p.N) {
+          uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n;
+          if (n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
+            const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<uintx2*>(dst) = o;
+          } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (n + t < p.N) dst[t] = f32_to_bf16(v[t]);
+          }
+        }
+      }
+    }
+  }
+}
+
 template <int KIND>
 __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
-  constexpr int ESZ = KIND == kFp8 ? 1 : 2;      // bytes per A element
-  constexpr int KS = kStageBytes / ESZ;          // K elements per stage
-  __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][kTM * kPitch];
-  __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][kTN * kPitch];
+  constexpr int ESZ = KIND == kFp8 ? 1 : 2;  // bytes per activation element
+  constexpr int KS = kRow / ESZ;             // K elements per stage
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [2][(kTM + kTN) * kRow]
+  constexpr int kBufBytes = (kTM + kTN) * kRow;
 
   if (KIND == kFp8 && p.require_pow2_scales) {
     if (!(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;  // the exact kernel runs
   }
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int li = lane & 15, kb = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, kb = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
 
+  // Workgroup id -> tile: consecutive ids of one XCD take 8 neighbouring channel tiles of one
+  // token tile, then the next token tile, so a token tile and 8 weight tiles stay hot in L2.
   int bid = blockIdx.x;
   {
     const int total = gridDim.x;
-    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;  // one XCD: a contiguous run
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
   }
-  const int tm = bid % p.tiles_m, tn = bid / p.tiles_m;
+  int tm, tn;
+  {
+    const int G = 8;
+    const int full = (p.tiles_n / G) * G;           // channel tiles covered by complete groups
+    const int per_group = G * p.tiles_m;
+    if (bid < (full / G) * per_group) {
+      const int g = bid / per_group, r = bid % per_group;
+      tn = g * G + r % G;
+      tm = r / G;
+    } else {
+      const int r = bid - (full / G) * per_group, w = p.tiles_n - full;  // last, narrower group
+      tn = full + r % w;
+      tm = r / w;
+    }
+  }
   const int batch = blockIdx.y;
   const int m0 = tm * kTM, n0 = tn * kTN;
 
-  const uint8_t* A = p.a + (size_t)batch * p.M * p.K * ESZ;
-  const uint8_t* B = p.b + (size_t)batch * p.K * p.N;  // kS8 only uses the batch offset
+  const uint32_t a_pitch = (uint32_t)p.K * ESZ;
+  const __amdgpu_buffer_rsrc_t ra =
+      tile_rsrc(p.a + (size_t)batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
+  const __amdgpu_buffer_rsrc_t rb =
+      KIND == kFp8 ? tile_rsrc(p.b, (uint32_t)p.N * (uint32_t)p.K)
+                   : tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
 
-  floatx4 acc[4][4];
+  // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
+  // of row l/8 with global chunk (l%8) ^ (row & 7).  Wave w owns rows [w*64, w*64+64) of a
+  // 256-row tile: 8 instructions per tile per stage.
+  const int ld_row = lane >> 3;                       // 0..7 within an instruction
+  const int ld_chunk = (lane & 7) ^ (ld_row & 7);     // rows start at multiples of 8, so row&7 == ld_row
+  uint32_t voff_a[8], voff_b[8];
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
-#pragma unroll
-    for (int y = 0; y < 4; ++y) acc[x][y] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 8; ++j) {
+    const int r = wave * 64 + j * 8 + ld_row;
+    voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk * 16;
+    if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk * 16;
+  }
+  const bool k_tail = (a_pitch % kRow) != 0;  // last stage is partial: chunks past K must read as 0
 
-  uintx4 ga[4];
-  uintx4 gb[4];      // kFp8: 4 chunks of the B tile; kS8: 8 dwords = rows of 4 channels
-  auto gload = [&](int k0) {
+  // ---- s8 weights: item = (8-row block kblk, 4-channel quad nq); 512 items, 2 per thread
+  uint32_t wreg[2][8];
+  auto s8_load = [&](int k0) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int c = tid + 256 * q, row = c >> 3, col = (c & 7) * 16;  // 8 chunks of 16 B per row
-      const int m = m0 + row;
-      const int kbyte = k0 * ESZ + col;
-      ga[q] = uintx4{0u, 0u, 0u, 0u};
-      if (m < p.M && kbyte < p.K * ESZ)
-        ga[q] = *reinterpret_cast<const uintx4*>(A + (size_t)m * p.K * ESZ + kbyte);
-      if (KIND == kFp8) {
-        const int n = n0 + row;
-        gb[q] = uintx4{0u, 0u, 0u, 0u};
-        if (n < p.N && kbyte < p.K) gb[q] = *reinterpret_cast<const uintx4*>(p.b + (size_t)n * p.K + kbyte);
-      }
-    }
-    if (KIND == kS8) {
-      const int kblk = tid >> 5, nq = tid & 31;  // 8 row blocks x 32 channel quads
-      const int n = n0 + nq * 4;
+    for (int it = 0; it < 2; ++it) {
+      const int item = tid + 256 * it, nq = item & 63, kblk = item >> 6;
+      const uint32_t col = (uint32_t)(n0 + nq * 4);
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
-        const int k = k0 + kblk * 8 + r;
-        uint32_t v = 0u;
-        if (k < p.K && n < p.N) v = *reinterpret_cast<const uint32_t*>(B + (size_t)k * p.N + n);
-        gb[r >> 2][r & 3] = v;
+        const uint32_t k = (uint32_t)(k0 + kblk * 8 + r);
+        uint32_t voff = k * (uint32_t)p.N + col;
+        if (col >= (uint32_t)p.N || k >= (uint32_t)p.K) voff = kOutOfRange;  // would alias other rows
+        wreg[it][r] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, 0, 0);
       }
     }
   };
-  auto lstore = [&](int buf) {
+  auto s8_store = [&](uint8_t* bt) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int c = tid + 256 * q, row = c >> 3, col = (c & 7) * 16;
-      *reinterpret_cast<uintx4*>(&lds_a[buf][row * kPitch + col]) = ga[q];
-      if (KIND == kFp8) *reinterpret_cast<uintx4*>(&lds_b[buf][row * kPitch + col]) = gb[q];
-    }
-    if (KIND == kS8) {
-      const int kblk = tid >> 5, nq = tid & 31;
+    for (int it = 0; it < 2; ++it) {
+      const int item = tid + 256 * it, nq = item & 63, kblk = item >> 6;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float f[8];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((gb[r >> 2][r & 3] >> (8 * e)) & 0xffu);
-        uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                    pack_bf16x2(f[6], f[7])};
-        *reinterpret_cast<uintx4*>(&lds_b[buf][(nq * 4 + e) * kPitch + kblk * 16]) = v;
+        for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((wreg[it][r] >> (8 * e)) & 0xffu);
+        const uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                          pack_bf16x2(f[6], f[7])};
+        const int n = nq * 4 + e;
+        *reinterpret_cast<uintx4*>(bt + n * kRow + ((kblk ^ (n & 7)) << 4)) = v;
       }
     }
   };
 
+  auto issue_loads = [&](int buf, int k0) {
+    uint8_t* at = lds + buf * kBufBytes;
+    uint8_t* bt = at + kTM * kRow;
+    const uint32_t kbyte = (uint32_t)k0 * ESZ;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool past_k = k_tail && kbyte + ld_chunk * 16 >= a_pitch;
+      load_to_lds(ra, at + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
+      if (KIND == kFp8)
+        load_to_lds(rb, bt + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
+    }
+    if (KIND == kS8) s8_load(k0);
+  };
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int y = 0; y < 4; ++y)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[x][y][v] = 0.0f;
+
   const int stages = (p.K + KS - 1) / KS;
-  gload(0);
-  lstore(0);
+  issue_loads(0, 0);
+  if (KIND == kS8) s8_store(lds + kTM * kRow);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+
+  // fragment addressing: row r of a tile, 16-byte chunk c -> r*128 + ((c ^ (r&7)) << 4)
+  const int frag_sw = l32 & 7;  // tile rows of a fragment start at multiples of 32
   for (int s = 0; s < stages; ++s) {
     const int buf = s & 1;
-    if (s + 1 < stages) gload((s + 1) * KS);
+    const uint8_t* at = lds + buf * kBufBytes + (wm * 128 + l32) * kRow;
+    const uint8_t* bt = lds + buf * kBufBytes + kTM * kRow + (wn * 128 + l32) * kRow;
+    if (s + 1 < stages) issue_loads(buf ^ 1, (s + 1) * KS);
     if (KIND == kFp8) {
-      intx8 fa[4], fb[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const uint8_t* ra = &lds_a[buf][(wm * 64 + t * 16 + li) * kPitch + kb * 32];
-        const uint8_t* rb = &lds_b[buf][(wn * 64 + t * 16 + li) * kPitch + kb * 32];
-        uintx4 a0 = *reinterpret_cast<const uintx4*>(ra), a1 = *reinterpret_cast<const uintx4*>(ra + 16);
-        uintx4 b0 = *reinterpret_cast<const uintx4*>(rb), b1 = *reinterpret_cast<const uintx4*>(rb + 16);
-        fa[t] = intx8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-        fb[t] = intx8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-      }
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[nt], fa[mt], acc[nt][mt],
-                                                                         0, 0, 0, 0, 0, 0);
-    } else {
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        bf16x8 fa[4], fb[4];
+        const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
+        intx8 fa[4], fb[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          fa[t] = *reinterpret_cast<const bf16x8*>(
-              &lds_a[buf][(wm * 64 + t * 16 + li) * kPitch + ks * 64 + kb * 16]);
-          fb[t] = *reinterpret_cast<const bf16x8*>(
-              &lds_b[buf][(wn * 64 + t * 16 + li) * kPitch + ks * 64 + kb * 16]);
+          const uintx4 a0 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c0);
+          const uintx4 a1 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c1);
+          const uintx4 b0 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c0);
+          const uintx4 b1 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c1);
+          fa[t] = intx8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+          fb[t] = intx8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
         }
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
           for (int mt = 0; mt < 4; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
+            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt],
+                                                                          0, 0, 0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int c = ((2 * ks + kb) ^ frag_sw) << 4;
+        bf16x8 fa[4], fb[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          fa[t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
+          fb[t] = *reinterpret_cast<const bf16x8*>(bt + t * 32 * kRow + c);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+            acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
       }
     }
-    if (s + 1 < stages) lstore(buf ^ 1);
+    if (KIND == kS8 && s + 1 < stages) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 
-  // ---- epilogue: lane (li, kb), register t of tile (nt, mt):
-  //      token m0 + wm*64 + mt*16 + li, channel n0 + wn*64 + nt*16 + 4*kb + t
   float alpha = 1.0f;
   if (KIND == kFp8) alpha = *p.a_scale * *p.b_scale;
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int m = m0 + wm * 64 + mt * 16 + li;
-    if (m >= p.M) continue;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int n = n0 + wn * 64 + nt * 16 + 4 * kb;
-      if (n >= p.N) continue;
-      float v[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        float x = acc[nt][mt][t];
-        if (KIND == kFp8) {
-          x = x * alpha;
-        } else {
-          const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + n + t;
-          x = (n + t < p.N) ? x * (p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si])
-                                                   : ((const float*)p.scales)[si])
-                            : 0.0f;
-        }
-        float bv = 0.0f;
-        if (p.bias && n + t < p.N)
-          bv = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n + t]) : ((const float*)p.bias)[n + t];
-        v[t] = epilogue_dispatch(x, bv, p.epilogue, p.bf16_dot, p.bf16_ops);
-      }
-      uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n;
-      if (n + 3 < p.N && (p.N & 3) == 0) {
-        uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<uintx2*>(dst) = o;
-      } else {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-          if (n + t < p.N) dst[t] = f32_to_bf16(v[t]);
-      }
-    }
+  // The common case (f32-typed dot and epilogue ops) gets one fully unrolled store routine per
+  // activation, so the 256 accumulators are read with static register indices; the bf16-typed
+  // op chains share one generic routine.
+  const int act = p.epilogue & ~1;
+  if (!p.bf16_dot && !p.bf16_ops) {
+    if (act == kEpiGelu) store_tile<KIND, kEpiGelu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
+    else if (act == kEpiSilu) store_tile<KIND, kEpiSilu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
+    else if (act == kEpiRelu) store_tile<KIND, kEpiRelu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
+    else store_tile<KIND, kEpiDefault>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
+  } else {
+    store_tile<KIND, -1>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
   }
 }
 
@@ -267,6 +355,23 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   p.out[idx] = f32_to_bf16(epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
+template <int KIND>
+int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
+  constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow;  // 128 KiB
+  static bool configured = false;  // per kernel instantiation; benign if two threads race
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+    if (e != hipSuccess)
+      return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", what, kLds,
+                  hipGetErrorString(e));
+    configured = true;
+  }
+  dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
+  hipLaunchKernelGGL(tiled_dot_kernel<KIND>, grid, dim3(256), kLds, stream, tp);
+  return CheckLaunch(what);
+}
+
 }  // namespace
 
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
@@ -276,6 +381,8 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
       p.dequant_type != XLA_FFI_DataType_F32)
     return -1;
   if (p.K % 8 != 0 || p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 4)) return -1;
+  // 32-bit buffer offsets per batch
+  if ((double)p.M * p.K * 2 >= 2147483000.0 || (double)p.K * p.N >= 2147483000.0) return -1;
   TiledParams tp{};
   tp.a = (const uint8_t*)p.lhs;
   tp.b = (const uint8_t*)p.weights;
@@ -291,10 +398,8 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.epilogue = p.epilogue;
   tp.tiles_m = (tp.M + kTM - 1) / kTM;
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
-  dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)p.batch);
-  hipLaunchKernelGGL(tiled_dot_kernel<kS8>, grid, dim3(256), 0, stream, tp);
   SetLastKernel("dequant_dot_tiled_s8_factored");
-  return CheckLaunch("dequant_dot_tiled_s8");
+  return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
 
 size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim) {
@@ -339,7 +444,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
 
   const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled
   const bool nk = p.rhs_contracting_dim == 1;
-  bool tiled_ok = p.K % 16 == 0 && p.K > 0 && ((uintptr_t)p.a % 16 == 0) && force != 1;
+  bool tiled_ok = p.K % 16 == 0 && p.K > 0 && ((uintptr_t)p.a % 16 == 0) && force != 1 &&
+                  (double)p.M * p.K < 2147483000.0 && (double)p.N * p.K < 2147483000.0;
   const uint8_t* b_nk = (const uint8_t*)p.b;
   if (tiled_ok && !nk) {
     if (p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
@@ -364,9 +470,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;
-    dim3 grid((unsigned)(tt.tiles_m * tt.tiles_n), 1);
-    hipLaunchKernelGGL(tiled_dot_kernel<kFp8>, grid, dim3(256), 0, stream, tt);
-    int rc = CheckLaunch("fp8_scaled_dot_tiled");
+    int rc = launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
     if (rc) return rc;
     if (deq_bf16) {
       // runs only if a scale is not a power of two (decided on the device, no host read)
