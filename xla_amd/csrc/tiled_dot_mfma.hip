@@ -72,60 +72,6 @@ __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t r, uint8_t* d
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(uintptr_t)dst, 16, voff, 0, 0, 0);
 }
 
-// Writes one wave's 128x128 quarter.  Register v of tile (nt, mt) in lane (l32, kb) is
-//   token   m_base + mt*32 + l32,   channel n_base + nt*32 + (v/4)*8 + kb*4 + v%4.
-// ACT >= 0: f32-typed ops with that activation (bias folded in as an add of 0 when absent);
-// ACT < 0: any typing, through epilogue_dispatch.
-template <int KIND, int ACT>
-__device__ __forceinline__ void store_tile(const TiledParams& p, const floatx16 (&acc)[4][4], float alpha,
-                                           int batch, int m_base, int n_base, int l32, int kb) {
-  const bool n_vec = (p.N & 3) == 0;
-#pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
-#pragma unroll
-    for (int vq = 0; vq < 4; ++vq) {
-      const int n = n_base + nt * 32 + vq * 8 + kb * 4;
-      float sc[4], bs[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const bool ok = n + t < p.N;
-        sc[t] = alpha;
-        if (KIND == kS8) {
-          const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
-          sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
-        }
-        bs[t] = 0.0f;
-        if (p.bias) {
-          const int bi = ok ? n + t : 0;
-          bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
-        }
-      }
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const int m = m_base + mt * 32 + l32;
-        float v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const float x = acc[nt][mt][vq * 4 + t] * sc[t];
-          if (ACT >= 0) v[t] = epilogue_value<false, false>(x, bs[t], ACT | 1);
-          else v[t] = epilogue_dispatch(x, bs[t], p.epilogue, p.bf16_dot, p.bf16_ops);
-        }
-        if (m < p.M && n < p.N) {
-          uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n;
-          if (n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
-            const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-            *reinterpret_cast<uintx2*>(dst) = o;
-          } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-              if (n + t < p.N) dst[t] = f32_to_bf16(v[t]);
-          }
-        }
-      }
-    }
-  }
-}
-
 template <int KIND>
 __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
   constexpr int ESZ = KIND == kFp8 ? 1 : 2;  // bytes per activation element
@@ -299,19 +245,71 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
     __syncthreads();
   }
 
+  // ---- epilogue, staged through LDS (free now: every wave passed the last barrier).
+  // Register v of tile (nt, mt) in lane (l32, kb) is token mt*32 + l32, channel
+  // nt*32 + (v/4)*8 + kb*4 + v%4 of the wave's 128x128 quarter.  Each wave owns 32 KiB of
+  // LDS and handles 64 channels per pass: it writes them as [128 tokens][16 chunks of 4 f32]
+  // (chunks XOR-swizzled by token), then reads the block back with 16 lanes per token row, so
+  // that a row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever
+  // indexed statically.  The rolled read loop carries the (runtime) epilogue.
   float alpha = 1.0f;
   if (KIND == kFp8) alpha = *p.a_scale * *p.b_scale;
-  // The common case (f32-typed dot and epilogue ops) gets one fully unrolled store routine per
-  // activation, so the 256 accumulators are read with static register indices; the bf16-typed
-  // op chains share one generic routine.
-  const int act = p.epilogue & ~1;
-  if (!p.bf16_dot && !p.bf16_ops) {
-    if (act == kEpiGelu) store_tile<KIND, kEpiGelu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
-    else if (act == kEpiSilu) store_tile<KIND, kEpiSilu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
-    else if (act == kEpiRelu) store_tile<KIND, kEpiRelu>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
-    else store_tile<KIND, kEpiDefault>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
-  } else {
-    store_tile<KIND, -1>(p, acc, alpha, batch, m0 + wm * 128, n0 + wn * 128, l32, kb);
+  float* stage = reinterpret_cast<float*>(lds + wave * 32768);
+  const int rd_chunk = lane & 15, rd_row = lane >> 4;  // read side: chunk of 4 channels, row within 4
+  const bool n_vec = (p.N & 3) == 0;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+    for (int ntl = 0; ntl < 2; ++ntl) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        const int m = mt * 32 + l32;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int c = ntl * 8 + vq * 2 + kb;
+          const floatx16& a = acc[pass * 2 + ntl][mt];
+          const floatx4 v = {a[vq * 4], a[vq * 4 + 1], a[vq * 4 + 2], a[vq * 4 + 3]};
+          *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
+        }
+      }
+    }
+    // channels of this lane on the read side: fixed for the whole pass
+    const int n = n0 + wn * 128 + pass * 64 + rd_chunk * 4;
+    float sc[4], bs[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bool ok = n + t < p.N;
+      sc[t] = alpha;
+      if (KIND == kS8) {
+        const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
+        sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
+      }
+      bs[t] = 0.0f;
+      if (p.bias) {
+        const int bi = ok ? n + t : 0;
+        bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
+      }
+    }
+    for (int it = 0; it < 32; ++it) {
+      const int ml = it * 4 + rd_row;
+      const floatx4 x = *reinterpret_cast<const floatx4*>(stage + ml * 64 + ((rd_chunk ^ (ml & 15)) << 2));
+      float v[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        v[t] = epilogue_dispatch(x[t] * sc[t], bs[t], p.epilogue, p.bf16_dot, p.bf16_ops);
+      const int m = m0 + wm * 128 + ml;
+      if (m < p.M && n < p.N) {
+        uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n;
+        if (n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
+          const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          *reinterpret_cast<uintx2*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (n + t < p.N) dst[t] = f32_to_bf16(v[t]);
+        }
+      }
+    }
   }
 }
 
