@@ -125,17 +125,27 @@ enum : int { kEpiDefault = 0, kEpiBias = 1, kEpiRelu = 2, kEpiBiasRelu = 3, kEpi
 // FloatNormalization makes of them, xla/service/cpu/cpu_compiler.cc:804-817);
 // otherwise they run in f32 and only the final convert rounds.  GELU op order:
 // gemm_rewriter_fp8_test.cc:1123-1141; SiLU: gemm_rewriter.cc:995-1002.
+// The dot result as the epilogue sees it: rounded to the dot's type, then (optionally) the
+// bias add in the epilogue's type.
 template <bool BF16_DOT, bool BF16_OPS>
-__device__ __forceinline__ float epilogue_value(float acc, float bias, int epi) {
+__device__ __forceinline__ float epilogue_pre(float acc, float bias, bool has_bias) {
   auto R = [](float v) { return BF16_OPS ? round_bf16(v) : v; };
   float x = BF16_DOT ? round_bf16(acc) : acc;
   x = R(x);
-  if (epi & 1) x = R(x + R(bias));
-  switch (epi & ~1) {
-    case kEpiRelu:
+  const float xb = R(x + R(bias));
+  return has_bias ? xb : x;
+}
+
+// The activation, every op rounded to the epilogue's type.  `act` is one of 0, kEpiRelu,
+// kEpiGelu, kEpiSilu (2, 4, 6).
+template <bool BF16_OPS>
+__device__ __forceinline__ float epilogue_act(float x, int act) {
+  auto R = [](float v) { return BF16_OPS ? round_bf16(v) : v; };
+  switch (act) {
+    case 2:  // relu; NaN passes through
       x = x > 0.0f ? x : (x != x ? x : 0.0f);
       break;
-    case kEpiGelu: {
+    case 4: {  // tanh-approximated gelu
       float m0 = R(x * x);
       float m1 = R(x * m0);
       float m2 = R(m1 * R(0.044715f));
@@ -147,7 +157,7 @@ __device__ __forceinline__ float epilogue_value(float acc, float bias, int epi) 
       x = R(x * m4);
       break;
     }
-    case kEpiSilu: {
+    case 6: {  // silu
       float ex = R(exp_xla(-x));
       float dn = R(1.0f + ex);
       float sg = R(1.0f / dn);
@@ -158,6 +168,11 @@ __device__ __forceinline__ float epilogue_value(float acc, float bias, int epi) 
       break;
   }
   return x;
+}
+
+template <bool BF16_DOT, bool BF16_OPS>
+__device__ __forceinline__ float epilogue_value(float acc, float bias, int epi) {
+  return epilogue_act<BF16_OPS>(epilogue_pre<BF16_DOT, BF16_OPS>(acc, bias, (epi & 1) != 0), epi & ~1);
 }
 
 __device__ __forceinline__ float epilogue_dispatch(float acc, float bias, int epi, bool bf16_dot,

@@ -25,6 +25,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "device_numerics.h"
 #include "launch.h"
 
@@ -70,6 +72,61 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 constexpr uint32_t kOutOfRange = 0x80000000u;  // every buffer here is smaller than 2 GiB
 __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t r, uint8_t* dst, uint32_t voff) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(uintptr_t)dst, 16, voff, 0, 0, 0);
+}
+
+// Read side of the staged epilogue: 32 iterations of one ds_read_b128, four epilogue values
+// and an 8-byte store per lane.  The activation and the two rounding modes are template
+// parameters, so the loop body is branch-free; the variant is picked once per pass.
+struct DrainArgs {
+  const float* stage;
+  int rd_chunk, rd_row, m_base, n, M, N;
+  uint16_t* out;  // start of this batch's [M,N] block
+  bool n_vec, has_bias;
+  float sc[4], bs[4];
+};
+
+template <bool BF16_DOT, bool BF16_OPS, int ACT>
+__device__ __forceinline__ void drain_rows(const DrainArgs& d) {
+#pragma unroll 4
+  for (int it = 0; it < 32; ++it) {
+    const int ml = it * 4 + d.rd_row;
+    const floatx4 x = *reinterpret_cast<const floatx4*>(d.stage + ml * 64 + ((d.rd_chunk ^ (ml & 15)) << 2));
+    float v[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      v[t] = epilogue_act<BF16_OPS>(epilogue_pre<BF16_DOT, BF16_OPS>(x[t] * d.sc[t], d.bs[t], d.has_bias), ACT);
+    }
+    const int m = d.m_base + ml;
+    if (m < d.M && d.n < d.N) {
+      uint16_t* dst = d.out + (size_t)m * d.N + d.n;
+      if (d.n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
+        const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        *reinterpret_cast<uintx2*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (d.n + t < d.N) dst[t] = f32_to_bf16(v[t]);
+      }
+    }
+  }
+}
+
+template <bool BF16_DOT, bool BF16_OPS>
+__device__ __forceinline__ void drain_act(const DrainArgs& d, int act) {
+  switch (act) {
+    case kEpiRelu: drain_rows<BF16_DOT, BF16_OPS, kEpiRelu>(d); break;
+    case kEpiGelu: drain_rows<BF16_DOT, BF16_OPS, kEpiGelu>(d); break;
+    case kEpiSilu: drain_rows<BF16_DOT, BF16_OPS, kEpiSilu>(d); break;
+    default: drain_rows<BF16_DOT, BF16_OPS, 0>(d); break;
+  }
+}
+
+__device__ __forceinline__ void drain_dispatch(const DrainArgs& d, int act, bool bf16_dot, bool bf16_ops) {
+  if (bf16_ops) {
+    if (bf16_dot) drain_act<true, true>(d, act); else drain_act<false, true>(d, act);
+  } else {
+    if (bf16_dot) drain_act<true, false>(d, act); else drain_act<false, false>(d, act);
+  }
 }
 
 template <int KIND>
@@ -189,61 +246,77 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[x][y][v] = 0.0f;
 
+  // ---- main loop.  A stage is NKS MFMA steps.  Fragments are double-buffered in registers:
+  // the LDS reads of step i+1 are issued before the 16 MFMAs of step i, so the matrix cores
+  // run while the next operands arrive.  Once per stage, before the MFMAs of the stage's last
+  // step, the workgroup synchronises: every wave's reads of the stage buffer are complete (so
+  // it may be refilled) and the next stage's tiles have landed (so its first fragments may be
+  // read).  The refill for stage s+2 is issued right after that point.
+  constexpr int NKS = KIND == kFp8 ? 2 : 4;
+  const int frag_sw = l32 & 7;  // tile rows of a fragment start at multiples of 32
+  const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 128 + l32) * kRow;
+  typedef typename std::conditional<KIND == kFp8, intx8, bf16x8>::type frag_t;
+  frag_t fa[2][4], fb[2][4];
+  auto read_frags = [&](int set, int buf, int ks) {
+    const uint8_t* at = lds + buf * kBufBytes + row_a;
+    const uint8_t* bt = lds + buf * kBufBytes + row_b;
+    if constexpr (KIND == kFp8) {
+      const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uintx4 a0 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c0);
+        const uintx4 a1 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c1);
+        const uintx4 b0 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c0);
+        const uintx4 b1 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c1);
+        fa[set][t] = intx8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+        fb[set][t] = intx8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+      }
+    } else {
+      const int c = ((2 * ks + kb) ^ frag_sw) << 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        fa[set][t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
+        fb[set][t] = *reinterpret_cast<const bf16x8*>(bt + t * 32 * kRow + c);
+      }
+    }
+  };
+  auto mfma_all = [&](int set) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        if constexpr (KIND == kFp8)
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[set][nt], fa[set][mt], acc[nt][mt],
+                                                                        0, 0, 0, 0, 0, 0);
+        else
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][nt], fa[set][mt], acc[nt][mt], 0, 0, 0);
+      }
+  };
+
   const int stages = (p.K + KS - 1) / KS;
   issue_loads(0, 0);
   if (KIND == kS8) s8_store(lds + kTM * kRow);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
-
-  // fragment addressing: row r of a tile, 16-byte chunk c -> r*128 + ((c ^ (r&7)) << 4)
-  const int frag_sw = l32 & 7;  // tile rows of a fragment start at multiples of 32
+  if (stages > 1) issue_loads(1, KS);
+  read_frags(0, 0, 0);
   for (int s = 0; s < stages; ++s) {
     const int buf = s & 1;
-    const uint8_t* at = lds + buf * kBufBytes + (wm * 128 + l32) * kRow;
-    const uint8_t* bt = lds + buf * kBufBytes + kTM * kRow + (wn * 128 + l32) * kRow;
-    if (s + 1 < stages) issue_loads(buf ^ 1, (s + 1) * KS);
-    if (KIND == kFp8) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
-        intx8 fa[4], fb[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const uintx4 a0 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c0);
-          const uintx4 a1 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c1);
-          const uintx4 b0 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c0);
-          const uintx4 b1 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c1);
-          fa[t] = intx8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-          fb[t] = intx8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-        }
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-          for (int mt = 0; mt < 4; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt],
-                                                                          0, 0, 0, 0, 0, 0);
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + 1 < NKS) {
+        read_frags((ks + 1) & 1, buf, ks + 1);
+      } else if (s + 1 < stages) {
+        if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        read_frags(0, buf ^ 1, 0);
+        if (s + 2 < stages) issue_loads(buf, (s + 2) * KS);
       }
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int c = ((2 * ks + kb) ^ frag_sw) << 4;
-        bf16x8 fa[4], fb[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          fa[t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
-          fb[t] = *reinterpret_cast<const bf16x8*>(bt + t * 32 * kRow + c);
-        }
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-          for (int mt = 0; mt < 4; ++mt)
-            acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
-      }
+      mfma_all(ks & 1);
     }
-    if (KIND == kS8 && s + 1 < stages) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
   }
+  __syncthreads();  // the epilogue reuses the stage buffers
 
   // ---- epilogue, staged through LDS (free now: every wave passed the last barrier).
   // Register v of tile (nt, mt) in lane (l32, kb) is token mt*32 + l32, channel
@@ -290,26 +363,20 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
         bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
       }
     }
-    for (int it = 0; it < 32; ++it) {
-      const int ml = it * 4 + rd_row;
-      const floatx4 x = *reinterpret_cast<const floatx4*>(stage + ml * 64 + ((rd_chunk ^ (ml & 15)) << 2));
-      float v[4];
+    DrainArgs d;
+    d.stage = stage;
+    d.rd_chunk = rd_chunk;
+    d.rd_row = rd_row;
+    d.m_base = m0 + wm * 128;
+    d.n = n;
+    d.M = p.M;
+    d.N = p.N;
+    d.out = p.out + (size_t)batch * p.M * p.N;
+    d.n_vec = n_vec;
+    d.has_bias = p.bias != nullptr;
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
-        v[t] = epilogue_dispatch(x[t] * sc[t], bs[t], p.epilogue, p.bf16_dot, p.bf16_ops);
-      const int m = m0 + wm * 128 + ml;
-      if (m < p.M && n < p.N) {
-        uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n;
-        if (n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
-          const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          *reinterpret_cast<uintx2*>(dst) = o;
-        } else {
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-            if (n + t < p.N) dst[t] = f32_to_bf16(v[t]);
-        }
-      }
-    }
+    for (int t = 0; t < 4; ++t) d.sc[t] = sc[t], d.bs[t] = bs[t];
+    drain_dispatch(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops);
   }
 }
 
