@@ -178,18 +178,20 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
                    : tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
 
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
-  // of row l/8 with global chunk (l%8) ^ (row & 7).  Wave w owns rows [w*64, w*64+64) of a
+  // of row l/8 with global chunk (l%8) ^ ((row >> 1) & 7): any 16 consecutive rows then cover all 64
+  // banks with one 16-byte chunk each, which is what ds_read_b128 needs for its full rate (the
+  // hardware serves 16 lanes per clock).  Wave w owns rows [w*64, w*64+64) of a
   // 256-row tile: 8 instructions per tile per stage.
   const int ld_row = lane >> 3;                       // 0..7 within an instruction
-  const int ld_chunk = (lane & 7) ^ (ld_row & 7);     // rows start at multiples of 8, so row&7 == ld_row
+  // rows of instruction j start at a multiple of 8: (row >> 1) & 7 == 4 * (j & 1) + ld_row / 2
+  const int ld_chunk[2] = {(lane & 7) ^ (ld_row >> 1), (lane & 7) ^ (4 + (ld_row >> 1))};
   uint32_t voff_a[8], voff_b[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int r = wave * 64 + j * 8 + ld_row;
-    voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk * 16;
-    if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk * 16;
+    voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk[j & 1] * 16;
+    if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
   }
-  const bool k_tail = (a_pitch % kRow) != 0;  // last stage is partial: chunks past K must read as 0
 
   // ---- s8 weights: item = (8-row block kblk, 4-channel quad nq); 512 items, 2 per thread
   uint32_t wreg[2][8];
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
         const uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
                           pack_bf16x2(f[6], f[7])};
         const int n = nq * 4 + e;
-        *reinterpret_cast<uintx4*>(bt + n * kRow + ((kblk ^ (n & 7)) << 4)) = v;
+        *reinterpret_cast<uintx4*>(bt + n * kRow + ((kblk ^ ((n >> 1) & 7)) << 4)) = v;
       }
     }
   };
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
     const uint32_t kbyte = (uint32_t)k0 * ESZ;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const bool past_k = k_tail && kbyte + ld_chunk * 16 >= a_pitch;
+      const bool past_k = kbyte + ld_chunk[j & 1] * 16 >= a_pitch;
       load_to_lds(ra, at + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
       if (KIND == kFp8)
         load_to_lds(rb, bt + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
   // it may be refilled) and the next stage's tiles have landed (so its first fragments may be
   // read).  The refill for stage s+2 is issued right after that point.
   constexpr int NKS = KIND == kFp8 ? 2 : 4;
-  const int frag_sw = l32 & 7;  // tile rows of a fragment start at multiples of 32
+  const int frag_sw = (l32 >> 1) & 7;  // tile rows of a fragment start at multiples of 32
   const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 128 + l32) * kRow;
   typedef typename std::conditional<KIND == kFp8, intx8, bf16x8>::type frag_t;
   frag_t fa[2][4], fb[2][4];
@@ -293,26 +295,46 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
       }
   };
 
+  // Instruction order inside a step: the scheduler is asked to put one LDS read (and, in the
+  // refill step, one global->LDS load) behind every MFMA, so that the matrix pipe starts at
+  // once after a barrier and the LDS / memory pipes are fed evenly instead of in bursts.
+  auto interleave = [&](bool with_loads) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);               // one ds_read
+      if (with_loads) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+    }
+  };
+
   const int stages = (p.K + KS - 1) / KS;
   issue_loads(0, 0);
   if (KIND == kS8) s8_store(lds + kTM * kRow);
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
-  if (stages > 1) issue_loads(1, KS);
+  issue_loads(1, KS);  // past K: lands as zeros, never read
   read_frags(0, 0, 0);
-  for (int s = 0; s < stages; ++s) {
+  for (int s = 0; s + 1 < stages; ++s) {
     const int buf = s & 1;
 #pragma unroll
+    for (int ks = 0; ks + 1 < NKS; ++ks) {
+      read_frags((ks + 1) & 1, buf, ks + 1);
+      mfma_all(ks & 1);
+      if (KIND == kFp8) interleave(false);
+    }
+    if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    read_frags(0, buf ^ 1, 0);
+    issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
+    mfma_all((NKS - 1) & 1);
+    if (KIND == kFp8) interleave(true);
+  }
+  {  // last stage: nothing left to fetch
+    const int buf = (stages - 1) & 1;
+#pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      if (ks + 1 < NKS) {
-        read_frags((ks + 1) & 1, buf, ks + 1);
-      } else if (s + 1 < stages) {
-        if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-        read_frags(0, buf ^ 1, 0);
-        if (s + 2 < stages) issue_loads(buf, (s + 2) * KS);
-      }
+      if (ks + 1 < NKS) read_frags((ks + 1) & 1, buf, ks + 1);
       mfma_all(ks & 1);
     }
   }
