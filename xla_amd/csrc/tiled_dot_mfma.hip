@@ -3,11 +3,11 @@
 //   kFp8 : out[m,n] = epi( a_scale*b_scale * sum_k A8[m,k] * B8[n,k] )   f8e4m3fn x f8e4m3fn
 //   kS8  : out[b,m,n] = epi( scale[b,n] * sum_k A[b,m,k] * W[b,k,n] )    bf16 x s8 (per channel)
 //
-// A workgroup of 4 waves (2x2) owns a 256x256 output tile, each wave a 128x128 quarter held
-// in 256 accumulator registers, and walks K in stages of 128 bytes per activation row (128
-// fp8 or 64 bf16 values).  Both operand tiles of a stage sit in LDS with the contracting
+// A workgroup of 8 waves (2x4, two per SIMD) owns a 256x256 output tile, each wave a 128x64
+// part held in 128 accumulator registers, and walks K in stages of 128 bytes per activation
+// row (128 fp8 or 64 bf16 values).  Both operand tiles of a stage sit in LDS with the contracting
 // dimension contiguous (128-byte rows, 16-byte chunks XOR-swizzled by row so that the
-// 128-bit fragment reads of 8 consecutive rows hit 8 different bank groups).  The
+// 128-bit fragment reads of 16 consecutive rows cover all 64 banks once).  The
 // activation tile -- and the fp8 weight tile, stored [N,K] -- go from global memory
 // straight into LDS (buffer_load ... lds: no staging registers, out-of-range rows arrive as
 // zeros); the swizzle is applied by permuting which global chunk each lane fetches.  The s8
@@ -74,7 +74,7 @@ __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t r, uint8_t* d
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(uintptr_t)dst, 16, voff, 0, 0, 0);
 }
 
-// Read side of the staged epilogue: 32 iterations of one ds_read_b128, four epilogue values
+// Read side of the staged epilogue: 16 iterations of one ds_read_b128, four epilogue values
 // and an 8-byte store per lane.  The activation and the two rounding modes are template
 // parameters, so the loop body is branch-free; the variant is picked once per pass.
 struct DrainArgs {
@@ -88,7 +88,7 @@ struct DrainArgs {
 template <bool BF16_DOT, bool BF16_OPS, int ACT>
 __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
 #pragma unroll 4
-  for (int it = 0; it < 32; ++it) {
+  for (int it = 0; it < 16; ++it) {
     const int ml = it * 4 + d.rd_row;
     const floatx4 x = *reinterpret_cast<const floatx4*>(d.stage + ml * 64 + ((d.rd_chunk ^ (ml & 15)) << 2));
     float v[4];
@@ -130,7 +130,7 @@ __device__ __forceinline__ void drain_dispatch(const DrainArgs& d, int act, bool
 }
 
 template <int KIND>
-__global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
+__global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr int ESZ = KIND == kFp8 ? 1 : 2;  // bytes per activation element
   constexpr int KS = kRow / ESZ;             // K elements per stage
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [2][(kTM + kTN) * kRow]
@@ -141,9 +141,9 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
   }
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..7, two per SIMD
   const int l32 = lane & 31, kb = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;  // wave tile: tokens [wm*128,+128) x channels [wn*64,+64)
 
   // Workgroup id -> tile: consecutive ids of one XCD take 8 neighbouring channel tiles of one
   // token tile, then the next token tile, so a token tile and 8 weight tiles stay hot in L2.
@@ -178,51 +178,44 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
                    : tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
 
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
-  // of row l/8 with global chunk (l%8) ^ ((row >> 1) & 7): any 16 consecutive rows then cover all 64
-  // banks with one 16-byte chunk each, which is what ds_read_b128 needs for its full rate (the
-  // hardware serves 16 lanes per clock).  Wave w owns rows [w*64, w*64+64) of a
-  // 256-row tile: 8 instructions per tile per stage.
+  // of row l/8 with global chunk (l%8) ^ ((row >> 1) & 7): any 16 consecutive rows then cover
+  // all 64 banks with one 16-byte chunk each, which is what ds_read_b128 needs for its full
+  // rate (the hardware serves 16 lanes per clock).  Wave w owns rows [w*32, w*32+32) of a
+  // 256-row tile: 4 instructions per tile per stage.
   const int ld_row = lane >> 3;                       // 0..7 within an instruction
   // rows of instruction j start at a multiple of 8: (row >> 1) & 7 == 4 * (j & 1) + ld_row / 2
   const int ld_chunk[2] = {(lane & 7) ^ (ld_row >> 1), (lane & 7) ^ (4 + (ld_row >> 1))};
-  uint32_t voff_a[8], voff_b[8];
+  uint32_t voff_a[4], voff_b[4];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int r = wave * 64 + j * 8 + ld_row;
+  for (int j = 0; j < 4; ++j) {
+    const int r = wave * 32 + j * 8 + ld_row;
     voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk[j & 1] * 16;
     if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
   }
 
-  // ---- s8 weights: item = (8-row block kblk, 4-channel quad nq); 512 items, 2 per thread
-  uint32_t wreg[2][8];
+  // ---- s8 weights: a thread takes 4 channels (quad nq) of the 8 rows of block kblk
+  uint32_t wreg[8];
+  const int w_nq = tid & 63, w_kblk = tid >> 6;
   auto s8_load = [&](int k0) {
+    const uint32_t col = (uint32_t)(n0 + w_nq * 4);
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int item = tid + 256 * it, nq = item & 63, kblk = item >> 6;
-      const uint32_t col = (uint32_t)(n0 + nq * 4);
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const uint32_t k = (uint32_t)(k0 + kblk * 8 + r);
-        uint32_t voff = k * (uint32_t)p.N + col;
-        if (col >= (uint32_t)p.N || k >= (uint32_t)p.K) voff = kOutOfRange;  // would alias other rows
-        wreg[it][r] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, 0, 0);
-      }
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t k = (uint32_t)(k0 + w_kblk * 8 + r);
+      uint32_t voff = k * (uint32_t)p.N + col;
+      if (col >= (uint32_t)p.N || k >= (uint32_t)p.K) voff = kOutOfRange;  // would alias other rows
+      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, 0, 0);
     }
   };
   auto s8_store = [&](uint8_t* bt) {
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-      const int item = tid + 256 * it, nq = item & 63, kblk = item >> 6;
+    for (int e = 0; e < 4; ++e) {
+      float f[8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float f[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((wreg[it][r] >> (8 * e)) & 0xffu);
-        const uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                          pack_bf16x2(f[6], f[7])};
-        const int n = nq * 4 + e;
-        *reinterpret_cast<uintx4*>(bt + n * kRow + ((kblk ^ ((n >> 1) & 7)) << 4)) = v;
-      }
+      for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((wreg[r] >> (8 * e)) & 0xffu);
+      const uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                        pack_bf16x2(f[6], f[7])};
+      const int n = w_nq * 4 + e;
+      *reinterpret_cast<uintx4*>(bt + n * kRow + ((w_kblk ^ ((n >> 1) & 7)) << 4)) = v;
     }
   };
 
@@ -231,80 +224,69 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
     uint8_t* bt = at + kTM * kRow;
     const uint32_t kbyte = (uint32_t)k0 * ESZ;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const bool past_k = kbyte + ld_chunk[j & 1] * 16 >= a_pitch;
-      load_to_lds(ra, at + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
+    for (int j = 0; j < 4; ++j) {
+      const bool past_k = kbyte + ld_chunk[j & 1] * 16 >= a_pitch;  // chunks past K must read as 0
+      load_to_lds(ra, at + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
       if (KIND == kFp8)
-        load_to_lds(rb, bt + (wave * 64 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
+        load_to_lds(rb, bt + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
     }
     if (KIND == kS8) s8_load(k0);
   };
 
-  floatx16 acc[4][4];
+  floatx16 acc[2][4];
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+  for (int x = 0; x < 2; ++x)
 #pragma unroll
     for (int y = 0; y < 4; ++y)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[x][y][v] = 0.0f;
 
-  // ---- main loop.  A stage is NKS MFMA steps.  Fragments are double-buffered in registers:
-  // the LDS reads of step i+1 are issued before the 16 MFMAs of step i, so the matrix cores
-  // run while the next operands arrive.  Once per stage, before the MFMAs of the stage's last
-  // step, the workgroup synchronises: every wave's reads of the stage buffer are complete (so
-  // it may be refilled) and the next stage's tiles have landed (so its first fragments may be
-  // read).  The refill for stage s+2 is issued right after that point.
+  // ---- main loop.  A stage is NKS MFMA steps of 8 MFMAs per wave; a step reads its six
+  // fragments (4 token tiles, 2 channel tiles) and multiplies.  Nothing is software-pipelined
+  // inside a wave: the two waves of a SIMD alternate, one multiplying while the other's LDS
+  // reads are in flight.  Once per stage, between the reads and the MFMAs of its last step,
+  // the workgroup synchronises: every wave's reads of the stage buffer are complete (so it
+  // may be refilled) and the next stage's tiles have landed.  The refill for stage s+2 is
+  // issued right behind that barrier, interleaved with the MFMAs.
   constexpr int NKS = KIND == kFp8 ? 2 : 4;
   const int frag_sw = (l32 >> 1) & 7;  // tile rows of a fragment start at multiples of 32
-  const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 128 + l32) * kRow;
+  const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 64 + l32) * kRow;
   typedef typename std::conditional<KIND == kFp8, intx8, bf16x8>::type frag_t;
-  frag_t fa[2][4], fb[2][4];
-  auto read_frags = [&](int set, int buf, int ks) {
+  frag_t fa[4], fb[2];
+  auto read_frags = [&](int buf, int ks) {
     const uint8_t* at = lds + buf * kBufBytes + row_a;
     const uint8_t* bt = lds + buf * kBufBytes + row_b;
     if constexpr (KIND == kFp8) {
       const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
+      auto rd = [&](const uint8_t* base) {
+        const uintx4 x0 = *reinterpret_cast<const uintx4*>(base + c0);
+        const uintx4 x1 = *reinterpret_cast<const uintx4*>(base + c1);
+        return intx8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+      };
+      fb[0] = rd(bt);
+      fa[0] = rd(at);
+      fb[1] = rd(bt + 32 * kRow);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const uintx4 a0 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c0);
-        const uintx4 a1 = *reinterpret_cast<const uintx4*>(at + t * 32 * kRow + c1);
-        const uintx4 b0 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c0);
-        const uintx4 b1 = *reinterpret_cast<const uintx4*>(bt + t * 32 * kRow + c1);
-        fa[set][t] = intx8{(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-        fb[set][t] = intx8{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-      }
+      for (int t = 1; t < 4; ++t) fa[t] = rd(at + t * 32 * kRow);
     } else {
       const int c = ((2 * ks + kb) ^ frag_sw) << 4;
+      fb[0] = *reinterpret_cast<const bf16x8*>(bt + c);
+      fa[0] = *reinterpret_cast<const bf16x8*>(at + c);
+      fb[1] = *reinterpret_cast<const bf16x8*>(bt + 32 * kRow + c);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        fa[set][t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
-        fb[set][t] = *reinterpret_cast<const bf16x8*>(bt + t * 32 * kRow + c);
-      }
+      for (int t = 1; t < 4; ++t) fa[t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
     }
   };
-  auto mfma_all = [&](int set) {
+  auto mfma_all = [&]() {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
+      for (int nt = 0; nt < 2; ++nt) {
         if constexpr (KIND == kFp8)
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[set][nt], fa[set][mt], acc[nt][mt],
-                                                                        0, 0, 0, 0, 0, 0);
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, 0, 0, 0);
         else
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][nt], fa[set][mt], acc[nt][mt], 0, 0, 0);
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
       }
-  };
-
-  // Instruction order inside a step: the scheduler is asked to put one LDS read (and, in the
-  // refill step, one global->LDS load) behind every MFMA, so that the matrix pipe starts at
-  // once after a barrier and the LDS / memory pipes are fed evenly instead of in bursts.
-  auto interleave = [&](bool with_loads) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);               // one ds_read
-      if (with_loads) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
-    }
   };
 
   const int stages = (p.K + KS - 1) / KS;
@@ -313,91 +295,92 @@ __global__ __launch_bounds__(256) void tiled_dot_kernel(TiledParams p) {
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
   issue_loads(1, KS);  // past K: lands as zeros, never read
-  read_frags(0, 0, 0);
   for (int s = 0; s + 1 < stages; ++s) {
     const int buf = s & 1;
 #pragma unroll
     for (int ks = 0; ks + 1 < NKS; ++ks) {
-      read_frags((ks + 1) & 1, buf, ks + 1);
-      mfma_all(ks & 1);
-      if (KIND == kFp8) interleave(false);
+      read_frags(buf, ks);
+      mfma_all();
     }
+    read_frags(buf, NKS - 1);
     if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    read_frags(0, buf ^ 1, 0);
     issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
-    mfma_all((NKS - 1) & 1);
-    if (KIND == kFp8) interleave(true);
+    mfma_all();
+    if (KIND == kFp8) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+      }
+    }
   }
   {  // last stage: nothing left to fetch
     const int buf = (stages - 1) & 1;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      if (ks + 1 < NKS) read_frags((ks + 1) & 1, buf, ks + 1);
-      mfma_all(ks & 1);
+      read_frags(buf, ks);
+      mfma_all();
     }
   }
   __syncthreads();  // the epilogue reuses the stage buffers
 
   // ---- epilogue, staged through LDS (free now: every wave passed the last barrier).
   // Register v of tile (nt, mt) in lane (l32, kb) is token mt*32 + l32, channel
-  // nt*32 + (v/4)*8 + kb*4 + v%4 of the wave's 128x128 quarter.  Each wave owns 32 KiB of
-  // LDS and handles 64 channels per pass: it writes them as [128 tokens][16 chunks of 4 f32]
-  // (chunks XOR-swizzled by token), then reads the block back with 16 lanes per token row, so
-  // that a row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever
-  // indexed statically.  The rolled read loop carries the (runtime) epilogue.
+  // nt*32 + (v/4)*8 + kb*4 + v%4 of the wave's 128x64 tile.  Each wave owns 16 KiB of LDS and
+  // handles 64 tokens per pass: it writes them as [64 tokens][16 chunks of 4 f32] (chunks
+  // XOR-swizzled by token), then reads the block back with 16 lanes per token row, so that a
+  // row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever indexed
+  // statically.  The rolled read loop carries the epilogue.
   float alpha = 1.0f;
   if (KIND == kFp8) alpha = *p.a_scale * *p.b_scale;
-  float* stage = reinterpret_cast<float*>(lds + wave * 32768);
+  float* stage = reinterpret_cast<float*>(lds + wave * 16384);
   const int rd_chunk = lane & 15, rd_row = lane >> 4;  // read side: chunk of 4 channels, row within 4
   const bool n_vec = (p.N & 3) == 0;
+  // channels of this lane on the read side: the same in both passes
+  const int n = n0 + wn * 64 + rd_chunk * 4;
+  DrainArgs d;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const bool ok = n + t < p.N;
+    d.sc[t] = alpha;
+    if (KIND == kS8) {
+      const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
+      d.sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
+    }
+    d.bs[t] = 0.0f;
+    if (p.bias) {
+      const int bi = ok ? n + t : 0;
+      d.bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
+    }
+  }
+  d.stage = stage;
+  d.rd_chunk = rd_chunk;
+  d.rd_row = rd_row;
+  d.n = n;
+  d.M = p.M;
+  d.N = p.N;
+  d.out = p.out + (size_t)batch * p.M * p.N;
+  d.n_vec = n_vec;
+  d.has_bias = p.bias != nullptr;
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
-    for (int ntl = 0; ntl < 2; ++ntl) {
+    for (int mtl = 0; mtl < 2; ++mtl) {
+      const int m = mtl * 32 + l32;
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const int m = mt * 32 + l32;
+      for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq) {
-          const int c = ntl * 8 + vq * 2 + kb;
-          const floatx16& a = acc[pass * 2 + ntl][mt];
+          const int c = nt * 8 + vq * 2 + kb;
+          const floatx16& a = acc[nt][pass * 2 + mtl];
           const floatx4 v = {a[vq * 4], a[vq * 4 + 1], a[vq * 4 + 2], a[vq * 4 + 3]};
           *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
         }
       }
     }
-    // channels of this lane on the read side: fixed for the whole pass
-    const int n = n0 + wn * 128 + pass * 64 + rd_chunk * 4;
-    float sc[4], bs[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const bool ok = n + t < p.N;
-      sc[t] = alpha;
-      if (KIND == kS8) {
-        const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
-        sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
-      }
-      bs[t] = 0.0f;
-      if (p.bias) {
-        const int bi = ok ? n + t : 0;
-        bs[t] = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[bi]) : ((const float*)p.bias)[bi];
-      }
-    }
-    DrainArgs d;
-    d.stage = stage;
-    d.rd_chunk = rd_chunk;
-    d.rd_row = rd_row;
-    d.m_base = m0 + wm * 128;
-    d.n = n;
-    d.M = p.M;
-    d.N = p.N;
-    d.out = p.out + (size_t)batch * p.M * p.N;
-    d.n_vec = n_vec;
-    d.has_bias = p.bias != nullptr;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) d.sc[t] = sc[t], d.bs[t] = bs[t];
+    d.m_base = m0 + wm * 128 + pass * 64;
     drain_dispatch(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops);
   }
 }
@@ -455,7 +438,7 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
     configured = true;
   }
   dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
-  hipLaunchKernelGGL(tiled_dot_kernel<KIND>, grid, dim3(256), kLds, stream, tp);
+  hipLaunchKernelGGL(tiled_dot_kernel<KIND>, grid, dim3(512), kLds, stream, tp);
   return CheckLaunch(what);
 }
 
