@@ -139,26 +139,35 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   const int k_begin = slice * p.rows_per_slice + wave * rows_per_wave;
   const int k_stop = k_begin + rows_per_wave;           // may run past K: those rows load zeros
 
-  float sc[NV];  // kRounded: scale (x16 for s4) of each owned channel, for the current group
-  auto load_scales = [&](int k0) {
-    uint32_t raw[NV * SSZ / 4];
-    if (GROUP32) {
-      const uint32_t g = (uint32_t)min(k0, p.K - 1) / (uint32_t)p.group;  // scalar
-      buffer_load_words<NV * SSZ / 4>(rs, voff_s, g * (uint32_t)p.N * SSZ, raw);
-    } else {
-      const uint32_t g = (uint32_t)min(k0 + 8 * kb, p.K - 1) / (uint32_t)p.group;  // per lane
-      buffer_load_words<NV * SSZ / 4>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, raw);
-    }
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      float v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
-                           : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
-      sc[j] = WBITS == 4 ? v * 16.0f : v;  // the s4 convert yields value/16
-    }
-  };
-
+  // ---- software pipeline: everything step k0+32 needs from memory -- weights, activations
+  // and (when it opens a new scale group) the scales -- is requested before the arithmetic
+  // of step k0 starts, so a step never waits for a load issued after its own.
+  constexpr int SW = NV * SSZ / 4;  // dwords of raw scales per lane
   uint32_t wq[2][8][WORDS];
-  auto load_rows = [&](int buf, int k0) {
+  uintx4 aq[2][MT];
+  uint32_t sraw[2][SW];
+  float sc[NV];  // kRounded: scale (x16 for s4) of each owned channel, for the current group
+
+  // GROUP32: a step opens a new group every `steps_per_group` steps (and at the wave's first)
+  const int steps_per_group = GROUP32 ? p.group / 32 : 1;
+  auto opens_group = [&](int k0) {  // scalar
+    return !GROUP32 || k0 == k_begin || ((k0 >> 5) % steps_per_group) == 0;
+  };
+  auto load_step = [&](int buf, int k0) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      aq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt] + (uint32_t)k0 * 2u, 0, 0);
+    if (MODE == kRounded) {
+      if (GROUP32) {
+        if (opens_group(k0)) {
+          const uint32_t g = (uint32_t)min(k0, p.K - 1) / (uint32_t)p.group;  // scalar
+          buffer_load_words<SW>(rs, voff_s, g * (uint32_t)p.N * SSZ, sraw[buf]);
+        }
+      } else {
+        const uint32_t g = (uint32_t)min(k0 + 8 * kb, p.K - 1) / (uint32_t)p.group;  // per lane
+        buffer_load_words<SW>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, sraw[buf]);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 8; ++r)
       buffer_load_words<WORDS>(rw, voff_w + (uint32_t)(k0 + r) * pitch, 0, wq[buf][r]);
@@ -169,18 +178,20 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt] + (uint32_t)k0 * 2u, 0, 0);
+      uintx4 v = aq[buf][mt];
       if (k0 + 32 > p.K) {  // scalar condition: only a step that crosses the end of K
         const bool ok = k0 + 8 * kb < p.K;
         v = uintx4{ok ? v[0] : 0u, ok ? v[1] : 0u, ok ? v[2] : 0u, ok ? v[3] : 0u};
       }
       bop[mt] = __builtin_bit_cast(bf16x8, v);
     }
-    if (MODE == kRounded) {
-      if (GROUP32) {
-        if (k0 % p.group == 0 || k0 == k_begin) load_scales(k0);  // scalar condition
-      } else {
-        load_scales(k0);
+    if (MODE == kRounded && opens_group(k0)) {
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const uint32_t* raw = sraw[buf];
+        float v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
+                             : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
+        sc[j] = WBITS == 4 ? v * 16.0f : v;  // the s4 convert yields value/16
       }
     }
 #pragma unroll
@@ -218,11 +229,11 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   };
 
   if (k_begin < p.K) {
-    load_rows(0, k_begin);
+    load_step(0, k_begin);
     for (int k0 = k_begin; k0 < k_stop; k0 += 64) {
-      load_rows(1, k0 + 32);
+      load_step(1, k0 + 32);
       compute(0, k0);
-      load_rows(0, k0 + 64);
+      load_step(0, k0 + 64);
       compute(1, k0 + 32);
     }
   }

@@ -402,6 +402,48 @@ __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __r
   }
 }
 
+// [K,N] -> [N,K] byte transpose, 128x128 tiles, for N % 4 == 0, K % 16 == 0 and aligned
+// pointers.  A thread reads 4 rows x 4 bytes (lanes along N: 128 contiguous bytes per row and
+// half wave), transposes the 4x4 block with byte permutes, and parks the four column dwords in
+// LDS as [n][k/4], the dword index XOR-swizzled by n/4 so the 32 lanes of a row group hit 32
+// banks.  Then two threads per output row gather its 32 dwords and store 128 contiguous bytes.
+__global__ __launch_bounds__(256) void transpose_bytes_fast_kernel(const uint8_t* __restrict__ src,
+                                                                   uint8_t* __restrict__ dst, int K, int N) {
+  __shared__ uint32_t tile[128 * 32];
+  const int k0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int b = tid + 256 * i, nb = b & 31, kb = b >> 5;
+    uint32_t r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int k = k0 + 4 * kb + q, n = n0 + 4 * nb;
+      r[q] = (k < K && n < N) ? *reinterpret_cast<const uint32_t*>(src + (size_t)k * N + n) : 0u;
+    }
+    // bytes of v_perm's pool: 0-3 = second operand, 4-7 = first operand
+    const uint32_t a01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);  // r0b0 r1b0 r0b1 r1b1
+    const uint32_t c01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);  // r0b2 r1b2 r0b3 r1b3
+    const uint32_t a23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t c23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    const uint32_t col[4] = {__builtin_amdgcn_perm(a23, a01, 0x05040100u), __builtin_amdgcn_perm(a23, a01, 0x07060302u),
+                             __builtin_amdgcn_perm(c23, c01, 0x05040100u), __builtin_amdgcn_perm(c23, c01, 0x07060302u)};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile[(4 * nb + j) * 32 + (kb ^ nb)] = col[j];
+  }
+  __syncthreads();
+  const int n = tid >> 1, half = tid & 1;
+  if (n0 + n >= N) return;
+  uint8_t* out = dst + (size_t)(n0 + n) * K + k0 + half * 64;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uintx4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = tile[n * 32 + ((half * 16 + q * 4 + e) ^ (n >> 2))];
+    if (k0 + half * 64 + q * 16 < K) *reinterpret_cast<uintx4*>(out + q * 16) = v;  // K % 16 == 0
+  }
+}
+
 // Exact, slow f8 scaled dot for scales that are not powers of two under a bf16-typed
 // dequantise multiply: each operand value is rounded to bf16 after its scale, as the HLO does.
 __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b_is_nk, int deq_bf16,
@@ -519,9 +561,15 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const uint8_t* b_nk = (const uint8_t*)p.b;
   if (tiled_ok && !nk) {
     if (p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
-      dim3 tgrid((unsigned)((p.N + 63) / 64), (unsigned)((p.K + 63) / 64));
-      hipLaunchKernelGGL(transpose_bytes_kernel, tgrid, dim3(256), 0, stream, (const uint8_t*)p.b,
-                         (uint8_t*)p.workspace, (int)p.K, (int)p.N);
+      if (p.N % 4 == 0 && ((uintptr_t)p.b % 4 == 0)) {
+        dim3 tgrid((unsigned)((p.N + 127) / 128), (unsigned)((p.K + 127) / 128));
+        hipLaunchKernelGGL(transpose_bytes_fast_kernel, tgrid, dim3(256), 0, stream, (const uint8_t*)p.b,
+                           (uint8_t*)p.workspace, (int)p.K, (int)p.N);
+      } else {
+        dim3 tgrid((unsigned)((p.N + 63) / 64), (unsigned)((p.K + 63) / 64));
+        hipLaunchKernelGGL(transpose_bytes_kernel, tgrid, dim3(256), 0, stream, (const uint8_t*)p.b,
+                           (uint8_t*)p.workspace, (int)p.K, (int)p.N);
+      }
       int rc = CheckLaunch("fp8_scaled_dot_transpose");
       if (rc) return rc;
       b_nk = (const uint8_t*)p.workspace;
