@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 HBM_PEAK_XLA_GBS = 6810.0      # what XLA's own device file assumes (mi350.txtpb:28)
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}
+# HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this script, each scaled by what the same counter read for the --calibrate-copy kernel (figures
+# and factors: profiles/decode_c2_hbm_traffic.md).  None where no such run has been made.
+MEASURED_TRAFFIC_BYTES = {"C2 M=64": 138326809, "C2 M=32": 131555915}
 K2, N2, GROUP2 = 8192, 28672, 128
 MS2 = (1, 8, 32, 64)
 
@@ -41,6 +45,9 @@ def main():
     ap.add_argument("--skip-other", action="store_true", help="only the headline workload")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baseline leg")
     ap.add_argument("--reps", type=int, default=20, help="launches per event-timed batch")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times, so that a rocprofv3 --pmc run of this "
+                         "command shows what FETCH_SIZE / WRITE_SIZE read for a known number of bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path shards by output channels with no "
@@ -69,6 +76,17 @@ def main():
             t = e0.elapsed_time(e1) / reps
             best = t if best is None else min(best, t)
         return best  # ms
+
+    # ---- what a plain copy reaches on this machine (context for every HBM fraction below) ------
+    ca = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    cb = torch.empty_like(ca)
+    copy_ms = ev_time(lambda: cb.copy_(ca), 5)
+    copy_gbs = 2 * ca.numel() / (copy_ms * 1e-3) / 1e9
+    if args.calibrate_copy:
+        for _ in range(3):
+            cb[:1 << 28].copy_(ca[:1 << 28])     # 256 MiB read + 256 MiB written per launch
+        torch.cuda.synchronize()
+    del ca, cb
 
     # ---- configuration 2 on the device -------------------------------------------------------
     w_packed = torch.randint(0, 256, (K2 * N2 // 2,), dtype=torch.uint8, device=dev)   # nibbles ~U{-8..7}
@@ -106,7 +124,10 @@ def main():
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "workload": dom["workload"],
                 "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
                 "frac_of_xla_device_file_peak": round(dom["GB/s"] / HBM_PEAK_XLA_GBS, 4),
-                "traffic": None, "launch_ms": dom["ms"], "algorithmic_bytes": dom["bytes"]}
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dom["workload"]), "launch_ms": dom["ms"],
+                "algorithmic_bytes": dom["bytes"],
+                "device_copy_GB/s": round(copy_gbs, 1),
+                "frac_of_device_copy_rate": round(dom["GB/s"] / copy_gbs, 4)}
 
     # ---- the other four configurations (informational) -----------------------------------------
     other = []
