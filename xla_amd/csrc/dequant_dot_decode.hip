@@ -462,9 +462,15 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
       if (int s = GetOption("dequant_dot_slices")) {
         slices = s;
       } else {
-        const int want = p.M <= 8 ? 768 : 384;  // workgroups; partial sums cost slices*M*N*4 bytes
-        while (dp.strips * slices * p.batch < want && p.K / (slices * 2) >= 64 * waves &&
-               slices * 2 * p.M <= 32)
+        // workgroups wanted; the partial sums cost slices*M*N*4 bytes written and read again,
+        // which is allowed to reach a quarter of the weight bytes when the strips alone would leave
+        // most CUs idle
+        const int want = p.M <= 8 ? 768 : 384;
+        const double weight_bytes = (double)p.K * row_bytes;
+        // and no slice so thin that a wave gets fewer than four 32-row steps
+        while (dp.strips * slices * p.batch < want && p.K / (slices * 2) >= 128 * waves &&
+               (slices * 2 * p.M <= 32 ||
+                (dp.strips * p.batch <= 64 && 2.0 * (slices * 2) * p.M * p.N * 4.0 <= 0.25 * weight_bytes)))
           slices *= 2;
       }
       if (slices > 1 && (!p.workspace ||
