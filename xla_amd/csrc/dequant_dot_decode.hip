@@ -54,11 +54,6 @@ __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf
   return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];
 }
 
-// s4 nibble (two's complement, in the low 4 bits of `v`) -> f32 value/16, one instruction
-__device__ __forceinline__ float s4_to_f32_div16(uint32_t v) {
-  return __builtin_amdgcn_cvt_off_f32_i4((int)v);
-}
-
 // Buffer descriptor over [base, base+bytes): loads through it return 0 past the end, which is
 // how rows beyond K and tokens beyond M drop out of the main loop without any branch.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -146,7 +141,8 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   uint32_t wq[2][8][WORDS];
   uintx4 aq[2][MT];
   uint32_t sraw[2][SW];
-  float sc[NV];  // kRounded: scale (x16 for s4) of each owned channel, for the current group
+  float sc[NV];  // kRounded: scale of each owned channel for the current group (s4: see compute)
+  float cc[NV];  // s4: the constant term that removes the conversion offset
 
   // GROUP32: a step opens a new group every `steps_per_group` steps (and at the wave's first)
   const int steps_per_group = GROUP32 ? p.group / 32 : 1;
@@ -191,39 +187,70 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
         const uint32_t* raw = sraw[buf];
         float v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
                              : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
-        sc[j] = WBITS == 4 ? v * 16.0f : v;  // the s4 convert yields value/16
+        if (WBITS == 4) {
+          // nibble j of a dword arrives as the f16 value 1024 + u (even j) or 1024 + 16u (odd j),
+          // u = w + 8: w*s = (1024 + u)*s - 1032*s = (1024 + 16u)*(s/16) - 72*s, one fma each,
+          // exact for any scale with an 8-bit significand and |1040*s| finite
+          sc[j] = (j & 1) ? v * 0.0625f : v;
+          cc[j] = (j & 1) ? v * -72.0f : v * -1032.0f;
+        } else {
+          sc[j] = v;
+        }
       }
     }
 #pragma unroll
     for (int q = 0; q < WORDS; ++q) {
-      // s4: one shift exposes the odd nibbles; byte selects then come for free with the convert
-      uint32_t lo[8], hi[8];
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        lo[r] = wq[buf][r][q];
-        hi[r] = lo[r] >> 4;
-        if (WBITS == 4) asm volatile("" : "+v"(hi[r]));  // keep it one shift, not one per nibble
-      }
-#pragma unroll
-      for (int e = 0; e < NPW; ++e) {
-        const int j = q * NPW + e;
-        float f[8];
+      if constexpr (WBITS == 4) {
+        // Two nibbles become the two f16 halves of one dword in a single three-input bit
+        // operation: where the mask is set the result is x ^ C (the nibble with its sign bit
+        // flipped: offset binary), elsewhere C (the f16 exponent of 1024).  Masks 0x000f000f /
+        // 0x00f000f0 pick nibbles (0,4) / (1,5) of x and (2,6) / (3,7) of x >> 8.  The product
+        // with the scale and the removal of the offset are one v_fma_mix_f32 per weight.
+        typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+        halfx2 pr[8][4];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-          if (WBITS == 4) {
-            const uint32_t src = (e & 1) ? hi[r] : lo[r];
-            f[r] = s4_to_f32_div16((src >> (8 * (e >> 1))) & 0xffu);
-          } else {
-            f[r] = (float)(int8_t)((lo[r] >> (8 * e)) & 0xffu);
-          }
-          if (MODE == kRounded) f[r] = f[r] * sc[j];
+          const uint32_t x = wq[buf][r][q], y = x >> 8;
+          pr[r][0] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+          pr[r][1] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a));
+          pr[r][2] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(y, 0x000f000fu, 0x64086408u, 0x6a));
+          pr[r][3] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(y, 0x00f000f0u, 0x64806480u, 0x6a));
         }
-        uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                    pack_bf16x2(f[6], f[7])};
-        const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+        for (int e = 0; e < 8; ++e) {
+          const int j = q * 8 + e;
+          const float sj = MODE == kRounded ? sc[j] : ((e & 1) ? 0.0625f : 1.0f);
+          const float cj = MODE == kRounded ? cc[j] : ((e & 1) ? -72.0f : -1032.0f);
+          float f[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][e & 3][e >> 2], sj, cj);
+          uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                      pack_bf16x2(f[6], f[7])};
+          const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+        }
+      } else {
+        uint32_t lo[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) lo[r] = wq[buf][r][q];
+#pragma unroll
+        for (int e = 0; e < NPW; ++e) {
+          const int j = q * NPW + e;
+          float f[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            f[r] = (float)(int8_t)((lo[r] >> (8 * e)) & 0xffu);
+            if (MODE == kRounded) f[r] = f[r] * sc[j];
+          }
+          uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                      pack_bf16x2(f[6], f[7])};
+          const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+        }
       }
     }
   };
@@ -252,7 +279,6 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
       const int r = pass * kChunk + c;
       const int j = r % NV, mt = (r / NV) / 4, t = (r / NV) % 4;
       float v = acc[j][mt][t];
-      if (MODE == kFactored && WBITS == 4) v *= 16.0f;  // undo value/16 (exact)
       lds[(wave * kChunk + c) * 64 + lane] = v;
     }
     __syncthreads();
