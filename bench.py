@@ -51,7 +51,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (the path shards by output channels with no "
-                 "exchange step; see DESIGN.md); --gpus %d is not supported" % args.gpus)
+                 "exchange step, so more GPUs would only run independent column slices); --gpus %d is not supported" % args.gpus)
 
     import torch
     from xla_amd import ffi, ops
@@ -162,7 +162,7 @@ def main():
         b8 = (torch.randn((8192, 8192), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
         s64 = torch.full((), 1 / 64, device=dev)
         b3 = torch.randn((8192,), device=dev).to(torch.bfloat16)
-        entry("C3 fp8 [8192,8192]x[8192,8192] (rhs [K,N])",
+        entry("C3 fp8 [8192,8192]x[8192,8192] (rhs [K,N], as in the HLO)",
               ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", build_only=True),
               2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
         entry("C3 fp8, rhs given as [N,K]",

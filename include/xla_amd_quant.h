@@ -182,7 +182,8 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
 /* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
  * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, 3 tiled),
  * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "fp8_dot_kernel" (1 exact, 2 tiled),
- * "quantize_variant".  Returns 0, or -1 for an unknown key. */
+ * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass).  Returns 0, or -1 for
+ * an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
 
 #ifdef __cplusplus

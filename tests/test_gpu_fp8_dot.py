@@ -70,6 +70,30 @@ def test_c3_shape_reduced(oracle, M, K, N, nk):
     assert n_floor <= got.size // 100
 
 
+def test_rhs_layouts_take_their_own_paths(oracle):
+    """[N,K] streams as it is, [K,N] with whole 16-channel chunks is transposed on the way out of
+    LDS, any other [K,N] (or a forced one) through a pre-pass; all three must agree with the oracle."""
+    say("fp8_scaled_dot rhs layouts")
+    w = workloads.c3_fp8(192, 640, 272)
+    ref = reference(oracle, w)
+    seen = set()
+    for nk, layout in [(True, 0), (False, 0), (False, 1)]:
+        ffi.set_option("fp8_dot_layout", layout)
+        try:
+            got, kern = run(w, nk=nk)
+        finally:
+            ffi.set_option("fp8_dot_layout", 0)
+        seen.add(kern)
+        n_floor = check_dot(got, ref, floor_for(w), kern)
+        assert n_floor <= got.size // 100
+    assert seen == {"fp8_scaled_dot_tiled", "fp8_scaled_dot_tiled_kn", "fp8_scaled_dot_tiled+transpose"}, seen
+    w2 = workloads.c3_fp8(64, 128, 200)  # 200 % 16 != 0: no direct [K,N] path
+    got, kern = run(w2, nk=False)
+    assert kern == "fp8_scaled_dot_tiled+transpose", kern
+    # K = 128: many outputs sit on the flat tail of GELU, where only the floor clause is meaningful
+    assert check_dot(got, reference(oracle, w2), floor_for(w2), kern) <= got.size // 25
+
+
 def test_fp8_one_hot_exact(oracle):
     """A = selector rows of 1.0: outputs are single B values times the scales, exactly."""
     say("fp8_scaled_dot one-hot")

@@ -33,14 +33,14 @@
 namespace xla_amd {
 namespace {
 
-enum : int { kFp8 = 0, kS8 = 1 };
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2 };  // kFp8KN: fp8 with the weights given [K,N]
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
 
 struct TiledParams {
   const uint8_t* a;     // kFp8: f8 [M,K]; kS8: bf16 [batch,M,K]
-  const uint8_t* b;     // kFp8: f8 [N,K]; kS8: s8 [batch,K,N]
+  const uint8_t* b;     // kFp8: f8 [N,K]; kFp8KN: f8 [K,N]; kS8: s8 [batch,K,N]
   const float* a_scale; // kFp8 device scalars
   const float* b_scale;
   const void* scales;   // kS8: [scale_batch, N]
@@ -131,12 +131,14 @@ __device__ __forceinline__ void drain_dispatch(const DrainArgs& d, int act, bool
 
 template <int KIND>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
-  constexpr int ESZ = KIND == kFp8 ? 1 : 2;  // bytes per activation element
+  constexpr bool F8 = KIND != kS8;       // both operands f8e4m3fn
+  constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
+  constexpr int ESZ = F8 ? 1 : 2;  // bytes per activation element
   constexpr int KS = kRow / ESZ;             // K elements per stage
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [2][(kTM + kTN) * kRow]
   constexpr int kBufBytes = (kTM + kTN) * kRow;
 
-  if (KIND == kFp8 && p.require_pow2_scales) {
+  if (F8 && p.require_pow2_scales) {
     if (!(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;  // the exact kernel runs
   }
 
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const __amdgpu_buffer_rsrc_t ra =
       tile_rsrc(p.a + (size_t)batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
   const __amdgpu_buffer_rsrc_t rb =
-      KIND == kFp8 ? tile_rsrc(p.b, (uint32_t)p.N * (uint32_t)p.K)
+      F8 ? tile_rsrc(p.b, (uint32_t)p.N * (uint32_t)p.K)
                    : tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
 
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
@@ -191,6 +193,15 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const int r = wave * 32 + j * 8 + ld_row;
     voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk[j & 1] * 16;
     if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
+    if (BKN) {
+      // [K,N]: instruction j of this wave moves 4 rows of K x 256 channels; lane l fills slot l%16
+      // of row l/16 with global chunk (l%16) ^ ((k & 7) << 1): eight consecutive rows then spread a
+      // pair of neighbouring chunks over all 16 slots, which the transposing reads below need
+      const int kr = wave * 16 + j * 4 + (lane >> 4);  // row of the stage (0..127)
+      const int ch = (lane & 15) ^ ((kr & 7) << 1);
+      const uint32_t col = (uint32_t)(n0 + ch * 16);
+      voff_b[j] = col < (uint32_t)p.N ? (uint32_t)kr * (uint32_t)p.N + col : kOutOfRange;  // N % 16 == 0
+    }
   }
 
   // ---- s8 weights: a thread takes 4 channels (quad nq) of the 8 rows of block kblk
@@ -229,6 +240,11 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       load_to_lds(ra, at + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
       if (KIND == kFp8)
         load_to_lds(rb, bt + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
+      if (BKN) {
+        // rows k0 + kr; a row past K lies past the end of the buffer by itself
+        const uint32_t v = voff_b[j] == kOutOfRange ? kOutOfRange : voff_b[j] + (uint32_t)k0 * (uint32_t)p.N;
+        load_to_lds(rb, bt + (wave * 16 + j * 4) * 256, v);
+      }
     }
     if (KIND == kS8) s8_load(k0);
   };
@@ -248,24 +264,50 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // the workgroup synchronises: every wave's reads of the stage buffer are complete (so it
   // may be refilled) and the next stage's tiles have landed.  The refill for stage s+2 is
   // issued right behind that barrier, interleaved with the MFMAs.
-  constexpr int NKS = KIND == kFp8 ? 2 : 4;
+  constexpr int NKS = F8 ? 2 : 4;
   const int frag_sw = (l32 >> 1) & 7;  // tile rows of a fragment start at multiples of 32
   const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 64 + l32) * kRow;
-  typedef typename std::conditional<KIND == kFp8, intx8, bf16x8>::type frag_t;
+  typedef typename std::conditional<F8, intx8, bf16x8>::type frag_t;
   frag_t fa[4], fb[2];
+  // kFp8KN: per-lane parts of the transposing reads' addresses (see read_frags)
+  const int tr_m = (lane & 15) >> 1, tr_par = lane & 1, tr_g = (lane >> 4) & 1;
+  const int bkn_base = (32 * kb + tr_m) * 256 + 8 * tr_par;
+  const int bkn_cx[2] = {((wn * 4 + 0 + tr_g) ^ (tr_m << 1)) << 4, ((wn * 4 + 2 + tr_g) ^ (tr_m << 1)) << 4};
   auto read_frags = [&](int buf, int ks) {
     const uint8_t* at = lds + buf * kBufBytes + row_a;
     const uint8_t* bt = lds + buf * kBufBytes + row_b;
-    if constexpr (KIND == kFp8) {
+    if constexpr (F8) {
       const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
       auto rd = [&](const uint8_t* base) {
         const uintx4 x0 = *reinterpret_cast<const uintx4*>(base + c0);
         const uintx4 x1 = *reinterpret_cast<const uintx4*>(base + c1);
         return intx8{(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
       };
-      fb[0] = rd(bt);
-      fa[0] = rd(at);
-      fb[1] = rd(bt + 32 * kRow);
+      if constexpr (BKN) {
+        // Weight tile [k][256 channels] in LDS, read with the transposing 64-bit load: in every
+        // group of 16 lanes, lane i hands in the address of 8 bytes (row i of a 16x8 block) and
+        // lane j receives column j of the even rows (j < 8) or column j-8 of the odd rows.  Even
+        // lanes point at 8 consecutive k of one channel octet, odd lanes at the same k of the next
+        // octet, so the 16 lanes end up with 8 consecutive k of 16 consecutive channels: the MFMA
+        // operand layout.  Four such loads give a lane its 32 values of k.
+        typedef int intx2 __attribute__((ext_vector_type(2)));
+        typedef __attribute__((address_space(3))) intx2* tr_ptr_t;
+        const uint8_t* wt = lds + buf * kBufBytes + kTM * kRow + bkn_base + ks * (64 * 256);
+        auto rdt = [&](int nt) {
+          intx2 q[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            q[i] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr_t)(uintptr_t)(wt + bkn_cx[nt] + i * (8 * 256)));
+          return intx8{q[0][0], q[0][1], q[1][0], q[1][1], q[2][0], q[2][1], q[3][0], q[3][1]};
+        };
+        fb[0] = rdt(0);
+        fa[0] = rd(at);
+        fb[1] = rdt(1);
+      } else {
+        fb[0] = rd(bt);
+        fa[0] = rd(at);
+        fb[1] = rd(bt + 32 * kRow);
+      }
 #pragma unroll
       for (int t = 1; t < 4; ++t) fa[t] = rd(at + t * 32 * kRow);
     } else {
@@ -282,7 +324,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        if constexpr (KIND == kFp8)
+        if constexpr (F8)
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, 0, 0, 0);
         else
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
@@ -308,7 +350,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     __syncthreads();
     issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
     mfma_all();
-    if (KIND == kFp8) {
+    if (F8) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
@@ -334,7 +376,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever indexed
   // statically.  The rolled read loop carries the epilogue.
   float alpha = 1.0f;
-  if (KIND == kFp8) alpha = *p.a_scale * *p.b_scale;
+  if (F8) alpha = *p.a_scale * *p.b_scale;
   float* stage = reinterpret_cast<float*>(lds + wave * 16384);
   const int rd_chunk = lane & 15, rd_row = lane >> 4;  // read side: chunk of 4 channels, row within 4
   const bool n_vec = (p.N & 3) == 0;
@@ -559,7 +601,11 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   bool tiled_ok = p.K % 16 == 0 && p.K > 0 && ((uintptr_t)p.a % 16 == 0) && force != 1 &&
                   (double)p.M * p.K < 2147483000.0 && (double)p.N * p.K < 2147483000.0;
   const uint8_t* b_nk = (const uint8_t*)p.b;
-  if (tiled_ok && !nk) {
+  // a [K,N] rhs with whole 16-channel chunks goes in as it is: the kernel stages it K-major and
+  // transposes on the way out of LDS (fp8_dot_layout = 1 forces the transposing pre-pass instead)
+  const bool kn_direct = tiled_ok && !nk && p.N % 16 == 0 && ((uintptr_t)p.b % 16 == 0) &&
+                         GetOption("fp8_dot_layout") != 1;
+  if (tiled_ok && !nk && !kn_direct) {
     if (p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
       if (p.N % 4 == 0 && ((uintptr_t)p.b % 4 == 0)) {
         dim3 tgrid((unsigned)((p.N + 127) / 128), (unsigned)((p.K + 127) / 128));
@@ -588,7 +634,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;
-    int rc = launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
+    int rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn")
+                       : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
     if (rc) return rc;
     if (deq_bf16) {
       // runs only if a scale is not a power of two (decided on the device, no host read)
@@ -596,7 +643,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       rc = CheckLaunch("fp8_scaled_dot_exact");
       if (rc) return rc;
     }
-    SetLastKernel(nk ? "fp8_scaled_dot_tiled" : "fp8_scaled_dot_tiled+transpose");
+    SetLastKernel(nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose");
     return 0;
   }
   hipLaunchKernelGGL(fp8_dot_exact_kernel, egrid, dim3(256), 0, stream, tp, nk ? 1 : 0, deq_bf16 ? 1 : 0, 0);
