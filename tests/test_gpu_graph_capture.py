@@ -1,0 +1,85 @@
+"""The handlers declare XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE: XLA may record them
+into a command buffer (a HIP graph) once and replay it step after step
+(xla/ffi/api/c_api.h:428-437, 528-533; xla/backends/gpu/runtime/custom_call_thunk.cc:659-666).
+That only works if a call enqueues the same kernels for the same shapes, never synchronises,
+never reads device data on the host and allocates nothing.  Here a decode step, a quantize and
+a scaled dot are captured into one graph through the native call-frame replay, the operands
+are then changed in place, and every replay must equal what eager calls give on the same data."""
+import sys
+
+import pytest
+import torch
+
+from xla_amd import ffi, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def test_handlers_replay_from_a_hip_graph():
+    say("graph capture of dequant_dot (split-K + finalize), rowwise_quantize_fp8, fp8_scaled_dot")
+    dev = torch.device("cuda:0")
+    torch.manual_seed(7)
+    K, N = 2048, 1024
+    lhs = torch.randn((8, K), device=dev).to(torch.bfloat16)
+    w4 = torch.randint(0, 256, (K * N // 2,), dtype=torch.uint8, device=dev)
+    sc = torch.empty((K // 128, N), device=dev).uniform_(1e-3, 2e-2).to(torch.bfloat16)
+    bias = torch.randn((N,), device=dev).to(torch.bfloat16)
+    x = torch.randn((256, 1024), device=dev).to(torch.bfloat16)
+    gamma = torch.empty((1024,), device=dev).uniform_(0.5, 1.5).to(torch.bfloat16)
+    a8 = (torch.randn((256, 512), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+    b8 = (torch.randn((512, 256), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+    s64 = torch.full((), 1 / 64, device=dev)
+
+    calls = [ops.dequant_dot(lhs, w4, sc, bias, weight_dtype="s4", weight_shape=(K, N), epilogue="BIAS_SILU",
+                             dequant_type="bf16", build_only=True),
+             ops.rowwise_quantize_fp8(x, gamma, build_only=True),
+             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="GELU", build_only=True)]
+
+    def results():
+        out = []
+        for c in calls:
+            r = c.result if isinstance(c.result, (list, tuple)) else [c.result]
+            out += [t.clone().view(torch.uint8) if t.dtype != torch.float32 else t.clone() for t in r]
+        return out
+
+    # eager warm-up: first launches may set kernel attributes, which must not happen under capture
+    for c in calls:
+        c.run()
+    torch.cuda.synchronize()
+
+    replay = ffi.Replay([(c.target, c.frame) for c in calls])
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for c in calls:
+            c.frame.host.stream = side.cuda_stream
+        with torch.cuda.graph(graph, stream=side):
+            replay.run(1)
+    torch.cuda.current_stream().wait_stream(side)
+
+    for round_ in range(3):
+        # new operand values in the same buffers, eager work and a synchronisation between replays
+        lhs.copy_(torch.randn((8, K), device=dev).to(torch.bfloat16))
+        x.copy_(torch.randn((256, 1024), device=dev).to(torch.bfloat16) * (round_ + 1))
+        a8.copy_((torch.randn((256, 512), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn))
+        torch.cuda.synchronize()
+        for c in calls:
+            c.run()
+        torch.cuda.synchronize()
+        want = results()
+        for c in calls:  # wipe the outputs so that a replay that does nothing cannot pass
+            for t in (c.result if isinstance(c.result, (list, tuple)) else [c.result]):
+                t.view(torch.uint8).zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = results()
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert torch.equal(g, w), "replay %d: result %d differs from the eager call" % (round_, i)
+    assert ffi.last_kernel()  # the library recorded which kernels it chose
