@@ -68,7 +68,8 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  * (xla/backends/gpu/transforms/gemm_rewriter.cc:1235-1591, executed by
  * CublasLtMatmulThunk -> hipBLASLt, xla/stream_executor/rocm/hip_blas_lt.cc:468-484).
  *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1);
- *         a_scale F32 []; b_scale F32 []; bias BF16|F32 [N] (only with BIAS*)
+ *         a_scale F32 [] or [M] (one per row of a, as a row-wise quantizer produces them);
+ *         b_scale F32 [] or [N] (one per output channel); bias BF16|F32 [N] (only with BIAS*)
  *   rets: out BF16 [M,N]
  *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
  *          rhs_contracting_dim i64 (default 0)
@@ -139,8 +140,8 @@ XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t
 typedef struct XlaAmdFp8ScaledDot {
   const void* a;       /* f8e4m3fn [M,K] */
   const void* b;       /* f8e4m3fn [K,N] or [N,K] */
-  const float* a_scale; /* device scalars */
-  const float* b_scale;
+  const float* a_scale; /* device: one value, or M values when a_scale_per_row */
+  const float* b_scale; /* device: one value, or N values when b_scale_per_channel */
   const void* bias;
   void* out;           /* bf16 [M,N] */
   void* workspace;     /* optional scratch, see xla_amd_fp8_scaled_dot_workspace_bytes */
@@ -150,6 +151,8 @@ typedef struct XlaAmdFp8ScaledDot {
   int32_t bias_dtype;
   int32_t dequant_type, dot_type, epilogue_type;
   int32_t epilogue;
+  int32_t a_scale_per_row;     /* a_scale is f32[M]: row m of a is scaled by a_scale[m] */
+  int32_t b_scale_per_channel; /* b_scale is f32[N]: output channel n of b by b_scale[n] */
 } XlaAmdFp8ScaledDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);

@@ -73,7 +73,7 @@ def lib():
         L.xo_dequant_dot.argtypes = [vp, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64, i64,
                                      i64, i32, i32, i32, vp]
         L.xo_fp8_scaled_dot.restype = i32
-        L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, f32, f32, i32, vp, i32, i64, i64, i64,
+        L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64,
                                         i32, i32, i32, vp]
         L.xo_rmsnorm_quantize_fp8.restype = i32
         L.xo_rmsnorm_quantize_fp8.argtypes = [vp, vp, f32, i64, i64, vp, vp]
@@ -212,9 +212,14 @@ def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=N
         bias = _c(bias, np.uint16 if bias_ty == "bf16" else np.float32)
         assert bias.size == N
         bp = _ptr(bias)
+    # a scale is one value, or one per row of a (a_scale) / per output channel (b_scale)
+    sa = _c(np.asarray(a_scale, np.float32).reshape(-1), np.float32)
+    sb = _c(np.asarray(b_scale, np.float32).reshape(-1), np.float32)
+    a_rows, b_cols = np.ndim(a_scale) == 1, np.ndim(b_scale) == 1
+    assert sa.size == (M if a_rows else 1) and sb.size == (N if b_cols else 1)
     out = np.empty((M, N), np.uint16)
-    rc = lib().xo_fp8_scaled_dot(_ptr(a8), _ptr(b8), int(b_is_nk), float(a_scale), float(b_scale),
-                                 TYPES[mul_ty], bp, TYPES[bias_ty], M, K, N, TYPES[dot_ty],
+    rc = lib().xo_fp8_scaled_dot(_ptr(a8), _ptr(b8), int(b_is_nk), _ptr(sa), int(a_rows), _ptr(sb),
+                                 int(b_cols), TYPES[mul_ty], bp, TYPES[bias_ty], M, K, N, TYPES[dot_ty],
                                  TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
     assert rc == 0
     return out

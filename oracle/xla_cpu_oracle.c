@@ -385,42 +385,54 @@ XO_API int xo_dequant_dot(const uint16_t* A, const void* w, int w_bits,
 
 /*
  * out[m,n] = epilogue( sum_k A'[m,k] * B'[k,n] ),
- *   A' = round_mul_ty(f32(A8) * round_mul_ty(a_scale)), same for B'.
+ *   A'[m,k] = round_mul_ty(f32(A8[m,k]) * round_mul_ty(sa_m)), B'[k,n] likewise with sb_n.
  * A8: f8e4m3fn [M,K] row-major.  B8: f8e4m3fn, [K,N] row-major when
  * b_is_nk == 0, or [N,K] row-major (contracting dimension minor) when 1.
+ * a_scale points at one value (a_rows == 0: the per-tensor scale of
+ * gemm_rewriter_fp8_test.cc:1099-1135) or at M values (a_rows != 0: one per
+ * row of A, the broadcast along dimension 0 that a row-wise quantizer's
+ * scales are applied with); b_scale at one value or, with b_cols != 0, at N
+ * values, one per output channel.
  */
 XO_API int xo_fp8_scaled_dot(const uint8_t* A8, const uint8_t* B8, int b_is_nk,
-                             float a_scale, float b_scale, int mul_ty,
-                             const void* bias, int bias_ty, int64_t M, int64_t K,
-                             int64_t N, int dot_ty, int ep_ty, int epi,
-                             uint16_t* out) {
-  float lutA[256], lutB[256];
-  float sa = rnd(a_scale, mul_ty), sb = rnd(b_scale, mul_ty);
-  for (int c = 0; c < 256; ++c) {
-    volatile float pa = xo_f8e4m3fn_to_f32((uint8_t)c) * sa;
-    volatile float pb = xo_f8e4m3fn_to_f32((uint8_t)c) * sb;
-    lutA[c] = rnd(pa, mul_ty);
-    lutB[c] = rnd(pb, mul_ty);
+                             const float* a_scale, int a_rows, const float* b_scale,
+                             int b_cols, int mul_ty, const void* bias, int bias_ty,
+                             int64_t M, int64_t K, int64_t N, int dot_ty, int ep_ty,
+                             int epi, uint16_t* out) {
+  float f8v[256];
+  for (int c = 0; c < 256; ++c) f8v[c] = xo_f8e4m3fn_to_f32((uint8_t)c);
+  /* the dequantised A once: M*K floats */
+  float* Ad = (float*)malloc(sizeof(float) * (size_t)(M > 0 ? M : 1) * (size_t)(K > 0 ? K : 1));
+  if (!Ad) return -1;
+  for (int64_t m = 0; m < M; ++m) {
+    float sa = rnd(a_scale[a_rows ? m : 0], mul_ty);
+    for (int64_t k = 0; k < K; ++k) {
+      volatile float pa = f8v[A8[(size_t)m * K + k]] * sa;
+      Ad[(size_t)m * K + k] = rnd(pa, mul_ty);
+    }
   }
   int rc = 0;
 #pragma omp parallel
   {
-    float* col = (float*)malloc(sizeof(float) * (size_t)K);
+    float* col = (float*)malloc(sizeof(float) * (size_t)(K > 0 ? K : 1));
     if (!col) rc = -1;
 #pragma omp for schedule(static)
     for (int64_t n = 0; n < N; ++n) {
       if (rc) continue;
-      for (int64_t k = 0; k < K; ++k)
-        col[k] = lutB[b_is_nk ? B8[(size_t)n * K + k] : B8[(size_t)k * N + n]];
+      float sb = rnd(b_scale[b_cols ? n : 0], mul_ty);
+      for (int64_t k = 0; k < K; ++k) {
+        volatile float pb = f8v[b_is_nk ? B8[(size_t)n * K + k] : B8[(size_t)k * N + n]] * sb;
+        col[k] = rnd(pb, mul_ty);
+      }
       float bv = 0.0f;
       if (bias)
         bv = bias_ty == XO_BF16 ? xo_bf16_to_f32(((const uint16_t*)bias)[n])
                                 : ((const float*)bias)[n];
       for (int64_t m = 0; m < M; ++m) {
-        const uint8_t* a = A8 + (size_t)m * K;
+        const float* a = Ad + (size_t)m * K;
         float acc = 0.0f;
         for (int64_t k = 0; k < K; ++k) {
-          float p = lutA[a[k]] * col[k];
+          float p = a[k] * col[k];
           acc = acc + p;
         }
         out[(size_t)m * N + n] = epilogue(acc, dot_ty, ep_ty, bias != NULL, bv, epi);
@@ -428,6 +440,7 @@ XO_API int xo_fp8_scaled_dot(const uint8_t* A8, const uint8_t* B8, int b_is_nk,
     }
     free(col);
   }
+  free(Ad);
   return rc;
 }
 

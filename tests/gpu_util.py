@@ -19,7 +19,7 @@ def dev_s8(a):
 
 
 def dev_f32(a):
-    return torch.from_numpy(np.ascontiguousarray(a, np.float32).copy()).cuda()
+    return torch.from_numpy(np.array(a, np.float32, order="C")).cuda()  # keeps a 0-d array 0-d
 
 
 def host_bf16(t):

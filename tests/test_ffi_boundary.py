@@ -111,9 +111,18 @@ def test_shape_validation_happens_before_any_launch():
          (dtypes.F32, FAKE, ())]
     with pytest.raises(ffi.FfiError, match="xla_amd.fp8_scaled_dot: result shape must be M,N"):
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a, [(dtypes.BF16, FAKE, (4, 5))]))
-    with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0 but got 1"):
+    # a scale is one value, or a vector along the operand's free dimension
+    with pytest.raises(ffi.FfiError, match="xla_amd.fp8_scaled_dot: a rank-1 a_scale must have M elements"):
         a2 = list(a)
-        a2[2] = (dtypes.F32, FAKE, (1,))
+        a2[2] = (dtypes.F32, FAKE, (3,))
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
+    with pytest.raises(ffi.FfiError, match="xla_amd.fp8_scaled_dot: a rank-1 b_scale must have N elements"):
+        a2 = list(a)
+        a2[3] = (dtypes.F32, FAKE, (8,))
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
+    with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0..1 but got 2"):
+        a2 = list(a)
+        a2[2] = (dtypes.F32, FAKE, (4, 1))
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
 
 

@@ -51,8 +51,9 @@ def floor_for(w, exact_kernel=False):
     neighbours of 4.0, but not of 16.0).  Each product therefore carries an error of up to
     2^-13 of its group's maximum; summed as a random walk that is 2^-13 * sqrt(sum (a*b)^2),
     taken with a factor 2 of slack and 1.2 for the slope of GELU/SiLU."""
-    a = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * float(w["a_scale"])
-    b = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * float(w["b_scale"])
+    sa, sb = np.asarray(w["a_scale"], np.float64), np.asarray(w["b_scale"], np.float64)
+    a = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * (sa[:, None] if sa.ndim else sa)
+    b = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * (sb[None, :] if sb.ndim else sb)
     f32_order = dot_floor(a, b, w["a"].shape[1])
     if exact_kernel:
         return f32_order
@@ -92,6 +93,52 @@ def test_rhs_layouts_take_their_own_paths(oracle):
     assert kern == "fp8_scaled_dot_tiled+transpose", kern
     # K = 128: many outputs sit on the flat tail of GELU, where only the floor clause is meaningful
     assert check_dot(got, reference(oracle, w2), floor_for(w2), kern) <= got.size // 25
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("which", ["a", "b", "ab"])
+def test_vector_scales(oracle, which, nk):
+    """a_scale per row of a and/or b_scale per output channel, on ragged tiles."""
+    say("fp8_scaled_dot vector scales %s nk=%s" % (which, nk))
+    M, K, N = 300, 512, 272
+    w = workloads.c3_fp8(M, K, N)
+    rng = np.random.default_rng(17)
+    if "a" in which:
+        w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+    if "b" in which:
+        w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    got, kern = run(w, nk=nk)
+    assert kern.startswith("fp8_scaled_dot_tiled"), kern
+    n_floor = check_dot(got, reference(oracle, w), floor_for(w), kern)
+    assert n_floor <= got.size // 100
+    # the slow kernel takes the same vectors (and is the one a bf16-typed multiply gets)
+    got, kern = run(w, nk=nk, force=1)
+    assert kern == "fp8_scaled_dot_exact", kern
+    check_dot(got, reference(oracle, w), floor_for(w, exact_kernel=True), kern)
+    got, kern = run(w, nk=nk, dequant_type="bf16")
+    assert kern == "fp8_scaled_dot_exact", kern
+    check_dot(got, reference(oracle, w, dequant_type="bf16"), floor_for(w, exact_kernel=True), kern)
+
+
+def test_quantized_rows_feed_the_dot(oracle):
+    """rowwise_quantize_fp8 -> fp8_scaled_dot: the quantizer's codes and per-row scales go
+    straight in as a and a_scale.  Codes and scales are bit-exact against the oracle, so the
+    dot is compared on the oracle's own chain."""
+    say("rowwise_quantize_fp8 feeding fp8_scaled_dot")
+    R, C, N = 200, 1024, 256
+    x = workloads.c4_quantize(R, C)
+    q, s = ops.rowwise_quantize_fp8(dev_bf16(x["x"]), dev_bf16(x["gamma"]), eps=1e-6)
+    w = workloads.c3_fp8(R, C, N)
+    b, sb = dev_u8(w["b"]), dev_f32(np.array(w["b_scale"], np.float32))
+    out = ops.fp8_scaled_dot(q, b, s, sb, dev_bf16(w["bias"]), epilogue="BIAS_GELU")
+    torch.cuda.synchronize()
+    kern = ffi.last_kernel()
+    assert kern.startswith("fp8_scaled_dot_tiled"), kern
+    q_ref, s_ref = oracle.rmsnorm_quantize_fp8(x["x"], x["gamma"], eps=1e-6)
+    assert np.array_equal(q.cpu().numpy().view(np.uint8), q_ref) and np.array_equal(s.cpu().numpy(), s_ref)
+    w.update(a=q_ref, a_scale=s_ref)
+    n_floor = check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    assert n_floor <= out.numel() // 100
 
 
 def test_fp8_one_hot_exact(oracle):

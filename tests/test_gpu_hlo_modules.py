@@ -68,6 +68,42 @@ def test_c3_module():
     check_dot(host_bf16(out), ref, dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "C3 module")
 
 
+def test_c3_module_vector_scales():
+    say("module C3 with per-row / per-channel scales")
+    M, K, N = 128, 256, 144
+    w = workloads.c3_fp8(M, K, N)
+    text = hm.c3_fp8(M, K, N, vector_scales=True)
+    rng = np.random.default_rng(8)
+    sa = rng.uniform(0.004, 0.04, M).astype(np.float32)
+    sb = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(w["a"]), dev_u8(w["b"]), dev_f32(sa), dev_f32(sb), dev_bf16(w["bias"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"]
+    ref = reference(text, [w["a"], w["b"], sa, sb, w["bias"]])
+    fa = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * sa[:, None]
+    fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * sb[None, :]
+    check_dot(host_bf16(out), ref, dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "C3 vector scales")
+
+
+def test_quantize_then_fp8_dot_module(oracle):
+    """RMSNorm + quantize feeding an f8 dot: two custom calls after the pass, against the op-by-op
+    evaluation of the original module."""
+    say("module quantize -> fp8 dot")
+    R, C, N = 96, 512, 128
+    x = workloads.c4_quantize(R, C)
+    w = workloads.c3_fp8(R, C, N)
+    sw = np.array(1 / 64, np.float32)
+    text = hm.quantize_then_fp8_dot(R, C, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(x["x"]), dev_bf16(x["gamma"]), dev_u8(w["b"]), dev_f32(sw)])
+    torch.cuda.synchronize()
+    assert rw == ["q -> xla_amd.rowwise_quantize_fp8 [rmsnorm]", "dot -> xla_amd.fp8_scaled_dot [DEFAULT]"]
+    ref = reference(text, [x["x"], x["gamma"], w["b"], sw])
+    q, s = oracle.rmsnorm_quantize_fp8(x["x"], x["gamma"], eps=1e-6)
+    fa = np.abs(dtypes.f8e4m3fn_to_f32(q).astype(np.float64)) * s[:, None]
+    fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) / 64
+    check_dot(host_bf16(out), ref, dot_floor(fa, fb, C) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "quantize -> dot")
+
+
 @pytest.mark.parametrize("rmsnorm", [True, False])
 def test_c4_module_bit_exact(rmsnorm):
     say("module C4 rmsnorm=%s" % rmsnorm)

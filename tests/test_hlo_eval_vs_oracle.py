@@ -40,6 +40,29 @@ def test_c3(oracle, typed):
     assert np.array_equal(got, ref)
 
 
+def test_c3_vector_scales(oracle):
+    """a_scale per row of a, b_scale per output channel: the broadcasts run along dimension 0
+    of a and dimension 1 of b."""
+    M, K, N = 12, 64, 20
+    w = workloads.c3_fp8(M, K, N)
+    rng = np.random.default_rng(4)
+    sa = rng.uniform(0.005, 0.05, M).astype(np.float32)
+    sb = rng.uniform(0.005, 0.05, N).astype(np.float32)
+    got = run_module(hm.c3_fp8(M, K, N, vector_scales=True), [w["a"], w["b"], sa, sb, w["bias"]])
+    ref = oracle.fp8_scaled_dot(w["a"], w["b"], sa, sb, bias=w["bias"], epilogue="gelu_tanh")
+    assert np.array_equal(got, ref)
+
+
+def test_quantize_then_fp8_dot(oracle):
+    R, C, N = 6, 96, 10
+    x = workloads.c4_quantize(R, C)
+    w = workloads.c3_fp8(R, C, N)
+    sw = np.array(1 / 32, np.float32)
+    got = run_module(hm.quantize_then_fp8_dot(R, C, N), [x["x"], x["gamma"], w["b"], sw])
+    q, s = oracle.rmsnorm_quantize_fp8(x["x"], x["gamma"], eps=1e-6)
+    assert np.array_equal(got, oracle.fp8_scaled_dot(q, w["b"], s, sw))
+
+
 @pytest.mark.parametrize("rows,cols", [(4, 256), (3, 1000), (2, 33)])
 def test_c4(oracle, rows, cols):
     w = workloads.c4_quantize(rows, cols)

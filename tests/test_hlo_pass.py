@@ -101,6 +101,37 @@ def test_c3_fp8_bias_gelu(typed, code):
         check(new, r"%a_scale.f32 = f32\[\] convert\(%a_scale\)", r"%b_scale.f32 = f32\[\] convert\(%b_scale\)")
 
 
+def test_c3_fp8_vector_scales():
+    """Scales broadcast along the free dimension of each operand (rows of a, channels of b)
+    go in as rank-1 operands; along the contracting dimension they do not factor out of the
+    sum and the dot is left alone, with the reason logged."""
+    text = hm.c3_fp8(64, 128, 32, vector_scales=True)
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"] and rf == []
+    check(new, r"custom-call\(%a, %b, %a_scale, %b_scale, %bias\), custom_call_target=\"xla_amd.fp8_scaled_dot\"")
+    assert "%a_scale = f32[64] parameter(2)" in new and "%b_scale = f32[32] parameter(3)" in new
+    bad = text.replace("%a_scale = f32[64] parameter(2)", "%a_scale = f32[128] parameter(2)") \
+              .replace("broadcast(%a_scale), dimensions={0}", "broadcast(%a_scale), dimensions={1}")
+    new, rw, rf = hlo.rewrite(bad)
+    assert rw == [] and "custom-call" not in new
+    assert len(rf) == 1 and "lhs scales vary along the contracting dimension" in rf[0]
+    bad = text.replace("%b_scale = f32[32] parameter(3)", "%b_scale = f32[128] parameter(3)") \
+              .replace("broadcast(%b_scale), dimensions={1}", "broadcast(%b_scale), dimensions={0}")
+    new, rw, rf = hlo.rewrite(bad)
+    assert rw == [] and len(rf) == 1 and "rhs scales vary along the contracting dimension" in rf[0]
+
+
+def test_quantizer_feeding_a_dot_becomes_two_calls():
+    """The quantizer's broadcast scales are reused by the dequantising multiply of the next dot:
+    both patterns are taken, the dot reads the quantizer's two results, and none of the
+    RMSNorm / amax / divide chain survives."""
+    new, rw, rf = hlo.rewrite(hm.quantize_then_fp8_dot(64, 256, 32))
+    assert rw == ["q -> xla_amd.rowwise_quantize_fp8 [rmsnorm]", "dot -> xla_amd.fp8_scaled_dot [DEFAULT]"] and rf == []
+    check(new, r"custom-call\(%x, %gamma\), custom_call_target=\"xla_amd.rowwise_quantize_fp8\"",
+          r"custom-call\(%q.codes, %w, %scale.scales, %w_scale\), custom_call_target=\"xla_amd.fp8_scaled_dot\"")
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+
+
 def test_c4_quantize_rmsnorm_and_plain():
     new, rw, rf = hlo.rewrite(hm.c4_quantize())
     assert rw == ["q -> xla_amd.rowwise_quantize_fp8 [rmsnorm]"] and rf == []

@@ -182,6 +182,36 @@ def test_fp8_dot_one_hot(oracle):
     assert np.array_equal(as_f32(out), as_f32(want))       # value compare: -0 sums to +0
 
 
+def test_fp8_dot_vector_scales(oracle):
+    """Per-row a_scale and per-channel b_scale: a vector of equal values is the per-tensor
+    case bit for bit; power-of-two vectors scale row m / column n exactly (so each output is
+    the unscaled sum times sa[m]*sb[n] before the one rounding); general vectors against f64;
+    and a transposed index (scales along the wrong axis) must change the result."""
+    rng = np.random.default_rng(21)
+    M, K, N = 7, 48, 9
+    a8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 32, -448, 448))
+    b8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((K, N)) * 32, -448, 448))
+    for nk in (False, True):
+        bm = np.ascontiguousarray(b8.T) if nk else b8
+        same = oracle.fp8_scaled_dot(a8, bm, np.full(M, 0.3, np.float32), np.full(N, 0.7, np.float32), b_is_nk=nk)
+        assert np.array_equal(same, oracle.fp8_scaled_dot(a8, bm, np.float32(0.3), np.float32(0.7), b_is_nk=nk))
+        sa = (2.0 ** rng.integers(-6, 3, M)).astype(np.float32)
+        sb = (2.0 ** rng.integers(-6, 3, N)).astype(np.float32)
+        got = as_f32(oracle.fp8_scaled_dot(a8, bm, sa, sb, b_is_nk=nk))
+        unit = dtypes.f8e4m3fn_to_f32(a8).astype(np.float64) @ dtypes.f8e4m3fn_to_f32(b8).astype(np.float64)
+        # |sum| < 2^24 * 2^-6 granularity: the f32 sums of these f8 products are exact
+        want = as_f32(bf16((unit * sa[:, None] * sb[None, :]).astype(np.float32)))
+        assert np.array_equal(got, want)
+        sa = rng.uniform(0.01, 2.0, M).astype(np.float32)
+        sb = rng.uniform(0.01, 2.0, N).astype(np.float32)
+        got = as_f32(oracle.fp8_scaled_dot(a8, bm, sa, sb, b_is_nk=nk)).astype(np.float64)
+        ref = unit * sa[:, None].astype(np.float64) * sb[None, :]
+        assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -8 + 1e-6)
+        if not nk:
+            wrong = unit * sa[::-1, None].astype(np.float64) * sb[None, :]
+            assert not np.all(np.abs(got - wrong) <= np.abs(wrong) * 2.0 ** -8 + 1e-6)
+
+
 # ---- RMSNorm + quantize -----------------------------------------------------------
 
 def test_tree32_sum_order(oracle):

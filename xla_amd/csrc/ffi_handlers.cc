@@ -390,8 +390,8 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   const uint64_t f8 = Bit(XLA_FFI_DataType_F8E4M3FN);
   XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 2, "a");
   XLA_FFI_Buffer* b = d.Arg(1, f8, 2, 2, "b");
-  XLA_FFI_Buffer* sa = d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 0, "a_scale");
-  XLA_FFI_Buffer* sb = d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 0, "b_scale");
+  XLA_FFI_Buffer* sa = d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
+  XLA_FFI_Buffer* sb = d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
   XLA_FFI_Buffer* bias = f->args.size > 4 ? d.Arg(4, kFloatMask, 1, 1, "bias") : nullptr;
   XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16), 2, 2, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
@@ -412,10 +412,14 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
     else if (out->dims[0] != p.M || out->dims[1] != p.N) why = "result shape must be M,N";
     else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
     else if (((at.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
+    else if (sa->rank == 1 && sa->dims[0] != p.M) why = "a rank-1 a_scale must have M elements";
+    else if (sb->rank == 1 && sb->dims[0] != p.N) why = "a rank-1 b_scale must have N elements";
   }
   if (!why.empty()) return InvalidArgument(f->api, "xla_amd.fp8_scaled_dot: " + why);
   p.a = a->data; p.b = b->data;
   p.a_scale = (const float*)sa->data; p.b_scale = (const float*)sb->data;
+  p.a_scale_per_row = sa->rank == 1;
+  p.b_scale_per_channel = sb->rank == 1;
   p.bias = bias ? bias->data : nullptr;
   p.out = out->data;
   p.workspace = ws ? ws->data : nullptr;

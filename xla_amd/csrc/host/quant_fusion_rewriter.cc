@@ -2,7 +2,8 @@
 // each with one typed-FFI custom call to this library's kernels, in the place where XLA's
 // GemmFusion / GemmRewriter run (xla/service/gpu/gpu_compiler.cc:2113-2129):
 //
-//   convert(f8e4m3fn) [* or / broadcast(scalar)] -> dot [-> +bias] [-> relu|gelu|silu]
+//   convert(f8e4m3fn) [* or / broadcast(scalar) | * broadcast(per-row / per-channel vector)]
+//       -> dot [-> +bias] [-> relu|gelu|silu]
 //       => xla_amd.fp8_scaled_dot          (what gemm_rewriter.cc:190-336,1235-1591 turns into
 //                                           __cublas$lt$matmul$f8, epilogues :888-1007,1987-2304)
 //   convert(s8|s4) * broadcast(scale) -> dot [-> +bias] [-> activation]
@@ -272,23 +273,37 @@ Instr* AsF32Scalar(Computation* comp, Instr* s, const Instr* before) {
 // ---------------------------------------------------------------- f8 scaled dot
 struct F8Operand {
   Instr* value = nullptr;   // the f8e4m3fn tensor
-  Instr* scale = nullptr;   // scalar, null = 1
+  Instr* scale = nullptr;   // scalar or vector, null = 1
   bool divide = false;
+  int64_t scale_dim = -1;   // the operand dimension a rank-1 scale runs along; -1 for a scalar
   std::string type;         // element type of the convert / multiply
 };
+
+// broadcast(scalar), or broadcast(vector) along one dimension of a rank-2 operand
+bool ScaleBroadcast(const Instr* i, Instr** scale, int64_t* dim) {
+  *dim = -1;
+  if (ScalarBroadcast(i, scale)) return true;
+  if (!i->Is("broadcast") || i->shape.rank() != 2 || i->operands[0]->shape.rank() != 1) return false;
+  auto dims = i->DimsAttr("dimensions");
+  if (dims.size() != 1 || dims[0] < 0 || dims[0] > 1) return false;
+  *scale = i->operands[0];
+  *dim = dims[0];
+  return true;
+}
 
 bool MatchF8Operand(Instr* op, F8Operand* out) {
   Instr* src;
   if (ConvertFrom(op, "f8e4m3fn", &src)) {
-    *out = {src, nullptr, false, op->shape.dtype};
+    *out = {src, nullptr, false, -1, op->shape.dtype};
     return IsFloatTy(op->shape.dtype);
   }
   Instr *cv = nullptr, *sc = nullptr;
   if (op->Is("multiply")) {
-    if (!BinaryWith(op, "multiply", [&](Instr* s) { return ScalarBroadcast(s, &sc); }, &cv)) return false;
+    if (!BinaryWith(op, "multiply", [&](Instr* s) { return ScaleBroadcast(s, &sc, &out->scale_dim); }, &cv))
+      return false;
   } else if (op->Is("divide")) {
     Instr* b;
-    if (!Binary(op, "divide", &cv, &b) || !ScalarBroadcast(b, &sc)) return false;
+    if (!Binary(op, "divide", &cv, &b) || !ScaleBroadcast(b, &sc, &out->scale_dim)) return false;
     out->divide = true;
   } else {
     return false;
@@ -321,12 +336,25 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
 
   const int64_t M = a.value->shape.dims[0], K = a.value->shape.dims[1], N = b.value->shape.dims[1 - rc[0]];
+  // a vector of scales must run along the operand's free dimension (rows of a, output channels
+  // of b): along K it does not factor out of the sum
+  if (a.scale_dim == 1) return refuse("the lhs scales vary along the contracting dimension");
+  if (b.scale_dim == rc[0]) return refuse("the rhs scales vary along the contracting dimension");
+  if ((a.scale_dim >= 0 || b.scale_dim >= 0) && a.type != "f32")
+    return refuse("per-row / per-channel scales are taken with an f32 multiply only");
+  if ((a.scale_dim >= 0 && a.divide) || (b.scale_dim >= 0 && b.divide))
+    return refuse("a division by a vector of scales is not taken");
   auto scale_of = [&](const F8Operand& o) -> Instr* {
     Instr* s = o.scale;
     if (!s) {
       auto one = Make(comp->UniqueName("one"), "constant", Shape::Array("f32", {}), {});
       one->literal = "1";
       return comp->Insert(std::move(one), ep.tail);
+    }
+    if (o.scale_dim >= 0) {
+      if (s->shape.dtype == "f32") return s;
+      return comp->Insert(Make(comp->UniqueName(s->name + ".f32"), "convert", Shape::Array("f32", s->shape.dims), {s}),
+                          ep.tail);
     }
     s = AsF32Scalar(comp, s, ep.tail);
     if (o.divide) {
@@ -551,11 +579,11 @@ bool RewriteQuantize(const Module& mod, Computation* comp, Instr* q, RewriteLog*
                          {Shape::Array("f8e4m3fn", {R, C}), Shape::Array("f32", {R})}, cfg);
   Instr* s_new = EmitGte(comp, call, 1, s, s->name + ".scales");
   Instr* q_new = EmitGte(comp, call, 0, s, q->name + ".codes");
-  // every user of the scale other than the pattern's own broadcast keeps working on s_new
+  // every user of the scale works on s_new from here on; the pattern's own broadcast too, which
+  // may feed a dequantising multiply further down besides the divide that dies with q
   for (auto& i : comp->instrs)
-    if (i.get() != sb)
-      for (Instr*& op : i->operands)
-        if (op == s) op = s_new;
+    for (Instr*& op : i->operands)
+      if (op == s) op = s_new;
   if (s->is_root) { s->is_root = false; s_new->is_root = true; }
   comp->ReplaceAllUses(q, q_new);
   log->rewrites.push_back(q->name + " -> xla_amd.rowwise_quantize_fp8 [" + (rms ? "rmsnorm" : "plain") + "]");

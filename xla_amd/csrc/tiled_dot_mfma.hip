@@ -41,8 +41,8 @@ constexpr int kRow = 128;            // bytes of K per LDS row per stage
 struct TiledParams {
   const uint8_t* a;     // kFp8: f8 [M,K]; kS8: bf16 [batch,M,K]
   const uint8_t* b;     // kFp8: f8 [N,K]; kFp8KN: f8 [K,N]; kS8: s8 [batch,K,N]
-  const float* a_scale; // kFp8 device scalars
-  const float* b_scale;
+  const float* a_scale; // kFp8: one value, or M (a_per_row)
+  const float* b_scale; // kFp8: one value, or N (b_per_channel)
   const void* scales;   // kS8: [scale_batch, N]
   const void* bias;
   uint16_t* out;        // [batch, M, N]
@@ -51,6 +51,7 @@ struct TiledParams {
   int bf16_dot, bf16_ops, epilogue;
   int tiles_m, tiles_n;
   int require_pow2_scales;  // kFp8 with a bf16-typed dequantise multiply: exact only then
+  int a_per_row, b_per_channel;
 };
 
 __device__ __forceinline__ bool is_pow2_f32(float s) {
@@ -376,7 +377,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever indexed
   // statically.  The rolled read loop carries the epilogue.
   float alpha = 1.0f;
-  if (F8) alpha = *p.a_scale * *p.b_scale;
+  if (F8) alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
   float* stage = reinterpret_cast<float*>(lds + wave * 16384);
   const int rd_chunk = lane & 15, rd_row = lane >> 4;  // read side: chunk of 4 channels, row within 4
   const bool n_vec = (p.N & 3) == 0;
@@ -387,6 +388,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   for (int t = 0; t < 4; ++t) {
     const bool ok = n + t < p.N;
     d.sc[t] = alpha;
+    if (F8 && p.b_per_channel) d.sc[t] = alpha * p.b_scale[ok ? n + t : 0];
     if (KIND == kS8) {
       const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
       d.sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
@@ -406,6 +408,16 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.out = p.out + (size_t)batch * p.M * p.N;
   d.n_vec = n_vec;
   d.has_bias = p.bias != nullptr;
+  if (F8 && p.a_per_row) {
+    // one scale per token row: all 16 registers of a tile belong to the lane's one token
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int m = m0 + wm * 128 + mt * 32 + l32;
+      const float rs = p.a_scale[m < p.M ? m : p.M - 1];
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) acc[nt][mt] *= rs;
+    }
+  }
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
@@ -495,7 +507,7 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
   const int n = (int)(idx % p.N), m = (int)(idx / p.N);
-  float sa = *p.a_scale, sb = *p.b_scale;
+  float sa = p.a_scale[p.a_per_row ? m : 0], sb = p.b_scale[p.b_per_channel ? n : 0];
   if (deq_bf16) { sa = round_bf16(sa); sb = round_bf16(sb); }
   float acc = 0.0f;
   for (int k = 0; k < p.K; ++k) {
@@ -584,6 +596,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.b = (const uint8_t*)p.b;
   tp.a_scale = p.a_scale;
   tp.b_scale = p.b_scale;
+  tp.a_per_row = p.a_scale_per_row != 0;
+  tp.b_per_channel = p.b_scale_per_channel != 0;
   tp.bias = (p.epilogue & 1) ? p.bias : nullptr;
   tp.out = (uint16_t*)p.out;
   tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
@@ -595,10 +609,14 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   const bool deq_bf16 = p.dequant_type == XLA_FFI_DataType_BF16;
   tp.require_pow2_scales = deq_bf16;
+  // a vector of scales cannot be tested for powers of two in one place: with a bf16-typed
+  // multiply it takes the exact kernel
+  const bool vector_scales = tp.a_per_row || tp.b_per_channel;
 
   const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled
   const bool nk = p.rhs_contracting_dim == 1;
   bool tiled_ok = p.K % 16 == 0 && p.K > 0 && ((uintptr_t)p.a % 16 == 0) && force != 1 &&
+                  !(deq_bf16 && vector_scales) &&
                   (double)p.M * p.K < 2147483000.0 && (double)p.N * p.K < 2147483000.0;
   const uint8_t* b_nk = (const uint8_t*)p.b;
   // a [K,N] rhs with whole 16-channel chunks goes in as it is: the kernel stages it K-major and

@@ -71,12 +71,17 @@ ENTRY %main {{
 """
 
 
-def c3_fp8(M=8192, K=8192, N=8192, typed="f32"):
+def c3_fp8(M=8192, K=8192, N=8192, typed="f32", vector_scales=False):
     """f8 [M,K] . f8 [K,N] with per-tensor scales, + bias, GELU(tanh) -> bf16.  typed="f32":
     f32 ops and one final rounding; typed="bf16": every op bf16-typed (the shape of
-    gemm_rewriter_fp8_test.cc:1110-1141)."""
+    gemm_rewriter_fp8_test.cc:1110-1141).  vector_scales: a_scale is f32[M], one per row of a
+    (what a row-wise quantizer hands on), and b_scale f32[N], one per output channel."""
     t = typed
     scale_decl = (f"  %a_scale = {t}[] parameter(2)\n  %b_scale = {t}[] parameter(3)\n")
+    a_dims, b_dims = "", ""
+    if vector_scales:
+        scale_decl = (f"  %a_scale = {t}[{M}] parameter(2)\n  %b_scale = {t}[{N}] parameter(3)\n")
+        a_dims, b_dims = "0", "1"
     tail = (f"  ROOT %out = bf16[{M},{N}] convert(%gelu)\n" if t == "f32" else "")
     root = "" if t == "f32" else "ROOT "
     bias_line = (f"  %bias_t = f32[{N}] convert(%bias)\n" if t == "f32" else "")
@@ -89,8 +94,8 @@ ENTRY %main {{
 {scale_decl}  %bias = bf16[{N}] parameter(4)
   %a_t = {t}[{M},{K}] convert(%a)
   %b_t = {t}[{K},{N}] convert(%b)
-  %a_scale_b = {t}[{M},{K}] broadcast(%a_scale), dimensions={{}}
-  %b_scale_b = {t}[{K},{N}] broadcast(%b_scale), dimensions={{}}
+  %a_scale_b = {t}[{M},{K}] broadcast(%a_scale), dimensions={{{a_dims}}}
+  %b_scale_b = {t}[{K},{N}] broadcast(%b_scale), dimensions={{{b_dims}}}
   %a_deq = {t}[{M},{K}] multiply(%a_t, %a_scale_b)
   %b_deq = {t}[{K},{N}] multiply(%b_t, %b_scale_b)
   %dot = {t}[{M},{N}] dot(%a_deq, %b_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
@@ -167,6 +172,27 @@ ENTRY %main {{
   %clamped = f32[{R},{C}] clamp(%lo_b, %scaled, %hi_b)
   %q = f8e4m3fn[{R},{C}] convert(%clamped)
   ROOT %result = (f8e4m3fn[{R},{C}], f32[{R}]) tuple(%q, %scale)
+}}
+"""
+
+
+def quantize_then_fp8_dot(rows=16384, cols=8192, N=8192, eps=1e-6):
+    """One layer boundary: RMSNorm + row-wise f8e4m3fn quantisation of x[rows,cols] (the C4
+    pattern), whose codes and per-row scales are dequantised straight into a dot with f8
+    weights [cols,N] under a per-tensor scale -> bf16 [rows,N]."""
+    R, C = rows, cols
+    text = c4_quantize(rows, cols, rmsnorm=True, eps=eps).replace("HloModule c4_rowwise_quantize_fp8",
+                                                                  "HloModule quantize_then_fp8_dot")
+    head, _ = text.split("  ROOT %result")
+    return head + f"""  %w = f8e4m3fn[{C},{N}] parameter(2)
+  %w_scale = f32[] parameter(3)
+  %q_f32 = f32[{R},{C}] convert(%q)
+  %a_deq = f32[{R},{C}] multiply(%q_f32, %scale_b)
+  %w_f32 = f32[{C},{N}] convert(%w)
+  %w_scale_b = f32[{C},{N}] broadcast(%w_scale), dimensions={{}}
+  %w_deq = f32[{C},{N}] multiply(%w_f32, %w_scale_b)
+  %dot = f32[{R},{N}] dot(%a_deq, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
+  ROOT %out = bf16[{R},{N}] convert(%dot)
 }}
 """
 

@@ -88,14 +88,16 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
 def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, epilogue="DEFAULT",
                    dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto",
                    build_only=False):
-    """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K]; scales f32 []."""
+    """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K];
+    a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel)."""
     _check_cuda(a, b, a_scale, b_scale, bias)
     m, k = a.shape
     n = b.shape[1 - rhs_contracting_dim]
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
     args = [(dtypes.F8E4M3FN, a.data_ptr(), a.shape), (dtypes.F8E4M3FN, b.data_ptr(), b.shape),
-            (dtypes.F32, a_scale.data_ptr(), []), (dtypes.F32, b_scale.data_ptr(), [])]
+            (dtypes.F32, a_scale.data_ptr(), list(a_scale.shape)),
+            (dtypes.F32, b_scale.data_ptr(), list(b_scale.shape))]
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
     rets = [(dtypes.BF16, out.data_ptr(), [m, n])]
