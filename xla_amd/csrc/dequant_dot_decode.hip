@@ -113,16 +113,30 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   const int n_lane = strip * TN + li * NV;   // first channel of this lane (may be >= N: discarded)
   const uint32_t pitch = (uint32_t)(((size_t)p.N * WBITS) >> 3);  // bytes per row of W
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.w + (size_t)batch * p.K * pitch, (uint32_t)p.K * pitch);
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.lhs + (size_t)batch * p.M * p.K, (uint32_t)p.M * p.K * 2u);
+  // one descriptor per 16-token tile, each ending where the activations end: the per-lane offset
+  // is then the same for every tile (token li of the tile) and still range-checks tokens >= M
+  __amdgpu_buffer_rsrc_t ra[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int rows = max(p.M - 16 * mt, 0);
+    ra[mt] = make_rsrc(p.lhs + ((size_t)batch * p.M + (rows ? 16 * mt : 0)) * p.K, (uint32_t)rows * p.K * 2u);
+  }
   const int groups = p.K / p.group;
   const __amdgpu_buffer_rsrc_t rs =
       make_rsrc((const char*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N * SSZ,
                 (uint32_t)groups * p.N * SSZ);
-  const uint32_t voff_w = (uint32_t)(8 * kb) * pitch + (uint32_t)((n_lane * WBITS) >> 3);
-  uint32_t voff_a[MT];
+  // a lane whose channels lie beyond N (last strip) gets an offset no buffer reaches: all its
+  // loads return zeros and nothing is read outside the operands
+  constexpr uint32_t kNowhere = 0x80000000u;
+  const bool lane_live = n_lane < p.N;
+  const uint32_t voff_w = lane_live ? (uint32_t)(8 * kb) * pitch + (uint32_t)((n_lane * WBITS) >> 3) : kNowhere;
+  const uint32_t voff_a = ((uint32_t)li * p.K + 8 * kb) * 2u;
+  // rows r = 1..7 of a lane's block of 8 are reached through the scalar offset: K % 8 == 0, so
+  // the block is inside the weights exactly when its first row is, which the lane offset checks
+  uint32_t soff_w[8];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) voff_a[mt] = ((uint32_t)(mt * 16 + li) * p.K + 8 * kb) * 2u;
-  const uint32_t voff_s = (uint32_t)n_lane * SSZ;
+  for (int r = 0; r < 8; ++r) soff_w[r] = (uint32_t)r * pitch;
+  const uint32_t voff_s = lane_live ? (uint32_t)n_lane * SSZ : kNowhere;
 
   floatx4 acc[NV][MT];
 #pragma unroll
@@ -150,9 +164,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     return !GROUP32 || k0 == k_begin || ((k0 >> 5) % steps_per_group) == 0;
   };
   auto load_step = [&](int buf, int k0) {
+    const uint32_t va = voff_a + (uint32_t)k0 * 2u;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      aq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a[mt] + (uint32_t)k0 * 2u, 0, 0);
+    for (int mt = 0; mt < MT; ++mt) aq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], va, 0, 0);
     if (MODE == kRounded) {
       if (GROUP32) {
         if (opens_group(k0)) {
@@ -164,24 +178,28 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
         buffer_load_words<SW>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, sraw[buf]);
       }
     }
+    const uint32_t vw = voff_w + (uint32_t)k0 * pitch;
 #pragma unroll
-    for (int r = 0; r < 8; ++r)
-      buffer_load_words<WORDS>(rw, voff_w + (uint32_t)(k0 + r) * pitch, 0, wq[buf][r]);
+    for (int r = 0; r < 8; ++r) buffer_load_words<WORDS>(rw, vw, soff_w[r], wq[buf][r]);
   };
 
   auto compute = [&](int buf, int k0) {
     // activations: 8 consecutive k of token (16*mt + li); tokens >= M read past the buffer -> 0
+    uintx4 av[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) av[mt] = aq[buf][mt];
+    if (k0 + 32 > p.K) {  // scalar condition: only a step that crosses the end of K
+      asm volatile("");   // keeps this one branch: as selects it would cost 4 per tile in every step
+      const bool ok = k0 + 8 * kb < p.K;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        av[mt] = uintx4{ok ? av[mt][0] : 0u, ok ? av[mt][1] : 0u, ok ? av[mt][2] : 0u, ok ? av[mt][3] : 0u};
+    }
     bf16x8 bop[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      uintx4 v = aq[buf][mt];
-      if (k0 + 32 > p.K) {  // scalar condition: only a step that crosses the end of K
-        const bool ok = k0 + 8 * kb < p.K;
-        v = uintx4{ok ? v[0] : 0u, ok ? v[1] : 0u, ok ? v[2] : 0u, ok ? v[3] : 0u};
-      }
-      bop[mt] = __builtin_bit_cast(bf16x8, v);
-    }
+    for (int mt = 0; mt < MT; ++mt) bop[mt] = __builtin_bit_cast(bf16x8, av[mt]);
     if (MODE == kRounded && opens_group(k0)) {
+      asm volatile("");  // a branch, not 2*NV selects per step
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         const uint32_t* raw = sraw[buf];
@@ -207,29 +225,31 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
         // 0x00f000f0 pick nibbles (0,4) / (1,5) of x and (2,6) / (3,7) of x >> 8.  The product
         // with the scale and the removal of the offset are one v_fma_mix_f32 per weight.
         typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
-        halfx2 pr[8][4];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          const uint32_t x = wq[buf][r][q], y = x >> 8;
-          pr[r][0] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
-          pr[r][1] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a));
-          pr[r][2] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(y, 0x000f000fu, 0x64086408u, 0x6a));
-          pr[r][3] = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(y, 0x00f000f0u, 0x64806480u, 0x6a));
-        }
+        for (int sel = 0; sel < 4; ++sel) {  // nibble pairs (0,4), (1,5) of x, then (2,6), (3,7) of x >> 8
+          halfx2 pr[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int j = q * 8 + e;
-          const float sj = MODE == kRounded ? sc[j] : ((e & 1) ? 0.0625f : 1.0f);
-          const float cj = MODE == kRounded ? cc[j] : ((e & 1) ? -72.0f : -1032.0f);
-          float f[8];
+          for (int r = 0; r < 8; ++r) {
+            const uint32_t x = sel < 2 ? wq[buf][r][q] : wq[buf][r][q] >> 8;
+            pr[r] = __builtin_bit_cast(halfx2, (sel & 1) ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a)
+                                                         : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+          }
 #pragma unroll
-          for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][e & 3][e >> 2], sj, cj);
-          uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                      pack_bf16x2(f[6], f[7])};
-          const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+          for (int half = 0; half < 2; ++half) {
+            const int e = sel + 4 * half;
+            const int j = q * 8 + e;
+            const float sj = MODE == kRounded ? sc[j] : ((e & 1) ? 0.0625f : 1.0f);
+            const float cj = MODE == kRounded ? cc[j] : ((e & 1) ? -72.0f : -1032.0f);
+            float f[8];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+            for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][half], sj, cj);
+            uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                        pack_bf16x2(f[6], f[7])};
+            const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[j][mt], 0, 0, 0);
+          }
         }
       } else {
         uint32_t lo[8];
@@ -474,7 +494,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // buffer offsets are 32-bit: keep every operand (plus one loop overrun) below 2 GiB
-    const bool fits32 = (double)p.K * row_bytes + 128.0 * row_bytes < 2147483648.0 &&
+    const bool fits32 = (double)p.K * row_bytes + 1024.0 * row_bytes < 2147483648.0 &&
                         (double)p.M * p.K * 2 < 2147483648.0 &&
                         (double)(p.K / p.group) * p.N * 4 < 2147483648.0;
     const bool shape_ok = p.N % nv == 0 && row_bytes % vec == 0 && nv * mt <= 32 &&
