@@ -120,7 +120,7 @@ def test_quantize_empty_and_errors():
 
 
 def test_c4_full_size_bit_exact(oracle):
-    """BASELINE configuration 4 at full size, every code and scale against the oracle."""
+    """Configuration 4 (bf16 [16384,8192]) at full size, every code and scale against the oracle."""
     say("quantize C4 full 16384x8192")
     w = workloads.c4_quantize()
     q, s = run(w["x"], w["gamma"])
