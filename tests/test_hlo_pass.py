@@ -74,13 +74,21 @@ def test_c1_per_channel_s8():
 
 
 def test_c2_grouped_s4_with_bias_silu():
-    new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=8))
+    # one token: K is split over two workgroups per strip, the scratch result holds their sums
+    new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=1))
     assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
-    want_ws = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 28672, 21)
+    want_ws = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 1, 8192, 28672, 21)
+    assert want_ws == 2 * 1 * 28672 * 4
     check(new, r"custom-call\(%lhs, %w, %scales, %bias\)",
           r'epilogue = \\"BIAS_SILU\\", dequant_type = 16 : i32, dot_type = 11 : i32, epilogue_type = 11 : i32')
     assert "s8[%d]{0})" % want_ws in new
     assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+    # eight tokens: the 224 strips fill the machine, no split, no scratch, a plain array result
+    new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=8))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
+    assert ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 28672, 21) == 0
+    check(new, r"ROOT %\S+ = bf16\[8,28672\]\{1,0\} custom-call\(%lhs, %w, %scales, %bias\)")
+    assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
     # x * logistic(x) is the same activation before LogisticExpander has run
     text = hm.c2_s4_group(M=8)
     text = re.sub(r"  %neg = .*\n  %exp = .*\n  %one = .*\n  %one_b = .*\n  %den = .*\n  %sig = f32(\[\d+,\d+\]) divide.*\n",

@@ -49,7 +49,7 @@ int GetOption(const char* key) {
   return 0;
 }
 
-size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices);
+size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4);
 size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim);
 
 }  // namespace xla_amd
@@ -73,13 +73,7 @@ int xla_amd_launch_rowwise_quantize_fp8(const XlaAmdRowwiseQuantize* p, void* st
 
 size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, int64_t N,
                                            int32_t weight_dtype) {
-  (void)K;
-  (void)weight_dtype;
-  if (M > 64 || M <= 0) return 0;
-  // the decode kernels never use more than 64/M slices (capped at 16)
-  int slices = (int)(64 / M);
-  if (slices > 16) slices = 16;
-  return xla_amd::DequantDotWorkspaceBytes(batch, M, N, slices);
+  return xla_amd::DequantDotDecodeWorkspaceBytes(batch, M, K, N, weight_dtype == XLA_FFI_DataType_S4);
 }
 
 size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,

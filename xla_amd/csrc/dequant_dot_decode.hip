@@ -424,6 +424,37 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
   return slices > 1 ? (size_t)batch * slices * M * N * sizeof(float) : 0;
 }
 
+// K-slices for a decode launch.  One workgroup per CU is enough once the strips alone give about
+// that many (the kernel is bound by its own arithmetic, and every extra slice costs partial sums
+// and a second launch); up to four tokens a second slice still pays.  Fewer strips are split
+// until there are, as long as a wave keeps at least four 32-row steps and the partial sums
+// (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or a quarter
+// of the weight bytes when the strips would leave three quarters of the CUs idle.
+static int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
+  if (int s = GetOption("dequant_dot_slices")) return s;
+  const int64_t want = M <= 4 ? 448 : 192;
+  const double weight_bytes = (double)K * row_bytes;
+  int slices = 1;
+  while (strips * slices * batch < want && K / (slices * 2) >= 128 * waves &&
+         (slices * 2 * M <= 32 ||
+          (strips * batch <= 64 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes)))
+    slices *= 2;
+  return slices;
+}
+
+// What xla_amd_dequant_dot_workspace_bytes reports: the scratch the launch below will use for
+// this shape (the narrowest strips give the most slices), or what a forced slice count needs.
+size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4) {
+  if (M <= 0 || M > 64 || K < 32 || N <= 0 || batch <= 0) return 0;
+  const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  int vec = s4 ? 4 : (mt == 4 ? 4 : 8);
+  if (int v = GetOption("dequant_dot_vec")) vec = v;
+  const int nv = vec * (s4 ? 2 : 1);
+  const int64_t row_bytes = N * (s4 ? 1 : 2) / 2;
+  const int strips = (int)((N + 16 * nv - 1) / (16 * nv));
+  return DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, strips, row_bytes, 8));
+}
+
 int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
   const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4;
   if (!s4 && p.weight_dtype != XLA_FFI_DataType_S8)
@@ -503,22 +534,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
       int waves = 8;
       if (int wv = GetOption("dequant_dot_waves")) waves = wv == 4 ? 4 : 8;
       dp.strips = (int)((p.N + 16 * nv - 1) / (16 * nv));
-      // enough workgroups for ~2 per CU, but never slices that leave a wave without rows
-      int slices = 1;
-      if (int s = GetOption("dequant_dot_slices")) {
-        slices = s;
-      } else {
-        // workgroups wanted; the partial sums cost slices*M*N*4 bytes written and read again,
-        // which is allowed to reach a quarter of the weight bytes when the strips alone would leave
-        // most CUs idle
-        const int want = p.M <= 8 ? 768 : 384;
-        const double weight_bytes = (double)p.K * row_bytes;
-        // and no slice so thin that a wave gets fewer than four 32-row steps
-        while (dp.strips * slices * p.batch < want && p.K / (slices * 2) >= 128 * waves &&
-               (slices * 2 * p.M <= 32 ||
-                (dp.strips * p.batch <= 64 && 2.0 * (slices * 2) * p.M * p.N * 4.0 <= 0.25 * weight_bytes)))
-          slices *= 2;
-      }
+      int slices = DecodeSlices(p.batch, p.M, p.K, p.N, dp.strips, row_bytes, waves);
       if (slices > 1 && (!p.workspace ||
                          p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, slices)))
         slices = 1;
