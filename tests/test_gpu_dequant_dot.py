@@ -104,6 +104,24 @@ def test_s4_decode_variants(oracle, M, vec, slices):
     compare(oracle, w, got, "s4 %s slices=%d" % (kern, slices))
 
 
+@pytest.mark.parametrize("which", ["s4", "s8"])
+def test_sixteen_wave_workgroups(oracle, which):
+    """The whole-CU workgroup (16 waves splitting K, picked by itself only for wide N): ragged K
+    per wave, a ragged last strip and fewer tokens than a tile."""
+    say("dequant_dot 16-wave workgroups " + which)
+    if which == "s4":
+        w = workloads.c2_s4_group(M=5, K=4096 + 160, N=1000, group=32)
+    else:
+        w = workloads.c1_s8_channel(M=13, K=2048 + 72, N=520)
+    ffi.set_option("dequant_dot_waves", 16)
+    try:
+        got, kern = run_dot(w, force_kernel=2)
+    finally:
+        ffi.set_option("dequant_dot_waves", 0)
+    assert "_w16_" in kern, kern
+    compare(oracle, w, got, kern)
+
+
 def test_s4_unpack_and_dequant_bit_exact(oracle):
     """One-hot activations: every output is one dequantised weight, so nibble order, sign
     extension, the scale lookup and the bf16 rounding are checked exactly."""

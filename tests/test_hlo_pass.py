@@ -74,7 +74,7 @@ def test_c1_per_channel_s8():
 
 
 def test_c2_grouped_s4_with_bias_silu():
-    # one token: K is split over two workgroups per strip, the scratch result holds their sums
+    # one token: the scratch result covers the two K-slices per strip an 8-wave launch would use
     new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=1))
     assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
     want_ws = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 1, 8192, 28672, 21)
