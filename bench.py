@@ -61,9 +61,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
-    def ev_time(fn, reps):
+    def ev_time(fn, reps, warm=1):
         """Average device time of fn() over `reps` back-to-back launches, events on the stream."""
-        fn()
+        for _ in range(warm):
+            fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         best = None
@@ -133,7 +134,8 @@ def main():
     other = []
     if not args.skip_other:
         def entry(name, call, bytes_, flops, bound, dtype=None):
-            ms = ev_time(lambda: call.run(), max(3, args.reps // 4))
+            # the half-millisecond kernels get a few launches to settle the clocks before timing
+            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=5 if flops else 1)
             e = {"workload": name, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
                  "GB/s": round(bytes_ / (ms * 1e-3) / 1e9, 1)}
             e["frac_hbm"] = round(e["GB/s"] / HBM_PEAK_GBS, 4)
