@@ -70,9 +70,13 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1);
  *         a_scale F32 [] or [M] (one per row of a, as a row-wise quantizer produces them);
  *         b_scale F32 [] or [N] (one per output channel); bias BF16|F32 [N] (only with BIAS*)
- *   rets: out BF16 [M,N]
+ *         d_scale F32 [] (last; only when out is F8E4M3FN)
+ *   rets: out BF16 [M,N], or F8E4M3FN [M,N] = convert(clamp(-448, v / d_scale, 448)) for the
+ *         f32 value v after the epilogue (the D scaling of gemm_rewriter_fp8_test.cc:1665-1690,
+ *         which GemmRewriter leaves unfused on ROCm, :1710)
  *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
- *          rhs_contracting_dim i64 (default 0)
+ *          rhs_contracting_dim i64 (default 0);
+ *          d_scale_multiplies pred (default false): v * d_scale instead (:1730-1748)
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* call_frame);
 
@@ -153,6 +157,10 @@ typedef struct XlaAmdFp8ScaledDot {
   int32_t epilogue;
   int32_t a_scale_per_row;     /* a_scale is f32[M]: row m of a is scaled by a_scale[m] */
   int32_t b_scale_per_channel; /* b_scale is f32[N]: output channel n of b by b_scale[n] */
+  int32_t out_dtype;           /* 0 or XLA_FFI_DataType_BF16: bf16 out; XLA_FFI_DataType_F8E4M3FN:
+                                  out = convert(clamp(-448, v / *d_scale, 448)), one byte each */
+  int32_t d_scale_multiplies;  /* the f8 result is v * *d_scale instead of v / *d_scale */
+  const float* d_scale;        /* device scalar, only with an F8E4M3FN result */
 } XlaAmdFp8ScaledDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);

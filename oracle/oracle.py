@@ -74,7 +74,7 @@ def lib():
                                      i64, i32, i32, i32, vp]
         L.xo_fp8_scaled_dot.restype = i32
         L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64,
-                                        i32, i32, i32, vp]
+                                        i32, i32, i32, vp, vp, i32, vp, vp]
         L.xo_rmsnorm_quantize_fp8.restype = i32
         L.xo_rmsnorm_quantize_fp8.argtypes = [vp, vp, f32, i64, i64, vp, vp]
         L.xo_num_threads.restype = i32
@@ -201,7 +201,10 @@ def dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, bias=None, bias_ty="
 
 
 def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=None,
-                   bias_ty="bf16", dot_ty="f32", ep_ty="f32", epilogue="none"):
+                   bias_ty="bf16", dot_ty="f32", ep_ty="f32", epilogue="none", d_scale=None,
+                   d_scale_divides=True):
+    """bf16 result [M,N]; with d_scale the f8e4m3fn result convert(clamp(v / d_scale)) (or
+    v * d_scale) and the f32 values v before the scaling, as a pair."""
     a8 = _c(a8, np.uint8)
     b8 = _c(b8, np.uint8)
     M, K = a8.shape
@@ -217,12 +220,19 @@ def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=N
     sb = _c(np.asarray(b_scale, np.float32).reshape(-1), np.float32)
     a_rows, b_cols = np.ndim(a_scale) == 1, np.ndim(b_scale) == 1
     assert sa.size == (M if a_rows else 1) and sb.size == (N if b_cols else 1)
-    out = np.empty((M, N), np.uint16)
+    if d_scale is None:
+        out = np.empty((M, N), np.uint16)
+        tail = (_ptr(out), None, 0, None, None)
+    else:
+        assert dot_ty == "f32" and ep_ty == "f32"
+        sd = _c(np.asarray(d_scale, np.float32).reshape(1), np.float32)
+        out8, val = np.empty((M, N), np.uint8), np.empty((M, N), np.float32)
+        tail = (None, _ptr(sd), int(bool(d_scale_divides)), _ptr(out8), _ptr(val))
     rc = lib().xo_fp8_scaled_dot(_ptr(a8), _ptr(b8), int(b_is_nk), _ptr(sa), int(a_rows), _ptr(sb),
                                  int(b_cols), TYPES[mul_ty], bp, TYPES[bias_ty], M, K, N, TYPES[dot_ty],
-                                 TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
+                                 TYPES[ep_ty], EPILOGUES[epilogue], *tail)
     assert rc == 0
-    return out
+    return out if d_scale is None else (out8, val)
 
 
 def rmsnorm_quantize_fp8(x_bf16, gamma_bf16, eps=1e-6):

@@ -270,8 +270,8 @@ static inline float rnd(float v, int ty) {
  * (a convert sits between them when the types differ); the result is finally
  * converted to bf16.  Op order of GELU follows gemm_rewriter_fp8_test.cc:1123-1141,
  * SiLU follows gemm_rewriter.cc:995-1002 after LogisticExpander. */
-static inline uint16_t epilogue(float acc, int dot_ty, int ep_ty, int has_bias,
-                                float bias, int epi) {
+static inline float epilogue_value(float acc, int dot_ty, int ep_ty, int has_bias,
+                                   float bias, int epi) {
   float x = rnd(acc, dot_ty);
   x = rnd(x, ep_ty); /* convert(dot) -> ep_ty; identity when equal or widening */
   if (has_bias) x = rnd(x + rnd(bias, ep_ty), ep_ty);
@@ -303,7 +303,26 @@ static inline uint16_t epilogue(float acc, int dot_ty, int ep_ty, int has_bias,
     default:
       break;
   }
-  return xo_f32_to_bf16(x);
+  return x;
+}
+
+static inline uint16_t epilogue(float acc, int dot_ty, int ep_ty, int has_bias,
+                                float bias, int epi) {
+  return xo_f32_to_bf16(epilogue_value(acc, dot_ty, ep_ty, has_bias, bias, epi));
+}
+
+/* The f8 result of a dot whose value v (f32-typed ops throughout) is scaled by a per-tensor
+ * factor, clamped and converted: convert(clamp(-448, v / z | v * z, 448)), the tail of
+ * gemm_rewriter_fp8_test.cc:1665-1690 (divide) and :1730-1748 (multiply).  Clamp is
+ * min(max(x, lo), hi) with NaN passed on. */
+static inline uint8_t scaled_f8_result(float v, float z, int divides) {
+  volatile float t = divides ? v / z : v * z;
+  float c = t;
+  if (c == c) {
+    if (c < -448.0f) c = -448.0f;
+    if (c > 448.0f) c = 448.0f;
+  }
+  return xo_f32_to_f8e4m3fn(c);
 }
 
 XO_API uint16_t xo_epilogue_one(float acc, int dot_ty, int ep_ty, int has_bias,
@@ -392,13 +411,16 @@ XO_API int xo_dequant_dot(const uint16_t* A, const void* w, int w_bits,
  * gemm_rewriter_fp8_test.cc:1099-1135) or at M values (a_rows != 0: one per
  * row of A, the broadcast along dimension 0 that a row-wise quantizer's
  * scales are applied with); b_scale at one value or, with b_cols != 0, at N
- * values, one per output channel.
+ * values, one per output channel.  With out8 the result is f8e4m3fn after a
+ * per-tensor scaling by *d_scale (see scaled_f8_result); out_value, if given,
+ * receives the f32 value before that scaling, for tolerance checks.
  */
 XO_API int xo_fp8_scaled_dot(const uint8_t* A8, const uint8_t* B8, int b_is_nk,
                              const float* a_scale, int a_rows, const float* b_scale,
                              int b_cols, int mul_ty, const void* bias, int bias_ty,
                              int64_t M, int64_t K, int64_t N, int dot_ty, int ep_ty,
-                             int epi, uint16_t* out) {
+                             int epi, uint16_t* out, const float* d_scale, int d_divides,
+                             uint8_t* out8, float* out_value) {
   float f8v[256];
   for (int c = 0; c < 256; ++c) f8v[c] = xo_f8e4m3fn_to_f32((uint8_t)c);
   /* the dequantised A once: M*K floats */
@@ -435,7 +457,13 @@ XO_API int xo_fp8_scaled_dot(const uint8_t* A8, const uint8_t* B8, int b_is_nk,
           float p = a[k] * col[k];
           acc = acc + p;
         }
-        out[(size_t)m * N + n] = epilogue(acc, dot_ty, ep_ty, bias != NULL, bv, epi);
+        if (out8) { /* f8 result: f32-typed ops, then scale, clamp, convert */
+          float v = epilogue_value(acc, dot_ty, ep_ty, bias != NULL, bv, epi);
+          if (out_value) out_value[(size_t)m * N + n] = v;
+          out8[(size_t)m * N + n] = scaled_f8_result(v, *d_scale, d_divides);
+        } else {
+          out[(size_t)m * N + n] = epilogue(acc, dot_ty, ep_ty, bias != NULL, bv, epi);
+        }
       }
     }
     free(col);

@@ -59,3 +59,32 @@ def dot_floor(abs_a, abs_w, K):
     """2^-24 * sqrt(K) * sum_k |a_k w_kn|: the scale of the difference between two f32 summation
     orders of the same products (float64 inputs, [..,M,K] @ [..,K,N])."""
     return (2.0 ** -24) * np.sqrt(K) * (abs_a @ abs_w) * 1.25
+
+
+def f8_value(codes):
+    return dtypes.f8e4m3fn_to_f32(np.asarray(codes, np.uint8)).astype(np.float64)
+
+
+def check_f8_result(got_codes, ref_codes, ref_value, d_scale, divides, abs_floor, what=""):
+    """Parity rule for an f8 result convert(clamp(v / z)) of a dot: the oracle's v is only matched
+    to 2 bf16 ulp (or the floor), so a code is accepted when some value within that window of
+    the oracle's v is scaled, clamped and cast to it -- the cast is monotonic, so the code must
+    lie between the codes of the window's ends.  Returns how many codes differ from the oracle's."""
+    got_codes, ref_codes = np.asarray(got_codes, np.uint8), np.asarray(ref_codes, np.uint8)
+    v = np.asarray(ref_value, np.float64)
+    tol = np.maximum(np.abs(v) * 2.0 ** -7, abs_floor)      # 2 ulp of an 8-bit significand
+    z = float(d_scale)
+    def cast(x):
+        t = (x / z if divides else x * z).astype(np.float32)
+        return f8_value(dtypes.f32_to_f8e4m3fn(np.clip(t, -448, 448)))
+    lo, hi = cast(v - tol), cast(v + tol)
+    lo, hi = np.minimum(lo, hi), np.maximum(lo, hi)
+    g = f8_value(got_codes)
+    both_nan = np.isnan(g) & np.isnan(f8_value(ref_codes))
+    bad = ~(((g >= lo) & (g <= hi)) | both_nan)
+    if bad.any():
+        idx = np.argwhere(bad)[:8]
+        raise AssertionError("%s: %d of %d f8 codes outside the window: %s" % (
+            what, int(bad.sum()), bad.size,
+            [(tuple(i), float(g[tuple(i)]), float(lo[tuple(i)]), float(hi[tuple(i)])) for i in idx]))
+    return int((got_codes != ref_codes).sum())

@@ -120,6 +120,15 @@ def test_shape_validation_happens_before_any_launch():
         a2 = list(a)
         a2[3] = (dtypes.F32, FAKE, (8,))
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
+    # an f8e4m3fn result brings its per-tensor scale as the last operand
+    with pytest.raises(ffi.FfiError, match="an F8E4M3FN result takes a, b, a_scale, b_scale, \\[bias,\\] d_scale"):
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a, [(dtypes.F8E4M3FN, FAKE, (4, 4))]))
+    with pytest.raises(ffi.FfiError, match="a BF16 result takes a, b, a_scale, b_scale\\[, bias\\]"):
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.BF16, FAKE, (4,)), (dtypes.F32, FAKE, ())],
+                                                       [(dtypes.BF16, FAKE, (4, 4))], {"epilogue": ffi.Attr.str("BIAS")}))
+    with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0 but got 1 \\(d_scale\\)"):
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.F32, FAKE, (4,))],
+                                                       [(dtypes.F8E4M3FN, FAKE, (4, 4))]))
     with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0..1 but got 2"):
         a2 = list(a)
         a2[2] = (dtypes.F32, FAKE, (4, 1))

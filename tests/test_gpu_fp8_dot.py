@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_u8, dot_floor, host_bf16
+from tests.gpu_util import check_dot, check_f8_result, dev_bf16, dev_f32, dev_u8, dot_floor, host_bf16
 from xla_amd import dtypes, ffi, ops, workloads
 
 pytestmark = pytest.mark.gpu
@@ -139,6 +139,64 @@ def test_quantized_rows_feed_the_dot(oracle):
     w.update(a=q_ref, a_scale=s_ref)
     n_floor = check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
     assert n_floor <= out.numel() // 100
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("mode", ["divide", "multiply", "divide_by_odd_scale", "exact_kernel"])
+def test_f8_result(oracle, mode, nk):
+    """f8e4m3fn result = convert(clamp(v / d_scale)): codes inside the window the dot's own
+    tolerance allows, and nearly all of them equal to the oracle's."""
+    say("fp8_scaled_dot f8 result %s nk=%s" % (mode, nk))
+    M, K, N = 300, 512, 272
+    w = workloads.c3_fp8(M, K, N)
+    divides = mode != "multiply"
+    # all-ones significand: the reciprocal shortcut must step aside for the IEEE divide
+    z = {"divide": np.float32(0.0117), "multiply": np.float32(85.0),
+         "divide_by_odd_scale": np.frombuffer(np.uint32(0x3c7fffff).tobytes(), np.float32)[0],
+         "exact_kernel": np.float32(0.0117)}[mode]
+    a, b = dev_u8(w["a"]), dev_u8(np.ascontiguousarray(w["b"].T) if nk else w["b"])
+    s64 = dev_f32(np.array(1 / 64, np.float32))
+    ffi.set_option("fp8_dot_kernel", 1 if mode == "exact_kernel" else 0)
+    try:
+        out = ops.fp8_scaled_dot(a, b, s64, s64, dev_bf16(w["bias"]), rhs_contracting_dim=1 if nk else 0,
+                                 epilogue="BIAS_GELU", d_scale=dev_f32(np.array(z, np.float32)),
+                                 d_scale_multiplies=not divides)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+    kern = ffi.last_kernel()
+    assert out.dtype == torch.uint8
+    assert ("exact" in kern) == (mode == "exact_kernel") and (mode == "exact_kernel" or kern.endswith("_f8")), kern
+    ref, val = oracle.fp8_scaled_dot(w["a"], w["b"], 1 / 64, 1 / 64, bias=w["bias"], epilogue="gelu_tanh",
+                                     d_scale=z, d_scale_divides=divides)
+    differ = check_f8_result(out.cpu().numpy(), ref, val, z, divides, floor_for(w, exact_kernel=mode == "exact_kernel"), kern)
+    assert differ <= out.numel() // 50, differ
+
+
+def test_f8_result_special_values(oracle):
+    """NaN operands give NaN codes, a huge value over a tiny scale saturates at +-448, -0 stays -0;
+    a zero scale follows IEEE (x/0 = +-inf -> +-448, 0/0 = NaN)."""
+    say("fp8_scaled_dot f8 result special values")
+    M, K, N = 64, 64, 64
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), np.arange(M) % K] = 1.0           # selector rows: out[m, n] = b[m % K, n]
+    bvals = np.zeros((K, N), np.float32)
+    bvals[0, :] = 448.0
+    bvals[1, :] = -448.0
+    bvals[2, :] = 2.0 ** -9
+    bvals[3, :] = -0.0
+    b8 = dtypes.f32_to_f8e4m3fn(bvals)
+    b8[4, N - 1] = 0x7F                                # NaN: the whole last column (0 * NaN = NaN)
+    a8 = dtypes.f32_to_f8e4m3fn(a)
+    one = dev_f32(np.array(1.0, np.float32))
+    for z in (np.float32(1e-30), np.float32(0.0), np.float32(3.0)):
+        out = ops.fp8_scaled_dot(dev_u8(a8), dev_u8(b8), one, one, d_scale=dev_f32(np.array(z, np.float32)))
+        torch.cuda.synchronize()
+        ref, _ = oracle.fp8_scaled_dot(a8, b8, 1.0, 1.0, d_scale=z)
+        got = out.cpu().numpy()
+        nan = (ref & 0x7F) == 0x7F
+        assert np.array_equal(nan, (got & 0x7F) == 0x7F), z
+        assert np.array_equal(got[~nan], ref[~nan]), z
 
 
 def test_fp8_one_hot_exact(oracle):

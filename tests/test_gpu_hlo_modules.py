@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import hlo_eval
-from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_s8, dev_u8, dot_floor, host_bf16
+from tests.gpu_util import check_dot, check_f8_result, dev_bf16, dev_f32, dev_s8, dev_u8, dot_floor, host_bf16
 from xla_amd import dtypes, hlo, hlo_modules as hm, hlo_runner, workloads
 
 pytestmark = pytest.mark.gpu
@@ -83,6 +83,25 @@ def test_c3_module_vector_scales():
     fa = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * sa[:, None]
     fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * sb[None, :]
     check_dot(host_bf16(out), ref, dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "C3 vector scales")
+
+
+def test_c3_module_f8_result(oracle):
+    say("module C3 with an f8 result")
+    M, K, N = 128, 256, 144
+    w = workloads.c3_fp8(M, K, N)
+    s, z = np.array(1 / 64, np.float32), np.array(0.0171, np.float32)
+    text = hm.c3_fp8_f8_result(M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(w["a"]), dev_u8(w["b"]), dev_f32(s), dev_f32(s),
+                                                   dev_bf16(w["bias"]), dev_f32(z)])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result]"]
+    ref = reference(text, [w["a"], w["b"], s, s, w["bias"], z])
+    _, val = oracle.fp8_scaled_dot(w["a"], w["b"], s, s, bias=w["bias"], epilogue="gelu_tanh", d_scale=z)
+    fa = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) / 64
+    fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) / 64
+    floor = dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb))
+    got = out.cpu().numpy().view(np.uint8)
+    assert check_f8_result(got, ref, val, z, True, floor, "C3 f8 result") <= got.size // 50
 
 
 def test_quantize_then_fp8_dot_module(oracle):

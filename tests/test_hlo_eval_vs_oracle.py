@@ -53,6 +53,17 @@ def test_c3_vector_scales(oracle):
     assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("multiply", [False, True])
+def test_c3_f8_result(oracle, multiply):
+    M, K, N = 12, 64, 20
+    w = workloads.c3_fp8(M, K, N)
+    s, z = np.array(1 / 64, np.float32), np.array(0.0213 if not multiply else 37.5, np.float32)
+    got = run_module(hm.c3_fp8_f8_result(M, K, N, multiply=multiply), [w["a"], w["b"], s, s, w["bias"], z])
+    ref, _ = oracle.fp8_scaled_dot(w["a"], w["b"], s, s, bias=w["bias"], epilogue="gelu_tanh", d_scale=z,
+                                   d_scale_divides=not multiply)
+    assert np.array_equal(got, ref)
+
+
 def test_quantize_then_fp8_dot(oracle):
     R, C, N = 6, 96, 10
     x = workloads.c4_quantize(R, C)

@@ -129,6 +129,22 @@ def test_c3_fp8_vector_scales():
     assert rw == [] and len(rf) == 1 and "rhs scales vary along the contracting dimension" in rf[0]
 
 
+def test_c3_fp8_with_f8_result():
+    """divide (or multiply) by a per-tensor scale -> clamp(+-448) -> convert(f8e4m3fn) after the
+    epilogue is taken into the call: the scale is the last operand, the result is f8
+    (gemm_rewriter_fp8_test.cc:1665-1690; the reference leaves it unfused on ROCm, :1710)."""
+    for mul in (False, True):
+        new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 32, multiply=mul))
+        assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result]"] and rf == []
+        check(new, r"\(f8e4m3fn\[64,32\]\{1,0\}, s8\[4096\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
+              r"d_scale_multiplies = %s" % ("true" if mul else "false"))
+        assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+    # a clamp to anything but +-448 is not the f8 saturation: left alone, with the reason
+    bad = hm.c3_fp8_f8_result(64, 128, 32).replace("constant(448)", "constant(240)")
+    new, rw, rf = hlo.rewrite(bad)
+    assert rw == [] and any("is f32, the kernels produce bf16" in r for r in rf)
+
+
 def test_quantizer_feeding_a_dot_becomes_two_calls():
     """The quantizer's broadcast scales are reused by the dequantising multiply of the next dot:
     both patterns are taken, the dot reads the quantizer's two results, and none of the

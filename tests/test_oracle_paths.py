@@ -212,6 +212,29 @@ def test_fp8_dot_vector_scales(oracle):
             assert not np.all(np.abs(got - wrong) <= np.abs(wrong) * 2.0 ** -8 + 1e-6)
 
 
+def test_fp8_dot_f8_result(oracle):
+    """f8 result = convert(clamp(v / z)): v must be the bf16-result path's value before its
+    rounding, the codes the numpy restatement of divide / clamp / cast on those v (the cast itself
+    is pinned by the reference's vectors), multiply is not divide, and clamping saturates."""
+    rng = np.random.default_rng(33)
+    M, K, N = 9, 64, 12
+    a8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 32, -448, 448))
+    b8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((K, N)) * 32, -448, 448))
+    bias = bf16(rng.standard_normal(N))
+    kw = dict(bias=bias, epilogue="gelu_tanh")
+    z = np.float32(0.0137)
+    codes, v = oracle.fp8_scaled_dot(a8, b8, 1 / 64, 1 / 64, d_scale=z, **kw)
+    assert np.array_equal(bf16(v), oracle.fp8_scaled_dot(a8, b8, 1 / 64, 1 / 64, **kw))
+    want = dtypes.f32_to_f8e4m3fn(np.clip((v / z).astype(np.float32), -448, 448))
+    assert np.array_equal(codes, want)
+    codes_m, v_m = oracle.fp8_scaled_dot(a8, b8, 1 / 64, 1 / 64, d_scale=z, d_scale_divides=False, **kw)
+    assert np.array_equal(v_m, v)
+    assert np.array_equal(codes_m, dtypes.f32_to_f8e4m3fn(np.clip((v * z).astype(np.float32), -448, 448)))
+    assert not np.array_equal(codes_m, codes)
+    sat, v2 = oracle.fp8_scaled_dot(a8, b8, 1.0, 1.0, d_scale=np.float32(1e-3))   # |v| / 1e-3 >> 448
+    assert set(np.unique(sat[np.abs(v2) > 1.0])) <= {0x7E, 0xFE}                  # +-448, never NaN
+
+
 # ---- RMSNorm + quantize -----------------------------------------------------------
 
 def test_tree32_sum_order(oracle):

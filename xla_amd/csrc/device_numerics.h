@@ -75,6 +75,25 @@ __device__ __forceinline__ uint32_t pack_f8x4(float a, float b, float c, float d
   return (uint32_t)r;
 }
 
+// y / s, correctly rounded, from the correctly rounded reciprocal rs = RN(1/s):
+// q0 = RN(y*rs); r = y - q0*s exactly (fma); q1 = RN(q0 + r*rs).  With rs
+// correctly rounded and no overflow/underflow in range this is RN(y/s)
+// (Markstein); the caller takes the plain IEEE divide when ordinary_divisor(s) is false.
+__device__ __forceinline__ float div_by_ordinary(float y, float s, float rs) {
+  float q0 = y * rs;
+  float r = __builtin_fmaf(-q0, s, y);
+  // s > 0 here, so the quotient carries the sign of y even when it is zero (-0/s = -0, which the
+  // correction step would turn into +0)
+  return __builtin_copysignf(__builtin_fmaf(r, rs, q0), y);
+}
+
+// A positive divisor shared by many quotients for which div_by_ordinary is exact: a normal
+// number well inside the exponent range whose significand is not all ones.
+__device__ __forceinline__ bool ordinary_divisor(float s) {
+  const uint32_t sb = f32_to_bits(s);
+  return sb > 0x0d800000u && sb < 0x71800000u && (sb & 0x7fffffu) != 0x7fffffu;
+}
+
 // xla/codegen/intrinsic/tanh.cc:48-108 rational, then the |x| >= 20 -> +-1 rule of :33-46.
 __device__ __forceinline__ float tanh_xla(float x) {
   const float kClamp = 7.99881172180175781f;

@@ -385,20 +385,31 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
 
 XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Error* err;
-  if (Preamble(f, 4, 5, 1, 2, &err)) return err;
+  if (Preamble(f, 4, 6, 1, 2, &err)) return err;
   Decoder d{f};
   const uint64_t f8 = Bit(XLA_FFI_DataType_F8E4M3FN);
   XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 2, "a");
   XLA_FFI_Buffer* b = d.Arg(1, f8, 2, 2, "b");
   XLA_FFI_Buffer* sa = d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
   XLA_FFI_Buffer* sb = d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
-  XLA_FFI_Buffer* bias = f->args.size > 4 ? d.Arg(4, kFloatMask, 1, 1, "bias") : nullptr;
-  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16), 2, 2, "out");
+  // an F8E4M3FN result brings its scale as the last operand; a bias, if any, sits before it
+  const bool out_f8 = f->rets.types[0] == XLA_FFI_RetType_BUFFER &&
+                      static_cast<XLA_FFI_Buffer*>(f->rets.rets[0])->dtype == XLA_FFI_DataType_F8E4M3FN;
+  const int64_t n_bias = f->args.size - 4 - (out_f8 ? 1 : 0);
+  if (n_bias < 0 || n_bias > 1)
+    return InvalidArgument(f->api, out_f8 ? "xla_amd.fp8_scaled_dot: an F8E4M3FN result takes a, b, a_scale, b_scale, "
+                                            "[bias,] d_scale"
+                                          : "xla_amd.fp8_scaled_dot: a BF16 result takes a, b, a_scale, b_scale[, bias]");
+  XLA_FFI_Buffer* bias = n_bias ? d.Arg(4, kFloatMask, 1, 1, "bias") : nullptr;
+  XLA_FFI_Buffer* sd = out_f8 ? d.Arg(4 + (int)n_bias, Bit(XLA_FFI_DataType_F32), 0, 0, "d_scale") : nullptr;
+  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F8E4M3FN), 2, 2, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
   CommonAttrs at;
   DecodeCommonAttrs(d, &at);
   int64_t rcd = 0;
   d.Int("rhs_contracting_dim", &rcd);
+  bool d_mul = false;
+  d.Scalar("d_scale_multiplies", XLA_FFI_DataType_PRED, &d_mul, 1);
   if (!d.ok()) return d.Error();
 
   XlaAmdFp8ScaledDot p{};
@@ -420,6 +431,9 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   p.a_scale = (const float*)sa->data; p.b_scale = (const float*)sb->data;
   p.a_scale_per_row = sa->rank == 1;
   p.b_scale_per_channel = sb->rank == 1;
+  p.out_dtype = out->dtype;
+  p.d_scale = sd ? (const float*)sd->data : nullptr;
+  p.d_scale_multiplies = d_mul;
   p.bias = bias ? bias->data : nullptr;
   p.out = out->data;
   p.workspace = ws ? ws->data : nullptr;

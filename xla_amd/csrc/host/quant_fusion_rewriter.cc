@@ -108,6 +108,8 @@ struct Epilogue {
   Instr* bias = nullptr;     // [N] operand, bf16 or f32 (null if none)
   std::string act = "";      // "", RELU, GELU, SILU
   std::string ops_type;      // element type of the bias add / activation ops
+  Instr* d_scale = nullptr;  // f8 result: the scalar the value is divided (or multiplied) by
+  bool d_multiplies = false;
   std::string Name() const {
     std::string a = act.empty() ? "" : act;
     if (bias) return a.empty() ? "BIAS" : "BIAS_" + a;
@@ -155,7 +157,7 @@ bool MatchSilu(Instr* out, Instr* x) {
 // Walks forward from the dot: optional convert, optional + broadcast(bias) along the minor
 // dimension, optional activation, optional final convert to bf16.  Returns false when what
 // leaves the chain is not bf16.
-bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why) {
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result = false) {
   Instr* cur = dot;
   const int64_t rank = dot->shape.rank();
   ep->ops_type = dot->shape.dtype;
@@ -233,6 +235,29 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why) {
   }
   if (cur != after_dot && cur != dot) ep->ops_type = cur->shape.dtype;
   if (!ep->bias && ep->act.empty()) ep->ops_type = dot->shape.dtype;  // nothing between dot and result
+  // f8 result: convert(clamp(-448, cur / broadcast(z) | cur * broadcast(z), 448)) on f32-typed ops
+  // (gemm_rewriter_fp8_test.cc:1665-1690, :1730-1748)
+  if (allow_f8_result && cur->shape.dtype == "f32" && dot->shape.dtype == "f32" && ep->ops_type == "f32") {
+    Instr* sc = SoleUser(cur);
+    Instr *val = nullptr, *z = nullptr, *bz = nullptr;
+    bool mul = false, ok = false;
+    if (sc && Binary(sc, "divide", &val, &bz) && val == cur && ScalarBroadcast(bz, &z)) ok = true;
+    else if (sc && BinaryWith(sc, "multiply", [&](Instr* b) { return ScalarBroadcast(b, &z); }, &val) && val == cur)
+      ok = mul = true;
+    if (ok && z->shape.dtype == "f32") {
+      Instr* cl = SoleUser(sc);
+      if (cl && cl->Is("clamp") && cl->operands.size() == 3 && cl->operands[1] == sc &&
+          IsConst(cl->operands[0], -448.0) && IsConst(cl->operands[2], 448.0)) {
+        Instr* cv = SoleUser(cl);
+        if (cv && cv->Is("convert") && cv->shape.dtype == "f8e4m3fn") {
+          ep->d_scale = z;
+          ep->d_multiplies = mul;
+          ep->tail = cv;
+          return true;
+        }
+      }
+    }
+  }
   step_convert();
   if (cur->shape.dtype != "bf16") {
     *why = "the value leaving the dot pattern is " + cur->shape.dtype + ", the kernels produce bf16";
@@ -333,7 +358,7 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   if (!IsFloatTy(dot->shape.dtype)) return refuse("dot result type " + dot->shape.dtype);
   Epilogue ep;
   std::string why;
-  if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/true)) return refuse(why);
 
   const int64_t M = a.value->shape.dims[0], K = a.value->shape.dims[1], N = b.value->shape.dims[1 - rc[0]];
   // a vector of scales must run along the operand's free dimension (rows of a, output channels
@@ -367,15 +392,17 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   };
   std::vector<Instr*> ops = {a.value, b.value, scale_of(a), scale_of(b)};
   if (ep.bias) ops.push_back(ep.bias);
-  std::vector<Shape> results = {Shape::Array("bf16", {M, N})};
+  if (ep.d_scale) ops.push_back(ep.d_scale);
+  std::vector<Shape> results = {Shape::Array(ep.d_scale ? "f8e4m3fn" : "bf16", {M, N})};
   size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0]) : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
   std::string cfg = CommonConfig(ep, a.type, dot->shape.dtype) + ", rhs_contracting_dim = " +
                     std::to_string(rc[0]) + " : i64";
+  if (ep.d_scale) cfg += std::string(", d_scale_multiplies = ") + (ep.d_multiplies ? "true" : "false");
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, results, cfg);
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
-  log->rewrites.push_back(dot->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + "]");
+  log->rewrites.push_back(dot->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + (ep.d_scale ? ", f8 result" : "") + "]");
   return true;
 }
 

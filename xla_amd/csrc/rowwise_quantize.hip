@@ -41,19 +41,6 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// y / s, correctly rounded, from the correctly rounded reciprocal rs = RN(1/s):
-// q0 = RN(y*rs); r = y - q0*s exactly (fma); q1 = RN(q0 + r*rs).  With rs
-// correctly rounded and no overflow/underflow in range this is RN(y/s)
-// (Markstein); the caller takes the plain IEEE divide when s is outside the
-// safe range or has an all-ones significand.
-__device__ __forceinline__ float div_by_row_scale(float y, float s, float rs) {
-  float q0 = y * rs;
-  float r = __builtin_fmaf(-q0, s, y);
-  // s > 0 here, so the quotient carries the sign of y even when it is zero (-0/s = -0, which the
-  // correction step would turn into +0)
-  return __builtin_copysignf(__builtin_fmaf(r, rs, q0), y);
-}
-
 // CH: consecutive 8-element chunks owned by a lane inside one group;
 // G: groups.  A group spans kThreads*CH*8 consecutive elements.  VEC: rows are
 // 16-byte aligned and cols % 8 == 0, so chunks move as 128-bit accesses.
@@ -201,8 +188,7 @@ __global__ __launch_bounds__(kThreads) void rowwise_quantize_kernel(
   // The reciprocal shortcut is exact only for an ordinary s; otherwise (zero, NaN, huge,
   // tiny, all-ones significand) every quotient takes the IEEE divide and the software cast,
   // which also reproduces the NaN codes the unguarded HLO yields for an all-zero row.
-  const uint32_t sb = f32_to_bits(s);
-  const bool fast = sb > 0x0d800000u && sb < 0x71800000u && (sb & 0x7fffffu) != 0x7fffffu;
+  const bool fast = ordinary_divisor(s);
   const float rs = 1.0f / s;
 
 #pragma unroll
@@ -215,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void rowwise_quantize_kernel(
         float d[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          float t = div_by_row_scale(v[g][c][i], s, rs);
+          float t = div_by_ordinary(v[g][c][i], s, rs);
           d[i] = __builtin_amdgcn_fmed3f(t, -448.0f, 448.0f);
         }
         out[0] = pack_f8x4(d[0], d[1], d[2], d[3]);

@@ -52,6 +52,9 @@ struct TiledParams {
   int tiles_m, tiles_n;
   int require_pow2_scales;  // kFp8 with a bf16-typed dequantise multiply: exact only then
   int a_per_row, b_per_channel;
+  uint8_t* out8;         // kFp8 with an f8e4m3fn result: [M,N] codes (out is unused then)
+  const float* d_scale;  // its per-tensor scale, a device scalar
+  int d_divides;         // the value is divided by the scale (else multiplied)
 };
 
 __device__ __forceinline__ bool is_pow2_f32(float s) {
@@ -82,11 +85,16 @@ struct DrainArgs {
   const float* stage;
   int rd_chunk, rd_row, m_base, n, M, N;
   uint16_t* out;  // start of this batch's [M,N] block
+  uint8_t* out8;  // f8e4m3fn result instead (d_mode != 0)
+  // 0: bf16 result; f8 result = convert(clamp(t)): 1: t = v * dz, 2: t = v / dz through the
+  // shared reciprocal (dz ordinary), 3: t = v / dz by the IEEE divide
+  int d_mode;
+  float dz, drz, dlim;  // the scale, its reciprocal, and 1792 * dz
   bool n_vec, has_bias;
   float sc[4], bs[4];
 };
 
-template <bool BF16_DOT, bool BF16_OPS, int ACT>
+template <bool BF16_DOT, bool BF16_OPS, int ACT, bool OUT_F8>
 __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
 #pragma unroll 4
   for (int it = 0; it < 16; ++it) {
@@ -98,7 +106,45 @@ __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
       v[t] = epilogue_act<BF16_OPS>(epilogue_pre<BF16_DOT, BF16_OPS>(x[t] * d.sc[t], d.bs[t], d.has_bias), ACT);
     }
     const int m = d.m_base + ml;
-    if (m < d.M && d.n < d.N) {
+    if (OUT_F8) {
+      float q[4];
+      bool special = d.d_mode == 3;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        if (d.d_mode == 1) {
+          q[t] = v[t] * d.dz;
+        } else if (d.d_mode == 2) {
+          // beyond +-1792*dz the quotient is clamped anyway; inside, the shortcut cannot overflow
+          q[t] = div_by_ordinary(__builtin_amdgcn_fmed3f(v[t], -d.dlim, d.dlim), d.dz, d.drz);
+        } else {
+          q[t] = v[t] / d.dz;
+        }
+        special |= v[t] != v[t] || q[t] != q[t];
+      }
+      uint32_t codes;
+      if (!special) {
+        codes = pack_f8x4(__builtin_amdgcn_fmed3f(q[0], -448.0f, 448.0f), __builtin_amdgcn_fmed3f(q[1], -448.0f, 448.0f),
+                          __builtin_amdgcn_fmed3f(q[2], -448.0f, 448.0f), __builtin_amdgcn_fmed3f(q[3], -448.0f, 448.0f));
+      } else {  // NaN in or out, or a scale the shortcut does not cover: op by op, software cast
+        codes = 0u;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          float c = d.d_mode == 1 ? v[t] * d.dz : v[t] / d.dz;
+          if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+          codes |= f32_to_f8e4m3fn_any(c) << (8 * t);
+        }
+      }
+      if (m < d.M && d.n < d.N) {
+        uint8_t* dst = d.out8 + (size_t)m * d.N + d.n;
+        if (d.n_vec) {
+          *reinterpret_cast<uint32_t*>(dst) = codes;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (d.n + t < d.N) dst[t] = (uint8_t)(codes >> (8 * t));
+        }
+      }
+    } else if (m < d.M && d.n < d.N) {
       uint16_t* dst = d.out + (size_t)m * d.N + d.n;
       if (d.n_vec) {  // N % 4 == 0 and n % 4 == 0: the run of 4 is whole and 8-byte aligned
         const uintx2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
@@ -112,25 +158,28 @@ __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
   }
 }
 
-template <bool BF16_DOT, bool BF16_OPS>
+template <bool BF16_DOT, bool BF16_OPS, bool OUT_F8>
 __device__ __forceinline__ void drain_act(const DrainArgs& d, int act) {
   switch (act) {
-    case kEpiRelu: drain_rows<BF16_DOT, BF16_OPS, kEpiRelu>(d); break;
-    case kEpiGelu: drain_rows<BF16_DOT, BF16_OPS, kEpiGelu>(d); break;
-    case kEpiSilu: drain_rows<BF16_DOT, BF16_OPS, kEpiSilu>(d); break;
-    default: drain_rows<BF16_DOT, BF16_OPS, 0>(d); break;
+    case kEpiRelu: drain_rows<BF16_DOT, BF16_OPS, kEpiRelu, OUT_F8>(d); break;
+    case kEpiGelu: drain_rows<BF16_DOT, BF16_OPS, kEpiGelu, OUT_F8>(d); break;
+    case kEpiSilu: drain_rows<BF16_DOT, BF16_OPS, kEpiSilu, OUT_F8>(d); break;
+    default: drain_rows<BF16_DOT, BF16_OPS, 0, OUT_F8>(d); break;
   }
 }
 
+template <bool OUT_F8>
 __device__ __forceinline__ void drain_dispatch(const DrainArgs& d, int act, bool bf16_dot, bool bf16_ops) {
-  if (bf16_ops) {
-    if (bf16_dot) drain_act<true, true>(d, act); else drain_act<false, true>(d, act);
+  if (OUT_F8) {  // an f8 result is scaled from f32-typed ops only (checked on the host)
+    drain_act<false, false, true>(d, act);
+  } else if (bf16_ops) {
+    if (bf16_dot) drain_act<true, true, false>(d, act); else drain_act<false, true, false>(d, act);
   } else {
-    if (bf16_dot) drain_act<true, false>(d, act); else drain_act<false, false>(d, act);
+    if (bf16_dot) drain_act<true, false, false>(d, act); else drain_act<false, false, false>(d, act);
   }
 }
 
-template <int KIND>
+template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr bool F8 = KIND != kS8;       // both operands f8e4m3fn
   constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
@@ -406,6 +455,16 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.M = p.M;
   d.N = p.N;
   d.out = p.out + (size_t)batch * p.M * p.N;
+  d.out8 = nullptr;
+  d.d_mode = 0;
+  d.dz = d.drz = d.dlim = 1.0f;
+  if (OUT_F8) {
+    d.out8 = p.out8;
+    d.dz = *p.d_scale;
+    d.drz = 1.0f / d.dz;
+    d.dlim = 1792.0f * d.dz;
+    d.d_mode = !p.d_divides ? 1 : ordinary_divisor(d.dz) ? 2 : 3;
+  }
   d.n_vec = n_vec;
   d.has_bias = p.bias != nullptr;
   if (F8 && p.a_per_row) {
@@ -435,7 +494,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
     d.m_base = m0 + wm * 128 + pass * 64;
-    drain_dispatch(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops);
+    drain_dispatch<OUT_F8>(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops);
   }
 }
 
@@ -518,15 +577,22 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   }
   float bias = 0.0f;
   if (p.bias) bias = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n]) : ((const float*)p.bias)[n];
-  p.out[idx] = f32_to_bf16(epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops));
+  const float v = epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
+  if (p.out8) {
+    float c = p.d_divides ? v / *p.d_scale : v * *p.d_scale;
+    if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+    p.out8[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
+  } else {
+    p.out[idx] = f32_to_bf16(v);
+  }
 }
 
-template <int KIND>
+template <int KIND, bool OUT_F8 = false>
 int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
   constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow;  // 128 KiB
   static bool configured = false;  // per kernel instantiation; benign if two threads race
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND>,
+    hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND, OUT_F8>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
     if (e != hipSuccess)
       return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", what, kLds,
@@ -534,7 +600,7 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
     configured = true;
   }
   dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
-  hipLaunchKernelGGL(tiled_dot_kernel<KIND>, grid, dim3(512), kLds, stream, tp);
+  hipLaunchKernelGGL((tiled_dot_kernel<KIND, OUT_F8>), grid, dim3(512), kLds, stream, tp);
   return CheckLaunch(what);
 }
 
@@ -590,6 +656,14 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   }
   if (!p.a || !p.b || !p.a_scale || !p.b_scale || !p.out)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: null buffer");
+  const bool out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
+  if (!out_f8 && p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: the result is BF16 or F8E4M3FN");
+  if (out_f8 && !p.d_scale)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: an F8E4M3FN result needs d_scale");
+  if (out_f8 && (p.dot_type != XLA_FFI_DataType_F32 || p.epilogue_type != XLA_FFI_DataType_F32))
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT,
+                "fp8_scaled_dot: an F8E4M3FN result is scaled from f32-typed dot and epilogue ops");
 
   TiledParams tp{};
   tp.a = (const uint8_t*)p.a;
@@ -599,7 +673,10 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.a_per_row = p.a_scale_per_row != 0;
   tp.b_per_channel = p.b_scale_per_channel != 0;
   tp.bias = (p.epilogue & 1) ? p.bias : nullptr;
-  tp.out = (uint16_t*)p.out;
+  tp.out = out_f8 ? nullptr : (uint16_t*)p.out;
+  tp.out8 = out_f8 ? (uint8_t*)p.out : nullptr;
+  tp.d_scale = p.d_scale;
+  tp.d_divides = p.d_scale_multiplies ? 0 : 1;
   tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
   tp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
   tp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
@@ -652,8 +729,13 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;
-    int rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn")
-                       : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
+    int rc;
+    if (out_f8)
+      rc = kn_direct ? launch_tiled<kFp8KN, true>(tt, 1, stream, "fp8_scaled_dot_tiled_kn_f8")
+                     : launch_tiled<kFp8, true>(tt, 1, stream, "fp8_scaled_dot_tiled_f8");
+    else
+      rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn")
+                     : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
     if (rc) return rc;
     if (deq_bf16) {
       // runs only if a scale is not a power of two (decided on the device, no host read)
@@ -661,7 +743,10 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       rc = CheckLaunch("fp8_scaled_dot_exact");
       if (rc) return rc;
     }
-    SetLastKernel(nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose");
+    if (out_f8)
+      SetLastKernel(nk ? "fp8_scaled_dot_tiled_f8" : kn_direct ? "fp8_scaled_dot_tiled_kn_f8" : "fp8_scaled_dot_tiled+transpose_f8");
+    else
+      SetLastKernel(nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose");
     return 0;
   }
   hipLaunchKernelGGL(fp8_dot_exact_kernel, egrid, dim3(256), 0, stream, tp, nk ? 1 : 0, deq_bf16 ? 1 : 0, 0);

@@ -122,6 +122,26 @@ ENTRY %main {{
 """
 
 
+def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False):
+    """The f32-typed C3 module with an f8e4m3fn result: the GELU value is divided (or multiplied)
+    by a per-tensor scale, clamped to +-448 and converted -- the D scaling of
+    gemm_rewriter_fp8_test.cc:1665-1690 (divide) / :1730-1748 (multiply)."""
+    text = c3_fp8(M, K, N, typed="f32", vector_scales=vector_scales)
+    head, _ = text.split(f"  ROOT %out = bf16[{M},{N}] convert(%gelu)")
+    op = "multiply" if multiply else "divide"
+    return head + f"""  %d_scale = f32[] parameter(5)
+  %d_scale_b = f32[{M},{N}] broadcast(%d_scale), dimensions={{}}
+  %scaled = f32[{M},{N}] {op}(%gelu, %d_scale_b)
+  %lo = f32[] constant(-448)
+  %lo_b = f32[{M},{N}] broadcast(%lo), dimensions={{}}
+  %hi = f32[] constant(448)
+  %hi_b = f32[{M},{N}] broadcast(%hi), dimensions={{}}
+  %clamped = f32[{M},{N}] clamp(%lo_b, %scaled, %hi_b)
+  ROOT %out = f8e4m3fn[{M},{N}] convert(%clamped)
+}}
+"""
+
+
 def c4_quantize(rows=16384, cols=8192, rmsnorm=True, eps=1e-6):
     """RMSNorm (f32 math, bf16 result) -> per-row amax -> scale = amax/448 -> clamp -> f8e4m3fn."""
     R, C = rows, cols

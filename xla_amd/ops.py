@@ -87,20 +87,25 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
 
 def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, epilogue="DEFAULT",
                    dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto",
-                   build_only=False):
+                   d_scale=None, d_scale_multiplies=False, build_only=False):
     """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K];
-    a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel)."""
-    _check_cuda(a, b, a_scale, b_scale, bias)
+    a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel).
+    With d_scale (f32 []) the result is f8e4m3fn codes (uint8): convert(clamp(out / d_scale)),
+    or out * d_scale with d_scale_multiplies."""
+    _check_cuda(a, b, a_scale, b_scale, bias, d_scale)
     m, k = a.shape
     n = b.shape[1 - rhs_contracting_dim]
+    out_f8 = d_scale is not None
     if out is None:
-        out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+        out = torch.empty((m, n), dtype=torch.uint8 if out_f8 else torch.bfloat16, device=a.device)
     args = [(dtypes.F8E4M3FN, a.data_ptr(), a.shape), (dtypes.F8E4M3FN, b.data_ptr(), b.shape),
             (dtypes.F32, a_scale.data_ptr(), list(a_scale.shape)),
             (dtypes.F32, b_scale.data_ptr(), list(b_scale.shape))]
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
-    rets = [(dtypes.BF16, out.data_ptr(), [m, n])]
+    if out_f8:
+        args.append((dtypes.F32, d_scale.data_ptr(), list(d_scale.shape)))
+    rets = [(dtypes.F8E4M3FN if out_f8 else dtypes.BF16, out.data_ptr(), [m, n])]
     if scratch == "auto":
         nbytes = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(m, k, n, rhs_contracting_dim)
         scratch = _scratch(nbytes, a.device)
@@ -110,8 +115,10 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
              "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
              "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type]),
              "rhs_contracting_dim": ffi.Attr.i64(rhs_contracting_dim)}
+    if out_f8:
+        attrs["d_scale_multiplies"] = ffi.Attr.pred(d_scale_multiplies)
     call = Call("xla_amd.fp8_scaled_dot", ffi.Frame(host(), args, rets, attrs), out,
-                keep=(a, b, a_scale, b_scale, bias, scratch))
+                keep=(a, b, a_scale, b_scale, bias, d_scale, scratch))
     return call if build_only else call.run()
 
 
