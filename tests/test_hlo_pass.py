@@ -338,3 +338,45 @@ def test_quantize_near_misses_are_refused_with_reasons():
         "%rinv = f32[8] divide(%one_b, %rt)", "%rinv = f32[8] multiply(%one_b, %rt)")
     _, rw, rf = hlo.rewrite(rs)
     assert rw == [] and "not the RMSNorm form" in rf[0]
+
+
+def test_mutated_modules_are_rejected_or_stay_printable():
+    """Line deletions, duplications, swaps and token edits of the canonical modules: the parser
+    either rejects the text with an error or the pass returns a module that parses again."""
+    import random
+    rng = random.Random(5)
+    tokens = ["(", ")", "{", "}", "[", "]", ",", "=", "%", ":", " ", "0", "f32", "s4", "f8e4m3fn", "broadcast",
+              "dot", "-", "448", "dimensions={0}", "ROOT ", "parameter(0)", "tuple", "clamp"]
+    base = [hm.c1_s8_channel(16, 512, 256), hm.c2_s4_group(8, 1024, 512), hm.c3_fp8(64, 128, 32, vector_scales=True),
+            hm.c3_fp8_f8_result(64, 128, 32), hm.c4_quantize(24, 2048), hm.c5_s8_batched(2, 128, 256, 512),
+            hm.quantize_then_fp8_dot(64, 256, 32)]
+    accepted = rejected = 0
+    for text in base:
+        lines = text.split("\n")
+        for _ in range(40):
+            b = list(lines)
+            kind = rng.random()
+            if kind < 0.3:
+                del b[rng.randrange(len(b))]
+            elif kind < 0.5:
+                i = rng.randrange(len(b))
+                b.insert(i, b[i])
+            elif kind < 0.7:
+                i, k = rng.randrange(len(b)), rng.randrange(len(b))
+                b[i], b[k] = b[k], b[i]
+            else:
+                i = rng.randrange(len(b))
+                if b[i]:
+                    p = rng.randrange(len(b[i]))
+                    b[i] = b[i][:p] + rng.choice(tokens) + b[i][p + rng.randrange(3):]
+            try:
+                new, _, _ = hlo.rewrite("\n".join(b))
+            except hlo.HloError:
+                rejected += 1
+                continue
+            accepted += 1
+            hlo.print_module(new)
+            hlo.to_json(new)
+    assert accepted > 20 and rejected > 20, (accepted, rejected)
+    with pytest.raises(hlo.HloError, match="computation without a name"):
+        hlo.rewrite(hm.c1_s8_channel(16, 512, 256).replace("ENTRY %main {", "ENTRY :%main {"))

@@ -370,6 +370,7 @@ std::unique_ptr<Module> Parse(const std::string& text, std::string* error) {
       if (nb == std::string::npos) return fail("computation without a name");
       size_t ne = nb;
       while (ne < h.size() && IsIdentChar(h[ne])) ++ne;
+      if (ne == nb) return fail("computation without a name");
       c->name = h.substr(nb, ne - nb);
       comp = c.get();
       mod->computations.push_back(std::move(c));
