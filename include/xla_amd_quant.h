@@ -74,6 +74,8 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  *   rets: out BF16 [M,N], or F8E4M3FN [M,N] = convert(clamp(-448, v / d_scale, 448)) for the
  *         f32 value v after the epilogue (the D scaling of gemm_rewriter_fp8_test.cc:1665-1690,
  *         which GemmRewriter leaves unfused on ROCm, :1710)
+ *         then optionally amax F32 [] = max |v| (reduce-maximum of abs, NaN passed on:
+ *         gemm_rewriter_fp8_test.cc:2559-2600), only next to an F8E4M3FN out
  *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
  *          rhs_contracting_dim i64 (default 0);
  *          d_scale_multiplies pred (default false): v * d_scale instead (:1730-1748)
@@ -161,6 +163,8 @@ typedef struct XlaAmdFp8ScaledDot {
                                   out = convert(clamp(-448, v / *d_scale, 448)), one byte each */
   int32_t d_scale_multiplies;  /* the f8 result is v * *d_scale instead of v / *d_scale */
   const float* d_scale;        /* device scalar, only with an F8E4M3FN result */
+  float* amax;                 /* optional device scalar result with an F8E4M3FN result:
+                                  max |v| over all outputs, NaN if any v is NaN */
 } XlaAmdFp8ScaledDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);

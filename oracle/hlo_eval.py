@@ -142,8 +142,13 @@ def evaluate(module_json, args):
             v = _round(r, ty)
         elif op == "reduce":
             dims = _dims(ins["attrs"]["dimensions"])
-            assert dims == [np.asarray(x[0]).ndim - 1], "only reductions over the minor dimension"
             kind = reducer_kind(ins["attrs"]["to_apply"])
+            if kind == "maximum" and sorted(dims) == list(range(np.asarray(x[0]).ndim)):
+                # over everything: order-free, NaN passed on (np.max and np.maximum both do)
+                v = _round(np.maximum(np.max(np.asarray(x[0], np.float32)), np.asarray(x[1], np.float32)), ty)
+                env[ins["name"]] = v
+                continue
+            assert dims == [np.asarray(x[0]).ndim - 1], "only reductions over the minor dimension"
             if kind == "add":
                 v = _round(_tree32_sum_last(x[0]), ty)
             elif kind == "maximum":

@@ -126,6 +126,10 @@ def test_shape_validation_happens_before_any_launch():
     with pytest.raises(ffi.FfiError, match="a BF16 result takes a, b, a_scale, b_scale\\[, bias\\]"):
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.BF16, FAKE, (4,)), (dtypes.F32, FAKE, ())],
                                                        [(dtypes.BF16, FAKE, (4, 4))], {"epilogue": ffi.Attr.str("BIAS")}))
+    with pytest.raises(ffi.FfiError, match="results are out\\[, amax\\]\\[, scratch\\]"):
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.F32, FAKE, ())],
+                                                       [(dtypes.F8E4M3FN, FAKE, (4, 4)), (dtypes.U8, FAKE, (64,)),
+                                                        (dtypes.F32, FAKE, ())]))
     with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0 but got 1 \\(d_scale\\)"):
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.F32, FAKE, (4,))],
                                                        [(dtypes.F8E4M3FN, FAKE, (4, 4))]))

@@ -173,6 +173,37 @@ def test_f8_result(oracle, mode, nk):
     assert differ <= out.numel() // 50, differ
 
 
+@pytest.mark.parametrize("force", [0, 1])
+def test_f8_result_amax(oracle, force):
+    """amax next to the f8 result: max |v| over the ragged result, from atomics into a result the
+    call itself zeroes -- so two calls in a row, the second on smaller values, must not see the first."""
+    say("fp8_scaled_dot f8 result with amax, kernel option %d" % force)
+    M, K, N = 300, 512, 272
+    w = workloads.c3_fp8(M, K, N)
+    z = np.float32(0.0117)
+    a, b, bias = dev_u8(w["a"]), dev_u8(w["b"]), dev_bf16(w["bias"])
+    ffi.set_option("fp8_dot_kernel", force)
+    try:
+        for scale in (1 / 64, 1 / 512):
+            s = dev_f32(np.array(scale, np.float32))
+            out, amax = ops.fp8_scaled_dot(a, b, s, s, bias, epilogue="BIAS_GELU", amax=True,
+                                           d_scale=dev_f32(np.array(z, np.float32)))
+            torch.cuda.synchronize()
+            _, val = oracle.fp8_scaled_dot(w["a"], w["b"], scale, scale, bias=w["bias"], epilogue="gelu_tanh", d_scale=z)
+            want = float(np.max(np.abs(val)))
+            assert abs(float(amax) - want) <= want * 2.0 ** -7, (float(amax), want)
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+    # a NaN anywhere makes the maximum NaN
+    bn = w["b"].copy()
+    bn[7, 5] = 0x7F
+    s = dev_f32(np.array(1 / 64, np.float32))
+    _, amax = ops.fp8_scaled_dot(a, dev_u8(bn), s, s, bias, epilogue="BIAS_GELU", amax=True,
+                                 d_scale=dev_f32(np.array(z, np.float32)))
+    torch.cuda.synchronize()
+    assert np.isnan(float(amax))
+
+
 def test_f8_result_special_values(oracle):
     """NaN operands give NaN codes, a huge value over a tiny scale saturates at +-448, -0 stays -0;
     a zero scale follows IEEE (x/0 = +-inf -> +-448, 0/0 = NaN)."""

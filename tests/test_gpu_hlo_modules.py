@@ -104,6 +104,22 @@ def test_c3_module_f8_result(oracle):
     assert check_f8_result(got, ref, val, z, True, floor, "C3 f8 result") <= got.size // 50
 
 
+def test_c3_module_f8_result_with_amax(oracle):
+    say("module C3 with an f8 result and its amax")
+    M, K, N = 128, 256, 144
+    w = workloads.c3_fp8(M, K, N)
+    s, z = np.array(1 / 64, np.float32), np.array(0.0171, np.float32)
+    text = hm.c3_fp8_f8_result(M, K, N, amax=True)
+    (out, amax), rw, _ = hlo_runner.compile_and_run(text, [dev_u8(w["a"]), dev_u8(w["b"]), dev_f32(s), dev_f32(s),
+                                                           dev_bf16(w["bias"]), dev_f32(z)])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result, amax]"]
+    ref_codes, ref_amax = reference(text, [w["a"], w["b"], s, s, w["bias"], z])
+    ref_amax = float(np.asarray(ref_amax).reshape(-1)[0])
+    assert abs(float(amax) - ref_amax) <= ref_amax * 2.0 ** -7
+    assert (out.cpu().numpy().view(np.uint8) != ref_codes).sum() <= out.numel() // 50
+
+
 def test_quantize_then_fp8_dot_module(oracle):
     """RMSNorm + quantize feeding an f8 dot: two custom calls after the pass, against the op-by-op
     evaluation of the original module."""

@@ -64,6 +64,16 @@ def test_c3_f8_result(oracle, multiply):
     assert np.array_equal(got, ref)
 
 
+def test_c3_f8_result_with_amax(oracle):
+    M, K, N = 12, 64, 20
+    w = workloads.c3_fp8(M, K, N)
+    s, z = np.array(1 / 64, np.float32), np.array(0.0213, np.float32)
+    codes, amax = run_module(hm.c3_fp8_f8_result(M, K, N, amax=True), [w["a"], w["b"], s, s, w["bias"], z])
+    ref, val = oracle.fp8_scaled_dot(w["a"], w["b"], s, s, bias=w["bias"], epilogue="gelu_tanh", d_scale=z)
+    assert np.array_equal(codes, ref)
+    assert np.float32(amax) == np.max(np.abs(val)) and amax > 0
+
+
 def test_quantize_then_fp8_dot(oracle):
     R, C, N = 6, 96, 10
     x = workloads.c4_quantize(R, C)

@@ -139,6 +139,12 @@ def test_c3_fp8_with_f8_result():
         check(new, r"\(f8e4m3fn\[64,32\]\{1,0\}, s8\[4096\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
               r"d_scale_multiplies = %s" % ("true" if mul else "false"))
         assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+    # the result's own amax (reduce-maximum of abs over both dimensions) becomes a second result
+    new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 32, amax=True))
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result, amax]"] and rf == []
+    check(new, r"\(f8e4m3fn\[64,32\]\{1,0\}, f32\[\], s8\[4096\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
+          r"ROOT %result = .* tuple\(%out.out, %amax.amax\)")
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter", "tuple"]
     # a clamp to anything but +-448 is not the f8 saturation: left alone, with the reason
     bad = hm.c3_fp8_f8_result(64, 128, 32).replace("constant(448)", "constant(240)")
     new, rw, rf = hlo.rewrite(bad)

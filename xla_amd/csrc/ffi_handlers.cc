@@ -385,7 +385,7 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
 
 XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Error* err;
-  if (Preamble(f, 4, 6, 1, 2, &err)) return err;
+  if (Preamble(f, 4, 6, 1, 3, &err)) return err;
   Decoder d{f};
   const uint64_t f8 = Bit(XLA_FFI_DataType_F8E4M3FN);
   XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 2, "a");
@@ -403,7 +403,16 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Buffer* bias = n_bias ? d.Arg(4, kFloatMask, 1, 1, "bias") : nullptr;
   XLA_FFI_Buffer* sd = out_f8 ? d.Arg(4 + (int)n_bias, Bit(XLA_FFI_DataType_F32), 0, 0, "d_scale") : nullptr;
   XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F8E4M3FN), 2, 2, "out");
-  XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
+  // after out: an f32 scalar is the amax of an f8 result, a byte vector is scratch
+  XLA_FFI_Buffer* amax = nullptr;
+  XLA_FFI_Buffer* ws = nullptr;
+  for (int64_t i = 1; i < f->rets.size; ++i) {
+    const bool scalar_f32 = f->rets.types[i] == XLA_FFI_RetType_BUFFER &&
+                            static_cast<XLA_FFI_Buffer*>(f->rets.rets[i])->dtype == XLA_FFI_DataType_F32;
+    if (scalar_f32 && out_f8 && !amax && !ws) amax = d.Ret((int)i, Bit(XLA_FFI_DataType_F32), 0, 0, "amax");
+    else if (!ws) ws = d.Ret((int)i, kBytesMask, 1, 1, "scratch");
+    else return InvalidArgument(f->api, "xla_amd.fp8_scaled_dot: results are out[, amax][, scratch]");
+  }
   CommonAttrs at;
   DecodeCommonAttrs(d, &at);
   int64_t rcd = 0;
@@ -434,6 +443,7 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   p.out_dtype = out->dtype;
   p.d_scale = sd ? (const float*)sd->data : nullptr;
   p.d_scale_multiplies = d_mul;
+  p.amax = amax ? (float*)amax->data : nullptr;
   p.bias = bias ? bias->data : nullptr;
   p.out = out->data;
   p.workspace = ws ? ws->data : nullptr;

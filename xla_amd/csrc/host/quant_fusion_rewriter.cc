@@ -110,6 +110,7 @@ struct Epilogue {
   std::string ops_type;      // element type of the bias add / activation ops
   Instr* d_scale = nullptr;  // f8 result: the scalar the value is divided (or multiplied) by
   bool d_multiplies = false;
+  Instr* amax = nullptr;     // f8 result: reduce-maximum of abs(value) over everything, if the module has one
   std::string Name() const {
     std::string a = act.empty() ? "" : act;
     if (bias) return a.empty() ? "BIAS" : "BIAS_" + a;
@@ -157,7 +158,8 @@ bool MatchSilu(Instr* out, Instr* x) {
 // Walks forward from the dot: optional convert, optional + broadcast(bias) along the minor
 // dimension, optional activation, optional final convert to bf16.  Returns false when what
 // leaves the chain is not bf16.
-bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result = false) {
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_result_in = nullptr) {
+  const bool allow_f8_result = f8_result_in != nullptr;
   Instr* cur = dot;
   const int64_t rank = dot->shape.rank();
   ep->ops_type = dot->shape.dtype;
@@ -238,7 +240,27 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_res
   // f8 result: convert(clamp(-448, cur / broadcast(z) | cur * broadcast(z), 448)) on f32-typed ops
   // (gemm_rewriter_fp8_test.cc:1665-1690, :1730-1748)
   if (allow_f8_result && cur->shape.dtype == "f32" && dot->shape.dtype == "f32" && ep->ops_type == "f32") {
+    // the value may also feed its own amax: reduce(abs(cur), -inf) over both dimensions with a
+    // maximum (gemm_rewriter_fp8_test.cc:2559-2600)
     Instr* sc = SoleUser(cur);
+    Instr* amax = nullptr;
+    if (!sc && cur->users.size() == 2) {
+      for (int which = 0; which < 2 && !amax; ++which) {
+        Instr* ab = cur->users[which];
+        Instr* rd = ab->Is("abs") ? SoleUser(ab) : nullptr;
+        if (!rd || !rd->Is("reduce") || rd->operands.size() != 2 || rd->operands[0] != ab) continue;
+        if (rd->DimsAttr("dimensions") != std::vector<int64_t>{0, 1} || !rd->operands[1]->Is("constant") ||
+            rd->operands[1]->literal != "-inf")
+          continue;
+        const std::string* to = rd->Attr("to_apply");
+        std::string name = to ? *to : "";
+        if (!name.empty() && name[0] == '%') name = name.substr(1);
+        const Computation* body = f8_result_in->FindComputation(name);
+        if (!body || !body->root() || !body->root()->Is("maximum")) continue;
+        amax = rd;
+        sc = cur->users[1 - which];
+      }
+    }
     Instr *val = nullptr, *z = nullptr, *bz = nullptr;
     bool mul = false, ok = false;
     if (sc && Binary(sc, "divide", &val, &bz) && val == cur && ScalarBroadcast(bz, &z)) ok = true;
@@ -252,6 +274,7 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_res
         if (cv && cv->Is("convert") && cv->shape.dtype == "f8e4m3fn") {
           ep->d_scale = z;
           ep->d_multiplies = mul;
+          ep->amax = amax;
           ep->tail = cv;
           return true;
         }
@@ -342,7 +365,7 @@ bool MatchF8Operand(Instr* op, F8Operand* out) {
   return true;
 }
 
-bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
+bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
   F8Operand a, b;
   if (!MatchF8Operand(dot->operands[0], &a) || !MatchF8Operand(dot->operands[1], &b)) return false;
   auto refuse = [&](const std::string& why) {
@@ -358,7 +381,7 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   if (!IsFloatTy(dot->shape.dtype)) return refuse("dot result type " + dot->shape.dtype);
   Epilogue ep;
   std::string why;
-  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/true)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, /*f8_result_in=*/&mod)) return refuse(why);
 
   const int64_t M = a.value->shape.dims[0], K = a.value->shape.dims[1], N = b.value->shape.dims[1 - rc[0]];
   // a vector of scales must run along the operand's free dimension (rows of a, output channels
@@ -394,6 +417,7 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   if (ep.bias) ops.push_back(ep.bias);
   if (ep.d_scale) ops.push_back(ep.d_scale);
   std::vector<Shape> results = {Shape::Array(ep.d_scale ? "f8e4m3fn" : "bf16", {M, N})};
+  if (ep.amax) results.push_back(Shape::Array("f32", {}));
   size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0]) : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
   std::string cfg = CommonConfig(ep, a.type, dot->shape.dtype) + ", rhs_contracting_dim = " +
@@ -402,7 +426,9 @@ bool RewriteF8Dot(Computation* comp, Instr* dot, const RewriteOptions& opt, Rewr
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, results, cfg);
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
-  log->rewrites.push_back(dot->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + (ep.d_scale ? ", f8 result" : "") + "]");
+  if (ep.amax) comp->ReplaceAllUses(ep.amax, EmitGte(comp, call, 1, ep.tail, ep.amax->name + ".amax"));
+  log->rewrites.push_back(dot->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + (ep.d_scale ? ", f8 result" : "") +
+                          (ep.amax ? ", amax" : "") + "]");
   return true;
 }
 
@@ -630,7 +656,7 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         Instr* i = up.get();
         bool did = false;
         if (i->Is("dot") && i->operands.size() == 2) {
-          did = RewriteF8Dot(comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
+          did = RewriteF8Dot(*mod, comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
         } else if (i->Is("convert") && i->shape.dtype == "f8e4m3fn") {
           did = RewriteQuantize(*mod, comp.get(), i, log);
         }

@@ -55,6 +55,7 @@ struct TiledParams {
   uint8_t* out8;         // kFp8 with an f8e4m3fn result: [M,N] codes (out is unused then)
   const float* d_scale;  // its per-tensor scale, a device scalar
   int d_divides;         // the value is divided by the scale (else multiplied)
+  float* amax;           // optional f32 scalar result: max |v| over the f8 result's values
 };
 
 __device__ __forceinline__ bool is_pow2_f32(float s) {
@@ -90,12 +91,16 @@ struct DrainArgs {
   // shared reciprocal (dz ordinary), 3: t = v / dz by the IEEE divide
   int d_mode;
   float dz, drz, dlim;  // the scale, its reciprocal, and 1792 * dz
+  bool want_amax;       // f8 result: also the largest |v| of the whole result
   bool n_vec, has_bias;
   float sc[4], bs[4];
 };
 
+// Returns, for an f8 result, the largest |v| this lane produced as a bit pattern (NaN sorts above
+// every number, which is how maximum propagates it); 0 otherwise.
 template <bool BF16_DOT, bool BF16_OPS, int ACT, bool OUT_F8>
-__device__ __forceinline__ void drain_rows(const DrainArgs& d) {
+__device__ __forceinline__ uint32_t drain_rows(const DrainArgs& d) {
+  uint32_t amax = 0u;
 #pragma unroll 4
   for (int it = 0; it < 16; ++it) {
     const int ml = it * 4 + d.rd_row;
@@ -107,6 +112,11 @@ __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
     }
     const int m = d.m_base + ml;
     if (OUT_F8) {
+      if (d.want_amax && m < d.M) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (d.n + t < d.N) amax = max(amax, f32_to_bits(v[t]) & 0x7fffffffu);
+      }
       float q[4];
       bool special = d.d_mode == 3;
 #pragma unroll
@@ -156,27 +166,28 @@ __device__ __forceinline__ void drain_rows(const DrainArgs& d) {
       }
     }
   }
+  return amax;
 }
 
 template <bool BF16_DOT, bool BF16_OPS, bool OUT_F8>
-__device__ __forceinline__ void drain_act(const DrainArgs& d, int act) {
+__device__ __forceinline__ uint32_t drain_act(const DrainArgs& d, int act) {
   switch (act) {
-    case kEpiRelu: drain_rows<BF16_DOT, BF16_OPS, kEpiRelu, OUT_F8>(d); break;
-    case kEpiGelu: drain_rows<BF16_DOT, BF16_OPS, kEpiGelu, OUT_F8>(d); break;
-    case kEpiSilu: drain_rows<BF16_DOT, BF16_OPS, kEpiSilu, OUT_F8>(d); break;
-    default: drain_rows<BF16_DOT, BF16_OPS, 0, OUT_F8>(d); break;
+    case kEpiRelu: return drain_rows<BF16_DOT, BF16_OPS, kEpiRelu, OUT_F8>(d);
+    case kEpiGelu: return drain_rows<BF16_DOT, BF16_OPS, kEpiGelu, OUT_F8>(d);
+    case kEpiSilu: return drain_rows<BF16_DOT, BF16_OPS, kEpiSilu, OUT_F8>(d);
+    default: return drain_rows<BF16_DOT, BF16_OPS, 0, OUT_F8>(d);
   }
 }
 
 template <bool OUT_F8>
-__device__ __forceinline__ void drain_dispatch(const DrainArgs& d, int act, bool bf16_dot, bool bf16_ops) {
-  if (OUT_F8) {  // an f8 result is scaled from f32-typed ops only (checked on the host)
-    drain_act<false, false, true>(d, act);
-  } else if (bf16_ops) {
+__device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, bool bf16_dot, bool bf16_ops) {
+  if (OUT_F8) return drain_act<false, false, true>(d, act);  // f32-typed ops only (checked on the host)
+  if (bf16_ops) {
     if (bf16_dot) drain_act<true, true, false>(d, act); else drain_act<false, true, false>(d, act);
   } else {
     if (bf16_dot) drain_act<true, false, false>(d, act); else drain_act<false, false, false>(d, act);
   }
+  return 0u;
 }
 
 template <int KIND, bool OUT_F8>
@@ -456,6 +467,8 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.N = p.N;
   d.out = p.out + (size_t)batch * p.M * p.N;
   d.out8 = nullptr;
+  d.want_amax = OUT_F8 && p.amax != nullptr;
+  uint32_t amax_bits = 0u;
   d.d_mode = 0;
   d.dz = d.drz = d.dlim = 1.0f;
   if (OUT_F8) {
@@ -494,7 +507,12 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
     d.m_base = m0 + wm * 128 + pass * 64;
-    drain_dispatch<OUT_F8>(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops);
+    amax_bits = max(amax_bits, drain_dispatch<OUT_F8>(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops));
+  }
+  if (OUT_F8 && p.amax) {  // one atomic per wave into the result a fill kernel zeroed
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, off));
+    if (lane == 0) atomicMax(reinterpret_cast<unsigned*>(p.amax), amax_bits);
   }
 }
 
@@ -579,6 +597,7 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   if (p.bias) bias = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n]) : ((const float*)p.bias)[n];
   const float v = epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
   if (p.out8) {
+    if (p.amax) atomicMax(reinterpret_cast<unsigned*>(p.amax), f32_to_bits(v) & 0x7fffffffu);
     float c = p.d_divides ? v / *p.d_scale : v * *p.d_scale;
     if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
     p.out8[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
@@ -586,6 +605,8 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
     p.out[idx] = f32_to_bf16(v);
   }
 }
+
+__global__ void store_u32_kernel(uint32_t* dst, uint32_t value) { *dst = value; }
 
 template <int KIND, bool OUT_F8 = false>
 int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
@@ -651,6 +672,11 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   if ((p.epilogue & 1) && !p.bias)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: BIAS epilogue without a bias");
   if (p.M == 0 || p.N == 0) {
+    if (p.amax && p.out_dtype == XLA_FFI_DataType_F8E4M3FN) {  // maximum over nothing: its init, -inf
+      hipLaunchKernelGGL(store_u32_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<uint32_t*>(p.amax), 0xff800000u);
+      int rc = CheckLaunch("fp8_scaled_dot_amax_init");
+      if (rc) return rc;
+    }
     SetLastKernel("fp8_scaled_dot:empty");
     return 0;
   }
@@ -677,6 +703,12 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.out8 = out_f8 ? (uint8_t*)p.out : nullptr;
   tp.d_scale = p.d_scale;
   tp.d_divides = p.d_scale_multiplies ? 0 : 1;
+  tp.amax = out_f8 ? p.amax : nullptr;
+  if (tp.amax) {  // the kernels fold their maxima into it with atomics (a kernel, not a memset: graphs)
+    hipLaunchKernelGGL(store_u32_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<uint32_t*>(tp.amax), 0u);
+    int rc = CheckLaunch("fp8_scaled_dot_amax_init");
+    if (rc) return rc;
+  }
   tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
   tp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
   tp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;

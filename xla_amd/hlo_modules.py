@@ -122,13 +122,23 @@ ENTRY %main {{
 """
 
 
-def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False):
+def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False, amax=False):
     """The f32-typed C3 module with an f8e4m3fn result: the GELU value is divided (or multiplied)
     by a per-tensor scale, clamped to +-448 and converted -- the D scaling of
     gemm_rewriter_fp8_test.cc:1665-1690 (divide) / :1730-1748 (multiply)."""
     text = c3_fp8(M, K, N, typed="f32", vector_scales=vector_scales)
     head, _ = text.split(f"  ROOT %out = bf16[{M},{N}] convert(%gelu)")
     op = "multiply" if multiply else "divide"
+    if amax:  # the result's own amax beside it (gemm_rewriter_fp8_test.cc:2559-2600)
+        head = head.replace("ENTRY %main {", "%max_f32 {\n  %a = f32[] parameter(0)\n  %b = f32[] parameter(1)\n"
+                            "  ROOT %m = f32[] maximum(%a, %b)\n}\n\nENTRY %main {")
+        root, tail = "", f"""  %abs_v = f32[{M},{N}] abs(%gelu)
+  %ninf = f32[] constant(-inf)
+  %amax = f32[] reduce(%abs_v, %ninf), dimensions={{0,1}}, to_apply=%max_f32
+  ROOT %result = (f8e4m3fn[{M},{N}], f32[]) tuple(%out, %amax)
+"""
+    else:
+        root, tail = "ROOT ", ""
     return head + f"""  %d_scale = f32[] parameter(5)
   %d_scale_b = f32[{M},{N}] broadcast(%d_scale), dimensions={{}}
   %scaled = f32[{M},{N}] {op}(%gelu, %d_scale_b)
@@ -137,8 +147,8 @@ def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False
   %hi = f32[] constant(448)
   %hi_b = f32[{M},{N}] broadcast(%hi), dimensions={{}}
   %clamped = f32[{M},{N}] clamp(%lo_b, %scaled, %hi_b)
-  ROOT %out = f8e4m3fn[{M},{N}] convert(%clamped)
-}}
+  {root}%out = f8e4m3fn[{M},{N}] convert(%clamped)
+{tail}}}
 """
 
 

@@ -87,11 +87,12 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
 
 def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, epilogue="DEFAULT",
                    dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto",
-                   d_scale=None, d_scale_multiplies=False, build_only=False):
+                   d_scale=None, d_scale_multiplies=False, amax=False, build_only=False):
     """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K];
     a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel).
     With d_scale (f32 []) the result is f8e4m3fn codes (uint8): convert(clamp(out / d_scale)),
-    or out * d_scale with d_scale_multiplies."""
+    or out * d_scale with d_scale_multiplies; with amax=True the call also returns max |out| (f32 [])
+    as a second tensor."""
     _check_cuda(a, b, a_scale, b_scale, bias, d_scale)
     m, k = a.shape
     n = b.shape[1 - rhs_contracting_dim]
@@ -106,6 +107,12 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
     if out_f8:
         args.append((dtypes.F32, d_scale.data_ptr(), list(d_scale.shape)))
     rets = [(dtypes.F8E4M3FN if out_f8 else dtypes.BF16, out.data_ptr(), [m, n])]
+    amax_t = None
+    if amax:
+        if not out_f8:
+            raise ValueError("amax comes with an f8 result (d_scale)")
+        amax_t = torch.empty((), dtype=torch.float32, device=a.device)
+        rets.append((dtypes.F32, amax_t.data_ptr(), []))
     if scratch == "auto":
         nbytes = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(m, k, n, rhs_contracting_dim)
         scratch = _scratch(nbytes, a.device)
@@ -117,8 +124,8 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
              "rhs_contracting_dim": ffi.Attr.i64(rhs_contracting_dim)}
     if out_f8:
         attrs["d_scale_multiplies"] = ffi.Attr.pred(d_scale_multiplies)
-    call = Call("xla_amd.fp8_scaled_dot", ffi.Frame(host(), args, rets, attrs), out,
-                keep=(a, b, a_scale, b_scale, bias, d_scale, scratch))
+    call = Call("xla_amd.fp8_scaled_dot", ffi.Frame(host(), args, rets, attrs),
+                (out, amax_t) if amax else out, keep=(a, b, a_scale, b_scale, bias, d_scale, scratch))
     return call if build_only else call.run()
 
 
