@@ -21,7 +21,7 @@ def say(msg):
 
 
 def test_handlers_replay_from_a_hip_graph():
-    say("graph capture of dequant_dot (split-K + finalize), rowwise_quantize_fp8, fp8_scaled_dot")
+    say("graph capture of dequant_dot (split-K + finalize), rowwise_quantize_fp8, fp8_scaled_dot (bf16 and f8 + amax)")
     dev = torch.device("cuda:0")
     torch.manual_seed(7)
     K, N = 2048, 1024
@@ -38,7 +38,10 @@ def test_handlers_replay_from_a_hip_graph():
     calls = [ops.dequant_dot(lhs, w4, sc, bias, weight_dtype="s4", weight_shape=(K, N), epilogue="BIAS_SILU",
                              dequant_type="bf16", build_only=True),
              ops.rowwise_quantize_fp8(x, gamma, build_only=True),
-             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="GELU", build_only=True)]
+             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="GELU", build_only=True),
+             # f8 result with its amax: a one-thread kernel zeroes the amax, then atomics fold into it
+             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="RELU", d_scale=torch.full((), 0.05, device=dev),
+                                amax=True, build_only=True)]
 
     def results():
         out = []
@@ -75,7 +78,7 @@ def test_handlers_replay_from_a_hip_graph():
         want = results()
         for c in calls:  # wipe the outputs so that a replay that does nothing cannot pass
             for t in (c.result if isinstance(c.result, (list, tuple)) else [c.result]):
-                t.view(torch.uint8).zero_()
+                t.reshape(-1).view(torch.uint8).zero_()
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
