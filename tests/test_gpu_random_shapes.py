@@ -1,0 +1,98 @@
+"""Seeded random shapes through every handler against the oracle: ragged M, K, N and group sizes,
+every epilogue, both typings -- whatever kernel the launcher picks for them."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import dev_bf16
+from tests.test_gpu_dequant_dot import compare, run_dot
+from tests.test_gpu_fp8_dot import EPI, floor_for, reference, run
+from tests.gpu_util import check_dot
+from xla_amd import dtypes, ffi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+EPILOGUES = ["DEFAULT", "BIAS", "RELU", "BIAS_RELU", "GELU", "BIAS_GELU", "SILU", "BIAS_SILU"]
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def test_dequant_dot_random_shapes(oracle):
+    rng = np.random.default_rng(2024)
+    kernels = set()
+    for case in range(36):
+        bits = int(rng.choice([4, 8]))
+        M = int(rng.choice([1, 2, 5, 8, 13, 16, 17, 31, 32, 40, 64, 65, 100, 200]))
+        group = int(rng.choice([8, 16, 32, 64, 128]))
+        K = group * int(rng.integers(1, 40))
+        N = int(rng.choice([8, 24, 64, 100, 128, 136, 256, 520, 1000]))
+        per_channel = bool(rng.integers(0, 2))
+        if per_channel:
+            group = K
+        if bits == 4 and (K * N) % 2:
+            N += 1
+        epilogue = EPILOGUES[int(rng.integers(0, 8))]
+        typed = "bf16" if rng.integers(0, 2) else "f32"
+        if typed == "f32" and not per_channel:
+            typed = "bf16"          # grouped scales under an f32 multiply go to the generic kernel only
+        say("dequant_dot #%d s%d M=%d K=%d N=%d group=%d %s %s" % (case, bits, M, K, N, group, epilogue, typed))
+        lhs = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+        wq = rng.integers(-8 if bits == 4 else -127, 8 if bits == 4 else 128, size=(K, N)).astype(np.int8)
+        sc = rng.uniform(1e-3, 2e-2, size=(K // group, N)).astype(np.float32)
+        if per_channel:
+            sc = sc.reshape(N)
+        w = dict(lhs=lhs, weights=wq, scales=dtypes.f32_to_bf16(sc) if typed == "bf16" else sc,
+                 bias=dtypes.f32_to_bf16(rng.standard_normal(N).astype(np.float32)) if "BIAS" in epilogue else None,
+                 weight_dtype="s%d" % bits, weight_shape=(K, N), group=group, dequant_type=typed, epilogue=epilogue)
+        got, kern = run_dot(w)
+        kernels.add(kern.split("_v")[0])
+        compare(oracle, w, got, "#%d %s" % (case, kern))
+    assert len(kernels) >= 3, kernels    # decode, tiled and generic all took part
+
+
+def test_fp8_dot_random_shapes(oracle):
+    rng = np.random.default_rng(77)
+    for case in range(16):
+        M = int(rng.choice([1, 7, 16, 100, 256, 300]))
+        K = 16 * int(rng.integers(1, 40)) if rng.integers(0, 4) else int(rng.integers(1, 300))
+        N = int(rng.choice([16, 40, 64, 200, 256, 272]))
+        nk = bool(rng.integers(0, 2))
+        w = workloads.c3_fp8(M, K, N)
+        w["epilogue"] = EPILOGUES[int(rng.integers(0, 8))]
+        if "BIAS" not in w["epilogue"]:
+            w["bias"] = None
+        vec = int(rng.integers(0, 4))
+        if vec & 1:
+            w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+        if vec & 2:
+            w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+        say("fp8_scaled_dot #%d M=%d K=%d N=%d nk=%s %s scales=%d" % (case, M, K, N, nk, w["epilogue"], vec))
+        got, kern = run(w, nk=nk)
+        n_floor = check_dot(got, reference(oracle, w), floor_for(w, exact_kernel="exact" in kern), "#%d %s" % (case, kern))
+        assert n_floor <= max(8, got.size // 20)
+
+
+def test_rowwise_quantize_random_shapes(oracle):
+    rng = np.random.default_rng(5)
+    for case in range(12):
+        R = int(rng.integers(1, 40))
+        C = int(rng.choice([8, 33, 256, 1000, 1024, 4096, 5000, 8192, 16384]))
+        rms = bool(rng.integers(0, 2))
+        say("rowwise_quantize_fp8 #%d R=%d C=%d rmsnorm=%s" % (case, R, C, rms))
+        x = dtypes.f32_to_bf16((rng.standard_normal((R, C)) * rng.choice([1e-3, 1.0, 300.0])).astype(np.float32))
+        g = dtypes.f32_to_bf16(rng.uniform(0.5, 1.5, C).astype(np.float32))
+        q, s = ops.rowwise_quantize_fp8(dev_bf16(x), dev_bf16(g) if rms else None, eps=1e-6)
+        torch.cuda.synchronize()
+        if rms:
+            q_ref, s_ref = oracle.rmsnorm_quantize_fp8(x, g, eps=1e-6)
+        else:  # without RMSNorm the pattern is amax / 448, divide, clamp, convert: plain numpy
+            xf = dtypes.bf16_to_f32(x)
+            s_ref = (np.abs(xf).max(axis=1) / np.float32(448)).astype(np.float32)
+            q_ref = oracle.f32_to_f8e4m3fn(np.clip((xf / s_ref[:, None]).astype(np.float32), -448, 448))
+        assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32)), case
+        assert np.array_equal(q.cpu().numpy().view(np.uint8), q_ref), case
