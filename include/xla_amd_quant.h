@@ -67,7 +67,9 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  * f8e4m3fn scaled dot.  Replaces `__cublas$lt$matmul$f8`
  * (xla/backends/gpu/transforms/gemm_rewriter.cc:1235-1591, executed by
  * CublasLtMatmulThunk -> hipBLASLt, xla/stream_executor/rocm/hip_blas_lt.cc:468-484).
- *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1);
+ *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1); or both
+ *         with one leading batch dimension ([B,M,K], [B,K,N]|[B,N,K], out [B,M,N]: the batched
+ *         dot of gemm_rewriter_fp8_test.cc:941-957), then with per-tensor scales only;
  *         a_scale F32 [] or [M] (one per row of a, as a row-wise quantizer produces them);
  *         b_scale F32 [] or [N] (one per output channel); bias BF16|F32 [N] (only with BIAS*)
  *         d_scale F32 [] (last; only when out is F8E4M3FN)
@@ -165,6 +167,8 @@ typedef struct XlaAmdFp8ScaledDot {
   const float* d_scale;        /* device scalar, only with an F8E4M3FN result */
   float* amax;                 /* optional device scalar result with an F8E4M3FN result:
                                   max |v| over all outputs, NaN if any v is NaN */
+  int64_t batch;               /* 0 or 1: a [M,K], b [K,N]|[N,K]; B > 1: a [B,M,K], b [B,K,N]|[B,N,K],
+                                  out [B,M,N], scales per tensor only; negative: empty batch */
 } XlaAmdFp8ScaledDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);

@@ -204,6 +204,39 @@ def test_f8_result_amax(oracle, force):
     assert np.isnan(float(amax))
 
 
+@pytest.mark.parametrize("nk,N", [(True, 272), (False, 272), (False, 200)])
+def test_batched(oracle, nk, N):
+    """One leading batch dimension: every batch against the oracle, bf16 and f8 results (with the
+    amax over all batches); a [K,N] rhs whose N has no whole 16-channel chunks takes the exact kernel."""
+    say("fp8_scaled_dot batched nk=%s N=%d" % (nk, N))
+    B, M, K = 3, 150, 256
+    ws = [workloads.c3_fp8(M, K, N) for _ in range(B)]
+    rng = np.random.default_rng(3)
+    for i, w in enumerate(ws):   # different data per batch
+        w["a"] = np.roll(w["a"], 17 * i, axis=0)
+        w["b"] = np.roll(w["b"], 5 * i, axis=1)
+    a = dev_u8(np.stack([w["a"] for w in ws]))
+    b = dev_u8(np.stack([np.ascontiguousarray(w["b"].T) if nk else w["b"] for w in ws]))
+    s64, bias = dev_f32(np.array(1 / 64, np.float32)), dev_bf16(ws[0]["bias"])
+    out = ops.fp8_scaled_dot(a, b, s64, s64, bias, rhs_contracting_dim=1 if nk else 0, epilogue="BIAS_GELU")
+    torch.cuda.synchronize()
+    kern = ffi.last_kernel()
+    assert ("exact" in kern) == (N % 16 != 0), kern
+    got = host_bf16(out)
+    for i, w in enumerate(ws):
+        check_dot(got[i], reference(oracle, w), floor_for(w, exact_kernel="exact" in kern), "batch %d %s" % (i, kern))
+    z = np.float32(0.0117)
+    out8, amax = ops.fp8_scaled_dot(a, b, s64, s64, bias, rhs_contracting_dim=1 if nk else 0, epilogue="BIAS_GELU",
+                                    d_scale=dev_f32(np.array(z, np.float32)), amax=True)
+    torch.cuda.synchronize()
+    want_amax = 0.0
+    for i, w in enumerate(ws):
+        ref, val = oracle.fp8_scaled_dot(w["a"], w["b"], 1 / 64, 1 / 64, bias=w["bias"], epilogue="gelu_tanh", d_scale=z)
+        check_f8_result(out8[i].cpu().numpy(), ref, val, z, True, floor_for(w, exact_kernel="exact" in kern), "f8 batch %d" % i)
+        want_amax = max(want_amax, float(np.max(np.abs(val))))
+    assert abs(float(amax) - want_amax) <= want_amax * 2.0 ** -7
+
+
 def test_f8_result_special_values(oracle):
     """NaN operands give NaN codes, a huge value over a tiny scale saturates at +-448, -0 stays -0;
     a zero scale follows IEEE (x/0 = +-inf -> +-448, 0/0 = NaN)."""

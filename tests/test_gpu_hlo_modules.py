@@ -120,6 +120,25 @@ def test_c3_module_f8_result_with_amax(oracle):
     assert (out.cpu().numpy().view(np.uint8) != ref_codes).sum() <= out.numel() // 50
 
 
+def test_batched_fp8_module(oracle):
+    say("module batched fp8 dot")
+    B, M, K, N = 4, 64, 128, 48
+    rng = np.random.default_rng(12)
+    a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((B, M, K)) * 32, -448, 448).astype(np.float32))
+    b = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((B, K, N)) * 32, -448, 448).astype(np.float32))
+    sa, sb = np.array(0.03, np.float32), np.array(0.011, np.float32)
+    text = hm.fp8_batched(B, M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(a), dev_u8(b), dev_f32(sa), dev_f32(sb)])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [DEFAULT]"]
+    ref = reference(text, [a, b, sa, sb])
+    got = host_bf16(out)
+    for i in range(B):
+        fa = np.abs(dtypes.f8e4m3fn_to_f32(a[i]).astype(np.float64)) * 0.03
+        fb = np.abs(dtypes.f8e4m3fn_to_f32(b[i]).astype(np.float64)) * 0.011
+        check_dot(got[i], ref[i], dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "batch %d" % i)
+
+
 def test_quantize_then_fp8_dot_module(oracle):
     """RMSNorm + quantize feeding an f8 dot: two custom calls after the pass, against the op-by-op
     evaluation of the original module."""

@@ -74,6 +74,19 @@ def test_c3_f8_result_with_amax(oracle):
     assert np.float32(amax) == np.max(np.abs(val)) and amax > 0
 
 
+@pytest.mark.parametrize("nk", [False, True])
+def test_batched_fp8_dot(oracle, nk):
+    B, M, K, N = 3, 5, 48, 7
+    rng = np.random.default_rng(8)
+    a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((B, M, K)) * 32, -448, 448).astype(np.float32))
+    b = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((B, K, N)) * 32, -448, 448).astype(np.float32))
+    sa, sb = np.array(0.03, np.float32), np.array(0.011, np.float32)
+    bb = np.ascontiguousarray(b.transpose(0, 2, 1)) if nk else b
+    got = run_module(hm.fp8_batched(B, M, K, N, rhs_nk=nk), [a, bb, sa, sb])
+    for i in range(B):
+        assert np.array_equal(got[i], oracle.fp8_scaled_dot(a[i], b[i], sa, sb))
+
+
 def test_quantize_then_fp8_dot(oracle):
     R, C, N = 6, 96, 10
     x = workloads.c4_quantize(R, C)

@@ -151,6 +151,21 @@ def test_c3_fp8_with_f8_result():
     assert rw == [] and any("is f32, the kernels produce bf16" in r for r in rf)
 
 
+def test_batched_fp8_dot():
+    """One leading batch dimension on both operands (gemm_rewriter_fp8_test.cc:941-957): operands
+    and result keep their rank, rhs_contracting_dim counts inside the matrix; per-row scales
+    on a batched dot are left alone."""
+    for nk in (False, True):
+        new, rw, rf = hlo.rewrite(hm.fp8_batched(10, 16, 32, 16, rhs_nk=nk))
+        assert rw == ["dot -> xla_amd.fp8_scaled_dot [DEFAULT]"] and rf == []
+        check(new, r"bf16\[10,16,16\]\{2,1,0\}.* custom-call\(%x, %y, %x_scale, %y_scale\)",
+              r"rhs_contracting_dim = %d : i64" % (1 if nk else 0))
+    bad = hm.fp8_batched(10, 16, 32, 16).replace("%x_scale = f32[] parameter(2)", "%x_scale = f32[16] parameter(2)") \
+            .replace("broadcast(%x_scale), dimensions={}", "broadcast(%x_scale), dimensions={1}")
+    new, rw, rf = hlo.rewrite(bad)
+    assert rw == [] and "custom-call" not in new
+
+
 def test_quantizer_feeding_a_dot_becomes_two_calls():
     """The quantizer's broadcast scales are reused by the dequantising multiply of the next dot:
     both patterns are taken, the dot reads the quantizer's two results, and none of the

@@ -388,8 +388,8 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   if (Preamble(f, 4, 6, 1, 3, &err)) return err;
   Decoder d{f};
   const uint64_t f8 = Bit(XLA_FFI_DataType_F8E4M3FN);
-  XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 2, "a");
-  XLA_FFI_Buffer* b = d.Arg(1, f8, 2, 2, "b");
+  XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 3, "a");
+  XLA_FFI_Buffer* b = d.Arg(1, f8, 2, 3, "b");
   XLA_FFI_Buffer* sa = d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
   XLA_FFI_Buffer* sb = d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
   // an F8E4M3FN result brings its scale as the last operand; a bias, if any, sits before it
@@ -402,7 +402,7 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
                                           : "xla_amd.fp8_scaled_dot: a BF16 result takes a, b, a_scale, b_scale[, bias]");
   XLA_FFI_Buffer* bias = n_bias ? d.Arg(4, kFloatMask, 1, 1, "bias") : nullptr;
   XLA_FFI_Buffer* sd = out_f8 ? d.Arg(4 + (int)n_bias, Bit(XLA_FFI_DataType_F32), 0, 0, "d_scale") : nullptr;
-  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F8E4M3FN), 2, 2, "out");
+  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F8E4M3FN), 2, 3, "out");
   // after out: an f32 scalar is the amax of an f8 result, a byte vector is scratch
   XLA_FFI_Buffer* amax = nullptr;
   XLA_FFI_Buffer* ws = nullptr;
@@ -422,14 +422,19 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   if (!d.ok()) return d.Error();
 
   XlaAmdFp8ScaledDot p{};
-  p.M = a->dims[0];
-  p.K = a->dims[1];
+  const int lead = a->rank == 3 ? 1 : 0;  // one leading batch dimension, on all three or on none
+  p.M = a->dims[lead];
+  p.K = a->dims[lead + 1];
+  p.batch = lead ? (a->dims[0] > 0 ? a->dims[0] : -1) : 1;  // -1: an empty batch, nothing to do
   std::string why;
   if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
+  else if (b->rank != a->rank || out->rank != a->rank) why = "a, b and out must have the same rank";
+  else if (lead && (b->dims[0] != p.batch || out->dims[0] != p.batch)) why = "batch dimensions differ";
+  else if (lead && (sa->rank != 0 || sb->rank != 0)) why = "a batched dot takes per-tensor scales";
   else {
-    p.N = b->dims[1 - rcd];
-    if (b->dims[rcd] != p.K) why = "contracting dimensions differ";
-    else if (out->dims[0] != p.M || out->dims[1] != p.N) why = "result shape must be M,N";
+    p.N = b->dims[lead + 1 - rcd];
+    if (b->dims[lead + rcd] != p.K) why = "contracting dimensions differ";
+    else if (out->dims[lead] != p.M || out->dims[lead + 1] != p.N) why = "result shape must be M,N";
     else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
     else if (((at.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
     else if (sa->rank == 1 && sa->dims[0] != p.M) why = "a rank-1 a_scale must have M elements";

@@ -249,7 +249,9 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_
         Instr* ab = cur->users[which];
         Instr* rd = ab->Is("abs") ? SoleUser(ab) : nullptr;
         if (!rd || !rd->Is("reduce") || rd->operands.size() != 2 || rd->operands[0] != ab) continue;
-        if (rd->DimsAttr("dimensions") != std::vector<int64_t>{0, 1} || !rd->operands[1]->Is("constant") ||
+        std::vector<int64_t> all_dims;
+        for (int64_t i = 0; i < rank; ++i) all_dims.push_back(i);
+        if (rd->DimsAttr("dimensions") != all_dims || !rd->operands[1]->Is("constant") ||
             rd->operands[1]->literal != "-inf")
           continue;
         const std::string* to = rd->Attr("to_apply");
@@ -373,17 +375,30 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
     return false;
   };
   if (a.type != b.type) return refuse("operands are dequantised in different types");
-  if (dot->shape.rank() != 2 || a.value->shape.rank() != 2 || b.value->shape.rank() != 2)
-    return refuse("only rank-2 dots are supported");
-  if (!dot->DimsAttr("lhs_batch_dims").empty()) return refuse("batch dimensions are not supported");
+  // [M,K] . [K,N]|[N,K], or the same with one leading batch dimension on both operands
+  // (gemm_rewriter_fp8_test.cc:941-957)
+  const int64_t rank = dot->shape.rank();
+  if ((rank != 2 && rank != 3) || a.value->shape.rank() != rank || b.value->shape.rank() != rank)
+    return refuse("only rank-2 dots and rank-3 dots with one batch dimension are supported");
+  const int64_t lead = rank - 2;
+  const std::vector<int64_t> want_batch = lead ? std::vector<int64_t>{0} : std::vector<int64_t>{};
+  if (dot->DimsAttr("lhs_batch_dims") != want_batch || dot->DimsAttr("rhs_batch_dims") != want_batch)
+    return refuse(lead ? "the batch dimension must be the leading one of both operands"
+                       : "batch dimensions are not supported on rank-2 operands");
   auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
-  if (lc.size() != 1 || rc.size() != 1 || lc[0] != 1) return refuse("lhs must contract its minor dimension");
+  if (lc.size() != 1 || rc.size() != 1 || lc[0] != rank - 1 || rc[0] < lead)
+    return refuse("lhs must contract its minor dimension");
+  rc[0] -= lead;  // from here on: 0 = rhs [K,N], 1 = rhs [N,K]
+  if (lead && (a.scale_dim >= 0 || b.scale_dim >= 0)) return refuse("a batched dot takes per-tensor scales");
   if (!IsFloatTy(dot->shape.dtype)) return refuse("dot result type " + dot->shape.dtype);
   Epilogue ep;
   std::string why;
   if (!MatchEpilogue(dot, &ep, &why, /*f8_result_in=*/&mod)) return refuse(why);
 
-  const int64_t M = a.value->shape.dims[0], K = a.value->shape.dims[1], N = b.value->shape.dims[1 - rc[0]];
+  const int64_t M = a.value->shape.dims[lead], K = a.value->shape.dims[lead + 1];
+  const int64_t N = b.value->shape.dims[lead + 1 - rc[0]];
+  std::vector<int64_t> out_dims = {M, N};
+  if (lead) out_dims.insert(out_dims.begin(), a.value->shape.dims[0]);
   // a vector of scales must run along the operand's free dimension (rows of a, output channels
   // of b): along K it does not factor out of the sum
   if (a.scale_dim == 1) return refuse("the lhs scales vary along the contracting dimension");
@@ -416,7 +431,7 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
   std::vector<Instr*> ops = {a.value, b.value, scale_of(a), scale_of(b)};
   if (ep.bias) ops.push_back(ep.bias);
   if (ep.d_scale) ops.push_back(ep.d_scale);
-  std::vector<Shape> results = {Shape::Array(ep.d_scale ? "f8e4m3fn" : "bf16", {M, N})};
+  std::vector<Shape> results = {Shape::Array(ep.d_scale ? "f8e4m3fn" : "bf16", out_dims)};
   if (ep.amax) results.push_back(Shape::Array("f32", {}));
   size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0]) : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));

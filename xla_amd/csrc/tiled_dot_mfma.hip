@@ -237,8 +237,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const __amdgpu_buffer_rsrc_t ra =
       tile_rsrc(p.a + (size_t)batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
   const __amdgpu_buffer_rsrc_t rb =
-      F8 ? tile_rsrc(p.b, (uint32_t)p.N * (uint32_t)p.K)
-                   : tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
+      tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);  // bytes, either layout
 
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
   // of row l/8 with global chunk (l%8) ^ ((row >> 1) & 7): any 16 consecutive rows then cover
@@ -472,7 +471,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.d_mode = 0;
   d.dz = d.drz = d.dlim = 1.0f;
   if (OUT_F8) {
-    d.out8 = p.out8;
+    d.out8 = p.out8 + (size_t)batch * p.M * p.N;
     d.dz = *p.d_scale;
     d.drz = 1.0f / d.dz;
     d.dlim = 1792.0f * d.dz;
@@ -584,6 +583,11 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
   const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+  // one batch per blockIdx.y
+  p.a += (size_t)blockIdx.y * p.M * p.K;
+  p.b += (size_t)blockIdx.y * p.K * p.N;
+  if (p.out) p.out += (size_t)blockIdx.y * total;
+  if (p.out8) p.out8 += (size_t)blockIdx.y * total;
   float sa = p.a_scale[p.a_per_row ? m : 0], sb = p.b_scale[p.b_per_channel ? n : 0];
   if (deq_bf16) { sa = round_bf16(sa); sb = round_bf16(sb); }
   float acc = 0.0f;
@@ -671,7 +675,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: unknown epilogue %d", p.epilogue);
   if ((p.epilogue & 1) && !p.bias)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: BIAS epilogue without a bias");
-  if (p.M == 0 || p.N == 0) {
+  if (p.M == 0 || p.N == 0 || p.batch < 0) {
     if (p.amax && p.out_dtype == XLA_FFI_DataType_F8E4M3FN) {  // maximum over nothing: its init, -inf
       hipLaunchKernelGGL(store_u32_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<uint32_t*>(p.amax), 0xff800000u);
       int rc = CheckLaunch("fp8_scaled_dot_amax_init");
@@ -724,6 +728,10 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
 
   const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled
   const bool nk = p.rhs_contracting_dim == 1;
+  const int batch = p.batch > 1 ? (int)p.batch : 1;
+  if (p.batch > 65535) return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: more than 65535 batches");
+  if (batch > 1 && vector_scales)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: a batched dot takes per-tensor scales");
   bool tiled_ok = p.K % 16 == 0 && p.K > 0 && ((uintptr_t)p.a % 16 == 0) && force != 1 &&
                   !(deq_bf16 && vector_scales) &&
                   (double)p.M * p.K < 2147483000.0 && (double)p.N * p.K < 2147483000.0;
@@ -733,7 +741,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const bool kn_direct = tiled_ok && !nk && p.N % 16 == 0 && ((uintptr_t)p.b % 16 == 0) &&
                          GetOption("fp8_dot_layout") != 1;
   if (tiled_ok && !nk && !kn_direct) {
-    if (p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
+    // (the pre-pass handles one matrix: a batched [K,N] rhs with ragged N takes the exact kernel)
+    if (batch == 1 && p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
       if (p.N % 4 == 0 && ((uintptr_t)p.b % 4 == 0)) {
         dim3 tgrid((unsigned)((p.N + 127) / 128), (unsigned)((p.K + 127) / 128));
         hipLaunchKernelGGL(transpose_bytes_fast_kernel, tgrid, dim3(256), 0, stream, (const uint8_t*)p.b,
@@ -757,17 +766,17 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
                 "for a [K,N] rhs, a workspace of K*N bytes");
   if (p.K == 0) tiled_ok = false;
 
-  dim3 egrid((unsigned)(((size_t)p.M * p.N + 255) / 256));
+  dim3 egrid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)batch);
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;
     int rc;
     if (out_f8)
-      rc = kn_direct ? launch_tiled<kFp8KN, true>(tt, 1, stream, "fp8_scaled_dot_tiled_kn_f8")
-                     : launch_tiled<kFp8, true>(tt, 1, stream, "fp8_scaled_dot_tiled_f8");
+      rc = kn_direct ? launch_tiled<kFp8KN, true>(tt, batch, stream, "fp8_scaled_dot_tiled_kn_f8")
+                     : launch_tiled<kFp8, true>(tt, batch, stream, "fp8_scaled_dot_tiled_f8");
     else
-      rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn")
-                     : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
+      rc = kn_direct ? launch_tiled<kFp8KN>(tt, batch, stream, "fp8_scaled_dot_tiled_kn")
+                     : launch_tiled<kFp8>(tt, batch, stream, "fp8_scaled_dot_tiled");
     if (rc) return rc;
     if (deq_bf16) {
       // runs only if a scale is not a power of two (decided on the device, no host read)

@@ -122,6 +122,30 @@ ENTRY %main {{
 """
 
 
+def fp8_batched(B=10, M=16, K=32, N=16, rhs_nk=False):
+    """Batched f8 dot with per-tensor scales -> bf16 (the shape of gemm_rewriter_fp8_test.cc:941-957,
+    with the result converted to bf16)."""
+    bshape = f"{B},{N},{K}" if rhs_nk else f"{B},{K},{N}"
+    rcd = 2 if rhs_nk else 1
+    return f"""HloModule fp8_batched_scaled_dot
+
+ENTRY %main {{
+  %x = f8e4m3fn[{B},{M},{K}] parameter(0)
+  %y = f8e4m3fn[{bshape}] parameter(1)
+  %x_scale = f32[] parameter(2)
+  %y_scale = f32[] parameter(3)
+  %x_f32 = f32[{B},{M},{K}] convert(%x)
+  %y_f32 = f32[{bshape}] convert(%y)
+  %x_scale_b = f32[{B},{M},{K}] broadcast(%x_scale), dimensions={{}}
+  %y_scale_b = f32[{bshape}] broadcast(%y_scale), dimensions={{}}
+  %x_unscaled = f32[{B},{M},{K}] multiply(%x_f32, %x_scale_b)
+  %y_unscaled = f32[{bshape}] multiply(%y_f32, %y_scale_b)
+  %dot = f32[{B},{M},{N}] dot(%x_unscaled, %y_unscaled), lhs_contracting_dims={{2}}, rhs_contracting_dims={{{rcd}}}, lhs_batch_dims={{0}}, rhs_batch_dims={{0}}
+  ROOT %out = bf16[{B},{M},{N}] convert(%dot)
+}}
+"""
+
+
 def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False, amax=False):
     """The f32-typed C3 module with an f8e4m3fn result: the GELU value is divided (or multiplied)
     by a per-tensor scale, clamped to +-448 and converted -- the D scaling of

@@ -94,11 +94,11 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
     or out * d_scale with d_scale_multiplies; with amax=True the call also returns max |out| (f32 [])
     as a second tensor."""
     _check_cuda(a, b, a_scale, b_scale, bias, d_scale)
-    m, k = a.shape
-    n = b.shape[1 - rhs_contracting_dim]
+    *lead, m, k = a.shape          # one leading batch dimension, or none
+    n = b.shape[len(lead) + 1 - rhs_contracting_dim]
     out_f8 = d_scale is not None
     if out is None:
-        out = torch.empty((m, n), dtype=torch.uint8 if out_f8 else torch.bfloat16, device=a.device)
+        out = torch.empty((*lead, m, n), dtype=torch.uint8 if out_f8 else torch.bfloat16, device=a.device)
     args = [(dtypes.F8E4M3FN, a.data_ptr(), a.shape), (dtypes.F8E4M3FN, b.data_ptr(), b.shape),
             (dtypes.F32, a_scale.data_ptr(), list(a_scale.shape)),
             (dtypes.F32, b_scale.data_ptr(), list(b_scale.shape))]
@@ -106,7 +106,7 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
     if out_f8:
         args.append((dtypes.F32, d_scale.data_ptr(), list(d_scale.shape)))
-    rets = [(dtypes.F8E4M3FN if out_f8 else dtypes.BF16, out.data_ptr(), [m, n])]
+    rets = [(dtypes.F8E4M3FN if out_f8 else dtypes.BF16, out.data_ptr(), [*lead, m, n])]
     amax_t = None
     if amax:
         if not out_f8:
