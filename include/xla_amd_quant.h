@@ -70,6 +70,8 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1); or both
  *         with one leading batch dimension ([B,M,K], [B,K,N]|[B,N,K], out [B,M,N]: the batched
  *         dot of gemm_rewriter_fp8_test.cc:941-957), then with per-tensor scales only;
+ *         a_scale, b_scale F8E8M0FNU [M,K/32], [N,K/32] with b = [N,K]: block-scaled (MXFP8)
+ *         operands, "__op$block_scaled_dot" of block_scaling_rewriter.h:48-69; otherwise
  *         a_scale F32 [] or [M] (one per row of a, as a row-wise quantizer produces them);
  *         b_scale F32 [] or [N] (one per output channel); bias BF16|F32 [N] (only with BIAS*)
  *         d_scale F32 [] (last; only when out is F8E4M3FN)
@@ -167,6 +169,10 @@ typedef struct XlaAmdFp8ScaledDot {
   const float* d_scale;        /* device scalar, only with an F8E4M3FN result */
   float* amax;                 /* optional device scalar result with an F8E4M3FN result:
                                   max |v| over all outputs, NaN if any v is NaN */
+  const void* a_block_scales;  /* MXFP8: f8e8m0fnu [M, K/32], one scale per 32 elements of K of a;   */
+  const void* b_block_scales;  /* f8e8m0fnu [N, K/32] for b = [N,K]; both or neither; a_scale and   */
+  int32_t block;               /* b_scale are unused then; block must be 32                          */
+  int32_t reserved0;
   int64_t batch;               /* 0 or 1: a [M,K], b [K,N]|[N,K]; B > 1: a [B,M,K], b [B,K,N]|[B,N,K],
                                   out [B,M,N], scales per tensor only; negative: empty batch */
 } XlaAmdFp8ScaledDot;

@@ -85,7 +85,7 @@ def evaluate(module_json, args):
             v = args[int(ins["literal"])]
             if ty == "bf16":
                 v = O.bf16_to_f32(v)
-            elif ty == "f8e4m3fn":
+            elif ty in ("f8e4m3fn", "f8e8m0fnu"):
                 v = np.ascontiguousarray(v, np.uint8)
             elif ty in ("s8", "s4"):
                 v = np.ascontiguousarray(v, np.int8)
@@ -155,6 +155,14 @@ def evaluate(module_json, args):
                 v = _round(np.maximum(np.max(np.asarray(x[0], np.float32), axis=-1), np.asarray(x[1], np.float32)), ty)
             else:
                 raise NotImplementedError("reduce with " + kind)
+        elif op == "custom-call" and ins["attrs"].get("custom_call_target", "").strip('"') == "__op$block_scaled_dot":
+            # what BlockScalingRewriter expands it to (block_scaling_rewriter.cc:194-219, :521-571):
+            # convert, multiply by the scale of each block of the minor dimension, contract minor with minor
+            a8, b8, sa, sb = x
+            blk = a8.shape[-1] // sa.shape[-1]
+            ad = _round(O.f8e4m3fn_to_f32(a8) * np.repeat(O.f8e8m0fnu_to_f32(sa), blk, axis=-1), ty)
+            bd = _round(O.f8e4m3fn_to_f32(b8) * np.repeat(O.f8e8m0fnu_to_f32(sb), blk, axis=-1), ty)
+            v = _round(_dot(ad, bd, [ad.ndim - 1], [bd.ndim - 1], [], []), ty)
         elif op == "tuple":
             v = list(x)
         elif op == "get-tuple-element":

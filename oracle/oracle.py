@@ -75,6 +75,10 @@ def lib():
         L.xo_fp8_scaled_dot.restype = i32
         L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64,
                                         i32, i32, i32, vp, vp, i32, vp, vp]
+        L.xo_f8e8m0fnu_to_f32.restype = f32
+        L.xo_f8e8m0fnu_to_f32.argtypes = [c.c_uint8]
+        L.xo_block_scaled_dot.restype = i32
+        L.xo_block_scaled_dot.argtypes = [vp, vp, vp, vp, i64, vp, i32, i64, i64, i64, i32, i32, i32, vp]
         L.xo_rmsnorm_quantize_fp8.restype = i32
         L.xo_rmsnorm_quantize_fp8.argtypes = [vp, vp, f32, i64, i64, vp, vp]
         L.xo_num_threads.restype = i32
@@ -233,6 +237,32 @@ def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=N
                                  TYPES[ep_ty], EPILOGUES[epilogue], *tail)
     assert rc == 0
     return out if d_scale is None else (out8, val)
+
+
+def f8e8m0fnu_to_f32(codes):
+    codes = np.asarray(codes, np.uint8)
+    return np.array([lib().xo_f8e8m0fnu_to_f32(int(v)) for v in codes.reshape(-1)], np.float32).reshape(codes.shape)
+
+
+def block_scaled_dot(a8, b8_nk, a_sc, b_sc, block=32, bias=None, bias_ty="bf16", dot_ty="f32", ep_ty="f32",
+                     epilogue="none"):
+    """bf16 [M,N] = epilogue(dot(a8 * 2^(a_sc-127), b8 * 2^(b_sc-127))): a8 [M,K], b8 [N,K] f8e4m3fn codes,
+    scales f8e8m0fnu codes, one per `block` elements of K."""
+    a8, b8 = _c(a8, np.uint8), _c(b8_nk, np.uint8)
+    M, K = a8.shape
+    N = b8.shape[0]
+    assert b8.shape[1] == K and K % block == 0
+    a_sc, b_sc = _c(a_sc, np.uint8), _c(b_sc, np.uint8)
+    assert a_sc.shape == (M, K // block) and b_sc.shape == (N, K // block)
+    bp = None
+    if bias is not None:
+        bias = _c(bias, np.uint16 if bias_ty == "bf16" else np.float32)
+        bp = _ptr(bias)
+    out = np.empty((M, N), np.uint16)
+    rc = lib().xo_block_scaled_dot(_ptr(a8), _ptr(b8), _ptr(a_sc), _ptr(b_sc), block, bp, TYPES[bias_ty], M, K, N,
+                                   TYPES[dot_ty], TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
+    assert rc == 0
+    return out
 
 
 def rmsnorm_quantize_fp8(x_bf16, gamma_bf16, eps=1e-6):

@@ -472,6 +472,70 @@ XO_API int xo_fp8_scaled_dot(const uint8_t* A8, const uint8_t* B8, int b_is_nk,
   return rc;
 }
 
+/* -------------------------------------------------- block-scaled (MX) dot */
+
+/* f8e8m0fnu -> f32: 2^(e-127); 0xFF is NaN; there is no zero and no sign
+ * (convert_test.cc:2114-2140: 1.0 <-> 127, 2^127 <-> 254, 2^-126 <-> 1). */
+XO_API float xo_f8e8m0fnu_to_f32(uint8_t e) {
+  if (e == 0xFF) return u2f(0x7fc00000u);
+  if (e == 0) return u2f(0x00400000u); /* 2^-127, a subnormal f32 */
+  return u2f((uint32_t)e << 23);
+}
+
+/*
+ * "__op$block_scaled_dot" as BlockScalingRewriter expands it when no library
+ * kernel applies (block_scaling_rewriter.cc:194-219, :521-571): each operand
+ * is converted to the result type and multiplied by its scale, one scale per
+ * `block` consecutive elements of the contracting (minor) dimension, then the
+ * two are contracted.  A8: f8e4m3fn [M,K]; B8: f8e4m3fn [N,K]; a_sc: f8e8m0fnu
+ * [M,K/block]; b_sc: [N,K/block].  The scales are powers of two and an f8 value
+ * has a 4-bit significand, so the multiplies are exact in f32 and in bf16
+ * alike; the dot adds in f32 and the epilogue rounds as for the other dots.
+ */
+XO_API int xo_block_scaled_dot(const uint8_t* A8, const uint8_t* B8, const uint8_t* a_sc,
+                               const uint8_t* b_sc, int64_t block, const void* bias, int bias_ty,
+                               int64_t M, int64_t K, int64_t N, int dot_ty, int ep_ty, int epi,
+                               uint16_t* out) {
+  if (block <= 0 || K % block) return -2;
+  const int64_t nb = K / block;
+  float* Ad = (float*)malloc(sizeof(float) * (size_t)(M > 0 ? M : 1) * (size_t)(K > 0 ? K : 1));
+  if (!Ad) return -1;
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t k = 0; k < K; ++k) {
+      volatile float p = xo_f8e4m3fn_to_f32(A8[(size_t)m * K + k]) * xo_f8e8m0fnu_to_f32(a_sc[(size_t)m * nb + k / block]);
+      Ad[(size_t)m * K + k] = p;
+    }
+  int rc = 0;
+#pragma omp parallel
+  {
+    float* col = (float*)malloc(sizeof(float) * (size_t)(K > 0 ? K : 1));
+    if (!col) rc = -1;
+#pragma omp for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+      if (rc) continue;
+      for (int64_t k = 0; k < K; ++k) {
+        volatile float p = xo_f8e4m3fn_to_f32(B8[(size_t)n * K + k]) * xo_f8e8m0fnu_to_f32(b_sc[(size_t)n * nb + k / block]);
+        col[k] = p;
+      }
+      float bv = 0.0f;
+      if (bias)
+        bv = bias_ty == XO_BF16 ? xo_bf16_to_f32(((const uint16_t*)bias)[n]) : ((const float*)bias)[n];
+      for (int64_t m = 0; m < M; ++m) {
+        const float* a = Ad + (size_t)m * K;
+        float acc = 0.0f;
+        for (int64_t k = 0; k < K; ++k) {
+          float p = a[k] * col[k];
+          acc = acc + p;
+        }
+        out[(size_t)m * N + n] = epilogue(acc, dot_ty, ep_ty, bias != NULL, bv, epi);
+      }
+    }
+    free(col);
+  }
+  free(Ad);
+  return rc;
+}
+
 /* ------------------------------------------------- RMSNorm + fp8 quantize */
 
 /* Sum of n values as TreeReductionRewriter(32) shapes it: windows of 32

@@ -133,6 +133,21 @@ def test_shape_validation_happens_before_any_launch():
     with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0 but got 1 \\(d_scale\\)"):
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a + [(dtypes.F32, FAKE, (4,))],
                                                        [(dtypes.F8E4M3FN, FAKE, (4, 4))]))
+    # block scales: f8e8m0fnu [rows, K/32] on both operands, rhs [N,K]
+    mx = [(dtypes.F8E4M3FN, FAKE, (4, 64)), (dtypes.F8E4M3FN, FAKE, (8, 64)), (dtypes.F8E8M0FNU, FAKE, (4, 2)),
+          (dtypes.F8E8M0FNU, FAKE, (8, 2))]
+    with pytest.raises(ffi.FfiError, match="block scales go with unbatched a \\[M,K\\] and b \\[N,K\\]"):
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, mx, [(dtypes.BF16, FAKE, (4, 64))]))
+    with pytest.raises(ffi.FfiError, match="block scales must be \\[M,K/32\\] and \\[N,K/32\\]"):
+        bad = list(mx)
+        bad[3] = (dtypes.F8E8M0FNU, FAKE, (8, 3))
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, bad, [(dtypes.BF16, FAKE, (4, 8))],
+                                                       {"rhs_contracting_dim": ffi.Attr.i64(1)}))
+    with pytest.raises(ffi.FfiError, match="Wrong buffer dtype: expected F8E8M0FNU but got F32 \\(b_scale\\)"):
+        bad = list(mx)
+        bad[3] = (dtypes.F32, FAKE, (8, 2))
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, bad, [(dtypes.BF16, FAKE, (4, 8))],
+                                                       {"rhs_contracting_dim": ffi.Attr.i64(1)}))
     with pytest.raises(ffi.FfiError, match="Wrong buffer rank: expected 0..1 but got 2"):
         a2 = list(a)
         a2[2] = (dtypes.F32, FAKE, (4, 1))

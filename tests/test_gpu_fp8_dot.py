@@ -237,6 +237,68 @@ def test_batched(oracle, nk, N):
     assert abs(float(amax) - want_amax) <= want_amax * 2.0 ** -7
 
 
+def mx_case(M, K, N, seed):
+    rng = np.random.default_rng(seed)
+    a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 8, -448, 448).astype(np.float32))
+    b = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((N, K)) * 8, -448, 448).astype(np.float32))
+    sa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    sb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    return a, b, sa, sb
+
+
+def mx_floor(a, b, sa, sb, exact_kernel):
+    ad = np.abs(dtypes.f8e4m3fn_to_f32(a).astype(np.float64)) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, axis=1)
+    bd = np.abs(dtypes.f8e4m3fn_to_f32(b).astype(np.float64)) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, axis=1)
+    fl = dot_floor(ad, bd.T, a.shape[1])
+    return fl if exact_kernel else fl + 1.2 * 2.0 ** -12 * np.sqrt((ad * ad) @ (bd * bd).T)
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 512, 272), (256, 1024, 256), (100, 96, 40)])
+def test_mxfp8_block_scales(oracle, M, K, N):
+    """f8e8m0fnu scales per 32 elements of K on both operands, multiplied in by the matrix cores;
+    K that is not a multiple of 128 (and the forced slow kernel) take the exact kernel, which
+    must match the oracle bit for bit: every product and partial sum is the same f32 operation."""
+    say("fp8_scaled_dot MXFP8 M=%d K=%d N=%d" % (M, K, N))
+    a, b, sa, sb = mx_case(M, K, N, 7)
+    ref = oracle.block_scaled_dot(a, b, sa, sb)
+    da, db, dsa, dsb = dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb)
+    out = ops.fp8_scaled_dot(da, db, dsa, dsb, rhs_contracting_dim=1)
+    torch.cuda.synchronize()
+    kern = ffi.last_kernel()
+    assert kern == ("fp8_scaled_dot_tiled_mx" if K % 128 == 0 else "fp8_scaled_dot_exact"), kern
+    n_floor = check_dot(host_bf16(out), ref, mx_floor(a, b, sa, sb, "exact" in kern), kern)
+    assert n_floor <= out.numel() // 50
+    ffi.set_option("fp8_dot_kernel", 1)
+    try:
+        out = ops.fp8_scaled_dot(da, db, dsa, dsb, rhs_contracting_dim=1)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+    assert ffi.last_kernel() == "fp8_scaled_dot_exact"
+    assert np.array_equal(host_bf16(out), ref)
+
+
+def test_mxfp8_one_block_at_a_time(oracle):
+    """Data in a single 32-element block of K, a different scale on every block: each block must
+    come out multiplied by its own two scales exactly (products of small integers, exact sums)."""
+    say("fp8_scaled_dot MXFP8 block by block")
+    M, K, N = 64, 256, 64
+    rng = np.random.default_rng(2)
+    ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    bi = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    sa = np.repeat((121 + np.arange(K // 32)).astype(np.uint8)[None, :], M, axis=0)
+    sb = np.repeat((130 - np.arange(K // 32)).astype(np.uint8)[None, :], N, axis=0)
+    sb[:, :] += (np.arange(N) % 3).astype(np.uint8)[:, None]
+    for j in range(K // 32):
+        a1 = np.zeros_like(ai)
+        a1[:, 32 * j:32 * j + 32] = ai[:, 32 * j:32 * j + 32]
+        a8, b8 = dtypes.f32_to_f8e4m3fn(a1), dtypes.f32_to_f8e4m3fn(bi)
+        out = ops.fp8_scaled_dot(dev_u8(a8), dev_u8(b8), dev_u8(sa), dev_u8(sb), rhs_contracting_dim=1)
+        torch.cuda.synchronize()
+        assert ffi.last_kernel() == "fp8_scaled_dot_tiled_mx"
+        assert np.array_equal(host_bf16(out), oracle.block_scaled_dot(a8, b8, sa, sb)), j
+
+
 def test_f8_result_special_values(oracle):
     """NaN operands give NaN codes, a huge value over a tiny scale saturates at +-448, -0 stays -0;
     a zero scale follows IEEE (x/0 = +-inf -> +-448, 0/0 = NaN)."""

@@ -139,6 +139,24 @@ def test_batched_fp8_module(oracle):
         check_dot(got[i], ref[i], dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "batch %d" % i)
 
 
+def test_mxfp8_module(oracle):
+    say("module MXFP8 block-scaled dot")
+    M, K, N = 128, 256, 96
+    rng = np.random.default_rng(6)
+    a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 8, -448, 448).astype(np.float32))
+    b = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((N, K)) * 8, -448, 448).astype(np.float32))
+    sa = rng.integers(118, 134, (M, K // 32)).astype(np.uint8)
+    sb = rng.integers(118, 134, (N, K // 32)).astype(np.uint8)
+    text = hm.mxfp8_block_scaled_dot(M, K, N)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb)])
+    torch.cuda.synchronize()
+    assert rw == ["result -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]"]
+    ref = reference(text, [a, b, sa, sb])
+    ad = np.abs(dtypes.f8e4m3fn_to_f32(a).astype(np.float64)) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, axis=1)
+    bd = np.abs(dtypes.f8e4m3fn_to_f32(b).astype(np.float64)) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, axis=1)
+    check_dot(host_bf16(out), ref, dot_floor(ad, bd.T, K) + 1.2 * 2.0 ** -12 * np.sqrt((ad * ad) @ (bd * bd).T), "MXFP8 module")
+
+
 def test_quantize_then_fp8_dot_module(oracle):
     """RMSNorm + quantize feeding an f8 dot: two custom calls after the pass, against the op-by-op
     evaluation of the original module."""

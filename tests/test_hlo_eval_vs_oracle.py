@@ -87,6 +87,17 @@ def test_batched_fp8_dot(oracle, nk):
         assert np.array_equal(got[i], oracle.fp8_scaled_dot(a[i], b[i], sa, sb))
 
 
+def test_mxfp8_block_scaled_dot(oracle):
+    M, K, N = 7, 96, 5
+    rng = np.random.default_rng(10)
+    a8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 8, -448, 448).astype(np.float32))
+    b8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((N, K)) * 8, -448, 448).astype(np.float32))
+    sa = rng.integers(120, 134, (M, K // 32)).astype(np.uint8)
+    sb = rng.integers(120, 134, (N, K // 32)).astype(np.uint8)
+    got = run_module(hm.mxfp8_block_scaled_dot(M, K, N), [a8, b8, sa, sb])
+    assert np.array_equal(got, oracle.block_scaled_dot(a8, b8, sa, sb))
+
+
 def test_quantize_then_fp8_dot(oracle):
     R, C, N = 6, 96, 10
     x = workloads.c4_quantize(R, C)

@@ -237,3 +237,12 @@ def test_bf16_to_f32_exhaustive(oracle):
     got = oracle.bf16_to_f32(h)
     want = torch.from_numpy(h.copy()).view(torch.bfloat16).float().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_f8e8m0fnu_decode(oracle):
+    """convert_test.cc:2114-2140 (ConvertF32F8e8m0fnuRoundtrip): 1.0 <-> code 127, 2^127 is the
+    largest value (254), 2^-126 the smallest normal (1), there is no zero, no sign, 0xFF is NaN."""
+    v = oracle.f8e8m0fnu_to_f32(np.arange(256, dtype=np.uint8))
+    assert v[127] == 1.0 and v[254] == 2.0 ** 127 and v[1] == 2.0 ** -126 and np.isnan(v[255])
+    assert v[0] == 2.0 ** -127 and np.all(v[:255] > 0)
+    assert np.all(v[1:255] == 2.0 * v[0:254])      # every code doubles the one below

@@ -235,6 +235,39 @@ def test_fp8_dot_f8_result(oracle):
     assert set(np.unique(sat[np.abs(v2) > 1.0])) <= {0x7E, 0xFE}                  # +-448, never NaN
 
 
+def test_block_scaled_dot(oracle):
+    """MXFP8: against f64 on the dequantised operands; all scales 1.0 is the plain dot of the two
+    code matrices; doubling one block's scale adds exactly that block's contribution once more;
+    scales along the wrong axis (transposed scale matrix semantics) must change the result."""
+    rng = np.random.default_rng(44)
+    M, K, N = 6, 128, 9
+    a8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((M, K)) * 8, -448, 448).astype(np.float32))
+    b8 = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal((N, K)) * 8, -448, 448).astype(np.float32))
+    sa = rng.integers(120, 134, (M, K // 32)).astype(np.uint8)
+    sb = rng.integers(120, 134, (N, K // 32)).astype(np.uint8)
+    af, bf = dtypes.f8e4m3fn_to_f32(a8).astype(np.float64), dtypes.f8e4m3fn_to_f32(b8).astype(np.float64)
+    ad = af * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, axis=1)
+    bd = bf * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, axis=1)
+    ref = ad @ bd.T
+    got = as_f32(oracle.block_scaled_dot(a8, b8, sa, sb)).astype(np.float64)
+    assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -8 + 1e-6)
+    one_a, one_b = np.full_like(sa, 127), np.full_like(sb, 127)
+    plain = oracle.block_scaled_dot(a8, b8, one_a, one_b)
+    assert np.array_equal(plain, oracle.fp8_scaled_dot(a8, b8, 1.0, 1.0, b_is_nk=True))
+    # small integers: every sum is exact, so doubling block 2 of row 3 adds its part exactly once more
+    ai = dtypes.f32_to_f8e4m3fn(rng.integers(-3, 4, (M, K)).astype(np.float32))
+    bi = dtypes.f32_to_f8e4m3fn(rng.integers(-3, 4, (N, K)).astype(np.float32))
+    base = as_f32(oracle.block_scaled_dot(ai, bi, one_a, one_b))
+    bumped = one_a.copy()
+    bumped[3, 2] = 128
+    part = dtypes.f8e4m3fn_to_f32(ai)[3, 64:96] @ dtypes.f8e4m3fn_to_f32(bi)[:, 64:96].T
+    want = base.copy()
+    want[3] += part
+    assert np.array_equal(as_f32(oracle.block_scaled_dot(ai, bi, bumped, one_b)), want)
+    wrong = (af * np.repeat(2.0 ** (sa[::-1].astype(np.float64) - 127), 32, axis=1)) @ bd.T
+    assert not np.all(np.abs(got - wrong) <= np.abs(wrong) * 2.0 ** -8 + 1e-6)
+
+
 # ---- RMSNorm + quantize -----------------------------------------------------------
 
 def test_tree32_sum_order(oracle):

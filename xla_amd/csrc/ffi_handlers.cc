@@ -52,6 +52,7 @@ const char* DTypeName(int d) {
     case XLA_FFI_DataType_F8E4M3FNUZ: return "F8E4M3FNUZ";
     case XLA_FFI_DataType_F8E5M2FNUZ: return "F8E5M2FNUZ";
     case XLA_FFI_DataType_F8E4M3B11FNUZ: return "F8E4M3B11FNUZ";
+    case XLA_FFI_DataType_F8E8M0FNU: return "F8E8M0FNU";
     default: return "INVALID";
   }
 }
@@ -390,8 +391,13 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   const uint64_t f8 = Bit(XLA_FFI_DataType_F8E4M3FN);
   XLA_FFI_Buffer* a = d.Arg(0, f8, 2, 3, "a");
   XLA_FFI_Buffer* b = d.Arg(1, f8, 2, 3, "b");
-  XLA_FFI_Buffer* sa = d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
-  XLA_FFI_Buffer* sb = d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
+  // per-tensor / per-row / per-channel f32 scales, or f8e8m0fnu block scales [rows, K/32] on both
+  const bool mx = f->args.size > 3 && f->args.types[2] == XLA_FFI_ArgType_BUFFER &&
+                  static_cast<XLA_FFI_Buffer*>(f->args.args[2])->dtype == XLA_FFI_DataType_F8E8M0FNU;
+  XLA_FFI_Buffer* sa = mx ? d.Arg(2, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 2, "a_scale")
+                          : d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
+  XLA_FFI_Buffer* sb = mx ? d.Arg(3, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 2, "b_scale")
+                          : d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
   // an F8E4M3FN result brings its scale as the last operand; a bias, if any, sits before it
   const bool out_f8 = f->rets.types[0] == XLA_FFI_RetType_BUFFER &&
                       static_cast<XLA_FFI_Buffer*>(f->rets.rets[0])->dtype == XLA_FFI_DataType_F8E4M3FN;
@@ -428,6 +434,7 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   p.batch = lead ? (a->dims[0] > 0 ? a->dims[0] : -1) : 1;  // -1: an empty batch, nothing to do
   std::string why;
   if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
+  else if (mx && (lead || rcd != 1)) why = "block scales go with unbatched a [M,K] and b [N,K]";
   else if (b->rank != a->rank || out->rank != a->rank) why = "a, b and out must have the same rank";
   else if (lead && (b->dims[0] != p.batch || out->dims[0] != p.batch)) why = "batch dimensions differ";
   else if (lead && (sa->rank != 0 || sb->rank != 0)) why = "a batched dot takes per-tensor scales";
@@ -437,14 +444,22 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
     else if (out->dims[lead] != p.M || out->dims[lead + 1] != p.N) why = "result shape must be M,N";
     else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
     else if (((at.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
-    else if (sa->rank == 1 && sa->dims[0] != p.M) why = "a rank-1 a_scale must have M elements";
-    else if (sb->rank == 1 && sb->dims[0] != p.N) why = "a rank-1 b_scale must have N elements";
+    else if (mx && (p.K % 32 != 0 || sa->dims[0] != p.M || sb->dims[0] != p.N || sa->dims[1] != p.K / 32 ||
+                    sb->dims[1] != p.K / 32))
+      why = "block scales must be [M,K/32] and [N,K/32]";
+    else if (!mx && sa->rank == 1 && sa->dims[0] != p.M) why = "a rank-1 a_scale must have M elements";
+    else if (!mx && sb->rank == 1 && sb->dims[0] != p.N) why = "a rank-1 b_scale must have N elements";
   }
   if (!why.empty()) return InvalidArgument(f->api, "xla_amd.fp8_scaled_dot: " + why);
   p.a = a->data; p.b = b->data;
-  p.a_scale = (const float*)sa->data; p.b_scale = (const float*)sb->data;
-  p.a_scale_per_row = sa->rank == 1;
-  p.b_scale_per_channel = sb->rank == 1;
+  if (mx) {
+    p.a_block_scales = sa->data; p.b_block_scales = sb->data;
+    p.block = 32;
+  } else {
+    p.a_scale = (const float*)sa->data; p.b_scale = (const float*)sb->data;
+    p.a_scale_per_row = sa->rank == 1;
+    p.b_scale_per_channel = sb->rank == 1;
+  }
   p.out_dtype = out->dtype;
   p.d_scale = sd ? (const float*)sd->data : nullptr;
   p.d_scale_multiplies = d_mul;

@@ -9,6 +9,8 @@
 //   convert(s8|s4) * broadcast(scale) -> dot [-> +bias] [-> activation]
 //       => xla_amd.dequant_dot             (what gemm_fusion.cc:1629-1702 wraps into __triton_gemm;
 //                                           pattern zoo: fusion_emitter_int4_device_test.cc:85-449)
+//   custom-call "__op$block_scaled_dot" (f8e4m3fn operands, f8e8m0fnu scales per 32 of K)
+//       => xla_amd.fp8_scaled_dot with block scales (block_scaling_rewriter.h:48-69)
 //   [RMSNorm ->] reduce-max(abs) -> /448 -> divide -> clamp -> convert(f8e4m3fn)
 //       => xla_amd.rowwise_quantize_fp8    (today: several reduction/loop fusions,
 //                                           codegen/emitters/reduction.cc:840-991)
@@ -447,6 +449,43 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
   return true;
 }
 
+// ---------------------------------------------------------------- block-scaled (MXFP8) dot
+// custom-call(lhs f8e4m3fn [M,K], rhs f8e4m3fn [N,K], lhs_scale f8e8m0fnu [M,K/32], rhs_scale
+// [N,K/32]), custom_call_target="__op$block_scaled_dot" -> bf16 [M,N]
+// (block_scaling_rewriter.h:48-69) becomes xla_amd.fp8_scaled_dot with the scales as they are:
+// the matrix cores multiply them in.  BlockScalingRewriter would expand it into converts,
+// multiplies and a dot on anything but cuDNN (block_scaling_rewriter.cc:548-571).
+bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
+  const std::string* target = cc->Attr("custom_call_target");
+  if (!target || *target != "\"__op$block_scaled_dot\"") return false;
+  auto refuse = [&](const std::string& why) {
+    log->refusals.push_back(cc->name + ": block-scaled dot found but not rewritten: " + why);
+    return false;
+  };
+  if (cc->operands.size() != 4) return refuse("expected lhs, rhs and a scale for each");
+  Instr *a = cc->operands[0], *b = cc->operands[1], *sa = cc->operands[2], *sb = cc->operands[3];
+  if (a->shape.dtype != "f8e4m3fn" || b->shape.dtype != "f8e4m3fn" || sa->shape.dtype != "f8e8m0fnu" ||
+      sb->shape.dtype != "f8e8m0fnu")
+    return refuse("operands must be f8e4m3fn with f8e8m0fnu scales");
+  if (a->shape.rank() != 2 || b->shape.rank() != 2 || sa->shape.rank() != 2 || sb->shape.rank() != 2 ||
+      cc->shape.is_tuple || cc->shape.rank() != 2)
+    return refuse("only unbatched rank-2 operands are supported");
+  const int64_t M = a->shape.dims[0], K = a->shape.dims[1], N = b->shape.dims[0];
+  if (b->shape.dims[1] != K || K % 32 != 0 || sa->shape.dims != std::vector<int64_t>{M, K / 32} ||
+      sb->shape.dims != std::vector<int64_t>{N, K / 32})
+    return refuse("scales must be one per 32 elements of the contracting (minor) dimension");
+  if (cc->Attr("backend_config")) return refuse("a backend_config (explicit block size, global scale) is not taken");
+  if (cc->shape.dtype != "bf16" || cc->shape.dims != std::vector<int64_t>{M, N})
+    return refuse("the result is " + cc->shape.dtype + ", the kernels produce bf16 [M,N]");
+  Epilogue ep;
+  ep.ops_type = "f32";
+  std::string cfg = CommonConfig(ep, "f32", "f32") + ", rhs_contracting_dim = 1 : i64";
+  Instr* call = EmitCall(comp, cc, "xla_amd.fp8_scaled_dot", {a, b, sa, sb}, {Shape::Array("bf16", {M, N})}, cfg);
+  comp->ReplaceAllUses(cc, call);
+  log->rewrites.push_back(cc->name + " -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]");
+  return true;
+}
+
 // ---------------------------------------------------------------- weight-only dequantize dot
 struct QWeights {
   Instr* w = nullptr;       // s8 or s4 tensor [B,]K,N
@@ -672,6 +711,8 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         bool did = false;
         if (i->Is("dot") && i->operands.size() == 2) {
           did = RewriteF8Dot(*mod, comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
+        } else if (i->Is("custom-call")) {
+          did = RewriteBlockScaledDot(comp.get(), i, log);
         } else if (i->Is("convert") && i->shape.dtype == "f8e4m3fn") {
           did = RewriteQuantize(*mod, comp.get(), i, log);
         }

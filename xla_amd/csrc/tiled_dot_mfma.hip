@@ -33,7 +33,9 @@
 namespace xla_amd {
 namespace {
 
-enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2 };  // kFp8KN: fp8 with the weights given [K,N]
+// kFp8KN: fp8 with the weights given [K,N]; kFp8MX: fp8 [M,K] x [N,K] with one f8e8m0fnu scale per
+// 32 elements of K on both operands (MXFP8), multiplied in by the matrix cores themselves
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3 };
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
@@ -56,7 +58,13 @@ struct TiledParams {
   const float* d_scale;  // its per-tensor scale, a device scalar
   int d_divides;         // the value is divided by the scale (else multiplied)
   float* amax;           // optional f32 scalar result: max |v| over the f8 result's values
+  const uint8_t* a_block_scales;  // kFp8MX: f8e8m0fnu [M, K/32]
+  const uint8_t* b_block_scales;  // kFp8MX: f8e8m0fnu [N, K/32]
 };
+
+__device__ __forceinline__ float e8m0_to_f32(uint32_t e) {
+  return e == 0xffu ? bits_to_f32(0x7fc00000u) : e == 0u ? bits_to_f32(0x00400000u) : bits_to_f32(e << 23);
+}
 
 __device__ __forceinline__ bool is_pow2_f32(float s) {
   const uint32_t u = f32_to_bits(s);
@@ -194,12 +202,14 @@ template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr bool F8 = KIND != kS8;       // both operands f8e4m3fn
   constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
+  constexpr bool MX = KIND == kFp8MX;    // block scales ride along with every stage
+  constexpr bool BNK = KIND == kFp8 || MX;  // f8 weights [N,K]: staged like the activations
   constexpr int ESZ = F8 ? 1 : 2;  // bytes per activation element
   constexpr int KS = kRow / ESZ;             // K elements per stage
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [2][(kTM + kTN) * kRow]
   constexpr int kBufBytes = (kTM + kTN) * kRow;
 
-  if (F8 && p.require_pow2_scales) {
+  if (F8 && !MX && p.require_pow2_scales) {
     if (!(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;  // the exact kernel runs
   }
 
@@ -239,6 +249,12 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const __amdgpu_buffer_rsrc_t rb =
       tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);  // bytes, either layout
 
+  // kFp8MX: scales [rows, K/32]; lane l of wave w owns tile row (w & 3) * 64 + l of its operand
+  const int nblk = p.K >> 5;
+  const __amdgpu_buffer_rsrc_t rsa = tile_rsrc(MX ? p.a_block_scales : p.a, MX ? (uint32_t)p.M * (uint32_t)nblk : 0u);
+  const __amdgpu_buffer_rsrc_t rsb = tile_rsrc(MX ? p.b_block_scales : p.a, MX ? (uint32_t)p.N * (uint32_t)nblk : 0u);
+  const uint32_t sc_voff = (uint32_t)((wave < 4 ? m0 : n0) + (wave & 3) * 64 + lane) * (uint32_t)nblk;
+
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
   // of row l/8 with global chunk (l%8) ^ ((row >> 1) & 7): any 16 consecutive rows then cover
   // all 64 banks with one 16-byte chunk each, which is what ds_read_b128 needs for its full
@@ -252,7 +268,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   for (int j = 0; j < 4; ++j) {
     const int r = wave * 32 + j * 8 + ld_row;
     voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk[j & 1] * 16;
-    if (KIND == kFp8) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
+    if (BNK) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
     if (BKN) {
       // [K,N]: instruction j of this wave moves 4 rows of K x 256 channels; lane l fills slot l%16
       // of row l/16 with global chunk (l%16) ^ ((k & 7) << 1): eight consecutive rows then spread a
@@ -298,7 +314,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     for (int j = 0; j < 4; ++j) {
       const bool past_k = kbyte + ld_chunk[j & 1] * 16 >= a_pitch;  // chunks past K must read as 0
       load_to_lds(ra, at + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_a[j] + kbyte);
-      if (KIND == kFp8)
+      if (BNK)
         load_to_lds(rb, bt + (wave * 32 + j * 8) * kRow, past_k ? kOutOfRange : voff_b[j] + kbyte);
       if (BKN) {
         // rows k0 + kr; a row past K lies past the end of the buffer by itself
@@ -307,6 +323,14 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
     if (KIND == kS8) s8_load(k0);
+    if (MX) {
+      // the stage's four scale bytes of every tile row, one dword per row: waves 0-3 fetch the
+      // 256 token rows, waves 4-7 the 256 channel rows (64 lanes x 4 bytes land contiguously)
+      const uint32_t blk = (uint32_t)k0 >> 5;
+      const uint32_t v = blk < (uint32_t)nblk ? sc_voff + blk : kOutOfRange;  // K % 128 == 0
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wave < 4 ? rsa : rsb, (lds_ptr_t)(uintptr_t)(lds + 2 * kBufBytes + buf * 2048 + wave * 256),
+                                               4, v, 0, 0, 0);
+    }
   };
 
   floatx16 acc[2][4];
@@ -329,6 +353,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const int row_a = (wm * 128 + l32) * kRow, row_b = kTM * kRow + (wn * 64 + l32) * kRow;
   typedef typename std::conditional<F8, intx8, bf16x8>::type frag_t;
   frag_t fa[4], fb[2];
+  int sa_e[4] = {0, 0, 0, 0}, sb_e[2] = {0, 0};  // kFp8MX: f8e8m0fnu scale of each fragment
   // kFp8KN: per-lane parts of the transposing reads' addresses (see read_frags)
   const int tr_m = (lane & 15) >> 1, tr_par = lane & 1, tr_g = (lane >> 4) & 1;
   const int bkn_base = (32 * kb + tr_m) * 256 + 8 * tr_par;
@@ -337,7 +362,12 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const uint8_t* at = lds + buf * kBufBytes + row_a;
     const uint8_t* bt = lds + buf * kBufBytes + row_b;
     if constexpr (F8) {
-      const int c0 = ((4 * ks + 2 * kb) ^ frag_sw) << 4, c1 = ((4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
+      // The matrix core applies the scale handed in by lanes 0-31 to the first 16 bytes of every
+      // lane of the row and the one from lanes 32-63 to the second 16 (measured; without scales
+      // any split of the 64 k works as long as both operands use the same).  So with block scales
+      // a lane takes 16 bytes of each of the step's two 32-element blocks, otherwise 32 in a run.
+      const int c0 = ((MX ? 4 * ks + kb : 4 * ks + 2 * kb) ^ frag_sw) << 4;
+      const int c1 = ((MX ? 4 * ks + 2 + kb : 4 * ks + 2 * kb + 1) ^ frag_sw) << 4;
       auto rd = [&](const uint8_t* base) {
         const uintx4 x0 = *reinterpret_cast<const uintx4*>(base + c0);
         const uintx4 x1 = *reinterpret_cast<const uintx4*>(base + c1);
@@ -370,6 +400,14 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
 #pragma unroll
       for (int t = 1; t < 4; ++t) fa[t] = rd(at + t * 32 * kRow);
+      if constexpr (MX) {
+        // lanes 0-31 hand in the scale of block 2*ks of the stage, lanes 32-63 that of block 2*ks + 1
+        const uint8_t* sc = lds + 2 * kBufBytes + buf * 2048 + 2 * ks + kb;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) sa_e[t] = sc[(wm * 128 + t * 32 + l32) * 4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) sb_e[t] = sc[1024 + (wn * 64 + t * 32 + l32) * 4];
+      }
     } else {
       const int c = ((2 * ks + kb) ^ frag_sw) << 4;
       fb[0] = *reinterpret_cast<const bf16x8*>(bt + c);
@@ -384,7 +422,10 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        if constexpr (F8)
+        if constexpr (MX)
+          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, sb_e[nt], 0,
+                                                                         sa_e[mt]);
+        else if constexpr (F8)
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, 0, 0, 0);
         else
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
@@ -436,7 +477,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // row leaves as 128 contiguous bytes of bf16 and the accumulators are only ever indexed
   // statically.  The rolled read loop carries the epilogue.
   float alpha = 1.0f;
-  if (F8) alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+  if (F8 && !MX) alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
   float* stage = reinterpret_cast<float*>(lds + wave * 16384);
   const int rd_chunk = lane & 15, rd_row = lane >> 4;  // read side: chunk of 4 channels, row within 4
   const bool n_vec = (p.N & 3) == 0;
@@ -447,7 +488,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   for (int t = 0; t < 4; ++t) {
     const bool ok = n + t < p.N;
     d.sc[t] = alpha;
-    if (F8 && p.b_per_channel) d.sc[t] = alpha * p.b_scale[ok ? n + t : 0];
+    if (F8 && !MX && p.b_per_channel) d.sc[t] = alpha * p.b_scale[ok ? n + t : 0];
     if (KIND == kS8) {
       const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
       d.sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
@@ -479,7 +520,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   }
   d.n_vec = n_vec;
   d.has_bias = p.bias != nullptr;
-  if (F8 && p.a_per_row) {
+  if (F8 && !MX && p.a_per_row) {
     // one scale per token row: all 16 registers of a tile belong to the lane's one token
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
@@ -588,10 +629,17 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   p.b += (size_t)blockIdx.y * p.K * p.N;
   if (p.out) p.out += (size_t)blockIdx.y * total;
   if (p.out8) p.out8 += (size_t)blockIdx.y * total;
-  float sa = p.a_scale[p.a_per_row ? m : 0], sb = p.b_scale[p.b_per_channel ? n : 0];
+  const bool mx = p.a_block_scales != nullptr;
+  float sa = 1.0f, sb = 1.0f;
+  if (!mx) { sa = p.a_scale[p.a_per_row ? m : 0]; sb = p.b_scale[p.b_per_channel ? n : 0]; }
   if (deq_bf16) { sa = round_bf16(sa); sb = round_bf16(sb); }
+  const int nblk = p.K >> 5;
   float acc = 0.0f;
   for (int k = 0; k < p.K; ++k) {
+    if (mx && (k & 31) == 0) {
+      sa = e8m0_to_f32(p.a_block_scales[(size_t)m * nblk + (k >> 5)]);
+      sb = e8m0_to_f32(p.b_block_scales[(size_t)n * nblk + (k >> 5)]);
+    }
     float av = f8e4m3fn_to_f32(p.a[(size_t)m * p.K + k]) * sa;
     float bv = f8e4m3fn_to_f32(b_is_nk ? p.b[(size_t)n * p.K + k] : p.b[(size_t)k * p.N + n]) * sb;
     if (deq_bf16) { av = round_bf16(av); bv = round_bf16(bv); }
@@ -614,7 +662,7 @@ __global__ void store_u32_kernel(uint32_t* dst, uint32_t value) { *dst = value; 
 
 template <int KIND, bool OUT_F8 = false>
 int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
-  constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow;  // 128 KiB
+  constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow + (KIND == kFp8MX ? 4096 : 0);  // 128 KiB (+ scales)
   static bool configured = false;  // per kernel instantiation; benign if two threads race
   if (!configured) {
     hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND, OUT_F8>,
@@ -684,7 +732,19 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     SetLastKernel("fp8_scaled_dot:empty");
     return 0;
   }
-  if (!p.a || !p.b || !p.a_scale || !p.b_scale || !p.out)
+  const bool mx = p.a_block_scales || p.b_block_scales;
+  if (mx) {
+    if (!p.a_block_scales || !p.b_block_scales || p.block != 32 || p.K % 32 != 0)
+      return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT,
+                  "fp8_scaled_dot: block scales come for both operands, one per 32 elements of K");
+    if (p.rhs_contracting_dim != 1)
+      return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: a block-scaled rhs is [N,K]");
+    if (p.a_scale_per_row || p.b_scale_per_channel || p.batch > 1 || p.out_dtype == XLA_FFI_DataType_F8E4M3FN ||
+        p.dequant_type != XLA_FFI_DataType_F32)
+      return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED,
+                  "fp8_scaled_dot: block scales go with an unbatched bf16 result and no other scales");
+  }
+  if (!p.a || !p.b || (!mx && (!p.a_scale || !p.b_scale)) || !p.out)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: null buffer");
   const bool out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
   if (!out_f8 && p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16)
@@ -707,6 +767,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.out8 = out_f8 ? (uint8_t*)p.out : nullptr;
   tp.d_scale = p.d_scale;
   tp.d_divides = p.d_scale_multiplies ? 0 : 1;
+  tp.a_block_scales = (const uint8_t*)p.a_block_scales;
+  tp.b_block_scales = (const uint8_t*)p.b_block_scales;
   tp.amax = out_f8 ? p.amax : nullptr;
   if (tp.amax) {  // the kernels fold their maxima into it with atomics (a kernel, not a memset: graphs)
     hipLaunchKernelGGL(store_u32_kernel, dim3(1), dim3(1), 0, stream, reinterpret_cast<uint32_t*>(tp.amax), 0u);
@@ -760,6 +822,10 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     }
   }
   if (tiled_ok && ((uintptr_t)b_nk % 16 != 0)) tiled_ok = false;
+  // the stage's scales move as one dword per row: K % 128 == 0 and 4-byte aligned scale tensors
+  if (mx && (p.K % 128 != 0 || ((uintptr_t)p.a_block_scales % 4) || ((uintptr_t)p.b_block_scales % 4) ||
+             (double)p.M * (p.K / 32) >= 2147483000.0 || (double)p.N * (p.K / 32) >= 2147483000.0))
+    tiled_ok = false;
   if (force == 2 && !tiled_ok)
     return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
                 "fp8_scaled_dot: the tiled kernel needs K %% 16 == 0, 16-byte aligned operands and, "
@@ -771,7 +837,9 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     TiledParams tt = tp;
     tt.b = b_nk;
     int rc;
-    if (out_f8)
+    if (mx)
+      rc = launch_tiled<kFp8MX>(tt, 1, stream, "fp8_scaled_dot_tiled_mx");
+    else if (out_f8)
       rc = kn_direct ? launch_tiled<kFp8KN, true>(tt, batch, stream, "fp8_scaled_dot_tiled_kn_f8")
                      : launch_tiled<kFp8, true>(tt, batch, stream, "fp8_scaled_dot_tiled_f8");
     else
@@ -784,7 +852,9 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       rc = CheckLaunch("fp8_scaled_dot_exact");
       if (rc) return rc;
     }
-    if (out_f8)
+    if (mx)
+      SetLastKernel("fp8_scaled_dot_tiled_mx");
+    else if (out_f8)
       SetLastKernel(nk ? "fp8_scaled_dot_tiled_f8" : kn_direct ? "fp8_scaled_dot_tiled_kn_f8" : "fp8_scaled_dot_tiled+transpose_f8");
     else
       SetLastKernel(nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose");

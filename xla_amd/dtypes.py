@@ -16,10 +16,11 @@ PRED, S8, S16, S32, S64 = 1, 2, 3, 4, 5
 U8, U16, U32, U64 = 6, 7, 8, 9
 F16, F32, F64, BF16 = 10, 11, 12, 16
 F8E5M2, F8E4M3FN, S4, U4 = 19, 20, 21, 22
+F8E8M0FNU = 33
 
 DTYPE_NAMES = {PRED: "PRED", S8: "S8", S16: "S16", S32: "S32", S64: "S64", U8: "U8", U16: "U16",
                U32: "U32", U64: "U64", F16: "F16", F32: "F32", F64: "F64", BF16: "BF16",
-               F8E5M2: "F8E5M2", F8E4M3FN: "F8E4M3FN", S4: "S4", U4: "U4"}
+               F8E5M2: "F8E5M2", F8E4M3FN: "F8E4M3FN", S4: "S4", U4: "U4", F8E8M0FNU: "F8E8M0FNU"}
 HLO_NAMES = {k: v.lower() for k, v in DTYPE_NAMES.items()}
 FROM_HLO_NAME = {v: k for k, v in HLO_NAMES.items()}
 

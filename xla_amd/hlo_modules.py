@@ -146,6 +146,21 @@ ENTRY %main {{
 """
 
 
+def mxfp8_block_scaled_dot(M=8192, K=8192, N=8192):
+    """MXFP8: f8e4m3fn operands [M,K] and [N,K] with one f8e8m0fnu scale per 32 elements of K, as
+    the "__op$block_scaled_dot" custom call of block_scaling_rewriter.h:48-69 -> bf16 [M,N]."""
+    return f"""HloModule mxfp8_block_scaled_dot
+
+ENTRY %main {{
+  %lhs = f8e4m3fn[{M},{K}] parameter(0)
+  %rhs = f8e4m3fn[{N},{K}] parameter(1)
+  %lhs_scale = f8e8m0fnu[{M},{K // 32}] parameter(2)
+  %rhs_scale = f8e8m0fnu[{N},{K // 32}] parameter(3)
+  ROOT %result = bf16[{M},{N}] custom-call(%lhs, %rhs, %lhs_scale, %rhs_scale), custom_call_target="__op$block_scaled_dot"
+}}
+"""
+
+
 def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False, amax=False):
     """The f32-typed C3 module with an f8e4m3fn result: the GELU value is divided (or multiplied)
     by a per-tensor scale, clamped to +-448 and converted -- the D scaling of

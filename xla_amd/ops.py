@@ -89,7 +89,8 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
                    dequant_type="f32", dot_type="f32", epilogue_type="f32", out=None, scratch="auto",
                    d_scale=None, d_scale_multiplies=False, amax=False, build_only=False):
     """out = epilogue((a*a_scale) . (b*b_scale)); a f8 [M,K]; b f8 [K,N] or [N,K];
-    a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel).
+    a_scale f32 [] or [M] (per row of a), b_scale f32 [] or [N] (per output channel); or both uint8
+    f8e8m0fnu block scales [M,K/32], [N,K/32] with b = [N,K] (MXFP8).
     With d_scale (f32 []) the result is f8e4m3fn codes (uint8): convert(clamp(out / d_scale)),
     or out * d_scale with d_scale_multiplies; with amax=True the call also returns max |out| (f32 [])
     as a second tensor."""
@@ -99,9 +100,11 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
     out_f8 = d_scale is not None
     if out is None:
         out = torch.empty((*lead, m, n), dtype=torch.uint8 if out_f8 else torch.bfloat16, device=a.device)
+    # uint8 scales are f8e8m0fnu block scales [rows, K/32] (MXFP8); float32 ones per tensor / row / channel
+    scale_ty = dtypes.F8E8M0FNU if a_scale.dtype == torch.uint8 else dtypes.F32
     args = [(dtypes.F8E4M3FN, a.data_ptr(), a.shape), (dtypes.F8E4M3FN, b.data_ptr(), b.shape),
-            (dtypes.F32, a_scale.data_ptr(), list(a_scale.shape)),
-            (dtypes.F32, b_scale.data_ptr(), list(b_scale.shape))]
+            (scale_ty, a_scale.data_ptr(), list(a_scale.shape)),
+            (scale_ty, b_scale.data_ptr(), list(b_scale.shape))]
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
     if out_f8:
