@@ -401,12 +401,16 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
 #pragma unroll
       for (int t = 1; t < 4; ++t) fa[t] = rd(at + t * 32 * kRow);
       if constexpr (MX) {
-        // lanes 0-31 hand in the scale of block 2*ks of the stage, lanes 32-63 that of block 2*ks + 1
-        const uint8_t* sc = lds + 2 * kBufBytes + buf * 2048 + 2 * ks + kb;
+        // Lanes 0-31 hand in the scale of block 2*ks of the stage, lanes 32-63 that of block
+        // 2*ks + 1.  A row's four bytes are read once per stage and shifted by the lane's half, so
+        // that byte 0 serves step 0 and byte 2 step 1 (picked by the instruction's op_sel).
+        if (ks == 0) {
+          const uint32_t* sc = reinterpret_cast<const uint32_t*>(lds + 2 * kBufBytes + buf * 2048);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) sa_e[t] = sc[(wm * 128 + t * 32 + l32) * 4];
+          for (int t = 0; t < 4; ++t) sa_e[t] = (int)(sc[wm * 128 + t * 32 + l32] >> (8 * kb));
 #pragma unroll
-        for (int t = 0; t < 2; ++t) sb_e[t] = sc[1024 + (wn * 64 + t * 32 + l32) * 4];
+          for (int t = 0; t < 2; ++t) sb_e[t] = (int)(sc[256 + wn * 64 + t * 32 + l32] >> (8 * kb));
+        }
       }
     } else {
       const int c = ((2 * ks + kb) ^ frag_sw) << 4;
@@ -417,15 +421,19 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       for (int t = 1; t < 4; ++t) fa[t] = *reinterpret_cast<const bf16x8*>(at + t * 32 * kRow + c);
     }
   };
-  auto mfma_all = [&]() {
+  auto mfma_all = [&](int ks) {
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        if constexpr (MX)
-          acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, sb_e[nt], 0,
-                                                                         sa_e[mt]);
-        else if constexpr (F8)
+        if constexpr (MX) {
+          if (ks == 0)
+            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, sb_e[nt],
+                                                                           0, sa_e[mt]);
+          else
+            acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 2, sb_e[nt],
+                                                                           2, sa_e[mt]);
+        } else if constexpr (F8)
           acc[nt][mt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0, 0, 0, 0);
         else
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[nt], fa[mt], acc[nt][mt], 0, 0, 0);
@@ -443,14 +451,14 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
 #pragma unroll
     for (int ks = 0; ks + 1 < NKS; ++ks) {
       read_frags(buf, ks);
-      mfma_all();
+      mfma_all(ks);
     }
     read_frags(buf, NKS - 1);
     if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
-    mfma_all();
+    mfma_all(NKS - 1);
     if (F8) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -464,7 +472,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       read_frags(buf, ks);
-      mfma_all();
+      mfma_all(ks);
     }
   }
   __syncthreads();  // the epilogue reuses the stage buffers
