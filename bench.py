@@ -134,8 +134,8 @@ def main():
     other = []
     if not args.skip_other:
         def entry(name, call, bytes_, flops, bound, dtype=None):
-            # the half-millisecond kernels get a few launches to settle the clocks before timing
-            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=5 if flops else 1)
+            # the half-millisecond kernels get 20 ms of launches to settle the clocks before timing
+            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=40 if flops else 1)
             e = {"workload": name, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
                  "GB/s": round(bytes_ / (ms * 1e-3) / 1e9, 1)}
             e["frac_hbm"] = round(e["GB/s"] / HBM_PEAK_GBS, 4)
@@ -171,6 +171,15 @@ def main():
               ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", rhs_contracting_dim=1,
                                  build_only=True),
               2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+        # the same call with GELU from its closed form (opt-in: the far negative tail then differs
+        # from the reference's own cancellation by more than 2 bf16 ulp of results below 1e-5)
+        ffi.set_option("tiled_epilogue", 1)
+        try:
+            entry("C3 fp8 (rhs [K,N]), opt-in closed-form GELU",
+                  ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", build_only=True),
+                  2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+        finally:
+            ffi.set_option("tiled_epilogue", 0)
         del a8, b8
         # C5: batched s8 per-channel prefill
         a5 = torch.randn((8, 512, 4096), device=dev).to(torch.bfloat16)

@@ -207,8 +207,10 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
 /* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
  * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, 3 tiled),
  * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "fp8_dot_kernel" (1 exact, 2 tiled),
- * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass).  Returns 0, or -1 for
- * an unknown key. */
+ * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1: the
+ * tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
+ * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the
+ * reference's cancellation to 2 bf16 ulp).  Returns 0, or -1 for an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
 
 #ifdef __cplusplus

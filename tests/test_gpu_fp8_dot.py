@@ -325,6 +325,31 @@ def test_f8_result_special_values(oracle):
         assert np.array_equal(got[~nan], ref[~nan]), z
 
 
+@pytest.mark.parametrize("epilogue", ["BIAS_GELU", "SILU"])
+def test_closed_form_activations_opt_in(oracle, epilogue):
+    """Option "tiled_epilogue" = 1: x * sigmoid(.) with the hardware exponential.  Same values as the
+    op-by-op default to 2 bf16 ulp wherever the result is not negligible; in the far negative tail
+    (results below 2e-5 in magnitude) the reference's own cancellation is the larger error, so
+    there only an absolute bound holds."""
+    say("fp8_scaled_dot closed-form " + epilogue)
+    w = workloads.c3_fp8(256, 512, 384)
+    w["epilogue"] = epilogue
+    if "BIAS" not in epilogue:
+        w["bias"] = None
+    strict, _ = run(w)
+    ffi.set_option("tiled_epilogue", 1)
+    try:
+        got, kern = run(w)
+    finally:
+        ffi.set_option("tiled_epilogue", 0)
+    assert kern.startswith("fp8_scaled_dot_tiled")
+    assert not np.array_equal(got, strict)                      # it did take the other path
+    n_floor = check_dot(got, reference(oracle, w), floor_for(w) + 2e-5, kern)
+    big = np.abs(dtypes.bf16_to_f32(strict)) > 1e-3
+    from tests.gpu_util import bf16_ordinal
+    assert np.all(np.abs(bf16_ordinal(got[big]) - bf16_ordinal(strict[big])) <= 2)
+
+
 def test_fp8_one_hot_exact(oracle):
     """A = selector rows of 1.0: outputs are single B values times the scales, exactly."""
     say("fp8_scaled_dot one-hot")

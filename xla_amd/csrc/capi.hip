@@ -21,7 +21,7 @@ struct Option {
 Option g_options[] = {{"dequant_dot_kernel", {0}}, {"dequant_dot_vec", {0}},
                       {"dequant_dot_slices", {0}}, {"dequant_dot_waves", {0}},
                       {"fp8_dot_kernel", {0}},
-                      {"quantize_variant", {0}}, {"fp8_dot_layout", {0}}};
+                      {"quantize_variant", {0}}, {"fp8_dot_layout", {0}}, {"tiled_epilogue", {0}}};
 }  // namespace
 
 int Fail(int code, const char* fmt, ...) {

@@ -60,6 +60,7 @@ struct TiledParams {
   float* amax;           // optional f32 scalar result: max |v| over the f8 result's values
   const uint8_t* a_block_scales;  // kFp8MX: f8e8m0fnu [M, K/32]
   const uint8_t* b_block_scales;  // kFp8MX: f8e8m0fnu [N, K/32]
+  int closed_form_epilogue;       // option "tiled_epilogue" = 1
 };
 
 __device__ __forceinline__ float e8m0_to_f32(uint32_t e) {
@@ -100,13 +101,14 @@ struct DrainArgs {
   int d_mode;
   float dz, drz, dlim;  // the scale, its reciprocal, and 1792 * dz
   bool want_amax;       // f8 result: also the largest |v| of the whole result
+  bool closed_form;     // f32-typed gelu / silu from x * sigmoid(.) instead of the HLO's op sequence
   bool n_vec, has_bias;
   float sc[4], bs[4];
 };
 
 // Returns, for an f8 result, the largest |v| this lane produced as a bit pattern (NaN sorts above
 // every number, which is how maximum propagates it); 0 otherwise.
-template <bool BF16_DOT, bool BF16_OPS, int ACT, bool OUT_F8>
+template <bool BF16_DOT, bool BF16_OPS, int ACT, bool OUT_F8, bool DIRECT = false>
 __device__ __forceinline__ uint32_t drain_rows(const DrainArgs& d) {
   uint32_t amax = 0u;
 #pragma unroll 4
@@ -116,7 +118,8 @@ __device__ __forceinline__ uint32_t drain_rows(const DrainArgs& d) {
     float v[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      v[t] = epilogue_act<BF16_OPS>(epilogue_pre<BF16_DOT, BF16_OPS>(x[t] * d.sc[t], d.bs[t], d.has_bias), ACT);
+      const float pre = epilogue_pre<BF16_DOT, BF16_OPS>(x[t] * d.sc[t], d.bs[t], d.has_bias);
+      v[t] = DIRECT ? epilogue_act_direct(pre, ACT) : epilogue_act<BF16_OPS>(pre, ACT);
     }
     const int m = d.m_base + ml;
     if (OUT_F8) {
@@ -179,6 +182,10 @@ __device__ __forceinline__ uint32_t drain_rows(const DrainArgs& d) {
 
 template <bool BF16_DOT, bool BF16_OPS, bool OUT_F8>
 __device__ __forceinline__ uint32_t drain_act(const DrainArgs& d, int act) {
+  if (!BF16_OPS && d.closed_form) {  // opt-in: f32-typed gelu / silu from their closed forms
+    if (act == kEpiGelu) return drain_rows<BF16_DOT, BF16_OPS, kEpiGelu, OUT_F8, true>(d);
+    if (act == kEpiSilu) return drain_rows<BF16_DOT, BF16_OPS, kEpiSilu, OUT_F8, true>(d);
+  }
   switch (act) {
     case kEpiRelu: return drain_rows<BF16_DOT, BF16_OPS, kEpiRelu, OUT_F8>(d);
     case kEpiGelu: return drain_rows<BF16_DOT, BF16_OPS, kEpiGelu, OUT_F8>(d);
@@ -516,6 +523,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.out = p.out + (size_t)batch * p.M * p.N;
   d.out8 = nullptr;
   d.want_amax = OUT_F8 && p.amax != nullptr;
+  d.closed_form = p.closed_form_epilogue != 0;
   uint32_t amax_bits = 0u;
   d.d_mode = 0;
   d.dz = d.drz = d.dlim = 1.0f;
@@ -711,6 +719,7 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.epilogue = p.epilogue;
   tp.tiles_m = (tp.M + kTM - 1) / kTM;
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
+  tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
   SetLastKernel("dequant_dot_tiled_s8_factored");
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
@@ -792,6 +801,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   const bool deq_bf16 = p.dequant_type == XLA_FFI_DataType_BF16;
   tp.require_pow2_scales = deq_bf16;
+  tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
   // a vector of scales cannot be tested for powers of two in one place: with a bf16-typed
   // multiply it takes the exact kernel
   const bool vector_scales = tp.a_per_row || tp.b_per_channel;
