@@ -94,7 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   constexpr int R = NV * 4 * MT;        // accumulator registers per lane
   constexpr int TN = 16 * NV;           // channels per wave tile
   constexpr int SSZ = SCALE_BF16 ? 2 : 4;
-  __shared__ float lds[WAVES * 16 * 64];  // one 16-register chunk of every wave's tile
+  // the waves' tiles are added through LDS kChunk accumulator registers at a time: 64 KiB where
+  // the split of a chunk over the waves allows it, so a 64-token tile needs four passes
+  constexpr int kChunk = (WAVES == 8 && NV % 4 == 0 && R % 32 == 0) ? 32 : 16;
+  __shared__ float lds[WAVES * kChunk * 64];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, in an SGPR
@@ -285,15 +288,32 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     }
   }
 
-  // ---- add the waves' tiles through LDS, kChunk accumulator registers per pass; in each pass
-  // wave w finishes registers [w*RPW, (w+1)*RPW) of the chunk.  Register index
-  // r = (mt*4 + t)*NV + j; in the accumulator tile, lane (li, kb) register t of instruction j
-  // is channel strip*TN + (4*kb + t)*NV + j, token 16*mt + li.
-  constexpr int kChunk = 16;
+  // ---- add the waves' tiles through LDS; in each pass wave w finishes registers
+  // [w*RPW, (w+1)*RPW) of the chunk.  Register index r = (mt*4 + t)*NV + j; in the accumulator
+  // tile, lane (li, kb) register t of instruction j is channel strip*TN + (4*kb + t)*NV + j,
+  // token 16*mt + li.
   constexpr int RPW = kChunk / WAVES;
+  constexpr int PASSES = R / kChunk;
   static_assert(R % kChunk == 0 && kChunk % WAVES == 0 && NV % RPW == 0, "reduction split");
+  // bias and per-channel scales of every pass are requested now, in one batch, so that no pass
+  // waits for memory between its barriers
+  float bq[PASSES * RPW], fq[PASSES * RPW], res[PASSES * RPW];
 #pragma unroll
-  for (int pass = 0; pass < R / kChunk; ++pass) {
+  for (int pass = 0; pass < PASSES; ++pass) {
+    const int r0 = pass * kChunk + wave * RPW;
+    const int n0 = strip * TN + (4 * kb + (r0 / NV) % 4) * NV + r0 % NV;
+    const bool live = p.slices == 1 && n0 < p.N;
+#pragma unroll
+    for (int u = 0; u < RPW; ++u) {
+      bq[pass * RPW + u] = live && p.bias ? load_scale(p.bias, n0 + u, p.bias_is_bf16) : 0.0f;
+      fq[pass * RPW + u] =
+          MODE == kFactored && live
+              ? load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n0 + u, p.scale_is_bf16)
+              : 1.0f;
+    }
+  }
+#pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
 #pragma unroll
     for (int c = 0; c < kChunk; ++c) {
       const int r = pass * kChunk + c;
@@ -302,35 +322,32 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
       lds[(wave * kChunk + c) * 64 + lane] = v;
     }
     __syncthreads();
-    const int r0 = pass * kChunk + wave * RPW;  // first register this wave finishes
-    const int j0 = r0 % NV, mt = (r0 / NV) / 4, t = (r0 / NV) % 4;
-    const int m = mt * 16 + li;
-    const int n0 = strip * TN + (4 * kb + t) * NV + j0;
-    float sum[RPW];
 #pragma unroll
     for (int u = 0; u < RPW; ++u) {
       float s = 0.0f;
 #pragma unroll
       for (int w2 = 0; w2 < WAVES; ++w2) s = s + lds[(w2 * kChunk + wave * RPW + u) * 64 + lane];
-      sum[u] = s;
+      res[pass * RPW + u] = MODE == kFactored ? s * fq[pass * RPW + u] : s;
     }
-    __syncthreads();
+    if (pass + 1 < PASSES) __syncthreads();
+  }
+  // the epilogue is chosen once for all of the lane's outputs
+  if (p.slices == 1) epilogue_all_dispatch<PASSES * RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
+#pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
+    const int r0 = pass * kChunk + wave * RPW;  // first register this wave finished in the pass
+    const int j0 = r0 % NV, mt = (r0 / NV) / 4, t = (r0 / NV) % 4;
+    const int m = mt * 16 + li;
+    const int n0 = strip * TN + (4 * kb + t) * NV + j0;
     if (m >= p.M || n0 >= p.N) continue;
     if (p.slices > 1) {
       float* dst = p.workspace + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
 #pragma unroll
-      for (int u = 0; u < RPW; ++u) dst[u] = sum[u];
+      for (int u = 0; u < RPW; ++u) dst[u] = res[pass * RPW + u];
     } else {
       uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n0;
 #pragma unroll
-      for (int u = 0; u < RPW; ++u) {
-        float v = sum[u];
-        if (MODE == kFactored)
-          v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n0 + u,
-                             p.scale_is_bf16);
-        const float b = p.bias ? load_scale(p.bias, n0 + u, p.bias_is_bf16) : 0.0f;
-        dst[u] = f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
-      }
+      for (int u = 0; u < RPW; ++u) dst[u] = f32_to_bf16(res[pass * RPW + u]);
     }
   }
 }

@@ -230,5 +230,37 @@ __device__ __forceinline__ float epilogue_dispatch(float acc, float bias, int ep
                   : epilogue_value<false, false>(acc, bias, epi);
 }
 
+// COUNT values through one epilogue, chosen once: straight-line code for the one variant that
+// runs, instead of a COUNT-fold copy of the whole dispatch.
+template <bool BF16_DOT, bool BF16_OPS, int ACT, int COUNT>
+__device__ __forceinline__ void epilogue_all(float* v, const float* bias, bool has_bias) {
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i)
+    v[i] = epilogue_act<BF16_OPS>(epilogue_pre<BF16_DOT, BF16_OPS>(v[i], bias[i], has_bias), ACT);
+}
+
+template <bool BF16_DOT, bool BF16_OPS, int COUNT>
+__device__ __forceinline__ void epilogue_all_act(float* v, const float* bias, int epi) {
+  const bool has_bias = (epi & 1) != 0;
+  switch (epi & ~1) {
+    case kEpiRelu: epilogue_all<BF16_DOT, BF16_OPS, kEpiRelu, COUNT>(v, bias, has_bias); break;
+    case kEpiGelu: epilogue_all<BF16_DOT, BF16_OPS, kEpiGelu, COUNT>(v, bias, has_bias); break;
+    case kEpiSilu: epilogue_all<BF16_DOT, BF16_OPS, kEpiSilu, COUNT>(v, bias, has_bias); break;
+    default: epilogue_all<BF16_DOT, BF16_OPS, 0, COUNT>(v, bias, has_bias); break;
+  }
+}
+
+template <int COUNT>
+__device__ __forceinline__ void epilogue_all_dispatch(float* v, const float* bias, int epi, bool bf16_dot,
+                                                      bool bf16_ops) {
+  if (bf16_ops) {
+    if (bf16_dot) epilogue_all_act<true, true, COUNT>(v, bias, epi);
+    else epilogue_all_act<false, true, COUNT>(v, bias, epi);
+  } else {
+    if (bf16_dot) epilogue_all_act<true, false, COUNT>(v, bias, epi);
+    else epilogue_all_act<false, false, COUNT>(v, bias, epi);
+  }
+}
+
 }  // namespace xla_amd
 #endif  // XLA_AMD_CSRC_DEVICE_NUMERICS_H_
