@@ -25,7 +25,7 @@ def run(x_u16, gamma_u16, eps=1e-6):
     return q.cpu().numpy(), s.cpu().numpy()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("rows,cols", [(64, 8192), (33, 4096), (7, 2048), (5, 1024), (3, 16384), (9, 256)])
 def test_rmsnorm_quantize_bit_exact(oracle, variant, rows, cols):
     say("quantize rmsnorm variant=%d rows=%d cols=%d" % (variant, rows, cols))
