@@ -81,8 +81,11 @@ def main():
     # ---- what a plain copy reaches on this machine (context for every HBM fraction below) ------
     ca = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     cb = torch.empty_like(ca)
-    copy_ms = ev_time(lambda: cb.copy_(ca), 5)
+    st = torch.cuda.current_stream().cuda_stream
+    copy_ms = ev_time(lambda: ffi.debug_stream(cb.data_ptr(), ca.data_ptr(), ca.numel(), st), 10, warm=3)
     copy_gbs = 2 * ca.numel() / (copy_ms * 1e-3) / 1e9
+    read_ms = ev_time(lambda: ffi.debug_stream(None, ca.data_ptr(), ca.numel(), st), 10, warm=3)
+    read_gbs = ca.numel() / (read_ms * 1e-3) / 1e9
     if args.calibrate_copy:
         for _ in range(3):
             cb[:1 << 28].copy_(ca[:1 << 28])     # 256 MiB read + 256 MiB written per launch
@@ -127,8 +130,8 @@ def main():
                 "frac_of_xla_device_file_peak": round(dom["GB/s"] / HBM_PEAK_XLA_GBS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get(dom["workload"]), "launch_ms": dom["ms"],
                 "algorithmic_bytes": dom["bytes"],
-                "device_copy_GB/s": round(copy_gbs, 1),
-                "frac_of_device_copy_rate": round(dom["GB/s"] / copy_gbs, 4)}
+                "device_copy_GB/s": round(copy_gbs, 1), "device_read_GB/s": round(read_gbs, 1),
+                "frac_of_device_read_rate": round(dom["GB/s"] / read_gbs, 4)}
 
     # ---- the other four configurations (informational) -----------------------------------------
     other = []

@@ -213,6 +213,13 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * reference's cancellation to 2 bf16 ulp).  Returns 0, or -1 for an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
 
+/* Measurement aid for benchmarks (no counterpart in the reference): streams `bytes` (a multiple of 16,
+ * buffers 16-byte aligned) from `src` on `stream` -- copied to `dst`, or only read when `dst` is
+ * null -- with the access shape that reaches the highest HBM rate on MI355X, so that a benchmark can
+ * print what a plain stream achieves on the same machine next to a kernel's own rate.  Returns 0 or
+ * an XLA_FFI_Error_Code. */
+XLA_AMD_EXPORT int xla_amd_debug_stream(void* dst, const void* src, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

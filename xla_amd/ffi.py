@@ -24,7 +24,7 @@ EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
     "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_fp8_scaled_dot",
     "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
     "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
-    "xla_amd_debug_set_option"]
+    "xla_amd_debug_set_option", "xla_amd_debug_stream"]
 
 STAGE_INSTANTIATE, STAGE_PREPARE, STAGE_INITIALIZE, STAGE_EXECUTE, STAGE_RECORD = range(5)
 ATTR_ARRAY, ATTR_DICTIONARY, ATTR_SCALAR, ATTR_STRING = 1, 2, 3, 4
@@ -248,6 +248,7 @@ def library():
         L.xla_amd_last_error.restype = C.c_char_p
         L.xla_amd_last_kernel.restype = C.c_char_p
         L.xla_amd_debug_set_option.argtypes = [C.c_char_p, C.c_int]
+        L.xla_amd_debug_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
         L.xla_amd_fp8_scaled_dot_workspace_bytes.restype = C.c_size_t
@@ -427,6 +428,13 @@ def query_metadata(target, host):
 
 def last_kernel():
     return library().xla_amd_last_kernel().decode()
+
+
+def debug_stream(dst_ptr, src_ptr, nbytes, stream):
+    """Launches the library's yardstick stream kernel (copy, or read only when dst_ptr is 0/None)."""
+    rc = library().xla_amd_debug_stream(dst_ptr or None, src_ptr, nbytes, stream)
+    if rc != 0:
+        raise RuntimeError(library().xla_amd_last_error().decode())
 
 
 def set_option(key, value):
