@@ -238,6 +238,36 @@ def test_batched_decode(oracle):
     compare(oracle, w, got, "batched decode")
 
 
+@pytest.mark.parametrize("M,K,N", [(200, 1024, 512), (65, 256, 264), (128, 2048, 256)])
+def test_s4_group_scales_more_than_64_tokens(oracle, M, K, N):
+    """Prefill-sized M on s4 weights with grouped scales: the decode kernel once per 64 tokens,
+    and the result equals, bit for bit, separate calls on the same token rows."""
+    say("dequant_dot s4 group chunked M=%d K=%d N=%d" % (M, K, N))
+    w = workloads.c2_s4_group(M=M, K=K, N=N)
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s4") and kern.endswith(":x64"), kern
+    compare(oracle, w, got, "s4 chunked M=%d" % M)
+    for m0 in range(0, M, 64):
+        part = dict(w, lhs=np.ascontiguousarray(w["lhs"][m0:m0 + 64]))
+        alone, _ = run_dot(part)
+        assert np.array_equal(alone, got[m0:m0 + 64]), "rows %d.. differ from a call of their own" % m0
+
+
+def test_batched_grouped_s8_more_than_64_tokens(oracle):
+    """Batched s8 weights with per-group scales (not the tiled kernel's per-channel case), 70 tokens."""
+    say("dequant_dot batched grouped s8 chunked")
+    rng = np.random.default_rng(77)
+    B, M, K, N, g = 2, 70, 256, 128, 64
+    w = dict(lhs=dtypes.f32_to_bf16(rng.standard_normal((B, M, K)).astype(np.float32)),
+             weights=rng.integers(-127, 128, size=(B, K, N)).astype(np.int8),
+             scales=dtypes.f32_to_bf16(rng.uniform(1e-3, 1e-2, size=(B, K // g, N)).astype(np.float32)),
+             bias=None, weight_dtype="s8", weight_shape=(B, K, N), group=g, dequant_type="bf16",
+             epilogue="DEFAULT")
+    got, kern = run_dot(w)
+    assert kern.startswith("dequant_dot_decode_s8") and kern.endswith(":x64"), kern
+    compare(oracle, w, got, "batched grouped s8 chunked")
+
+
 def test_c5_full_size_sampled_blocks(oracle):
     """Configuration 5 at full size; the oracle evaluates random (expert, row block, column block)
     sub-problems of the same inputs."""

@@ -28,6 +28,7 @@
 //    multiplies the f32 sum once.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include "device_numerics.h"
 #include "launch.h"
@@ -462,6 +463,10 @@ static int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int stri
 // What xla_amd_dequant_dot_workspace_bytes reports: the scratch the launch below will use for
 // this shape (the narrowest strips give the most slices), or what a forced slice count needs.
 size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4) {
+  if (M > 64 && s4) {  // runs as one batch-1 launch per 64 tokens, all sharing the scratch
+    M = 64;
+    batch = 1;
+  }
   if (M <= 0 || M > 64 || K < 32 || N <= 0 || batch <= 0) return 0;
   const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
   int vec = s4 ? 4 : (mt == 4 ? 4 : 8);
@@ -531,9 +536,10 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
 
-  if (force != 1 && force != 3 && aligned && mode_ok && p.M <= 64 && p.K >= 32) {
-    // VEC bytes per lane per row -> NV channels per lane; needs N % NV == 0 and 16-byte rows
-    const int mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+  // Strip layout of the decode kernels for M tokens, and whether this shape fits them.
+  // VEC bytes per lane per row -> NV channels per lane; needs N % NV == 0 and 16-byte rows
+  auto decode_shape = [&](int64_t M, int* mt_out, int* vec_out, int* nv_out) {
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
     // Narrow strips (4 bytes of s4 = 8 channels, 8 bytes of s8 per lane) measured fastest on
     // MI355X: the loop is bound by the dequantising VALU work, not by load width, and narrow
     // strips give more workgroups to spread over the 256 CUs.
@@ -543,10 +549,46 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // buffer offsets are 32-bit: keep every operand (plus one loop overrun) below 2 GiB
     const bool fits32 = (double)p.K * row_bytes + 1024.0 * row_bytes < 2147483648.0 &&
-                        (double)p.M * p.K * 2 < 2147483648.0 &&
+                        (double)M * p.K * 2 < 2147483648.0 &&
                         (double)(p.K / p.group) * p.N * 4 < 2147483648.0;
-    const bool shape_ok = p.N % nv == 0 && row_bytes % vec == 0 && nv * mt <= 32 &&
-                          (vec == 4 || vec == 8 || vec == 16) && fits32;
+    *mt_out = mt; *vec_out = vec; *nv_out = nv;
+    return p.N % nv == 0 && row_bytes % vec == 0 && nv * mt <= 32 && (vec == 4 || vec == 8 || vec == 16) && fits32;
+  };
+
+  // More than 64 tokens on weights the tiled kernel does not take (s4, grouped scales): the
+  // decode kernel runs once per 64 tokens (and per batch).  Every token row is computed exactly as
+  // in a call of its own, so the chunks compose bit for bit; each pass streams the weights again,
+  // which at 8192 x 28672 s4 still reaches 0.55 PFLOP/s against 2-3 TFLOP/s of the generic kernel.
+  int mt64, vec64, nv64;
+  if (force != 1 && force != 3 && aligned && mode_ok && p.M > 64 && p.K >= 32 && p.N % 2 == 0 &&
+      decode_shape(64, &mt64, &vec64, &nv64)) {
+    const size_t wbytes = (size_t)p.K * p.N * (s4 ? 1 : 2) / 2;
+    const size_t ssz = p.scale_dtype == XLA_FFI_DataType_BF16 ? 2 : 4;
+    const size_t sbytes = p.scale_batch == p.batch && p.batch > 1 ? (size_t)(p.K / p.group) * p.N * ssz : 0;
+    XlaAmdDequantDot sub = p;
+    sub.batch = 1;
+    sub.scale_batch = 1;
+    char name[128] = "";
+    for (int64_t b = 0; b < p.batch; ++b) {
+      sub.weights = (const char*)p.weights + b * wbytes;
+      sub.scales = (const char*)p.scales + b * sbytes;
+      for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
+        sub.M = p.M - m0 < 64 ? p.M - m0 : 64;
+        sub.lhs = (const uint16_t*)p.lhs + ((size_t)b * p.M + m0) * p.K;
+        sub.out = (uint16_t*)p.out + ((size_t)b * p.M + m0) * p.N;
+        const int rc = LaunchDequantDot(sub, stream);
+        if (rc) return rc;
+        if (!name[0]) snprintf(name, sizeof(name), "%s:x64", xla_amd_last_kernel());
+      }
+    }
+    SetLastKernel(name);
+    return 0;
+  }
+
+  if (force != 1 && force != 3 && aligned && mode_ok && p.M <= 64 && p.K >= 32) {
+    int mt, vec, nv;
+    const bool shape_ok = decode_shape(p.M, &mt, &vec, &nv);
+    const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     if (shape_ok) {
       dp.strips = (int)((p.N + 16 * nv - 1) / (16 * nv));
       // Up to 16 tokens, when the strips alone give (nearly) a workgroup per CU, the workgroup is
