@@ -38,9 +38,11 @@ def test_c1_module():
     check_dot(host_bf16(out), ref, fl, "C1 module")
 
 
-def test_c2_module():
-    say("module C2")
-    M, K, N = 8, 1024, 512
+@pytest.mark.parametrize("M", [8, 130])
+def test_c2_module(M):
+    """M = 130: a prefill-sized token count on the s4 weights (one decode launch per 64 tokens)."""
+    say("module C2 M=%d" % M)
+    K, N = 1024, 512
     w = workloads.c2_s4_group(M, K, N)
     text = hm.c2_s4_group(M, K, N)
     out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_u8(w["weights_packed"]),
