@@ -238,12 +238,56 @@ def test_batched_decode(oracle):
     compare(oracle, w, got, "batched decode")
 
 
-@pytest.mark.parametrize("M,K,N", [(200, 1024, 512), (65, 256, 264), (128, 2048, 256)])
-def test_s4_group_scales_more_than_64_tokens(oracle, M, K, N):
-    """Prefill-sized M on s4 weights with grouped scales: the decode kernel once per 64 tokens,
-    and the result equals, bit for bit, separate calls on the same token rows."""
+@pytest.mark.parametrize("M,K,N,group", [(200, 1024, 512, 128), (65, 264, 264, 8), (300, 2048, 1000, 64),
+                                         (512, 512, 256, 512), (130, 1000, 72, 8)])
+def test_s4_group_scales_tiled(oracle, M, K, N, group):
+    """Prefill-sized M on s4 weights with bf16 scales per power-of-two group: the tiled MFMA kernel,
+    weights dequantised (one rounding each) on the way into LDS."""
+    say("dequant_dot s4 tiled M=%d K=%d N=%d group=%d" % (M, K, N, group))
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=group)
+    got, kern = run_dot(w, force_kernel=3)   # at these sizes the cost model would pick the decode passes
+    assert kern == "dequant_dot_tiled_s4_rounded", kern
+    compare(oracle, w, got, "s4 tiled M=%d" % M)
+
+
+def test_s4_more_than_64_tokens_picks_the_cheaper_kernel():
+    """8192 x 28672 s4 weights: decode passes up to a few hundred tokens, the tiled kernel beyond."""
+    say("dequant_dot s4 kernel choice at the C2 weight shape")
+    K, N = 8192, 28672
+    dev = torch.device("cuda:0")
+    wt = torch.zeros(K * N // 2, dtype=torch.uint8, device=dev)
+    sc = torch.ones((K // 128, N), dtype=torch.bfloat16, device=dev)
+    for M, want in ((128, "dequant_dot_decode_s4_v4_m64_rounded:x64"), (1024, "dequant_dot_tiled_s4_rounded")):
+        lhs = torch.zeros((M, K), dtype=torch.bfloat16, device=dev)
+        out = ops.dequant_dot(lhs, wt, sc, None, weight_dtype="s4", weight_shape=(K, N), epilogue="DEFAULT",
+                              dequant_type="bf16")
+        torch.cuda.synchronize()
+        assert ffi.last_kernel() == want, (M, ffi.last_kernel())
+        assert not bool(out.any())
+
+
+def test_s4_tiled_dequantised_weights_bit_exact(oracle):
+    """One-hot activations pick single dequantised weights out of the tiled kernel: bf16(w * s) exactly."""
+    say("dequant_dot s4 tiled one-hot")
+    M, K, N, g = 128, 128, 256, 32
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=g)
+    lhs = np.zeros((M, K), np.float32)
+    lhs[np.arange(M), np.arange(M) % K] = 1.0
+    w = dict(w, lhs=dtypes.f32_to_bf16(lhs), bias=None, epilogue="DEFAULT")
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_s4_rounded", kern
+    sc = np.repeat(dtypes.bf16_to_f32(w["scales"]), g, axis=0)
+    want = dtypes.f32_to_bf16((w["weights"].astype(np.float32) * sc).astype(np.float32))[np.arange(M) % K]
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("M,K,N,group", [(200, 768, 512, 96), (65, 480, 264, 24)])
+def test_s4_group_scales_more_than_64_tokens(oracle, M, K, N, group):
+    """Prefill-sized M on s4 weights the tiled kernel does not take (groups that are no power of
+    two): the decode kernel once per 64 tokens, and the result equals, bit for bit, separate calls
+    on the same token rows."""
     say("dequant_dot s4 group chunked M=%d K=%d N=%d" % (M, K, N))
-    w = workloads.c2_s4_group(M=M, K=K, N=N)
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=group)
     got, kern = run_dot(w)
     assert kern.startswith("dequant_dot_decode_s4") and kern.endswith(":x64"), kern
     compare(oracle, w, got, "s4 chunked M=%d" % M)

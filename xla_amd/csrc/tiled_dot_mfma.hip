@@ -2,6 +2,8 @@
 //
 //   kFp8 : out[m,n] = epi( a_scale*b_scale * sum_k A8[m,k] * B8[n,k] )   f8e4m3fn x f8e4m3fn
 //   kS8  : out[b,m,n] = epi( scale[b,n] * sum_k A[b,m,k] * W[b,k,n] )    bf16 x s8 (per channel)
+//   kS4  : out[b,m,n] = epi( sum_k A[b,m,k] * bf16(W[b,k,n] * scale[b,k/g,n]) )   bf16 x s4, bf16 scales per
+//          group of g rows, every dequantised weight rounded once (the bf16-typed multiply)
 //
 // A workgroup of 8 waves (2x4, two per SIMD) owns a 256x256 output tile, each wave a 128x64
 // part held in 128 accumulator registers, and walks K in stages of 128 bytes per activation
@@ -35,7 +37,7 @@ namespace {
 
 // kFp8KN: fp8 with the weights given [K,N]; kFp8MX: fp8 [M,K] x [N,K] with one f8e8m0fnu scale per
 // 32 elements of K on both operands (MXFP8), multiplied in by the matrix cores themselves
-enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3 };
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4 };
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
@@ -45,7 +47,8 @@ struct TiledParams {
   const uint8_t* b;     // kFp8: f8 [N,K]; kFp8KN: f8 [K,N]; kS8: s8 [batch,K,N]
   const float* a_scale; // kFp8: one value, or M (a_per_row)
   const float* b_scale; // kFp8: one value, or N (b_per_channel)
-  const void* scales;   // kS8: [scale_batch, N]
+  const void* scales;   // kS8: [scale_batch, N]; kS4: bf16 [scale_batch, K/group, N]
+  int group_shift;      // kS4: log2 of the scale group (rows of K)
   const void* bias;
   uint16_t* out;        // [batch, M, N]
   int M, K, N;
@@ -207,7 +210,8 @@ __device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, 
 
 template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
-  constexpr bool F8 = KIND != kS8;       // both operands f8e4m3fn
+  constexpr bool WQ = KIND == kS8 || KIND == kS4;  // integer weights [K,N], dequantised on the way into LDS
+  constexpr bool F8 = !WQ;               // both operands f8e4m3fn
   constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
   constexpr bool MX = KIND == kFp8MX;    // block scales ride along with every stage
   constexpr bool BNK = KIND == kFp8 || MX;  // f8 weights [N,K]: staged like the activations
@@ -253,8 +257,8 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const uint32_t a_pitch = (uint32_t)p.K * ESZ;
   const __amdgpu_buffer_rsrc_t ra =
       tile_rsrc(p.a + (size_t)batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
-  const __amdgpu_buffer_rsrc_t rb =
-      tile_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);  // bytes, either layout
+  const uint32_t b_bytes = KIND == kS4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N;
+  const __amdgpu_buffer_rsrc_t rb = tile_rsrc(p.b + (size_t)batch * b_bytes, b_bytes);  // bytes, either layout
 
   // kFp8MX: scales [rows, K/32]; lane l of wave w owns tile row (w & 3) * 64 + l of its operand
   const int nblk = p.K >> 5;
@@ -313,6 +317,63 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     }
   };
 
+  // ---- s4 weights: two per byte along N, so a dword is 8 channels of one row.  Lane l of wave w
+  // takes block (l & 7) of 8 rows of octet (w & 3) * 8 + (l >> 3) -- the 8 lanes that share an
+  // octet write one whole 128-byte LDS row per channel -- and waves 0-3 / 4-7 dequantise nibble
+  // pairs (0,4),(1,5) / (2,6),(3,7) of the same dwords.  The group's 8 bf16 scales ride along.
+  uintx4 s4_scales = {0u, 0u, 0u, 0u};
+  const int q_kblk = lane & 7, q_oct = (wave & 3) * 8 + (lane >> 3), q_half = wave >> 2;
+  const uint32_t s4_pitch = (uint32_t)p.N >> 1;
+  const __amdgpu_buffer_rsrc_t rsc4 =
+      tile_rsrc(KIND == kS4 ? (const uint8_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * p.N * 2
+                            : p.a,
+                KIND == kS4 ? (uint32_t)(p.K >> p.group_shift) * (uint32_t)p.N * 2u : 0u);
+  auto s4_load = [&](int k0) {
+    const uint32_t col = (uint32_t)(n0 + q_oct * 8);
+    const uint32_t kfirst = (uint32_t)(k0 + q_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
+    const bool live = col < (uint32_t)p.N && kfirst < (uint32_t)p.K;  // N % 8 == 0
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, live ? (kfirst + r) * s4_pitch + (col >> 1) : kOutOfRange, 0, 0);
+    s4_scales = __builtin_amdgcn_raw_buffer_load_b128(
+        rsc4, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) * 2u : kOutOfRange, 0, 0);
+  };
+  auto s4_store = [&](uint8_t* bt) {
+    typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl) {
+      // nibbles (e, e + 4), e = 2 * q_half + sl, as the f16 pair (1024 + u, 1024 + u) or, for odd
+      // e, (1024 + 16 u, 1024 + 16 u), u = w + 8: see dequant_dot_decode.hip
+      halfx2 pr[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const uint32_t x = q_half ? wreg[r] >> 8 : wreg[r];
+        pr[r] = __builtin_bit_cast(halfx2, sl ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a)
+                                              : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+      }
+#pragma unroll
+      for (int hi = 0; hi < 2; ++hi) {
+        const int e_lo = sl + 4 * hi;  // nibble index when q_half == 0; + 2 otherwise
+        const uint32_t sw0 = s4_scales[(e_lo) >> 1], sw1 = s4_scales[(e_lo + 2) >> 1];
+        const uint32_t sw = q_half ? sw1 : sw0;  // e and e + 2 have the same parity: same half of the dword
+        const float v = (e_lo & 1) ? bf16hi_to_f32(sw) : bf16lo_to_f32(sw);
+        const float sj = sl ? v * 0.0625f : v;
+        const float cj = sl ? v * -72.0f : v * -1032.0f;
+        float f[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][hi], sj, cj);
+        const uintx4 o = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                          pack_bf16x2(f[6], f[7])};
+        const int n = q_oct * 8 + e_lo + 2 * q_half;
+        *reinterpret_cast<uintx4*>(bt + n * kRow + ((q_kblk ^ ((n >> 1) & 7)) << 4)) = o;
+      }
+    }
+  };
+  auto wq_store = [&](uint8_t* bt) {
+    if constexpr (KIND == kS8) s8_store(bt);
+    if constexpr (KIND == kS4) s4_store(bt);
+  };
+
   auto issue_loads = [&](int buf, int k0) {
     uint8_t* at = lds + buf * kBufBytes;
     uint8_t* bt = at + kTM * kRow;
@@ -330,6 +391,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
     if (KIND == kS8) s8_load(k0);
+    if (KIND == kS4) s4_load(k0);
     if (MX) {
       // the stage's four scale bytes of every tile row, one dword per row: waves 0-3 fetch the
       // 256 token rows, waves 4-7 the 256 channel rows (64 lanes x 4 bytes land contiguously)
@@ -449,7 +511,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
 
   const int stages = (p.K + KS - 1) / KS;
   issue_loads(0, 0);
-  if (KIND == kS8) s8_store(lds + kTM * kRow);
+  if (WQ) wq_store(lds + kTM * kRow);
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
   issue_loads(1, KS);  // past K: lands as zeros, never read
@@ -461,7 +523,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       mfma_all(ks);
     }
     read_frags(buf, NKS - 1);
-    if (KIND == kS8) s8_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+    if (WQ) wq_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
@@ -698,9 +760,26 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
 // (the caller then falls back), 0 on success, or an error code.
 int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
-  if (p.weight_dtype != XLA_FFI_DataType_S8 || p.group != p.K ||
-      p.dequant_type != XLA_FFI_DataType_F32)
-    return -1;
+  // s4 with bf16 scales per power-of-two group of rows and a bf16-typed dequantise multiply, or
+  // s8 with per-channel scales and an f32-typed one
+  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4 && p.dequant_type == XLA_FFI_DataType_BF16 &&
+                  p.scale_dtype == XLA_FFI_DataType_BF16 && p.group >= 8 && (p.group & (p.group - 1)) == 0 &&
+                  p.N % 8 == 0 && ((uintptr_t)p.scales % 16) == 0 &&
+                  (double)(p.K / p.group) * p.N * 2 < 2147483000.0;
+  const bool s8 = p.weight_dtype == XLA_FFI_DataType_S8 && p.group == p.K && p.dequant_type == XLA_FFI_DataType_F32;
+  if (!s4 && !s8) return -1;
+  if (s4 && GetOption("dequant_dot_kernel") != 3) {
+    // The decode kernel, run once per 64 tokens, streams and dequantises the weights on every
+    // pass but fills the machine at any M; the tiled kernel dequantises once per 256 tokens but
+    // needs 256 tiles per round.  Estimates in microseconds fitted on MI355X (8192 x 28672:
+    // 53 per decode pass, 316 per round of tiles); the cheaper one runs.
+    const double passes = (double)p.batch * (double)((p.M + 63) / 64);
+    const double decode_us = passes * (6.0 + (double)p.K * (double)p.N * 2.0e-7);
+    const double tiles = (double)p.batch * (double)((p.M + kTM - 1) / kTM) * (double)((p.N + kTN - 1) / kTN);
+    const double rounds = (double)(int64_t)((tiles + 255.0) / 256.0);
+    const double tiled_us = rounds * (10.0 + (double)p.K * 0.0374);
+    if (decode_us <= tiled_us) return -1;
+  }
   if (p.K % 8 != 0 || p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 4)) return -1;
   // 32-bit buffer offsets per batch
   if ((double)p.M * p.K * 2 >= 2147483000.0 || (double)p.K * p.N >= 2147483000.0) return -1;
@@ -720,6 +799,11 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.tiles_m = (tp.M + kTM - 1) / kTM;
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
+  if (s4) {
+    tp.group_shift = __builtin_ctzll((unsigned long long)p.group);
+    SetLastKernel("dequant_dot_tiled_s4_rounded");
+    return launch_tiled<kS4>(tp, (int)p.batch, stream, "dequant_dot_tiled_s4");
+  }
   SetLastKernel("dequant_dot_tiled_s8_factored");
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
