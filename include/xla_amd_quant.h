@@ -207,7 +207,8 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
 /* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
  * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, also in passes of 64
  * tokens, 3 tiled whenever it covers the shape),
- * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "fp8_dot_kernel" (1 exact, 2 tiled),
+ * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "dequant_dot_skew" (shares of K of a SIMD's
+ * waves, oldest first, as decimal digits), "fp8_dot_kernel" (1 exact, 2 tiled),
  * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1: the
  * tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the

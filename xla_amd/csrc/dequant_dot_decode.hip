@@ -49,6 +49,9 @@ struct DecodeParams {
   int scale_is_bf16, bias_is_bf16, scale_batched;
   int bf16_dot, bf16_ops, epilogue;
   int strips, slices, rows_per_slice;  // rows_per_slice: multiple of 32 * WAVES
+  // Rows of a slice that a wave of age class c (wave index / 4) takes, multiples of 64: the
+  // waves w, w+4, w+8, ... share a SIMD, which serves the oldest wave first.
+  int class_rows[4];
 };
 
 __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
@@ -148,8 +151,13 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int rows_per_wave = p.rows_per_slice / WAVES;  // multiple of 64
-  const int k_begin = slice * p.rows_per_slice + wave * rows_per_wave;
+  // the slice is cut into four blocks, one per SIMD; inside a block the age classes follow each other
+  const int cls = wave >> 2;
+  int k_begin = slice * p.rows_per_slice + (wave & 3) * (p.rows_per_slice >> 2);
+#pragma unroll
+  for (int c = 0; c < WAVES / 4; ++c)
+    if (c < cls) k_begin += p.class_rows[c];
+  const int rows_per_wave = p.class_rows[cls];
   const int k_stop = k_begin + rows_per_wave;           // may run past K: those rows load zeros
 
   // ---- software pipeline: everything step k0+32 needs from memory -- weights, activations
@@ -438,6 +446,35 @@ static int RowsPerSlice(int K, int slices, int waves) {
   return (per + unit - 1) / unit * unit;
 }
 
+// Splits a SIMD's quarter of a slice between its waves' age classes in proportion to weights
+// (option "dequant_dot_skew": four decimal digits, oldest class first; 0 = the default), in units
+// of 64 rows; the youngest class takes what rounding leaves.
+static void ClassRows(int rows_per_slice, int waves, int* out) {
+  const int classes = waves / 4;
+  const int units = rows_per_slice / 4 / 64;  // 64-row units per SIMD block, a multiple of `classes`
+  // Defaults from a sweep on 8192 x 28672 s4: with equal shares the four waves of a SIMD left the
+  // main loop at 11.7, 15.8, 20.2 and 24.5 us (in-kernel clock), the last one running alone at a
+  // little over half the SIMD's rate; 4:3:2:1 brings 1 token from 28.3 to 25.9 us, 3:2 for two
+  // classes 32 tokens from 38.0 to 36.8 (64 tokens: no change, one wave already fills the SIMD).
+  int w[4] = {1, 1, 1, 1};
+  if (classes == 4) { w[0] = 4; w[1] = 3; w[2] = 2; w[3] = 1; }
+  if (classes == 2) { w[0] = 3; w[1] = 2; }
+  if (int v = GetOption("dequant_dot_skew")) {
+    w[0] = v / 1000 % 10; w[1] = v / 100 % 10; w[2] = v / 10 % 10; w[3] = v % 10;
+    if (classes == 2) { w[0] = v / 10 % 10; w[1] = v % 10; }
+  }
+  int total = 0;
+  for (int c = 0; c < classes; ++c) total += w[c] > 0 ? w[c] : (w[c] = 1);
+  int left = units;
+  for (int c = 0; c < 4; ++c) out[c] = 0;
+  for (int c = 0; c < classes; ++c) {
+    int u = c + 1 == classes ? left : (units * w[c] + total / 2) / total;
+    if (u > left) u = left;
+    out[c] = u * 64;
+    left -= u;
+  }
+}
+
 size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices) {
   return slices > 1 ? (size_t)batch * slices * M * N * sizeof(float) : 0;
 }
@@ -605,6 +642,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
         slices = 1;
       dp.slices = slices;
       dp.rows_per_slice = RowsPerSlice(dp.K, slices, waves);
+      ClassRows(dp.rows_per_slice, waves, dp.class_rows);
       if (waves == 16) {  // one 16-token tile, 8 channels per lane: the whole CU as one workgroup
         if (s4 && mode == kRounded)
           return launch_decode<4, 4, 1, 16, kRounded>(dp, (int)p.batch, stream, "dequant_dot_decode_s4_v4_m16_w16_rounded");
