@@ -149,6 +149,13 @@ def main():
             e["bound"] = bound
             other.append(e)
 
+        # C2's weights at a prefill-sized token count (not a BASELINE configuration: the tiled s4 kernel)
+        lhs2k = torch.randn((2048, K2), device=dev).to(torch.bfloat16)
+        entry("C2 weights, 2048 tokens (s4 prefill)",
+              ops.dequant_dot(lhs2k, w_packed, scales, bias, weight_dtype="s4", weight_shape=(K2, N2),
+                              epilogue="BIAS_SILU", dequant_type="bf16", build_only=True),
+              c2_bytes(2048), 2 * 2048 * K2 * N2, "mfma", "bf16")
+        del lhs2k
         # C1: s8 per-channel decode
         a = torch.randn((16, 4096), device=dev).to(torch.bfloat16)
         w8 = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
