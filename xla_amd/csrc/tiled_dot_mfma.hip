@@ -318,11 +318,13 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   };
 
   // ---- s4 weights: two per byte along N, so a dword is 8 channels of one row.  Lane l of wave w
-  // takes block (l & 7) of 8 rows of octet (w & 3) * 8 + (l >> 3) -- the 8 lanes that share an
-  // octet write one whole 128-byte LDS row per channel -- and waves 0-3 / 4-7 dequantise nibble
-  // pairs (0,4),(1,5) / (2,6),(3,7) of the same dwords.  The group's 8 bf16 scales ride along.
+  // takes block l >> 3 of 8 rows of octet (w & 3) * 8 + (l & 7): the four lanes of a quad read 16
+  // contiguous bytes of one row (with the block index in the low lane bits instead, a quad touched
+  // four rows and the kernel was 11 % slower), and the 8 lanes of a row block write 8 different
+  // 16-byte chunks.  Waves 0-3 / 4-7 dequantise nibble pairs (0,4),(1,5) / (2,6),(3,7) of the same
+  // dwords.  The group's 8 bf16 scales ride along.
   uintx4 s4_scales = {0u, 0u, 0u, 0u};
-  const int q_kblk = lane & 7, q_oct = (wave & 3) * 8 + (lane >> 3), q_half = wave >> 2;
+  const int q_kblk = lane >> 3, q_oct = (wave & 3) * 8 + (lane & 7), q_half = wave >> 2;
   const uint32_t s4_pitch = (uint32_t)p.N >> 1;
   const __amdgpu_buffer_rsrc_t rsc4 =
       tile_rsrc(KIND == kS4 ? (const uint8_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * p.N * 2
@@ -772,12 +774,12 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
     // The decode kernel, run once per 64 tokens, streams and dequantises the weights on every
     // pass but fills the machine at any M; the tiled kernel dequantises once per 256 tokens but
     // needs 256 tiles per round.  Estimates in microseconds fitted on MI355X (8192 x 28672:
-    // 53 per decode pass, 316 per round of tiles); the cheaper one runs.
+    // 53 per decode pass, 287 per round of tiles); the cheaper one runs.
     const double passes = (double)p.batch * (double)((p.M + 63) / 64);
     const double decode_us = passes * (6.0 + (double)p.K * (double)p.N * 2.0e-7);
     const double tiles = (double)p.batch * (double)((p.M + kTM - 1) / kTM) * (double)((p.N + kTN - 1) / kTN);
     const double rounds = (double)(int64_t)((tiles + 255.0) / 256.0);
-    const double tiled_us = rounds * (10.0 + (double)p.K * 0.0374);
+    const double tiled_us = rounds * (10.0 + (double)p.K * 0.0338);
     if (decode_us <= tiled_us) return -1;
   }
   if (p.K % 8 != 0 || p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 4)) return -1;
