@@ -84,7 +84,7 @@ def compare(oracle, w, got, what):
 
 # ---- decode kernels (M <= 64) --------------------------------------------------------------
 
-@pytest.mark.parametrize("M", [1, 8, 32, 64])
+@pytest.mark.parametrize("M", [1, 8, 32, 40, 48, 64])
 def test_c2_shape_reduced_n(oracle, M):
     """Configuration 2 with full K and group 128, N cut to 1024 so the oracle stays fast."""
     say("dequant_dot C2 s4 M=%d K=8192 N=1024" % M)

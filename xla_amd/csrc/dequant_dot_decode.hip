@@ -505,8 +505,8 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
     batch = 1;
   }
   if (M <= 0 || M > 64 || K < 32 || N <= 0 || batch <= 0) return 0;
-  const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-  int vec = s4 ? 4 : (mt == 4 ? 4 : 8);
+  const int mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 48 ? 3 : 4;
+  int vec = s4 ? 4 : (mt >= 3 ? 4 : 8);
   if (int v = GetOption("dequant_dot_vec")) vec = v;
   const int nv = vec * (s4 ? 2 : 1);
   const int64_t row_bytes = N * (s4 ? 1 : 2) / 2;
@@ -576,11 +576,11 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
   // Strip layout of the decode kernels for M tokens, and whether this shape fits them.
   // VEC bytes per lane per row -> NV channels per lane; needs N % NV == 0 and 16-byte rows
   auto decode_shape = [&](int64_t M, int* mt_out, int* vec_out, int* nv_out) {
-    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 48 ? 3 : 4;  // 16-token tiles
     // Narrow strips (4 bytes of s4 = 8 channels, 8 bytes of s8 per lane) measured fastest on
     // MI355X: the loop is bound by the dequantising VALU work, not by load width, and narrow
     // strips give more workgroups to spread over the 256 CUs.
-    int vec = s4 ? 4 : (mt == 4 ? 4 : 8);
+    int vec = s4 ? 4 : (mt >= 3 ? 4 : 8);
     if (int v = GetOption("dequant_dot_vec")) vec = v;
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
@@ -658,17 +658,21 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
       XLA_AMD_DECODE(4, 4, 1, kRounded, "dequant_dot_decode_s4_v4_m16_rounded")
       XLA_AMD_DECODE(4, 8, 2, kRounded, "dequant_dot_decode_s4_v8_m32_rounded")
       XLA_AMD_DECODE(4, 4, 2, kRounded, "dequant_dot_decode_s4_v4_m32_rounded")
+      XLA_AMD_DECODE(4, 4, 3, kRounded, "dequant_dot_decode_s4_v4_m48_rounded")
       XLA_AMD_DECODE(4, 4, 4, kRounded, "dequant_dot_decode_s4_v4_m64_rounded")
       XLA_AMD_DECODE(4, 8, 1, kFactored, "dequant_dot_decode_s4_v8_m16_factored")
       XLA_AMD_DECODE(4, 4, 2, kFactored, "dequant_dot_decode_s4_v4_m32_factored")
+      XLA_AMD_DECODE(4, 4, 3, kFactored, "dequant_dot_decode_s4_v4_m48_factored")
       XLA_AMD_DECODE(4, 4, 4, kFactored, "dequant_dot_decode_s4_v4_m64_factored")
       XLA_AMD_DECODE(8, 16, 1, kRounded, "dequant_dot_decode_s8_v16_m16_rounded")
       XLA_AMD_DECODE(8, 8, 1, kRounded, "dequant_dot_decode_s8_v8_m16_rounded")
       XLA_AMD_DECODE(8, 8, 2, kRounded, "dequant_dot_decode_s8_v8_m32_rounded")
+      XLA_AMD_DECODE(8, 4, 3, kRounded, "dequant_dot_decode_s8_v4_m48_rounded")
       XLA_AMD_DECODE(8, 4, 4, kRounded, "dequant_dot_decode_s8_v4_m64_rounded")
       XLA_AMD_DECODE(8, 16, 1, kFactored, "dequant_dot_decode_s8_v16_m16_factored")
       XLA_AMD_DECODE(8, 8, 1, kFactored, "dequant_dot_decode_s8_v8_m16_factored")
       XLA_AMD_DECODE(8, 8, 2, kFactored, "dequant_dot_decode_s8_v8_m32_factored")
+      XLA_AMD_DECODE(8, 4, 3, kFactored, "dequant_dot_decode_s8_v4_m48_factored")
       XLA_AMD_DECODE(8, 4, 4, kFactored, "dequant_dot_decode_s8_v4_m64_factored")
 #undef XLA_AMD_DECODE
       dp.strips = 1; dp.slices = 1;
