@@ -149,7 +149,7 @@ def main():
             e["bound"] = bound
             other.append(e)
 
-        # C2's weights at a prefill-sized token count (not a BASELINE configuration: the tiled s4 kernel)
+        # C2's weights at a prefill-sized token count (informational: the tiled s4 kernel)
         lhs2k = torch.randn((2048, K2), device=dev).to(torch.bfloat16)
         entry("C2 weights, 2048 tokens (s4 prefill)",
               ops.dequant_dot(lhs2k, w_packed, scales, bias, weight_dtype="s4", weight_shape=(K2, N2),
