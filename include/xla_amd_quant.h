@@ -222,6 +222,12 @@ XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
  * an XLA_FFI_Error_Code. */
 XLA_AMD_EXPORT int xla_amd_debug_stream(void* dst, const void* src, size_t bytes, void* stream);
 
+/* Self-check for tests (no counterpart in the reference; allocates and synchronises): evaluates the
+ * epilogue's tanh -- whose quotient uses the f32 division sequence without operand scaling and
+ * fix-up -- and a copy with the plain quotient on all 2^32 f32 bit patterns on the current device
+ * and returns how many results differ (0 is the only acceptable answer), or -1 on a HIP error. */
+XLA_AMD_EXPORT long long xla_amd_debug_tanh_division_mismatches(void);
+
 #ifdef __cplusplus
 }
 #endif

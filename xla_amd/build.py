@@ -15,7 +15,7 @@ LIB = os.path.join(ROOT, "xla_amd", "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 KERNEL_SOURCES = ["capi.hip", "rowwise_quantize.hip", "dequant_dot_decode.hip", "tiled_dot_mfma.hip",
-                  "ffi_handlers.cc"]
+                  "self_check.hip", "ffi_handlers.cc"]
 HOST_SOURCES = ["host/ffi_host.cc", "host/hlo_ir.cc", "host/hlo_parser.cc", "host/quant_fusion_rewriter.cc",
                 "host/host_capi.cc"]
 

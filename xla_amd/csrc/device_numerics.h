@@ -94,6 +94,18 @@ __device__ __forceinline__ bool ordinary_divisor(float s) {
   return sb > 0x0d800000u && sb < 0x71800000u && (sb & 0x7fffffu) != 0x7fffffu;
 }
 
+// n / d as the f32 division expands on this target (reciprocal refined once, quotient corrected
+// twice), minus the operand scaling and the special-case fix-up: bit-identical to n / d when d is
+// a normal number in [2^-8, 2] and n is 0 or 2^-40 <= |n| <= 2, where the scaling factors are 1
+// and the fix-up passes the value through.
+__device__ __forceinline__ float div_well_scaled(float n, float d) {
+  float r = __builtin_amdgcn_rcpf(d);
+  r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+  const float q0 = n * r;
+  const float q1 = __builtin_fmaf(__builtin_fmaf(-d, q0, n), r, q0);
+  return __builtin_fmaf(__builtin_fmaf(-d, q1, n), r, q1);
+}
+
 // xla/codegen/intrinsic/tanh.cc:48-108 rational, then the |x| >= 20 -> +-1 rule of :33-46.
 __device__ __forceinline__ float tanh_xla(float x) {
   const float kClamp = 7.99881172180175781f;
@@ -112,7 +124,8 @@ __device__ __forceinline__ float tanh_xla(float x) {
   q = x2 * q + 1.18534705686654e-04f;
   q = x2 * q + 2.26843463243900e-03f;
   q = x2 * q + 4.89352518554385e-03f;
-  float r = ax < 0.0004f ? x : p / q;
+  // q is in [4.89e-3, 0.95] and |p| <= 0.95; below |x| = 4e-4 (|p| < 2e-6) the quotient is not used
+  float r = ax < 0.0004f ? x : div_well_scaled(p, q);
   return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
 }
 

@@ -1,0 +1,60 @@
+// Exhaustive device-side self-checks of numerics shortcuts, callable from tests through the C ABI.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_numerics.h"
+#include "launch.h"
+
+namespace xla_amd {
+namespace {
+
+// tanh_xla as in device_numerics.h, but with the plain f32 quotient p / q
+__device__ float tanh_plain_quotient(float x) {
+  const float kClamp = 7.99881172180175781f;
+  float ax = __builtin_fabsf(x);
+  float xc = __builtin_fminf(__builtin_fmaxf(x, -kClamp), kClamp);
+  float x2 = xc * xc;
+  float p = -2.76076847742355e-16f;
+  p = x2 * p + 2.00018790482477e-13f;
+  p = x2 * p + -8.60467152213735e-11f;
+  p = x2 * p + 5.12229709037114e-08f;
+  p = x2 * p + 1.48572235717979e-05f;
+  p = x2 * p + 6.37261928875436e-04f;
+  p = x2 * p + 4.89352455891786e-03f;
+  p = xc * p;
+  float q = 1.19825839466702e-06f;
+  q = x2 * q + 1.18534705686654e-04f;
+  q = x2 * q + 2.26843463243900e-03f;
+  q = x2 * q + 4.89352518554385e-03f;
+  float r = ax < 0.0004f ? x : p / q;
+  return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
+}
+
+// block b compares the 2^20 bit patterns b * 2^20 ...; NaN results count as equal to each other
+__global__ __launch_bounds__(256) void tanh_division_check_kernel(unsigned long long* mismatches) {
+  const uint32_t base = blockIdx.x * 1048576u;
+  unsigned long long n = 0;
+  for (uint32_t i = threadIdx.x; i < 1048576u; i += 256) {
+    const float x = bits_to_f32(base + i);
+    const uint32_t a = f32_to_bits(tanh_plain_quotient(x)), b = f32_to_bits(tanh_xla(x));
+    const bool nan_both = (a & 0x7fffffffu) > 0x7f800000u && (b & 0x7fffffffu) > 0x7f800000u;
+    if (a != b && !nan_both) ++n;
+  }
+  if (n) atomicAdd(mismatches, n);
+}
+
+}  // namespace
+}  // namespace xla_amd
+
+extern "C" long long xla_amd_debug_tanh_division_mismatches(void) {
+  unsigned long long* dev = nullptr;
+  unsigned long long host = 0;
+  if (hipMalloc(&dev, sizeof(host)) != hipSuccess) return -1;
+  long long result = -1;
+  if (hipMemset(dev, 0, sizeof(host)) == hipSuccess) {
+    hipLaunchKernelGGL(xla_amd::tanh_division_check_kernel, dim3(4096), dim3(256), 0, 0, dev);
+    if (hipMemcpy(&host, dev, sizeof(host), hipMemcpyDeviceToHost) == hipSuccess) result = (long long)host;
+  }
+  (void)hipFree(dev);
+  return result;
+}

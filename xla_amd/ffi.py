@@ -24,7 +24,8 @@ EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
     "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_fp8_scaled_dot",
     "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
     "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
-    "xla_amd_debug_set_option", "xla_amd_debug_stream"]
+    "xla_amd_debug_set_option", "xla_amd_debug_stream",
+    "xla_amd_debug_tanh_division_mismatches"]
 
 STAGE_INSTANTIATE, STAGE_PREPARE, STAGE_INITIALIZE, STAGE_EXECUTE, STAGE_RECORD = range(5)
 ATTR_ARRAY, ATTR_DICTIONARY, ATTR_SCALAR, ATTR_STRING = 1, 2, 3, 4
@@ -249,6 +250,8 @@ def library():
         L.xla_amd_last_kernel.restype = C.c_char_p
         L.xla_amd_debug_set_option.argtypes = [C.c_char_p, C.c_int]
         L.xla_amd_debug_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.xla_amd_debug_tanh_division_mismatches.restype = C.c_longlong
+        L.xla_amd_debug_tanh_division_mismatches.argtypes = []
         L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
         L.xla_amd_fp8_scaled_dot_workspace_bytes.restype = C.c_size_t
