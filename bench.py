@@ -28,7 +28,7 @@ MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}
 # HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
 # this script, each scaled by what the same counter read for the --calibrate-copy kernel (figures
 # and factors: profiles/decode_c2_hbm_traffic.md).  None where no such run has been made.
-MEASURED_TRAFFIC_BYTES = {"C2 M=64": 137880449, "C2 M=32": 131389977}
+MEASURED_TRAFFIC_BYTES = {"C2 M=64": 137883648, "C2 M=32": 131388569}
 K2, N2, GROUP2 = 8192, 28672, 128
 MS2 = (1, 8, 32, 64)
 
