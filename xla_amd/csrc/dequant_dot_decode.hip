@@ -52,6 +52,7 @@ struct DecodeParams {
   // Rows of a slice that a wave of age class c (wave index / 4) takes, multiples of 64: the
   // waves w, w+4, w+8, ... share a SIMD, which serves the oldest wave first.
   int class_rows[4];
+  int weights_shared;  // every batch reads the same weights and scales (token chunks of one matrix)
 };
 
 __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 
   const int n_lane = strip * TN + li * NV;   // first channel of this lane (may be >= N: discarded)
   const uint32_t pitch = (uint32_t)(((size_t)p.N * WBITS) >> 3);  // bytes per row of W
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.w + (size_t)batch * p.K * pitch, (uint32_t)p.K * pitch);
+  const __amdgpu_buffer_rsrc_t rw =
+      make_rsrc(p.w + (p.weights_shared ? (size_t)0 : (size_t)batch * p.K * pitch), (uint32_t)p.K * pitch);
   // one descriptor per 16-token tile, each ending where the activations end: the per-lane offset
   // is then the same for every tile (token li of the tile) and still range-checks tokens >= M
   __amdgpu_buffer_rsrc_t ra[MT];
@@ -514,7 +516,9 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
   return DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, strips, row_bytes, 8));
 }
 
-int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
+// weights_shared: `batch` counts 64-token chunks of one [batch * M, K] activation matrix that all
+// use the same weights and scales (only the decode kernels take it).
+static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, bool weights_shared) {
   const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4;
   if (!s4 && p.weight_dtype != XLA_FFI_DataType_S8)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: weights must be S4 or S8");
@@ -560,6 +564,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
   dp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
   dp.epilogue = p.epilogue;
   dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
+  dp.weights_shared = weights_shared;
   const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
   const bool per_channel = p.group == p.K;
 
@@ -568,7 +573,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
                        ((uintptr_t)p.weights % 16 == 0);
   const bool mode_ok = mode == kRounded || per_channel;
 
-  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64) {
+  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
@@ -609,11 +614,17 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
     for (int64_t b = 0; b < p.batch; ++b) {
       sub.weights = (const char*)p.weights + b * wbytes;
       sub.scales = (const char*)p.scales + b * sbytes;
-      for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
-        sub.M = p.M - m0 < 64 ? p.M - m0 : 64;
+      // the whole 64-token chunks go out as one launch with the chunk index in the grid (the
+      // workgroups of all chunks then pack onto the CUs together), the remainder as a second one
+      const int64_t whole = p.M / 64;
+      for (int part = 0; part < 2; ++part) {
+        const int64_t m0 = part == 0 ? 0 : whole * 64;
+        sub.M = part == 0 ? 64 : p.M - m0;
+        sub.batch = part == 0 ? whole : 1;
+        if (sub.M == 0 || sub.batch == 0) continue;
         sub.lhs = (const uint16_t*)p.lhs + ((size_t)b * p.M + m0) * p.K;
         sub.out = (uint16_t*)p.out + ((size_t)b * p.M + m0) * p.N;
-        const int rc = LaunchDequantDot(sub, stream);
+        const int rc = LaunchDequantDotImpl(sub, stream, true);
         if (rc) return rc;
         if (!name[0]) snprintf(name, sizeof(name), "%s:x64", xla_amd_last_kernel());
       }
@@ -678,6 +689,8 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
       dp.strips = 1; dp.slices = 1;
     }
   }
+  if (weights_shared)
+    return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot: a token chunk did not fit the decode kernel");
   if (force == 2 || force == 3)
     return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
                 "dequant_dot: the requested kernel does not cover this shape");
@@ -690,5 +703,7 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) {
     return CheckLaunch("dequant_dot_generic");
   }
 }
+
+int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) { return LaunchDequantDotImpl(p, stream, false); }
 
 }  // namespace xla_amd
