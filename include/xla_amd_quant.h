@@ -147,6 +147,20 @@ XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* s
 XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K,
                                                           int64_t N, int32_t weight_dtype);
 
+/*
+ * xla_amd_launch_dequant_dot for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * p->workspace and p->workspace_bytes are ignored: where the decode kernels split K across
+ * workgroups, the f32 partial sums go into a fixed 8 MiB array in device memory that is part of
+ * the library's code object (every GPU the library runs on holds its own copy until the process
+ * ends); its address is looked up once per device on the first call there.  A shape whose partial
+ * sums need more (xla_amd_dequant_dot_workspace_bytes > 8 MiB) is refused with
+ * XLA_FFI_Error_Code_RESOURCE_EXHAUSTED.  The call itself allocates nothing and results are
+ * bit-identical to xla_amd_launch_dequant_dot with a sufficient workspace.  All calls on one GPU
+ * share the array: calls that may overlap on one GPU (different streams) race on it.
+ */
+XLA_AMD_EXPORT int xla_amd_launch_dequant_dot_static_scratch(const XlaAmdDequantDot* p, void* stream);
+
 typedef struct XlaAmdFp8ScaledDot {
   const void* a;       /* f8e4m3fn [M,K] */
   const void* b;       /* f8e4m3fn [K,N] or [N,K] */

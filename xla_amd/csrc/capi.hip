@@ -78,6 +78,11 @@ int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream) {
   return xla_amd::LaunchDequantDot(*p, (hipStream_t)stream);
 }
 
+int xla_amd_launch_dequant_dot_static_scratch(const XlaAmdDequantDot* p, void* stream) {
+  if (!p) return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot_static_scratch: null params");
+  return xla_amd::LaunchDequantDotStaticScratch(*p, (hipStream_t)stream);
+}
+
 int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream) {
   if (!p) return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: null params");
   return xla_amd::LaunchFp8ScaledDot(*p, (hipStream_t)stream);

@@ -30,6 +30,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "device_numerics.h"
 #include "launch.h"
 
@@ -705,5 +707,53 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
 }
 
 int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream) { return LaunchDequantDotImpl(p, stream, false); }
+
+// ---- the same launch for callers that cannot allocate: the split-K partial sums go into a
+// fixed array in device memory that comes with the code object instead of a workspace argument.
+// Every GPU the library runs on holds its own copy of the array until the process ends.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device.  The array's name is only a host-side handle;
+// the address is looked up once per device (with that device current) and kept.
+static int StaticScratchPointer(void** out) {
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot_static_scratch: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot_static_scratch: device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot_static_scratch: hipGetSymbolAddress: %s",
+                  hipGetErrorString(e));
+    ptrs[dev] = ptr;
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+
+int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream) {
+  const size_t need = p.batch > 0 && p.M > 0 && p.K > 0 && p.N > 0
+                          ? DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4)
+                          : 0;
+  if (need > kStaticScratchBytes)
+    return Fail(XLA_FFI_Error_Code_RESOURCE_EXHAUSTED,
+                "dequant_dot_static_scratch: this shape splits K through %zu bytes of partial sums, the static "
+                "scratch holds %zu; use xla_amd_launch_dequant_dot with a workspace",
+                need, kStaticScratchBytes);
+  void* ptr = nullptr;
+  if (int rc = StaticScratchPointer(&ptr)) return rc;
+  XlaAmdDequantDot q = p;
+  q.workspace = ptr;
+  q.workspace_bytes = kStaticScratchBytes;
+  return LaunchDequantDotImpl(q, stream, false);
+}
 
 }  // namespace xla_amd

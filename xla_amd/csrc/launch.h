@@ -22,6 +22,8 @@ int GetOption(const char* key);
 
 int LaunchRowwiseQuantize(const XlaAmdRowwiseQuantize& p, hipStream_t stream, int variant);
 int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream);
+// Same, with the split-K partial sums in the library's static device array (allocates nothing).
+int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream);
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
 
 inline bool IsF32OrBf16(int32_t t) {

@@ -21,7 +21,8 @@ HANDLER_SYMBOLS = {
     "xla_amd.rowwise_quantize_fp8": "xla_amd_rowwise_quantize_fp8",
 }
 EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
-    "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_fp8_scaled_dot",
+    "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch",
+    "xla_amd_launch_fp8_scaled_dot",
     "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
     "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
     "xla_amd_debug_set_option", "xla_amd_debug_stream",
@@ -229,6 +230,16 @@ class NativeHost:
         return host_library().xla_amd_host_find_handler(self._h, target.encode(), platform.encode())
 
 
+class LaunchDequantDot(C.Structure):
+    """XlaAmdDequantDot of include/xla_amd_quant.h (the launcher layer below the handlers)."""
+    _fields_ = [("lhs", C.c_void_p), ("weights", C.c_void_p), ("scales", C.c_void_p), ("bias", C.c_void_p),
+                ("out", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+                ("batch", C.c_int64), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("group", C.c_int64), ("scale_batch", C.c_int64), ("weight_dtype", C.c_int32),
+                ("scale_dtype", C.c_int32), ("bias_dtype", C.c_int32), ("dequant_type", C.c_int32),
+                ("dot_type", C.c_int32), ("epilogue_type", C.c_int32), ("epilogue", C.c_int32)]
+
+
 _lib = None
 
 
@@ -254,6 +265,9 @@ def library():
         L.xla_amd_debug_tanh_division_mismatches.argtypes = []
         L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
+        for sym in ("xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch"):
+            getattr(L, sym).restype = C.c_int
+            getattr(L, sym).argtypes = [C.POINTER(LaunchDequantDot), C.c_void_p]
         L.xla_amd_fp8_scaled_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_fp8_scaled_dot_workspace_bytes.argtypes = [C.c_int64] * 3 + [C.c_int32]
         _lib = L
