@@ -195,7 +195,7 @@ def main():
         a5 = torch.randn((8, 512, 4096), device=dev).to(torch.bfloat16)
         w5 = torch.randint(-127, 128, (8, 4096, 14336), dtype=torch.int8, device=dev)
         s5 = torch.empty((8, 14336), device=dev).uniform_(1e-3, 1e-2)
-        entry("C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, build_only=True),
+        entry("C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, scale_group_size=0, build_only=True),
               8 * (4096 * 14336 + 512 * 4096 * 2 + 14336 * 4 + 512 * 14336 * 2),
               2 * 8 * 512 * 4096 * 14336, "mfma", "bf16")
         del a5, w5

@@ -60,6 +60,10 @@ extern "C" {
  *                   fusion_emitter_int4_device_test.cc:93-104)
  *     dot_type      i32: 11 (default) or 16 -- element type of the dot instruction
  *     epilogue_type i32: 11 (default) or 16 -- element type of the bias add / activation ops
+ *     scale_group_size i64: rows of K that share one scale; 0 = all of them (one scale per output
+ *                   channel: scales [N] or [B,N]), g > 0: scales [K/g,N] or [B,K/g,N].  The rewrite
+ *                   pass always sets it.  Without it the grouping is read off the scales' shape,
+ *                   and a batched call whose rank-2 scales fit both readings is refused.
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame);
 

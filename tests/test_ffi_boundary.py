@@ -235,3 +235,22 @@ def test_native_host_registry_and_errors():
     rp = ffi.Replay([("xla_amd.rowwise_quantize_fp8", quant_frame(host, n_rets=1))])
     with pytest.raises(ffi.FfiError, match="call 0: .*Wrong number of results"):
         rp.run(3)
+
+
+def test_batched_rank2_scales_need_scale_group_size_when_both_readings_fit():
+    """[x,N] scales on a batched dequant_dot are per batch or per group; with x == batch and x | K the
+    shape alone cannot tell, so the handler asks for the attribute the rewrite pass always emits."""
+    host = ffi.Host()
+    args = [(dtypes.BF16, FAKE, (4, 2, 64)), (dtypes.S8, FAKE, (4, 64, 8)), (dtypes.F32, FAKE, (4, 8))]
+    rets = [(dtypes.BF16, FAKE, (4, 2, 8))]
+    with pytest.raises(ffi.FfiError, match=r"can be read per batch or per group of 16 rows: set scale_group_size"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, args, rets))
+    # the attribute is validated against the scales' shape before anything is launched
+    with pytest.raises(ffi.FfiError, match=r"scales must be \[K/scale_group_size,N\]"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, args, rets, {"scale_group_size": ffi.Attr.i64(32)}))
+    with pytest.raises(ffi.FfiError, match="scale_group_size must divide K"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, args, rets, {"scale_group_size": ffi.Attr.i64(48)}))
+    with pytest.raises(ffi.FfiError, match="rank-1 scales go with scale_group_size = 0"):
+        a1 = [(dtypes.BF16, FAKE, (2, 64)), (dtypes.S8, FAKE, (64, 8)), (dtypes.F32, FAKE, (8,))]
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, a1, [(dtypes.BF16, FAKE, (2, 8))],
+                                                    {"scale_group_size": ffi.Attr.i64(16)}))

@@ -36,7 +36,8 @@ def run_dot(w, force_kernel=0, slices=0, vec=0):
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
                               weight_shape=w["weight_shape"], epilogue=w["epilogue"],
                               dequant_type=w["dequant_type"], dot_type=w.get("dot_type", "f32"),
-                              epilogue_type=w.get("epilogue_type", "f32"))
+                              epilogue_type=w.get("epilogue_type", "f32"),
+                              scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"])
         torch.cuda.synchronize()
     finally:
         for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec"):

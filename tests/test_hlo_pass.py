@@ -416,3 +416,56 @@ def test_mutated_modules_are_rejected_or_stay_printable():
     assert accepted > 20 and rejected > 20, (accepted, rejected)
     with pytest.raises(hlo.HloError, match="computation without a name"):
         hlo.rewrite(hm.c1_s8_channel(16, 512, 256).replace("ENTRY %main {", "ENTRY :%main {"))
+
+
+def test_amax_consumer_ahead_of_the_convert_stays_defined_before_use():
+    """XLA prints in post-order, so a user of the amax reduce may sit above the clamp/convert chain
+    that ends the pattern; after the rewrite it must still follow the custom call it now reads."""
+    text = hm.c3_fp8_f8_result(64, 128, 32, amax=True)
+    # move the amax reduce (and a consumer of it) in front of the divide/clamp/convert chain
+    lines = text.split("\n")
+    take = [i for i, l in enumerate(lines) if l.strip().startswith(("%abs_v", "%ninf", "%amax ="))]
+    moved = [lines[i] for i in take]
+    for i in reversed(take):
+        del lines[i]
+    at = next(i for i, l in enumerate(lines) if l.strip().startswith("%d_scale ="))
+    extra = ["  %two = f32[] constant(2)", "  %amax2 = f32[] multiply(%amax, %two)"]
+    lines[at:at] = moved + extra
+    text = "\n".join(lines).replace("tuple(%out, %amax)", "tuple(%out, %amax2)")
+    assert text.index("%amax2 =") < text.index("%clamped =")
+    hlo.print_module(text)  # the input itself is well formed
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result, amax]"] and rf == []
+    again = hlo.print_module(new)  # the parser refuses a use before its definition
+    assert again == new
+    check(new, r"custom-call\(", r"%amax.amax = f32\[\] get-tuple-element", r"%amax2 = f32\[\] multiply\(%amax.amax, %two\)",
+          r"ROOT %result = .* tuple\(%out.out, %amax2\)")
+
+
+def test_rewrite_keeps_side_effects_and_what_was_already_unused():
+    text = hm.c3_fp8(16, 32, 16)
+    text = text.replace("  %a_t =", "  %tok = token[] after-all()\n"
+                        "  %side = token[] custom-call(%tok), custom_call_target=\"my_side_effect\", "
+                        "custom_call_has_side_effect=true\n"
+                        "  %unused = f32[] constant(7)\n  %a_t =", 1)
+    new, rw, rf = hlo.rewrite(text)
+    assert len(rw) == 1 and rf == []
+    ops = opcodes(new)
+    assert "after-all" in ops and ops.count("custom-call") == 2
+    assert "%unused = f32[] constant(7)" in new and "my_side_effect" in new
+    # nothing of the matched pattern survives
+    assert "tanh" not in ops and "dot" not in ops and "convert" not in ops
+
+
+@pytest.mark.parametrize("c1,ok", [("0.797884583", True), ("0.79788456", True), ("0.8", False), ("0.79", False),
+                                   ("0.7979", True), ("0.79795", False)])
+def test_gelu_constants_are_held_to_128_epsilon_of_their_type(c1, ok):
+    """gemm_rewriter.cc:472-503: |actual - expected| < |actual + expected| * 128 eps(type)."""
+    text = hm.c3_fp8(16, 32, 16).replace("constant(0.797884583)", "constant(%s)" % c1)
+    _, rw, _ = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [%s]" % ("BIAS_GELU" if ok else "BIAS")] or (not ok and rw == [])
+    if not ok:
+        assert not any("GELU" in r for r in rw)
+    # a bf16 constant is as coarse as its type: 0.796875 is bf16(0.7978...), within 128 * 2^-7
+    bf = hm.c3_fp8(16, 32, 16, typed="bf16").replace("constant(0.797884583)", "constant(0.796875)")
+    assert hlo.rewrite(bf)[1] == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"]

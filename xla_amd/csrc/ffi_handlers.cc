@@ -334,6 +334,8 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
   CommonAttrs a;
   DecodeCommonAttrs(d, &a);
+  int64_t group_size = 0;
+  const bool has_group_size = d.Int("scale_group_size", &group_size);
   if (!d.ok()) return d.Error();
 
   const bool batched = lhs->rank == 3;
@@ -353,18 +355,40 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
   else if (((a.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
   if (why.empty()) {
-    // scales: [N] | [G,N] | [B,N] | [B,G,N]; a rank-2 [x,N] is per-batch when batched and
-    // x == batch, otherwise per-group
+    // scales: [N] | [G,N] | [B,N] | [B,G,N].  scale_group_size says which: 0 = one scale per output
+    // channel (then a rank-2 [x,N] is per batch), g > 0 = one per g rows of K (then a rank-2 [x,N]
+    // is [K/g,N], shared by the batch).  Without the attribute a rank-2 [x,N] on a batched call is
+    // taken per batch when x == batch and per group otherwise, and refused when both readings fit.
     int64_t groups = 1;
     p.scale_batch = 1;
-    if (sc->rank == 3) {
+    if (has_group_size) {
+      if (group_size < 0 || (group_size > 0 && p.K % group_size != 0)) why = "scale_group_size must divide K";
+      else {
+        groups = group_size == 0 || p.K == 0 ? 1 : p.K / group_size;
+        const bool per_channel = group_size == 0;
+        if (sc->rank == 3) {
+          p.scale_batch = sc->dims[0];
+          if (sc->dims[1] != groups) why = "scales must be [batch,K/scale_group_size,N]";
+        } else if (sc->rank == 2) {
+          if (per_channel) p.scale_batch = sc->dims[0];
+          else if (sc->dims[0] != groups) why = "scales must be [K/scale_group_size,N]";
+        } else if (groups != 1) {
+          why = "rank-1 scales go with scale_group_size = 0";
+        }
+      }
+    } else if (sc->rank == 3) {
       p.scale_batch = sc->dims[0];
       groups = sc->dims[1];
     } else if (sc->rank == 2) {
-      if (batched && sc->dims[0] == p.batch) p.scale_batch = p.batch;
-      else groups = sc->dims[0];
+      const int64_t x = sc->dims[0];
+      if (batched && x == p.batch && p.batch > 1 && x < p.K && p.K % x == 0)
+        why = "rank-2 scales [" + std::to_string(x) + ",N] can be read per batch or per group of " +
+              std::to_string(p.K / x) + " rows: set scale_group_size, or pass rank-3 scales";
+      else if (batched && x == p.batch) p.scale_batch = p.batch;
+      else groups = x;
     }
-    if (groups <= 0 || (p.K > 0 && p.K % groups != 0)) why = "the number of scale groups must divide K";
+    if (!why.empty()) {
+    } else if (groups <= 0 || (p.K > 0 && p.K % groups != 0)) why = "the number of scale groups must divide K";
     else if (p.scale_batch != 1 && p.scale_batch != p.batch) why = "scales batch dimension differs";
     else p.group = p.K > 0 ? p.K / groups : 1;
   }

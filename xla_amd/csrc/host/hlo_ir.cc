@@ -125,19 +125,77 @@ void Computation::ReplaceAllUses(Instr* from, Instr* to) {
   RecomputeUsers();
 }
 
-int Computation::RemoveDead() {
+bool HasSideEffect(const Instr& i) {
+  static const char* const kOps[] = {"after-all", "infeed", "outfeed", "send", "send-done", "recv", "recv-done",
+                                     "rng", "rng-get-and-update-state", "partition-id", "replica-id",
+                                     "all-reduce", "all-reduce-start", "all-reduce-done", "all-gather",
+                                     "all-gather-start", "all-gather-done", "all-to-all", "ragged-all-to-all",
+                                     "collective-permute", "collective-permute-start", "collective-permute-done",
+                                     "collective-broadcast", "reduce-scatter", "async-start", "async-update",
+                                     "async-done", "copy-start", "copy-done", "set-dimension-size",
+                                     "add-dependency", "opt-barrier", "while", "conditional", "call"};
+  for (const char* op : kOps)
+    if (i.opcode == op) return true;
+  if (i.opcode == "custom-call") {
+    const std::string* v = i.Attr("custom_call_has_side_effect");
+    return v && *v == "true";
+  }
+  return false;
+}
+
+std::set<const Instr*> Computation::Unused() {
+  RecomputeUsers();
+  std::set<const Instr*> out;
+  const Instr* r = root();
+  for (const auto& i : instrs)
+    if (i.get() != r && i->users.empty() && i->opcode != "parameter") out.insert(i.get());
+  return out;
+}
+
+int Computation::RemoveDead(const std::set<const Instr*>& keep) {
   int removed = 0;
   for (;;) {
     RecomputeUsers();
     Instr* r = root();
     auto it = std::find_if(instrs.begin(), instrs.end(), [&](const std::unique_ptr<Instr>& p) {
-      return p.get() != r && p->users.empty() && p->opcode != "parameter";
+      return p.get() != r && p->users.empty() && p->opcode != "parameter" && !HasSideEffect(*p) &&
+             !keep.count(p.get());
     });
     if (it == instrs.end()) break;
     instrs.erase(it);
     ++removed;
   }
   return removed;
+}
+
+void Computation::SortDefBeforeUse() {
+  std::vector<std::unique_ptr<Instr>> old = std::move(instrs);
+  instrs.clear();
+  std::unordered_map<const Instr*, size_t> index;
+  for (size_t i = 0; i < old.size(); ++i) index[old[i].get()] = i;
+  std::vector<char> state(old.size(), 0);  // 0 new, 1 on the stack, 2 emitted
+  // iterative post-order from each instruction in list order
+  for (size_t start = 0; start < old.size(); ++start) {
+    if (state[start]) continue;
+    std::vector<std::pair<size_t, size_t>> stack = {{start, 0}};
+    state[start] = 1;
+    while (!stack.empty()) {
+      auto& [at, next] = stack.back();
+      Instr* ins = old[at].get();
+      if (next < ins->operands.size()) {
+        auto it = index.find(ins->operands[next++]);
+        if (it != index.end() && state[it->second] == 0) {
+          state[it->second] = 1;
+          stack.push_back({it->second, 0});
+        }
+        continue;
+      }
+      state[at] = 2;
+      instrs.push_back(std::move(old[at]));
+      stack.pop_back();
+    }
+  }
+  RecomputeUsers();
 }
 
 std::string Computation::UniqueName(const std::string& base) const {

@@ -7,6 +7,7 @@
 #include <stdint.h>
 
 #include <memory>
+#include <set>
 #include <string>
 #include <utility>
 #include <vector>
@@ -47,6 +48,10 @@ struct Instr {
   int64_t user_count() const { return (int64_t)users.size(); }
 };
 
+// Side effects as HloInstruction::HasSideEffect sees them (xla/hlo/ir/hlo_instruction.cc): the
+// opcode itself, or custom_call_has_side_effect=true on a custom call.
+bool HasSideEffect(const Instr& i);
+
 struct Computation {
   std::string name;
   bool is_entry = false;
@@ -59,8 +64,15 @@ struct Computation {
   Instr* Insert(std::unique_ptr<Instr> ins, const Instr* before);
   // Every use of `from` (and its root flag) moves to `to`.
   void ReplaceAllUses(Instr* from, Instr* to);
-  // Drops instructions nothing uses (parameters and the root stay).  Returns how many.
-  int RemoveDead();
+  // Instructions nothing uses right now (root and parameters left out): what a later
+  // RemoveDead must not touch because the module came that way.
+  std::set<const Instr*> Unused();
+  // Drops instructions that nothing uses any more, except the root, parameters, instructions with
+  // side effects (HasSideEffect) and those in `keep`.  Returns how many.
+  int RemoveDead(const std::set<const Instr*>& keep);
+  // Stable re-ordering so that every operand precedes its users: instructions keep their relative
+  // order except where an operand has to move up in front of an earlier user.
+  void SortDefBeforeUse();
   std::string UniqueName(const std::string& base) const;
 };
 

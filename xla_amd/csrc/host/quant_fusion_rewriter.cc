@@ -59,11 +59,25 @@ bool ConstScalar(const Instr* i, double* v) {
   return end && *end == 0 && !lit.empty();
 }
 
-bool IsConst(const Instr* i, double want, double rel_tol = 0) {
+bool IsConst(const Instr* i, double want) {
+  double v;
+  return ConstScalar(i, &v) && v == want;
+}
+
+// A constant close to `want` by the rule of BcastConstScalarNear (gemm_rewriter.cc:472-503):
+// |actual - want| < |actual + want| * 128 * epsilon of the constant's own element type.
+bool IsConstNear(const Instr* i, double want) {
   double v;
   if (!ConstScalar(i, &v)) return false;
-  if (rel_tol == 0) return v == want;
-  return fabs(v - want) <= rel_tol * fabs(want);
+  const Instr* c = i;
+  while (!c->Is("constant")) c = c->operands[0];
+  double eps;
+  if (c->shape.dtype == "f16") eps = 0x1p-10;
+  else if (c->shape.dtype == "bf16") eps = 0x1p-7;
+  else if (c->shape.dtype == "f32") eps = 0x1p-23;
+  else if (c->shape.dtype == "f64") eps = 0x1p-52;
+  else return false;
+  return fabs(v - want) < fabs(v + want) * 128 * eps;
 }
 
 // broadcast of a rank-0 value (dimensions={})
@@ -133,12 +147,12 @@ bool MatchGelu(Instr* out, Instr* x) {
   if (!BinaryWith(onep, "add", [](Instr* s) { return IsConst(s, 1.0); }, &th)) return false;
   if (!th->Is("tanh")) return false;
   Instr* inner;
-  if (!BinaryWith(th->operands[0], "multiply", [](Instr* s) { return IsConst(s, 0.7978845608, 1e-2); }, &inner))
+  if (!BinaryWith(th->operands[0], "multiply", [](Instr* s) { return IsConstNear(s, 0.7978845608028654); }, &inner))
     return false;
   Instr* cube_term;
   if (!BinaryWith(inner, "add", [&](Instr* s) { return s == x; }, &cube_term)) return false;
   Instr* cube;
-  if (!BinaryWith(cube_term, "multiply", [](Instr* s) { return IsConst(s, 0.044715, 1e-2); }, &cube)) return false;
+  if (!BinaryWith(cube_term, "multiply", [](Instr* s) { return IsConstNear(s, 0.044715); }, &cube)) return false;
   Instr* sq;
   if (!BinaryWith(cube, "multiply", [&](Instr* s) { return s == x; }, &sq)) return false;
   Instr *a, *b;
@@ -590,7 +604,11 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
                   ? opt.dequant_workspace_bytes(B, M, K, N, q.w->shape.dtype == "s4" ? 21 : 2)
                   : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
-  Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results, CommonConfig(ep, q.type, dot->shape.dtype));
+  // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
+  const int64_t group_size = rank == 2 && q.scale->shape.rank() == 2 ? K / q.scale->shape.dims[0] : 0;
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results,
+                         CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
+                             std::to_string(group_size) + " : i64");
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype + "]");
@@ -705,7 +723,8 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
     bool again = true;
     while (again) {
       again = false;
-      comp->RecomputeUsers();
+      // what nothing used before this sweep stays: only what a rewrite orphans is removed
+      const std::set<const Instr*> unused_before = comp->Unused();
       for (auto& up : comp->instrs) {
         Instr* i = up.get();
         bool did = false;
@@ -718,7 +737,9 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         }
         if (did) {
           ++changed;
-          comp->RemoveDead();
+          comp->RemoveDead(unused_before);
+          // a redirected user (of an amax, of the scales) may sit above the new call
+          comp->SortDefBeforeUse();
           again = true;
           break;  // the instruction list changed under the loop
         }

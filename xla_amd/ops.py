@@ -57,8 +57,10 @@ def _scratch(nbytes, device):
 
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
-                out=None, scratch="auto", build_only=False):
-    """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K]."""
+                scale_group_size=None, out=None, scratch="auto", build_only=False):
+    """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
+    scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
+    the handler reads the grouping off the scales' shape."""
     _check_cuda(lhs, weights, scales, bias)
     wdt = dtypes.S4 if weight_dtype == "s4" else dtypes.S8
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
@@ -80,6 +82,8 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     attrs = {"epilogue": ffi.Attr.str(epilogue), "dequant_type": ffi.Attr.i32(_TYPE_ATTR[dequant_type]),
              "dot_type": ffi.Attr.i32(_TYPE_ATTR[dot_type]),
              "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type])}
+    if scale_group_size is not None:
+        attrs["scale_group_size"] = ffi.Attr.i64(scale_group_size)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
                 keep=(lhs, weights, scales, bias, scratch))
     return call if build_only else call.run()
