@@ -1,0 +1,80 @@
+// Declarations shared by the decode (weight-streaming) dequantize-dot kernels.
+#ifndef XLA_AMD_CSRC_DECODE_COMMON_H_
+#define XLA_AMD_CSRC_DECODE_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "device_numerics.h"
+#include "launch.h"
+
+namespace xla_amd {
+
+enum : int { kRounded = 0, kFactored = 1 };
+
+struct DecodeParams {
+  const uint16_t* lhs;   // [batch, M, K]
+  const uint8_t* w;      // [batch, K, N] packed
+  const void* scales;    // [scale_batch, K/group, N]
+  const void* bias;      // [N] or null
+  uint16_t* out;         // [batch, M, N]
+  float* workspace;      // [batch, slices, M, N] when slices > 1
+  int M, K, N, group;
+  int scale_is_bf16, bias_is_bf16, scale_batched;
+  int bf16_dot, bf16_ops, epilogue;
+  int strips, slices, rows_per_slice;  // rows_per_slice: multiple of 32 * WAVES
+  // Rows of a slice that a wave of age class c (wave index / 4) takes, multiples of 64: the
+  // waves w, w+4, w+8, ... share a SIMD, which serves the oldest wave first.
+  int class_rows[4];
+  int weights_shared;  // every batch reads the same weights and scales (token chunks of one matrix)
+  // s4x kernels: a unit is four scale groups of rows; a SIMD's waves take class_units[age class]
+  // consecutive units each, SIMD b starting at unit b * units_per_simd of the slice
+  int units_per_simd;
+  int class_units[4];
+};
+
+static __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
+  return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];
+}
+
+// Buffer descriptor over [base, base+bytes): loads through it return 0 past the end, which is
+// how rows beyond K and tokens beyond M drop out of the main loop without any branch.
+static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// N32 consecutive dwords (1, 2 or a multiple of 4) at voff + soff.  The hardware range-checks
+// the per-lane offset only, so soff must be 0 wherever running past the end is possible.
+template <int N32>
+static __device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff,
+                                                  uint32_t* dst) {
+  if constexpr (N32 >= 4) {
+#pragma unroll
+    for (int q = 0; q < N32 / 4; ++q) {
+      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff + 16 * q, soff, 0);
+      dst[4 * q] = v[0]; dst[4 * q + 1] = v[1]; dst[4 * q + 2] = v[2]; dst[4 * q + 3] = v[3];
+    }
+  } else if constexpr (N32 == 2) {
+    uintx2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    dst[0] = v[0]; dst[1] = v[1];
+  } else {
+    dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+  }
+}
+
+
+// Sums the K-slices of dp.workspace in slice order and applies scale, bias and activation
+// (dequant_dot_decode.hip); mode: kRounded or kFactored.
+int LaunchDecodeFinalize(const DecodeParams& dp, int batch, hipStream_t stream, int mode);
+
+// K-slices a decode launch uses for this shape, and the f32 partial sums they need.
+int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves);
+size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices);
+
+// s4 weights with bf16 group scales under a bf16-typed multiply (dequant_dot_decode_s4x.hip).
+// Returns -1 when the shape is not covered, else the launch status.  dp comes filled except for
+// the strip / slice layout.
+int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream);
+
+}  // namespace xla_amd
+#endif  // XLA_AMD_CSRC_DECODE_COMMON_H_

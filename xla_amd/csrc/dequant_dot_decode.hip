@@ -32,59 +32,12 @@
 
 #include <mutex>
 
+#include "decode_common.h"
 #include "device_numerics.h"
 #include "launch.h"
 
 namespace xla_amd {
 namespace {
-
-enum : int { kRounded = 0, kFactored = 1 };
-
-struct DecodeParams {
-  const uint16_t* lhs;   // [batch, M, K]
-  const uint8_t* w;      // [batch, K, N] packed
-  const void* scales;    // [scale_batch, K/group, N]
-  const void* bias;      // [N] or null
-  uint16_t* out;         // [batch, M, N]
-  float* workspace;      // [batch, slices, M, N] when slices > 1
-  int M, K, N, group;
-  int scale_is_bf16, bias_is_bf16, scale_batched;
-  int bf16_dot, bf16_ops, epilogue;
-  int strips, slices, rows_per_slice;  // rows_per_slice: multiple of 32 * WAVES
-  // Rows of a slice that a wave of age class c (wave index / 4) takes, multiples of 64: the
-  // waves w, w+4, w+8, ... share a SIMD, which serves the oldest wave first.
-  int class_rows[4];
-  int weights_shared;  // every batch reads the same weights and scales (token chunks of one matrix)
-};
-
-__device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
-  return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];
-}
-
-// Buffer descriptor over [base, base+bytes): loads through it return 0 past the end, which is
-// how rows beyond K and tokens beyond M drop out of the main loop without any branch.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-
-// N32 consecutive dwords (1, 2 or a multiple of 4) at voff + soff.  The hardware range-checks
-// the per-lane offset only, so soff must be 0 wherever running past the end is possible.
-template <int N32>
-__device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff,
-                                                  uint32_t* dst) {
-  if constexpr (N32 >= 4) {
-#pragma unroll
-    for (int q = 0; q < N32 / 4; ++q) {
-      uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff + 16 * q, soff, 0);
-      dst[4 * q] = v[0]; dst[4 * q + 1] = v[1]; dst[4 * q + 2] = v[2]; dst[4 * q + 3] = v[3];
-    }
-  } else if constexpr (N32 == 2) {
-    uintx2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
-    dst[0] = v[0]; dst[1] = v[1];
-  } else {
-    dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
-  }
-}
 
 // WBITS: 4 or 8.  VEC: bytes a lane reads per row (4, 8, 16).  MT: 16-token tiles.  WAVES: waves
 // per workgroup, splitting the workgroup's rows.  SCALE_BF16: element type of the scales.
@@ -441,7 +394,13 @@ int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const c
 
 }  // namespace
 
-int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream);  // dequant_dot_mfma.hip
+int LaunchDecodeFinalize(const DecodeParams& dp, int batch, hipStream_t stream, int mode) {
+  dim3 fgrid((unsigned)(((size_t)dp.M * dp.N + 255) / 256), (unsigned)batch);
+  hipLaunchKernelGGL(dequant_dot_finalize_kernel, fgrid, dim3(256), 0, stream, dp, mode);
+  return CheckLaunch("dequant_dot_finalize");
+}
+
+int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream);  // tiled_dot_mfma.hip
 
 // Rows of K each workgroup takes so that `slices` workgroups cover K; multiple of 64*waves.
 static int RowsPerSlice(int K, int slices, int waves) {
@@ -489,7 +448,7 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
 // until there are, as long as a wave keeps at least four 32-row steps and the partial sums
 // (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or a quarter
 // of the weight bytes when the strips would leave three quarters of the CUs idle.
-static int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
+int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
   if (int s = GetOption("dequant_dot_slices")) return s;
   const int64_t want = M <= 4 ? 448 : 192;
   const double weight_bytes = (double)K * row_bytes;
@@ -639,6 +598,12 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     int mt, vec, nv;
     const bool shape_ok = decode_shape(p.M, &mt, &vec, &nv);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
+    // s4 with bf16 group scales and a bf16-typed multiply: the kernels that dequantise through the
+    // 4x4x4 matrix instruction
+    if (shape_ok && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1) {
+      const int rc = LaunchDequantDotDecodeS4x(dp, p, stream);
+      if (rc >= 0) return rc;
+    }
     if (shape_ok) {
       dp.strips = (int)((p.N + 16 * nv - 1) / (16 * nv));
       // Up to 16 tokens, when the strips alone give (nearly) a workgroup per CU, the workgroup is
