@@ -19,9 +19,10 @@ def say(msg):
     sys.stdout.flush()
 
 
-def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, side=0, depth=0):
+def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0):
     """x: 1 keeps s4 weights off the kernels that dequantise through the 4x4x4 matrix instruction
-    (default: off whenever a strip width `vec` of the other kernels is asked for)."""
+    (default: off whenever a strip width `vec` of the other kernels is asked for); pair: 1 takes the
+    two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never."""
     lhs = dev_bf16(w["lhs"])
     if w["weight_dtype"] == "s4":
         wt = dev_u8(w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"]))
@@ -35,7 +36,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, side=0, depth=0):
     ffi.set_option("dequant_dot_slices", slices)
     ffi.set_option("dequant_dot_vec", vec)
     ffi.set_option("dequant_dot_x", (1 if vec else 0) if x is None else x)
-    ffi.set_option("dequant_dot_side", side)
+    ffi.set_option("dequant_dot_pair", pair)
     ffi.set_option("dequant_dot_depth", depth)
     try:
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
@@ -45,7 +46,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, side=0, depth=0):
                               scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"])
         torch.cuda.synchronize()
     finally:
-        for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec", "dequant_dot_x", "dequant_dot_side",
+        for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec", "dequant_dot_x", "dequant_dot_pair",
                   "dequant_dot_depth"):
             ffi.set_option(k, 0)
     return host_bf16(out), ffi.last_kernel()
@@ -111,29 +112,29 @@ def test_s4_decode_variants(oracle, M, vec, slices):
     compare(oracle, w, got, "s4 %s slices=%d" % (kern, slices))
 
 
-@pytest.mark.parametrize("M,side,depth,slices,K,N,group", [
-    (1, 4, 4, 1, 2048, 768, 64), (3, 4, 2, 2, 2048, 768, 64), (8, 2, 4, 1, 2048 + 256, 800, 128),
-    (8, 1, 2, 1, 1024, 1024, 128), (16, 1, 4, 1, 2048, 768, 128), (16, 4, 4, 4, 4096, 256, 32),
-    (20, 1, 2, 2, 2048 + 128, 736, 64), (33, 1, 4, 1, 1536, 512, 128), (48, 1, 2, 1, 1024, 640, 64),
-    (64, 1, 2, 2, 2048, 768, 128), (64, 2, 2, 1, 1024, 512, 32)])
-def test_s4x_variants(oracle, M, side, depth, slices, K, N, group):
-    """The kernels that scale and transpose through the 4x4x4 matrix instruction: groups side by
-    side, prefetch depth, K-slices, a ragged last strip (N % 128 != 0) and a K that is no whole
-    number of units or of waves' shares."""
-    say("dequant_dot s4x M=%d side=%d depth=%d slices=%d K=%d N=%d group=%d" % (M, side, depth, slices, K, N, group))
+@pytest.mark.parametrize("M,pair,depth,slices,K,N,group", [
+    (1, 2, 4, 1, 2048, 768, 128), (3, 2, 2, 2, 2048, 768, 64), (8, 1, 2, 0, 2048 + 256, 800, 128),
+    (8, 2, 2, 1, 1024, 1024, 128), (16, 2, 4, 1, 2048, 768, 128), (16, 1, 2, 0, 4096, 256, 64),
+    (20, 2, 2, 2, 2048 + 128, 736, 64), (33, 2, 4, 1, 1536, 512, 128), (48, 2, 2, 1, 1024, 640, 64),
+    (64, 2, 2, 2, 2048, 768, 128), (5, 1, 2, 0, 1024 + 64, 1120, 64), (13, 1, 2, 0, 8192, 512, 128)])
+def test_s4x_variants(oracle, M, pair, depth, slices, K, N, group):
+    """The kernels that scale and transpose through the 4x4x4 matrix instruction: one workgroup per
+    128-channel strip or two per 256-channel strip handing over inside the kernel, prefetch depth,
+    K-slices, a ragged last strip and a K that is no whole number of waves' shares."""
+    say("dequant_dot s4x M=%d pair=%d depth=%d slices=%d K=%d N=%d group=%d" % (M, pair, depth, slices, K, N, group))
     w = workloads.c2_s4_group(M=M, K=K, N=N, group=group)
-    got, kern = run_dot(w, force_kernel=2, slices=slices, side=side, depth=depth)
-    assert kern.startswith("dequant_dot_decode_s4x_") and "_side%d_" % side in kern, kern
+    got, kern = run_dot(w, force_kernel=2, slices=slices, pair=pair, depth=depth)
+    assert kern.startswith("dequant_dot_decode_s4x_") and kern.endswith("_pair") == (pair == 1), kern
     compare(oracle, w, got, "%s slices=%d" % (kern, slices))
 
 
-@pytest.mark.parametrize("side", [1, 4])
-def test_s4x_unpack_and_dequant_bit_exact(oracle, side):
+@pytest.mark.parametrize("pair", [2, 1])
+def test_s4x_unpack_and_dequant_bit_exact(oracle, pair):
     """One-hot activations through the matrix-instruction dequantisation: every output is one
     dequantised weight -- nibble order, sign, the f16 scale operand and the bf16 rounding, exactly;
     scales across the whole f16 window and both signs."""
-    say("dequant_dot s4x one-hot side=%d" % side)
-    K, N, group = 512, 256, 64
+    say("dequant_dot s4x one-hot pair=%d" % pair)
+    K, N, group = 512, 512, 64
     rng = np.random.default_rng(5)
     wv = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
     wv[:16, :16] = np.arange(-8, 8, dtype=np.int8)[:, None]
@@ -141,26 +142,26 @@ def test_s4x_unpack_and_dequant_bit_exact(oracle, side):
     expo = rng.integers(-22, 3, size=(K // group, N)).astype(np.float32)
     sign = rng.choice([-1.0, 1.0], size=(K // group, N)).astype(np.float32)
     sc = dtypes.f32_to_bf16(sign * mant * np.exp2(expo))
-    for m0 in range(0, K, 64):
-        a = np.zeros((64, K), np.float32)
-        a[np.arange(64), m0 + np.arange(64)] = 1.0
+    for m0 in range(0, K, 16):
+        a = np.zeros((16, K), np.float32)
+        a[np.arange(16), m0 + np.arange(16)] = 1.0
         w = dict(lhs=dtypes.f32_to_bf16(a), weights=wv, weights_packed=dtypes.pack_s4(wv), scales=sc,
                  bias=None, weight_dtype="s4", weight_shape=(K, N), group=group, dequant_type="bf16",
                  epilogue="DEFAULT")
-        got, kern = run_dot(w, force_kernel=2, side=side)
-        assert kern.startswith("dequant_dot_decode_s4x_"), kern
-        prod = wv[m0:m0 + 64].astype(np.float32) * np.repeat(dtypes.bf16_to_f32(sc), group, axis=0)[m0:m0 + 64]
+        got, kern = run_dot(w, force_kernel=2, pair=pair)
+        assert kern.startswith("dequant_dot_decode_s4x_") and kern.endswith("_pair") == (pair == 1), kern
+        prod = wv[m0:m0 + 16].astype(np.float32) * np.repeat(dtypes.bf16_to_f32(sc), group, axis=0)[m0:m0 + 16]
         want = dtypes.f32_to_bf16(prod)
         assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want)), kern
 
 
-@pytest.mark.parametrize("M,side", [(4, 4), (24, 1)])
-def test_s4x_scales_outside_the_f16_window(oracle, M, side):
+@pytest.mark.parametrize("M,pair", [(4, 1), (4, 2), (24, 2)])
+def test_s4x_scales_outside_the_f16_window(oracle, M, pair):
     """Zero scales stay on the fast path; huge, tiny, subnormal, infinite and NaN scales flag their
     channel, which the kernel then recomputes with ordinary arithmetic: every channel must still
-    match the oracle."""
-    say("dequant_dot s4x odd scales M=%d side=%d" % (M, side))
-    K, N, group = 1024, 256, 128
+    match the oracle -- also when the flagged rows lie in only one of the two workgroups of a strip."""
+    say("dequant_dot s4x odd scales M=%d pair=%d" % (M, pair))
+    K, N, group = 1024, 512, 128
     w = workloads.c2_s4_group(M=M, K=K, N=N, group=group)
     sc = dtypes.bf16_to_f32(w["scales"]).copy()
     sc[0, 3] = 0.0
@@ -171,20 +172,49 @@ def test_s4x_scales_outside_the_f16_window(oracle, M, side):
     sc[5, 129] = np.inf
     sc[6, 200] = np.nan
     sc[7, 255] = -3.0e4
+    sc[0, 300] = 64.0
+    sc[7, 301] = 2.0 ** -25
     w["scales"] = dtypes.f32_to_bf16(sc)
-    got, kern = run_dot(w, force_kernel=2, side=side)
-    assert kern.startswith("dequant_dot_decode_s4x_"), kern
+    got, kern = run_dot(w, force_kernel=2, pair=pair)
+    assert kern.startswith("dequant_dot_decode_s4x_") and kern.endswith("_pair") == (pair == 1), kern
     ref = oracle_dot(oracle, w)
     ok_cols = np.ones(N, bool)
     ok_cols[[129, 200]] = False
     a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
     wd = np.abs(w["weights"].astype(np.float64)) * np.abs(np.repeat(np.nan_to_num(sc.astype(np.float64), nan=0.0, posinf=0.0), group, axis=0))
-    from tests.gpu_util import check_dot, dot_floor
     check_dot(got[:, ok_cols], ref[:, ok_cols], dot_floor(a, wd, K)[:, ok_cols], kern)
     # an infinite or NaN scale makes the whole channel non-finite, on both sides
     g, r = dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(ref)
     assert not np.isfinite(r[:, [129, 200]]).any() and not np.isfinite(g[:, [129, 200]]).any()
     assert np.array_equal(np.isnan(g[:, [129, 200]]), np.isnan(r[:, [129, 200]]))
+
+
+def test_s4x_pair_same_call_frame_replayed(oracle):
+    """The hand-over flag is lowered by the finisher, so the very same call frame (same workspace,
+    same flag value) can run again and again -- what a captured graph does -- with new activations
+    each time; the workspace starts out holding arbitrary bytes."""
+    say("dequant_dot s4x pair replay")
+    M, K, N = 8, 2048, 1024
+    w = workloads.c2_s4_group(M=M, K=K, N=N)
+    lhs = dev_bf16(w["lhs"])
+    wt, sc, bias = dev_u8(w["weights_packed"]), dev_bf16(w["scales"]), dev_bf16(w["bias"])
+    nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S4)
+    ffi.set_option("dequant_dot_pair", 1)
+    try:
+        nbytes = max(nbytes, ffi.library().xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S4))
+        scratch = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+        call = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype="s4", weight_shape=(K, N), epilogue="BIAS_SILU",
+                               dequant_type="bf16", scratch=scratch, build_only=True)
+        rng = np.random.default_rng(9)
+        for it in range(4):
+            a = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+            lhs.copy_(dev_bf16(a))
+            out = call.run()
+            torch.cuda.synchronize()
+            assert ffi.last_kernel() == "dequant_dot_decode_s4x_m16_pair", ffi.last_kernel()
+            compare(oracle, dict(w, lhs=a), host_bf16(out), "pair replay %d" % it)
+    finally:
+        ffi.set_option("dequant_dot_pair", 0)
 
 
 @pytest.mark.parametrize("which", ["s4", "s8"])
@@ -340,7 +370,7 @@ def test_s4_more_than_64_tokens_picks_the_cheaper_kernel():
     dev = torch.device("cuda:0")
     wt = torch.zeros(K * N // 2, dtype=torch.uint8, device=dev)
     sc = torch.ones((K // 128, N), dtype=torch.bfloat16, device=dev)
-    for M, want in ((128, "dequant_dot_decode_s4x_m64_side1_d2:x64"), (1024, "dequant_dot_tiled_s4_rounded")):
+    for M, want in ((128, "dequant_dot_decode_s4x_m64_d2:x64"), (1024, "dequant_dot_tiled_s4_rounded")):
         lhs = torch.zeros((M, K), dtype=torch.bfloat16, device=dev)
         out = ops.dequant_dot(lhs, wt, sc, None, weight_dtype="s4", weight_shape=(K, N), epilogue="DEFAULT",
                               dequant_type="bf16")

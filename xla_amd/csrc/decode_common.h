@@ -31,6 +31,14 @@ struct DecodeParams {
   // consecutive units each, SIMD b starting at unit b * units_per_simd of the slice
   int units_per_simd;
   int class_units[4];
+  // s4x kernels, two workgroups per strip handing over inside the kernel: the producer's sums go to
+  // workspace[batch * strips + strip][16 x 256 floats], then flags[batch * strips + strip] is set
+  // to epoch (never 0)
+  int pair;
+  int rows_first;       // rows the producer takes; the finisher takes rows_per_slice from there on
+  int units_per_simd2;  // the finisher's units per SIMD; its class split is class_units[2..3]
+  unsigned long long* flags;
+  unsigned long long epoch;
 };
 
 static __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
@@ -75,6 +83,10 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
 // Returns -1 when the shape is not covered, else the launch status.  dp comes filled except for
 // the strip / slice layout.
 int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream);
+// Whether LaunchDequantDotDecodeS4x would split the rows of this shape over two workgroups that hand
+// over inside the kernel, and the workspace that takes.
+bool S4xPairShape(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t group);
+size_t S4xPairWorkspaceBytes(int64_t batch, int64_t M, int64_t N);
 
 }  // namespace xla_amd
 #endif  // XLA_AMD_CSRC_DECODE_COMMON_H_

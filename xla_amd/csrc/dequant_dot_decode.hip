@@ -474,7 +474,11 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
   const int nv = vec * (s4 ? 2 : 1);
   const int64_t row_bytes = N * (s4 ? 1 : 2) / 2;
   const int strips = (int)((N + 16 * nv - 1) / (16 * nv));
-  return DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, strips, row_bytes, 8));
+  size_t bytes = DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, strips, row_bytes, 8));
+  // s4 up to 16 tokens may run as two workgroups per 256-channel strip that hand over through the
+  // workspace (the group size is not known here: the smallest one that path takes decides)
+  if (s4 && S4xPairShape(batch, M, K, N, 64)) bytes = bytes > S4xPairWorkspaceBytes(batch, M, N) ? bytes : S4xPairWorkspaceBytes(batch, M, N);
+  return bytes;
 }
 
 // weights_shared: `batch` counts 64-token chunks of one [batch * M, K] activation matrix that all

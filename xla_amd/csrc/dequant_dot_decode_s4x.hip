@@ -25,15 +25,20 @@
 // inf, NaN), which are recomputed at the end by a plain loop: every input gets the reference's
 // result.
 //
-// Lane (kb, q, i) = (lane >> 4, (lane >> 2) & 3, lane & 3) loads rows i and i + 4 of an 8-row
-// block, 16 bytes (32 channels) of each.  SIDE scale groups are walked side by side: the four
-// kb sit in SIDE different groups, 4 / SIDE consecutive 8-row blocks in each.  SIDE = 4 rebuilds
-// the scale operands once per group / 8 steps, but spreads a step's activations over four cache
-// lines per token (fine for a few tokens); SIDE = 1 reads 64 contiguous bytes per token and step.
+// Consuming side: lane (kb, q, i) = (lane >> 4, (lane >> 2) & 3, lane & 3) takes rows 8 kb + i and
+// 8 kb + i + 4 of a 32-row step, 16 bytes (32 channels) of each.  Loading side: weights and
+// activations go global -> LDS by direct loads whose lanes are laid out for the memory system, not
+// for the arithmetic: consecutive lanes read consecutive 16-byte pieces of one row.  With COLS = 2 a
+// wave covers 256 channels, so every load instruction takes whole 128-byte lines (measured on
+// MI355X for this matrix: 64-byte pieces per workgroup stream at 5.4 TB/s at best, whole lines
+// at 6.8 TB/s); the rows are then split over two workgroups per strip, and the second adds the
+// first one's partial sums, handed over through the workspace, before the epilogue.
 //
 // Bound: HBM.  Algorithmic bytes: K*N/2 (weights) + scales, bias, lhs and out once each.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <atomic>
 
 #include "decode_common.h"
 #include "device_numerics.h"
@@ -46,29 +51,35 @@ typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 typedef uint16_t ushortx2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// MT: 16-token tiles.  WAVES: waves per workgroup (they split the rows).  SIDE: scale groups side
-// by side (1, 2 or 4).  DEPTH: steps whose loads are in flight or in use (>= 2).
-template <int MT, int WAVES, int SIDE, int DEPTH>
+// MT: 16-token tiles.  WAVES: waves per workgroup (they split the rows).  COLS: 128-channel columns
+// a wave covers (1 or 2).  DEPTH: steps whose loads are in flight or in use (>= 2).
+template <int MT, int WAVES, int COLS, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(DecodeParams p) {
-  constexpr int R = 32 * MT;      // accumulator registers per lane: 32 channels x MT token tiles
-  constexpr int KBG = 4 / SIDE;   // 8-row blocks of one group in a step
+  constexpr int R = 32 * MT * COLS;  // accumulator registers per lane: 32 channels x MT token tiles per column
   constexpr int kChunk = (WAVES <= 8) ? 32 : 16;
+  constexpr int TN = 128 * COLS;     // channels per strip
+  constexpr int WROW = 64 * COLS;    // bytes of a weight row a wave covers
   constexpr float kUnscale = 0x1p-12f;
-  // Weights and activations travel global -> LDS without passing registers: per wave DEPTH slots of
-  // one step's data, [32 rows][64 bytes] of weights and MT tiles of [16 tokens][64 bytes] of
-  // activations.  The same memory later carries the waves' partial tiles to be added.
-  constexpr int kSlot = 2048 + MT * 1024;
+  // Per wave DEPTH slots of one step's data, [32 rows][WROW bytes] of weights and MT tiles of
+  // [16 tokens][64 bytes] of activations.  The same memory later carries the waves' partial tiles.
+  constexpr int kWBytes = 32 * WROW;
+  constexpr int kSlot = kWBytes + MT * 1024;
   constexpr int kRingBytes = WAVES * DEPTH * kSlot, kSumBytes = WAVES * kChunk * 64 * 4;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kRingBytes > kSumBytes ? kRingBytes : kSumBytes];
   float* const lds = (float*)smem;
-  __shared__ uint32_t lds_bad[4];
+  __shared__ uint32_t lds_bad[4 * COLS];
+  __shared__ int lds_partner;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4, q = (lane >> 2) & 3, i = lane & 3;
-  if (threadIdx.x < 4) lds_bad[threadIdx.x] = 0;
+  if (threadIdx.x < 4 * COLS) lds_bad[threadIdx.x] = 0;
+  // Consecutive workgroup ids land on different XCDs (round robin over 8): 128-channel strips are
+  // renumbered so that neighbours, which share cache lines, share an L2.  The two workgroups of a
+  // 256-channel strip keep consecutive ids (they share no lines, and the one that waits must be
+  // dispatched after the one it waits for).
   int bid = blockIdx.x;
-  {
+  if (!p.pair) {
     const int total = gridDim.x;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
   }
@@ -77,6 +88,8 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   const int batch = blockIdx.y;
   const int group = p.group;
   const int groups = p.K / group;
+  // two workgroups per strip that hand over inside the kernel: slice 0 produces, slice 1 finishes
+  const bool producer = p.pair && slice == 0, finisher = p.pair && slice == 1;
 
   const uint32_t pitch = (uint32_t)p.N >> 1;
   const __amdgpu_buffer_rsrc_t rw =
@@ -87,33 +100,29 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
       (const char*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N * 2, (uint32_t)groups * p.N * 2u);
 
   constexpr uint32_t kNowhere = 0x80000000u;
-  const int n_chunk = strip * 128 + 32 * q;  // the lane's 32 channels (N % 32 == 0: all inside or none)
-  const bool lane_live = n_chunk < p.N;
-  const int side = kb / KBG;                                   // which of the SIDE groups
-  const int lane_row = side * group + (kb % KBG) * 8;          // first row of the lane's block in a step
-  // Loading side: lane l fetches 16 bytes of row (l >> 2) of a 16-row half step, chunk l & 3, so four
-  // neighbouring lanes read 64 contiguous bytes; row R = 8 * kb' + r of a step is row r of block kb'.
-  // The data of lane l lands at slot + 16 * l: the slot is a row-major [32 rows][64 bytes] tile.
-  uint32_t voff_w[2];
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int Rr = 16 * half + (lane >> 2), kbl = Rr >> 3;
-    const int row = (kbl / KBG) * group + (kbl % KBG) * 8 + (Rr & 7);
-    const int nl = strip * 128 + 32 * (lane & 3);
-    voff_w[half] = nl < p.N ? (uint32_t)row * pitch + (uint32_t)(nl >> 1) : kNowhere;
-  }
+  // Loading side: LPR lanes cover one row (16 bytes each), so a load instruction takes 64 / LPR whole
+  // rows of WROW contiguous bytes; lane l deposits at slot + 16 * l: the slot is a row-major
+  // [32 rows][WROW bytes] tile.  32-channel pieces beyond N (N % 32 == 0) read as zeros.
+  constexpr int LPR = 4 * COLS, RPI = 64 / LPR, NLD = 32 / RPI;
+  const uint32_t voff_w = strip * TN + 32 * (lane % LPR) < p.N
+                              ? (uint32_t)(lane / LPR) * pitch + (uint32_t)((strip * TN + 32 * (lane % LPR)) >> 1)
+                              : kNowhere;
   uint8_t* const my_ring = smem + wave * (DEPTH * kSlot);
-  // Reading side: rows 8 * kb + i and 8 * kb + i + 4, chunk q
-  const uint32_t rd_off = (uint32_t)(64 * (8 * kb + i) + 16 * q);
-  // activations, loading side: lane l fetches 16 bytes (8 rows) of token l >> 2 for the block kb' = l & 3
-  // and deposits them at 16 * l; reading side: token li, block kb
-  const uint32_t voff_a =
-      ((uint32_t)(lane >> 2) * p.K + (uint32_t)(((lane & 3) / KBG) * group + ((lane & 3) % KBG) * 8)) * 2u;
+  // Consuming side: rows 8 * kb + i and 8 * kb + i + 4, column c, piece q
+  const uint32_t rd_off = (uint32_t)(WROW * (8 * kb + i) + 16 * q);
+  // activations, loading side: lane l fetches 16 bytes (8 rows) of token l >> 2 for the block l & 3
+  // and deposits them at 16 * l; consuming side: token li, block kb
+  const uint32_t voff_a = ((uint32_t)(lane >> 2) * p.K + (uint32_t)((lane & 3) * 8)) * 2u;
   const uint32_t rd_off_a = (uint32_t)(64 * li + 16 * kb);
-  // as column j = i of B and D the lane stands for channels n_chunk + 8d + sm + h, sm = (0,4,2,6)[i];
-  // one dword of a scales row holds the pair h = 0, 1
+  // as column j = i of B and D the lane stands for channels 128c + 32q + 8d + sm + h of the strip,
+  // sm = (0,4,2,6)[i]; one dword of a scales row holds the pair h = 0, 1
   const int sm = (i & 1) * 4 + (i >> 1) * 2;
-  const uint32_t voff_s = lane_live ? ((uint32_t)side * p.N + (uint32_t)(n_chunk + sm)) * 2u : kNowhere;
+  uint32_t voff_s[COLS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) {
+    const int n = strip * TN + 128 * c + 32 * q;
+    voff_s[c] = n < p.N ? (uint32_t)(n + sm) * 2u : kNowhere;
+  }
   // byte selectors that put a 16-bit scale where s_j sits in column j = i of B (0x0c selects zero):
   // sel[h][r]: register r of the column, taking the low (h = 0) or high (h = 1) half of the source
   const uint32_t pos = (i & 1) ? 0x01000c0cu : 0x0c0c0100u;   // value in the high / low half
@@ -121,108 +130,124 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   const uint32_t sel10 = sel00 == 0x0c0c0c0cu ? sel00 : sel00 + ((i & 1) ? 0x02020000u : 0x00000202u);
   const uint32_t sel11 = sel01 == 0x0c0c0c0cu ? sel01 : sel01 + ((i & 1) ? 0x02020000u : 0x00000202u);
 
-  floatx4 acc[4][2][MT];
+  floatx4 acc[COLS][4][2][MT];
 #pragma unroll
-  for (int d = 0; d < 4; ++d)
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[d][h][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  // this wave's units (SIDE groups of rows each)
-  const int macro = SIDE * group;
-  const int spg = group / (8 * KBG);  // steps per unit, a multiple of DEPTH
-  const int units = p.rows_per_slice / macro;
-  const int cls = wave >> 2;
-  int first = (wave & 3) * p.units_per_simd;
-#pragma unroll
-  for (int c = 0; c < (WAVES + 3) / 4; ++c)
-    if (c < cls) first += p.class_units[c];
-  int cnt = min(first + p.class_units[cls], units) - first;
-  const int k_begin = slice * p.rows_per_slice + first * macro;
-  if (k_begin >= p.K) cnt = 0;
-
-  uint32_t sraw[4];
-  halfx4 Bm[4][2];
-  floatx4 Cm[4][2];
-  uint32_t bad = 0;
-
-  auto load_scales = [&](int km) {  // groups km / group + side of the lane's four channel pairs
-    const uint32_t vs = voff_s + (uint32_t)(km / group) * (uint32_t)p.N * 2u;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) sraw[d] = __builtin_amdgcn_raw_buffer_load_b32(rs, vs + 16u * d, 0, 0);
-  };
-  auto load_step = [&](int buf, int row) {  // row: first row of the step in the first of the SIDE groups
-    uint8_t* const slot = my_ring + buf * kSlot;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(uintptr_t)(slot + 2048 + mt * 1024), 16,
-                                               voff_a + (uint32_t)(row + 16 * mt * p.K) * 2u, 0, 0, 0);
-    const uint32_t rp = (uint32_t)row * pitch;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(uintptr_t)slot, 16, voff_w[0] + rp, 0, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(uintptr_t)(slot + 1024), 16, voff_w[1] + rp, 0, 0, 0);
-  };
-  // B and C of the eight channels the lane stands for, from sraw
-  auto prepare = [&]() {
-    const halfx4 off0 = {(_Float16)-1032.0f, (_Float16)-1032.0f, (_Float16)-1032.0f, (_Float16)-1032.0f};
-    const halfx4 off1 = {(_Float16)-1152.0f, (_Float16)-1152.0f, (_Float16)-1152.0f, (_Float16)-1152.0f};
-    // all eight exponents in [105, 129] (2^-22 <= |s| < 8)?  Both halves of a dword at once, in
-    // unsigned 16-bit lanes: |bits| - (105 << 7) wraps below the window and exceeds 25 << 7 above it
-    ushortx2 worst = {0, 0};
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const ushortx2 ax = __builtin_bit_cast(ushortx2, sraw[d] & 0x7fff7fffu);
-      worst = __builtin_elementwise_max(worst, (ushortx2)(ax - (ushortx2){105u << 7, 105u << 7}));
-    }
-    const bool fast = __builtin_amdgcn_ballot_w64(max(worst[0], worst[1]) >= (25u << 7)) == 0;  // wave-uniform
-    if (fast) {
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        // bf16 (8 exponent, 7 mantissa bits) -> f16 (5, 10) times 2^12 (low half) | 2^8 (high half):
-        // shift the fields up by three and re-bias the exponent by 100 | 104, in 16-bit lanes (the six
-        // exponent bits that survive the shift are enough inside the window)
-        const uint32_t x = sraw[d];
-        const ushortx2 ax = __builtin_bit_cast(ushortx2, x & 0x7fff7fffu);
-        const ushortx2 t = (ushortx2)((ushortx2)(ax << (ushortx2){3, 3}) - (ushortx2){(uint16_t)(100u << 10), (uint16_t)(104u << 10)});
-        const uint32_t pair = __builtin_bit_cast(uint32_t, t) | (x & 0x80008000u);
-        Bm[d][0] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel00), __builtin_amdgcn_perm(pair, pair, sel01)});
-        Bm[d][1] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel10), __builtin_amdgcn_perm(pair, pair, sel11)});
-      }
-    } else {
-      asm volatile("");
-#pragma unroll
-      for (int d = 0; d < 4; ++d)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const float s = h ? bf16hi_to_f32(sraw[d]) : bf16lo_to_f32(sraw[d]);
-          const float a = __builtin_fabsf(s);
-          const bool ok = (a >= 0x1p-22f && a < 8.0f) || a == 0.0f;
-          if (!ok) bad |= 1u << (2 * d + h);
-          const float sv = ok ? s * (h ? 256.0f : 4096.0f) : 0.0f;
-          const uint32_t pair = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sv, sv));
-          Bm[d][h] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel00), __builtin_amdgcn_perm(pair, pair, sel01)});
-        }
-    }
+  for (int c = 0; c < COLS; ++c)
 #pragma unroll
     for (int d = 0; d < 4; ++d)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        Cm[d][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(h ? off1 : off0, Bm[d][h], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[c][d][h][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // this wave's units (one scale group of rows each).  The producer of a pair takes fewer rows than
+  // the finisher (rows_first against the rest), so that its sums are on their way while the finisher
+  // still streams; class_units[2..3] and units_per_simd2 describe the finisher's split then.
+  const int spg = group >> 5;  // steps per unit, a multiple of DEPTH
+  const int slice_begin = finisher ? p.rows_first : slice * p.rows_per_slice;
+  const int slice_rows = producer ? p.rows_first : p.rows_per_slice;
+  const int units = slice_rows / group;
+  const int cls = wave >> 2;
+  const int ups = finisher ? p.units_per_simd2 : p.units_per_simd;
+  const int cu0 = finisher ? p.class_units[2] : p.class_units[0];
+  const int cu1 = finisher ? p.class_units[3] : p.class_units[1];
+  const int first = (wave & 3) * ups + (cls ? cu0 : 0);
+  int cnt = min(first + (cls ? cu1 : cu0), units) - first;
+  const int k_begin = slice_begin + first * group;
+  if (k_begin >= p.K) cnt = 0;
+
+  uint32_t sraw[COLS][4];
+  halfx4 Bm[COLS][4][2];
+  floatx4 Cm[COLS][4][2];
+  uint32_t bad = 0;
+
+  auto load_scales = [&](int km) {  // group km / group of the lane's channel pairs
+    const uint32_t vs = (uint32_t)(km / group) * (uint32_t)p.N * 2u;
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) sraw[c][d] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_s[c] + vs + 16u * d, 0, 0);
+  };
+  auto load_step = [&](int buf, int row) {  // row: first row of the step
+    uint8_t* const slot = my_ring + buf * kSlot;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(uintptr_t)(slot + kWBytes + mt * 1024), 16,
+                                               voff_a + (uint32_t)(row + 16 * mt * p.K) * 2u, 0, 0, 0);
+    // (the offsets are spelled out rather than kept in an array indexed by j: with such an argument
+    // to this builtin inside a lambda the compiler's host pass drops the kernel's launch stub)
+    const uint32_t rp = (uint32_t)row * pitch;
+#pragma unroll
+    for (int j = 0; j < NLD; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(uintptr_t)(slot + 1024 * j), 16,
+                                               voff_w + rp + (uint32_t)(RPI * j) * pitch, 0, 0, 0);
+  };
+  // B and C of the channels the lane stands for, from sraw
+  auto prepare = [&]() {
+    const halfx4 off0 = {(_Float16)-1032.0f, (_Float16)-1032.0f, (_Float16)-1032.0f, (_Float16)-1032.0f};
+    const halfx4 off1 = {(_Float16)-1152.0f, (_Float16)-1152.0f, (_Float16)-1152.0f, (_Float16)-1152.0f};
+    // all exponents in [105, 129] (2^-22 <= |s| < 8)?  Both halves of a dword at once, in
+    // unsigned 16-bit lanes: |bits| - (105 << 7) wraps below the window and exceeds 25 << 7 above it
+    ushortx2 worst = {0, 0};
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const ushortx2 ax = __builtin_bit_cast(ushortx2, sraw[c][d] & 0x7fff7fffu);
+        worst = __builtin_elementwise_max(worst, (ushortx2)(ax - (ushortx2){105u << 7, 105u << 7}));
+      }
+    const bool fast = __builtin_amdgcn_ballot_w64(max(worst[0], worst[1]) >= (25u << 7)) == 0;  // wave-uniform
+    if (fast) {
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          // bf16 (8 exponent, 7 mantissa bits) -> f16 (5, 10) times 2^12 (low half) | 2^8 (high half):
+          // shift the fields up by three and re-bias the exponent by 100 | 104, in 16-bit lanes (the six
+          // exponent bits that survive the shift are enough inside the window)
+          const uint32_t x = sraw[c][d];
+          const ushortx2 ax = __builtin_bit_cast(ushortx2, x & 0x7fff7fffu);
+          const ushortx2 t = (ushortx2)((ushortx2)(ax << (ushortx2){3, 3}) - (ushortx2){(uint16_t)(100u << 10), (uint16_t)(104u << 10)});
+          const uint32_t pair = __builtin_bit_cast(uint32_t, t) | (x & 0x80008000u);
+          Bm[c][d][0] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel00), __builtin_amdgcn_perm(pair, pair, sel01)});
+          Bm[c][d][1] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel10), __builtin_amdgcn_perm(pair, pair, sel11)});
+        }
+    } else {
+      asm volatile("");
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const float s = h ? bf16hi_to_f32(sraw[c][d]) : bf16lo_to_f32(sraw[c][d]);
+            const float a = __builtin_fabsf(s);
+            const bool ok = (a >= 0x1p-22f && a < 8.0f) || a == 0.0f;
+            if (!ok) bad |= 1u << (8 * c + 2 * d + h);
+            const float sv = ok ? s * (h ? 256.0f : 4096.0f) : 0.0f;
+            const uint32_t pair = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sv, sv));
+            Bm[c][d][h] = __builtin_bit_cast(halfx4, uintx2{__builtin_amdgcn_perm(pair, pair, sel00), __builtin_amdgcn_perm(pair, pair, sel01)});
+          }
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          Cm[c][d][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(h ? off1 : off0, Bm[c][d][h], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
   };
   auto compute = [&](int buf, int row) {
     // the step's data has landed once at most the loads of the DEPTH - 1 later steps are outstanding
     // (loads complete in order; the scale loads in between only make this wait longer)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (MT + 2)) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (MT + NLD)) : "memory");
     const uint8_t* const slot = my_ring + buf * kSlot;
     uintx4 av[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) av[mt] = *(const uintx4*)(slot + 2048 + mt * 1024 + rd_off_a);
-    uintx4 wq[2];
-    wq[0] = *(const uintx4*)(slot + rd_off);
-    wq[1] = *(const uintx4*)(slot + rd_off + 256);
-    if (row + (SIDE - 1) * group + 8 * KBG > p.K) {  // scalar: only a step that reaches the end of K
+    for (int mt = 0; mt < MT; ++mt) av[mt] = *(const uintx4*)(slot + kWBytes + mt * 1024 + rd_off_a);
+    if (row + 32 > p.K) {  // scalar: only a step that reaches the end of K
       asm volatile("");
-      const bool ok = row + lane_row < p.K;
+      const bool ok = row + 8 * kb < p.K;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
         av[mt] = uintx4{ok ? av[mt][0] : 0u, ok ? av[mt][1] : 0u, ok ? av[mt][2] : 0u, ok ? av[mt][3] : 0u};
@@ -231,50 +256,54 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) bop[mt] = __builtin_bit_cast(bf16x8, av[mt]);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      floatx4 D[2][2];
+    for (int c = 0; c < COLS; ++c) {
+      uintx4 wq[2];
+      wq[0] = *(const uintx4*)(slot + rd_off + 64 * c);
+      wq[1] = *(const uintx4*)(slot + rd_off + 64 * c + 4 * WROW);
 #pragma unroll
-      for (int rho = 0; rho < 2; ++rho) {
-        const uint32_t x = wq[rho][d];
-        const uint32_t y = x >> 8;
-        // nibbles (0,4), (2,6) as 1024 + u; (1,5), (3,7) as 1024 + 16u
-        const uint32_t p0 = __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a);
-        const uint32_t p1 = __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a);
-        const uint32_t p2 = __builtin_amdgcn_bitop3_b32(y, 0x000f000fu, 0x64086408u, 0x6a);
-        const uint32_t p3 = __builtin_amdgcn_bitop3_b32(y, 0x00f000f0u, 0x64806480u, 0x6a);
-        D[0][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p0, p2}), Bm[d][0], Cm[d][0], 0, 0, 0);
-        D[1][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p1, p3}), Bm[d][1], Cm[d][1], 0, 0, 0);
-      }
+      for (int d = 0; d < 4; ++d) {
+        floatx4 D[2][2];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uintx4 a = {pack_bf16x2(D[h][0][0], D[h][0][1]), pack_bf16x2(D[h][0][2], D[h][0][3]),
-                          pack_bf16x2(D[h][1][0], D[h][1][1]), pack_bf16x2(D[h][1][2], D[h][1][3])};
-        const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+        for (int rho = 0; rho < 2; ++rho) {
+          const uint32_t x = wq[rho][d];
+          const uint32_t y = x >> 8;
+          // nibbles (0,4), (2,6) as 1024 + u; (1,5), (3,7) as 1024 + 16u
+          const uint32_t p0 = __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a);
+          const uint32_t p1 = __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a);
+          const uint32_t p2 = __builtin_amdgcn_bitop3_b32(y, 0x000f000fu, 0x64086408u, 0x6a);
+          const uint32_t p3 = __builtin_amdgcn_bitop3_b32(y, 0x00f000f0u, 0x64806480u, 0x6a);
+          D[0][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p0, p2}), Bm[c][d][0], Cm[c][d][0], 0, 0, 0);
+          D[1][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p1, p3}), Bm[c][d][1], Cm[c][d][1], 0, 0, 0);
+        }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[d][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[d][h][mt], 0, 0, 0);
+        for (int h = 0; h < 2; ++h) {
+          const uintx4 a = {pack_bf16x2(D[h][0][0], D[h][0][1]), pack_bf16x2(D[h][0][2], D[h][0][3]),
+                            pack_bf16x2(D[h][1][0], D[h][1][1]), pack_bf16x2(D[h][1][2], D[h][1][3])};
+          const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[c][d][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[c][d][h][mt], 0, 0, 0);
+        }
       }
     }
   };
 
   if (cnt > 0) {
-    // first row of step t of the unit at km; steps past the unit's last run on into the next unit
-    auto step_row = [&](int km, int t) { return t < spg ? km + 8 * KBG * t : km + macro + 8 * KBG * (t - spg); };
     load_scales(k_begin);
 #pragma unroll
-    for (int j = 0; j < DEPTH - 1; ++j) load_step(j, step_row(k_begin, j));
+    for (int j = 0; j < DEPTH - 1; ++j) load_step(j, k_begin + 32 * j);
     for (int u = 0; u < cnt; ++u) {
-      const int km = k_begin + u * macro;
+      const int km = k_begin + u * group;
       prepare();
-      load_scales(km + macro);  // past the last group the loads return zeros
+      load_scales(km + group);  // past the last group the loads return zeros
       // at least one round: the scale loads just issued are then known to be DEPTH steps of
       // loads old when the next unit waits for them, and that wait leaves the steps in flight alone
       int t = 0;
       do {
 #pragma unroll
         for (int j = 0; j < DEPTH; ++j) {
-          load_step((j + DEPTH - 1) % DEPTH, step_row(km, t + j + DEPTH - 1));
-          compute(j, km + 8 * KBG * (t + j));
+          load_step((j + DEPTH - 1) % DEPTH, km + 32 * (t + j + DEPTH - 1));
+          compute(j, km + 32 * (t + j));
         }
         t += DEPTH;
       } while (t < spg);
@@ -282,30 +311,34 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   }
   if (bad) {  // rare: channels whose scale does not fit the f16 operand
 #pragma unroll
-    for (int d = 0; d < 4; ++d)
+    for (int c = 0; c < COLS; ++c)
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-        if (bad & (1u << (2 * d + h))) {
-          const int ch = 32 * q + 8 * d + sm + h;
-          atomicOr(&lds_bad[ch >> 5], 1u << (ch & 31));
-        }
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          if (bad & (1u << (8 * c + 2 * d + h))) {
+            const int ch = 128 * c + 32 * q + 8 * d + sm + h;
+            atomicOr(&lds_bad[ch >> 5], 1u << (ch & 31));
+          }
   }
 
   // loads for steps past the wave's last may still be on their way into the ring
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();  // every wave is done with its ring: the memory now carries the partial tiles
-  // ---- add the waves' tiles through LDS.  Register r = mt * 32 + c holds channel
-  // strip * 128 + 32 * (lane >> 4) + c, token 16 * mt + (lane & 15): a lane owns 32 consecutive
-  // channels.  In the MFMA tiles c = 8d + e sits in acc[d][e & 1][mt][v], v = 2 * ((e >> 1) & 1) + (e >> 2).
+  // ---- add the waves' tiles through LDS.  Register r = (c * MT + mt) * 32 + e32 holds channel
+  // strip * TN + 128 * c + 32 * (lane >> 4) + e32, token 16 * mt + (lane & 15): a lane owns 32
+  // consecutive channels per column.  In the MFMA tiles e32 = 8d + e sits in
+  // acc[c][d][e & 1][mt][v], v = 2 * ((e >> 1) & 1) + (e >> 2).
   constexpr int RPW = kChunk / WAVES;
   constexpr int PASSES = R / kChunk;
   static_assert(R % kChunk == 0 && kChunk % WAVES == 0 && 32 % RPW == 0, "reduction split");
+  const bool finishes = p.slices == 1 || finisher;  // this workgroup applies the epilogue and writes the result
   float bq[PASSES * RPW], res[PASSES * RPW];
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
     const int r0 = pass * kChunk + wave * RPW;
-    const int n0 = strip * 128 + 32 * kb + r0 % 32;
-    const bool live = p.slices == 1 && n0 < p.N;
+    const int n0 = strip * TN + 128 * (r0 / (32 * MT)) + 32 * kb + r0 % 32;
+    const bool live = finishes && n0 < p.N;
 #pragma unroll
     for (int u = 0; u < RPW; ++u)
       bq[pass * RPW + u] = live && p.bias ? load_scale(p.bias, n0 + u, p.bias_is_bf16) : 0.0f;
@@ -313,10 +346,10 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
 #pragma unroll
-    for (int c = 0; c < kChunk; ++c) {
-      const int r = pass * kChunk + c;
-      const int mt = r / 32, ch = r % 32, d = ch / 8, e = ch % 8;
-      lds[(wave * kChunk + c) * 64 + lane] = acc[d][e & 1][mt][2 * ((e >> 1) & 1) + (e >> 2)];
+    for (int cc = 0; cc < kChunk; ++cc) {
+      const int r = pass * kChunk + cc;
+      const int c = r / (32 * MT), mt = (r / 32) % MT, ch = r % 32, d = ch / 8, e = ch % 8;
+      lds[(wave * kChunk + cc) * 64 + lane] = acc[c][d][e & 1][mt][2 * ((e >> 1) & 1) + (e >> 2)];
     }
     __syncthreads();
 #pragma unroll
@@ -328,14 +361,54 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     }
     if (pass + 1 < PASSES) __syncthreads();
   }
-  if (p.slices == 1) epilogue_all_dispatch<PASSES * RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
+
+  // ---- hand-over between the two workgroups of a strip.  The producer's sums and the flag go out
+  // as device-scope stores, the finisher reads them with device-scope loads: no cache maintenance.
+  // The producer has the lower workgroup id of the two, so it was dispatched first and never waits
+  // for anything; should the flag still not show after a long bounded wait, the finisher computes
+  // the whole strip by the plain loop below instead.
+  // The sums travel in the threads' own order -- [pass][wave][lane][RPW floats], 64 KiB... per strip
+  // R * 64 floats -- so that every wave stores and loads 64 x 16 contiguous bytes.
+  static_assert(RPW == 4 || COLS == 1, "the hand-over moves 16 bytes per lane and pass");
+  const __amdgpu_buffer_rsrc_t rh = make_rsrc(p.workspace + ((size_t)batch * p.strips + strip) * (R * 64), R * 64 * 4);
+  constexpr int kDeviceScope = 16;  // sc1: the access is performed where every XCD sees it
+  unsigned long long* const flag = p.flags + (size_t)batch * p.strips + strip;
+  bool partner_ok = true;
+  if (finisher) {
+    if (threadIdx.x == 0) {
+      int ok = 0;
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) { ok = 1; break; }
+        __builtin_amdgcn_s_sleep(8);
+      }
+      lds_partner = ok;
+    }
+    __syncthreads();
+    partner_ok = lds_partner != 0;
+    if (partner_ok) {
+      uintx4 other[PASSES];
+#pragma unroll
+      for (int pass = 0; pass < PASSES; ++pass)
+        other[pass] = __builtin_amdgcn_raw_buffer_load_b128(rh, (uint32_t)(((pass * WAVES + wave) * 64 + lane) * 16), 0, kDeviceScope);
+#pragma unroll
+      for (int pass = 0; pass < PASSES; ++pass)
+#pragma unroll
+        for (int u = 0; u < RPW; ++u) res[pass * RPW + u] = bits_to_f32(other[pass][u]) + res[pass * RPW + u];
+    }
+  }
+  if (finishes) epilogue_all_dispatch<PASSES * RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
     const int r0 = pass * kChunk + wave * RPW;
-    const int m = (r0 / 32) * 16 + li;
-    const int n0 = strip * 128 + 32 * kb + r0 % 32;
+    const int m = ((r0 / 32) % MT) * 16 + li;
+    const int n0 = strip * TN + 128 * (r0 / (32 * MT)) + 32 * kb + r0 % 32;
     if (m >= p.M || n0 >= p.N) continue;
-    if (p.slices > 1) {
+    if (producer) {
+      if constexpr (RPW == 4)
+        __builtin_amdgcn_raw_buffer_store_b128(uintx4{f32_to_bits(res[pass * RPW]), f32_to_bits(res[pass * RPW + 1]),
+                                                      f32_to_bits(res[pass * RPW + 2]), f32_to_bits(res[pass * RPW + 3])},
+                                               rh, (uint32_t)(((pass * WAVES + wave) * 64 + lane) * 16), 0, kDeviceScope);
+    } else if (!finishes) {
       float* dst = p.workspace + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = res[pass * RPW + u];
@@ -346,106 +419,177 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     }
   }
 
-  // ---- flagged channels: the whole wave recomputes each (token, channel) over the slice's rows with
-  // ordinary arithmetic, in a fixed order, and overwrites what the loop above produced for it
+  // ---- flagged channels (or, after a failed hand-over, every channel): the whole wave recomputes
+  // each (token, channel) over the rows with ordinary arithmetic, in a fixed order, and overwrites
+  // what the loop above produced for it.  The stores above must have landed first.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if ((lds_bad[0] | lds_bad[1] | lds_bad[2] | lds_bad[3]) == 0) return;
-  const int ks = slice * p.rows_per_slice, ke = min(ks + p.rows_per_slice, p.K);
-  const uint16_t* sc16 = (const uint16_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N;
-  const uint8_t* wb = p.w + (p.weights_shared ? (size_t)0 : (size_t)batch * p.K * pitch);
-  for (int ch = wave; ch < 128; ch += WAVES) {
-    const int n = strip * 128 + ch;
-    if (!((lds_bad[ch >> 5] >> (ch & 31)) & 1u) || n >= p.N) continue;
-    for (int m = 0; m < p.M; ++m) {
-      const uint16_t* arow = p.lhs + ((size_t)batch * p.M + m) * p.K;
-      float v = 0.0f;
-      for (int k = ks + lane; k < ke; k += 64) {
-        const uint32_t nib = (wb[(size_t)k * pitch + (n >> 1)] >> (4 * (n & 1))) & 0xfu;
-        const float wv = round_bf16((float)((int)(nib ^ 8u) - 8) * bf16_to_f32(sc16[(size_t)(k / group) * p.N + n]));
-        v = v + bf16_to_f32(arow[k]) * wv;
-      }
+  uint32_t any_bad = partner_ok ? 0u : 1u;
 #pragma unroll
-      for (int sh = 32; sh >= 1; sh >>= 1) v = v + __shfl_xor(v, sh);
-      if (lane != 0) continue;
-      if (p.slices > 1) {
-        p.workspace[(((size_t)batch * p.slices + slice) * p.M + m) * p.N + n] = v;
-      } else {
-        const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-        p.out[((size_t)batch * p.M + m) * p.N + n] = f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  for (int c = 0; c < 4 * COLS; ++c) any_bad |= lds_bad[c];
+  if (any_bad) {
+    const int ks = partner_ok ? slice_begin : 0;
+    const int ke = partner_ok ? min(ks + slice_rows, p.K) : p.K;
+    const uint16_t* sc16 = (const uint16_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N;
+    const uint8_t* wb = p.w + (p.weights_shared ? (size_t)0 : (size_t)batch * p.K * pitch);
+    for (int ch = wave; ch < TN; ch += WAVES) {
+      const int n = strip * TN + ch;
+      if ((partner_ok && !((lds_bad[ch >> 5] >> (ch & 31)) & 1u)) || n >= p.N) continue;
+      for (int m = 0; m < p.M; ++m) {
+        const uint16_t* arow = p.lhs + ((size_t)batch * p.M + m) * p.K;
+        float v = 0.0f;
+        for (int k = ks + lane; k < ke; k += 64) {
+          const uint32_t nib = (wb[(size_t)k * pitch + (n >> 1)] >> (4 * (n & 1))) & 0xfu;
+          const float wv = round_bf16((float)((int)(nib ^ 8u) - 8) * bf16_to_f32(sc16[(size_t)(k / group) * p.N + n]));
+          v = v + bf16_to_f32(arow[k]) * wv;
+        }
+#pragma unroll
+        for (int sh = 32; sh >= 1; sh >>= 1) v = v + __shfl_xor(v, sh);
+        if (lane != 0) continue;
+        // where the thread that owns (m, n) keeps it in the hand-over buffer
+        const int hr = ((ch >> 7) * MT + (m >> 4)) * 32 + (ch & 31);
+        float* const hslot = p.workspace + ((size_t)batch * p.strips + strip) * (R * 64) +
+                             (((hr / kChunk) * WAVES + (hr % kChunk) / RPW) * 64 + 16 * ((ch & 127) >> 5) + (m & 15)) * RPW +
+                             (hr % kChunk) % RPW;
+        if (producer) {
+          __hip_atomic_store(hslot, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (!finishes) {
+          p.workspace[(((size_t)batch * p.slices + slice) * p.M + m) * p.N + n] = v;
+        } else {
+          if (finisher && partner_ok) v = __hip_atomic_load(hslot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + v;
+          const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+          p.out[((size_t)batch * p.M + m) * p.N + n] = f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+        }
       }
     }
   }
+  if (p.pair) {
+    // the producer raises the flag once all its sums have landed; the finisher lowers it again so
+    // that a replay of the same launch (a captured graph) waits for the producer's new sums
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+      __hip_atomic_store(flag, producer ? p.epoch : 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
-template <int MT, int WAVES, int SIDE, int DEPTH>
+template <int MT, int WAVES, int COLS, int DEPTH>
 int launch_s4x(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
-  hipLaunchKernelGGL((dequant_dot_decode_s4x_kernel<MT, WAVES, SIDE, DEPTH>), grid, dim3(WAVES * 64), 0, stream, dp);
+  hipLaunchKernelGGL((dequant_dot_decode_s4x_kernel<MT, WAVES, COLS, DEPTH>), grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
   if (rc) return rc;
-  if (dp.slices > 1) rc = LaunchDecodeFinalize(dp, batch, stream, kRounded);
+  if (dp.slices > 1 && !dp.pair) rc = LaunchDecodeFinalize(dp, batch, stream, kRounded);
   SetLastKernel(name);
   return rc;
 }
 
 }  // namespace
 
+// Bytes of workspace the in-kernel hand-over between the two workgroups of a 256-channel strip
+// needs: the producer's f32 sums, 16 KiB per (batch, strip), and one 8-byte flag each.
+size_t S4xPairWorkspaceBytes(int64_t batch, int64_t M, int64_t N) {
+  (void)M;  // the producer's sums travel as whole 16-token tiles: 16 x 256 floats per strip
+  return (size_t)batch * ((N + 255) / 256) * (16 * 256 * 4 + 8);
+}
+
+// Whole 128-byte lines per load and two workgroups per 256-channel strip: up to 16 tokens (the
+// accumulators and scale operands of two columns fill the registers).  Chosen by itself when those
+// workgroups fill most of the machine and every wave gets at least one group of rows; option
+// "dequant_dot_pair" = 1 takes it wherever the shape allows, 2 never.
+bool S4xPairShape(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t group) {
+  const int mode = GetOption("dequant_dot_pair");
+  if (mode == 2 || M < 1 || M > 16 || N % 32 != 0 || group % 64 != 0 || K < 2 * group) return false;
+  if (mode == 1) return true;
+  const int64_t wgs = batch * ((N + 255) / 256) * 2;
+  return K / 2 >= 8 * group && wgs >= 128 && wgs <= 1024;
+}
+
 int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream) {
-  if (p.weight_dtype != XLA_FFI_DataType_S4 || !dp.scale_is_bf16 || p.M > 64 || p.N % 32 != 0 || p.group % 32 != 0)
+  if (p.weight_dtype != XLA_FFI_DataType_S4 || !dp.scale_is_bf16 || p.M > 64 || p.N % 32 != 0 || p.group % 64 != 0)
     return -1;
   const int mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : p.M <= 48 ? 3 : 4;
-  int side = 1;  // groups side by side cost more in scattered activation reads than they save in scale set-up
-  if (int v = GetOption("dequant_dot_side")) side = v;
-  if (side != 1 && side != 2 && side != 4) return -1;
-  while (side < 4 && p.group / (8 * (4 / side)) < 2) side *= 2;  // at least two steps per unit
-  const int macro = side * (int)p.group;
-  const int spg = (int)p.group / (8 * (4 / side));   // steps per unit
+  const int group = (int)p.group;
+  const int spg = group / 32;   // steps per unit
   int depth = 2;  // two steps in the ring measured faster than four at every token count
   if (int v = GetOption("dequant_dot_depth")) depth = v;
-  while (depth > 2 && spg % depth != 0) --depth;
-  if (p.K < macro || spg % depth != 0) return -1;
+  if (mt > 2 && depth > 2) depth = 2;  // 48 and 64 tokens: the ring leaves room for two steps
+  if ((depth != 2 && depth != 4) || p.K < group || spg % depth != 0) return -1;
   const int64_t row_bytes = p.N / 2;
   if ((double)p.K * row_bytes + 1024.0 * row_bytes >= 2147483648.0 || (double)p.M * p.K * 2 >= 2147483648.0 ||
       (double)(p.K / p.group + 8) * p.N * 2 >= 2147483648.0)
     return -1;
   const int waves = 8;
-  dp.strips = (int)((p.N + 127) / 128);
-  // once the strips alone (nearly) fill the CUs, K-slices only add a second launch
-  int slices = dp.strips * p.batch >= 192 && !GetOption("dequant_dot_slices")
-                   ? 1 : DecodeSlices(p.batch, p.M, p.K, p.N, dp.strips, row_bytes, waves);
-  if (slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, slices)))
-    slices = 1;
-  while (slices > 1 && p.K / slices < macro) slices /= 2;
-  dp.slices = slices;
-  const int per = (int)((p.K + slices - 1) / slices);
-  dp.rows_per_slice = (per + macro - 1) / macro * macro;
-  const int units = dp.rows_per_slice / macro;
-  dp.units_per_simd = (units + 3) / 4;
-  // a SIMD serves its older wave first: the older class may take the larger share
+  const int b = (int)p.batch;
+  // a SIMD serves its older wave first: the older class takes the larger share of the rows
   int w0 = 7, w1 = 5;
   if (int v = GetOption("dequant_dot_skew")) { w0 = v / 10 % 10; w1 = v % 10; }
   if (w0 + w1 <= 0) { w0 = 1; w1 = 1; }
-  int u0 = (dp.units_per_simd * w0 + (w0 + w1) / 2) / (w0 + w1);
-  if (u0 > dp.units_per_simd) u0 = dp.units_per_simd;
-  dp.class_units[0] = u0;
-  dp.class_units[1] = dp.units_per_simd - u0;
-  dp.class_units[2] = dp.class_units[3] = 0;
-  const int b = (int)p.batch;
-#define XLA_AMD_S4X(MT_, SIDE_, DEPTH_, NAME) \
-  if (mt == MT_ && side == SIDE_ && depth == DEPTH_) return launch_s4x<MT_, 8, SIDE_, DEPTH_>(dp, b, stream, NAME);
-#define XLA_AMD_S4X_SIDES(MT_, DEPTH_, TOKENS)                                        \
-  XLA_AMD_S4X(MT_, 1, DEPTH_, "dequant_dot_decode_s4x_" TOKENS "_side1_d" #DEPTH_)   \
-  XLA_AMD_S4X(MT_, 2, DEPTH_, "dequant_dot_decode_s4x_" TOKENS "_side2_d" #DEPTH_)   \
-  XLA_AMD_S4X(MT_, 4, DEPTH_, "dequant_dot_decode_s4x_" TOKENS "_side4_d" #DEPTH_)
-  if (mt > 2 && depth > 2) depth = 2;  // 48 and 64 tokens: the accumulators leave room for two steps
-  if (spg % depth != 0) return -1;
-  XLA_AMD_S4X_SIDES(1, 4, "m16")
-  XLA_AMD_S4X_SIDES(1, 2, "m16")
-  XLA_AMD_S4X_SIDES(2, 4, "m32")
-  XLA_AMD_S4X_SIDES(2, 2, "m32")
-  XLA_AMD_S4X_SIDES(3, 2, "m48")
-  XLA_AMD_S4X_SIDES(4, 2, "m64")
-#undef XLA_AMD_S4X_SIDES
+  auto split_rows = [&](int slices) {
+    dp.slices = slices;
+    const int per = (int)((p.K + slices - 1) / slices);
+    dp.rows_per_slice = (per + group - 1) / group * group;
+    const int units = dp.rows_per_slice / group;
+    dp.units_per_simd = (units + 3) / 4;
+    int u0 = (dp.units_per_simd * w0 + (w0 + w1) / 2) / (w0 + w1);
+    if (u0 > dp.units_per_simd) u0 = dp.units_per_simd;
+    dp.class_units[0] = u0;
+    dp.class_units[1] = dp.units_per_simd - u0;
+    dp.class_units[2] = dp.class_units[3] = 0;
+  };
+  dp.pair = 0;
+  dp.flags = nullptr;
+  dp.epoch = 0;
+  dp.rows_first = 0;
+  dp.units_per_simd2 = 0;
+  const bool forced_slices = GetOption("dequant_dot_slices") != 0;
+  if (mt == 1 && depth == 2 && !forced_slices && S4xPairShape(p.batch, p.M, p.K, p.N, p.group) && p.workspace &&
+      ((uintptr_t)p.workspace % 8) == 0 && p.workspace_bytes >= S4xPairWorkspaceBytes(p.batch, p.M, p.N)) {
+    static std::atomic<unsigned long long> counter{0};
+    static const unsigned long long nonce = 0x9e3779b97f4a7c15ull * (unsigned long long)(uintptr_t)&counter ^ 0xd1b54a32d192ed03ull;
+    dp.strips = (int)((p.N + 255) / 256);
+    dp.pair = 1;
+    dp.flags = (unsigned long long*)((char*)p.workspace + (size_t)p.batch * dp.strips * (16 * 256 * 4));
+    dp.epoch = (nonce + 2 * counter.fetch_add(1, std::memory_order_relaxed)) | 1ull;  // never 0
+    // Rows are split evenly ("dequant_dot_share" sets the producer's sixteenths): giving the producer
+    // less, so that its sums are in memory before the finisher asks, measured slower at every token
+    // count -- the finisher's own loop is what the kernel waits for.
+    int share = 8;
+    if (int v = GetOption("dequant_dot_share")) share = v;
+    const int groups_total = (int)((p.K + group - 1) / group);
+    int g0 = (groups_total * share + 8) / 16;
+    if (g0 < 1) g0 = 1;
+    if (g0 > groups_total - 1) g0 = groups_total - 1;
+    auto class_split = [&](int units, int* ups, int* c0, int* c1) {
+      *ups = (units + 3) / 4;
+      int u0 = (*ups * w0 + (w0 + w1) / 2) / (w0 + w1);
+      if (u0 > *ups) u0 = *ups;
+      *c0 = u0;
+      *c1 = *ups - u0;
+    };
+    dp.slices = 2;
+    dp.rows_first = g0 * group;
+    dp.rows_per_slice = (groups_total - g0) * group;   // the finisher's rows (to the end of K, rounded up to a group)
+    class_split(g0, &dp.units_per_simd, &dp.class_units[0], &dp.class_units[1]);
+    class_split(groups_total - g0, &dp.units_per_simd2, &dp.class_units[2], &dp.class_units[3]);
+    return launch_s4x<1, 8, 2, 2>(dp, b, stream, "dequant_dot_decode_s4x_m16_pair");
+  }
+  dp.strips = (int)((p.N + 127) / 128);
+  // once the strips alone (nearly) fill the CUs, K-slices only add a second launch
+  int slices = dp.strips * p.batch >= 192 && !forced_slices
+                   ? 1 : DecodeSlices(p.batch, p.M, p.K, p.N, dp.strips, row_bytes, waves);
+  if (slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, slices)))
+    slices = 1;
+  while (slices > 1 && p.K / slices < group) slices /= 2;
+  split_rows(slices);
+#define XLA_AMD_S4X(MT_, DEPTH_, NAME) \
+  if (mt == MT_ && depth == DEPTH_) return launch_s4x<MT_, 8, 1, DEPTH_>(dp, b, stream, NAME);
+  XLA_AMD_S4X(1, 2, "dequant_dot_decode_s4x_m16_d2")
+  XLA_AMD_S4X(1, 4, "dequant_dot_decode_s4x_m16_d4")
+  XLA_AMD_S4X(2, 2, "dequant_dot_decode_s4x_m32_d2")
+  XLA_AMD_S4X(2, 4, "dequant_dot_decode_s4x_m32_d4")
+  XLA_AMD_S4X(3, 2, "dequant_dot_decode_s4x_m48_d2")
+  XLA_AMD_S4X(4, 2, "dequant_dot_decode_s4x_m64_d2")
 #undef XLA_AMD_S4X
   return -1;
 }
