@@ -77,6 +77,19 @@ def evaluate(module_json, args):
         root = next(i for i in body["instructions"] if i["root"])
         return root["opcode"]
 
+    by_name = {i["name"]: i for i in entry["instructions"]}
+    uses = {}
+    for i in entry["instructions"]:
+        for o in i["operands"]:
+            uses[o] = uses.get(o, 0) + 1
+
+    def contracted_product(add):
+        for k, o in enumerate(add["operands"]):
+            m = by_name[o]
+            if m["opcode"] == "multiply" and m["shape"].get("dtype") == "f32" and uses[o] == 1 and not m["root"]:
+                return k
+        return None
+
     for ins in entry["instructions"]:
         op, sh = ins["opcode"], ins["shape"]
         ty = sh.get("dtype")
@@ -113,6 +126,12 @@ def evaluate(module_json, args):
             v = np.broadcast_to(np.reshape(x[0], shape), sh["dims"])
         elif op in ("reshape", "bitcast"):
             v = np.reshape(x[0], sh["dims"])
+        elif op == "add" and ty == "f32" and contracted_product(ins) is not None:
+            # an f32 multiply whose only user is this f32 add: one fused kernel on the CPU backend,
+            # whose LLVM may contract the pair (cpu_aot_loader.cc:49-55) -- O.mul_add_f32 decides
+            k = contracted_product(ins)
+            m = by_name[ins["operands"][k]]
+            v = O.mul_add_f32(env[m["operands"][0]], env[m["operands"][1]], x[1 - k])
         elif op in ("multiply", "add", "subtract", "divide", "maximum", "minimum"):
             a, b = np.asarray(x[0], np.float32), np.asarray(x[1], np.float32)
             with np.errstate(all="ignore"):

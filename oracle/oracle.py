@@ -59,6 +59,12 @@ def lib():
         L.xo_tanh_f32.argtypes = [f32]
         L.xo_exp_f32.restype = f32
         L.xo_exp_f32.argtypes = [f32]
+        L.xo_mul_add_f32_n.restype = None
+        L.xo_mul_add_f32_n.argtypes = [vp, vp, vp, c.c_size_t, vp]
+        L.xo_set_fp_contract.restype = None
+        L.xo_set_fp_contract.argtypes = [i32]
+        L.xo_get_fp_contract.restype = i32
+        L.xo_get_fp_contract.argtypes = []
         for name in ("xo_pack_s4", "xo_unpack_s4", "xo_unpack_u4", "xo_f32_to_bf16_n",
                      "xo_f32_to_f8e4m3fn_n", "xo_f8e4m3fn_to_f32_n", "xo_tanh_f32_n",
                      "xo_exp_f32_n"):
@@ -145,6 +151,31 @@ def unpack_u4(b, n):
     b = _c(b, np.uint8).reshape(-1)
     out = np.empty(n, np.uint8)
     lib().xo_unpack_u4(_ptr(b), n, _ptr(out))
+    return out
+
+
+class fp_contract:
+    """`with fp_contract(False):` -- the f32 polynomials and the f32-typed GELU with every multiply
+    and add rounded separately (a host without fma); the default fuses them, as the reference's
+    CPU backend does wherever the host has the instruction (cpu_aot_loader.cc:49-55)."""
+
+    def __init__(self, on):
+        self.on = int(bool(on))
+
+    def __enter__(self):
+        self.before = lib().xo_get_fp_contract()
+        lib().xo_set_fp_contract(self.on)
+
+    def __exit__(self, *exc):
+        lib().xo_set_fp_contract(self.before)
+
+
+def mul_add_f32(a, b, c):
+    """a * b + c elementwise with the rounding of one f32 kernel: fused when fp_contract is on."""
+    a, b, c = np.broadcast_arrays(np.asarray(a, np.float32), np.asarray(b, np.float32), np.asarray(c, np.float32))
+    a, b, c = _c(a, np.float32), _c(b, np.float32), _c(c, np.float32)
+    out = np.empty_like(a)
+    lib().xo_mul_add_f32_n(_ptr(a), _ptr(b), _ptr(c), a.size, _ptr(out))
     return out
 
 

@@ -32,9 +32,11 @@
  *     k (this file adds in increasing k, one rounding per multiply and per add)
  *   - xo_rmsnorm_quantize_fp8: the order of additions inside one 32-wide
  *     window of the sum of squares (this file adds left to right)
- *   - xo_tanh_f32 / xo_exp_f32: whether the host contracts mul+add into fma
- *     (this file does not: it must be compiled with -ffp-contract=off and
- *     without -ffast-math, which also keeps every sum in its written order)
+ *   - xo_tanh_f32 / xo_exp_f32 and the f32-typed GELU: which multiply-add pairs
+ *     the host's LLVM contracts into fma (fusion is allowed there; this file
+ *     fuses exactly the pairs written as mul_add when xo_set_fp_contract(1),
+ *     none when 0; it must be compiled with -ffp-contract=off and without
+ *     -ffast-math so that nothing else fuses or reorders)
  */
 #include <math.h>
 #include <stddef.h>
@@ -190,8 +192,24 @@ XO_API void xo_f8e4m3fn_to_f32_n(const uint8_t* in, size_t n, float* out) {
 
 /* ------------------------------------------------------- transcendental */
 
-/* tanh.cc:48-108 then :33-46.  Separate multiplies and adds (the emitter
- * issues FMul/FAdd); the fma clamp constant is the default on x86 with FMA. */
+/* Multiply feeding an add inside one f32 kernel.  The CPU backend builds its
+ * target machine with fused multiply-add allowed (cpu_aot_loader.cc:49-55,
+ * used from cpu_compiler.cc:1364 and :2200: AllowFPOpFusion = Fast), so on a
+ * host with an fma instruction such a pair is ONE rounding; on a host without
+ * it is two.  xo_set_fp_contract(1) (the default: every x86-64 and aarch64
+ * host of the last decade) gives the first, 0 the second. */
+static int xo_fp_contract = 1;
+XO_API void xo_set_fp_contract(int on) { xo_fp_contract = on != 0; }
+XO_API int xo_get_fp_contract(void) { return xo_fp_contract; }
+static inline float mul_add(float a, float b, float c) {
+  if (xo_fp_contract) return fmaf(a, b, c);
+  volatile float t = a * b;
+  volatile float r = t + c;
+  return r;
+}
+
+/* tanh.cc:48-108 then :33-46.  The emitter issues FMul then FAdd per Horner
+ * step (mul_add above); the fma clamp constant is the default on x86 with FMA. */
 XO_API float xo_tanh_f32(float x) {
   const float plus_clamp = 7.99881172180175781f;
   static const float num[7] = {-2.76076847742355e-16f, 2.00018790482477e-13f,
@@ -207,17 +225,18 @@ XO_API float xo_tanh_f32(float x) {
   if (!(xc <= plus_clamp)) xc = plus_clamp;
   if (x != x) xc = x;
   volatile float x2 = xc * xc;
-  volatile float p = num[0];
-  for (int i = 1; i < 7; ++i) { volatile float t = x2 * p; p = t + num[i]; }
+  float p = num[0];
+  for (int i = 1; i < 7; ++i) p = mul_add(x2, p, num[i]);
   volatile float n = xc * p;
-  volatile float q = den[0];
-  for (int i = 1; i < 4; ++i) { volatile float t = x2 * q; q = t + den[i]; }
+  float q = den[0];
+  for (int i = 1; i < 4; ++i) q = mul_add(x2, q, den[i]);
   float r = use_approx ? x : (n / q);
   if (ax >= 20.0f) r = copysignf(1.0f, x);
   return r;
 }
 
-/* polynomial_approximations.cc:173-296 (Cephes expf, MulAdd = mul then add). */
+/* polynomial_approximations.cc:173-296 (Cephes expf; its MulAdd is FMul then
+ * FAdd, and in - C1*n is FMul then FSub: all mul_add above). */
 XO_API float xo_exp_f32(float x) {
   const float C1 = 0.693359375f, C2 = -2.12194440e-4f;
   const float p0 = 1.9875691500E-4f, p1 = 1.3981999507E-3f, p2 = 8.3334519073E-3f,
@@ -226,28 +245,28 @@ XO_API float xo_exp_f32(float x) {
   float in = x;
   if (in < -87.8f) in = -87.8f;
   if (in > 88.8f) in = 88.8f;
-  volatile float t0 = in * 1.44269504088896341f;
-  volatile float t1 = t0 + 0.5f;
-  float n = floorf(t1);
+  float n = floorf(mul_add(in, 1.44269504088896341f, 0.5f));
   if (n < -127.0f) n = -127.0f;
   if (n > 127.0f) n = 127.0f;
-  volatile float a = C1 * n;
-  volatile float xr = in - a;
-  volatile float b = C2 * n;
-  xr = xr - b;
-  volatile float z = xr * p0; z = z + p1;
-  z = z * xr; z = z + p2;
-  z = z * xr; z = z + p3;
-  z = z * xr; z = z + p4;
-  z = z * xr; z = z + p5;
+  float xr = mul_add(-C1, n, in);
+  xr = mul_add(-C2, n, xr);
+  float z = mul_add(xr, p0, p1);
+  z = mul_add(z, xr, p2);
+  z = mul_add(z, xr, p3);
+  z = mul_add(z, xr, p4);
+  z = mul_add(z, xr, p5);
   volatile float xx = xr * xr;
-  z = z * xx; z = z + xr;
-  z = 1.0f + z;
+  z = mul_add(z, xx, xr);
+  volatile float z1 = 1.0f + z;
   int32_t ni = (int32_t)n;
   float pow2 = u2f((uint32_t)(ni + 0x7f) << 23);
-  return z * pow2;
+  return z1 * pow2;
 }
 
+/* a[i]*b[i] + c[i] as one elementwise kernel holds it (see mul_add). */
+XO_API void xo_mul_add_f32_n(const float* a, const float* b, const float* c, size_t n, float* out) {
+  for (size_t i = 0; i < n; ++i) out[i] = mul_add(a[i], b[i], c[i]);
+}
 XO_API void xo_tanh_f32_n(const float* in, size_t n, float* out) {
   for (size_t i = 0; i < n; ++i) out[i] = xo_tanh_f32(in[i]);
 }
@@ -283,8 +302,9 @@ static inline float epilogue_value(float acc, int dot_ty, int ep_ty, int has_bia
       float c0 = rnd(0.044715f, ep_ty), c1 = rnd(0.797884583f, ep_ty);
       float m0 = rnd(x * x, ep_ty);
       float m1 = rnd(x * m0, ep_ty);
-      float m2 = rnd(m1 * c0, ep_ty);
-      float a0 = rnd(x + m2, ep_ty);
+      /* f32-typed ops sit in one kernel: m1*c0 feeds only the add (mul_add);
+       * bf16-typed ops round the product to bf16 in between, nothing fuses */
+      float a0 = ep_ty == XO_BF16 ? rnd(x + rnd(m1 * c0, ep_ty), ep_ty) : mul_add(m1, c0, x);
       float m3 = rnd(a0 * c1, ep_ty);
       float th = rnd(xo_tanh_f32(m3), ep_ty);
       float a2 = rnd(th + 1.0f, ep_ty);

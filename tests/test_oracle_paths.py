@@ -41,6 +41,30 @@ def test_exp_matches_libm(oracle):
         oracle.exp_f32(np.array([89.0], np.float32))[0] > 3e38
 
 
+def test_fused_and_separate_roundings_are_both_the_reference(oracle):
+    """The CPU backend may fuse a multiply into the add it feeds (cpu_aot_loader.cc:49-55), so the
+    oracle carries both spellings.  They are different functions (some inputs differ) and both stay
+    within a few f32 ulp of each other and of libm; an fma is never less accurate than the pair."""
+    x = np.linspace(-9, 9, 400001).astype(np.float32)
+    fused_t, fused_e = oracle.tanh_f32(x), oracle.exp_f32(x)
+    with oracle.fp_contract(False):
+        sep_t, sep_e = oracle.tanh_f32(x), oracle.exp_f32(x)
+    assert oracle.lib().xo_get_fp_contract() == 1
+    assert np.any(fused_t != sep_t) and np.any(fused_e != sep_e)
+    assert np.max(np.abs(fused_t.astype(np.float64) - sep_t)) <= 4 * 2.0 ** -23
+    assert np.max(np.abs(fused_e.astype(np.float64) / sep_e - 1)) <= 4 * 2.0 ** -23
+    want_t, want_e = np.tanh(x.astype(np.float64)), np.exp(x.astype(np.float64))
+    assert np.mean(np.abs(fused_t - want_t)) <= np.mean(np.abs(sep_t - want_t)) * 1.02
+    assert np.mean(np.abs(fused_e / want_e - 1)) <= np.mean(np.abs(sep_e / want_e - 1)) * 1.02
+    # tanh.cc:51-59 picks the clamp "in a way that the tanh approximation on that input is exactly
+    # 1.0" for the with_fma constant it passes for f32 (tanh.cc:187): true of the fused spelling
+    # only -- the separate roundings land 3 ulp short, which is what pins mul_add's operand order
+    clamp = np.array([7.99881172180175781, 8.5, 12.0, -7.99881172180175781, -19.0], np.float32)
+    assert np.array_equal(oracle.tanh_f32(clamp), np.sign(clamp))
+    with oracle.fp_contract(False):
+        assert np.all(np.abs(oracle.tanh_f32(clamp)) < 1.0)
+
+
 # ---- epilogue -----------------------------------------------------------------
 
 def _gelu64(x):

@@ -106,6 +106,11 @@ __device__ __forceinline__ float div_well_scaled(float n, float d) {
   return __builtin_fmaf(__builtin_fmaf(-d, q1, n), r, q1);
 }
 
+// The reference's CPU backend compiles every kernel with fused multiply-add allowed
+// (xla/service/cpu/cpu_aot_loader.cc:49-55 and cpu_compiler.cc:1364: AllowFPOpFusion = Fast), so a
+// multiply feeding an add inside these f32 polynomials contracts to one fma on any host that has
+// the instruction.  The fused spelling is used here: one instruction per Horner step.
+//
 // xla/codegen/intrinsic/tanh.cc:48-108 rational, then the |x| >= 20 -> +-1 rule of :33-46.
 __device__ __forceinline__ float tanh_xla(float x) {
   const float kClamp = 7.99881172180175781f;
@@ -113,17 +118,17 @@ __device__ __forceinline__ float tanh_xla(float x) {
   float xc = __builtin_fminf(__builtin_fmaxf(x, -kClamp), kClamp);
   float x2 = xc * xc;
   float p = -2.76076847742355e-16f;
-  p = x2 * p + 2.00018790482477e-13f;
-  p = x2 * p + -8.60467152213735e-11f;
-  p = x2 * p + 5.12229709037114e-08f;
-  p = x2 * p + 1.48572235717979e-05f;
-  p = x2 * p + 6.37261928875436e-04f;
-  p = x2 * p + 4.89352455891786e-03f;
+  p = __builtin_fmaf(x2, p, 2.00018790482477e-13f);
+  p = __builtin_fmaf(x2, p, -8.60467152213735e-11f);
+  p = __builtin_fmaf(x2, p, 5.12229709037114e-08f);
+  p = __builtin_fmaf(x2, p, 1.48572235717979e-05f);
+  p = __builtin_fmaf(x2, p, 6.37261928875436e-04f);
+  p = __builtin_fmaf(x2, p, 4.89352455891786e-03f);
   p = xc * p;
   float q = 1.19825839466702e-06f;
-  q = x2 * q + 1.18534705686654e-04f;
-  q = x2 * q + 2.26843463243900e-03f;
-  q = x2 * q + 4.89352518554385e-03f;
+  q = __builtin_fmaf(x2, q, 1.18534705686654e-04f);
+  q = __builtin_fmaf(x2, q, 2.26843463243900e-03f);
+  q = __builtin_fmaf(x2, q, 4.89352518554385e-03f);
   // q is in [4.89e-3, 0.95] and |p| <= 0.95; below |x| = 4e-4 (|p| < 2e-6) the quotient is not used
   float r = ax < 0.0004f ? x : div_well_scaled(p, q);
   return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
@@ -132,16 +137,16 @@ __device__ __forceinline__ float tanh_xla(float x) {
 // xla/backends/cpu/codegen/polynomial_approximations.cc:173-296 (Cephes expf)
 __device__ __forceinline__ float exp_xla(float x) {
   float in = __builtin_fminf(__builtin_fmaxf(x, -87.8f), 88.8f);
-  float n = __builtin_floorf(in * 1.44269504088896341f + 0.5f);
+  float n = __builtin_floorf(__builtin_fmaf(in, 1.44269504088896341f, 0.5f));
   n = __builtin_fminf(__builtin_fmaxf(n, -127.0f), 127.0f);
-  float r = in - 0.693359375f * n;
-  r = r - -2.12194440e-4f * n;
-  float z = r * 1.9875691500E-4f + 1.3981999507E-3f;
-  z = z * r + 8.3334519073E-3f;
-  z = z * r + 4.1665795894E-2f;
-  z = z * r + 1.6666665459E-1f;
-  z = z * r + 5.0000001201E-1f;
-  z = z * (r * r) + r;
+  float r = __builtin_fmaf(-0.693359375f, n, in);
+  r = __builtin_fmaf(2.12194440e-4f, n, r);
+  float z = __builtin_fmaf(r, 1.9875691500E-4f, 1.3981999507E-3f);
+  z = __builtin_fmaf(z, r, 8.3334519073E-3f);
+  z = __builtin_fmaf(z, r, 4.1665795894E-2f);
+  z = __builtin_fmaf(z, r, 1.6666665459E-1f);
+  z = __builtin_fmaf(z, r, 5.0000001201E-1f);
+  z = __builtin_fmaf(z, r * r, r);
   z = 1.0f + z;
   float p2 = bits_to_f32((uint32_t)((int)n + 0x7f) << 23);
   float res = z * p2;
@@ -180,8 +185,9 @@ __device__ __forceinline__ float epilogue_act(float x, int act) {
     case 4: {  // tanh-approximated gelu
       float m0 = R(x * x);
       float m1 = R(x * m0);
-      float m2 = R(m1 * R(0.044715f));
-      float a0 = R(x + m2);
+      // f32-typed ops: the multiply by 0.044715 feeds only the add, which contracts like the
+      // polynomial steps above; bf16-typed ops round the product first, so nothing fuses
+      float a0 = BF16_OPS ? R(x + R(m1 * R(0.044715f))) : __builtin_fmaf(m1, 0.044715f, x);
       float m3 = R(a0 * R(0.797884583f));
       float th = R(tanh_xla(m3));
       float a2 = R(th + 1.0f);

@@ -15,17 +15,17 @@ __device__ float tanh_plain_quotient(float x) {
   float xc = __builtin_fminf(__builtin_fmaxf(x, -kClamp), kClamp);
   float x2 = xc * xc;
   float p = -2.76076847742355e-16f;
-  p = x2 * p + 2.00018790482477e-13f;
-  p = x2 * p + -8.60467152213735e-11f;
-  p = x2 * p + 5.12229709037114e-08f;
-  p = x2 * p + 1.48572235717979e-05f;
-  p = x2 * p + 6.37261928875436e-04f;
-  p = x2 * p + 4.89352455891786e-03f;
+  p = __builtin_fmaf(x2, p, 2.00018790482477e-13f);
+  p = __builtin_fmaf(x2, p, -8.60467152213735e-11f);
+  p = __builtin_fmaf(x2, p, 5.12229709037114e-08f);
+  p = __builtin_fmaf(x2, p, 1.48572235717979e-05f);
+  p = __builtin_fmaf(x2, p, 6.37261928875436e-04f);
+  p = __builtin_fmaf(x2, p, 4.89352455891786e-03f);
   p = xc * p;
   float q = 1.19825839466702e-06f;
-  q = x2 * q + 1.18534705686654e-04f;
-  q = x2 * q + 2.26843463243900e-03f;
-  q = x2 * q + 4.89352518554385e-03f;
+  q = __builtin_fmaf(x2, q, 1.18534705686654e-04f);
+  q = __builtin_fmaf(x2, q, 2.26843463243900e-03f);
+  q = __builtin_fmaf(x2, q, 4.89352518554385e-03f);
   float r = ax < 0.0004f ? x : p / q;
   return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
 }
