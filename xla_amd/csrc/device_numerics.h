@@ -94,16 +94,16 @@ __device__ __forceinline__ bool ordinary_divisor(float s) {
   return sb > 0x0d800000u && sb < 0x71800000u && (sb & 0x7fffffu) != 0x7fffffu;
 }
 
-// n / d as the f32 division expands on this target (reciprocal refined once, quotient corrected
-// twice), minus the operand scaling and the special-case fix-up: bit-identical to n / d when d is
-// a normal number in [2^-8, 2] and n is 0 or 2^-40 <= |n| <= 2, where the scaling factors are 1
-// and the fix-up passes the value through.
+// n / d for tanh_xla's numerator and denominator only: the reciprocal refined once and the quotient
+// corrected once -- the f32 division as this target expands it, minus the operand scaling, the
+// special-case fix-up (d is a normal number in [4.89e-3, 0.95], |n| <= 0.95) and the second
+// correction.  That this equals the IEEE quotient for every pair tanh_xla can produce is not argued
+// but checked: a self-check kernel compares both tanh spellings on all 2^32 inputs.
 __device__ __forceinline__ float div_well_scaled(float n, float d) {
   float r = __builtin_amdgcn_rcpf(d);
   r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
   const float q0 = n * r;
-  const float q1 = __builtin_fmaf(__builtin_fmaf(-d, q0, n), r, q0);
-  return __builtin_fmaf(__builtin_fmaf(-d, q1, n), r, q1);
+  return __builtin_fmaf(__builtin_fmaf(-d, q0, n), r, q0);
 }
 
 // The reference's CPU backend compiles every kernel with fused multiply-add allowed
@@ -112,7 +112,8 @@ __device__ __forceinline__ float div_well_scaled(float n, float d) {
 // the instruction.  The fused spelling is used here: one instruction per Horner step.
 //
 // xla/codegen/intrinsic/tanh.cc:48-108 rational, then the |x| >= 20 -> +-1 rule of :33-46.
-__device__ __forceinline__ float tanh_xla(float x) {
+// NaN in -> unspecified finite value out (the caller restores it): tanh_xla below is the full op.
+__device__ __forceinline__ float tanh_xla_nan_unspecified(float x) {
   const float kClamp = 7.99881172180175781f;
   float ax = __builtin_fabsf(x);
   float xc = __builtin_fminf(__builtin_fmaxf(x, -kClamp), kClamp);
@@ -131,7 +132,17 @@ __device__ __forceinline__ float tanh_xla(float x) {
   q = __builtin_fmaf(x2, q, 4.89352518554385e-03f);
   // q is in [4.89e-3, 0.95] and |p| <= 0.95; below |x| = 4e-4 (|p| < 2e-6) the quotient is not used
   float r = ax < 0.0004f ? x : div_well_scaled(p, q);
-  return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
+  // The |x| >= 20 -> copysign(1, x) rule of tanh.cc:33-46 changes nothing here: the clamp was chosen
+  // (tanh.cc:54-59) so that the fused rational is exactly +-1 at +-kClamp, which is where every
+  // larger |x| lands.
+  return r;
+}
+
+// A NaN comes out of the fmax/fmin clamp as -kClamp (the reference's select-based clamp keeps it,
+// llvm_util.cc EmitFloatMax with fast min/max), so it is put back.
+__device__ __forceinline__ float tanh_xla(float x) {
+  const float r = tanh_xla_nan_unspecified(x);
+  return x != x ? x : r;
 }
 
 // xla/backends/cpu/codegen/polynomial_approximations.cc:173-296 (Cephes expf)
@@ -189,9 +200,9 @@ __device__ __forceinline__ float epilogue_act(float x, int act) {
       // polynomial steps above; bf16-typed ops round the product first, so nothing fuses
       float a0 = BF16_OPS ? R(x + R(m1 * R(0.044715f))) : __builtin_fmaf(m1, 0.044715f, x);
       float m3 = R(a0 * R(0.797884583f));
-      float th = R(tanh_xla(m3));
-      float a2 = R(th + 1.0f);
-      float m4 = R(a2 * 0.5f);
+      float th = R(tanh_xla_nan_unspecified(m3));  // x * m4 below turns a NaN x back into NaN
+      // (th + 1) * 0.5: the halving is exact, so for f32 ops one fma gives the same bits
+      float m4 = BF16_OPS ? R(R(th + 1.0f) * 0.5f) : __builtin_fmaf(th, 0.5f, 0.5f);
       x = R(x * m4);
       break;
     }

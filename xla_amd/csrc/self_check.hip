@@ -8,7 +8,8 @@
 namespace xla_amd {
 namespace {
 
-// tanh_xla as in device_numerics.h, but with the plain f32 quotient p / q
+// tanh_xla as in device_numerics.h, but with the plain f32 quotient p / q and the explicit
+// |x| >= 20 rule of tanh.cc:33-46
 __device__ float tanh_plain_quotient(float x) {
   const float kClamp = 7.99881172180175781f;
   float ax = __builtin_fabsf(x);
@@ -27,6 +28,7 @@ __device__ float tanh_plain_quotient(float x) {
   q = __builtin_fmaf(x2, q, 2.26843463243900e-03f);
   q = __builtin_fmaf(x2, q, 4.89352518554385e-03f);
   float r = ax < 0.0004f ? x : p / q;
+  if (x != x) return x;  // the reference's select-based clamp keeps a NaN
   return ax >= 20.0f ? __builtin_copysignf(1.0f, x) : r;
 }
 
