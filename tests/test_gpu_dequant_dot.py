@@ -19,7 +19,7 @@ def say(msg):
     sys.stdout.flush()
 
 
-def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0):
+def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0):
     """x: 1 keeps s4 weights off the kernels that dequantise through the 4x4x4 matrix instruction
     (default: off whenever a strip width `vec` of the other kernels is asked for); pair: 1 takes the
     two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never."""
@@ -38,6 +38,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0):
     ffi.set_option("dequant_dot_x", (1 if vec else 0) if x is None else x)
     ffi.set_option("dequant_dot_pair", pair)
     ffi.set_option("dequant_dot_depth", depth)
+    ffi.set_option("dequant_dot_steps", steps)
     try:
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
                               weight_shape=w["weight_shape"], epilogue=w["epilogue"],
@@ -47,7 +48,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0):
         torch.cuda.synchronize()
     finally:
         for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec", "dequant_dot_x", "dequant_dot_pair",
-                  "dequant_dot_depth"):
+                  "dequant_dot_depth", "dequant_dot_steps"):
             ffi.set_option(k, 0)
     return host_bf16(out), ffi.last_kernel()
 
@@ -215,6 +216,75 @@ def test_s4x_pair_same_call_frame_replayed(oracle):
             compare(oracle, dict(w, lhs=a), host_bf16(out), "pair replay %d" % it)
     finally:
         ffi.set_option("dequant_dot_pair", 0)
+
+
+@pytest.mark.parametrize("M,steps,K,N,epilogue,bf16_vectors", [
+    (16, 0, 4096, 4096, "DEFAULT", False), (1, 1, 1024, 640, "BIAS_GELU", False), (5, 2, 1024, 648, "BIAS_SILU", True),
+    (16, 4, 4096, 200, "RELU", True), (8, 1, 4096, 384, "BIAS", False), (3, 4, 1024, 128, "DEFAULT", False),
+    (12, 2, 512, 1000, "BIAS_RELU", False), (16, 1, 256, 136, "SILU", True)])
+def test_s8x_variants(oracle, M, steps, K, N, epilogue, bf16_vectors):
+    """The single-launch s8 kernel for small matrices: 1 to 16 K-slices per strip adding up inside the
+    kernel, a ragged last strip, every epilogue, f32 and bf16 scale and bias vectors."""
+    say("dequant_dot s8x M=%d steps=%d K=%d N=%d %s bf16_vectors=%s" % (M, steps, K, N, epilogue, bf16_vectors))
+    w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    w["epilogue"] = epilogue
+    rng = np.random.default_rng(11)
+    if "BIAS" in epilogue:
+        w["bias"] = rng.standard_normal(N).astype(np.float32)
+        if bf16_vectors:
+            w["bias"] = dtypes.f32_to_bf16(w["bias"])
+    if bf16_vectors:
+        w["scales"] = dtypes.f32_to_bf16(w["scales"])
+    got, kern = run_dot(w, force_kernel=2, steps=steps)
+    assert kern.startswith("dequant_dot_decode_s8x_m16_s") and (steps == 0 or kern.endswith("s%d" % steps)), kern
+    compare(oracle, w, got, kern)
+
+
+def test_s8x_one_hot_integer_exact_and_batched(oracle):
+    """One-hot activations: every output is one weight times its channel's scale, exactly -- byte
+    order inside the 8-byte pieces, row order inside a step, the slices' and waves' shares of K.
+    Then two batches with their own weights and scales against the oracle."""
+    say("dequant_dot s8x one-hot, batched")
+    K, N = 512, 256
+    rng = np.random.default_rng(12)
+    wv = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+    sc = np.exp2(rng.integers(-6, 3, size=N)).astype(np.float32)
+    for m0 in range(0, K, 16):
+        a = np.zeros((16, K), np.float32)
+        a[np.arange(16), m0 + np.arange(16)] = 1.0
+        w = dict(lhs=dtypes.f32_to_bf16(a), weights=wv, scales=sc, bias=None, weight_dtype="s8",
+                 weight_shape=(K, N), group=K, dequant_type="f32", epilogue="DEFAULT")
+        got, kern = run_dot(w, force_kernel=2, steps=1)
+        assert kern == "dequant_dot_decode_s8x_m16_s1", kern
+        want = dtypes.f32_to_bf16(wv[m0:m0 + 16].astype(np.float32) * sc[None, :])
+        assert np.array_equal(got, want), (kern, m0)
+    w = workloads.c5_s8_batched(B=2, M=7, K=1024, N=392)
+    got, kern = run_dot(w, force_kernel=2, steps=2)
+    assert kern == "dequant_dot_decode_s8x_m16_s2", kern
+    compare(oracle, w, got, kern)
+
+
+def test_s8x_same_call_frame_replayed(oracle):
+    """The producers' flags are lowered by the strip's last workgroup, so the very same call frame
+    (same workspace, same flag value) can run again and again -- what a captured graph does -- with
+    new activations each time; the workspace starts out holding arbitrary bytes."""
+    say("dequant_dot s8x replay")
+    M, K, N = 16, 4096, 1024
+    w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    lhs, wt, sc = dev_bf16(w["lhs"]), dev_s8(w["weights"]), dev_f32(w["scales"])
+    nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S8)
+    assert nbytes > 0
+    scratch = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+    call = ops.dequant_dot(lhs, wt, sc, None, weight_dtype="s8", weight_shape=(K, N), epilogue="DEFAULT",
+                           dequant_type="f32", scratch=scratch, build_only=True)
+    rng = np.random.default_rng(9)
+    for it in range(4):
+        a = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+        lhs.copy_(dev_bf16(a))
+        out = call.run()
+        torch.cuda.synchronize()
+        assert ffi.last_kernel().startswith("dequant_dot_decode_s8x_m16_s"), ffi.last_kernel()
+        compare(oracle, dict(w, lhs=a), host_bf16(out), "s8x replay %d" % it)
 
 
 @pytest.mark.parametrize("which", ["s4", "s8"])

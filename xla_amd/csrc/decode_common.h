@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "device_numerics.h"
 #include "launch.h"
 
@@ -33,7 +35,7 @@ struct DecodeParams {
   int class_units[4];
   // s4x kernels, two workgroups per strip handing over inside the kernel: the producer's sums go to
   // workspace[batch * strips + strip][16 x 256 floats], then flags[batch * strips + strip] is set
-  // to epoch (never 0)
+  // to epoch (never 0).  s8x kernels: slices - 1 producers per strip, each with sums and a flag.
   int pair;
   int rows_first;       // rows the producer takes; the finisher takes rows_per_slice from there on
   int units_per_simd2;  // the finisher's units per SIMD; its class split is class_units[2..3]
@@ -71,6 +73,16 @@ static __device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t 
 }
 
 
+// A value no earlier launch of this process used and never 0: what the workgroups of one launch
+// write into their hand-over flags, so that whatever an earlier call (or nobody) left in the
+// workspace cannot be mistaken for it.
+inline unsigned long long NextHandOverEpoch() {
+  static std::atomic<unsigned long long> counter{0};
+  static const unsigned long long nonce =
+      0x9e3779b97f4a7c15ull * (unsigned long long)(uintptr_t)&counter ^ 0xd1b54a32d192ed03ull;
+  return (nonce + 2 * counter.fetch_add(1, std::memory_order_relaxed)) | 1ull;
+}
+
 // Sums the K-slices of dp.workspace in slice order and applies scale, bias and activation
 // (dequant_dot_decode.hip); mode: kRounded or kFactored.
 int LaunchDecodeFinalize(const DecodeParams& dp, int batch, hipStream_t stream, int mode);
@@ -87,6 +99,13 @@ int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
 // over inside the kernel, and the workspace that takes.
 bool S4xPairShape(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t group);
 size_t S4xPairWorkspaceBytes(int64_t batch, int64_t M, int64_t N);
+
+// s8 weights with per-channel scales under an f32-typed multiply, up to 16 tokens, small matrices:
+// one launch whose K-slices add up inside the kernel (dequant_dot_decode_s8x.hip).  Returns -1 when
+// the shape is not covered or the workspace is smaller than S8xWorkspaceBytes (0: shape not covered
+// or nothing needed).
+int LaunchDequantDotDecodeS8x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream);
+size_t S8xWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N);
 
 }  // namespace xla_amd
 #endif  // XLA_AMD_CSRC_DECODE_COMMON_H_

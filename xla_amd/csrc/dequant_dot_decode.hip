@@ -478,6 +478,8 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
   // s4 up to 16 tokens may run as two workgroups per 256-channel strip that hand over through the
   // workspace (the group size is not known here: the smallest one that path takes decides)
   if (s4 && S4xPairShape(batch, M, K, N, 64)) bytes = bytes > S4xPairWorkspaceBytes(batch, M, N) ? bytes : S4xPairWorkspaceBytes(batch, M, N);
+  // small s8 matrices up to 16 tokens: the slices of a strip hand over inside the kernel
+  if (!s4 && S8xWorkspaceBytes(batch, M, K, N) > bytes) bytes = S8xWorkspaceBytes(batch, M, K, N);
   return bytes;
 }
 
@@ -606,6 +608,11 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     // 4x4x4 matrix instruction
     if (shape_ok && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1) {
       const int rc = LaunchDequantDotDecodeS4x(dp, p, stream);
+      if (rc >= 0) return rc;
+    }
+    // small s8 matrices with per-channel scales under an f32-typed multiply: one launch
+    if (shape_ok && !s4 && mode == kFactored && per_channel && !weights_shared) {
+      const int rc = LaunchDequantDotDecodeS8x(dp, p, stream);
       if (rc >= 0) return rc;
     }
     if (shape_ok) {

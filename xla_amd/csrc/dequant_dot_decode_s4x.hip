@@ -545,12 +545,10 @@ int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
   const bool forced_slices = GetOption("dequant_dot_slices") != 0;
   if (mt == 1 && depth == 2 && !forced_slices && S4xPairShape(p.batch, p.M, p.K, p.N, p.group) && p.workspace &&
       ((uintptr_t)p.workspace % 8) == 0 && p.workspace_bytes >= S4xPairWorkspaceBytes(p.batch, p.M, p.N)) {
-    static std::atomic<unsigned long long> counter{0};
-    static const unsigned long long nonce = 0x9e3779b97f4a7c15ull * (unsigned long long)(uintptr_t)&counter ^ 0xd1b54a32d192ed03ull;
     dp.strips = (int)((p.N + 255) / 256);
     dp.pair = 1;
     dp.flags = (unsigned long long*)((char*)p.workspace + (size_t)p.batch * dp.strips * (16 * 256 * 4));
-    dp.epoch = (nonce + 2 * counter.fetch_add(1, std::memory_order_relaxed)) | 1ull;  // never 0
+    dp.epoch = NextHandOverEpoch();
     // Rows are split evenly ("dequant_dot_share" sets the producer's sixteenths): giving the producer
     // less, so that its sums are in memory before the finisher asks, measured slower at every token
     // count -- the finisher's own loop is what the kernel waits for.
