@@ -7,9 +7,10 @@
  *
  * Inside an XLA build include "xla/ffi/api/c_api.h" *before* this file: the
  * guard below is XLA's own, so this file then contributes nothing and the
- * handlers compile against the real header.  tests/test_ffi_abi.py checks
- * sizeof/offsetof of every struct against the real header when an XLA tree is
- * present.
+ * handlers compile against the real header.  tests/test_ffi_boundary.py
+ * compares sizeof/offsetof and the enum values with the real header when an
+ * XLA tree is present; tests/test_ffi_reference_headers.py registers and
+ * decodes through the real api.h / ffi.h.
  */
 #ifndef XLA_FFI_API_C_API_H_
 #define XLA_FFI_API_C_API_H_

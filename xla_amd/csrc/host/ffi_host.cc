@@ -29,10 +29,13 @@ HOST_EXPORT XLA_FFI_Error* xla_amd_host_replay(XLA_FFI_Handler* const* handlers,
 
 // ---- a native XLA_FFI_Api table: what xla/ffi/ffi_api.cc:668-706 provides inside XLA, reduced
 // to what the handlers of this library call (errors, stream, registration).
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <map>
 #include <mutex>
 #include <string>
-#include <unordered_map>
-#include <vector>
+#include <utility>
 
 struct XLA_FFI_Error {
   XLA_FFI_Error_Code code;
@@ -42,16 +45,44 @@ struct XLA_FFI_Error {
 namespace {
 
 struct Registration {
-  std::string name, platform;
+  XLA_FFI_Metadata metadata;
   XLA_FFI_Handler_Bundle bundle;
-  XLA_FFI_Handler_Traits traits;
 };
+
+// One registry per process, keyed by (target, canonical platform), like the static handler map
+// of xla/ffi/ffi_registry.cc:40-43: XLA_FFI_Handler_Register carries no context, and handlers
+// registered from static initialisers (XLA_FFI_REGISTER_HANDLER) must land somewhere.
+struct Registry {
+  std::mutex mu;
+  std::map<std::pair<std::string, std::string>, Registration> map;
+};
+Registry& StaticRegistry() {
+  static Registry* r = new Registry();
+  return *r;
+}
 
 struct HostState {
   XLA_FFI_Api api;
   void* stream = nullptr;
-  std::vector<Registration> registry;
 };
+
+// xla/service/platform_util.cc:64-91 as a ROCm build resolves it.
+std::string CanonicalPlatformName(std::string platform) {
+  for (char& c : platform) c = (char)tolower((unsigned char)c);
+  if (platform == "cpu") return "host";
+  if (platform == "gpu") return "rocm";
+  if (platform == "oneapi") return "sycl";
+  return platform;
+}
+
+XLA_FFI_Error* InvalidArgument(const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  return new XLA_FFI_Error{XLA_FFI_Error_Code_INVALID_ARGUMENT, buf};
+}
 
 // ctx of every frame built for this host points at the HostState
 XLA_FFI_Error* ErrorCreate(XLA_FFI_Error_Create_Args* a) { return new XLA_FFI_Error{a->errc, a->message}; }
@@ -65,13 +96,80 @@ XLA_FFI_Error* StreamGet(XLA_FFI_Stream_Get_Args* a) {
   a->stream = reinterpret_cast<HostState*>(a->ctx)->stream;
   return nullptr;
 }
-HostState* g_registering = nullptr;  // Handler_Register carries no ctx; set around the call
+
+// The registration-time handshake of xla/ffi/invoke.cc:174-233: a call frame that carries nothing
+// but a metadata extension; the handler fills in the API version it was built against and its
+// traits and returns without doing any work.
+XLA_FFI_Error* GetMetadata(const XLA_FFI_Api* api, XLA_FFI_Handler* handler, XLA_FFI_Metadata* metadata) {
+  *metadata = XLA_FFI_Metadata{};
+  metadata->struct_size = XLA_FFI_Metadata_STRUCT_SIZE;
+  metadata->api_version.struct_size = XLA_FFI_Api_Version_STRUCT_SIZE;
+  XLA_FFI_Metadata_Extension ext{};
+  ext.extension_base.struct_size = XLA_FFI_Metadata_Extension_STRUCT_SIZE;
+  ext.extension_base.type = XLA_FFI_Extension_Metadata;
+  ext.metadata = metadata;
+  XLA_FFI_CallFrame frame{};
+  frame.struct_size = XLA_FFI_CallFrame_STRUCT_SIZE;
+  frame.extension_start = &ext.extension_base;
+  frame.api = api;
+  frame.ctx = nullptr;
+  frame.stage = XLA_FFI_ExecutionStage_EXECUTE;
+  frame.args.struct_size = XLA_FFI_Args_STRUCT_SIZE;
+  frame.rets.struct_size = XLA_FFI_Rets_STRUCT_SIZE;
+  frame.attrs.struct_size = XLA_FFI_Attrs_STRUCT_SIZE;
+  return (*handler)(&frame);
+}
+
+bool SameMetadata(const XLA_FFI_Metadata& a, const XLA_FFI_Metadata& b) {
+  return a.api_version.major_version == b.api_version.major_version &&
+         a.api_version.minor_version == b.api_version.minor_version && a.traits == b.traits &&
+         a.state_type_id.type_id == b.state_type_id.type_id;
+}
+bool SameBundle(const XLA_FFI_Handler_Bundle& a, const XLA_FFI_Handler_Bundle& b) {
+  return a.instantiate == b.instantiate && a.prepare == b.prepare && a.initialize == b.initialize &&
+         a.execute == b.execute && a.record == b.record;
+}
+
+const XLA_FFI_Api* g_registering_api = nullptr;  // the table handed to the metadata query
+
+// RegisterHandler of xla/ffi/ffi_registry.cc:87-158, rule for rule: canonical platform, an execute
+// stage is required, the handler's API version must lie in [0.1, this API's], explicit traits are
+// OR-ed into the handler's own, and a second registration of the same key is accepted only when it
+// is the very same handler with the same metadata.
 XLA_FFI_Error* HandlerRegister(XLA_FFI_Handler_Register_Args* a) {
-  if (!g_registering) return new XLA_FFI_Error{XLA_FFI_Error_Code_FAILED_PRECONDITION, "no host is registering"};
-  if (!a->bundle.execute) return new XLA_FFI_Error{XLA_FFI_Error_Code_INVALID_ARGUMENT, "execute handler is required"};
-  Registration r{std::string(a->name.ptr, a->name.len), std::string(a->platform.ptr, a->platform.len), a->bundle, a->traits};
-  for (char& c : r.platform) c = (char)tolower(c);
-  g_registering->registry.push_back(r);
+  const std::string name(a->name.ptr, a->name.len), platform(a->platform.ptr, a->platform.len);
+  const std::string canonical = CanonicalPlatformName(platform);
+  if (!a->bundle.execute)
+    return InvalidArgument("FFI handler for %s on a platform %s must provide an execute implementation",
+                           name.c_str(), platform.c_str());
+  XLA_FFI_Metadata metadata;
+  if (XLA_FFI_Error* e = GetMetadata(g_registering_api, a->bundle.execute, &metadata)) return e;
+  const std::pair<int, int> version{metadata.api_version.major_version, metadata.api_version.minor_version};
+  const std::pair<int, int> lo{0, 1}, hi{XLA_FFI_API_MAJOR, XLA_FFI_API_MINOR};
+  if (version < lo || version > hi)
+    return InvalidArgument(
+        "XLA FFI handler registration for %s on platform %s (canonical %s) failed because the handler's API "
+        "version (%d.%d) is incompatible with the framework's API version (%d.%d). Minimum supported API "
+        "version is (%d.%d).",
+        name.c_str(), platform.c_str(), canonical.c_str(), version.first, version.second, hi.first, hi.second,
+        lo.first, lo.second);
+  metadata.traits |= a->traits;
+  if (a->bundle.instantiate) {
+    XLA_FFI_Metadata im;
+    if (XLA_FFI_Error* e = GetMetadata(g_registering_api, a->bundle.instantiate, &im)) return e;
+    metadata.state_type_id = im.state_type_id;
+  }
+  Registry& reg = StaticRegistry();
+  std::lock_guard<std::mutex> lock(reg.mu);
+  auto [it, emplaced] = reg.map.try_emplace({name, canonical}, Registration{metadata, a->bundle});
+  if (!emplaced) {
+    if (!SameMetadata(it->second.metadata, metadata))
+      return InvalidArgument("Duplicate FFI handler registration for %s on platform %s (canonical %s) with different metadata",
+                             name.c_str(), platform.c_str(), canonical.c_str());
+    if (!SameBundle(it->second.bundle, a->bundle))
+      return InvalidArgument("Duplicate FFI handler registration for %s on platform %s (canonical %s) with different bundle addresses",
+                             name.c_str(), platform.c_str(), canonical.c_str());
+  }
   return nullptr;
 }
 template <typename Args>
@@ -107,6 +205,7 @@ HOST_EXPORT void* xla_amd_host_create(void) {
   t.XLA_FFI_RunId_Get = Unimplemented<XLA_FFI_RunId_Get_Args>;
   t.XLA_FFI_DeviceOrdinal_Get = Unimplemented<XLA_FFI_DeviceOrdinal_Get_Args>;
   t.XLA_FFI_InvokeContext_FindExtension = Unimplemented<XLA_FFI_InvokeContext_FindExtension_Args>;
+  if (!g_registering_api) g_registering_api = &h->api;  // any host's table serves the metadata query
   return h;
 }
 
@@ -127,19 +226,27 @@ HOST_EXPORT int xla_amd_host_take_error(XLA_FFI_Error* err, char* buf, size_t n)
   return code;
 }
 
-// Runs `register_fn(api)` (e.g. xla_amd_register_handlers) against this host's registry.
+// Runs `register_fn(api)` (e.g. xla_amd_register_handlers) against the process-wide registry.
 HOST_EXPORT XLA_FFI_Error* xla_amd_host_register(void* host, XLA_FFI_Error* (*register_fn)(const XLA_FFI_Api*)) {
-  static std::mutex mu;
-  std::lock_guard<std::mutex> lock(mu);
-  g_registering = reinterpret_cast<HostState*>(host);
-  XLA_FFI_Error* e = register_fn(&g_registering->api);
-  g_registering = nullptr;
-  return e;
+  return register_fn(&reinterpret_cast<HostState*>(host)->api);
 }
 
-// Looks a handler up by (target, platform) the way the registry does (xla/ffi/ffi_registry.cc:160-175).
+// Looks a handler up by (target, platform) the way the registry does (xla/ffi/ffi_registry.cc:160-186):
+// the platform name is canonicalised first.  Returns the execute stage, or null.
 HOST_EXPORT XLA_FFI_Handler* xla_amd_host_find_handler(void* host, const char* name, const char* platform) {
-  for (const Registration& r : reinterpret_cast<HostState*>(host)->registry)
-    if (r.name == name && r.platform == platform) return r.bundle.execute;
-  return nullptr;
+  (void)host;
+  Registry& reg = StaticRegistry();
+  std::lock_guard<std::mutex> lock(reg.mu);
+  auto it = reg.map.find({name, CanonicalPlatformName(platform)});
+  return it == reg.map.end() ? nullptr : it->second.bundle.execute;
+}
+
+// Traits the registry holds for a handler (its own OR-ed with those given at registration), -1 if
+// it is not registered.
+HOST_EXPORT int64_t xla_amd_host_handler_traits(void* host, const char* name, const char* platform) {
+  (void)host;
+  Registry& reg = StaticRegistry();
+  std::lock_guard<std::mutex> lock(reg.mu);
+  auto it = reg.map.find({name, CanonicalPlatformName(platform)});
+  return it == reg.map.end() ? -1 : (int64_t)it->second.metadata.traits;
 }

@@ -404,6 +404,8 @@ def host_library():
         L.xla_amd_host_register.argtypes = [C.c_void_p, C.c_void_p]
         L.xla_amd_host_find_handler.restype = C.c_void_p
         L.xla_amd_host_find_handler.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
+        L.xla_amd_host_handler_traits.restype = C.c_int64
+        L.xla_amd_host_handler_traits.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
         _host_lib = L
     return _host_lib
 
