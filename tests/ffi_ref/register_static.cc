@@ -19,12 +19,15 @@ static const XLA_FFI_Api* HostApi() {
   return xla_amd_host_api(host);
 }
 
-XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.dequant_dot", "ROCM", xla_amd_dequant_dot,
+// execute and record stages are the same symbol: at RECORD the handler asks for stream capture
+#define XLA_AMD_BUNDLE(fn) (XLA_FFI_Handler_Bundle{nullptr, nullptr, nullptr, fn, fn})
+
+XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.dequant_dot", "ROCM", XLA_AMD_BUNDLE(xla_amd_dequant_dot),
                          XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE);
-XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.fp8_scaled_dot", "ROCM", xla_amd_fp8_scaled_dot,
+XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.fp8_scaled_dot", "ROCM", XLA_AMD_BUNDLE(xla_amd_fp8_scaled_dot),
                          XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE);
-XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.rowwise_quantize_fp8", "ROCM", xla_amd_rowwise_quantize_fp8,
-                         XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE);
+XLA_FFI_REGISTER_HANDLER(HostApi(), "xla_amd.rowwise_quantize_fp8", "ROCM",
+                         XLA_AMD_BUNDLE(xla_amd_rowwise_quantize_fp8), XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE);
 
 // A second registration of the same handler under the same name is accepted (the library linked
 // twice); the same name with another handler is refused.  Returns the two error codes.
@@ -46,8 +49,10 @@ extern "C" int register_again(int* same_handler_code, int* other_handler_code) {
     return code;
   };
   *same_handler_code = code_of(xla::ffi::Ffi::RegisterStaticHandler(
-      api, "xla_amd.dequant_dot", "rocm", xla_amd_dequant_dot, XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE));
+      api, "xla_amd.dequant_dot", "rocm", XLA_AMD_BUNDLE(xla_amd_dequant_dot),
+      XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE));
   *other_handler_code = code_of(xla::ffi::Ffi::RegisterStaticHandler(
-      api, "xla_amd.dequant_dot", "ROCM", xla_amd_fp8_scaled_dot, XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE));
+      api, "xla_amd.dequant_dot", "ROCM", XLA_AMD_BUNDLE(xla_amd_fp8_scaled_dot),
+      XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE));
   return 0;
 }

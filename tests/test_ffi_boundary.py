@@ -154,6 +154,30 @@ def test_shape_validation_happens_before_any_launch():
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
 
 
+def test_record_stage_asks_for_stream_capture():
+    """At the RECORD stage (XLA building a command buffer, custom_call_thunk.cc:577-684) a handler finds
+    the record extension on its invoke context and asks for stream capture of its execute stage;
+    it decodes nothing and launches nothing (the buffers here are fake)."""
+    host = ffi.NativeHost()
+    before = host.set_recording(True)
+    try:
+        ffi.invoke("xla_amd.rowwise_quantize_fp8", quant_frame(host, stage=ffi.STAGE_RECORD))
+        args = [(dtypes.BF16, FAKE, (2, 8)), (dtypes.S8, FAKE, (8, 4)), (dtypes.F32, FAKE, (4,))]
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, args, [(dtypes.BF16, FAKE, (2, 4))], stage=ffi.STAGE_RECORD))
+        a = [(dtypes.F8E4M3FN, FAKE, (4, 8)), (dtypes.F8E4M3FN, FAKE, (8, 4)), (dtypes.F32, FAKE, ()), (dtypes.F32, FAKE, ())]
+        ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a, [(dtypes.BF16, FAKE, (4, 4))], stage=ffi.STAGE_RECORD))
+    finally:
+        after = host.set_recording(False)
+    assert after - before == 3
+    # outside a recording there is no extension to answer to
+    with pytest.raises(ffi.FfiError, match=r"\[record\] the call carries no usable record extension"):
+        ffi.invoke("xla_amd.rowwise_quantize_fp8", quant_frame(host, stage=ffi.STAGE_RECORD))
+    assert host.set_recording(False) == after
+    # a host whose function table lacks the lookup reports that instead
+    with pytest.raises(ffi.FfiError, match="not implemented by this host"):
+        ffi.invoke("xla_amd.rowwise_quantize_fp8", quant_frame(ffi.Host(), stage=ffi.STAGE_RECORD))
+
+
 def test_stream_get_failure_is_propagated():
     host = ffi.Host(fail_stream_get=True)
     with pytest.raises(ffi.FfiError, match="GPU context is not available"):

@@ -2,15 +2,22 @@
 into a command buffer (a HIP graph) once and replay it step after step
 (xla/ffi/api/c_api.h:428-437, 528-533; xla/backends/gpu/runtime/custom_call_thunk.cc:659-666).
 That only works if a call enqueues the same kernels for the same shapes, never synchronises,
-never reads device data on the host and allocates nothing.  Here a decode step, a quantize and
-a scaled dot are captured into one graph through the native call-frame replay, the operands
-are then changed in place, and every replay must equal what eager calls give on the same data."""
+never reads device data on the host and allocates nothing.  Here decode steps of every kind
+(two workgroups per strip handing over inside the kernel, K-slices adding up inside the kernel,
+K-slices with a second launch, more than 64 tokens as several launches), a quantize and scaled dots
+are captured into one graph through the native call-frame replay; the operands are then changed
+in place, and every replay must equal what eager calls give on the same data AND what the oracle
+computes from it."""
 import sys
 
+import numpy as np
 import pytest
 import torch
 
-from xla_amd import ffi, ops
+from tests.gpu_util import check_dot, dev_bf16, dev_f32, dev_s8, dev_u8, host_bf16
+from tests.test_gpu_dequant_dot import compare
+from tests.test_gpu_fp8_dot import floor_for as fp8_floor_for
+from xla_amd import dtypes, ffi, ops, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -20,28 +27,50 @@ def say(msg):
     sys.stdout.flush()
 
 
-def test_handlers_replay_from_a_hip_graph():
-    say("graph capture of dequant_dot (split-K + finalize), rowwise_quantize_fp8, fp8_scaled_dot (bf16 and f8 + amax)")
+def test_handlers_replay_from_a_hip_graph(oracle):
+    say("graph capture of dequant_dot (pair hand-over, s8 in-kernel slices, split-K + finalize, 70 tokens), "
+        "rowwise_quantize_fp8, fp8_scaled_dot (bf16 and f8 + amax)")
     dev = torch.device("cuda:0")
-    torch.manual_seed(7)
-    K, N = 2048, 1024
-    lhs = torch.randn((8, K), device=dev).to(torch.bfloat16)
-    w4 = torch.randint(0, 256, (K * N // 2,), dtype=torch.uint8, device=dev)
-    sc = torch.empty((K // 128, N), device=dev).uniform_(1e-3, 2e-2).to(torch.bfloat16)
-    bias = torch.randn((N,), device=dev).to(torch.bfloat16)
-    x = torch.randn((256, 1024), device=dev).to(torch.bfloat16)
-    gamma = torch.empty((1024,), device=dev).uniform_(0.5, 1.5).to(torch.bfloat16)
-    a8 = (torch.randn((256, 512), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
-    b8 = (torch.randn((512, 256), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
-    s64 = torch.full((), 1 / 64, device=dev)
+    rng = np.random.default_rng(7)
+    # the decode calls, each with the numpy workload the oracle reads
+    dots = []
+    for w, opts in ((workloads.c2_s4_group(M=8, K=2048, N=1024), {"dequant_dot_pair": 1}),  # pair hand-over
+                    (workloads.c2_s4_group(M=20, K=2048, N=768, group=64), {"dequant_dot_slices": 2}),  # finalize launch
+                    (workloads.c2_s4_group(M=70, K=1024, N=512), {}),                     # 64 + 6 tokens
+                    (workloads.c1_s8_channel(M=16, K=2048, N=1024), {})):                 # slices inside the kernel
+        lhs = dev_bf16(w["lhs"])
+        wt = dev_u8(w["weights_packed"]) if w["weight_dtype"] == "s4" else dev_s8(w["weights"])
+        sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
+        bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
+        for k, v in opts.items():
+            ffi.set_option(k, v)
+        try:
+            call = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"], weight_shape=w["weight_shape"],
+                                   epilogue=w["epilogue"], dequant_type=w["dequant_type"],
+                                   scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"],
+                                   build_only=True)
+            call.run()   # eager warm-up with the options that pick the kernel; the frame keeps its scratch
+            torch.cuda.synchronize()
+            kern = ffi.last_kernel()
+        finally:
+            for k in opts:
+                ffi.set_option(k, 0)
+        dots.append((w, lhs, call, opts, kern))
+    assert dots[0][4] == "dequant_dot_decode_s4x_m16_pair", dots[0][4]
+    assert dots[2][4].endswith(":x64"), dots[2][4]
+    assert dots[3][4].startswith("dequant_dot_decode_s8x_"), dots[3][4]
 
-    calls = [ops.dequant_dot(lhs, w4, sc, bias, weight_dtype="s4", weight_shape=(K, N), epilogue="BIAS_SILU",
-                             dequant_type="bf16", build_only=True),
-             ops.rowwise_quantize_fp8(x, gamma, build_only=True),
-             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="GELU", build_only=True),
-             # f8 result with its amax: a one-thread kernel zeroes the amax, then atomics fold into it
-             ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="RELU", d_scale=torch.full((), 0.05, device=dev),
-                                amax=True, build_only=True)]
+    q4 = workloads.c4_quantize(rows=256, cols=1024)
+    x, gamma = dev_bf16(q4["x"]), dev_bf16(q4["gamma"])
+    c3 = workloads.c3_fp8(256, 512, 256)
+    a8, b8 = dev_u8(c3["a"]), dev_u8(c3["b"])
+    s64 = torch.full((), 1 / 64, device=dev)
+    calls = [d[2] for d in dots] + [
+        ops.rowwise_quantize_fp8(x, gamma, build_only=True),
+        ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="GELU", build_only=True),
+        # f8 result with its amax: a one-thread kernel zeroes the amax, then atomics fold into it
+        ops.fp8_scaled_dot(a8, b8, s64, s64, None, epilogue="RELU", d_scale=torch.full((), 0.05, device=dev),
+                           amax=True, build_only=True)]
 
     def results():
         out = []
@@ -50,12 +79,21 @@ def test_handlers_replay_from_a_hip_graph():
             out += [t.clone().view(torch.uint8) if t.dtype != torch.float32 else t.clone() for t in r]
         return out
 
-    # eager warm-up: first launches may set kernel attributes, which must not happen under capture
-    for c in calls:
-        c.run()
+    # options that steer a call's kernel choice are set around that call, eagerly and under capture alike
+    def run_all_eager():
+        for i, c in enumerate(calls):
+            opts = dots[i][3] if i < len(dots) else {}
+            for k, v in opts.items():
+                ffi.set_option(k, v)
+            try:
+                c.run()
+            finally:
+                for k in opts:
+                    ffi.set_option(k, 0)
+
+    run_all_eager()   # first launches may set kernel attributes, which must not happen under capture
     torch.cuda.synchronize()
 
-    replay = ffi.Replay([(c.target, c.frame) for c in calls])
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -63,17 +101,30 @@ def test_handlers_replay_from_a_hip_graph():
         for c in calls:
             c.frame.host.stream = side.cuda_stream
         with torch.cuda.graph(graph, stream=side):
-            replay.run(1)
+            for i, c in enumerate(calls):
+                opts = dots[i][3] if i < len(dots) else {}
+                for k, v in opts.items():
+                    ffi.set_option(k, v)
+                try:
+                    ffi.Replay([(c.target, c.frame)]).run(1)
+                finally:
+                    for k in opts:
+                        ffi.set_option(k, 0)
     torch.cuda.current_stream().wait_stream(side)
 
     for round_ in range(3):
         # new operand values in the same buffers, eager work and a synchronisation between replays
-        lhs.copy_(torch.randn((8, K), device=dev).to(torch.bfloat16))
-        x.copy_(torch.randn((256, 1024), device=dev).to(torch.bfloat16) * (round_ + 1))
-        a8.copy_((torch.randn((256, 512), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn))
+        new_lhs = []
+        for w, lhs, _, _, _ in dots:
+            a = dtypes.f32_to_bf16(rng.standard_normal(w["lhs"].shape).astype(np.float32))
+            lhs.copy_(dev_bf16(a))
+            new_lhs.append(a)
+        xq = dtypes.f32_to_bf16((rng.standard_normal(q4["x"].shape) * (round_ + 1)).astype(np.float32))
+        x.copy_(dev_bf16(xq))
+        an = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal(c3["a"].shape) * 64, -448, 448).astype(np.float32))
+        a8.copy_(dev_u8(an))
         torch.cuda.synchronize()
-        for c in calls:
-            c.run()
+        run_all_eager()
         torch.cuda.synchronize()
         want = results()
         for c in calls:  # wipe the outputs so that a replay that does nothing cannot pass
@@ -85,4 +136,13 @@ def test_handlers_replay_from_a_hip_graph():
         got = results()
         for i, (g, w) in enumerate(zip(got, want)):
             assert torch.equal(g, w), "replay %d: result %d differs from the eager call" % (round_, i)
+        # ... and against the oracle, from the replay's own outputs
+        for (w, _, call, _, kern), a in zip(dots, new_lhs):
+            compare(oracle, dict(w, lhs=a), host_bf16(call.result), "replay %d %s" % (round_, kern))
+        q_ref, s_ref = oracle.rmsnorm_quantize_fp8(xq, q4["gamma"], eps=1e-6)
+        q_got, s_got = calls[len(dots)].result
+        assert np.array_equal(q_got.cpu().numpy(), q_ref) and np.array_equal(s_got.cpu().numpy(), s_ref), round_
+        ref = oracle.fp8_scaled_dot(an, c3["b"], 1 / 64, 1 / 64, epilogue="gelu_tanh")
+        floor = fp8_floor_for(dict(c3, a=an))
+        check_dot(host_bf16(calls[len(dots) + 1].result), ref, floor, "replay %d fp8 dot" % round_)
     assert ffi.last_kernel()  # the library recorded which kernels it chose

@@ -14,6 +14,7 @@
 
 #include "launch.h"
 #include "xla_amd_quant.h"
+#include "xla_ffi_record_abi.h"
 
 namespace xla_amd {
 namespace {
@@ -209,6 +210,33 @@ constexpr uint64_t Bit(int d) { return 1ull << d; }
 constexpr uint64_t kFloatMask = Bit(XLA_FFI_DataType_F32) | Bit(XLA_FFI_DataType_BF16);
 constexpr uint64_t kBytesMask = Bit(XLA_FFI_DataType_S8) | Bit(XLA_FFI_DataType_U8);
 
+// The RECORD stage (xla/backends/gpu/runtime/custom_call_thunk.cc:577-684): XLA is building a
+// command buffer and asks the handler to add its commands through the record extension.  These
+// handlers launch prebuilt kernels on a stream, so they ask for the alternative the record API
+// offers -- request_stream_capture (record_c_api.h:189-191) -- and XLA then traces the EXECUTE
+// stage into the command buffer, which is what it does for a handler without a record stage.
+// Nothing is launched here.
+XLA_FFI_Error* AnswerRecord(XLA_FFI_CallFrame* f) {
+  const XLA_FFI_Api* api = f->api;
+  const size_t need = offsetof(XLA_FFI_Api, XLA_FFI_InvokeContext_FindExtension) + sizeof(void*);
+  if (api->struct_size < need || api->XLA_FFI_InvokeContext_FindExtension == nullptr)
+    return InvalidArgument(api, "[record] this XLA_FFI_Api has no XLA_FFI_InvokeContext_FindExtension");
+  XLA_FFI_InvokeContext_FindExtension_Args a;
+  memset(&a, 0, sizeof(a));
+  a.struct_size = XLA_FFI_STRUCT_SIZE(XLA_FFI_InvokeContext_FindExtension_Args, extension);
+  a.ctx = f->ctx;
+  a.extension_type = XLA_FFI_Extension_Record;
+  if (XLA_FFI_Error* e = api->XLA_FFI_InvokeContext_FindExtension(&a)) return e;
+  const XLA_FFI_Record_Extension* ext = reinterpret_cast<const XLA_FFI_Record_Extension*>(a.extension);
+  if (ext == nullptr || ext->extension_base.struct_size < XLA_FFI_Record_Extension_STRUCT_SIZE ||
+      ext->extension_base.id.extension_type != XLA_FFI_Extension_Record ||
+      ext->extension_base.id.major_version != XLA_FFI_Extension_Record_MajorVersion ||
+      ext->record_frame == nullptr || ext->record_frame->api == nullptr ||
+      ext->record_frame->api->request_stream_capture == nullptr)
+    return InvalidArgument(api, "[record] the call carries no usable record extension (type 128, version 0.x)");
+  return ext->record_frame->api->request_stream_capture(ext->record_frame->record_ctx);
+}
+
 // Steps shared by all handlers up to operand decoding (api.h:2296-2424).  Returns true when
 // the caller should return *err (which may be null for the metadata query).
 bool Preamble(XLA_FFI_CallFrame* f, int min_args, int max_args, int min_rets, int max_rets,
@@ -235,6 +263,10 @@ bool Preamble(XLA_FFI_CallFrame* f, int min_args, int max_args, int min_rets, in
     ext->metadata->api_version.minor_version = XLA_FFI_API_MINOR;
     ext->metadata->traits = XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE;
     ext->metadata->state_type_id.type_id = 0;  // stateless
+    return true;
+  }
+  if (f->stage == XLA_FFI_ExecutionStage_RECORD) {
+    *err = AnswerRecord(f);
     return true;
   }
   if (f->stage != XLA_FFI_ExecutionStage_EXECUTE) {
@@ -541,6 +573,7 @@ XLA_FFI_Error* xla_amd_register_handlers(const XLA_FFI_Api* api) {
     args.name = XLA_FFI_ByteSpan{e.name, strlen(e.name)};
     args.platform = XLA_FFI_ByteSpan{"ROCM", 4};
     args.bundle.execute = e.fn;
+    args.bundle.record = e.fn;  // the RECORD stage asks for stream capture of the execute stage
     args.traits = XLA_FFI_HANDLER_TRAITS_COMMAND_BUFFER_COMPATIBLE;
     if (XLA_FFI_Error* err = api->XLA_FFI_Handler_Register(&args)) return err;
   }

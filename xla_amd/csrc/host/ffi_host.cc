@@ -7,6 +7,7 @@
 #include <ctype.h>
 
 #include "xla_ffi_abi.h"
+#include "xla_ffi_record_abi.h"
 
 #define HOST_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -64,6 +65,13 @@ Registry& StaticRegistry() {
 struct HostState {
   XLA_FFI_Api api;
   void* stream = nullptr;
+  // what a command-buffer recording attaches to the invoke context (custom_call_thunk.cc:610-618):
+  // a record extension whose function table only implements request_stream_capture
+  XLA_FFI_RecordApi record_api{};
+  XLA_FFI_RecordFrame record_frame{};
+  XLA_FFI_Record_Extension record_extension{};
+  bool recording = false;
+  int stream_capture_requests = 0;
 };
 
 // xla/service/platform_util.cc:64-91 as a ROCm build resolves it.
@@ -94,6 +102,18 @@ void ErrorDestroy(XLA_FFI_Error_Destroy_Args* a) { delete a->error; }
 XLA_FFI_Error* StreamGet(XLA_FFI_Stream_Get_Args* a) {
   if (!a->ctx) return new XLA_FFI_Error{XLA_FFI_Error_Code_INVALID_ARGUMENT, "XLA FFI GPU context is not available"};
   a->stream = reinterpret_cast<HostState*>(a->ctx)->stream;
+  return nullptr;
+}
+
+XLA_FFI_Error* FindExtension(XLA_FFI_InvokeContext_FindExtension_Args* a) {
+  a->extension = nullptr;
+  if (!a->ctx) return new XLA_FFI_Error{XLA_FFI_Error_Code_INVALID_ARGUMENT, "no invoke context"};
+  HostState* h = reinterpret_cast<HostState*>(a->ctx);
+  if (h->recording && a->extension_type == XLA_FFI_Extension_Record) a->extension = &h->record_extension.extension_base;
+  return nullptr;  // not found: a null extension, no error (ffi_api.cc XLA_FFI_InvokeContext_FindExtension)
+}
+XLA_FFI_Error* RequestStreamCapture(XLA_FFI_RecordContext* ctx) {
+  ++reinterpret_cast<HostState*>(ctx)->stream_capture_requests;
   return nullptr;
 }
 
@@ -204,7 +224,16 @@ HOST_EXPORT void* xla_amd_host_create(void) {
   t.XLA_FFI_Future_SetError = Unimplemented<XLA_FFI_Future_SetError_Args>;
   t.XLA_FFI_RunId_Get = Unimplemented<XLA_FFI_RunId_Get_Args>;
   t.XLA_FFI_DeviceOrdinal_Get = Unimplemented<XLA_FFI_DeviceOrdinal_Get_Args>;
-  t.XLA_FFI_InvokeContext_FindExtension = Unimplemented<XLA_FFI_InvokeContext_FindExtension_Args>;
+  t.XLA_FFI_InvokeContext_FindExtension = FindExtension;
+  h->record_api.request_stream_capture = RequestStreamCapture;
+  h->record_frame.record_ctx = reinterpret_cast<XLA_FFI_RecordContext*>(h);
+  h->record_frame.api = &h->record_api;
+  h->record_frame.action = XLA_FFI_RecordAction_Create;
+  h->record_extension.extension_base.struct_size = XLA_FFI_Record_Extension_STRUCT_SIZE;
+  h->record_extension.extension_base.id =
+      XLA_FFI_ExtensionId{XLA_FFI_Extension_Record, XLA_FFI_Extension_Record_MajorVersion, XLA_FFI_Extension_Record_MinorVersion};
+  h->record_extension.extension_base.next = nullptr;
+  h->record_extension.record_frame = &h->record_frame;
   if (!g_registering_api) g_registering_api = &h->api;  // any host's table serves the metadata query
   return h;
 }
@@ -212,6 +241,15 @@ HOST_EXPORT void* xla_amd_host_create(void) {
 HOST_EXPORT void xla_amd_host_destroy(void* host) { delete reinterpret_cast<HostState*>(host); }
 HOST_EXPORT const XLA_FFI_Api* xla_amd_host_api(void* host) { return &reinterpret_cast<HostState*>(host)->api; }
 HOST_EXPORT void xla_amd_host_set_stream(void* host, void* stream) { reinterpret_cast<HostState*>(host)->stream = stream; }
+
+// While `on`, frames of this host find a record extension on their invoke context, as a custom call
+// finds one while XLA records it into a command buffer.  Returns how often a handler has asked
+// for stream capture so far.
+HOST_EXPORT int xla_amd_host_set_recording(void* host, int on) {
+  HostState* h = reinterpret_cast<HostState*>(host);
+  h->recording = on != 0;
+  return h->stream_capture_requests;
+}
 
 // Copies the error's message into buf (NUL-terminated), destroys it and returns its code.
 HOST_EXPORT int xla_amd_host_take_error(XLA_FFI_Error* err, char* buf, size_t n) {

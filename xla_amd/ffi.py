@@ -226,6 +226,11 @@ class NativeHost:
         if err:
             raise FfiError(*self.take_error(err))
 
+    def set_recording(self, on):
+        """While on, frames of this host carry a record extension (what XLA attaches while it records
+        a command buffer).  Returns how many times a handler has asked for stream capture so far."""
+        return host_library().xla_amd_host_set_recording(self._h, int(bool(on)))
+
     def find_handler(self, target, platform="rocm"):
         return host_library().xla_amd_host_find_handler(self._h, target.encode(), platform.encode())
 
@@ -404,6 +409,8 @@ def host_library():
         L.xla_amd_host_register.argtypes = [C.c_void_p, C.c_void_p]
         L.xla_amd_host_find_handler.restype = C.c_void_p
         L.xla_amd_host_find_handler.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
+        L.xla_amd_host_set_recording.restype = C.c_int
+        L.xla_amd_host_set_recording.argtypes = [C.c_void_p, C.c_int]
         L.xla_amd_host_handler_traits.restype = C.c_int64
         L.xla_amd_host_handler_traits.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
         _host_lib = L
