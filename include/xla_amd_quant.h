@@ -222,29 +222,20 @@ XLA_AMD_EXPORT const char* xla_amd_last_error(void);
  * (e.g. "dequant_dot_decode_s4_m16"); for profiling scripts and tests. */
 XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
 
-/* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic process-wide
- * (value 0 restores the default).  Keys: "dequant_dot_kernel" (1 generic, 2 decode, also in passes of 64
- * tokens, 3 tiled whenever it covers the shape),
- * "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "dequant_dot_skew" (shares of K of a SIMD's
- * waves, oldest first, as decimal digits), "fp8_dot_kernel" (1 exact, 2 tiled),
- * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1: the
- * tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
+/* Tuning hook for benchmarks and tests: overrides a kernel-selection heuristic for calls made by the
+ * calling thread (value 0 restores the default); other threads are not affected.  Keys:
+ * "dequant_dot_kernel" (1 generic, 2 decode, also in passes of 64 tokens, 3 tiled whenever it covers
+ * the shape), "dequant_dot_vec", "dequant_dot_slices", "dequant_dot_waves", "dequant_dot_skew" (shares
+ * of K of a SIMD's waves, oldest first, as decimal digits), "dequant_dot_x" (1: s4 / s8 weights stay
+ * off the matrix-instruction-dequantising and the single-launch kernels), "dequant_dot_pair" (1: two
+ * workgroups per 256-channel strip wherever the shape allows, 2: never), "dequant_dot_share" (the
+ * first workgroup's sixteenths of K), "dequant_dot_depth" (ring depth 2 or 4), "dequant_dot_steps"
+ * (steps per wave of the single-launch s8 kernel: 1, 2, 4), "fp8_dot_kernel" (1 exact, 2 tiled),
+ * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1:
+ * the tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the
  * reference's cancellation to 2 bf16 ulp).  Returns 0, or -1 for an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
-
-/* Measurement aid for benchmarks (no counterpart in the reference): streams `bytes` (a multiple of 16,
- * buffers 16-byte aligned) from `src` on `stream` -- copied to `dst`, or only read when `dst` is
- * null -- with the access shape that reaches the highest HBM rate on MI355X, so that a benchmark can
- * print what a plain stream achieves on the same machine next to a kernel's own rate.  Returns 0 or
- * an XLA_FFI_Error_Code. */
-XLA_AMD_EXPORT int xla_amd_debug_stream(void* dst, const void* src, size_t bytes, void* stream);
-
-/* Self-check for tests (no counterpart in the reference; allocates and synchronises): evaluates the
- * epilogue's tanh -- whose quotient uses the f32 division sequence without operand scaling and
- * fix-up -- and a copy with the plain quotient on all 2^32 f32 bit patterns on the current device
- * and returns how many results differ (0 is the only acceptable answer), or -1 on a HIP error. */
-XLA_AMD_EXPORT long long xla_amd_debug_tanh_division_mismatches(void);
 
 #ifdef __cplusplus
 }

@@ -22,6 +22,13 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(ffi.EXPORTED_SYMBOLS), declared ^ set(ffi.EXPORTED_SYMBOLS)
     for sym in declared:
         assert getattr(lib, sym) is not None
+    # the test and benchmark aids live in a library of their own and nowhere in the product
+    header = open(os.path.join(ROOT, "include", "xla_amd_selfcheck.h")).read()
+    aids = set(re.findall(r"XLA_AMD_SELFCHECK_EXPORT[^;(]*?\b(xla_amd_\w+)\s*\(", header))
+    assert aids == set(ffi.SELFCHECK_SYMBOLS), aids ^ set(ffi.SELFCHECK_SYMBOLS)
+    for sym in aids:
+        assert getattr(ffi.selfcheck_library(), sym) is not None
+        assert not hasattr(lib, sym)
 
 
 def test_metadata_handshake():

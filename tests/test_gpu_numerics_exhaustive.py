@@ -13,4 +13,4 @@ def test_tanh_scaling_free_division_equals_ieee_division_on_every_f32():
     inputs: the epilogue keeps the reference's op-by-op value bit for bit."""
     print("[case] tanh division, all f32 inputs", flush=True)
     sys.stdout.flush()
-    assert ffi.library().xla_amd_debug_tanh_division_mismatches() == 0
+    assert ffi.selfcheck_library().xla_amd_selfcheck_tanh_division_mismatches() == 0

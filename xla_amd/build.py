@@ -3,6 +3,8 @@
 ``python -m xla_amd.build`` (or ``__graft_entry__.build()``) produces
   xla_amd/lib/libxla_amd_quant.so   kernels + launchers + XLA FFI handlers
   xla_amd/lib/libxla_amd_host.so    FFI call-frame host and HLO rewrite pass (host only)
+  xla_amd/lib/libxla_amd_selfcheck.so  test and benchmark aids (exhaustive numerics checks, stream
+                                    yardstick, empty kernel); not part of the product
 Nothing is compiled at import time; loaders fail loudly if a library is missing.
 """
 import os
@@ -15,7 +17,8 @@ LIB = os.path.join(ROOT, "xla_amd", "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 KERNEL_SOURCES = ["capi.hip", "rowwise_quantize.hip", "dequant_dot_decode.hip", "dequant_dot_decode_s4x.hip", "dequant_dot_decode_s8x.hip", "tiled_dot_mfma.hip",
-                  "self_check.hip", "ffi_handlers.cc"]
+                  "ffi_handlers.cc"]
+SELFCHECK_SOURCES = ["self_check.hip"]
 HOST_SOURCES = ["host/ffi_host.cc", "host/hlo_ir.cc", "host/quant_fusion_rewriter.cc",
                 "host/host_capi.cc"]
 
@@ -32,10 +35,10 @@ def _run(cmd):
     subprocess.run(cmd, check=True)
 
 
-def build_kernels(jobs=8):
+def build_kernels(jobs=8, sources=None, libname="libxla_amd_quant.so"):
     os.makedirs(LIB, exist_ok=True)
     objs, procs = [], []
-    for src in KERNEL_SOURCES:
+    for src in (sources or KERNEL_SOURCES):
         obj = os.path.join(LIB, os.path.basename(src) + ".o")
         cmd = [HIPCC, "-c", os.path.join(CSRC, src), "-o", obj] + DEVICE_FLAGS
         if src.endswith(".cc"):
@@ -50,9 +53,13 @@ def build_kernels(jobs=8):
     for p, s in procs:
         if p.wait() != 0:
             raise RuntimeError("hipcc failed on " + s)
-    out = os.path.join(LIB, "libxla_amd_quant.so")
+    out = os.path.join(LIB, libname)
     _run([HIPCC, "-shared", "-o", out] + objs + ["--offload-arch=gfx950", "-fPIC"])
     return out
+
+
+def build_selfcheck():
+    return build_kernels(sources=SELFCHECK_SOURCES, libname="libxla_amd_selfcheck.so")
 
 
 def build_host():
@@ -65,9 +72,9 @@ def build_host():
 
 
 def build_all():
-    return [build_kernels(), build_host()]
+    return [build_kernels(), build_selfcheck(), build_host()]
 
 
 if __name__ == "__main__":
     what = sys.argv[1] if len(sys.argv) > 1 else "all"
-    {"all": build_all, "kernels": build_kernels, "host": build_host}[what]()
+    {"all": build_all, "kernels": build_kernels, "host": build_host, "selfcheck": build_selfcheck}[what]()

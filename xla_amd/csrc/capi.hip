@@ -6,8 +6,6 @@
 #include <stdio.h>
 #include <string.h>
 
-#include <atomic>
-
 #include "launch.h"
 
 namespace xla_amd {
@@ -15,14 +13,16 @@ namespace {
 thread_local char g_error[512] = "";
 thread_local char g_kernel[128] = "";
 
+// Kernel-selection overrides of the calling thread (a launcher runs on the thread that calls it):
+// one thread's tuning sweep does not steer another thread's calls.
 struct Option {
   const char* key;
-  std::atomic<int> value;
+  int value;
 };
-Option g_options[] = {{"dequant_dot_kernel", {0}}, {"dequant_dot_vec", {0}},
-                      {"dequant_dot_slices", {0}}, {"dequant_dot_waves", {0}}, {"dequant_dot_skew", {0}}, {"dequant_dot_x", {0}}, {"dequant_dot_pair", {0}}, {"dequant_dot_share", {0}}, {"dequant_dot_depth", {0}}, {"dequant_dot_steps", {0}},
-                      {"fp8_dot_kernel", {0}},
-                      {"quantize_variant", {0}}, {"fp8_dot_layout", {0}}, {"tiled_epilogue", {0}}};
+thread_local Option g_options[] = {{"dequant_dot_kernel", 0}, {"dequant_dot_vec", 0},
+                      {"dequant_dot_slices", 0}, {"dequant_dot_waves", 0}, {"dequant_dot_skew", 0}, {"dequant_dot_x", 0}, {"dequant_dot_pair", 0}, {"dequant_dot_share", 0}, {"dequant_dot_depth", 0}, {"dequant_dot_steps", 0},
+                      {"fp8_dot_kernel", 0},
+                      {"quantize_variant", 0}, {"fp8_dot_layout", 0}, {"tiled_epilogue", 0}};
 }  // namespace
 
 int Fail(int code, const char* fmt, ...) {
@@ -46,24 +46,8 @@ int CheckLaunch(const char* what) {
 
 int GetOption(const char* key) {
   for (auto& o : g_options)
-    if (strcmp(o.key, key) == 0) return o.value.load(std::memory_order_relaxed);
+    if (strcmp(o.key, key) == 0) return o.value;
   return 0;
-}
-
-// Yardstick kernels for benchmarks: what a plain stream over HBM reaches on this machine.  One
-// 16-byte access per lane per launch-wide pass, workgroups of 256 owning contiguous 4 KiB, no grid
-// stride (the shape that measured fastest: 6.6-7.0 TB/s read, 6.2-6.4 TB/s copy on MI355X).
-typedef uint32_t StreamVec __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(256) void stream_read_kernel(const StreamVec* __restrict__ src, uint32_t* sink, size_t n) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  const StreamVec v = __builtin_nontemporal_load(src + i);
-  if ((v[0] ^ v[1] ^ v[2] ^ v[3]) == 0x9e3779b9u && sink) sink[0] = v[0];  // keeps the load alive
-}
-__global__ __launch_bounds__(256) void stream_copy_kernel(const StreamVec* __restrict__ src, StreamVec* __restrict__ dst, size_t n) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4);
@@ -107,25 +91,10 @@ size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
 const char* xla_amd_last_error(void) { return xla_amd::g_error; }
 const char* xla_amd_last_kernel(void) { return xla_amd::g_kernel; }
 
-int xla_amd_debug_stream(void* dst, const void* src, size_t bytes, void* stream) {
-  if (!src || bytes == 0 || bytes % 16 != 0 || ((uintptr_t)src % 16) != 0 || ((uintptr_t)dst % 16) != 0 ||
-      bytes / 16 > 0x7fffffffull * 256)
-    return xla_amd::Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "debug_stream: needs 16-byte aligned buffers and size");
-  const size_t n = bytes / 16;
-  const dim3 grid((unsigned)((n + 255) / 256));
-  if (dst)
-    hipLaunchKernelGGL(xla_amd::stream_copy_kernel, grid, dim3(256), 0, (hipStream_t)stream,
-                       (const xla_amd::StreamVec*)src, (xla_amd::StreamVec*)dst, n);
-  else
-    hipLaunchKernelGGL(xla_amd::stream_read_kernel, grid, dim3(256), 0, (hipStream_t)stream,
-                       (const xla_amd::StreamVec*)src, (uint32_t*)nullptr, n);
-  return xla_amd::CheckLaunch("debug_stream");
-}
-
 int xla_amd_debug_set_option(const char* key, int value) {
   for (auto& o : xla_amd::g_options)
     if (strcmp(o.key, key) == 0) {
-      o.value.store(value, std::memory_order_relaxed);
+      o.value = value;
       return 0;
     }
   return -1;

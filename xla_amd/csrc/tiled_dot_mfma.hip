@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "device_numerics.h"
@@ -743,14 +744,19 @@ __global__ void store_u32_kernel(uint32_t* dst, uint32_t value) { *dst = value; 
 template <int KIND, bool OUT_F8 = false>
 int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
   constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow + (KIND == kFp8MX ? 4096 : 0);  // 128 KiB (+ scales)
-  static bool configured = false;  // per kernel instantiation; benign if two threads race
-  if (!configured) {
+  // per kernel instantiation and device: one bit per device ordinal; two threads that race both set
+  // the attribute to the same value, which is harmless, and neither launches before it is set
+  static std::atomic<unsigned long long> configured{0};
+  int device = 0;
+  (void)hipGetDevice(&device);
+  const unsigned long long bit = 1ull << (device & 63);
+  if (!(configured.load(std::memory_order_acquire) & bit)) {
     hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND, OUT_F8>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
     if (e != hipSuccess)
       return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", what, kLds,
                   hipGetErrorString(e));
-    configured = true;
+    configured.fetch_or(bit, std::memory_order_release);
   }
   dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
   hipLaunchKernelGGL((tiled_dot_kernel<KIND, OUT_F8>), grid, dim3(512), kLds, stream, tp);

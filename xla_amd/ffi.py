@@ -25,8 +25,9 @@ EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
     "xla_amd_launch_fp8_scaled_dot",
     "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
     "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
-    "xla_amd_debug_set_option", "xla_amd_debug_stream",
-    "xla_amd_debug_tanh_division_mismatches"]
+    "xla_amd_debug_set_option"]
+SELFCHECK_SYMBOLS = ["xla_amd_selfcheck_tanh_division_mismatches", "xla_amd_selfcheck_stream",
+                     "xla_amd_selfcheck_launch_empty"]
 
 STAGE_INSTANTIATE, STAGE_PREPARE, STAGE_INITIALIZE, STAGE_EXECUTE, STAGE_RECORD = range(5)
 ATTR_ARRAY, ATTR_DICTIONARY, ATTR_SCALAR, ATTR_STRING = 1, 2, 3, 4
@@ -265,9 +266,6 @@ def library():
         L.xla_amd_last_error.restype = C.c_char_p
         L.xla_amd_last_kernel.restype = C.c_char_p
         L.xla_amd_debug_set_option.argtypes = [C.c_char_p, C.c_int]
-        L.xla_amd_debug_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
-        L.xla_amd_debug_tanh_division_mismatches.restype = C.c_longlong
-        L.xla_amd_debug_tanh_division_mismatches.argtypes = []
         L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
         for sym in ("xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch"):
@@ -456,11 +454,38 @@ def last_kernel():
     return library().xla_amd_last_kernel().decode()
 
 
+SELFCHECK_LIB_PATH = os.path.join(_LIB_DIR, "libxla_amd_selfcheck.so")
+_selfcheck_lib = None
+
+
+def selfcheck_library():
+    """Test and benchmark aids (exhaustive numerics checks, HBM stream yardstick, empty kernel): a
+    library of their own, because unlike the product they allocate and synchronise."""
+    global _selfcheck_lib
+    if _selfcheck_lib is None:
+        if not os.path.exists(SELFCHECK_LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m xla_amd.build selfcheck`" % SELFCHECK_LIB_PATH)
+        L = C.CDLL(SELFCHECK_LIB_PATH)
+        L.xla_amd_selfcheck_tanh_division_mismatches.restype = C.c_longlong
+        L.xla_amd_selfcheck_tanh_division_mismatches.argtypes = []
+        L.xla_amd_selfcheck_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.xla_amd_selfcheck_launch_empty.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        _selfcheck_lib = L
+    return _selfcheck_lib
+
+
 def debug_stream(dst_ptr, src_ptr, nbytes, stream):
-    """Launches the library's yardstick stream kernel (copy, or read only when dst_ptr is 0/None)."""
-    rc = library().xla_amd_debug_stream(dst_ptr or None, src_ptr, nbytes, stream)
-    if rc != 0:
-        raise RuntimeError(library().xla_amd_last_error().decode())
+    """Plain HBM stream (copy, or read-only with dst None) on `stream`: the benchmark's yardstick."""
+    rc = selfcheck_library().xla_amd_selfcheck_stream(dst_ptr or None, src_ptr, nbytes, stream)
+    if rc:
+        raise RuntimeError("xla_amd_selfcheck_stream failed: %d" % rc)
+
+
+def launch_empty(stream, count, workgroups=1):
+    """`count` launches of a kernel that does nothing, back to back on `stream`."""
+    rc = selfcheck_library().xla_amd_selfcheck_launch_empty(stream, count, workgroups)
+    if rc:
+        raise RuntimeError("xla_amd_selfcheck_launch_empty failed: %d" % rc)
 
 
 def set_option(key, value):
