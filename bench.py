@@ -10,12 +10,20 @@ the benchmark's shapes and distributions, and resident in HBM before the timed r
 
 Prints ONE JSON line: `value` = algorithmic bytes of a step / wall time per step (GB/s);
 `roofline` = the step's slowest kernel against the 8 TB/s HBM peak, timed with events on the
-launch stream; `cpu_baseline` = the CPU oracle on a column slice of the same workload;
-`kernels` / `other_configs` = every kernel of the step and the four other configurations.
+launch stream; `cpu_baseline` = the CPU oracle on the same workload; `kernels` = every kernel of
+the step; `other_configs` = the four other configurations, each with a `roofline` and a
+`cpu_baseline` of its own (the oracle on a stated sample of the same shape); `launch_floor_us` =
+what a kernel that does nothing costs per launch in the same back-to-back measurement.
+
+`traffic` figures (HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs) are read
+from profiles/hbm_traffic_per_launch.md, which names the hash of the kernel sources it was measured
+on; when the sources here hash differently the figures are stale and `traffic` is null.
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -25,10 +33,38 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 HBM_PEAK_XLA_GBS = 6810.0      # what XLA's own device file assumes (mi350.txtpb:28)
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}
-# HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
-# this script, each scaled by what the same counter read for the --calibrate-copy kernel (figures
-# and factors: profiles/decode_c2_hbm_traffic.md).  None where no such run has been made.
-MEASURED_TRAFFIC_BYTES = {"C2 M=64": 137883648, "C2 M=32": 131388569}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.md")
+
+
+def kernel_sources_hash():
+    """sha256 over the device sources and headers, in path order: identifies what a profile measured."""
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "xla_amd", "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        h.update(open(f, "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic():
+    """workload -> HBM bytes per launch from the committed profile summary; {} when that summary
+    was measured on other kernel sources (or is missing)."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return {}
+    m = re.search(r"kernel sources sha256: `?([0-9a-f]{64})`?", text)
+    if not m or m.group(1) != kernel_sources_hash():
+        return {}
+    table = {}
+    for line in text.splitlines():
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 5 and re.fullmatch(r"\d+", cells[-1]):
+            table[cells[0]] = int(cells[-1])
+    return table
+
+
 K2, N2, GROUP2 = 8192, 28672, 128
 MS2 = (1, 8, 32, 64)
 
@@ -115,6 +151,7 @@ def main():
     step_bytes = sum(c2_bytes(m) for m in MS2)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    traffic = measured_traffic()
     kernels = []
     for m, c in zip(MS2, calls):
         one = ffi.Replay([(c.target, c.frame)])
@@ -123,23 +160,30 @@ def main():
         gbs = c2_bytes(m) / (ms * 1e-3) / 1e9
         kernels.append({"workload": "C2 M=%d" % m, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
                         "bytes": c2_bytes(m), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
-                        "TFLOP/s": round(2 * m * K2 * N2 / (ms * 1e-3) / 1e12, 2)})
+                        "TFLOP/s": round(2 * m * K2 * N2 / (ms * 1e-3) / 1e12, 2),
+                        "traffic": traffic.get("C2 M=%d" % m)})
     dom = max(kernels, key=lambda k: k["ms"])
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "workload": dom["workload"],
                 "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
                 "frac_of_xla_device_file_peak": round(dom["GB/s"] / HBM_PEAK_XLA_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dom["workload"]), "launch_ms": dom["ms"],
+                "traffic": dom["traffic"], "launch_ms": dom["ms"],
                 "algorithmic_bytes": dom["bytes"],
                 "device_copy_GB/s": round(copy_gbs, 1), "device_read_GB/s": round(read_gbs, 1),
                 "frac_of_device_read_rate": round(dom["GB/s"] / read_gbs, 4)}
 
-    # ---- the other four configurations (informational) -----------------------------------------
+    # ---- the floor under every one-kernel figure: a kernel that does nothing, launched the same way
+    st = torch.cuda.current_stream().cuda_stream
+    floor_ms = ev_time(lambda: ffi.launch_empty(st, 50, 256), 4, warm=2) / 50
+
+    # ---- the other four configurations, each with its own roofline and CPU baseline ---------------
+    import numpy as np
     other = []
+    cpu_legs = {}   # workload -> function returning the cpu_baseline dict (run after the GPU part)
     if not args.skip_other:
-        def entry(name, call, bytes_, flops, bound, dtype=None):
+        def entry(key, name, call, bytes_, flops, bound, dtype=None):
             # the half-millisecond kernels get 20 ms of launches to settle the clocks before timing
-            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=40 if flops else 1)
-            e = {"workload": name, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
+            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=40 if bound == "mfma" else 2)
+            e = {"workload": name, "key": key, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
                  "GB/s": round(bytes_ / (ms * 1e-3) / 1e9, 1)}
             e["frac_hbm"] = round(e["GB/s"] / HBM_PEAK_GBS, 4)
             if flops:
@@ -147,11 +191,19 @@ def main():
                 if dtype:
                     e["frac_mfma"] = round(e["TFLOP/s"] / MFMA_PEAK_TFLOPS[dtype], 4)
             e["bound"] = bound
+            if bound == "hbm":
+                e["roofline"] = {"bound": "hbm", "achieved": e["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": e["frac_hbm"], "traffic": traffic.get(key), "algorithmic_bytes": bytes_}
+            else:
+                e["roofline"] = {"bound": "mfma", "achieved": e["TFLOP/s"], "peak": MFMA_PEAK_TFLOPS[dtype],
+                                 "unit": "TFLOP/s", "frac": e["frac_mfma"], "traffic": traffic.get(key),
+                                 "algorithmic_flops": flops}
+            e["cpu_baseline"] = None
             other.append(e)
 
         # C2's weights at a prefill-sized token count (informational: the tiled s4 kernel)
         lhs2k = torch.randn((2048, K2), device=dev).to(torch.bfloat16)
-        entry("C2 weights, 2048 tokens (s4 prefill)",
+        entry("C2 prefill", "C2 weights, 2048 tokens (s4 prefill)",
               ops.dequant_dot(lhs2k, w_packed, scales, bias, weight_dtype="s4", weight_shape=(K2, N2),
                               epilogue="BIAS_SILU", dequant_type="bf16", build_only=True),
               c2_bytes(2048), 2 * 2048 * K2 * N2, "mfma", "bf16")
@@ -160,13 +212,13 @@ def main():
         a = torch.randn((16, 4096), device=dev).to(torch.bfloat16)
         w8 = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
         sc = torch.empty((4096,), device=dev).uniform_(1e-3, 1e-2)
-        entry("C1 s8 [16,4096]x[4096,4096]", ops.dequant_dot(a, w8, sc, build_only=True),
+        entry("C1", "C1 s8 [16,4096]x[4096,4096]", ops.dequant_dot(a, w8, sc, build_only=True),
               4096 * 4096 + 2 * 16 * 4096 * 2 + 4096 * 4, 2 * 16 * 4096 * 4096, "hbm")
         # C4: RMSNorm + rowwise fp8 quantize
         x = torch.randn((16384, 8192), device=dev)
         x = torch.where(torch.rand_like(x) < 0.01, x * 50, x).to(torch.bfloat16)
         g = torch.empty((8192,), device=dev).uniform_(0.5, 1.5).to(torch.bfloat16)
-        entry("C4 rmsnorm+quantize [16384,8192]", ops.rowwise_quantize_fp8(x, g, build_only=True),
+        entry("C4", "C4 rmsnorm+quantize [16384,8192]", ops.rowwise_quantize_fp8(x, g, build_only=True),
               16384 * 8192 * 3 + 16384 * 4 + 8192 * 2, 0, "hbm")
         del x
         # C3: fp8 scaled dot + bias + GELU
@@ -174,20 +226,28 @@ def main():
         b8 = (torch.randn((8192, 8192), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
         s64 = torch.full((), 1 / 64, device=dev)
         b3 = torch.randn((8192,), device=dev).to(torch.bfloat16)
-        entry("C3 fp8 [8192,8192]x[8192,8192] (rhs [K,N], as in the HLO)",
+        c3_bytes, c3_flops = 2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3
+        entry("C3", "C3 fp8 [8192,8192]x[8192,8192] (rhs [K,N], as in the HLO)",
               ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", build_only=True),
-              2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
-        entry("C3 fp8, rhs given as [N,K]",
+              c3_bytes, c3_flops, "mfma", "fp8")
+        entry("C3 nk", "C3 fp8, rhs given as [N,K]",
               ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", rhs_contracting_dim=1,
                                  build_only=True),
-              2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+              c3_bytes, c3_flops, "mfma", "fp8")
+        # the reference's own test spelling: every op bf16-typed (gemm_rewriter_fp8_test.cc:1110-1141);
+        # power-of-two scales keep it on the tiled kernel, with an extra rounding per epilogue op
+        s64b = torch.full((), 1 / 64, device=dev)
+        entry("C3 bf16-typed", "C3 fp8 with bf16-typed dequantise, dot and epilogue ops",
+              ops.fp8_scaled_dot(a8, b8, s64b, s64b, b3, epilogue="BIAS_GELU", dequant_type="bf16", dot_type="bf16",
+                                 epilogue_type="bf16", build_only=True),
+              c3_bytes, c3_flops, "mfma", "fp8")
         # the same call with GELU from its closed form (opt-in: the far negative tail then differs
         # from the reference's own cancellation by more than 2 bf16 ulp of results below 1e-5)
         ffi.set_option("tiled_epilogue", 1)
         try:
-            entry("C3 fp8 (rhs [K,N]), opt-in closed-form GELU",
+            entry("C3 closed form", "C3 fp8 (rhs [K,N]), opt-in closed-form GELU: fails the 2-ulp rule in the far tail",
                   ops.fp8_scaled_dot(a8, b8, s64, s64, b3, epilogue="BIAS_GELU", build_only=True),
-                  2 * 8192 * 8192 + 8192 * 8192 * 2 + 8192 * 2, 2 * 8192 ** 3, "mfma", "fp8")
+                  c3_bytes, c3_flops, "mfma", "fp8")
         finally:
             ffi.set_option("tiled_epilogue", 0)
         del a8, b8
@@ -195,19 +255,18 @@ def main():
         a5 = torch.randn((8, 512, 4096), device=dev).to(torch.bfloat16)
         w5 = torch.randint(-127, 128, (8, 4096, 14336), dtype=torch.int8, device=dev)
         s5 = torch.empty((8, 14336), device=dev).uniform_(1e-3, 1e-2)
-        entry("C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, scale_group_size=0, build_only=True),
+        entry("C5", "C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, scale_group_size=0, build_only=True),
               8 * (4096 * 14336 + 512 * 4096 * 2 + 14336 * 4 + 512 * 14336 * 2),
               2 * 8 * 512 * 4096 * 14336, "mfma", "bf16")
         del a5, w5
 
-    # ---- CPU baseline: the oracle on a column slice of the same workload -------------------------
+    # ---- CPU baselines: the oracle on the same workload, or on a stated sample of it ------------
     cpu = None
     if not args.skip_cpu:
-        import numpy as np
         from oracle import oracle
-        from xla_amd import workloads
-        ncols = N2  # the whole workload: around ten seconds on 16 host threads
-        wl = workloads.c2_s4_group(M=max(MS2), K=K2, N=ncols)  # weights, scales, bias: generated once
+        from xla_amd import dtypes, workloads
+        cores = oracle.num_threads()
+        wl = workloads.c2_s4_group(M=max(MS2), K=K2, N=N2)  # weights, scales, bias: generated once
         t_cpu, b_cpu = 0.0, 0
         for m in MS2:
             lhs = np.ascontiguousarray(wl["lhs"][:m])
@@ -216,11 +275,51 @@ def main():
                                bias=wl["bias"], group=GROUP2, epilogue="silu")
             t_cpu += time.perf_counter() - t1
             b_cpu += c2_bytes(m)
-        cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(),
+        cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": cores,
                "kind": "port",
-               "sample": "C2 at M=1,8,32,64 on %d of %d output channels (full K), %.2f s of "
+               "sample": "C2 at M=1,8,32,64 on all %d output channels (full K), %.2f s of "
                          "CPU time; scalar restatement of the XLA CPU backend's op-by-op semantics, "
-                         "OpenMP over output channels" % (ncols, N2, t_cpu)}
+                         "OpenMP over output channels" % (N2, t_cpu)}
+        del wl
+
+        def timed(fn):
+            t1 = time.perf_counter()
+            fn()
+            return time.perf_counter() - t1
+
+        def base(value, unit, sample):
+            return {"value": value, "unit": unit, "cores": cores, "kind": "port", "sample": sample}
+
+        by_key = {e["key"]: e for e in other}
+        if "C1" in by_key:
+            w = workloads.c1_s8_channel()
+            t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))
+            by_key["C1"]["cpu_baseline"] = base(round(w["algorithmic_bytes"] / t / 1e9, 3), "GB/s",
+                                                "the whole [16,4096]x[4096,4096] workload, %.2f s" % t)
+        if "C2 prefill" in by_key:
+            w = workloads.c2_s4_group(M=64, K=K2, N=4096)
+            t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16",
+                                                 bias=w["bias"], group=GROUP2, epilogue="silu"))
+            by_key["C2 prefill"]["cpu_baseline"] = base(round(2 * 64 * K2 * 4096 / t / 1e12, 4), "TFLOP/s",
+                                                        "64 of 2048 tokens on 4096 of %d channels (full K), %.2f s" % (N2, t))
+        if "C4" in by_key:
+            w = workloads.c4_quantize(rows=8192, cols=8192)
+            t = timed(lambda: oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6))
+            by_key["C4"]["cpu_baseline"] = base(round(w["algorithmic_bytes"] / t / 1e9, 3), "GB/s",
+                                                "8192 of 16384 rows (all 8192 columns), %.2f s" % t)
+        c3_keys = [k for k in ("C3", "C3 nk", "C3 bf16-typed") if k in by_key]
+        if c3_keys:
+            w = workloads.c3_fp8(1024, 8192, 2048)
+            t = timed(lambda: oracle.fp8_scaled_dot(w["a"], w["b"], w["a_scale"], w["b_scale"], bias=w["bias"],
+                                                    epilogue="gelu_tanh"))
+            for k in c3_keys:
+                by_key[k]["cpu_baseline"] = base(round(2 * 1024 * 8192 * 2048 / t / 1e12, 4), "TFLOP/s",
+                                                 "1024 of 8192 rows x 2048 of 8192 channels (full K), f32-typed ops, %.2f s" % t)
+        if "C5" in by_key:
+            w = workloads.c5_s8_batched(B=1, M=64, K=4096, N=14336)
+            t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))
+            by_key["C5"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
+                                                "1 of 8 batches, 64 of 512 tokens (full K and N), %.2f s" % t)
 
     out = {
         "metric": "quant-dot HBM GB/s on the s4 group-128 decode dequantize-dot (% of MI355X roofline) "
@@ -234,6 +333,9 @@ def main():
                    "boundary": "XLA FFI handler xla_amd_dequant_dot via native call-frame replay"},
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "other_configs": other,
         "frac_of_hbm_peak_whole_step": round(value / HBM_PEAK_GBS, 4),
+        "launch_floor_us": round(floor_ms * 1e3, 3),
+        "kernel_sources_sha256": kernel_sources_hash(),
+        "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT) if traffic else None,
     }
     print(json.dumps(out))
 
