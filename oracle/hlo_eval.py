@@ -144,6 +144,11 @@ def evaluate(module_json, args):
             v = _round(np.abs(np.asarray(x[0], np.float32)), ty)
         elif op == "sqrt":
             v = _round(np.sqrt(np.asarray(x[0], np.float32)), ty)
+        elif op == "rsqrt":
+            # the portable definition (xla/codegen/intrinsic/rsqrt.cc:178-193): 1 / sqrt(x), each op rounded.
+            # PARITY UNPINNED against hosts that take the x86 approximation instruction plus Newton steps
+            with np.errstate(all="ignore"):
+                v = _round(np.float32(1) / np.sqrt(np.asarray(x[0], np.float32)), ty)
         elif op == "exponential":
             v = _round(O.exp_f32(np.asarray(x[0], np.float32)), ty)
         elif op == "tanh":

@@ -115,6 +115,9 @@ def test_c4(oracle, rows, cols):
     q_ref, s_ref = oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6)
     assert np.array_equal(s.view(np.uint32), s_ref.view(np.uint32))
     assert np.array_equal(q, q_ref)
+    # the rsqrt spelling under its portable definition 1 / sqrt: the same bits
+    q2, s2 = run_module(hm.c4_quantize(rows, cols, rsqrt=True), [w["x"], w["gamma"]])
+    assert np.array_equal(q2, q_ref) and np.array_equal(s2.view(np.uint32), s_ref.view(np.uint32))
 
 
 def test_c5(oracle):

@@ -209,6 +209,15 @@ def test_c4_quantize_rmsnorm_and_plain():
     check(new, r"custom-call\(%x\)", r"rmsnorm = false")
     # reduce-max seeded with 0 instead of -inf is the same amax of absolute values
     assert hlo.rewrite(hm.c4_quantize(rmsnorm=False).replace("constant(-inf)", "constant(0)"))[1]
+    # the reciprocal root as one rsqrt instruction: the same call, the same attributes (the CPU
+    # backend's portable definition of rsqrt is 1 / sqrt, xla/codegen/intrinsic/rsqrt.cc:178-193)
+    new_r, rw_r, rf_r = hlo.rewrite(hm.c4_quantize(rsqrt=True))
+    assert rw_r == ["q -> xla_amd.rowwise_quantize_fp8 [rmsnorm]"] and rf_r == []
+    assert new_r == hlo.rewrite(hm.c4_quantize())[0]
+    assert "rsqrt" in hm.c4_quantize(rsqrt=True) and "rsqrt" not in new_r
+    # rsqrt of something else is not the pattern
+    bad = hm.c4_quantize(8, 64, rsqrt=True).replace("rsqrt(%ms_eps)", "rsqrt(%ms)")
+    assert hlo.rewrite(bad)[1] == [] and "not the RMSNorm form" in hlo.rewrite(bad)[2][0]
 
 
 def test_c5_batched_s8():

@@ -666,11 +666,15 @@ bool RewriteQuantize(const Module& mod, Computation* comp, Instr* q, RewriteLog*
       if (ConvertFrom(gsrc, "bf16", &g) &&
           BinaryWith(t, "multiply", [&](Instr* b) { return BroadcastAlong(b, {0}, &rinv); }, &xf) &&
           ConvertFrom(xf, "bf16", &xin)) {
-        // rinv = 1 / sqrt(sum(xf*xf)/C + eps)
+        // rinv = 1 / sqrt(sum(xf*xf)/C + eps), or the same value spelled rsqrt(...): the CPU backend
+        // defines rsqrt as 1 / sqrt(x) wherever it does not use the x86 approximation instruction
+        // (xla/codegen/intrinsic/rsqrt.cc:178-193) and refines that approximation towards the same
+        // value (rsqrt.cc:195-224); the custom call computes the IEEE 1 / sqrt(x) for both spellings
         Instr *one, *rt;
-        if (Binary(rinv, "divide", &one, &rt) && IsConst(one, 1.0) && rt->Is("sqrt")) {
+        const bool as_divide = Binary(rinv, "divide", &one, &rt) && IsConst(one, 1.0) && rt->Is("sqrt");
+        if (as_divide || rinv->Is("rsqrt")) {
           Instr* ms = nullptr;
-          Instr* me = rt->operands[0];
+          Instr* me = as_divide ? rt->operands[0] : rinv->operands[0];
           if (BinaryWith(me, "add", [&](Instr* b) { return ConstScalar(b, &eps); }, &ms)) {
             Instr *ssum = nullptr, *cnt = nullptr;
             double cv = 0;
@@ -689,7 +693,7 @@ bool RewriteQuantize(const Module& mod, Computation* comp, Instr* q, RewriteLog*
         }
       }
     }
-    if (!rms) return refuse("y is computed from a multiply that is not the RMSNorm form x * (1/sqrt(mean(x^2)+eps)) * gamma");
+    if (!rms) return refuse("y is computed from a multiply that is not the RMSNorm form x * (1/sqrt(mean(x^2)+eps)) * gamma (or rsqrt of the same)");
   }
   if (x->shape.dtype != "bf16") return refuse("input must be bf16");
 

@@ -191,9 +191,13 @@ def c3_fp8_f8_result(M=8192, K=8192, N=8192, multiply=False, vector_scales=False
 """
 
 
-def c4_quantize(rows=16384, cols=8192, rmsnorm=True, eps=1e-6):
-    """RMSNorm (f32 math, bf16 result) -> per-row amax -> scale = amax/448 -> clamp -> f8e4m3fn."""
+def c4_quantize(rows=16384, cols=8192, rmsnorm=True, eps=1e-6, rsqrt=False):
+    """RMSNorm (f32 math, bf16 result) -> per-row amax -> scale = amax/448 -> clamp -> f8e4m3fn.
+    rsqrt: the reciprocal root spelled as one rsqrt instruction instead of 1 / sqrt."""
     R, C = rows, cols
+    root = (f"  %rinv = f32[{R}] rsqrt(%ms_eps)\n" if rsqrt else
+            f"  %rt = f32[{R}] sqrt(%ms_eps)\n  %one = f32[] constant(1)\n"
+            f"  %one_b = f32[{R}] broadcast(%one), dimensions={{}}\n  %rinv = f32[{R}] divide(%one_b, %rt)\n")
     if rmsnorm:
         norm = f"""  %gamma = bf16[{C}] parameter(1)
   %x_f32 = f32[{R},{C}] convert(%x)
@@ -206,11 +210,7 @@ def c4_quantize(rows=16384, cols=8192, rmsnorm=True, eps=1e-6):
   %eps = f32[] constant({eps!r})
   %eps_b = f32[{R}] broadcast(%eps), dimensions={{}}
   %ms_eps = f32[{R}] add(%ms, %eps_b)
-  %rt = f32[{R}] sqrt(%ms_eps)
-  %one = f32[] constant(1)
-  %one_b = f32[{R}] broadcast(%one), dimensions={{}}
-  %rinv = f32[{R}] divide(%one_b, %rt)
-  %rinv_b = f32[{R},{C}] broadcast(%rinv), dimensions={{0}}
+{root}  %rinv_b = f32[{R},{C}] broadcast(%rinv), dimensions={{0}}
   %xn = f32[{R},{C}] multiply(%x_f32, %rinv_b)
   %gamma_f32 = f32[{C}] convert(%gamma)
   %gamma_b = f32[{R},{C}] broadcast(%gamma_f32), dimensions={{1}}
