@@ -126,7 +126,7 @@ enum {
 
 typedef struct XlaAmdDequantDot {
   const void* lhs;     /* bf16 [batch,M,K] */
-  const void* weights; /* s8 [batch,K,N] or packed s4 */
+  const void* weights; /* s8 [batch,K,N] or packed s4 / u4 */
   const void* scales;  /* [batch or 1, K/group, N] */
   const void* bias;    /* [N] or NULL */
   void* out;           /* bf16 [batch,M,N] */
@@ -135,11 +135,14 @@ typedef struct XlaAmdDequantDot {
   int64_t batch, M, K, N;
   int64_t group;           /* K for per-channel scales */
   int64_t scale_batch;     /* 1 if the scales are shared by all batches, else batch */
-  int32_t weight_dtype;    /* S8 or S4 */
+  int32_t weight_dtype;    /* S8, S4 or U4 */
   int32_t scale_dtype;     /* F32 or BF16 */
   int32_t bias_dtype;      /* F32 or BF16 */
   int32_t dequant_type, dot_type, epilogue_type; /* F32 or BF16 */
   int32_t epilogue;        /* XLA_AMD_EPI_* */
+  /* U4 weights only, or NULL: one u4 zero point per scale, [scale_batch, K/group, N] packed two per
+   * byte like the weights; the dequantised weight is (w - zero_point) * scale */
+  const void* zero_points;
 } XlaAmdDequantDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);

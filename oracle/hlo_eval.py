@@ -100,8 +100,8 @@ def evaluate(module_json, args):
                 v = O.bf16_to_f32(v)
             elif ty in ("f8e4m3fn", "f8e8m0fnu"):
                 v = np.ascontiguousarray(v, np.uint8)
-            elif ty in ("s8", "s4"):
-                v = np.ascontiguousarray(v, np.int8)
+            elif ty in ("s8", "s4", "u4"):
+                v = np.ascontiguousarray(v, np.int8)   # unpacked values (u4: 0..15)
             else:
                 v = np.ascontiguousarray(v, np.float32)
             v = v.reshape(sh["dims"])
@@ -114,7 +114,7 @@ def evaluate(module_json, args):
                 s = O.f8e4m3fn_to_f32(s)
             if ty == "f8e4m3fn":
                 v = O.f32_to_f8e4m3fn(np.ascontiguousarray(s, np.float32))
-            elif ty in ("s8", "s4"):
+            elif ty in ("s8", "s4", "u4"):
                 v = np.ascontiguousarray(s, np.int8)
             else:
                 v = _round(np.asarray(s).astype(np.float32), ty)

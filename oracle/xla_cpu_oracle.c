@@ -361,12 +361,33 @@ XO_API uint16_t xo_epilogue_one(float acc, int dot_ty, int ep_ty, int has_bias,
  * or NULL.  out: bf16 [batch,M,N].  Additions over k in increasing k, one
  * rounding per product and per sum.  Returns 0, or -1 on a bad argument.
  */
+/* The same with 4-bit weights read as unsigned (w_unsigned != 0: u4, 0..15) and an optional zero
+ * point per scale (zero_points: u4 [batch,K/group,N] packed like the weights, or NULL):
+ *   W'[b,k,n] = round_mul_ty( round_mul_ty(f32(w) - f32(z)) * round_mul_ty(scale) )
+ * -- convert, subtract, multiply, each an op of type mul_ty; the difference of two integers below
+ * 16 is exact in either type. */
+XO_API int xo_dequant_dot_zp(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
+                             const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
+                             const void* bias, int bias_ty, int64_t batch, int64_t M,
+                             int64_t K, int64_t N, int64_t group, int dot_ty,
+                             int ep_ty, int epi, uint16_t* out);
+
 XO_API int xo_dequant_dot(const uint16_t* A, const void* w, int w_bits,
                           const void* scale, int scale_ty, int mul_ty,
                           const void* bias, int bias_ty, int64_t batch, int64_t M,
                           int64_t K, int64_t N, int64_t group, int dot_ty,
                           int ep_ty, int epi, uint16_t* out) {
+  return xo_dequant_dot_zp(A, w, w_bits, 0, NULL, scale, scale_ty, mul_ty, bias, bias_ty, batch, M, K, N,
+                           group, dot_ty, ep_ty, epi, out);
+}
+
+XO_API int xo_dequant_dot_zp(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
+                             const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
+                             const void* bias, int bias_ty, int64_t batch, int64_t M,
+                             int64_t K, int64_t N, int64_t group, int dot_ty,
+                             int ep_ty, int epi, uint16_t* out) {
   if (!(w_bits == 8 || w_bits == 4) || group <= 0 || K % group != 0) return -1;
+  if ((w_unsigned || zero_points) && w_bits != 4) return -1;
   const int64_t G = K / group;
   int rc = 0;
 #pragma omp parallel
@@ -387,13 +408,19 @@ XO_API int xo_dequant_dot(const uint16_t* A, const void* w, int w_bits,
             wi = ((const int8_t*)w)[idx];
           } else {
             uint8_t nib = (((const uint8_t*)w)[idx >> 1] >> (4 * (idx & 1))) & 0xF;
-            wi = (int8_t)(nib << 4) >> 4;
+            wi = w_unsigned ? (int)nib : (int8_t)(nib << 4) >> 4;
           }
           size_t sidx = ((size_t)b * G + k / group) * N + n;
           float s = scale_ty == XO_BF16 ? xo_bf16_to_f32(((const uint16_t*)scale)[sidx])
                                         : ((const float*)scale)[sidx];
           s = rnd(s, mul_ty);
-          float prod = (float)wi * s;
+          float wf = rnd((float)wi, mul_ty);
+          if (zero_points) {
+            float zf = rnd((float)((zero_points[sidx >> 1] >> (4 * (sidx & 1))) & 0xF), mul_ty);
+            volatile float d = wf - zf;
+            wf = rnd(d, mul_ty);
+          }
+          float prod = wf * s;
           col[k] = rnd(prod, mul_ty);
         }
         for (int64_t m = 0; m < M; ++m) {

@@ -161,6 +161,25 @@ def test_shape_validation_happens_before_any_launch():
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, a2, [(dtypes.BF16, FAKE, (4, 4))]))
 
 
+def test_zero_point_operand_is_recognised_by_its_type():
+    """lhs, weights, scales[, zero_points][, bias]: a U4 operand after the scales is the zero points."""
+    host = ffi.Host()
+    lhs, w4 = (dtypes.BF16, FAKE, (2, 64)), (dtypes.U4, FAKE, (64, 8))
+    sc, zp, bias = (dtypes.BF16, FAKE, (2, 8)), (dtypes.U4, FAKE, (2, 8)), (dtypes.BF16, FAKE, (8,))
+    out = [(dtypes.BF16, FAKE, (2, 8))]
+    with pytest.raises(ffi.FfiError, match="zero points go with U4 weights"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, (dtypes.S4, FAKE, (64, 8)), sc, zp], out))
+    with pytest.raises(ffi.FfiError, match="zero points must have the shape of the scales"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w4, sc, (dtypes.U4, FAKE, (4, 8))], out))
+    with pytest.raises(ffi.FfiError, match="a bias operand goes with a BIAS\\* epilogue"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w4, sc, zp, bias], out))
+    with pytest.raises(ffi.FfiError, match="five operands are lhs, weights, scales, zero_points \\(U4\\), bias"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w4, sc, bias, bias], out,
+                                                    {"epilogue": ffi.Attr.str("BIAS")}))
+    with pytest.raises(ffi.FfiError, match="Wrong buffer dtype"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, (dtypes.U8, FAKE, (64, 8)), sc], out))
+
+
 def test_record_stage_asks_for_stream_capture():
     """At the RECORD stage (XLA building a command buffer, custom_call_thunk.cc:577-684) a handler finds
     the record extension on its invoke context and asks for stream capture of its execute stage;

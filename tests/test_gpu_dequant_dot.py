@@ -24,10 +24,11 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
     (default: off whenever a strip width `vec` of the other kernels is asked for); pair: 1 takes the
     two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never."""
     lhs = dev_bf16(w["lhs"])
-    if w["weight_dtype"] == "s4":
+    if w["weight_dtype"] in ("s4", "u4"):
         wt = dev_u8(w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"]))
     else:
         wt = dev_s8(w["weights"])
+    zp = dev_u8(w["zero_points_packed"]) if w.get("zero_points_packed") is not None else None
     sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
     bias = None
     if w.get("bias") is not None:
@@ -43,7 +44,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
                               weight_shape=w["weight_shape"], epilogue=w["epilogue"],
                               dequant_type=w["dequant_type"], dot_type=w.get("dot_type", "f32"),
-                              epilogue_type=w.get("epilogue_type", "f32"),
+                              epilogue_type=w.get("epilogue_type", "f32"), zero_points=zp,
                               scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"])
         torch.cuda.synchronize()
     finally:
@@ -57,7 +58,7 @@ def oracle_dot(oracle, w):
     scale_ty = "bf16" if w["scales"].dtype == np.uint16 else "f32"
     wt = w["weights"]
     bits = 8
-    if w["weight_dtype"] == "s4":
+    if w["weight_dtype"] in ("s4", "u4"):
         wt, bits = (w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"])), 4
     epi = {"DEFAULT": "none", "BIAS": "none", "RELU": "relu", "BIAS_RELU": "relu", "GELU": "gelu_tanh",
            "BIAS_GELU": "gelu_tanh", "SILU": "silu", "BIAS_SILU": "silu"}[w["epilogue"]]
@@ -66,7 +67,8 @@ def oracle_dot(oracle, w):
                               scale_ty, w["dequant_type"], bias=bias,
                               bias_ty="bf16" if (bias is not None and bias.dtype == np.uint16) else "f32",
                               group=w["group"], dot_ty=w.get("dot_type", "f32"),
-                              ep_ty=w.get("epilogue_type", "f32"), epilogue=epi)
+                              ep_ty=w.get("epilogue_type", "f32"), epilogue=epi,
+                              unsigned=w["weight_dtype"] == "u4", zero_points=w.get("zero_points_packed"))
 
 
 def floor_for(w):
@@ -74,6 +76,9 @@ def floor_for(w):
     s = w["scales"]
     sv = (dtypes.bf16_to_f32(s) if s.dtype == np.uint16 else s).astype(np.float64)
     wi = np.abs(w["weights"].astype(np.float64))
+    if w.get("zero_points") is not None:   # the weights' magnitude is that of w - z
+        z = w["zero_points"].astype(np.float64)
+        wi = np.abs(w["weights"].astype(np.float64) - np.repeat(z.reshape(-1, z.shape[-1]), w["group"], axis=0).reshape(wi.shape))
     K = w["lhs"].shape[-1]
     if w["lhs"].ndim == 3:
         sv = sv.reshape(w["lhs"].shape[0], -1, sv.shape[-1])
@@ -544,3 +549,59 @@ def test_dequant_dot_error_paths():
         ops.dequant_dot(lhs, wt, torch.ones((5, 32), dtype=torch.float32, device="cuda"))
     out = ops.dequant_dot(torch.zeros((0, 64), dtype=torch.bfloat16, device="cuda"), wt, sc)
     assert out.shape == (0, 32)
+
+
+# ---- u4 weights with zero points -----------------------------------------------------------
+
+@pytest.mark.parametrize("M,K,N,group,vec,slices", [
+    (1, 4096, 1024, 128, 0, 0), (8, 2048, 768, 64, 4, 2), (16, 2048, 512, 32, 8, 1), (20, 1024, 640, 128, 4, 1),
+    (33, 1024, 512, 64, 0, 0), (64, 2048, 256, 128, 4, 2), (70, 1024, 512, 128, 0, 0), (5, 100, 42, 50, 0, 0)])
+def test_u4_zero_point_decode(oracle, M, K, N, group, vec, slices):
+    """Unsigned 4-bit weights with one zero point and one scale per group and channel, bf16-typed
+    convert / subtract / multiply: every decode strip width, K-slices, more than 64 tokens as
+    chunks, and a shape only the one-thread-per-output kernel takes."""
+    say("dequant_dot u4+zp M=%d K=%d N=%d group=%d vec=%d slices=%d" % (M, K, N, group, vec, slices))
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=group)
+    got, kern = run_dot(w, slices=slices, vec=vec)
+    if (K, N) == (100, 42):
+        assert kern == "dequant_dot_generic", kern
+    else:
+        assert kern.startswith("dequant_dot_decode_s4_") and (M <= 64 or kern.endswith(":x64")), kern
+    compare(oracle, w, got, "u4+zp %s" % kern)
+
+
+def test_u4_zero_point_one_hot_bit_exact(oracle):
+    """One-hot activations: every output is one dequantised weight bf16((w - z) * s), exactly --
+    the nibble order of weights and zero points, unsignedness, the group of each row."""
+    say("dequant_dot u4+zp one-hot")
+    K, N, group = 256, 256, 64
+    w = workloads.u4_zero_point_group(M=16, K=K, N=N, group=group)
+    w["weights"][:16, :16] = np.arange(16, dtype=np.int8)[:, None]
+    wu = w["weights"].astype(np.uint8)
+    w["weights_packed"] = (wu.reshape(-1)[0::2] | (wu.reshape(-1)[1::2] << 4)).astype(np.uint8)
+    w["bias"], w["epilogue"] = None, "DEFAULT"
+    diff = w["weights"].astype(np.float32) - np.repeat(w["zero_points"], group, axis=0).astype(np.float32)
+    want_all = dtypes.f32_to_bf16((diff * np.repeat(dtypes.bf16_to_f32(w["scales"]), group, axis=0)).astype(np.float32))
+    for m0 in range(0, K, 16):
+        a = np.zeros((16, K), np.float32)
+        a[np.arange(16), m0 + np.arange(16)] = 1.0
+        got, kern = run_dot(dict(w, lhs=dtypes.f32_to_bf16(a)), force_kernel=2)
+        assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want_all[m0:m0 + 16])), (kern, m0)
+
+
+@pytest.mark.parametrize("with_zero_points", [False, True])
+def test_u4_per_channel_f32_multiply(oracle, with_zero_points):
+    """u4 with one scale (and zero point) per output channel under an f32-typed multiply: the integers
+    (w - z) go through the matrix cores exactly and the scale multiplies the sum once."""
+    say("dequant_dot u4 per-channel f32 zero_points=%s" % with_zero_points)
+    M, K, N = 12, 1024, 384
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=K)
+    w["scales"] = dtypes.bf16_to_f32(w["scales"]).reshape(N)
+    w["dequant_type"] = "f32"
+    if not with_zero_points:
+        w["zero_points"] = w["zero_points_packed"] = None
+    else:
+        w["zero_points"] = w["zero_points"].reshape(1, N)
+    got, kern = run_dot(w, force_kernel=2)
+    assert kern.endswith("_factored"), kern
+    compare(oracle, w, got, "u4 per-channel %s" % kern)

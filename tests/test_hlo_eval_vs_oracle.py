@@ -125,3 +125,14 @@ def test_c5(oracle):
     got = run_module(hm.c5_s8_batched(2, 4, 64, 24), [w["lhs"], w["weights"], w["scales"]])
     ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
     assert np.array_equal(got, ref)
+
+
+def test_u4_zero_points(oracle):
+    """The asymmetric 4-bit module op by op (convert, subtract, multiply, each bf16-typed) against
+    the fused oracle function: bit for bit."""
+    w = workloads.u4_zero_point_group(M=3, K=128, N=24, group=32)
+    got = run_module(hm.u4_zero_point_group(3, 128, 24, 32),
+                     [w["lhs"], w["weights"], w["scales"], w["zero_points"].astype(np.int8), w["bias"]])
+    ref = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", bias=w["bias"],
+                             group=32, unsigned=True, zero_points=w["zero_points_packed"])
+    assert np.array_equal(got, ref)

@@ -483,3 +483,26 @@ def test_gelu_constants_are_held_to_128_epsilon_of_their_type(c1, ok):
     # a bf16 constant is as coarse as its type: 0.796875 is bf16(0.7978...), within 128 * 2^-7
     bf = hm.c3_fp8(16, 32, 16, typed="bf16").replace("constant(0.797884583)", "constant(0.796875)")
     assert hlo.rewrite(bf)[1] == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"]
+
+
+def test_u4_weights_with_zero_points():
+    """(convert(u4 w) - convert(u4 zero)) * scale, grouped: one call with the zero points as the
+    operand after the scales; near misses keep their reasons."""
+    text = hm.u4_zero_point_group(8, 256, 64, 64)
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, u4 with zero points]"] and rf == []
+    check(new, r"custom-call\(%lhs, %w, %scales, %zero, %bias\), custom_call_target=\"xla_amd.dequant_dot\"",
+          r"dequant_type = 16 : i32", r"scale_group_size = 64 : i64")
+    assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
+    # zero points of another shape than the scales
+    bad = text.replace("%zero = u4[4,64] parameter(3)", "%zero4 = u4[4,64] parameter(3)\n  %zero = u4[4,64] add(%zero4, %zero4)")
+    assert hlo.rewrite(bad)[1] == rw          # any u4 [G,N] value serves
+    # signed weights with zero points are not a pattern the kernels take
+    signed = text.replace("u4[256,64] parameter(1)", "s4[256,64] parameter(1)").replace("%w_g = u4[", "%w_g = s4[")
+    new2, rw2, rf2 = hlo.rewrite(signed)
+    assert rw2 == [] and any("zero points are taken with u4 weights only" in r for r in rf2)
+    # u4 without zero points
+    plain = hm.c2_s4_group(4, 256, 64, 64).replace("s4[", "u4[").replace("s8[", "u8[")
+    new3, rw3, rf3 = hlo.rewrite(plain)
+    assert rw3 == ["dot -> xla_amd.dequant_dot [BIAS_SILU, u4]"] and rf3 == []
+    check(new3, r"custom-call\(%lhs, %w, %scales, %bias\)")

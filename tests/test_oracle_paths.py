@@ -345,3 +345,46 @@ def test_quantize_zero_row_gives_nan_codes(oracle):
     x = np.zeros((1, 64), np.float32)
     q, s = oracle.rmsnorm_quantize_fp8(bf16(x), bf16(np.ones(64)), eps=1e-6)
     assert s[0] == 0.0 and np.all((q & 0x7F) == 0x7F)
+
+
+# ---- u4 weights with zero points ------------------------------------------------
+
+def _pack4(v):
+    v = np.ascontiguousarray(v, np.uint8).reshape(-1)
+    return (v[0::2] | (v[1::2] << 4)).astype(np.uint8)
+
+
+def test_u4_zero_point_dequantisation_one_hot_and_brute_force(oracle):
+    """(w - z) * s for unsigned 4-bit weights: one-hot activations read single dequantised weights
+    back (nibble order of weights AND zero points, the group a row belongs to, unsignedness, the
+    single bf16 rounding); a small dot against float64; and z = 8 turns u4 into s4 exactly."""
+    rng = np.random.default_rng(21)
+    K, N, g = 64, 24, 16
+    w = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    w[:16, 0] = np.arange(16)                      # every code in one column
+    z = rng.integers(0, 16, (K // g, N)).astype(np.uint8)
+    s32 = (rng.integers(128, 256, (K // g, N)) / 128.0 * np.exp2(rng.integers(-8, 2, (K // g, N)))).astype(np.float32)
+    s = dtypes.f32_to_bf16(s32)                    # exactly representable
+    eye = dtypes.f32_to_bf16(np.eye(K, dtype=np.float32))
+    got = oracle.dequant_dot(eye, _pack4(w), 4, s, "bf16", "bf16", group=g, unsigned=True, zero_points=_pack4(z))
+    diff = w.astype(np.float32) - np.repeat(z, g, axis=0).astype(np.float32)
+    want = dtypes.f32_to_bf16((diff * np.repeat(dtypes.bf16_to_f32(s), g, axis=0)).astype(np.float32))
+    assert np.array_equal(got, want)
+    # f32-typed multiply: no rounding of the product before the dot; one-hot rows still read it back,
+    # rounded once by the final convert
+    got32 = oracle.dequant_dot(eye, _pack4(w), 4, s32, "f32", "f32", group=g, unsigned=True, zero_points=_pack4(z))
+    assert np.array_equal(got32, dtypes.f32_to_bf16((diff * np.repeat(s32, g, axis=0)).astype(np.float32)))
+    # without zero points the unsigned code itself is the weight
+    got0 = oracle.dequant_dot(eye, _pack4(w), 4, s, "bf16", "bf16", group=g, unsigned=True)
+    assert np.array_equal(got0, dtypes.f32_to_bf16((w * np.repeat(dtypes.bf16_to_f32(s), g, axis=0)).astype(np.float32)))
+    # z = 8 everywhere is the signed reading of the same bits with the sign bit flipped
+    a = dtypes.f32_to_bf16(rng.standard_normal((5, K)).astype(np.float32))
+    z8 = np.full((K // g, N), 8, np.uint8)
+    as_u4 = oracle.dequant_dot(a, _pack4(w), 4, s, "bf16", "bf16", group=g, unsigned=True, zero_points=_pack4(z8))
+    as_s4 = oracle.dequant_dot(a, _pack4(w ^ 8), 4, s, "bf16", "bf16", group=g)
+    assert np.array_equal(as_u4, as_s4)
+    # a dot against float64 on the dequantised weights
+    got = dtypes.bf16_to_f32(oracle.dequant_dot(a, _pack4(w), 4, s, "bf16", "bf16", group=g, unsigned=True,
+                                                zero_points=_pack4(z))).astype(np.float64)
+    ref = dtypes.bf16_to_f32(a).astype(np.float64) @ dtypes.bf16_to_f32(want).astype(np.float64)
+    assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2)) < 2.0 ** -7

@@ -79,7 +79,7 @@ int xla_amd_launch_rowwise_quantize_fp8(const XlaAmdRowwiseQuantize* p, void* st
 
 size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, int64_t N,
                                            int32_t weight_dtype) {
-  return xla_amd::DequantDotDecodeWorkspaceBytes(batch, M, K, N, weight_dtype == XLA_FFI_DataType_S4);
+  return xla_amd::DequantDotDecodeWorkspaceBytes(batch, M, K, N, weight_dtype == XLA_FFI_DataType_S4 || weight_dtype == XLA_FFI_DataType_U4);
 }
 
 size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,

@@ -41,6 +41,10 @@ struct DecodeParams {
   int units_per_simd2;  // the finisher's units per SIMD; its class split is class_units[2..3]
   unsigned long long* flags;
   unsigned long long epoch;
+  // 4-bit weights are unsigned (u4, 0..15) and zero_points, if not null, holds one u4 value per
+  // scale ([scale_batch, K/group, N], packed like the weights): W' = (w - z) * scale
+  int w_unsigned;
+  const uint8_t* zero_points;
 };
 
 static __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {

@@ -101,6 +101,18 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
   for (int r = 0; r < 8; ++r) soff_w[r] = (uint32_t)r * pitch;
   const uint32_t voff_s = lane_live ? (uint32_t)n_lane * SSZ : kNowhere;
+  // u4 zero points: one nibble per scale, packed like the weights; the lane's NV channels are NV / 8
+  // dwords (4-bit weights give a lane at least 8 channels)
+  constexpr int ZW = WBITS == 4 ? (NV / 8 > 0 ? NV / 8 : 1) : 1;
+  const bool has_zp = WBITS == 4 && p.zero_points != nullptr;
+  const __amdgpu_buffer_rsrc_t rz =
+      make_rsrc(has_zp ? p.zero_points + (size_t)(p.scale_batched ? batch : 0) * groups * (p.N >> 1) : p.w,
+                has_zp ? (uint32_t)groups * (uint32_t)(p.N >> 1) : 0u);
+  const uint32_t voff_z = lane_live ? (uint32_t)(n_lane >> 1) : kNowhere;
+  // 4-bit values arrive as the f16 number 1024 + u (or 1024 + 16 u): u = w + 8 for s4 (one XOR also
+  // flips the nibble's sign bit), u = w for u4; what is subtracted again is 1024 + 8 resp. 1024 + z
+  const uint32_t c_even = p.w_unsigned ? 0x64006400u : 0x64086408u;
+  const uint32_t c_odd = p.w_unsigned ? 0x64006400u : 0x64806480u;
 
   floatx4 acc[NV][MT];
 #pragma unroll
@@ -124,6 +136,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   uint32_t wq[2][8][WORDS];
   uintx4 aq[2][MT];
   uint32_t sraw[2][SW];
+  uint32_t zraw[2][ZW];
   float sc[NV];  // kRounded: scale of each owned channel for the current group (s4: see compute)
   float cc[NV];  // s4: the constant term that removes the conversion offset
 
@@ -136,15 +149,17 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     const uint32_t va = voff_a + (uint32_t)k0 * 2u;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) aq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], va, 0, 0);
-    if (MODE == kRounded) {
+    if (MODE == kRounded || (WBITS == 4 && has_zp)) {
       if (GROUP32) {
         if (opens_group(k0)) {
           const uint32_t g = (uint32_t)min(k0, p.K - 1) / (uint32_t)p.group;  // scalar
-          buffer_load_words<SW>(rs, voff_s, g * (uint32_t)p.N * SSZ, sraw[buf]);
+          if (MODE == kRounded) buffer_load_words<SW>(rs, voff_s, g * (uint32_t)p.N * SSZ, sraw[buf]);
+          if (WBITS == 4 && has_zp) buffer_load_words<ZW>(rz, voff_z, g * (uint32_t)(p.N >> 1), zraw[buf]);
         }
       } else {
         const uint32_t g = (uint32_t)min(k0 + 8 * kb, p.K - 1) / (uint32_t)p.group;  // per lane
-        buffer_load_words<SW>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, sraw[buf]);
+        if (MODE == kRounded) buffer_load_words<SW>(rs, voff_s + g * (uint32_t)p.N * SSZ, 0, sraw[buf]);
+        if (WBITS == 4 && has_zp) buffer_load_words<ZW>(rz, voff_z + g * (uint32_t)(p.N >> 1), 0, zraw[buf]);
       }
     }
     const uint32_t vw = voff_w + (uint32_t)k0 * pitch;
@@ -167,19 +182,23 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) bop[mt] = __builtin_bit_cast(bf16x8, av[mt]);
-    if (MODE == kRounded && opens_group(k0)) {
+    if ((MODE == kRounded || (WBITS == 4 && has_zp)) && opens_group(k0)) {
       asm volatile("");  // a branch, not 2*NV selects per step
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
         const uint32_t* raw = sraw[buf];
-        float v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
-                             : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
+        float v = 1.0f;  // kFactored: the integers go through as they are
+        if (MODE == kRounded)
+          v = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(raw[j / 2]) : bf16lo_to_f32(raw[j / 2]))
+                         : bits_to_f32(raw[SCALE_BF16 ? 0 : j]);
         if (WBITS == 4) {
-          // nibble j of a dword arrives as the f16 value 1024 + u (even j) or 1024 + 16u (odd j),
-          // u = w + 8: w*s = (1024 + u)*s - 1032*s = (1024 + 16u)*(s/16) - 72*s, one fma each,
+          // nibble j of a dword arrives as the f16 value 1024 + u (even j) or 1024 + 16u (odd j);
+          // with zero point z (8 for s4, where u = w + 8):
+          // (u - z)*s = (1024 + u)*s - (1024 + z)*s = (1024 + 16u)*(s/16) - (64 + z)*s, one fma each,
           // exact for any scale with an 8-bit significand and |1040*s| finite
+          const float z = has_zp ? (float)((zraw[buf][j / 8] >> (4 * (j % 8))) & 0xfu) : (p.w_unsigned ? 0.0f : 8.0f);
           sc[j] = (j & 1) ? v * 0.0625f : v;
-          cc[j] = (j & 1) ? v * -72.0f : v * -1032.0f;
+          cc[j] = (j & 1) ? v * -(64.0f + z) : v * -(1024.0f + z);
         } else {
           sc[j] = v;
         }
@@ -200,15 +219,18 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
           for (int r = 0; r < 8; ++r) {
             const uint32_t x = sel < 2 ? wq[buf][r][q] : wq[buf][r][q] >> 8;
-            pr[r] = __builtin_bit_cast(halfx2, (sel & 1) ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a)
-                                                         : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+            pr[r] = __builtin_bit_cast(halfx2, (sel & 1) ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, c_odd, 0x6a)
+                                                         : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, c_even, 0x6a));
           }
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const int e = sel + 4 * half;
             const int j = q * 8 + e;
-            const float sj = MODE == kRounded ? sc[j] : ((e & 1) ? 0.0625f : 1.0f);
-            const float cj = MODE == kRounded ? cc[j] : ((e & 1) ? -72.0f : -1032.0f);
+            // (a factored multiply without zero points keeps its constants out of registers)
+            const bool from_regs = MODE == kRounded || has_zp;
+            const float z0 = p.w_unsigned ? 0.0f : 8.0f;
+            const float sj = from_regs ? sc[j] : ((e & 1) ? 0.0625f : 1.0f);
+            const float cj = from_regs ? cc[j] : ((e & 1) ? -(64.0f + z0) : -(1024.0f + z0));
             float f[8];
 #pragma unroll
             for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][half], sj, cj);
@@ -355,7 +377,11 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
       wi = (int8_t)p.w[e];
     } else {
       const uint32_t nib = (p.w[e >> 1] >> (4 * (e & 1))) & 0xfu;
-      wi = (int)(nib ^ 8u) - 8;
+      wi = p.w_unsigned ? (int)nib : (int)(nib ^ 8u) - 8;
+      if (p.zero_points) {
+        const size_t ze = sbase + (size_t)(k / p.group) * p.N + n;
+        wi -= (int)((p.zero_points[ze >> 1] >> (4 * (ze & 1))) & 0xfu);
+      }
     }
     float s = load_scale(p.scales, sbase + (size_t)(k / p.group) * p.N + n, p.scale_is_bf16);
     float wv = (float)wi * s;
@@ -486,9 +512,12 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
 // weights_shared: `batch` counts 64-token chunks of one [batch * M, K] activation matrix that all
 // use the same weights and scales (only the decode kernels take it).
 static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, bool weights_shared) {
-  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4;
+  const bool u4 = p.weight_dtype == XLA_FFI_DataType_U4;
+  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4 || u4;  // 4-bit weights, two per byte
   if (!s4 && p.weight_dtype != XLA_FFI_DataType_S8)
-    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: weights must be S4 or S8");
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: weights must be S4, U4 or S8");
+  if (p.zero_points && !u4)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: zero points come with U4 weights only");
   if (!IsF32OrBf16(p.scale_dtype) || !IsF32OrBf16(p.dequant_type) || !IsF32OrBf16(p.dot_type) ||
       !IsF32OrBf16(p.epilogue_type) || (p.bias && !IsF32OrBf16(p.bias_dtype)))
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: types must be F32 or BF16");
@@ -532,6 +561,8 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.epilogue = p.epilogue;
   dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
   dp.weights_shared = weights_shared;
+  dp.w_unsigned = u4;
+  dp.zero_points = (const uint8_t*)p.zero_points;
   const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
   const bool per_channel = p.group == p.K;
 
@@ -540,7 +571,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
                        ((uintptr_t)p.weights % 16 == 0);
   const bool mode_ok = mode == kRounded || per_channel;
 
-  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared) {
+  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
@@ -581,6 +612,8 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     for (int64_t b = 0; b < p.batch; ++b) {
       sub.weights = (const char*)p.weights + b * wbytes;
       sub.scales = (const char*)p.scales + b * sbytes;
+      if (p.zero_points)  // one nibble per scale
+        sub.zero_points = (const char*)p.zero_points + (sbytes ? b * ((size_t)(p.K / p.group) * p.N / 2) : 0);
       // the whole 64-token chunks go out as one launch with the chunk index in the grid (the
       // workgroups of all chunks then pack onto the CUs together), the remainder as a second one
       const int64_t whole = p.M / 64;
@@ -650,6 +683,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
       XLA_AMD_DECODE(4, 4, 3, kRounded, "dequant_dot_decode_s4_v4_m48_rounded")
       XLA_AMD_DECODE(4, 4, 4, kRounded, "dequant_dot_decode_s4_v4_m64_rounded")
       XLA_AMD_DECODE(4, 8, 1, kFactored, "dequant_dot_decode_s4_v8_m16_factored")
+      XLA_AMD_DECODE(4, 4, 1, kFactored, "dequant_dot_decode_s4_v4_m16_factored")
       XLA_AMD_DECODE(4, 4, 2, kFactored, "dequant_dot_decode_s4_v4_m32_factored")
       XLA_AMD_DECODE(4, 4, 3, kFactored, "dequant_dot_decode_s4_v4_m48_factored")
       XLA_AMD_DECODE(4, 4, 4, kFactored, "dequant_dot_decode_s4_v4_m64_factored")

@@ -356,12 +356,21 @@ extern "C" {
 
 XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Error* err;
-  if (Preamble(f, 3, 4, 1, 2, &err)) return err;
+  if (Preamble(f, 3, 5, 1, 2, &err)) return err;
   Decoder d{f};
   XLA_FFI_Buffer* lhs = d.Arg(0, Bit(XLA_FFI_DataType_BF16), 2, 3, "lhs");
-  XLA_FFI_Buffer* w = d.Arg(1, Bit(XLA_FFI_DataType_S8) | Bit(XLA_FFI_DataType_S4), 2, 3, "weights");
+  XLA_FFI_Buffer* w = d.Arg(1, Bit(XLA_FFI_DataType_S8) | Bit(XLA_FFI_DataType_S4) | Bit(XLA_FFI_DataType_U4), 2, 3,
+                            "weights");
   XLA_FFI_Buffer* sc = d.Arg(2, kFloatMask, 1, 3, "scales");
-  XLA_FFI_Buffer* bias = f->args.size > 3 ? d.Arg(3, kFloatMask, 1, 1, "bias") : nullptr;
+  // operands: lhs, weights, scales[, zero_points][, bias] -- a U4 operand after the scales is the
+  // zero points (one per scale), a float one the bias
+  const bool has_zp = f->args.size > 3 && f->args.types[3] == XLA_FFI_ArgType_BUFFER &&
+                      static_cast<XLA_FFI_Buffer*>(f->args.args[3])->dtype == XLA_FFI_DataType_U4;
+  XLA_FFI_Buffer* zp = has_zp ? d.Arg(3, Bit(XLA_FFI_DataType_U4), 1, 3, "zero_points") : nullptr;
+  const int bias_at = has_zp ? 4 : 3;
+  XLA_FFI_Buffer* bias = f->args.size > bias_at ? d.Arg(bias_at, kFloatMask, 1, 1, "bias") : nullptr;
+  if (!has_zp && f->args.size > 4 && d.ok())
+    return InvalidArgument(f->api, "xla_amd.dequant_dot: five operands are lhs, weights, scales, zero_points (U4), bias");
   XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16), 2, 3, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
   CommonAttrs a;
@@ -385,6 +394,9 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
     why = "result shape must be [batch,]M,N";
   else if (sc->dims[sc->rank - 1] != p.N) why = "scales must have N as their last dimension";
   else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
+  else if (zp && w->dtype != XLA_FFI_DataType_U4) why = "zero points go with U4 weights";
+  else if (zp && (zp->rank != sc->rank || memcmp(zp->dims, sc->dims, sizeof(int64_t) * sc->rank) != 0))
+    why = "zero points must have the shape of the scales (one per scale)";
   else if (((a.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
   if (why.empty()) {
     // scales: [N] | [G,N] | [B,N] | [B,G,N].  scale_group_size says which: 0 = one scale per output
@@ -428,6 +440,7 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
 
   p.lhs = lhs->data; p.weights = w->data; p.scales = sc->data;
   p.bias = bias ? bias->data : nullptr;
+  p.zero_points = zp ? zp->data : nullptr;
   p.out = out->data;
   p.workspace = ws ? ws->data : nullptr;
   p.workspace_bytes = ws ? (size_t)Elements(ws) : 0;
@@ -499,6 +512,7 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
     if (b->dims[lead + rcd] != p.K) why = "contracting dimensions differ";
     else if (out->dims[lead] != p.M || out->dims[lead + 1] != p.N) why = "result shape must be M,N";
     else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
+
     else if (((at.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
     else if (mx && (p.K % 32 != 0 || sa->dims[0] != p.M || sb->dims[0] != p.N || sa->dims[1] != p.K / 32 ||
                     sb->dims[1] != p.K / 32))

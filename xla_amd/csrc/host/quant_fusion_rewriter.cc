@@ -502,18 +502,37 @@ bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
 
 // ---------------------------------------------------------------- weight-only dequantize dot
 struct QWeights {
-  Instr* w = nullptr;       // s8 or s4 tensor [B,]K,N
+  Instr* w = nullptr;       // s8, s4 or u4 tensor [B,]K,N
   Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N], bf16 or f32
   std::string type;         // element type of the multiply
+  Instr* zero = nullptr;    // u4 zero points, shaped like the scales: (w - zero) * scale
 };
+
+// convert(s4 -> s8) or convert(u4 -> u8): how 4-bit values are often widened before the float convert
+bool IsByteWidening(const Instr* s) {
+  if (!s->Is("convert")) return false;
+  const std::string& from = s->operands[0]->shape.dtype;
+  return (s->shape.dtype == "s8" && from == "s4") || (s->shape.dtype == "u8" && from == "u4");
+}
 
 // integer tensor behind convert(s4->s8)? -> convert(->float)
 bool IntSource(Instr* cv, const std::string& float_ty, Instr** w) {
   if (!cv->Is("convert") || cv->shape.dtype != float_ty) return false;
   Instr* s = cv->operands[0];
-  if (s->shape.dtype == "s8" && s->Is("convert") && s->operands[0]->shape.dtype == "s4") s = s->operands[0];
-  if (s->shape.dtype != "s8" && s->shape.dtype != "s4") return false;
+  if (IsByteWidening(s)) s = s->operands[0];
+  if (s->shape.dtype != "s8" && s->shape.dtype != "s4" && s->shape.dtype != "u4") return false;
   *w = s;
+  return true;
+}
+
+// v = subtract(x, broadcast(convert(u4 zero points -> ty)) along bdims): peels the subtraction off
+bool PeelZeroPoint(Instr* v, const std::vector<int64_t>& bdims, const std::string& ty, Instr** x, Instr** zero) {
+  if (!v->Is("subtract") || v->operands.size() != 2 || v->shape.dtype != ty) return false;
+  Instr* zs = nullptr;
+  if (!BroadcastAlong(v->operands[1], bdims, &zs)) return false;
+  if (!zs->Is("convert") || zs->shape.dtype != ty || zs->operands[0]->shape.dtype != "u4") return false;
+  *x = v->operands[0];
+  *zero = zs->operands[0];
   return true;
 }
 
@@ -534,13 +553,16 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
     if (d3[0] * d3[1] != op->shape.dims[0] || d3[2] != op->shape.dims[1]) return false;
     Instr *sc = nullptr, *cv = nullptr;
     if (!BinaryWith(mul, "multiply", [&](Instr* s) { return BroadcastAlong(s, {0, 2}, &sc); }, &cv)) return false;
+    Instr* zero = nullptr;
+    PeelZeroPoint(cv, {0, 2}, ty, &cv, &zero);
     // the convert may sit before or after the reshape to [G,g,N]
     Instr* w = nullptr;
     if (cv->Is("convert") && cv->operands[0]->Is("reshape")) {
       Instr* rs = cv->operands[0];
       Instr* src = rs->operands[0];
-      if (src->shape.dtype == "s8" && src->Is("convert") && src->operands[0]->shape.dtype == "s4") src = src->operands[0];
-      if ((src->shape.dtype == "s8" || src->shape.dtype == "s4") && src->shape.rank() == 2) w = src;
+      if (IsByteWidening(src)) src = src->operands[0];
+      if ((src->shape.dtype == "s8" || src->shape.dtype == "s4" || src->shape.dtype == "u4") && src->shape.rank() == 2)
+        w = src;
     } else if (cv->Is("reshape")) {
       IntSource(cv->operands[0], ty, &w);
     }
@@ -550,17 +572,19 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
     }
     sc = LookThroughWidening(sc, ty);
     if (sc->shape.rank() != 2 || sc->shape.dims[0] != d3[0] || sc->shape.dims[1] != d3[2]) return false;
-    *out = {w, sc, ty};
+    *out = {w, sc, ty, zero};
     return true;
   }
   if (!op->Is("multiply")) return false;
   Instr *sc = nullptr, *cv = nullptr;
   const std::vector<int64_t> bdims = rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2};
   if (!BinaryWith(op, "multiply", [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
+  Instr* zero = nullptr;
+  PeelZeroPoint(cv, bdims, ty, &cv, &zero);
   Instr* w;
   if (!IntSource(cv, ty, &w) || w->shape.dims != op->shape.dims) return false;
   sc = LookThroughWidening(sc, ty);
-  *out = {w, sc, ty};
+  *out = {w, sc, ty, zero};
   return true;
 }
 
@@ -589,8 +613,12 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   if (lc != std::vector<int64_t>{rank - 1} || rc != std::vector<int64_t>{rank - 2})
     return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] contracting K (N minor); s4 with a "
                   "minor contracting or batch dimension is rejected as in gemm_fusion.cc:1572-1590");
-  if (q.w->shape.dtype == "s4" && q.w->shape.dims.back() % 2 != 0)
+  const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
+  if (four_bit && q.w->shape.dims.back() % 2 != 0)
     return refuse("s4 rows must hold an even number of values");
+  if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");
+  if (q.zero && q.zero->shape.dims != q.scale->shape.dims)
+    return refuse("zero points must have the shape of the scales (one per scale)");
   if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
   if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
@@ -598,10 +626,11 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   const int64_t B = rank == 3 ? lhs->shape.dims[0] : 1;
   const int64_t M = lhs->shape.dims[rank - 2], K = lhs->shape.dims[rank - 1], N = q.w->shape.dims[rank - 1];
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
+  if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
   std::vector<Shape> results = {Shape::Array("bf16", dot->shape.dims)};
   size_t ws = opt.dequant_workspace_bytes
-                  ? opt.dequant_workspace_bytes(B, M, K, N, q.w->shape.dtype == "s4" ? 21 : 2)
+                  ? opt.dequant_workspace_bytes(B, M, K, N, q.w->shape.dtype == "s4" ? 21 : q.w->shape.dtype == "u4" ? 22 : 2)
                   : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
   // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
@@ -611,7 +640,8 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
                              std::to_string(group_size) + " : i64");
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
-  log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype + "]");
+  log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
+                          (q.zero ? " with zero points" : "") + "]");
   return true;
 }
 

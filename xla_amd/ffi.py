@@ -243,7 +243,8 @@ class LaunchDequantDot(C.Structure):
                 ("batch", C.c_int64), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
                 ("group", C.c_int64), ("scale_batch", C.c_int64), ("weight_dtype", C.c_int32),
                 ("scale_dtype", C.c_int32), ("bias_dtype", C.c_int32), ("dequant_type", C.c_int32),
-                ("dot_type", C.c_int32), ("epilogue_type", C.c_int32), ("epilogue", C.c_int32)]
+                ("dot_type", C.c_int32), ("epilogue_type", C.c_int32), ("epilogue", C.c_int32),
+                ("zero_points", C.c_void_p)]
 
 
 _lib = None

@@ -71,6 +71,38 @@ ENTRY %main {{
 """
 
 
+def u4_zero_point_group(M=8, K=4096, N=4096, group=128, typed="bf16"):
+    """bf16 [M,K] . ((convert(u4 [K,N]) - convert(u4 zero[K/g,N])) * scale[K/g,N]) + bias -> bf16: the
+    asymmetric 4-bit weight-only form (one zero point and one scale per group and channel).
+    typed="bf16": convert, subtract and multiply are bf16-typed, one rounding per dequantised weight
+    (the difference of two integers below 16 is exact); typed="f32" is not taken by the kernels for
+    grouped scales and shows a refusal."""
+    G, t = K // group, typed
+    return f"""HloModule u4_zero_point_group_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = u4[{K},{N}] parameter(1)
+  %scales = {t}[{G},{N}] parameter(2)
+  %zero = u4[{G},{N}] parameter(3)
+  %bias = bf16[{N}] parameter(4)
+  %w_g = u4[{G},{group},{N}] reshape(%w)
+  %w_t = {t}[{G},{group},{N}] convert(%w_g)
+  %zero_t = {t}[{G},{N}] convert(%zero)
+  %zero_b = {t}[{G},{group},{N}] broadcast(%zero_t), dimensions={{0,2}}
+  %w_centered = {t}[{G},{group},{N}] subtract(%w_t, %zero_b)
+  %scales_b = {t}[{G},{group},{N}] broadcast(%scales), dimensions={{0,2}}
+  %w_deq_g = {t}[{G},{group},{N}] multiply(%w_centered, %scales_b)
+  %w_deq = {t}[{K},{N}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] dot(%lhs, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""
+
+
 def c3_fp8(M=8192, K=8192, N=8192, typed="f32", vector_scales=False):
     """f8 [M,K] . f8 [K,N] with per-tensor scales, + bias, GELU(tanh) -> bf16.  typed="f32":
     f32 ops and one final rounding; typed="bf16": every op bf16-typed (the shape of

@@ -57,12 +57,14 @@ def _scratch(nbytes, device):
 
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
-                scale_group_size=None, out=None, scratch="auto", build_only=False):
+                scale_group_size=None, zero_points=None, out=None, scratch="auto", build_only=False):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
     scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
-    the handler reads the grouping off the scales' shape."""
-    _check_cuda(lhs, weights, scales, bias)
-    wdt = dtypes.S4 if weight_dtype == "s4" else dtypes.S8
+    the handler reads the grouping off the scales' shape.
+    weight_dtype "u4": unsigned 4-bit weights, packed like s4; zero_points (uint8, packed u4, one per
+    scale) then makes the dequantised weight (w - zero_point) * scale."""
+    _check_cuda(lhs, weights, scales, bias, zero_points)
+    wdt = {"s4": dtypes.S4, "u4": dtypes.U4}.get(weight_dtype, dtypes.S8)
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
     n = wshape[-1]
     oshape = list(lhs.shape[:-1]) + [n]
@@ -71,6 +73,8 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     batch = lhs.shape[0] if lhs.dim() == 3 else 1
     args = [(dtypes.BF16, lhs.data_ptr(), lhs.shape), (wdt, weights.data_ptr(), wshape),
             (_FLOAT[scales.dtype], scales.data_ptr(), scales.shape)]
+    if zero_points is not None:
+        args.append((dtypes.U4, zero_points.data_ptr(), scales.shape))
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
     rets = [(dtypes.BF16, out.data_ptr(), oshape)]
@@ -85,7 +89,7 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     if scale_group_size is not None:
         attrs["scale_group_size"] = ffi.Attr.i64(scale_group_size)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
-                keep=(lhs, weights, scales, bias, scratch))
+                keep=(lhs, weights, scales, bias, scratch, zero_points))
     return call if build_only else call.run()
 
 

@@ -41,6 +41,21 @@ def c2_s4_group(M=1, K=8192, N=28672, group=128):
                 algorithmic_flops=2 * M * K * N)
 
 
+def u4_zero_point_group(M=8, K=4096, N=4096, group=128):
+    """bf16 A[M,K] . bf16((u4 W[K,N] - u4 zero[K/group,N]) * bf16 scale[K/group,N]) + bias -> bf16."""
+    a = dtypes.f32_to_bf16(_rng(60 + M).standard_normal((M, K)).astype(np.float32))
+    w = _rng(61).integers(0, 16, size=(K, N)).astype(np.uint8)
+    zero = _rng(62).integers(0, 16, size=(K // group, N)).astype(np.uint8)
+    scale = dtypes.f32_to_bf16(_rng(63).uniform(1e-3, 2e-2, size=(K // group, N)).astype(np.float32))
+    bias = dtypes.f32_to_bf16(_rng(64).standard_normal((N,)).astype(np.float32))
+    pack = lambda v: (v.reshape(-1)[0::2] | (v.reshape(-1)[1::2] << 4)).astype(np.uint8)
+    return dict(name="u4zp", lhs=a, weights=w.astype(np.int8), weights_packed=pack(w), scales=scale,
+                zero_points=zero, zero_points_packed=pack(zero), bias=bias, weight_dtype="u4",
+                weight_shape=(K, N), group=group, dequant_type="bf16", epilogue="BIAS",
+                algorithmic_bytes=K * N // 2 + (K // group) * N * 5 // 2 + N * 2 + M * K * 2 + M * N * 2,
+                algorithmic_flops=2 * M * K * N)
+
+
 def c3_fp8(M=8192, K=8192, N=8192):
     """f8 A[M,K] . f8 B[K,N], per-tensor f32 scales 1/64, + bias, GELU(tanh) -> bf16."""
     def f8(seed, shape):
