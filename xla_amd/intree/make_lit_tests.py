@@ -1,0 +1,83 @@
+"""Writes the hlo-opt lit tests of the in-tree pass (xla/backends/gpu/transforms/tests/*.hlo).
+
+Each file is one module of xla_amd.hlo_modules at a small shape with a RUN line for hlo-opt and
+CHECK lines taken from what the offline matcher (the same rules on HLO text) produces for it: the
+custom call line with its operands, target and attributes, or the refusal.  tests/
+test_intree_pass_in_step.py runs every committed file through the offline matcher again, so the
+expectations cannot drift.
+
+    python xla_amd/intree/make_lit_tests.py        # regenerates the files
+"""
+import os
+import re
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+OUT = os.path.join(HERE, "xla", "backends", "gpu", "transforms", "tests")
+
+
+def cases():
+    from xla_amd import hlo_modules as hm
+    gelu_far = hm.c3_fp8(64, 128, 32).replace("constant(0.044715)", "constant(0.05)")
+    return [
+        ("quant_fusion_rewriter_s8_per_channel", hm.c1_s8_channel(16, 256, 128)),
+        ("quant_fusion_rewriter_s4_grouped_silu", hm.c2_s4_group(8, 256, 64, 64)),
+        ("quant_fusion_rewriter_u4_zero_points", hm.u4_zero_point_group(8, 256, 64, 64)),
+        ("quant_fusion_rewriter_s8_batched", hm.c5_s8_batched(2, 8, 32, 16)),
+        ("quant_fusion_rewriter_fp8_bias_gelu", hm.c3_fp8(64, 128, 32)),
+        ("quant_fusion_rewriter_fp8_bf16_typed", hm.c3_fp8(64, 128, 32, typed="bf16")),
+        ("quant_fusion_rewriter_fp8_vector_scales", hm.c3_fp8(64, 128, 32, vector_scales=True)),
+        ("quant_fusion_rewriter_fp8_f8_result_amax", hm.c3_fp8_f8_result(64, 128, 32, amax=True)),
+        ("quant_fusion_rewriter_rowwise_quantize_rmsnorm", hm.c4_quantize(8, 64)),
+        ("quant_fusion_rewriter_rowwise_quantize_rsqrt", hm.c4_quantize(8, 64, rsqrt=True)),
+        ("quant_fusion_rewriter_rowwise_quantize_plain", hm.c4_quantize(8, 64, rmsnorm=False)),
+        ("quant_fusion_rewriter_quantize_then_dot", hm.quantize_then_fp8_dot(8, 64, 32)),
+        ("quant_fusion_rewriter_refuses_far_gelu_constant", gelu_far),
+    ]
+
+
+def expectations(text):
+    """CHECK lines for one module: its custom calls (operands, target, attributes) or, when nothing
+    was rewritten, CHECK-NOT of the targets."""
+    from xla_amd import hlo
+    new, rewrites, refusals = hlo.rewrite(text)
+    lines = []
+    for line in new.splitlines():
+        m = re.search(r"custom-call\((.*?)\), custom_call_target=\"(xla_amd\.[a-z0-9_]+)\".*backend_config=\"\{(.*)\}\"", line)
+        if not m:
+            continue
+        operands, target, cfg = m.group(1), m.group(2), m.group(3).replace('\\"', '"')
+        # operand names change under hlo-opt's renumbering: their count is what is checked
+        lines.append("// CHECK: custom-call(%s), custom_call_target=\"%s\"" % (
+            ", ".join("%{{.*}}" for _ in operands.split(",")), target))
+        lines.append("// CHECK-SAME: api_version=API_VERSION_TYPED_FFI")
+        for attr in cfg.split(", "):
+            key = attr.split(" = ")[0]
+            if key in ("epilogue", "rmsnorm", "scale_group_size", "rhs_contracting_dim", "d_scale_multiplies",
+                       "dequant_type", "dot_type", "epilogue_type"):
+                lines.append("// CHECK-SAME: %s" % attr.replace("\\", ""))
+    if not lines:
+        lines.append("// CHECK-NOT: xla_amd.")
+    return lines, rewrites, refusals
+
+
+def render(name, text):
+    lines, rewrites, refusals = expectations(text)
+    head = ["// RUN: hlo-opt %s --platform=gpu --passes=quant-fusion-rewriter | FileCheck %s",
+            "//",
+            "// The offline matcher says: " + ("; ".join(rewrites) if rewrites else "nothing rewritten")]
+    head += ["//   refused: " + r for r in refusals]
+    return "\n".join(head) + "\n\n" + "\n".join(lines) + "\n\n" + text.strip() + "\n"
+
+
+def main():
+    os.makedirs(OUT, exist_ok=True)
+    for name, text in cases():
+        with open(os.path.join(OUT, name + ".hlo"), "w") as f:
+            f.write(render(name, text))
+    print("wrote %d files to %s" % (len(cases()), OUT))
+
+
+if __name__ == "__main__":
+    main()
