@@ -214,6 +214,16 @@ def main():
         sc = torch.empty((4096,), device=dev).uniform_(1e-3, 1e-2)
         entry("C1", "C1 s8 [16,4096]x[4096,4096]", ops.dequant_dot(a, w8, sc, build_only=True),
               4096 * 4096 + 2 * 16 * 4096 * 2 + 4096 * 4, 2 * 16 * 4096 * 4096, "hbm")
+        # a mixture-of-experts decode step: 32 tokens sorted by expert over 8 experts' s8 weights
+        # (ragged dot, group sizes read on the device; informational -- not one of the five configurations)
+        ar = torch.randn((32, 4096), device=dev).to(torch.bfloat16)
+        wr = torch.randint(-127, 128, (8, 4096, 4096), dtype=torch.int8, device=dev)
+        sr = torch.empty((8, 4096), device=dev).uniform_(1e-3, 1e-2)
+        gsz = torch.tensor([4, 4, 4, 4, 4, 4, 4, 4], dtype=torch.int32, device=dev)
+        entry("ragged", "ragged s8 [32,4096] x [8,4096,4096], 8 groups of 4 rows",
+              ops.dequant_dot(ar, wr, sr, scale_group_size=0, group_sizes=gsz, build_only=True),
+              8 * 4096 * 4096 + 8 * 4096 * 4 + 32 * 4096 * 2 + 32 * 4096 * 2, 2 * 32 * 4096 * 4096, "hbm")
+        del wr
         # C4: RMSNorm + rowwise fp8 quantize
         x = torch.randn((16384, 8192), device=dev)
         x = torch.where(torch.rand_like(x) < 0.01, x * 50, x).to(torch.bfloat16)
@@ -302,6 +312,12 @@ def main():
                                                  bias=w["bias"], group=GROUP2, epilogue="silu"))
             by_key["C2 prefill"]["cpu_baseline"] = base(round(2 * 64 * K2 * 4096 / t / 1e12, 4), "TFLOP/s",
                                                         "64 of 2048 tokens on 4096 of %d channels (full K), %.2f s" % (N2, t))
+        if "ragged" in by_key:
+            w = workloads.ragged_s8_experts(M=32, K=4096, N=4096, groups=8, sizes=[4] * 8)
+            t = timed(lambda: oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32",
+                                                        w["group_sizes"]))
+            by_key["ragged"]["cpu_baseline"] = base(round(w["algorithmic_bytes"] / t / 1e9, 3), "GB/s",
+                                                    "the whole workload, %.2f s" % t)
         if "C4" in by_key:
             w = workloads.c4_quantize(rows=8192, cols=8192)
             t = timed(lambda: oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6))

@@ -143,6 +143,13 @@ typedef struct XlaAmdDequantDot {
   /* U4 weights only, or NULL: one u4 zero point per scale, [scale_batch, K/group, N] packed two per
    * byte like the weights; the dequantised weight is (w - zero_point) * scale */
   const void* zero_points;
+  /* Ragged dot (xla ragged-dot with the ragged dimension on the rows of lhs): NULL for an ordinary
+   * dot.  Otherwise `batch` row counts in device memory, S32 or S64 (group_sizes_dtype): lhs is
+   * [M,K] with its rows sorted by group, weights [batch,K,N] hold one matrix per group, out is
+   * [M,N]; group g takes rows [sum of the sizes before it, + its size), rows past the last group
+   * are a dot of nothing (epilogue(0)).  Never read on the host. */
+  const void* group_sizes;
+  int32_t group_sizes_dtype;
 } XlaAmdDequantDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);

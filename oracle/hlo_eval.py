@@ -102,6 +102,8 @@ def evaluate(module_json, args):
                 v = np.ascontiguousarray(v, np.uint8)
             elif ty in ("s8", "s4", "u4"):
                 v = np.ascontiguousarray(v, np.int8)   # unpacked values (u4: 0..15)
+            elif ty in ("s32", "s64"):
+                v = np.ascontiguousarray(v, np.int64)
             else:
                 v = np.ascontiguousarray(v, np.float32)
             v = v.reshape(sh["dims"])
@@ -137,6 +139,25 @@ def evaluate(module_json, args):
             with np.errstate(all="ignore"):
                 r = {"multiply": np.multiply, "add": np.add, "subtract": np.subtract, "divide": np.divide,
                      "maximum": np.maximum, "minimum": np.minimum}[op](a, b)
+            v = _round(r, ty)
+        elif op == "ragged-dot":
+            # lhs [M,K] rows sorted by group, rhs [G,K,N], group sizes [G]: row m of group g is
+            # lhs[m] . rhs[g], f32 sums in increasing k; rows no group owns are zero
+            # (ragged_dot_rewriter.cc:110-210 masks one dense dot per group)
+            a_ = np.asarray(x[0], np.float32)
+            b_ = np.asarray(x[1], np.float32)
+            sizes = [int(v) for v in np.asarray(x[2]).reshape(-1)]
+            assert _dims(ins["attrs"].get("lhs_contracting_dims", "")) == [1]
+            assert _dims(ins["attrs"].get("rhs_contracting_dims", "")) == [1]
+            assert _dims(ins["attrs"].get("lhs_ragged_dims", "")) == [0]
+            assert _dims(ins["attrs"].get("rhs_group_dims", "")) == [0]
+            r = np.zeros((a_.shape[0], b_.shape[2]), np.float32)
+            start = 0
+            for g, n in enumerate(sizes):
+                n = max(0, min(n, a_.shape[0] - start))
+                if n:
+                    r[start:start + n] = _dot(a_[start:start + n], b_[g], [1], [0], [], [])
+                start += n
             v = _round(r, ty)
         elif op == "negate":
             v = _round(-np.asarray(x[0], np.float32), ty)

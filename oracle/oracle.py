@@ -244,6 +244,38 @@ def dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, bias=None, bias_ty="
     return out if batched else out[0]
 
 
+def ragged_dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, group_sizes, **kw):
+    """Ragged dot (xla ragged-dot, ragged dimension = rows of lhs; expanded by the reference into one
+    masked dense dot per group, xla/hlo/transforms/expanders/ragged_dot_rewriter.cc:110-210):
+    a_bf16 [M,K] with rows sorted by group, w [G,K,N] (int8, or packed 4-bit per group), scale
+    [G,..,N]; row m of group g is lhs[m] . dequant(w[g]); rows past the last group are a dot of
+    nothing, i.e. epilogue(0).  Built from dequant_dot, one call per group."""
+    a = _c(a_bf16, np.uint16)
+    M, K = a.shape
+    sizes = [int(x) for x in np.asarray(group_sizes).reshape(-1)]
+    G = len(sizes)
+    scale = np.ascontiguousarray(scale)
+    N = scale.shape[-1]
+    w = np.ascontiguousarray(w)
+    wg = w.reshape(G, -1)
+    sg = scale.reshape(G, -1, N)
+    zp = kw.pop("zero_points", None)
+    zg = None if zp is None else np.ascontiguousarray(zp).reshape(G, -1)
+    out = np.empty((M, N), np.uint16)
+    start = 0
+    for g in range(G):
+        n = max(0, min(sizes[g], M - start))
+        if n:
+            out[start:start + n] = dequant_dot(a[start:start + n], wg[g], w_bits, sg[g], scale_ty, mul_ty,
+                                               zero_points=None if zg is None else zg[g], **kw)
+        start += n
+    if start < M:   # a dot of nothing: zero activations give the same rows
+        zero = np.zeros((M - start, K), np.uint16)
+        out[start:] = dequant_dot(zero, wg[0], w_bits, sg[0], scale_ty, mul_ty,
+                                  zero_points=None if zg is None else zg[0], **kw)
+    return out
+
+
 def fp8_scaled_dot(a8, b8, a_scale, b_scale, b_is_nk=False, mul_ty="f32", bias=None,
                    bias_ty="bf16", dot_ty="f32", ep_ty="f32", epilogue="none", d_scale=None,
                    d_scale_divides=True):

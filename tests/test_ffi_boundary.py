@@ -180,6 +180,22 @@ def test_zero_point_operand_is_recognised_by_its_type():
         ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, (dtypes.U8, FAKE, (64, 8)), sc], out))
 
 
+def test_ragged_dot_operands():
+    """An integer operand at the end is the group sizes of a ragged dot: lhs [M,K], weights [G,K,N]."""
+    host = ffi.Host()
+    lhs, w = (dtypes.BF16, FAKE, (6, 64)), (dtypes.S8, FAKE, (3, 64, 8))
+    sc, gs = (dtypes.F32, FAKE, (3, 8)), (dtypes.S32, FAKE, (3,))
+    out = [(dtypes.BF16, FAKE, (6, 8))]
+    with pytest.raises(ffi.FfiError, match="a ragged dot takes lhs \\[M,K\\] and weights \\[groups,K,N\\]"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, (dtypes.S8, FAKE, (64, 8)), (dtypes.F32, FAKE, (8,)), gs], out))
+    with pytest.raises(ffi.FfiError, match="group_sizes must have one entry per group of weights"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w, sc, (dtypes.S64, FAKE, (4,))], out))
+    with pytest.raises(ffi.FfiError, match="result shape must be"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w, sc, gs], [(dtypes.BF16, FAKE, (3, 6, 8))]))
+    with pytest.raises(ffi.FfiError, match="lhs and weights must have the same rank"):
+        ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, [lhs, w, sc], out))      # no group sizes: not ragged
+
+
 def test_record_stage_asks_for_stream_capture():
     """At the RECORD stage (XLA building a command buffer, custom_call_thunk.cc:577-684) a handler finds
     the record extension on its invoke context and asks for stream capture of its execute stage;

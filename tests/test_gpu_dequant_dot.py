@@ -605,3 +605,65 @@ def test_u4_per_channel_f32_multiply(oracle, with_zero_points):
     got, kern = run_dot(w, force_kernel=2)
     assert kern.endswith("_factored"), kern
     compare(oracle, w, got, "u4 per-channel %s" % kern)
+
+
+# ---- ragged dot (tokens sorted by expert, group sizes on the device) -----------------------------
+
+def run_ragged(w, sizes_dtype=torch.int32, force_kernel=0):
+    lhs, wt = dev_bf16(w["lhs"]), dev_s8(w["weights"])
+    sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
+    bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
+    gs = torch.from_numpy(np.asarray(w["group_sizes"], np.int64)).to(sizes_dtype).cuda()
+    ffi.set_option("dequant_dot_kernel", force_kernel)
+    try:
+        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype="s8", weight_shape=w["weight_shape"],
+                              epilogue=w["epilogue"], dequant_type=w["dequant_type"], scale_group_size=0,
+                              group_sizes=gs)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("dequant_dot_kernel", 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+def ragged_floor(w):
+    a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
+    wd = np.max(np.abs(w["weights"].astype(np.float64)) * w["scales"].astype(np.float64)[:, None, :], axis=0)
+    return dot_floor(a, wd, w["lhs"].shape[-1])
+
+
+@pytest.mark.parametrize("M,K,N,G,sizes,sizes_dtype", [
+    (32, 1024, 512, 8, None, torch.int32), (64, 512, 384, 4, [10, 0, 50, 4], torch.int64),
+    (16, 2048, 256, 16, None, torch.int32), (12, 256, 136, 3, [5, 0, 2], torch.int32),
+    (7, 512, 128, 2, [9, 9], torch.int32), (40, 512, 256, 5, [0, 0, 0, 0, 0], torch.int64)])
+def test_ragged_dot_decode(oracle, M, K, N, G, sizes, sizes_dtype):
+    """Rows sorted by expert, each group through its own weights: random splits with empty groups,
+    s32 and s64 sizes, rows that no group owns (epilogue(0) = the bias), sizes that overrun M (cut
+    at M) and a call whose groups are all empty."""
+    say("dequant_dot ragged M=%d K=%d N=%d G=%d sizes=%s" % (M, K, N, G, sizes))
+    w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+    got, kern = run_ragged(w, sizes_dtype)
+    assert kern.startswith("dequant_dot_decode_s8_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged %s" % kern)
+
+
+def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
+    """Every row of the ragged result is bit-identical to an ordinary call on its group's rows with
+    that group's weights (the same kernel does both); the one-thread-per-output kernel, which finds
+    each row's group by itself, agrees with the oracle too."""
+    say("dequant_dot ragged vs per-group calls, generic kernel")
+    w = workloads.ragged_s8_experts(M=24, K=1024, N=256, groups=4, sizes=[7, 1, 0, 11])
+    got, kern = run_ragged(w)
+    start = 0
+    for g, n in enumerate(w["group_sizes"]):
+        if n:
+            sub = dict(w, lhs=w["lhs"][start:start + n], weights=w["weights"][g], scales=w["scales"][g],
+                       weight_shape=w["weights"][g].shape)
+            one, k1 = run_dot(sub, force_kernel=2, x=1)
+            assert np.array_equal(got[start:start + n], one), (g, kern, k1)
+        start += n
+    assert np.array_equal(got[start:], np.broadcast_to(w["bias"], (24 - start, 256)))
+    got_generic, kern = run_ragged(w, force_kernel=1)
+    assert kern == "dequant_dot_generic", kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got_generic, ref, ragged_floor(w), "ragged generic")

@@ -136,3 +136,14 @@ def test_u4_zero_points(oracle):
     ref = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", bias=w["bias"],
                              group=32, unsigned=True, zero_points=w["zero_points_packed"])
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("sizes", [[3, 3, 3, 3], [5, 0, 2, 1], [0, 0, 12, 0]])
+def test_ragged_dot(oracle, sizes):
+    """The ragged-dot module op by op (the evaluator's own ragged-dot: one masked dense dot per group)
+    against the oracle's composition of per-group calls: bit for bit."""
+    w = workloads.ragged_s8_experts(M=12, K=64, N=24, groups=4, sizes=sizes)
+    got = run_module(hm.ragged_s8_experts(12, 64, 24, 4),
+                     [w["lhs"], w["weights"], w["scales"], w["bias"], w["group_sizes"]])
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    assert np.array_equal(got, ref)

@@ -506,3 +506,18 @@ def test_u4_weights_with_zero_points():
     new3, rw3, rf3 = hlo.rewrite(plain)
     assert rw3 == ["dot -> xla_amd.dequant_dot [BIAS_SILU, u4]"] and rf3 == []
     check(new3, r"custom-call\(%lhs, %w, %scales, %bias\)")
+
+
+def test_ragged_dot_over_expert_weights():
+    text = hm.ragged_s8_experts(16, 256, 64, 4)
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, s8, ragged over 4 groups]"] and rf == []
+    check(new, r"custom-call\(%lhs, %w, %scale, %bias, %sizes\), custom_call_target=\"xla_amd.dequant_dot\"",
+          r"scale_group_size = 0 : i64")
+    assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
+    assert hlo.rewrite(hm.ragged_s8_experts(16, 256, 64, 4, sizes_ty="s64"))[1] == rw
+    for bad, reason in ((hm.ragged_s8_experts(128, 256, 64, 4), "more than 64 rows"),
+                        (text.replace("lhs_ragged_dims={0}", "lhs_ragged_dims={1}"), "ragged dimension on the rows of lhs"),
+                        (text.replace("%sizes = s32[4]", "%sizes = u32[4]"), "group sizes must be s32 or s64")):
+        new2, rw2, rf2 = hlo.rewrite(bad)
+        assert rw2 == [] and any(reason in r for r in rf2), (rw2, rf2)

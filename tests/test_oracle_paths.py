@@ -388,3 +388,34 @@ def test_u4_zero_point_dequantisation_one_hot_and_brute_force(oracle):
                                                 zero_points=_pack4(z))).astype(np.float64)
     ref = dtypes.bf16_to_f32(a).astype(np.float64) @ dtypes.bf16_to_f32(want).astype(np.float64)
     assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2)) < 2.0 ** -7
+
+
+# ---- ragged dot -------------------------------------------------------------------
+
+def test_ragged_dot_composition_is_pinned(oracle):
+    """The ragged dot is one dense dot per group on that group's rows (ragged_dot_rewriter.cc:110-210).
+    Equal group sizes must give the batched dot reshaped; every row must equal a one-row dot with
+    its group's weights; rows past the last group are epilogue(0); float64 agrees."""
+    from xla_amd import workloads
+    G, K, N = 4, 64, 24
+    w = workloads.ragged_s8_experts(M=12, K=K, N=N, groups=G, sizes=[3, 3, 3, 3])
+    got = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"],
+                                    bias=w["bias"])
+    batched = oracle.dequant_dot(w["lhs"].reshape(G, 3, K), w["weights"], 8, w["scales"], "f32", "f32", bias=w["bias"])
+    assert np.array_equal(got, batched.reshape(12, N))
+    # uneven, with an empty group and unowned rows at the end
+    sizes = [5, 0, 2, 1]
+    got = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", sizes, bias=w["bias"])
+    owner = [0] * 5 + [2] * 2 + [3]
+    for m, g in enumerate(owner):
+        one = oracle.dequant_dot(w["lhs"][m:m + 1], w["weights"][g], 8, w["scales"][g], "f32", "f32", bias=w["bias"])
+        assert np.array_equal(got[m], one[0]), m
+    assert np.array_equal(got[8:], np.broadcast_to(w["bias"], (4, N)))     # a dot of nothing, plus the bias
+    a64 = dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)
+    for m, g in enumerate(owner):
+        ref = a64[m] @ (w["weights"][g].astype(np.float64) * w["scales"][g].astype(np.float64)) + dtypes.bf16_to_f32(w["bias"])
+        assert np.max(np.abs(dtypes.bf16_to_f32(got[m]) - ref) / np.maximum(np.abs(ref), 1e-2)) < 2.0 ** -7
+    # sizes that overrun M are cut at M
+    over = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", [10, 10, 0, 0], bias=w["bias"])
+    assert np.array_equal(over[:10], oracle.dequant_dot(w["lhs"][:10], w["weights"][0], 8, w["scales"][0], "f32", "f32", bias=w["bias"]))
+    assert np.array_equal(over[10:], oracle.dequant_dot(w["lhs"][10:], w["weights"][1], 8, w["scales"][1], "f32", "f32", bias=w["bias"]))

@@ -45,7 +45,27 @@ struct DecodeParams {
   // scale ([scale_batch, K/group, N], packed like the weights): W' = (w - z) * scale
   int w_unsigned;
   const uint8_t* zero_points;
+  // Ragged dot (lhs [M,K] with its rows sorted by group, weights [groups,K,N]): group_sizes holds
+  // `batch` row counts (s32, or s64 when group_sizes_64) in device memory; grid.y walks the groups,
+  // group g takes rows [sum of the sizes before it, + its size) of lhs and out, rows past the last
+  // group get epilogue(0).  Null for an ordinary (batched) dot.
+  const void* group_sizes;
+  int group_sizes_64;
+  int ragged_groups;  // number of groups (the kernels that do not carry it in grid.y)
 };
+
+// Rows of a ragged dot that group g covers, read on the device: [*begin, *begin + *rows), clamped to
+// [0, M] so that sizes that do not add up cannot reach outside the operands.
+static __device__ __forceinline__ void ragged_rows(const DecodeParams& p, int g, int* begin, int* rows) {
+  long long start = 0;
+  for (int i = 0; i < g; ++i)
+    start += p.group_sizes_64 ? ((const long long*)p.group_sizes)[i] : (long long)((const int*)p.group_sizes)[i];
+  long long n = p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+  start = start < 0 ? 0 : (start > p.M ? p.M : start);
+  n = n < 0 ? 0 : (n > p.M - start ? p.M - start : n);
+  *begin = (int)start;
+  *rows = (int)n;
+}
 
 static __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
   return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];

@@ -72,6 +72,14 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   const int slice = bid % p.slices;
   const int strip = bid / p.slices;
   const int batch = blockIdx.y;
+  // rows of lhs / out this workgroup works on: batch b of an ordinary dot owns rows [b*M, (b+1)*M) of
+  // the flattened [batch*M] rows; group b of a ragged dot owns the rows its group sizes say
+  int m_begin = batch * p.M, m_rows = p.M, tail_begin = -1;
+  if (p.group_sizes) {
+    ragged_rows(p, batch, &m_begin, &m_rows);
+    if (batch == (int)gridDim.y - 1) tail_begin = m_begin + m_rows;  // the last group also fills the rows no group owns
+    if (m_rows == 0 && (tail_begin < 0 || tail_begin >= p.M)) return;
+  }
 
   const int n_lane = strip * TN + li * NV;   // first channel of this lane (may be >= N: discarded)
   const uint32_t pitch = (uint32_t)(((size_t)p.N * WBITS) >> 3);  // bytes per row of W
@@ -82,8 +90,8 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   __amdgpu_buffer_rsrc_t ra[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int rows = max(p.M - 16 * mt, 0);
-    ra[mt] = make_rsrc(p.lhs + ((size_t)batch * p.M + (rows ? 16 * mt : 0)) * p.K, (uint32_t)rows * p.K * 2u);
+    const int rows = max(m_rows - 16 * mt, 0);
+    ra[mt] = make_rsrc(p.lhs + ((size_t)m_begin + (rows ? 16 * mt : 0)) * p.K, (uint32_t)rows * p.K * 2u);
   }
   const int groups = p.K / p.group;
   const __amdgpu_buffer_rsrc_t rs =
@@ -327,15 +335,25 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     const int j0 = r0 % NV, mt = (r0 / NV) / 4, t = (r0 / NV) % 4;
     const int m = mt * 16 + li;
     const int n0 = strip * TN + (4 * kb + t) * NV + j0;
-    if (m >= p.M || n0 >= p.N) continue;
+    if (m >= m_rows || n0 >= p.N) continue;
     if (p.slices > 1) {
       float* dst = p.workspace + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = res[pass * RPW + u];
     } else {
-      uint16_t* dst = p.out + ((size_t)batch * p.M + m) * p.N + n0;
+      uint16_t* dst = p.out + ((size_t)m_begin + m) * p.N + n0;
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = f32_to_bf16(res[pass * RPW + u]);
+    }
+  }
+  // ragged dot: rows past the last group are a dot of nothing -- epilogue(0) in this strip's channels
+  if (tail_begin >= 0 && tail_begin < p.M) {
+    const int tail_rows = p.M - tail_begin;
+    for (int idx = threadIdx.x; idx < tail_rows * TN; idx += WAVES * 64) {
+      const int n = strip * TN + idx % TN, m = tail_begin + idx / TN;
+      if (n >= p.N) continue;
+      const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+      p.out[(size_t)m * p.N + n] = f32_to_bf16(epilogue_dispatch(0.0f, b, p.epilogue, p.bf16_dot, p.bf16_ops));
     }
   }
 }
@@ -366,11 +384,21 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
   const int batch = blockIdx.y;
   if (idx >= total) return;
   const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+  // ragged dot (launched with one batch): the row's group picks the weights; rows no group owns add nothing
+  int wbatch = batch, k_end = p.K;
+  if (p.group_sizes) {
+    k_end = 0;
+    for (int g = 0; g < p.ragged_groups; ++g) {
+      int b0, rows;
+      ragged_rows(p, g, &b0, &rows);
+      if (m >= b0 && m < b0 + rows) { wbatch = g; k_end = p.K; break; }
+    }
+  }
   const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
-  const size_t wbase = (size_t)batch * p.K * p.N;
-  const size_t sbase = (size_t)(p.scale_batched ? batch : 0) * (p.K / p.group) * p.N;
+  const size_t wbase = (size_t)wbatch * p.K * p.N;
+  const size_t sbase = (size_t)(p.scale_batched ? wbatch : 0) * (p.K / p.group) * p.N;
   float acc = 0.0f;
-  for (int k = 0; k < p.K; ++k) {
+  for (int k = 0; k < k_end; ++k) {
     const size_t e = wbase + (size_t)k * p.N + n;
     int wi;
     if (wbits == 8) {
@@ -563,6 +591,13 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.weights_shared = weights_shared;
   dp.w_unsigned = u4;
   dp.zero_points = (const uint8_t*)p.zero_points;
+  const bool ragged = p.group_sizes != nullptr;
+  if (ragged && p.group_sizes_dtype != XLA_FFI_DataType_S32 && p.group_sizes_dtype != XLA_FFI_DataType_S64)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: group sizes must be S32 or S64");
+  if (ragged && weights_shared) return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot: ragged token chunks");
+  dp.group_sizes = p.group_sizes;
+  dp.group_sizes_64 = p.group_sizes_dtype == XLA_FFI_DataType_S64;
+  dp.ragged_groups = ragged ? (int)p.batch : 0;
   const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
   const bool per_channel = p.group == p.K;
 
@@ -571,7 +606,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
                        ((uintptr_t)p.weights % 16 == 0);
   const bool mode_ok = mode == kRounded || per_channel;
 
-  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4) {
+  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && !ragged) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
@@ -600,7 +635,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // in a call of its own, so the chunks compose bit for bit; each pass streams the weights again,
   // which at 8192 x 28672 s4 still reaches 0.55 PFLOP/s against 2-3 TFLOP/s of the generic kernel.
   int mt64, vec64, nv64;
-  if (force != 1 && force != 3 && aligned && mode_ok && p.M > 64 && p.K >= 32 && p.N % 2 == 0 &&
+  if (force != 1 && force != 3 && aligned && mode_ok && p.M > 64 && p.K >= 32 && p.N % 2 == 0 && !ragged &&
       decode_shape(64, &mt64, &vec64, &nv64)) {
     const size_t wbytes = (size_t)p.K * p.N * (s4 ? 1 : 2) / 2;
     const size_t ssz = p.scale_dtype == XLA_FFI_DataType_BF16 ? 2 : 4;
@@ -639,12 +674,12 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // s4 with bf16 group scales and a bf16-typed multiply: the kernels that dequantise through the
     // 4x4x4 matrix instruction
-    if (shape_ok && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1) {
+    if (shape_ok && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1 && !ragged) {
       const int rc = LaunchDequantDotDecodeS4x(dp, p, stream);
       if (rc >= 0) return rc;
     }
     // small s8 matrices with per-channel scales under an f32-typed multiply: one launch
-    if (shape_ok && !s4 && mode == kFactored && per_channel && !weights_shared) {
+    if (shape_ok && !s4 && mode == kFactored && per_channel && !weights_shared && !ragged) {
       const int rc = LaunchDequantDotDecodeS8x(dp, p, stream);
       if (rc >= 0) return rc;
     }
@@ -655,13 +690,14 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
       // leave it (measured 6-7 % faster than the best 8-wave split on C2 up to 8 tokens).
       const bool has_w16 = mt == 1 && nv == 8 && ((s4 && mode == kRounded) || (!s4 && mode == kFactored));
       int waves = 8;
-      if (has_w16 && dp.strips * p.batch >= 192 && p.K >= 2048 && !GetOption("dequant_dot_slices")) waves = 16;
+      if (has_w16 && dp.strips * p.batch >= 192 && p.K >= 2048 && !GetOption("dequant_dot_slices") && !ragged) waves = 16;
       if (int wv = GetOption("dequant_dot_waves")) waves = wv == 4 ? 4 : (wv == 16 && has_w16) ? 16 : 8;
       int slices = waves == 16 && !GetOption("dequant_dot_slices")
                        ? 1 : DecodeSlices(p.batch, p.M, p.K, p.N, dp.strips, row_bytes, waves);
       if (slices > 1 && (!p.workspace ||
                          p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, slices)))
         slices = 1;
+      if (ragged) slices = 1;  // every group is one workgroup per strip: its rows are only known on the device
       dp.slices = slices;
       dp.rows_per_slice = RowsPerSlice(dp.K, slices, waves);
       ClassRows(dp.rows_per_slice, waves, dp.class_rows);
@@ -709,7 +745,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // fallback: any shape
   {
     dp.slices = 1;
-    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)p.batch);
+    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)(ragged ? 1 : p.batch));
     hipLaunchKernelGGL(dequant_dot_generic_kernel, grid, dim3(256), 0, stream, dp, s4 ? 4 : 8, mode);
     SetLastKernel("dequant_dot_generic");
     return CheckLaunch("dequant_dot_generic");

@@ -356,20 +356,30 @@ extern "C" {
 
 XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Error* err;
-  if (Preamble(f, 3, 5, 1, 2, &err)) return err;
+  if (Preamble(f, 3, 6, 1, 2, &err)) return err;
   Decoder d{f};
+  // a ragged dot brings its group sizes (S32 or S64 [groups]) as the last operand
+  int64_t nargs = f->args.size;
+  XLA_FFI_Buffer* gs = nullptr;
+  if (nargs > 3 && f->args.types[nargs - 1] == XLA_FFI_ArgType_BUFFER) {
+    XLA_FFI_Buffer* last = static_cast<XLA_FFI_Buffer*>(f->args.args[nargs - 1]);
+    if (last->dtype == XLA_FFI_DataType_S32 || last->dtype == XLA_FFI_DataType_S64) {
+      gs = d.Arg((int)nargs - 1, Bit(XLA_FFI_DataType_S32) | Bit(XLA_FFI_DataType_S64), 1, 1, "group_sizes");
+      --nargs;
+    }
+  }
   XLA_FFI_Buffer* lhs = d.Arg(0, Bit(XLA_FFI_DataType_BF16), 2, 3, "lhs");
   XLA_FFI_Buffer* w = d.Arg(1, Bit(XLA_FFI_DataType_S8) | Bit(XLA_FFI_DataType_S4) | Bit(XLA_FFI_DataType_U4), 2, 3,
                             "weights");
   XLA_FFI_Buffer* sc = d.Arg(2, kFloatMask, 1, 3, "scales");
   // operands: lhs, weights, scales[, zero_points][, bias] -- a U4 operand after the scales is the
   // zero points (one per scale), a float one the bias
-  const bool has_zp = f->args.size > 3 && f->args.types[3] == XLA_FFI_ArgType_BUFFER &&
+  const bool has_zp = nargs > 3 && f->args.types[3] == XLA_FFI_ArgType_BUFFER &&
                       static_cast<XLA_FFI_Buffer*>(f->args.args[3])->dtype == XLA_FFI_DataType_U4;
   XLA_FFI_Buffer* zp = has_zp ? d.Arg(3, Bit(XLA_FFI_DataType_U4), 1, 3, "zero_points") : nullptr;
   const int bias_at = has_zp ? 4 : 3;
-  XLA_FFI_Buffer* bias = f->args.size > bias_at ? d.Arg(bias_at, kFloatMask, 1, 1, "bias") : nullptr;
-  if (!has_zp && f->args.size > 4 && d.ok())
+  XLA_FFI_Buffer* bias = nargs > bias_at ? d.Arg(bias_at, kFloatMask, 1, 1, "bias") : nullptr;
+  if (((!has_zp && nargs > 4) || nargs > 5) && d.ok())
     return InvalidArgument(f->api, "xla_amd.dequant_dot: five operands are lhs, weights, scales, zero_points (U4), bias");
   XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16), 2, 3, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
@@ -379,18 +389,23 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   const bool has_group_size = d.Int("scale_group_size", &group_size);
   if (!d.ok()) return d.Error();
 
-  const bool batched = lhs->rank == 3;
+  // ragged: lhs [M,K] (rows sorted by group), weights [groups,K,N], out [M,N]; the groups take the
+  // place of the batch for weights and scales
+  const bool ragged = gs != nullptr;
+  const bool batched = lhs->rank == 3 || ragged;
   XlaAmdDequantDot p{};
-  p.batch = batched ? lhs->dims[0] : 1;
+  p.batch = ragged ? (w->rank == 3 ? w->dims[0] : 0) : batched ? lhs->dims[0] : 1;
   p.M = lhs->dims[lhs->rank - 2];
   p.K = lhs->dims[lhs->rank - 1];
   p.N = w->dims[w->rank - 1];
   std::string why;
-  if (w->rank != lhs->rank) why = "lhs and weights must have the same rank";
+  if (ragged && (lhs->rank != 2 || w->rank != 3)) why = "a ragged dot takes lhs [M,K] and weights [groups,K,N]";
+  else if (ragged && gs->dims[0] != p.batch) why = "group_sizes must have one entry per group of weights";
+  else if (!ragged && w->rank != lhs->rank) why = "lhs and weights must have the same rank";
   else if (w->dims[w->rank - 2] != p.K) why = "contracting dimensions differ";
-  else if (batched && w->dims[0] != p.batch) why = "batch dimensions differ";
+  else if (!ragged && batched && w->dims[0] != p.batch) why = "batch dimensions differ";
   else if (out->rank != lhs->rank || out->dims[out->rank - 1] != p.N ||
-           out->dims[out->rank - 2] != p.M || (batched && out->dims[0] != p.batch))
+           out->dims[out->rank - 2] != p.M || (!ragged && batched && out->dims[0] != p.batch))
     why = "result shape must be [batch,]M,N";
   else if (sc->dims[sc->rank - 1] != p.N) why = "scales must have N as their last dimension";
   else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
@@ -441,6 +456,8 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   p.lhs = lhs->data; p.weights = w->data; p.scales = sc->data;
   p.bias = bias ? bias->data : nullptr;
   p.zero_points = zp ? zp->data : nullptr;
+  p.group_sizes = gs ? gs->data : nullptr;
+  p.group_sizes_dtype = gs ? gs->dtype : 0;
   p.out = out->data;
   p.workspace = ws ? ws->data : nullptr;
   p.workspace_bytes = ws ? (size_t)Elements(ws) : 0;

@@ -6,7 +6,7 @@
 //       -> dot [-> +bias] [-> relu|gelu|silu]
 //       => xla_amd.fp8_scaled_dot          (what gemm_rewriter.cc:190-336,1235-1591 turns into
 //                                           __cublas$lt$matmul$f8, epilogues :888-1007,1987-2304)
-//   convert(s8|s4) * broadcast(scale) -> dot [-> +bias] [-> activation]
+//   (convert(s8|s4|u4) [- zero points]) * broadcast(scale) -> dot | ragged-dot [-> +bias] [-> activation]
 //       => xla_amd.dequant_dot             (what gemm_fusion.cc:1629-1702 wraps into __triton_gemm;
 //                                           pattern zoo: fusion_emitter_int4_device_test.cc:85-449)
 //   custom-call "__op$block_scaled_dot" (f8e4m3fn operands, f8e8m0fnu scales per 32 of K)
@@ -645,6 +645,60 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   return true;
 }
 
+// ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N], group_sizes [G]) with the ragged dimension
+// on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call whose
+// kernels read the group sizes on the device.  Decode sizes only: up to 64 rows in all.
+bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
+  QWeights q;
+  std::string why;
+  if (!MatchQWeights(dot->operands[1], &q, &why)) {
+    if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
+    return false;
+  }
+  auto refuse = [&](const std::string& w) {
+    log->refusals.push_back(dot->name + ": quantized weights found but not rewritten: " + w);
+    return false;
+  };
+  Instr* lhs = dot->operands[0];
+  Instr* sizes = dot->operands[2];
+  Instr* inner;
+  if (lhs->Is("convert") && ConvertFrom(lhs, "bf16", &inner) && lhs->shape.dtype == "f32") lhs = inner;
+  if (lhs->shape.dtype != "bf16") return refuse("the activation must be bf16 (or its convert to f32)");
+  if (lhs->shape.rank() != 2 || q.w->shape.rank() != 3 || dot->shape.rank() != 2)
+    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] and a result [M,N]");
+  if (dot->DimsAttr("lhs_contracting_dims") != std::vector<int64_t>{1} ||
+      dot->DimsAttr("rhs_contracting_dims") != std::vector<int64_t>{1} ||
+      dot->DimsAttr("lhs_ragged_dims") != std::vector<int64_t>{0} ||
+      dot->DimsAttr("rhs_group_dims") != std::vector<int64_t>{0} || !dot->DimsAttr("lhs_batch_dims").empty())
+    return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
+                  "leading the weights");
+  const int64_t G = q.w->shape.dims[0], M = lhs->shape.dims[0], K = lhs->shape.dims[1], N = q.w->shape.dims[2];
+  if (q.w->shape.dims[1] != K) return refuse("contracting dimensions differ");
+  if ((sizes->shape.dtype != "s32" && sizes->shape.dtype != "s64") || sizes->shape.dims != std::vector<int64_t>{G})
+    return refuse("group sizes must be s32 or s64, one per group of weights");
+  if (M > 64) return refuse("a ragged dot over more than 64 rows is left to the grouped matmul");
+  const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
+  if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
+  if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");
+  if (q.zero && q.zero->shape.dims != q.scale->shape.dims)
+    return refuse("zero points must have the shape of the scales (one per scale)");
+  if (q.scale->shape.dims != std::vector<int64_t>{G, N})
+    return refuse("a ragged dot takes one scale per group and output channel");
+  if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
+  Epilogue ep;
+  if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
+  std::vector<Instr*> ops = {lhs, q.w, q.scale};
+  if (q.zero) ops.push_back(q.zero);
+  if (ep.bias) ops.push_back(ep.bias);
+  ops.push_back(sizes);
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, {Shape::Array("bf16", dot->shape.dims)},
+                         CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = 0 : i64");
+  comp->ReplaceAllUses(ep.tail, call);
+  log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
+                          (q.zero ? " with zero points" : "") + ", ragged over " + std::to_string(G) + " groups]");
+  return true;
+}
+
 // ---------------------------------------------------------------- row-wise fp8 quantize
 bool IsReduceOver(const Instr* r, const Module& m, const char* body_op, int64_t dim, Instr** src, Instr** init) {
   if (!r->Is("reduce") || r->operands.size() != 2 || r->DimsAttr("dimensions") != std::vector<int64_t>{dim}) return false;
@@ -764,6 +818,8 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         bool did = false;
         if (i->Is("dot") && i->operands.size() == 2) {
           did = RewriteF8Dot(*mod, comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
+        } else if (i->Is("ragged-dot") && i->operands.size() == 3) {
+          did = RewriteRaggedDequantDot(comp.get(), i, log);
         } else if (i->Is("custom-call")) {
           did = RewriteBlockScaledDot(comp.get(), i, log);
         } else if (i->Is("convert") && i->shape.dtype == "f8e4m3fn") {

@@ -103,6 +103,32 @@ ENTRY %main {{
 """
 
 
+def ragged_s8_experts(M=32, K=4096, N=4096, groups=8, sizes_ty="s32"):
+    """ragged-dot(bf16 [M,K], convert(s8 [G,K,N]) * f32 scale[G,N], group sizes [G]) + bias -> bf16:
+    a decode step of a mixture of experts whose tokens are sorted by expert (the shape of
+    ragged_dot_rewriter_test.cc:78-82 with quantised weights)."""
+    G = groups
+    return f"""HloModule ragged_s8_experts_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s8[{G},{K},{N}] parameter(1)
+  %scale = f32[{G},{N}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %sizes = {sizes_ty}[{G}] parameter(4)
+  %lhs_f32 = f32[{M},{K}] convert(%lhs)
+  %w_f32 = f32[{G},{K},{N}] convert(%w)
+  %scale_b = f32[{G},{K},{N}] broadcast(%scale), dimensions={{0,2}}
+  %w_deq = f32[{G},{K},{N}] multiply(%w_f32, %scale_b)
+  %dot = f32[{M},{N}] ragged-dot(%lhs_f32, %w_deq, %sizes), lhs_contracting_dims={{1}}, rhs_contracting_dims={{1}}, lhs_ragged_dims={{0}}, rhs_group_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""
+
+
 def c3_fp8(M=8192, K=8192, N=8192, typed="f32", vector_scales=False):
     """f8 [M,K] . f8 [K,N] with per-tensor scales, + bias, GELU(tanh) -> bf16.  typed="f32":
     f32 ops and one final rounding; typed="bf16": every op bf16-typed (the shape of

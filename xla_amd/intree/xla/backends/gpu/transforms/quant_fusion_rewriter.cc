@@ -586,6 +586,62 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   return true;
 }
 
+// ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N], group_sizes [G]) with the ragged dimension
+// on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call whose
+// kernels read the group sizes on the device.  Decode sizes only: up to 64 rows in all.
+bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::function<void(std::string)>& log) {
+  QWeights q;
+  std::string why;
+  if (!MatchQWeights(dot->mutable_operand(1), &q, &why)) {
+    if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
+    return false;
+  }
+  auto refuse = [&](const std::string& w) {
+    log(absl::StrCat(dot->name(), ": quantized weights found but not rewritten: ", w));
+    return false;
+  };
+  Instr* lhs = dot->mutable_operand(0);
+  Instr* sizes = dot->mutable_operand(2);
+  Instr* inner;
+  if (ConvertFrom(lhs, BF16, &inner) && Ty(lhs) == F32) lhs = inner;
+  if (Ty(lhs) != BF16) return refuse("the activation must be bf16 (or its convert to f32)");
+  if (Rank(lhs) != 2 || Rank(q.w) != 3 || Rank(dot) != 2)
+    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] and a result [M,N]");
+  const RaggedDotDimensionNumbers& rd = Cast<HloRaggedDotInstruction>(dot)->ragged_dot_dimension_numbers();
+  const DotDimensionNumbers& dn = rd.dot_dimension_numbers();
+  auto is = [](const auto& d, int64_t v) { return d.size() == 1 && d[0] == v; };
+  if (!is(dn.lhs_contracting_dimensions(), 1) || !is(dn.rhs_contracting_dimensions(), 1) ||
+      !is(rd.lhs_ragged_dimensions(), 0) || !is(rd.rhs_group_dimensions(), 0) || dn.lhs_batch_dimensions_size() != 0)
+    return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
+                  "leading the weights");
+  const int64_t G = q.w->shape().dimensions(0), M = lhs->shape().dimensions(0), K = lhs->shape().dimensions(1),
+                N = q.w->shape().dimensions(2);
+  if (q.w->shape().dimensions(1) != K) return refuse("contracting dimensions differ");
+  if ((Ty(sizes) != S32 && Ty(sizes) != S64) || Dims(sizes) != std::vector<int64_t>{G})
+    return refuse("group sizes must be s32 or s64, one per group of weights");
+  if (M > 64) return refuse("a ragged dot over more than 64 rows is left to the grouped matmul");
+  const bool four_bit = Ty(q.w) == S4 || Ty(q.w) == U4;
+  if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
+  if (q.zero && Ty(q.w) != U4) return refuse("zero points are taken with u4 weights only");
+  if (q.zero && Dims(q.zero) != Dims(q.scale))
+    return refuse("zero points must have the shape of the scales (one per scale)");
+  if (Dims(q.scale) != std::vector<int64_t>{G, N})
+    return refuse("a ragged dot takes one scale per group and output channel");
+  if (q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
+  Epilogue ep;
+  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false)) return refuse(why);
+  std::vector<Instr*> ops = {lhs, q.w, q.scale};
+  if (q.zero) ops.push_back(q.zero);
+  if (ep.bias) ops.push_back(ep.bias);
+  ops.push_back(sizes);
+  Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, {ShapeUtil::MakeShape(BF16, Dims(dot))},
+                         CommonConfig(ep, q.type, Ty(dot)) + ", scale_group_size = 0 : i64");
+  CHECK_OK(ep.tail->ReplaceAllUsesWith(call));
+  VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
+          << (q.zero ? " with zero points" : "") << ", ragged over " << G << " groups]";
+  return true;
+}
+
 // ---------------------------------------------------------------- row-wise fp8 quantize
 bool IsReduceOver(Instr* r, HloOpcode body_op, int64_t dim, Instr** src, Instr** init) {
   if (r->opcode() != HloOpcode::kReduce || r->operand_count() != 2 || r->dimensions().size() != 1 ||
@@ -691,6 +747,8 @@ absl::StatusOr<bool> QuantFusionRewriter::RunImpl(HloModule* module,
       bool did = false;
       if (i->opcode() == HloOpcode::kDot && i->operand_count() == 2) {
         did = RewriteF8Dot(comp, i, log) || RewriteDequantDot(comp, i, log);
+      } else if (i->opcode() == HloOpcode::kRaggedDot && i->operand_count() == 3) {
+        did = RewriteRaggedDequantDot(comp, i, log);
       } else if (i->opcode() == HloOpcode::kCustomCall) {
         did = RewriteBlockScaledDot(comp, i, log);
       } else if (i->opcode() == HloOpcode::kConvert && Ty(i) == F8E4M3FN) {

@@ -57,26 +57,32 @@ def _scratch(nbytes, device):
 
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
-                scale_group_size=None, zero_points=None, out=None, scratch="auto", build_only=False):
+                scale_group_size=None, zero_points=None, group_sizes=None, out=None, scratch="auto",
+                build_only=False):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
     scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
     the handler reads the grouping off the scales' shape.
     weight_dtype "u4": unsigned 4-bit weights, packed like s4; zero_points (uint8, packed u4, one per
-    scale) then makes the dequantised weight (w - zero_point) * scale."""
-    _check_cuda(lhs, weights, scales, bias, zero_points)
+    scale) then makes the dequantised weight (w - zero_point) * scale.
+    group_sizes (int32 or int64 [G], on the device): ragged dot -- lhs [M,K] with its rows sorted by
+    group, weights [G,K,N]; group g multiplies rows [sum(sizes[:g]), +sizes[g]) with weights[g]."""
+    _check_cuda(lhs, weights, scales, bias, zero_points, group_sizes)
     wdt = {"s4": dtypes.S4, "u4": dtypes.U4}.get(weight_dtype, dtypes.S8)
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
     n = wshape[-1]
     oshape = list(lhs.shape[:-1]) + [n]
     if out is None:
         out = torch.empty(oshape, dtype=torch.bfloat16, device=lhs.device)
-    batch = lhs.shape[0] if lhs.dim() == 3 else 1
+    batch = lhs.shape[0] if lhs.dim() == 3 else (wshape[0] if group_sizes is not None else 1)
     args = [(dtypes.BF16, lhs.data_ptr(), lhs.shape), (wdt, weights.data_ptr(), wshape),
             (_FLOAT[scales.dtype], scales.data_ptr(), scales.shape)]
     if zero_points is not None:
         args.append((dtypes.U4, zero_points.data_ptr(), scales.shape))
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
+    if group_sizes is not None:
+        args.append((dtypes.S64 if group_sizes.dtype == torch.int64 else dtypes.S32, group_sizes.data_ptr(),
+                     group_sizes.shape))
     rets = [(dtypes.BF16, out.data_ptr(), oshape)]
     if scratch == "auto":
         nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(batch, lhs.shape[-2], lhs.shape[-1], n, wdt)
@@ -89,7 +95,7 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     if scale_group_size is not None:
         attrs["scale_group_size"] = ffi.Attr.i64(scale_group_size)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
-                keep=(lhs, weights, scales, bias, scratch, zero_points))
+                keep=(lhs, weights, scales, bias, scratch, zero_points, group_sizes))
     return call if build_only else call.run()
 
 

@@ -56,6 +56,24 @@ def u4_zero_point_group(M=8, K=4096, N=4096, group=128):
                 algorithmic_flops=2 * M * K * N)
 
 
+def ragged_s8_experts(M=32, K=4096, N=4096, groups=8, sizes=None):
+    """bf16 A[M,K] (rows sorted by expert) . (s8 W[G,K,N] * f32 scale[G,N]) + bias -> bf16 [M,N];
+    `sizes`: rows per expert (default: a random split of M, some experts empty)."""
+    rng = _rng(70 + M)
+    a = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = _rng(71).integers(-127, 128, size=(groups, K, N)).astype(np.int8)
+    scale = _rng(72).uniform(1e-3, 1e-2, size=(groups, N)).astype(np.float32)
+    bias = dtypes.f32_to_bf16(_rng(73).standard_normal((N,)).astype(np.float32))
+    if sizes is None:
+        cuts = np.sort(rng.integers(0, M + 1, size=groups - 1))
+        sizes = np.diff(np.concatenate([[0], cuts, [M]]))
+    return dict(name="ragged", lhs=a, weights=w, scales=scale, bias=bias, weight_dtype="s8",
+                weight_shape=(groups, K, N), group=K, dequant_type="f32", epilogue="BIAS",
+                group_sizes=np.asarray(sizes, np.int32),
+                algorithmic_bytes=groups * K * N + groups * N * 4 + N * 2 + M * K * 2 + M * N * 2,
+                algorithmic_flops=2 * M * K * N)
+
+
 def c3_fp8(M=8192, K=8192, N=8192):
     """f8 A[M,K] . f8 B[K,N], per-tensor f32 scales 1/64, + bias, GELU(tanh) -> bf16."""
     def f8(seed, shape):
