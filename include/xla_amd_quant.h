@@ -154,8 +154,9 @@ typedef struct XlaAmdDequantDot {
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);
 
-/* Scratch bytes with which the decode kernels may split K across workgroups (0 = never
- * needed for this shape).  The rewrite pass sizes the custom call's second result with it,
+/* Scratch bytes with which the kernels may split K across workgroups (0 = never needed for this
+ * shape): the decode kernels' K-slices up to 64 tokens, and above that the tiled kernel's last round
+ * of tiles when it is at most half full (256 KiB of f32 sums per tile of that round).  The rewrite pass sizes the custom call's second result with it,
  * the way `__cublas$lt$matmul` carries its workspace (gemm_rewriter_fp8_test.cc:1167).
  * A call without (enough) scratch still works; it just cannot split K. */
 XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K,
@@ -244,7 +245,8 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1:
  * the tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the
- * reference's cancellation to 2 bf16 ulp).  Returns 0, or -1 for an unknown key. */
+ * reference's cancellation to 2 bf16 ulp), "tiled_tail" (1: the tiled dequantize-dot kernel never
+ * splits the tiles of its last round along K).  Returns 0, or -1 for an unknown key. */
 XLA_AMD_EXPORT int xla_amd_debug_set_option(const char* key, int value);
 
 #ifdef __cplusplus

@@ -19,10 +19,11 @@ def say(msg):
     sys.stdout.flush()
 
 
-def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0):
+def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0, tail=0):
     """x: 1 keeps s4 weights off the kernels that dequantise through the 4x4x4 matrix instruction
     (default: off whenever a strip width `vec` of the other kernels is asked for); pair: 1 takes the
-    two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never."""
+    two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never; tail: 1 keeps
+    the tiled kernel from splitting the tiles of its last round along K."""
     lhs = dev_bf16(w["lhs"])
     if w["weight_dtype"] in ("s4", "u4"):
         wt = dev_u8(w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"]))
@@ -40,6 +41,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
     ffi.set_option("dequant_dot_pair", pair)
     ffi.set_option("dequant_dot_depth", depth)
     ffi.set_option("dequant_dot_steps", steps)
+    ffi.set_option("tiled_tail", tail)
     try:
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
                               weight_shape=w["weight_shape"], epilogue=w["epilogue"],
@@ -49,7 +51,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
         torch.cuda.synchronize()
     finally:
         for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec", "dequant_dot_x", "dequant_dot_pair",
-                  "dequant_dot_depth", "dequant_dot_steps"):
+                  "dequant_dot_depth", "dequant_dot_steps", "tiled_tail"):
             ffi.set_option(k, 0)
     return host_bf16(out), ffi.last_kernel()
 
@@ -434,7 +436,7 @@ def test_s4_group_scales_tiled(oracle, M, K, N, group):
     say("dequant_dot s4 tiled M=%d K=%d N=%d group=%d" % (M, K, N, group))
     w = workloads.c2_s4_group(M=M, K=K, N=N, group=group)
     got, kern = run_dot(w, force_kernel=3)   # at these sizes the cost model would pick the decode passes
-    assert kern == "dequant_dot_tiled_s4_rounded", kern
+    assert kern == ("dequant_dot_tiled_s4_rounded:tail2" if K >= 2048 else "dequant_dot_tiled_s4_rounded"), kern
     compare(oracle, w, got, "s4 tiled M=%d" % M)
 
 
@@ -506,14 +508,85 @@ def test_c5_full_size_sampled_blocks(oracle):
     say("dequant_dot C5 full size")
     w = workloads.c5_s8_batched()
     got, kern = run_dot(w)
-    assert kern == "dequant_dot_tiled_s8_factored", kern
+    # 896 tiles: three rounds of 256 whole tiles, then the 128 tiles of expert 6's end and expert 7
+    # as two workgroups each
+    assert kern == "dequant_dot_tiled_s8_factored:tail2", kern
     rng = np.random.default_rng(0)
-    for _ in range(6):
+    for i in range(8):
         b = int(rng.integers(0, 8)); m0 = int(rng.integers(0, 512 - 32)); n0 = int(rng.integers(0, 14336 - 64))
+        if i >= 6:
+            b = 7   # split tiles for certain
         sub = dict(w, lhs=np.ascontiguousarray(w["lhs"][b, m0:m0 + 32]),
                    weights=np.ascontiguousarray(w["weights"][b][:, n0:n0 + 64]),
                    scales=np.ascontiguousarray(w["scales"][b, n0:n0 + 64]), weight_shape=(4096, 64))
         compare(oracle, sub, got[b, m0:m0 + 32, n0:n0 + 64], "C5 block b=%d m0=%d n0=%d" % (b, m0, n0))
+
+
+@pytest.mark.parametrize("which,B,M,K,N", [("s8", 1, 300, 2048, 700), ("s8", 2, 257, 2304, 520),
+                                           ("s4", 1, 300, 4096, 520)])
+def test_tiled_last_round_split_along_k(oracle, which, B, M, K, N):
+    """Few tiles (a last round at most half full): every tile runs as two workgroups, the second half
+    of K handing its f32 sums to the first through the scratch.  Checked against the oracle, and
+    against the same call with the split switched off (sums in another order: a bf16 ulp apart at most)."""
+    say("dequant_dot tiled, tail split, %s B=%d M=%d K=%d N=%d" % (which, B, M, K, N))
+    if which == "s8":
+        w = workloads.c5_s8_batched(B=B, M=M, K=K, N=N)
+    else:
+        w = workloads.c2_s4_group(M=M, K=K, N=N, group=128)
+    base = "dequant_dot_tiled_s8_factored" if which == "s8" else "dequant_dot_tiled_s4_rounded"
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == base + ":tail2", kern
+    compare(oracle, w, got, "tail split " + which)
+    whole, kern = run_dot(w, force_kernel=3, tail=1)
+    assert kern == base, kern
+    d = np.abs(dtypes.bf16_to_f32(got).astype(np.float64) - dtypes.bf16_to_f32(whole).astype(np.float64))
+    mag = np.maximum(np.abs(dtypes.bf16_to_f32(whole).astype(np.float64)), floor_for(w))
+    assert np.all(d <= mag * 2.0 ** -7), "split and whole tiles differ by more than a bf16 ulp"
+
+
+def test_tiled_last_round_split_after_full_rounds(oracle):
+    """264 tiles: one round of 256 whole tiles, then 8 tiles as 16 workgroups; the same call frame
+    runs three times with new activations (the finishing workgroups lower the flags again), on a
+    scratch that starts out holding arbitrary bytes."""
+    say("dequant_dot tiled, 256 + 8 tiles, replayed")
+    B, M, K, N = 3, 1024, 2048, 5632
+    w = workloads.c5_s8_batched(B=B, M=M, K=K, N=N)
+    lhs, wt, sc = dev_bf16(w["lhs"]), dev_s8(w["weights"]), dev_f32(w["scales"])
+    nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(B, M, K, N, dtypes.S8)
+    assert nbytes == 8 * (256 * 256 * 4 + 8), nbytes
+    scratch = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda")
+    call = ops.dequant_dot(lhs, wt, sc, None, weight_dtype="s8", weight_shape=(B, K, N), epilogue="DEFAULT",
+                           dequant_type="f32", scratch=scratch, build_only=True)
+    rng = np.random.default_rng(11)
+    for it in range(3):
+        a = dtypes.f32_to_bf16(rng.standard_normal((B, M, K)).astype(np.float32))
+        lhs.copy_(dev_bf16(a))
+        out = call.run()
+        torch.cuda.synchronize()
+        assert ffi.last_kernel() == "dequant_dot_tiled_s8_factored:tail2", ffi.last_kernel()
+        got = host_bf16(out)
+        for i in range(8):
+            # the split tiles are the last 8 of expert 2 in launch order; sample there and elsewhere
+            b = 2 if i < 5 else int(rng.integers(0, B))
+            m0 = int(rng.integers(0, M - 32)); n0 = int(rng.integers(0, N - 64))
+            sub = dict(w, lhs=np.ascontiguousarray(a[b, m0:m0 + 32]),
+                       weights=np.ascontiguousarray(w["weights"][b][:, n0:n0 + 64]),
+                       scales=np.ascontiguousarray(w["scales"][b, n0:n0 + 64]), weight_shape=(K, 64))
+            compare(oracle, sub, got[b, m0:m0 + 32, n0:n0 + 64], "replay %d block b=%d m0=%d n0=%d" % (it, b, m0, n0))
+        # every output once against the unsplit kernel
+        if it == 0:
+            ffi.set_option("tiled_tail", 1)
+            try:
+                whole = host_bf16(ops.dequant_dot(lhs, wt, sc, None, weight_dtype="s8", weight_shape=(B, K, N),
+                                                  epilogue="DEFAULT", dequant_type="f32"))
+                torch.cuda.synchronize()
+                assert ffi.last_kernel() == "dequant_dot_tiled_s8_factored", ffi.last_kernel()
+            finally:
+                ffi.set_option("tiled_tail", 0)
+            g, h = dtypes.bf16_to_f32(got).astype(np.float64), dtypes.bf16_to_f32(whole).astype(np.float64)
+            differ = g != h
+            assert np.all(np.abs(g - h)[differ] <= np.maximum(np.abs(h[differ]) * 2.0 ** -7, 1e-2))
+            assert not differ[:2].any(), "whole tiles must not depend on the split"
 
 
 @pytest.mark.parametrize("M", [1, 8, 32, 64])

@@ -4,7 +4,7 @@ into a command buffer (a HIP graph) once and replay it step after step
 That only works if a call enqueues the same kernels for the same shapes, never synchronises,
 never reads device data on the host and allocates nothing.  Here decode steps of every kind
 (two workgroups per strip handing over inside the kernel, K-slices adding up inside the kernel,
-K-slices with a second launch, more than 64 tokens as several launches), a quantize and scaled dots
+K-slices with a second launch, more than 64 tokens as several launches, prefill tiles split along K), a quantize and scaled dots
 are captured into one graph through the native call-frame replay; the operands are then changed
 in place, and every replay must equal what eager calls give on the same data AND what the oracle
 computes from it."""
@@ -28,7 +28,7 @@ def say(msg):
 
 
 def test_handlers_replay_from_a_hip_graph(oracle):
-    say("graph capture of dequant_dot (pair hand-over, s8 in-kernel slices, split-K + finalize, 70 tokens), "
+    say("graph capture of dequant_dot (pair hand-over, s8 in-kernel slices, split-K + finalize, 70 tokens, split tiles), "
         "rowwise_quantize_fp8, fp8_scaled_dot (bf16 and f8 + amax)")
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(7)
@@ -37,7 +37,8 @@ def test_handlers_replay_from_a_hip_graph(oracle):
     for w, opts in ((workloads.c2_s4_group(M=8, K=2048, N=1024), {"dequant_dot_pair": 1}),  # pair hand-over
                     (workloads.c2_s4_group(M=20, K=2048, N=768, group=64), {"dequant_dot_slices": 2}),  # finalize launch
                     (workloads.c2_s4_group(M=70, K=1024, N=512), {}),                     # 64 + 6 tokens
-                    (workloads.c1_s8_channel(M=16, K=2048, N=1024), {})):                 # slices inside the kernel
+                    (workloads.c1_s8_channel(M=16, K=2048, N=1024), {}),                  # slices inside the kernel
+                    (workloads.c5_s8_batched(B=1, M=300, K=2048, N=700), {})):            # tiles split along K
         lhs = dev_bf16(w["lhs"])
         wt = dev_u8(w["weights_packed"]) if w["weight_dtype"] == "s4" else dev_s8(w["weights"])
         sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
@@ -59,6 +60,7 @@ def test_handlers_replay_from_a_hip_graph(oracle):
     assert dots[0][4] == "dequant_dot_decode_s4x_m16_pair", dots[0][4]
     assert dots[2][4].endswith(":x64"), dots[2][4]
     assert dots[3][4].startswith("dequant_dot_decode_s8x_"), dots[3][4]
+    assert dots[4][4] == "dequant_dot_tiled_s8_factored:tail2", dots[4][4]
 
     q4 = workloads.c4_quantize(rows=256, cols=1024)
     x, gamma = dev_bf16(q4["x"]), dev_bf16(q4["gamma"])

@@ -111,6 +111,10 @@ inline unsigned long long NextHandOverEpoch() {
 // (dequant_dot_decode.hip); mode: kRounded or kFactored.
 int LaunchDecodeFinalize(const DecodeParams& dp, int batch, hipStream_t stream, int mode);
 
+// Scratch the tiled prefill kernel uses to split the tiles of its last round along K
+// (tiled_dot_mfma.hip); 0 when the shape is not split.
+size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N);
+
 // K-slices a decode launch uses for this shape, and the f32 partial sums they need.
 int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves);
 size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices);

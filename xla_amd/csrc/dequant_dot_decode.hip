@@ -787,7 +787,7 @@ static int StaticScratchPointer(void** out) {
 
 int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream) {
   const size_t need = p.batch > 0 && p.M > 0 && p.K > 0 && p.N > 0
-                          ? DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4)
+                          ? DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4)
                           : 0;
   if (need > kStaticScratchBytes)
     return Fail(XLA_FFI_Error_Code_RESOURCE_EXHAUSTED,

@@ -30,6 +30,7 @@
 #include <atomic>
 #include <type_traits>
 
+#include "decode_common.h"
 #include "device_numerics.h"
 #include "launch.h"
 
@@ -65,7 +66,18 @@ struct TiledParams {
   const uint8_t* a_block_scales;  // kFp8MX: f8e8m0fnu [M, K/32]
   const uint8_t* b_block_scales;  // kFp8MX: f8e8m0fnu [N, K/32]
   int closed_form_epilogue;       // option "tiled_epilogue" = 1
+  // Integer-weight kinds: the tiles of the last, at most half-full round of 256 are each split over
+  // two workgroups along K (grid: tail_first whole tiles, then tail_tiles second halves, then
+  // tail_tiles first halves; one dimension, batches flattened).  A second half leaves its f32
+  // accumulators in tail_sums and raises its flag; the first half, dispatched after it, adds them
+  // to its own (first half + second half) and finishes the tile.
+  int tail_first, tail_tiles;
+  float* tail_sums;                 // [tail_tiles][32][512] x 16 bytes
+  unsigned long long* tail_flags;   // [tail_tiles]
+  unsigned long long epoch;         // value a raised flag holds for this launch
 };
+
+constexpr size_t kTailSumsBytes = (size_t)kTM * kTN * sizeof(float);  // per split tile
 
 __device__ __forceinline__ float e8m0_to_f32(uint32_t e) {
   return e == 0xffu ? bits_to_f32(0x7fc00000u) : e == 0u ? bits_to_f32(0x00400000u) : bits_to_f32(e << 23);
@@ -233,8 +245,23 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // Workgroup id -> tile: consecutive ids of one XCD take 8 neighbouring channel tiles of one
   // token tile, then the next token tile, so a token tile and 8 weight tiles stay hot in L2.
   int bid = blockIdx.x;
+  int batch = blockIdx.y;
+  int role = 0;       // 0: all of K; 1: second half of K, hands over; 2: first half of K, finishes
+  int tail_slot = 0;
+  const int tiles_per_batch = p.tiles_m * p.tiles_n;  // == gridDim.x unless the tail is split
+  if (WQ && p.tail_tiles > 0) {
+    int t = blockIdx.x;
+    if (t >= p.tail_first) {
+      t -= p.tail_first;
+      role = t < p.tail_tiles ? 1 : 2;
+      tail_slot = role == 1 ? t : t - p.tail_tiles;
+      t = p.tail_first + tail_slot;
+    }
+    batch = t / tiles_per_batch;
+    bid = t % tiles_per_batch;
+  }
   {
-    const int total = gridDim.x;
+    const int total = tiles_per_batch;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
   }
   int tm, tn;
@@ -252,7 +279,6 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       tm = r / w;
     }
   }
-  const int batch = blockIdx.y;
   const int m0 = tm * kTM, n0 = tn * kTN;
 
   const uint32_t a_pitch = (uint32_t)p.K * ESZ;
@@ -513,41 +539,86 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   };
 
   const int stages = (p.K + KS - 1) / KS;
-  issue_loads(0, 0);
-  if (WQ) wq_store(lds + kTM * kRow);
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-  __syncthreads();
-  issue_loads(1, KS);  // past K: lands as zeros, never read
-  for (int s = 0; s + 1 < stages; ++s) {
-    const int buf = s & 1;
-#pragma unroll
-    for (int ks = 0; ks + 1 < NKS; ++ks) {
-      read_frags(buf, ks);
-      mfma_all(ks);
-    }
-    read_frags(buf, NKS - 1);
-    if (WQ) wq_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+  const int half = (stages + 1) >> 1;
+  int s_begin = role == 1 ? half : 0, s_end = role == 2 ? half : stages;
+  bool add_sums = false;
+  __shared__ int tail_arrived;
+  for (;;) {
+    issue_loads(0, s_begin * KS);
+    if (WQ) wq_store(lds + kTM * kRow);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    issue_loads(buf, (s + 2) * KS);  // past K in the last rounds: zeros into a buffer nobody reads
-    mfma_all(NKS - 1);
-    if (F8) {
+    issue_loads(1, (s_begin + 1) * KS);  // past K: lands as zeros, never read
+    for (int s = s_begin; s + 1 < s_end; ++s) {
+      const int buf = (s - s_begin) & 1;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+      for (int ks = 0; ks + 1 < NKS; ++ks) {
+        read_frags(buf, ks);
+        mfma_all(ks);
+      }
+      read_frags(buf, NKS - 1);
+      if (WQ) wq_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+      issue_loads(buf, (s + 2) * KS);  // past this workgroup's stages in the last rounds: into a buffer nobody reads
+      mfma_all(NKS - 1);
+      if (F8) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+        }
       }
     }
-  }
-  {  // last stage: nothing left to fetch
-    const int buf = (stages - 1) & 1;
+    {  // last stage: nothing left to fetch
+      const int buf = (s_end - 1 - s_begin) & 1;
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      read_frags(buf, ks);
-      mfma_all(ks);
+      for (int ks = 0; ks < NKS; ++ks) {
+        read_frags(buf, ks);
+        mfma_all(ks);
+      }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads issued past the end have landed
+    __syncthreads();  // the epilogue (or another pass of this loop) reuses the stage buffers
+    if (!WQ || role != 2) break;
+    // first half done: wait (bounded) for the second half's flag.  That workgroup has a lower id,
+    // so it was dispatched before this one and is running or done.
+    if (tid == 0) {
+      int ok = 0;
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        if (__hip_atomic_load(p.tail_flags + tail_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) { ok = 1; break; }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      tail_arrived = ok;
+    }
+    __syncthreads();
+    if (tail_arrived) { add_sums = true; break; }
+    // the flag never showed: this workgroup does the second half as well, in K order
+    role = 0;
+    s_begin = half;
+    s_end = stages;
   }
-  __syncthreads();  // the epilogue reuses the stage buffers
+  constexpr int kDeviceScope = 16;  // sc1: performed where every XCD sees it
+  const __amdgpu_buffer_rsrc_t rt =
+      tile_rsrc(reinterpret_cast<const uint8_t*>(p.tail_sums) + (size_t)tail_slot * kTailSumsBytes,
+                WQ && (role == 1 || add_sums) ? (uint32_t)kTailSumsBytes : 0u);
+  if (WQ && role == 1) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const floatx16& a = acc[nt][mt];
+            __builtin_amdgcn_raw_buffer_store_b128(
+                uintx4{f32_to_bits(a[vq * 4]), f32_to_bits(a[vq * 4 + 1]), f32_to_bits(a[vq * 4 + 2]), f32_to_bits(a[vq * 4 + 3])},
+                rt, (uint32_t)((((nt * 4 + mt) * 4 + vq) * 512 + tid) * 16), 0, kDeviceScope);
+          }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) __hip_atomic_store(p.tail_flags + tail_slot, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+  }
 
   // ---- epilogue, staged through LDS (free now: every wave passed the last barrier).
   // Register v of tile (nt, mt) in lane (l32, kb) is token mt*32 + l32, channel
@@ -613,23 +684,56 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   }
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
+    if (WQ && add_sums) {
+      // the other half of K: this pass's 16 chunks are fetched together and added on the way into LDS
+      // (first half + second half), so the accumulators themselves are never rewritten
+      uintx4 o[2][2][4];
 #pragma unroll
-    for (int mtl = 0; mtl < 2; ++mtl) {
-      const int m = mtl * 32 + l32;
+      for (int mtl = 0; mtl < 2; ++mtl)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+        for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const int c = nt * 8 + vq * 2 + kb;
-          const floatx16& a = acc[nt][pass * 2 + mtl];
-          const floatx4 v = {a[vq * 4], a[vq * 4 + 1], a[vq * 4 + 2], a[vq * 4 + 3]};
-          *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
+          for (int vq = 0; vq < 4; ++vq)
+            o[mtl][nt][vq] = __builtin_amdgcn_raw_buffer_load_b128(
+                rt, (uint32_t)((((nt * 4 + pass * 2 + mtl) * 4 + vq) * 512 + tid) * 16), 0, kDeviceScope);
+#pragma unroll
+      for (int mtl = 0; mtl < 2; ++mtl) {
+        const int m = mtl * 32 + l32;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int c = nt * 8 + vq * 2 + kb;
+            const floatx16& a = acc[nt][pass * 2 + mtl];
+            const uintx4& q = o[mtl][nt][vq];
+            const floatx4 v = {a[vq * 4] + bits_to_f32(q[0]), a[vq * 4 + 1] + bits_to_f32(q[1]),
+                               a[vq * 4 + 2] + bits_to_f32(q[2]), a[vq * 4 + 3] + bits_to_f32(q[3])};
+            *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int mtl = 0; mtl < 2; ++mtl) {
+        const int m = mtl * 32 + l32;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const int c = nt * 8 + vq * 2 + kb;
+            const floatx16& a = acc[nt][pass * 2 + mtl];
+            const floatx4 v = {a[vq * 4], a[vq * 4 + 1], a[vq * 4 + 2], a[vq * 4 + 3]};
+            *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
+          }
         }
       }
     }
     d.m_base = m0 + wm * 128 + pass * 64;
     amax_bits = max(amax_bits, drain_dispatch<OUT_F8>(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops));
   }
+  // lowered again so that a replay of the same launch (a captured graph) waits for new sums
+  if (WQ && add_sums && tid == 0)
+    __hip_atomic_store(p.tail_flags + tail_slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (OUT_F8 && p.amax) {  // one atomic per wave into the result a fill kernel zeroed
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, off));
@@ -702,40 +806,42 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
                                                             int only_if_not_pow2) {
   if (only_if_not_pow2 && is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;
   const size_t total = (size_t)p.M * p.N;
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int n = (int)(idx % p.N), m = (int)(idx / p.N);
   // one batch per blockIdx.y
   p.a += (size_t)blockIdx.y * p.M * p.K;
   p.b += (size_t)blockIdx.y * p.K * p.N;
   if (p.out) p.out += (size_t)blockIdx.y * total;
   if (p.out8) p.out8 += (size_t)blockIdx.y * total;
   const bool mx = p.a_block_scales != nullptr;
-  float sa = 1.0f, sb = 1.0f;
-  if (!mx) { sa = p.a_scale[p.a_per_row ? m : 0]; sb = p.b_scale[p.b_per_channel ? n : 0]; }
-  if (deq_bf16) { sa = round_bf16(sa); sb = round_bf16(sb); }
   const int nblk = p.K >> 5;
-  float acc = 0.0f;
-  for (int k = 0; k < p.K; ++k) {
-    if (mx && (k & 31) == 0) {
-      sa = e8m0_to_f32(p.a_block_scales[(size_t)m * nblk + (k >> 5)]);
-      sb = e8m0_to_f32(p.b_block_scales[(size_t)n * nblk + (k >> 5)]);
+  // the grid is bounded (a call that returns at the first line costs a few workgroups, not one
+  // per 256 outputs): each workgroup strides over the outputs
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+    float sa = 1.0f, sb = 1.0f;
+    if (!mx) { sa = p.a_scale[p.a_per_row ? m : 0]; sb = p.b_scale[p.b_per_channel ? n : 0]; }
+    if (deq_bf16) { sa = round_bf16(sa); sb = round_bf16(sb); }
+    float acc = 0.0f;
+    for (int k = 0; k < p.K; ++k) {
+      if (mx && (k & 31) == 0) {
+        sa = e8m0_to_f32(p.a_block_scales[(size_t)m * nblk + (k >> 5)]);
+        sb = e8m0_to_f32(p.b_block_scales[(size_t)n * nblk + (k >> 5)]);
+      }
+      float av = f8e4m3fn_to_f32(p.a[(size_t)m * p.K + k]) * sa;
+      float bv = f8e4m3fn_to_f32(b_is_nk ? p.b[(size_t)n * p.K + k] : p.b[(size_t)k * p.N + n]) * sb;
+      if (deq_bf16) { av = round_bf16(av); bv = round_bf16(bv); }
+      acc = acc + av * bv;
     }
-    float av = f8e4m3fn_to_f32(p.a[(size_t)m * p.K + k]) * sa;
-    float bv = f8e4m3fn_to_f32(b_is_nk ? p.b[(size_t)n * p.K + k] : p.b[(size_t)k * p.N + n]) * sb;
-    if (deq_bf16) { av = round_bf16(av); bv = round_bf16(bv); }
-    acc = acc + av * bv;
-  }
-  float bias = 0.0f;
-  if (p.bias) bias = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n]) : ((const float*)p.bias)[n];
-  const float v = epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
-  if (p.out8) {
-    if (p.amax) atomicMax(reinterpret_cast<unsigned*>(p.amax), f32_to_bits(v) & 0x7fffffffu);
-    float c = p.d_divides ? v / *p.d_scale : v * *p.d_scale;
-    if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
-    p.out8[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
-  } else {
-    p.out[idx] = f32_to_bf16(v);
+    float bias = 0.0f;
+    if (p.bias) bias = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n]) : ((const float*)p.bias)[n];
+    const float v = epilogue_dispatch(acc, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
+    if (p.out8) {
+      if (p.amax) atomicMax(reinterpret_cast<unsigned*>(p.amax), f32_to_bits(v) & 0x7fffffffu);
+      float c = p.d_divides ? v / *p.d_scale : v * *p.d_scale;
+      if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+      p.out8[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
+    } else {
+      p.out[idx] = f32_to_bf16(v);
+    }
   }
 }
 
@@ -759,11 +865,23 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
     configured.fetch_or(bit, std::memory_order_release);
   }
   dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
+  if (tp.tail_tiles > 0) grid = dim3((unsigned)(tp.tail_first + 2 * tp.tail_tiles), 1u);
   hipLaunchKernelGGL((tiled_dot_kernel<KIND, OUT_F8>), grid, dim3(512), kLds, stream, tp);
   return CheckLaunch(what);
 }
 
 }  // namespace
+
+// Scratch for splitting the tiles of the last round along K: worth it when that round is at most
+// half full and K is long enough for half of it to outweigh the hand-over (256 KiB per tile,
+// written and read once).  0: no split for this shape.
+size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
+  if (batch <= 0 || M <= 64 || K < 2048 || N <= 0) return 0;
+  const int64_t tiles = batch * ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
+  const int64_t tail = tiles % 256;
+  if (tail == 0 || tail > 128 || tiles + tail > 0x7fffffff) return 0;
+  return (size_t)tail * (kTailSumsBytes + sizeof(unsigned long long));
+}
 
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
 // (the caller then falls back), 0 on success, or an error code.
@@ -807,12 +925,25 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.tiles_m = (tp.M + kTM - 1) / kTM;
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
+  // the last round of 256 workgroups, when at most half full, runs as two workgroups per tile
+  {
+    const size_t need = TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
+    if (need && GetOption("tiled_tail") != 1 && p.workspace && ((uintptr_t)p.workspace % 16) == 0 &&
+        p.workspace_bytes >= need) {
+      const int64_t tiles = p.batch * (int64_t)tp.tiles_m * tp.tiles_n;
+      tp.tail_tiles = (int)(tiles % 256);
+      tp.tail_first = (int)(tiles - tp.tail_tiles);
+      tp.tail_sums = (float*)p.workspace;
+      tp.tail_flags = (unsigned long long*)((char*)p.workspace + (size_t)tp.tail_tiles * kTailSumsBytes);
+      tp.epoch = NextHandOverEpoch();
+    }
+  }
   if (s4) {
     tp.group_shift = __builtin_ctzll((unsigned long long)p.group);
-    SetLastKernel("dequant_dot_tiled_s4_rounded");
+    SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_s4_rounded:tail2" : "dequant_dot_tiled_s4_rounded");
     return launch_tiled<kS4>(tp, (int)p.batch, stream, "dequant_dot_tiled_s4");
   }
-  SetLastKernel("dequant_dot_tiled_s8_factored");
+  SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_s8_factored:tail2" : "dequant_dot_tiled_s8_factored");
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
 
@@ -942,7 +1073,8 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
                 "for a [K,N] rhs, a workspace of K*N bytes");
   if (p.K == 0) tiled_ok = false;
 
-  dim3 egrid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)batch);
+  const size_t eblocks = ((size_t)p.M * p.N + 255) / 256;
+  dim3 egrid((unsigned)(eblocks < 8192 ? (eblocks ? eblocks : 1) : 8192), (unsigned)batch);
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;
