@@ -115,8 +115,48 @@ def test_quantize_empty_and_errors():
     assert q.shape == (0, 128) and s.shape == (0,)
     with pytest.raises(ffi.FfiError, match="gamma must have one entry per column"):
         ops.rowwise_quantize_fp8(torch.zeros((2, 64), dtype=torch.bfloat16, device="cuda"), g)
-    with pytest.raises(ffi.FfiError, match="not supported"):
-        ops.rowwise_quantize_fp8(torch.zeros((1, 16392), dtype=torch.bfloat16, device="cuda"), None)
+    with pytest.raises(ffi.FfiError, match="rows longer than 1048576 elements are not supported"):
+        ops.rowwise_quantize_fp8(torch.zeros((1, (1 << 20) + 8), dtype=torch.bfloat16, device="cuda"), None)
+
+
+@pytest.mark.parametrize("rows,cols,kernel", [(9, 28672, "long"), (3, 16392, "long"), (2, 65536, "long"),
+                                              (4, 20001, "long_unaligned"), (1, 1 << 20, "long")])
+def test_rmsnorm_quantize_long_rows(oracle, rows, cols, kernel):
+    """Rows past 16384 elements (an FFN activation of 28672, a vocabulary-sized row): the kernel that
+    walks the row three times instead of holding it in registers; same codes and scales, bit for bit,
+    windows of 32 and the levels above them in the oracle's order."""
+    say("quantize rmsnorm long rows=%d cols=%d" % (rows, cols))
+    w = workloads.c4_quantize(rows, cols)
+    q, s = run(w["x"], w["gamma"])
+    assert ffi.last_kernel() == "rowwise_quantize_fp8:" + kernel, ffi.last_kernel()
+    q_ref, s_ref = oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6)
+    assert np.array_equal(s.view(np.uint32), s_ref.view(np.uint32))
+    assert np.array_equal(q, q_ref)
+
+
+def test_quantize_long_special_rows(oracle):
+    """Long rows without RMSNorm: an all-zero row (NaN codes), a row with a NaN (NaN scale and codes),
+    tiny and huge rows (the IEEE-division path)."""
+    say("quantize long special rows")
+    cols = 20480
+    rng = np.random.default_rng(6)
+    base = rng.standard_normal((5, cols)).astype(np.float32)
+    base[0] = 0.0
+    base[1] *= 1e-30
+    base[2] *= 1e30
+    base[4, 12345] = np.nan
+    x = dtypes.f32_to_bf16(base)
+    q, s = run(x, None)
+    assert ffi.last_kernel() == "rowwise_quantize_fp8:long", ffi.last_kernel()
+    xf = dtypes.bf16_to_f32(x)
+    amax = np.abs(xf[:4]).max(axis=1)
+    s_ref = (amax / np.float32(448)).astype(np.float32)
+    assert np.array_equal(s[:4].view(np.uint32), s_ref.view(np.uint32))
+    assert np.all((q[0] & 0x7F) == 0x7F)
+    with np.errstate(all="ignore"):
+        d = np.clip((xf[1:4] / s_ref[1:, None]).astype(np.float32), -448, 448)
+    assert np.array_equal(q[1:4], oracle.f32_to_f8e4m3fn(d))
+    assert np.isnan(s[4]) and np.all((q[4] & 0x7F) == 0x7F)
 
 
 def test_c4_full_size_bit_exact(oracle):

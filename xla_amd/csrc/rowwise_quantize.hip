@@ -413,6 +413,151 @@ __global__ __launch_bounds__(kThreads) void rowwise_quantize_chain_kernel(
   }
 }
 
+// Rows longer than the register-resident kernels take (more than 16384 elements): the same
+// arithmetic in three walks over the row, which a workgroup re-reads from L2 instead of keeping it
+// in registers -- sums of squares per 32-element window (left to right, as above) into LDS and the
+// upper levels there; then y and its maximum; then the codes.  A row of up to 2^20 elements has at
+// most 32768 first-level sums (128 KiB of LDS, sized by the launch).
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void rowwise_quantize_long_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, uint8_t* __restrict__ q,
+    float* __restrict__ scales, int rows, int cols, float eps, int rmsnorm) {
+  extern __shared__ float lvl[];  // [n1] first-level sums, then [ceil(n1 / 32)] for the level above
+  __shared__ float red[kThreads / 64];
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x;
+  if (row >= rows) return;
+  const uint16_t* xr = x + (size_t)row * cols;
+  uint8_t* qr = q + (size_t)row * cols;
+
+  // eight consecutive elements from e0 on (zeros past the end of the row)
+  auto load8 = [&](const uint16_t* src, int e0, float* out) {
+    if (VEC) {
+      uintx4 w = {0u, 0u, 0u, 0u};
+      if (e0 < cols) w = *reinterpret_cast<const uintx4*>(src + e0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        out[2 * i] = bf16lo_to_f32(w[i]);
+        out[2 * i + 1] = bf16hi_to_f32(w[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[i] = e0 + i < cols ? bf16_to_f32(src[e0 + i]) : 0.0f;
+    }
+  };
+
+  float rinv = 1.0f;
+  if (rmsnorm) {
+    const int n1 = (cols + 31) / 32;
+    for (int w = tid; w < n1; w += kThreads) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float v[8];
+        load8(xr, w * 32 + c * 8, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = acc + v[i] * v[i];
+      }
+      lvl[w] = acc;
+    }
+    __syncthreads();
+    float* src = lvl;
+    float* dst = lvl + n1;
+    int n = n1;
+    while (n > 1) {
+      const int m = (n + 31) / 32;
+      for (int w = tid; w < m; w += kThreads) {
+        const int lo = w * 32, hi = min(lo + 32, n);
+        float acc = 0.0f;
+        for (int i = lo; i < hi; ++i) acc = acc + src[i];
+        dst[w] = acc;
+      }
+      __syncthreads();
+      float* t = src;
+      src = dst;
+      dst = t;
+      n = m;
+    }
+    const float ms = src[0] / (float)cols;
+    rinv = 1.0f / __builtin_sqrtf(ms + eps);
+  }
+
+  // y = bf16((x * rinv) * gamma), or x itself
+  auto y8 = [&](int e0, float* y) {
+    load8(xr, e0, y);
+    if (rmsnorm) {
+      float gm[8];
+      load8(gamma, e0, gm);
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        const uint32_t pk = pack_bf16x2((y[i] * rinv) * gm[i], (y[i + 1] * rinv) * gm[i + 1]);
+        y[i] = bf16lo_to_f32(pk);
+        y[i + 1] = bf16hi_to_f32(pk);
+      }
+    }
+  };
+
+  float amax = 0.0f;
+  bool has_nan = false;
+  for (int e0 = tid * 8; e0 < cols; e0 += kThreads * 8) {
+    float y[8];
+    y8(e0, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float a = __builtin_fabsf(y[i]);
+      has_nan |= a != a;
+      amax = __builtin_fmaxf(amax, a);
+    }
+  }
+  amax = wave_max(amax);
+  const bool any_nan = __any(has_nan);
+  if ((tid & 63) == 0) red[tid >> 6] = any_nan ? bits_to_f32(0x7fc00000u) : amax;
+  __syncthreads();
+  {
+    float m = red[0];
+    bool nan_seen = m != m;
+#pragma unroll
+    for (int i = 1; i < kThreads / 64; ++i) {
+      const float t = red[i];
+      nan_seen |= t != t;
+      m = __builtin_fmaxf(m, t);
+    }
+    amax = nan_seen ? bits_to_f32(0x7fc00000u) : m;  // maximum propagates NaN in XLA
+  }
+  const float s = amax / 448.0f;
+  if (tid == 0) scales[row] = s;
+  const bool fast = ordinary_divisor(s);
+  const float rs = 1.0f / s;
+
+  for (int e0 = tid * 8; e0 < cols; e0 += kThreads * 8) {
+    float y[8];
+    y8(e0, y);
+    uint32_t out[2];
+    if (fast) {
+      float d[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d[i] = __builtin_amdgcn_fmed3f(div_by_ordinary(y[i], s, rs), -448.0f, 448.0f);
+      out[0] = pack_f8x4(d[0], d[1], d[2], d[3]);
+      out[1] = pack_f8x4(d[4], d[5], d[6], d[7]);
+    } else {
+      out[0] = out[1] = 0u;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float t = y[i] / s;
+        if (t == t) t = __builtin_fminf(__builtin_fmaxf(t, -448.0f), 448.0f);
+        out[i >> 2] |= f32_to_f8e4m3fn_any(t) << (8 * (i & 3));
+      }
+    }
+    if (VEC) {
+      *reinterpret_cast<uintx2*>(qr + e0) = uintx2{out[0], out[1]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (e0 + i < cols) qr[e0 + i] = (uint8_t)(out[i >> 2] >> (8 * (i & 3)));
+    }
+  }
+}
+
 template <int CH, int G, bool VEC>
 void launch_variant(const XlaAmdRowwiseQuantize& p, hipStream_t stream) {
   hipLaunchKernelGGL((rowwise_quantize_kernel<CH, G, VEC>), dim3((unsigned)p.rows), dim3(kThreads),
@@ -432,11 +577,32 @@ int LaunchRowwiseQuantize(const XlaAmdRowwiseQuantize& p, hipStream_t stream, in
   if (!p.x || !p.q || !p.scales || (p.rmsnorm && !p.gamma))
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "rowwise_quantize_fp8: null buffer");
   constexpr int64_t kMaxCols = 256 * 8 * 8;  // 8 chunks of 8 per lane
-  if (p.cols > kMaxCols)
-    return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED,
-                "rowwise_quantize_fp8: rows longer than 16384 elements are not supported");
   const bool vec = p.cols % 8 == 0 && ((uintptr_t)p.x % 16 == 0) && ((uintptr_t)p.q % 8 == 0) &&
                    (!p.rmsnorm || (uintptr_t)p.gamma % 16 == 0);
+  if (p.cols > kMaxCols) {
+    if (p.cols > (1 << 20))
+      return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED,
+                  "rowwise_quantize_fp8: rows longer than 1048576 elements are not supported");
+    const int64_t n1 = (p.cols + 31) / 32;
+    const size_t lds = p.rmsnorm ? (size_t)(n1 + (n1 + 31) / 32) * sizeof(float) : 0;
+    const void* fn = vec ? (const void*)rowwise_quantize_long_kernel<true> : (const void*)rowwise_quantize_long_kernel<false>;
+    if (lds > 48 * 1024) {
+      // per kernel and device; setting it twice to the same value is harmless
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
+      if (e != hipSuccess)
+        return Fail(XLA_FFI_Error_Code_INTERNAL, "rowwise_quantize_fp8: cannot reserve LDS: %s", hipGetErrorString(e));
+    }
+    if (vec)
+      hipLaunchKernelGGL((rowwise_quantize_long_kernel<true>), dim3((unsigned)p.rows), dim3(kThreads), lds, stream,
+                         (const uint16_t*)p.x, (const uint16_t*)p.gamma, (uint8_t*)p.q, p.scales, (int)p.rows,
+                         (int)p.cols, p.eps, p.rmsnorm);
+    else
+      hipLaunchKernelGGL((rowwise_quantize_long_kernel<false>), dim3((unsigned)p.rows), dim3(kThreads), lds, stream,
+                         (const uint16_t*)p.x, (const uint16_t*)p.gamma, (uint8_t*)p.q, p.scales, (int)p.rows,
+                         (int)p.cols, p.eps, p.rmsnorm);
+    SetLastKernel(vec ? "rowwise_quantize_fp8:long" : "rowwise_quantize_fp8:long_unaligned");
+    return CheckLaunch("rowwise_quantize_fp8");
+  }
   const int64_t chunks = (p.cols + 7) / 8;          // 8-element chunks in a row
   const int64_t per_lane = (chunks + 255) / 256;    // chunks a lane must own
   // variant 0: the chained kernel for aligned rows; 1, 2, 3: the earlier layouts below (kept for
