@@ -740,3 +740,30 @@ def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
     assert kern == "dequant_dot_generic", kern
     ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
     check_dot(got_generic, ref, ragged_floor(w), "ragged generic")
+
+
+@pytest.mark.parametrize("M,K,N,G,sizes", [
+    (200, 512, 256, 4, [70, 0, 129, 1]), (640, 1024, 512, 8, None), (130, 512, 128, 2, [130, 0]),
+    (100, 256, 128, 3, [10, 20, 30]), (300, 512, 256, 3, [0, 400, 7])])
+def test_ragged_dot_more_than_64_rows(oracle, M, K, N, G, sizes):
+    """A ragged dot over any number of rows: every group is walked in chunks of 64 rows (a group of
+    130 rows as 64 + 64 + 2, one group that owns all rows, sizes that overrun M, 40 rows that no
+    group owns); rows of one group are bit-identical to an ordinary call on them."""
+    say("dequant_dot ragged prefill M=%d K=%d N=%d G=%d sizes=%s" % (M, K, N, G, sizes))
+    w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+    got, kern = run_ragged(w)
+    assert kern == "dequant_dot_decode_s8_v4_m64_factored", kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged prefill %s" % kern)
+    start = 0
+    for g, n in enumerate(w["group_sizes"]):
+        n = int(min(n, M - start))
+        if n > 0:
+            rows = slice(start, start + min(n, 64))   # the first chunk of the group, as a call of its own
+            sub = dict(w, lhs=np.ascontiguousarray(w["lhs"][rows]), weights=w["weights"][g], scales=w["scales"][g],
+                       weight_shape=w["weights"][g].shape)
+            one, k1 = run_dot(sub, force_kernel=2, x=1)
+            if k1 == kern:   # same kernel (64 rows): same bits
+                assert np.array_equal(got[rows], one), (g, kern, k1)
+        start += n
+    assert np.array_equal(got[start:], np.broadcast_to(w["bias"], (M - start, N)))

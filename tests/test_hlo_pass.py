@@ -516,8 +516,9 @@ def test_ragged_dot_over_expert_weights():
           r"scale_group_size = 0 : i64")
     assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
     assert hlo.rewrite(hm.ragged_s8_experts(16, 256, 64, 4, sizes_ty="s64"))[1] == rw
-    for bad, reason in ((hm.ragged_s8_experts(128, 256, 64, 4), "more than 64 rows"),
-                        (text.replace("lhs_ragged_dims={0}", "lhs_ragged_dims={1}"), "ragged dimension on the rows of lhs"),
+    # any number of rows: the kernel walks a group in chunks of 64
+    assert hlo.rewrite(hm.ragged_s8_experts(640, 256, 64, 4))[1] == rw
+    for bad, reason in ((text.replace("lhs_ragged_dims={0}", "lhs_ragged_dims={1}"), "ragged dimension on the rows of lhs"),
                         (text.replace("%sizes = s32[4]", "%sizes = u32[4]"), "group sizes must be s32 or s64")):
         new2, rw2, rf2 = hlo.rewrite(bad)
         assert rw2 == [] and any(reason in r for r in rf2), (rw2, rf2)

@@ -52,6 +52,7 @@ struct DecodeParams {
   const void* group_sizes;
   int group_sizes_64;
   int ragged_groups;  // number of groups (the kernels that do not carry it in grid.y)
+  int ragged_chunks;  // grid.z of a ragged launch: 64-row chunks any one group may need (1 up to 64 rows)
 };
 
 // Rows of a ragged dot that group g covers, read on the device: [*begin, *begin + *rows), clamped to

@@ -77,7 +77,13 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   int m_begin = batch * p.M, m_rows = p.M, tail_begin = -1;
   if (p.group_sizes) {
     ragged_rows(p, batch, &m_begin, &m_rows);
-    if (batch == (int)gridDim.y - 1) tail_begin = m_begin + m_rows;  // the last group also fills the rows no group owns
+    // the last group also fills the rows no group owns (its first chunk does)
+    if (batch == (int)gridDim.y - 1 && blockIdx.z == 0) tail_begin = m_begin + m_rows;
+    // a group of more than 16 * MT rows is spread over grid.z: chunk c takes rows [c * 16 * MT, + 16 * MT)
+    // of the group; chunks past its end have nothing to do
+    const int skip = min((int)blockIdx.z * 16 * MT, m_rows);
+    m_begin += skip;
+    m_rows = min(m_rows - skip, 16 * MT);
     if (m_rows == 0 && (tail_begin < 0 || tail_begin >= p.M)) return;
   }
 
@@ -433,7 +439,7 @@ int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const c
   else
     kern = g32 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, true>
                : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, false>;
-  dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
+  dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch, (unsigned)(dp.ragged_chunks > 1 ? dp.ragged_chunks : 1));
   hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
   if (rc) return rc;
@@ -598,6 +604,11 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.group_sizes = p.group_sizes;
   dp.group_sizes_64 = p.group_sizes_dtype == XLA_FFI_DataType_S64;
   dp.ragged_groups = ragged ? (int)p.batch : 0;
+  // a ragged dot over more than 64 rows: every group in chunks of 64 rows (grid.z), since any group
+  // may own any number of them; a chunk past its group's end returns at once
+  dp.ragged_chunks = ragged && p.M > 64 ? (int)((p.M + 63) / 64) : 1;
+  if (ragged && (p.M + 63) / 64 > 65535)
+    return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes at most 4194240 rows");
   const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
   const bool per_channel = p.group == p.K;
 
@@ -668,9 +679,9 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     return 0;
   }
 
-  if (force != 1 && force != 3 && aligned && mode_ok && p.M <= 64 && p.K >= 32) {
+  if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= 64 || ragged) && p.K >= 32) {
     int mt, vec, nv;
-    const bool shape_ok = decode_shape(p.M, &mt, &vec, &nv);
+    const bool shape_ok = decode_shape(p.M > 64 ? 64 : p.M, &mt, &vec, &nv);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // s4 with bf16 group scales and a bf16-typed multiply: the kernels that dequantise through the
     // 4x4x4 matrix instruction

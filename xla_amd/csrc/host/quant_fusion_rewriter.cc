@@ -672,11 +672,10 @@ bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
       dot->DimsAttr("rhs_group_dims") != std::vector<int64_t>{0} || !dot->DimsAttr("lhs_batch_dims").empty())
     return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
                   "leading the weights");
-  const int64_t G = q.w->shape.dims[0], M = lhs->shape.dims[0], K = lhs->shape.dims[1], N = q.w->shape.dims[2];
+  const int64_t G = q.w->shape.dims[0], K = lhs->shape.dims[1], N = q.w->shape.dims[2];  // any number of rows
   if (q.w->shape.dims[1] != K) return refuse("contracting dimensions differ");
   if ((sizes->shape.dtype != "s32" && sizes->shape.dtype != "s64") || sizes->shape.dims != std::vector<int64_t>{G})
     return refuse("group sizes must be s32 or s64, one per group of weights");
-  if (M > 64) return refuse("a ragged dot over more than 64 rows is left to the grouped matmul");
   const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
   if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
   if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");

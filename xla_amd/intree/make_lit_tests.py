@@ -26,7 +26,7 @@ def cases():
         ("quant_fusion_rewriter_u4_zero_points", hm.u4_zero_point_group(8, 256, 64, 64)),
         ("quant_fusion_rewriter_s8_batched", hm.c5_s8_batched(2, 8, 32, 16)),
         ("quant_fusion_rewriter_s8_ragged_experts", hm.ragged_s8_experts(16, 256, 64, 4)),
-        ("quant_fusion_rewriter_refuses_long_ragged_dot", hm.ragged_s8_experts(128, 256, 64, 4)),
+        ("quant_fusion_rewriter_s8_ragged_experts_prefill", hm.ragged_s8_experts(640, 256, 64, 4)),
         ("quant_fusion_rewriter_fp8_bias_gelu", hm.c3_fp8(64, 128, 32)),
         ("quant_fusion_rewriter_fp8_bf16_typed", hm.c3_fp8(64, 128, 32, typed="bf16")),
         ("quant_fusion_rewriter_fp8_vector_scales", hm.c3_fp8(64, 128, 32, vector_scales=True)),

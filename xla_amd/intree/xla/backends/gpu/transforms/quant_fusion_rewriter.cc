@@ -614,12 +614,11 @@ bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::functi
       !is(rd.lhs_ragged_dimensions(), 0) || !is(rd.rhs_group_dimensions(), 0) || dn.lhs_batch_dimensions_size() != 0)
     return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
                   "leading the weights");
-  const int64_t G = q.w->shape().dimensions(0), M = lhs->shape().dimensions(0), K = lhs->shape().dimensions(1),
+  const int64_t G = q.w->shape().dimensions(0), K = lhs->shape().dimensions(1),  // any number of rows
                 N = q.w->shape().dimensions(2);
   if (q.w->shape().dimensions(1) != K) return refuse("contracting dimensions differ");
   if ((Ty(sizes) != S32 && Ty(sizes) != S64) || Dims(sizes) != std::vector<int64_t>{G})
     return refuse("group sizes must be s32 or s64, one per group of weights");
-  if (M > 64) return refuse("a ragged dot over more than 64 rows is left to the grouped matmul");
   const bool four_bit = Ty(q.w) == S4 || Ty(q.w) == U4;
   if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
   if (q.zero && Ty(q.w) != U4) return refuse("zero points are taken with u4 weights only");
