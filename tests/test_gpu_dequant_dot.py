@@ -683,15 +683,16 @@ def test_u4_per_channel_f32_multiply(oracle, with_zero_points):
 # ---- ragged dot (tokens sorted by expert, group sizes on the device) -----------------------------
 
 def run_ragged(w, sizes_dtype=torch.int32, force_kernel=0):
-    lhs, wt = dev_bf16(w["lhs"]), dev_s8(w["weights"])
+    lhs = dev_bf16(w["lhs"])
+    wt = dev_u8(w["weights_packed"]) if w["weight_dtype"] == "s4" else dev_s8(w["weights"])
     sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
     bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
     gs = torch.from_numpy(np.asarray(w["group_sizes"], np.int64)).to(sizes_dtype).cuda()
     ffi.set_option("dequant_dot_kernel", force_kernel)
     try:
-        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype="s8", weight_shape=w["weight_shape"],
-                              epilogue=w["epilogue"], dequant_type=w["dequant_type"], scale_group_size=0,
-                              group_sizes=gs)
+        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"], weight_shape=w["weight_shape"],
+                              epilogue=w["epilogue"], dequant_type=w["dequant_type"],
+                              scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"], group_sizes=gs)
         torch.cuda.synchronize()
     finally:
         ffi.set_option("dequant_dot_kernel", 0)
@@ -767,3 +768,20 @@ def test_ragged_dot_more_than_64_rows(oracle, M, K, N, G, sizes):
                 assert np.array_equal(got[rows], one), (g, kern, k1)
         start += n
     assert np.array_equal(got[start:], np.broadcast_to(w["bias"], (M - start, N)))
+
+
+@pytest.mark.parametrize("M,K,N,G,group,sizes", [
+    (32, 1024, 512, 4, 128, None), (16, 512, 256, 3, 64, [9, 0, 5]), (200, 512, 256, 4, 128, [70, 0, 129, 1])])
+def test_ragged_dot_s4_group_scales(oracle, M, K, N, G, group, sizes):
+    """4-bit experts with bf16 scales per group of rows and channel under a bf16-typed multiply (one
+    rounding per weight), at decode and prefill row counts."""
+    say("dequant_dot ragged s4 M=%d K=%d N=%d G=%d group=%d sizes=%s" % (M, K, N, G, group, sizes))
+    w = workloads.ragged_s4_group_experts(M=M, K=K, N=N, groups=G, group=group, sizes=sizes)
+    got, kern = run_ragged(w)
+    assert kern.startswith("dequant_dot_decode_s4_") and kern.endswith("_rounded"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                    bias=w["bias"], group=group)
+    a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
+    wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), group, axis=1), axis=0)
+    check_dot(got, ref, dot_floor(a, wd, K), "ragged s4 %s" % kern)

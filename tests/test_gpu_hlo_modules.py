@@ -205,6 +205,47 @@ def test_c5_module():
     check_dot(host_bf16(out), ref, dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K), "C5 module")
 
 
+@pytest.mark.parametrize("M", [24, 150])
+def test_ragged_experts_modules(M):
+    """ragged-dot modules (s8 experts with a scale per expert and channel; s4 experts with scales per
+    128 rows of K as well) through the pass and the registry; the group sizes are a device operand."""
+    say("module ragged experts M=%d" % M)
+    K, N, G = 512, 256, 4
+    for kind in ("s8", "s4"):
+        if kind == "s8":
+            w, text = workloads.ragged_s8_experts(M, K, N, G), hm.ragged_s8_experts(M, K, N, G)
+            ops_in = [dev_bf16(w["lhs"]), dev_s8(w["weights"]), dev_f32(w["scales"]), dev_bf16(w["bias"])]
+            ref_in = [w["lhs"], w["weights"], w["scales"], w["bias"], w["group_sizes"]]
+            wd = np.max(np.abs(w["weights"].astype(np.float64)) * w["scales"].astype(np.float64)[:, None, :], axis=0)
+        else:
+            w, text = workloads.ragged_s4_group_experts(M, K, N, G, 128), hm.ragged_s4_group_experts(M, K, N, G, 128)
+            ops_in = [dev_bf16(w["lhs"]), dev_u8(w["weights_packed"]), dev_bf16(w["scales"]), dev_bf16(w["bias"])]
+            ref_in = [w["lhs"], w["weights"], w["scales"], w["bias"], w["group_sizes"]]
+            wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                        np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+        sizes = torch.from_numpy(w["group_sizes"].astype(np.int32)).cuda()
+        out, rw, _ = hlo_runner.compile_and_run(text, ops_in + [sizes])
+        torch.cuda.synchronize()
+        assert rw == ["dot -> xla_amd.dequant_dot [BIAS, %s, ragged over 4 groups]" % kind], rw
+        ref = reference(text, ref_in)
+        fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+        check_dot(host_bf16(out), ref, fl, "ragged %s module M=%d" % (kind, M))
+
+
+def test_batched_s4_group_module():
+    say("module batched s4 group scales")
+    B, M, K, N = 3, 8, 512, 256
+    w = workloads.batched_s4_group(B, M, K, N, 128)
+    text = hm.batched_s4_group(B, M, K, N, 128)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_u8(w["weights_packed"]), dev_bf16(w["scales"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s4]"], rw
+    ref = reference(text, [w["lhs"], w["weights"], w["scales"]])
+    wd = np.abs(w["weights"].astype(np.float64)) * np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1)
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+    check_dot(host_bf16(out), ref, fl, "batched s4 group module")
+
+
 def test_unrewritten_module_does_not_run():
     say("module with nothing to rewrite")
     text = "HloModule m\nENTRY e {\n  a = f32[4] parameter(0)\n  ROOT b = f32[4] add(a, a)\n}\n"

@@ -147,3 +147,23 @@ def test_ragged_dot(oracle, sizes):
                      [w["lhs"], w["weights"], w["scales"], w["bias"], w["group_sizes"]])
     ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("sizes", [[3, 3, 3, 3], [5, 0, 6, 1]])
+def test_ragged_dot_s4_group_scales(oracle, sizes):
+    """4-bit experts with one bf16 scale per 32 rows of K and channel, bf16-typed multiply: the module
+    op by op against the oracle's per-group composition, bit for bit."""
+    w = workloads.ragged_s4_group_experts(M=12, K=128, N=24, groups=4, group=32, sizes=sizes)
+    got = run_module(hm.ragged_s4_group_experts(12, 128, 24, 4, 32),
+                     [w["lhs"], w["weights"], w["scales"], w["bias"], w["group_sizes"]])
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                    bias=w["bias"], group=32)
+    assert np.array_equal(got, ref)
+
+
+def test_batched_s4_group_scales(oracle):
+    w = workloads.batched_s4_group(B=3, M=4, K=128, N=24, group=32)
+    got = run_module(hm.batched_s4_group(3, 4, 128, 24, 32), [w["lhs"], w["weights"], w["scales"]])
+    ref = np.stack([oracle.dequant_dot(w["lhs"][b], dtypes.pack_s4(w["weights"][b]), 4, w["scales"][b], "bf16", "bf16",
+                                       group=32) for b in range(3)])
+    assert np.array_equal(got, ref)

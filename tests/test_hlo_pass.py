@@ -522,3 +522,22 @@ def test_ragged_dot_over_expert_weights():
                         (text.replace("%sizes = s32[4]", "%sizes = u32[4]"), "group sizes must be s32 or s64")):
         new2, rw2, rf2 = hlo.rewrite(bad)
         assert rw2 == [] and any(reason in r for r in rf2), (rw2, rf2)
+
+
+def test_grouped_scales_behind_a_batch_or_expert_dimension():
+    """reshape([B,K/g,g,N] product) -> [B,K,N]: grouped scales [B,K/g,N] on batched weights, and on the
+    expert weights of a ragged dot; scale_group_size carries g."""
+    new, rw, rf = hlo.rewrite(hm.batched_s4_group(2, 8, 256, 64, 64))
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s4]"] and rf == []
+    check(new, r"custom-call\(%lhs, %w, %scales\), custom_call_target=\"xla_amd.dequant_dot\"",
+          r"scale_group_size = 64 : i64")
+    assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
+    text = hm.ragged_s4_group_experts(16, 256, 64, 4, 64)
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, s4, ragged over 4 groups]"] and rf == []
+    check(new, r"custom-call\(%lhs, %w, %scales, %bias, %sizes\), custom_call_target=\"xla_amd.dequant_dot\"",
+          r"scale_group_size = 64 : i64")
+    assert sorted(set(opcodes(new))) == ["custom-call", "parameter"]
+    # scales of another expert count are not this pattern
+    bad = text.replace("%scales = bf16[4,4,64] parameter(2)", "%scales = bf16[2,4,64] parameter(2)")
+    assert hlo.rewrite(bad)[1] == []

@@ -546,22 +546,27 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
   const std::string ty = op->shape.dtype;
   if (!IsFloatTy(ty)) return false;
   const int64_t rank = op->shape.rank();
-  // grouped: reshape([G,g,N] product) -> [K,N]
-  if (op->Is("reshape") && rank == 2 && op->operands[0]->shape.rank() == 3 && op->operands[0]->Is("multiply")) {
+  // grouped: reshape([G,g,N] product) -> [K,N], or with a leading batch / expert dimension
+  // reshape([B,G,g,N] product) -> [B,K,N]
+  if (op->Is("reshape") && (rank == 2 || rank == 3) && op->operands[0]->shape.rank() == rank + 1 &&
+      op->operands[0]->Is("multiply")) {
     Instr* mul = op->operands[0];
-    const auto& d3 = mul->shape.dims;  // G, g, N
-    if (d3[0] * d3[1] != op->shape.dims[0] || d3[2] != op->shape.dims[1]) return false;
+    const int64_t lead = rank - 2;  // 0, or 1 with a batch dimension in front
+    std::vector<int64_t> d3(mul->shape.dims.begin() + lead, mul->shape.dims.end());  // G, g, N
+    if (d3[0] * d3[1] != op->shape.dims[lead] || d3[2] != op->shape.dims[lead + 1]) return false;
+    if (lead && mul->shape.dims[0] != op->shape.dims[0]) return false;
+    const std::vector<int64_t> bdims = lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2};
     Instr *sc = nullptr, *cv = nullptr;
-    if (!BinaryWith(mul, "multiply", [&](Instr* s) { return BroadcastAlong(s, {0, 2}, &sc); }, &cv)) return false;
+    if (!BinaryWith(mul, "multiply", [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
     Instr* zero = nullptr;
-    PeelZeroPoint(cv, {0, 2}, ty, &cv, &zero);
+    PeelZeroPoint(cv, bdims, ty, &cv, &zero);
     // the convert may sit before or after the reshape to [G,g,N]
     Instr* w = nullptr;
     if (cv->Is("convert") && cv->operands[0]->Is("reshape")) {
       Instr* rs = cv->operands[0];
       Instr* src = rs->operands[0];
       if (IsByteWidening(src)) src = src->operands[0];
-      if ((src->shape.dtype == "s8" || src->shape.dtype == "s4" || src->shape.dtype == "u4") && src->shape.rank() == 2)
+      if ((src->shape.dtype == "s8" || src->shape.dtype == "s4" || src->shape.dtype == "u4") && src->shape.rank() == rank)
         w = src;
     } else if (cv->Is("reshape")) {
       IntSource(cv->operands[0], ty, &w);
@@ -571,7 +576,8 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
       return false;
     }
     sc = LookThroughWidening(sc, ty);
-    if (sc->shape.rank() != 2 || sc->shape.dims[0] != d3[0] || sc->shape.dims[1] != d3[2]) return false;
+    if (sc->shape.rank() != rank || sc->shape.dims[lead] != d3[0] || sc->shape.dims[lead + 1] != d3[2]) return false;
+    if (lead && sc->shape.dims[0] != op->shape.dims[0]) return false;
     *out = {w, sc, ty, zero};
     return true;
   }
@@ -634,7 +640,8 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
                   : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
   // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
-  const int64_t group_size = rank == 2 && q.scale->shape.rank() == 2 ? K / q.scale->shape.dims[0] : 0;
+  const int64_t group_size = rank == 2 && q.scale->shape.rank() == 2 ? K / q.scale->shape.dims[0]
+                             : rank == 3 && q.scale->shape.rank() == 3 ? K / q.scale->shape.dims[1] : 0;
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results,
                          CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
                              std::to_string(group_size) + " : i64");
@@ -647,7 +654,7 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
 
 // ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N], group_sizes [G]) with the ragged dimension
 // on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call whose
-// kernels read the group sizes on the device.  Decode sizes only: up to 64 rows in all.
+// kernels read the group sizes on the device, for any number of rows.
 bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   QWeights q;
   std::string why;
@@ -681,8 +688,13 @@ bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");
   if (q.zero && q.zero->shape.dims != q.scale->shape.dims)
     return refuse("zero points must have the shape of the scales (one per scale)");
-  if (q.scale->shape.dims != std::vector<int64_t>{G, N})
-    return refuse("a ragged dot takes one scale per group and output channel");
+  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well)
+  const bool grouped = q.scale->shape.rank() == 3;
+  if (!(q.scale->shape.dims == std::vector<int64_t>{G, N}) &&
+      !(grouped && q.scale->shape.dims[0] == G && q.scale->shape.dims[2] == N && q.scale->shape.dims[1] > 0 &&
+        K % q.scale->shape.dims[1] == 0))
+    return refuse("a ragged dot takes scales [groups,N] or [groups,K/g,N]");
+  const int64_t group_size = grouped ? K / q.scale->shape.dims[1] : 0;
   if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
   if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
@@ -691,7 +703,8 @@ bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   if (ep.bias) ops.push_back(ep.bias);
   ops.push_back(sizes);
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, {Shape::Array("bf16", dot->shape.dims)},
-                         CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = 0 : i64");
+                         CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
+                             std::to_string(group_size) + " : i64");
   comp->ReplaceAllUses(ep.tail, call);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
                           (q.zero ? " with zero points" : "") + ", ragged over " + std::to_string(G) + " groups]");

@@ -129,6 +129,56 @@ ENTRY %main {{
 """
 
 
+def ragged_s4_group_experts(M=32, K=4096, N=4096, groups=8, group=128):
+    """ragged-dot(bf16 [M,K], bf16(convert(s4 [G,K,N]) * bf16 scale[G,K/g,N]), group sizes [G]) + bias
+    -> bf16: 4-bit experts with one scale per `group` rows of K and channel, the dequantise multiply
+    bf16-typed (one rounding per weight) as in c2_s4_group."""
+    G, Kg = groups, K // group
+    return f"""HloModule ragged_s4_group_experts_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s4[{G},{K},{N}] parameter(1)
+  %scales = bf16[{G},{Kg},{N}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %sizes = s32[{G}] parameter(4)
+  %w_s8 = s8[{G},{K},{N}] convert(%w)
+  %w_g = s8[{G},{Kg},{group},{N}] reshape(%w_s8)
+  %w_bf16 = bf16[{G},{Kg},{group},{N}] convert(%w_g)
+  %scales_b = bf16[{G},{Kg},{group},{N}] broadcast(%scales), dimensions={{0,1,3}}
+  %w_deq_g = bf16[{G},{Kg},{group},{N}] multiply(%w_bf16, %scales_b)
+  %w_deq = bf16[{G},{K},{N}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] ragged-dot(%lhs, %w_deq, %sizes), lhs_contracting_dims={{1}}, rhs_contracting_dims={{1}}, lhs_ragged_dims={{0}}, rhs_group_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""
+
+
+def batched_s4_group(B=4, M=8, K=1024, N=512, group=128):
+    """bf16 [B,M,K] . bf16(convert(s4 [B,K,N]) * bf16 scale[B,K/g,N]), batch dimension 0 -> bf16
+    [B,M,N]: equally sized experts with 4-bit weights and grouped scales."""
+    Kg = K // group
+    return f"""HloModule batched_s4_group_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{B},{M},{K}] parameter(0)
+  %w = s4[{B},{K},{N}] parameter(1)
+  %scales = bf16[{B},{Kg},{N}] parameter(2)
+  %w_s8 = s8[{B},{K},{N}] convert(%w)
+  %w_g = s8[{B},{Kg},{group},{N}] reshape(%w_s8)
+  %w_bf16 = bf16[{B},{Kg},{group},{N}] convert(%w_g)
+  %scales_b = bf16[{B},{Kg},{group},{N}] broadcast(%scales), dimensions={{0,1,3}}
+  %w_deq_g = bf16[{B},{Kg},{group},{N}] multiply(%w_bf16, %scales_b)
+  %w_deq = bf16[{B},{K},{N}] reshape(%w_deq_g)
+  %dot = f32[{B},{M},{N}] dot(%lhs, %w_deq), lhs_batch_dims={{0}}, rhs_batch_dims={{0}}, lhs_contracting_dims={{2}}, rhs_contracting_dims={{1}}
+  ROOT %out = bf16[{B},{M},{N}] convert(%dot)
+}}
+"""
+
+
 def c3_fp8(M=8192, K=8192, N=8192, typed="f32", vector_scales=False):
     """f8 [M,K] . f8 [K,N] with per-tensor scales, + bias, GELU(tanh) -> bf16.  typed="f32":
     f32 ops and one final rounding; typed="bf16": every op bf16-typed (the shape of

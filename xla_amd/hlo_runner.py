@@ -17,9 +17,10 @@ import torch
 from . import dtypes, ffi, hlo
 
 _TORCH = {"f32": torch.float32, "bf16": torch.bfloat16, "s8": torch.int8, "u8": torch.uint8,
-          "f8e4m3fn": torch.uint8, "f8e8m0fnu": torch.uint8, "s4": torch.uint8}
-_DT = {"f32": dtypes.F32, "bf16": dtypes.BF16, "s8": dtypes.S8, "u8": dtypes.U8, "s4": dtypes.S4,
-       "f8e4m3fn": dtypes.F8E4M3FN, "f8e8m0fnu": dtypes.F8E8M0FNU}
+          "f8e4m3fn": torch.uint8, "f8e8m0fnu": torch.uint8, "s4": torch.uint8, "u4": torch.uint8,
+          "s32": torch.int32, "s64": torch.int64}
+_DT = {"f32": dtypes.F32, "bf16": dtypes.BF16, "s8": dtypes.S8, "u8": dtypes.U8, "s4": dtypes.S4, "u4": dtypes.U4,
+       "s32": dtypes.S32, "s64": dtypes.S64, "f8e4m3fn": dtypes.F8E4M3FN, "f8e8m0fnu": dtypes.F8E8M0FNU}
 
 
 def parse_backend_config(cfg):

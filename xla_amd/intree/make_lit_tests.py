@@ -27,6 +27,8 @@ def cases():
         ("quant_fusion_rewriter_s8_batched", hm.c5_s8_batched(2, 8, 32, 16)),
         ("quant_fusion_rewriter_s8_ragged_experts", hm.ragged_s8_experts(16, 256, 64, 4)),
         ("quant_fusion_rewriter_s8_ragged_experts_prefill", hm.ragged_s8_experts(640, 256, 64, 4)),
+        ("quant_fusion_rewriter_s4_ragged_experts_group_scales", hm.ragged_s4_group_experts(16, 256, 64, 4, 64)),
+        ("quant_fusion_rewriter_s4_batched_group_scales", hm.batched_s4_group(2, 8, 256, 64, 64)),
         ("quant_fusion_rewriter_fp8_bias_gelu", hm.c3_fp8(64, 128, 32)),
         ("quant_fusion_rewriter_fp8_bf16_typed", hm.c3_fp8(64, 128, 32, typed="bf16")),
         ("quant_fusion_rewriter_fp8_vector_scales", hm.c3_fp8(64, 128, 32, vector_scales=True)),

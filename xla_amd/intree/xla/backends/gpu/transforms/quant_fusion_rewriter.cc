@@ -489,22 +489,27 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
   const PrimitiveType ty = Ty(op);
   if (!IsFloatTy(ty)) return false;
   const int64_t rank = Rank(op);
-  // grouped: reshape([G,g,N] product) -> [K,N]
-  if (op->opcode() == HloOpcode::kReshape && rank == 2 && Rank(op->operand(0)) == 3 &&
+  // grouped: reshape([G,g,N] product) -> [K,N], or with a leading batch / expert dimension
+  // reshape([B,G,g,N] product) -> [B,K,N]
+  if (op->opcode() == HloOpcode::kReshape && (rank == 2 || rank == 3) && Rank(op->operand(0)) == rank + 1 &&
       op->operand(0)->opcode() == HloOpcode::kMultiply) {
     Instr* mul = op->mutable_operand(0);
-    const std::vector<int64_t> d3 = Dims(mul);  // G, g, N
-    if (d3[0] * d3[1] != op->shape().dimensions(0) || d3[2] != op->shape().dimensions(1)) return false;
+    const int64_t lead = rank - 2;  // 0, or 1 with a batch dimension in front
+    const std::vector<int64_t> dm = Dims(mul);
+    const std::vector<int64_t> d3(dm.begin() + lead, dm.end());  // G, g, N
+    if (d3[0] * d3[1] != op->shape().dimensions(lead) || d3[2] != op->shape().dimensions(lead + 1)) return false;
+    if (lead && dm[0] != op->shape().dimensions(0)) return false;
+    const std::vector<int64_t> gdims = lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2};
     Instr *sc = nullptr, *cv = nullptr;
-    if (!BinaryWith(mul, HloOpcode::kMultiply, [&](Instr* s) { return BroadcastAlong(s, {0, 2}, &sc); }, &cv))
+    if (!BinaryWith(mul, HloOpcode::kMultiply, [&](Instr* s) { return BroadcastAlong(s, gdims, &sc); }, &cv))
       return false;
     Instr* zero = nullptr;
-    PeelZeroPoint(cv, {0, 2}, ty, &cv, &zero);
+    PeelZeroPoint(cv, gdims, ty, &cv, &zero);
     Instr* w = nullptr;  // the convert may sit before or after the reshape to [G,g,N]
     if (cv->opcode() == HloOpcode::kConvert && cv->operand(0)->opcode() == HloOpcode::kReshape) {
       Instr* src = cv->mutable_operand(0)->mutable_operand(0);
       if (IsByteWidening(src)) src = src->mutable_operand(0);
-      if (IsQuantTy(Ty(src)) && Rank(src) == 2) w = src;
+      if (IsQuantTy(Ty(src)) && Rank(src) == rank) w = src;
     } else if (cv->opcode() == HloOpcode::kReshape) {
       IntSource(cv->mutable_operand(0), ty, &w);
     }
@@ -513,7 +518,9 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
       return false;
     }
     sc = LookThroughWidening(sc, ty);
-    if (Rank(sc) != 2 || sc->shape().dimensions(0) != d3[0] || sc->shape().dimensions(1) != d3[2]) return false;
+    if (Rank(sc) != rank || sc->shape().dimensions(lead) != d3[0] || sc->shape().dimensions(lead + 1) != d3[2])
+      return false;
+    if (lead && sc->shape().dimensions(0) != op->shape().dimensions(0)) return false;
     *out = {w, sc, ty, zero};
     return true;
   }
@@ -576,7 +583,9 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   if (size_t ws = xla_amd_dequant_dot_workspace_bytes(B, M, K, N, (int32_t)Ty(q.w)))
     results.push_back(ShapeUtil::MakeShape(S8, {(int64_t)ws}));
   // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
-  const int64_t group_size = rank == 2 && Rank(q.scale) == 2 ? K / q.scale->shape().dimensions(0) : 0;
+  const int64_t group_size = rank == 2 && Rank(q.scale) == 2   ? K / q.scale->shape().dimensions(0)
+                             : rank == 3 && Rank(q.scale) == 3 ? K / q.scale->shape().dimensions(1)
+                                                               : 0;
   Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, results,
                          CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64"));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0) : call;
@@ -588,7 +597,7 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
 
 // ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N], group_sizes [G]) with the ragged dimension
 // on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call whose
-// kernels read the group sizes on the device.  Decode sizes only: up to 64 rows in all.
+// kernels read the group sizes on the device, for any number of rows.
 bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::function<void(std::string)>& log) {
   QWeights q;
   std::string why;
@@ -624,8 +633,13 @@ bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::functi
   if (q.zero && Ty(q.w) != U4) return refuse("zero points are taken with u4 weights only");
   if (q.zero && Dims(q.zero) != Dims(q.scale))
     return refuse("zero points must have the shape of the scales (one per scale)");
-  if (Dims(q.scale) != std::vector<int64_t>{G, N})
-    return refuse("a ragged dot takes one scale per group and output channel");
+  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well)
+  const bool grouped = Rank(q.scale) == 3;
+  if (!(Dims(q.scale) == std::vector<int64_t>{G, N}) &&
+      !(grouped && q.scale->shape().dimensions(0) == G && q.scale->shape().dimensions(2) == N &&
+        q.scale->shape().dimensions(1) > 0 && K % q.scale->shape().dimensions(1) == 0))
+    return refuse("a ragged dot takes scales [groups,N] or [groups,K/g,N]");
+  const int64_t group_size = grouped ? K / q.scale->shape().dimensions(1) : 0;
   if (q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
   if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false)) return refuse(why);
@@ -634,7 +648,7 @@ bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::functi
   if (ep.bias) ops.push_back(ep.bias);
   ops.push_back(sizes);
   Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, {ShapeUtil::MakeShape(BF16, Dims(dot))},
-                         CommonConfig(ep, q.type, Ty(dot)) + ", scale_group_size = 0 : i64");
+                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64"));
   CHECK_OK(ep.tail->ReplaceAllUsesWith(call));
   VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
           << (q.zero ? " with zero points" : "") << ", ragged over " << G << " groups]";

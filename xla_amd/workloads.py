@@ -74,6 +74,34 @@ def ragged_s8_experts(M=32, K=4096, N=4096, groups=8, sizes=None):
                 algorithmic_flops=2 * M * K * N)
 
 
+def ragged_s4_group_experts(M=32, K=4096, N=4096, groups=8, group=128, sizes=None):
+    """bf16 A[M,K] (rows sorted by expert) . bf16(s4 W[G,K,N] * bf16 scale[G,K/group,N]) + bias -> bf16."""
+    rng = _rng(80 + M)
+    a = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = _rng(81).integers(-8, 8, size=(groups, K, N)).astype(np.int8)
+    scale = dtypes.f32_to_bf16(_rng(82).uniform(1e-3, 2e-2, size=(groups, K // group, N)).astype(np.float32))
+    bias = dtypes.f32_to_bf16(_rng(83).standard_normal((N,)).astype(np.float32))
+    if sizes is None:
+        cuts = np.sort(rng.integers(0, M + 1, size=groups - 1))
+        sizes = np.diff(np.concatenate([[0], cuts, [M]]))
+    return dict(name="ragged_s4", lhs=a, weights=w, weights_packed=dtypes.pack_s4(w), scales=scale, bias=bias,
+                weight_dtype="s4", weight_shape=(groups, K, N), group=group, dequant_type="bf16", epilogue="BIAS",
+                group_sizes=np.asarray(sizes, np.int32),
+                algorithmic_bytes=groups * K * N // 2 + groups * (K // group) * N * 2 + N * 2 + M * K * 2 + M * N * 2,
+                algorithmic_flops=2 * M * K * N)
+
+
+def batched_s4_group(B=4, M=8, K=1024, N=512, group=128):
+    """bf16 A[B,M,K] . bf16(s4 W[B,K,N] * bf16 scale[B,K/group,N]) -> bf16 [B,M,N]."""
+    a = dtypes.f32_to_bf16(_rng(90 + M).standard_normal((B, M, K)).astype(np.float32))
+    w = _rng(91).integers(-8, 8, size=(B, K, N)).astype(np.int8)
+    scale = dtypes.f32_to_bf16(_rng(92).uniform(1e-3, 2e-2, size=(B, K // group, N)).astype(np.float32))
+    return dict(name="batched_s4", lhs=a, weights=w, weights_packed=dtypes.pack_s4(w), scales=scale, bias=None,
+                weight_dtype="s4", weight_shape=(B, K, N), group=group, dequant_type="bf16", epilogue="DEFAULT",
+                algorithmic_bytes=B * (K * N // 2 + (K // group) * N * 2 + M * K * 2 + M * N * 2),
+                algorithmic_flops=2 * B * M * K * N)
+
+
 def c3_fp8(M=8192, K=8192, N=8192):
     """f8 A[M,K] . f8 B[K,N], per-tensor f32 scales 1/64, + bias, GELU(tanh) -> bf16."""
     def f8(seed, shape):
