@@ -745,7 +745,7 @@ def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
 
 @pytest.mark.parametrize("M,K,N,G,sizes", [
     (200, 512, 256, 4, [70, 0, 129, 1]), (640, 1024, 512, 8, None), (130, 512, 128, 2, [130, 0]),
-    (100, 256, 128, 3, [10, 20, 30]), (300, 512, 256, 3, [0, 400, 7])])
+    (100, 256, 128, 3, [10, 20, 30]), (300, 512, 256, 4, [0, 400, 7, 0])])
 def test_ragged_dot_more_than_64_rows(oracle, M, K, N, G, sizes):
     """A ragged dot over any number of rows: every group is walked in chunks of 64 rows (a group of
     130 rows as 64 + 64 + 2, one group that owns all rows, sizes that overrun M, 40 rows that no
@@ -785,3 +785,35 @@ def test_ragged_dot_s4_group_scales(oracle, M, K, N, G, group, sizes):
     wd = np.max(np.abs(w["weights"].astype(np.float64)) *
                 np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), group, axis=1), axis=0)
     check_dot(got, ref, dot_floor(a, wd, K), "ragged s4 %s" % kern)
+
+
+@pytest.mark.parametrize("kind,M,K,N,G,sizes", [
+    ("s8", 640, 1024, 512, 4, None), ("s8", 700, 512, 300, 3, [256, 1, 300]), ("s8", 512, 512, 256, 2, [0, 512]),
+    ("s8", 400, 512, 256, 4, [500, 3, 3, 3]), ("s4", 600, 1024, 512, 3, None), ("s4", 300, 2048, 256, 2, [10, 200])])
+def test_ragged_dot_grouped_gemm(oracle, kind, M, K, N, G, sizes):
+    """Groups that average 96 rows or more: the tiled kernel as a grouped GEMM -- 256-row tiles per
+    group, found on the device from the group sizes (a group of 257 rows is two tiles, the second with
+    one live row; empty groups, one group owning everything, sizes that overrun M, rows nobody owns)."""
+    say("dequant_dot ragged grouped GEMM %s M=%d K=%d N=%d G=%d sizes=%s" % (kind, M, K, N, G, sizes))
+    if kind == "s8":
+        w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+        floor = ragged_floor(w)
+        want = "dequant_dot_tiled_s8_factored:ragged"
+    else:
+        w = workloads.ragged_s4_group_experts(M=M, K=K, N=N, groups=G, group=128, sizes=sizes)
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                        bias=w["bias"], group=128)
+        wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                    np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+        floor = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+        want = "dequant_dot_tiled_s4_rounded:ragged"
+    got, kern = run_ragged(w)
+    assert kern == want, kern
+    check_dot(got, ref, floor, "ragged grouped GEMM %s" % kind)
+    # the decode kernel in 64-row chunks computes the same module
+    chunks, kern2 = run_ragged(w, force_kernel=2)
+    assert kern2.startswith("dequant_dot_decode_"), kern2
+    check_dot(chunks, ref, floor, "ragged chunks %s" % kind)
+    owned = int(min(M, np.sum(np.clip(w["group_sizes"], 0, None))))
+    assert np.array_equal(got[owned:], np.broadcast_to(w["bias"], (M - owned, N)))

@@ -617,7 +617,11 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
                        ((uintptr_t)p.weights % 16 == 0);
   const bool mode_ok = mode == kRounded || per_channel;
 
-  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && !ragged) {
+  // A ragged dot takes the tiled kernel (a grouped GEMM: 256-row tiles per group) once the groups
+  // average 96 rows; below that most tiles would be nearly empty and the 64-row chunks of the decode
+  // kernel do less work.  The sizes themselves are only known on the device.
+  const bool ragged_tiles = ragged && (force == 3 || (p.batch > 0 && p.M / p.batch >= 96));
+  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && (!ragged || ragged_tiles)) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }

@@ -75,6 +75,12 @@ struct TiledParams {
   float* tail_sums;                 // [tail_tiles][32][512] x 16 bytes
   unsigned long long* tail_flags;   // [tail_tiles]
   unsigned long long epoch;         // value a raised flag holds for this launch
+  // Integer-weight kinds, ragged dot: a is [M,K] with rows sorted by group, b [groups,K,N], out [M,N].
+  // Group g owns rows [sum of the sizes before it, + its size), read on the device.  The grid holds
+  // tiles_n x ragged_slots workgroups; slot s is the s-th 256-row tile counted over all groups (a
+  // group of n rows has ceil(n / 256) of them), slots past the last tile return.
+  const void* group_sizes;
+  int group_sizes_64, ragged_groups, ragged_slots;
 };
 
 constexpr size_t kTailSumsBytes = (size_t)kTM * kTN * sizeof(float);  // per split tile
@@ -260,12 +266,39 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     batch = t / tiles_per_batch;
     bid = t % tiles_per_batch;
   }
-  {
+  const bool ragged = WQ && p.group_sizes != nullptr;
+  int m0r = 0, m_limit = p.M;  // ragged: first row of the tile and the end of its group's rows
+  if (ragged) {
+    // consecutive ids share a row tile (and with it an activation tile in L2)
+    const int slot0 = bid / p.tiles_n;
+    int slot = slot0;
+    long long start = 0;
+    bool found = false;
+    for (int g = 0; g < p.ragged_groups; ++g) {
+      long long n = p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+      n = n < 0 ? 0 : (n > p.M - start ? p.M - start : n);   // sizes that do not add up stay inside [0, M]
+      const int tiles_g = (int)((n + kTM - 1) / kTM);
+      if (slot < tiles_g) {
+        batch = g;
+        m0r = (int)start + slot * kTM;
+        m_limit = (int)(start + n);
+        found = true;
+        break;
+      }
+      slot -= tiles_g;
+      start += n;
+    }
+    if (!found) return;
+  }
+  if (!ragged) {
     const int total = tiles_per_batch;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;
   }
   int tm, tn;
-  {
+  if (ragged) {
+    tm = 0;
+    tn = bid % p.tiles_n;
+  } else {
     const int G = 8;
     const int full = (p.tiles_n / G) * G;           // channel tiles covered by complete groups
     const int per_group = G * p.tiles_m;
@@ -279,11 +312,12 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       tm = r / w;
     }
   }
-  const int m0 = tm * kTM, n0 = tn * kTN;
+  const int m0 = ragged ? m0r : tm * kTM, n0 = tn * kTN;
+  const int a_batch = ragged ? 0 : batch;  // a ragged dot has one [M,K] activation and one [M,N] result
 
   const uint32_t a_pitch = (uint32_t)p.K * ESZ;
   const __amdgpu_buffer_rsrc_t ra =
-      tile_rsrc(p.a + (size_t)batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
+      tile_rsrc(p.a + (size_t)a_batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
   const uint32_t b_bytes = KIND == kS4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N;
   const __amdgpu_buffer_rsrc_t rb = tile_rsrc(p.b + (size_t)batch * b_bytes, b_bytes);  // bytes, either layout
 
@@ -654,9 +688,9 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   d.rd_chunk = rd_chunk;
   d.rd_row = rd_row;
   d.n = n;
-  d.M = p.M;
+  d.M = m_limit;  // rows from here on belong to the next group (or lie past M): computed, never stored
   d.N = p.N;
-  d.out = p.out + (size_t)batch * p.M * p.N;
+  d.out = p.out + (size_t)a_batch * p.M * p.N;
   d.out8 = nullptr;
   d.want_amax = OUT_F8 && p.amax != nullptr;
   d.closed_form = p.closed_form_epilogue != 0;
@@ -847,6 +881,23 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
 
 __global__ void store_u32_kernel(uint32_t* dst, uint32_t value) { *dst = value; }
 
+// Ragged dot: rows past the last group are a dot of nothing, epilogue(0).  Workgroup (x, y) takes 256
+// channels and every gridDim.y-th of those rows; usually there are none and it returns at once.
+__global__ __launch_bounds__(256) void ragged_tail_rows_kernel(TiledParams p) {
+  long long start = 0;
+  for (int g = 0; g < p.ragged_groups; ++g) {
+    long long n = p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+    n = n < 0 ? 0 : (n > p.M - start ? p.M - start : n);
+    start += n;
+  }
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= p.N) return;
+  float bias = 0.0f;
+  if (p.bias) bias = p.bias_is_bf16 ? bf16_to_f32(((const uint16_t*)p.bias)[n]) : ((const float*)p.bias)[n];
+  const uint16_t v = f32_to_bf16(epilogue_dispatch(0.0f, bias, p.epilogue, p.bf16_dot, p.bf16_ops));
+  for (long long m = start + blockIdx.y; m < p.M; m += gridDim.y) p.out[(size_t)m * p.N + n] = v;
+}
+
 template <int KIND, bool OUT_F8 = false>
 int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
   constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow + (KIND == kFp8MX ? 4096 : 0);  // 128 KiB (+ scales)
@@ -894,7 +945,8 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
                   (double)(p.K / p.group) * p.N * 2 < 2147483000.0;
   const bool s8 = p.weight_dtype == XLA_FFI_DataType_S8 && p.group == p.K && p.dequant_type == XLA_FFI_DataType_F32;
   if (!s4 && !s8) return -1;
-  if (s4 && GetOption("dequant_dot_kernel") != 3) {
+  const bool ragged = p.group_sizes != nullptr;  // the caller has decided that the rows per group make tiles worth it
+  if (s4 && !ragged && GetOption("dequant_dot_kernel") != 3) {
     // The decode kernel, run once per 64 tokens, streams and dequantises the weights on every
     // pass but fills the machine at any M; the tiled kernel dequantises once per 256 tokens but
     // needs 256 tiles per round.  Estimates in microseconds fitted on MI355X (8192 x 28672:
@@ -925,6 +977,22 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.tiles_m = (tp.M + kTM - 1) / kTM;
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
+  if (s4) tp.group_shift = __builtin_ctzll((unsigned long long)p.group);  // sizes the scales' descriptor: set before any launch
+  if (ragged) {
+    // at most floor(M / 256) + groups tiles of rows, whatever the sizes turn out to be
+    tp.group_sizes = p.group_sizes;
+    tp.group_sizes_64 = p.group_sizes_dtype == XLA_FFI_DataType_S64;
+    tp.ragged_groups = (int)p.batch;
+    tp.ragged_slots = (int)(p.M / kTM + p.batch);
+    if ((double)tp.ragged_slots * tp.tiles_n > 2147483000.0) return -1;
+    tp.tiles_m = tp.ragged_slots;
+    tp.scale_batched = p.scale_batch == p.batch;  // one set of scales per group, also for a single group
+    const int rc = s4 ? launch_tiled<kS4>(tp, 1, stream, "dequant_dot_tiled_s4") : launch_tiled<kS8>(tp, 1, stream, "dequant_dot_tiled_s8");
+    if (rc) return rc;
+    hipLaunchKernelGGL(ragged_tail_rows_kernel, dim3((unsigned)((p.N + 255) / 256), 64u), dim3(256), 0, stream, tp);
+    SetLastKernel(s4 ? "dequant_dot_tiled_s4_rounded:ragged" : "dequant_dot_tiled_s8_factored:ragged");
+    return CheckLaunch("dequant_dot_ragged_tail_rows");
+  }
   // the last round of 256 workgroups, when at most half full, runs as two workgroups per tile
   {
     const size_t need = TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
@@ -939,7 +1007,6 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
     }
   }
   if (s4) {
-    tp.group_shift = __builtin_ctzll((unsigned long long)p.group);
     SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_s4_rounded:tail2" : "dequant_dot_tiled_s4_rounded");
     return launch_tiled<kS4>(tp, (int)p.batch, stream, "dequant_dot_tiled_s4");
   }
