@@ -268,7 +268,15 @@ def main():
         entry("C5", "C5 s8 [8,512,4096]x[8,4096,14336]", ops.dequant_dot(a5, w5, s5, scale_group_size=0, build_only=True),
               8 * (4096 * 14336 + 512 * 4096 * 2 + 14336 * 4 + 512 * 14336 * 2),
               2 * 8 * 512 * 4096 * 14336, "mfma", "bf16")
-        del a5, w5
+        # the same experts with routing: 4096 tokens sorted by expert, uneven group sizes read on the device
+        # (ragged dot as a grouped GEMM; informational -- not one of the five configurations)
+        a5r = torch.randn((4096, 4096), device=dev).to(torch.bfloat16)
+        gsz5 = torch.tensor([1024, 0, 512, 512, 100, 924, 512, 512], dtype=torch.int32, device=dev)
+        entry("ragged prefill", "ragged s8 [4096,4096] x [8,4096,14336], groups of 1024/0/512/512/100/924/512/512 rows",
+              ops.dequant_dot(a5r, w5, s5, scale_group_size=0, group_sizes=gsz5, build_only=True),
+              8 * (4096 * 14336 + 14336 * 4) + 4096 * 4096 * 2 + 4096 * 14336 * 2,
+              2 * 4096 * 4096 * 14336, "mfma", "bf16")
+        del a5, w5, a5r
 
     # ---- CPU baselines: the oracle on the same workload, or on a stated sample of it ------------
     cpu = None
@@ -336,6 +344,9 @@ def main():
             t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))
             by_key["C5"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
                                                 "1 of 8 batches, 64 of 512 tokens (full K and N), %.2f s" % t)
+            if "ragged prefill" in by_key:   # the same arithmetic per row and expert
+                by_key["ragged prefill"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
+                                                                "64 rows of one expert (full K and N), %.2f s" % t)
 
     out = {
         "metric": "quant-dot HBM GB/s on the s4 group-128 decode dequantize-dot (% of MI355X roofline) "
