@@ -208,9 +208,10 @@ typedef struct XlaAmdFp8ScaledDot {
 
 XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, void* stream);
 
-/* K*N bytes when the rhs is [K,N] (it is re-laid out with K minor first, the transpose
- * GemmRewriter inserts at gemm_rewriter.cc:1235-1591), else 0.  Without it a [K,N] rhs runs
- * on the slow exact kernel. */
+/* Scratch the call can use (0 = none).  A [K,N] rhs whose N is a multiple of 16 goes in as it is;
+ * any other [K,N] rhs is re-laid out with K minor first (the transpose GemmRewriter inserts at
+ * gemm_rewriter.cc:1235-1591), which takes K*N bytes -- without them such a rhs runs on the slow
+ * exact kernel. */
 XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                                              int32_t rhs_contracting_dim);
 

@@ -109,7 +109,9 @@ def test_c3_fp8_bias_gelu(typed, code):
     check(new, r"custom-call\(%a, %b, %a_scale\S*, %b_scale\S*, %bias\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
           r'epilogue = \\"BIAS_GELU\\", dequant_type = %d : i32, dot_type = %d : i32, epilogue_type = %d : i32, '
           r'rhs_contracting_dim = 0 : i64' % (code, code, code))
-    assert "s8[67108864]{0}" in new            # K*N bytes to re-lay the [K,N] rhs out with K minor
+    assert "s8[" not in new                    # N % 16 == 0: the [K,N] rhs goes in as it is, no scratch
+    ragged_n = hlo.rewrite(hm.c3_fp8(512, 4096, 1000, typed=typed))[0]
+    assert "s8[4096000]{0}" in ragged_n        # K*N bytes to re-lay a [K,N] rhs out with K minor when N % 16 != 0
     if typed == "bf16":                        # bf16 scalars are widened, as GemmRewriter does
         check(new, r"%a_scale.f32 = f32\[\] convert\(%a_scale\)", r"%b_scale.f32 = f32\[\] convert\(%b_scale\)")
 
@@ -138,20 +140,21 @@ def test_c3_fp8_with_f8_result():
     """divide (or multiply) by a per-tensor scale -> clamp(+-448) -> convert(f8e4m3fn) after the
     epilogue is taken into the call: the scale is the last operand, the result is f8
     (gemm_rewriter_fp8_test.cc:1665-1690; the reference leaves it unfused on ROCm, :1710)."""
+    # N = 40 is no multiple of 16: the [K,N] rhs is re-laid out through K*N bytes of scratch
     for mul in (False, True):
-        new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 32, multiply=mul))
+        new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 40, multiply=mul))
         assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result]"] and rf == []
-        check(new, r"\(f8e4m3fn\[64,32\]\{1,0\}, s8\[4096\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
+        check(new, r"\(f8e4m3fn\[64,40\]\{1,0\}, s8\[5120\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
               r"d_scale_multiplies = %s" % ("true" if mul else "false"))
         assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
     # the result's own amax (reduce-maximum of abs over both dimensions) becomes a second result
-    new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 32, amax=True))
+    new, rw, rf = hlo.rewrite(hm.c3_fp8_f8_result(64, 128, 40, amax=True))
     assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, f8 result, amax]"] and rf == []
-    check(new, r"\(f8e4m3fn\[64,32\]\{1,0\}, f32\[\], s8\[4096\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
+    check(new, r"\(f8e4m3fn\[64,40\]\{1,0\}, f32\[\], s8\[5120\]\{0\}\) custom-call\(%a, %b, %a_scale, %b_scale, %bias, %d_scale\)",
           r"ROOT %result = .* tuple\(%out.out, %amax.amax\)")
     assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter", "tuple"]
     # a clamp to anything but +-448 is not the f8 saturation: left alone, with the reason
-    bad = hm.c3_fp8_f8_result(64, 128, 32).replace("constant(448)", "constant(240)")
+    bad = hm.c3_fp8_f8_result(64, 128, 40).replace("constant(448)", "constant(240)")
     new, rw, rf = hlo.rewrite(bad)
     assert rw == [] and any("is f32, the kernels produce bf16" in r for r in rf)
 

@@ -1014,8 +1014,9 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
 
+// The transposed copy of a [K,N] rhs that cannot go in as it is: N no multiple of 16, or the pre-pass forced.
 size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim) {
-  return rhs_contracting_dim == 0 ? (size_t)K * N : 0;
+  return rhs_contracting_dim == 0 && (N % 16 != 0 || GetOption("fp8_dot_layout") == 1) ? (size_t)K * N : 0;
 }
 
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
