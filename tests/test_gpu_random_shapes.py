@@ -7,7 +7,8 @@ import pytest
 import torch
 
 from tests.gpu_util import dev_bf16
-from tests.test_gpu_dequant_dot import compare, run_dot
+from tests.test_gpu_dequant_dot import compare, ragged_floor, run_dot, run_ragged
+from tests.gpu_util import dot_floor
 from tests.test_gpu_fp8_dot import EPI, floor_for, reference, run
 from tests.gpu_util import check_dot
 from xla_amd import dtypes, ffi, ops, workloads
@@ -81,7 +82,7 @@ def test_rowwise_quantize_random_shapes(oracle):
     rng = np.random.default_rng(5)
     for case in range(12):
         R = int(rng.integers(1, 40))
-        C = int(rng.choice([8, 33, 256, 1000, 1024, 4096, 5000, 8192, 16384]))
+        C = int(rng.choice([8, 33, 256, 1000, 1024, 4096, 5000, 8192, 16384, 20000, 33001]))
         rms = bool(rng.integers(0, 2))
         say("rowwise_quantize_fp8 #%d R=%d C=%d rmsnorm=%s" % (case, R, C, rms))
         x = dtypes.f32_to_bf16((rng.standard_normal((R, C)) * rng.choice([1e-3, 1.0, 300.0])).astype(np.float32))
@@ -96,3 +97,36 @@ def test_rowwise_quantize_random_shapes(oracle):
             q_ref = oracle.f32_to_f8e4m3fn(np.clip((xf / s_ref[:, None]).astype(np.float32), -448, 448))
         assert np.array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32)), case
         assert np.array_equal(q.cpu().numpy().view(np.uint8), q_ref), case
+
+
+def test_ragged_dot_random_shapes(oracle):
+    """Random row counts, expert counts and splits (empty groups, sizes that overrun M, rows nobody
+    owns), s8 experts with a scale per channel and s4 experts with group scales: whichever of the
+    decode chunks and the grouped GEMM the launcher picks."""
+    rng = np.random.default_rng(31)
+    kernels = set()
+    for case in range(14):
+        s4 = bool(rng.integers(0, 2))
+        G = int(rng.integers(1, 7))
+        M = int(rng.choice([1, 7, 40, 64, 65, 130, 300, 520, 700]))
+        K = 128 * int(rng.integers(1, 9))
+        N = int(rng.choice([64, 128, 264, 512]))
+        sizes = rng.multinomial(int(M * rng.choice([0.6, 1.0, 1.3])), np.ones(G) / G)
+        if rng.integers(0, 3) == 0:
+            sizes[int(rng.integers(0, G))] = 0
+        say("ragged #%d %s M=%d K=%d N=%d G=%d sizes=%s" % (case, "s4" if s4 else "s8", M, K, N, G, list(sizes)))
+        if s4:
+            w = workloads.ragged_s4_group_experts(M=M, K=K, N=N, groups=G, group=128, sizes=sizes)
+            ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                            bias=w["bias"], group=128)
+            wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                        np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+            floor = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+        else:
+            w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+            ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+            floor = ragged_floor(w)
+        got, kern = run_ragged(w)
+        kernels.add("tiled" if "tiled" in kern else "decode")
+        check_dot(got, ref, floor, "ragged #%d %s" % (case, kern))
+    assert kernels == {"tiled", "decode"}, kernels
