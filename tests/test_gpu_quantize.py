@@ -119,15 +119,21 @@ def test_quantize_empty_and_errors():
         ops.rowwise_quantize_fp8(torch.zeros((1, (1 << 20) + 8), dtype=torch.bfloat16, device="cuda"), None)
 
 
-@pytest.mark.parametrize("rows,cols,kernel", [(9, 28672, "long"), (3, 16392, "long"), (2, 65536, "long"),
-                                              (4, 20001, "long_unaligned"), (1, 1 << 20, "long")])
-def test_rmsnorm_quantize_long_rows(oracle, rows, cols, kernel):
-    """Rows past 16384 elements (an FFN activation of 28672, a vocabulary-sized row): the kernel that
-    walks the row three times instead of holding it in registers; same codes and scales, bit for bit,
-    windows of 32 and the levels above them in the oracle's order."""
-    say("quantize rmsnorm long rows=%d cols=%d" % (rows, cols))
+@pytest.mark.parametrize("rows,cols,variant,kernel", [
+    (9, 28672, 0, "lds_row"), (3, 16392, 0, "lds_row"), (2, 65536, 0, "lds_row"), (5, 40008, 0, "lds_row"),
+    (9, 28672, 1, "long"), (2, 65544, 0, "long"), (4, 20001, 0, "long_unaligned"), (1, 1 << 20, 0, "long")])
+def test_rmsnorm_quantize_long_rows(oracle, rows, cols, variant, kernel):
+    """Rows past 16384 elements (an FFN activation of 28672, a vocabulary-sized row): up to 65536
+    aligned elements the row is held in LDS by one workgroup, beyond that (and for unaligned rows) a
+    kernel walks the row three times through L2; same codes and scales, bit for bit, windows of 32
+    and the levels above them in the oracle's order."""
+    say("quantize rmsnorm long rows=%d cols=%d variant=%d" % (rows, cols, variant))
     w = workloads.c4_quantize(rows, cols)
-    q, s = run(w["x"], w["gamma"])
+    ffi.set_option("quantize_variant", variant)
+    try:
+        q, s = run(w["x"], w["gamma"])
+    finally:
+        ffi.set_option("quantize_variant", 0)
     assert ffi.last_kernel() == "rowwise_quantize_fp8:" + kernel, ffi.last_kernel()
     q_ref, s_ref = oracle.rmsnorm_quantize_fp8(w["x"], w["gamma"], eps=1e-6)
     assert np.array_equal(s.view(np.uint32), s_ref.view(np.uint32))
@@ -147,7 +153,7 @@ def test_quantize_long_special_rows(oracle):
     base[4, 12345] = np.nan
     x = dtypes.f32_to_bf16(base)
     q, s = run(x, None)
-    assert ffi.last_kernel() == "rowwise_quantize_fp8:long", ffi.last_kernel()
+    assert ffi.last_kernel() == "rowwise_quantize_fp8:lds_row", ffi.last_kernel()
     xf = dtypes.bf16_to_f32(x)
     amax = np.abs(xf[:4]).max(axis=1)
     s_ref = (amax / np.float32(448)).astype(np.float32)

@@ -558,6 +558,147 @@ __global__ __launch_bounds__(kThreads) void rowwise_quantize_long_kernel(
   }
 }
 
+// Aligned rows of 16385 to 65536 elements: one workgroup of 1024 lanes per row, the row held in LDS
+// (up to 128 KiB) instead of in registers, so x still crosses HBM once.  First the row is copied in
+// (16 bytes per lane, consecutive lanes consecutive chunks); then a lane per 32-element window adds
+// its squares left to right and the upper levels follow as above; then every chunk is replaced in
+// place by y (gamma comes from L2 once) while the maximum is taken; then the codes are made from y.
+constexpr int kLdsRowThreads = 1024;
+__global__ __launch_bounds__(kLdsRowThreads) void rowwise_quantize_lds_row_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma, uint8_t* __restrict__ q,
+    float* __restrict__ scales, int rows, int cols, float eps, int rmsnorm) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+  __shared__ uint32_t red[kLdsRowThreads / 64];
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x;
+  if (row >= rows) return;
+  const int chunks = cols >> 3;                       // cols % 8 == 0
+  const int padded = (chunks + 3) & ~3;               // whole 32-element windows; the padding holds zeros
+  uintx4* const rowv = reinterpret_cast<uintx4*>(lds_raw);
+  float* const lvl = reinterpret_cast<float*>(lds_raw + (size_t)padded * 16);
+  const uintx4* xr = reinterpret_cast<const uintx4*>(x + (size_t)row * cols);
+  uint8_t* qr = q + (size_t)row * cols;
+
+  for (int i = tid; i < padded; i += kLdsRowThreads) rowv[i] = i < chunks ? xr[i] : uintx4{0u, 0u, 0u, 0u};
+  __syncthreads();
+
+  auto unpack8 = [](const uintx4& w, float* out) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = bf16lo_to_f32(w[i]);
+      out[2 * i + 1] = bf16hi_to_f32(w[i]);
+    }
+  };
+
+  float rinv = 1.0f;
+  if (rmsnorm) {
+    const int n1 = padded >> 2;
+    // every level is padded with zeros to whole windows of 32, so a window is always eight 16-byte
+    // reads (adding the zeros changes nothing: the sums are not negative)
+    const int n1p = (n1 + 31) & ~31;
+    for (int w = n1 + tid; w < n1p; w += kLdsRowThreads) lvl[w] = 0.0f;
+    for (int w = tid; w < n1; w += kLdsRowThreads) {
+      uintx4 c4[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) c4[c] = rowv[w * 4 + c];
+      float acc = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float v[8];
+        unpack8(c4[c], v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = acc + v[i] * v[i];
+      }
+      lvl[w] = acc;
+    }
+    __syncthreads();
+    float* src = lvl;
+    int n = n1, np = n1p;
+    while (n > 1) {
+      const int m = (n + 31) / 32, mp = (m + 31) & ~31;
+      float* dst = src + np;
+      for (int w = tid; w < mp; w += kLdsRowThreads) {
+        float acc = 0.0f;
+        if (w < m) {
+          const floatx4* win = reinterpret_cast<const floatx4*>(src + w * 32);
+          floatx4 v[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] = win[i];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc = (((acc + v[i][0]) + v[i][1]) + v[i][2]) + v[i][3];
+        }
+        dst[w] = acc;
+      }
+      __syncthreads();
+      src = dst;
+      n = m;
+      np = mp;
+    }
+    const float ms = src[0] / (float)cols;
+    rinv = 1.0f / __builtin_sqrtf(ms + eps);
+  }
+
+  // y replaces x in place as packed bf16 pairs; the maximum is taken over the absolute bit patterns
+  // (every NaN pattern exceeds every number, which is XLA's NaN-propagating maximum)
+  typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+  u16x2 mx = {0, 0};
+  const uintx4* gv = reinterpret_cast<const uintx4*>(gamma);
+  for (int i = tid; i < chunks; i += kLdsRowThreads) {
+    uintx4 w = rowv[i];
+    if (rmsnorm) {
+      const uintx4 g = gv[i];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w[e] = pack_bf16x2((bf16lo_to_f32(w[e]) * rinv) * bf16lo_to_f32(g[e]), (bf16hi_to_f32(w[e]) * rinv) * bf16hi_to_f32(g[e]));
+      rowv[i] = w;  // the same lane reads this chunk again below: no barrier needed
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) mx = __builtin_elementwise_max(mx, __builtin_bit_cast(u16x2, w[e] & 0x7fff7fffu));
+  }
+  uint32_t m16 = mx[0] > mx[1] ? (uint32_t)mx[0] : (uint32_t)mx[1];
+  m16 = wave_max_u32(m16);
+  if ((tid & 63) == 0) red[tid >> 6] = m16;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kLdsRowThreads / 64; ++i) m16 = red[i] > m16 ? red[i] : m16;
+  const float amax = m16 > 0x7f80u ? bits_to_f32(0x7fc00000u) : bits_to_f32(m16 << 16);
+  const float s = amax / 448.0f;
+  if (tid == 0) scales[row] = s;
+  const bool fast = ordinary_divisor(s);
+  const float rs = 1.0f / s;
+
+  for (int i = tid; i < chunks; i += kLdsRowThreads) {
+    const uintx4 w = rowv[i];
+    uint32_t out[2];
+    if (fast) {  // no clamp needed and the zero's sign restored, as in the kernel above
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t pa = w[2 * h], pb = w[2 * h + 1];
+        const float y[4] = {bf16lo_to_f32(pa), bf16hi_to_f32(pa), bf16lo_to_f32(pb), bf16hi_to_f32(pb)};
+        float d[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float q0 = y[e] * rs;
+          d[e] = __builtin_fmaf(__builtin_fmaf(-q0, s, y[e]), rs, q0);
+        }
+        const uint32_t codes = pack_f8x4(d[0], d[1], d[2], d[3]);
+        const uint32_t signs = __builtin_amdgcn_perm(pb, pa, 0x07050301u);  // high bytes of the four bf16
+        out[h] = (codes & 0x7f7f7f7fu) | (signs & 0x80808080u);
+      }
+    } else {
+      out[0] = out[1] = 0u;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t v = w[e >> 1];
+        float t = ((e & 1) ? bf16hi_to_f32(v) : bf16lo_to_f32(v)) / s;
+        if (t == t) t = __builtin_fminf(__builtin_fmaxf(t, -448.0f), 448.0f);
+        out[e >> 2] |= f32_to_f8e4m3fn_any(t) << (8 * (e & 3));
+      }
+    }
+    __builtin_nontemporal_store(uintx2{out[0], out[1]}, reinterpret_cast<uintx2*>(qr + (size_t)i * 8));
+  }
+}
+
 template <int CH, int G, bool VEC>
 void launch_variant(const XlaAmdRowwiseQuantize& p, hipStream_t stream) {
   hipLaunchKernelGGL((rowwise_quantize_kernel<CH, G, VEC>), dim3((unsigned)p.rows), dim3(kThreads),
@@ -584,6 +725,20 @@ int LaunchRowwiseQuantize(const XlaAmdRowwiseQuantize& p, hipStream_t stream, in
       return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED,
                   "rowwise_quantize_fp8: rows longer than 1048576 elements are not supported");
     const int64_t n1 = (p.cols + 31) / 32;
+    if (vec && p.cols <= 65536 && variant == 0) {
+      // the row (padded to whole windows) and two levels of window sums
+      // the row (padded to whole windows) and the levels of window sums, each padded to whole windows
+      const size_t lds_row = (size_t)n1 * 64 + (size_t)(((n1 + 31) & ~31) + 160) * sizeof(float);
+      hipError_t e = hipFuncSetAttribute((const void*)rowwise_quantize_lds_row_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+      if (e != hipSuccess)
+        return Fail(XLA_FFI_Error_Code_INTERNAL, "rowwise_quantize_fp8: cannot reserve LDS: %s", hipGetErrorString(e));
+      hipLaunchKernelGGL(rowwise_quantize_lds_row_kernel, dim3((unsigned)p.rows), dim3(kLdsRowThreads), lds_row, stream,
+                         (const uint16_t*)p.x, (const uint16_t*)p.gamma, (uint8_t*)p.q, p.scales, (int)p.rows,
+                         (int)p.cols, p.eps, p.rmsnorm);
+      SetLastKernel("rowwise_quantize_fp8:lds_row");
+      return CheckLaunch("rowwise_quantize_fp8");
+    }
     const size_t lds = p.rmsnorm ? (size_t)(n1 + (n1 + 31) / 32) * sizeof(float) : 0;
     const void* fn = vec ? (const void*)rowwise_quantize_long_kernel<true> : (const void*)rowwise_quantize_long_kernel<false>;
     if (lds > 48 * 1024) {
