@@ -817,3 +817,37 @@ def test_ragged_dot_grouped_gemm(oracle, kind, M, K, N, G, sizes):
     check_dot(chunks, ref, floor, "ragged chunks %s" % kind)
     owned = int(min(M, np.sum(np.clip(w["group_sizes"], 0, None))))
     assert np.array_equal(got[owned:], np.broadcast_to(w["bias"], (M - owned, N)))
+
+
+@pytest.mark.parametrize("bits,M,K,N,group,scale_ty,epilogue", [
+    (8, 5, 1024, 256, 128, "f32", "BIAS_GELU"), (8, 24, 512, 128, 32, "bf16", "DEFAULT"), (8, 40, 2048, 512, 64, "f32", "BIAS"),
+    (8, 64, 1024, 256, 256, "f32", "SILU"), (4, 8, 2048, 512, 128, "f32", "BIAS_SILU"), (4, 30, 1024, 256, 64, "bf16", "RELU"),
+    (8, 200, 512, 128, 64, "f32", "DEFAULT")])
+def test_group_scales_under_f32_multiply(oracle, bits, M, K, N, group, scale_ty, epilogue):
+    """convert(w) * scale[K/g,N] f32-typed: every product is an f32 in the reference; the kernel adds a
+    group's integers exactly and multiplies the group's sum by its scale (2^-24 per term apart, inside
+    the floor that summation order already needs).  s8 and s4, f32 and bf16 scales, up to 64 tokens
+    per launch (200 tokens: 64-token chunks)."""
+    say("dequant_dot group scales, f32 multiply: s%d M=%d K=%d N=%d group=%d %s %s" % (bits, M, K, N, group, scale_ty, epilogue))
+    rng = np.random.default_rng(100 + M)
+    sc = rng.uniform(1e-3, 2e-2, size=(K // group, N)).astype(np.float32)
+    w = dict(lhs=dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)),
+             weights=rng.integers(-8 if bits == 4 else -127, 8 if bits == 4 else 128, size=(K, N)).astype(np.int8),
+             scales=dtypes.f32_to_bf16(sc) if scale_ty == "bf16" else sc,
+             bias=dtypes.f32_to_bf16(rng.standard_normal(N).astype(np.float32)) if "BIAS" in epilogue else None,
+             weight_dtype="s%d" % bits, weight_shape=(K, N), group=group, dequant_type="f32", epilogue=epilogue)
+    got, kern = run_dot(w)
+    assert "_group_factored" in kern, kern
+    compare(oracle, w, got, "group-factored %s" % kern)
+    generic, kern2 = run_dot(w, force_kernel=1)   # one thread per output, every product rounded to f32
+    assert kern2 == "dequant_dot_generic", kern2
+    compare(oracle, w, generic, "generic")
+
+
+def test_u4_zero_points_group_scales_under_f32_multiply(oracle):
+    say("dequant_dot u4 + zero points, group scales, f32 multiply")
+    w = workloads.u4_zero_point_group(M=12, K=1024, N=256, group=128)
+    w = dict(w, dequant_type="f32")
+    got, kern = run_dot(w)
+    assert kern == "dequant_dot_decode_s4_v4_m16_group_factored", kern
+    compare(oracle, w, got, "u4 group-factored")

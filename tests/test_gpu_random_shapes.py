@@ -39,8 +39,8 @@ def test_dequant_dot_random_shapes(oracle):
             N += 1
         epilogue = EPILOGUES[int(rng.integers(0, 8))]
         typed = "bf16" if rng.integers(0, 2) else "f32"
-        if typed == "f32" and not per_channel:
-            typed = "bf16"          # grouped scales under an f32 multiply go to the generic kernel only
+        # (grouped scales under an f32 multiply: group-factored sums when the group is whole 32-row steps
+        # and the shape fits, the one-thread-per-output kernel otherwise)
         say("dequant_dot #%d s%d M=%d K=%d N=%d group=%d %s %s" % (case, bits, M, K, N, group, epilogue, typed))
         lhs = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
         wq = rng.integers(-8 if bits == 4 else -127, 8 if bits == 4 else 128, size=(K, N)).astype(np.int8)

@@ -12,7 +12,7 @@
 
 namespace xla_amd {
 
-enum : int { kRounded = 0, kFactored = 1 };
+enum : int { kRounded = 0, kFactored = 1, kGroupFactored = 2 };
 
 struct DecodeParams {
   const uint16_t* lhs;   // [batch, M, K]

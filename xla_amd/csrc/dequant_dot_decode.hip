@@ -26,6 +26,13 @@
 //  * kFactored: the multiply is f32-typed and the scale is constant along K
 //    (per output channel).  Integers go through the MFMA exactly and the scale
 //    multiplies the f32 sum once.
+//  * kGroupFactored: the multiply is f32-typed and the scales change every `group` rows of K
+//    (a multiple of 32).  The integers of one group go through the MFMA exactly into a sum of
+//    their own, which is folded into the result as sum * scale at the group's last step.  The
+//    reference rounds every product w * s to f32 before it adds; factoring the scale out moves
+//    each term by at most 2^-24 of itself, the size of the summation-order differences the
+//    comparison rule already carries (the bf16-typed multiply rounds to 2^-9 and is never
+//    factored).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -133,6 +140,26 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   for (int j = 0; j < NV; ++j)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // kGroupFactored: acc holds the current group's sum of integers, tot the scaled sums so far; the
+  // scales are wanted in the accumulators' layout (register t of instruction j in lane (li, kb) is
+  // channel (4 * kb + t) * NV + j of the strip): four runs of NV consecutive channels per lane
+  constexpr bool GF = MODE == kGroupFactored;
+  static_assert(!GF || GROUP32, "group-factored sums need whole steps per group");
+  constexpr int SWG = NV * SSZ / 4;
+  floatx4 tot[GF ? NV : 1][GF ? MT : 1];
+  uint32_t graw[GF ? 4 : 1][GF ? SWG : 1];
+  uint32_t voff_g[4];
+  if (GF) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) tot[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int n = strip * TN + (4 * kb + t) * NV;
+      voff_g[t] = n < p.N ? (uint32_t)n * SSZ : kNowhere;   // N % NV == 0: a run is inside N or not at all
+    }
+  }
 
   // the slice is cut into four blocks, one per SIMD; inside a block the age classes follow each other
   const int cls = wave >> 2;
@@ -158,6 +185,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   const int steps_per_group = GROUP32 ? p.group / 32 : 1;
   auto opens_group = [&](int k0) {  // scalar
     return !GROUP32 || k0 == k_begin || ((k0 >> 5) % steps_per_group) == 0;
+  };
+  auto closes_group = [&](int k0) {  // scalar: the next step opens a group, or there is no next step
+    return k0 + 32 >= k_stop || (((k0 >> 5) + 1) % steps_per_group) == 0;
   };
   auto load_step = [&](int buf, int k0) {
     const uint32_t va = voff_a + (uint32_t)k0 * 2u;
@@ -196,6 +226,12 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) bop[mt] = __builtin_bit_cast(bf16x8, av[mt]);
+    if (GF && opens_group(k0)) {  // the group's scales: wanted at its last step, four steps of latency to hide in
+      asm volatile("");
+      const uint32_t g = (uint32_t)min(k0, p.K - 1) / (uint32_t)p.group;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) buffer_load_words<SWG>(rs, voff_g[t], g * (uint32_t)p.N * SSZ, graw[t]);
+    }
     if ((MODE == kRounded || (WBITS == 4 && has_zp)) && opens_group(k0)) {
       asm volatile("");  // a branch, not 2*NV selects per step
 #pragma unroll
@@ -278,6 +314,21 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
         }
       }
     }
+    if (GF && closes_group(k0)) {
+      asm volatile("");
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const float sv = SCALE_BF16 ? ((j & 1) ? bf16hi_to_f32(graw[t][j / 2]) : bf16lo_to_f32(graw[t][j / 2]))
+                                      : bits_to_f32(graw[t][SCALE_BF16 ? 0 : j]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            tot[j][mt][t] = __builtin_fmaf(acc[j][mt][t], sv, tot[j][mt][t]);
+            acc[j][mt][t] = 0.0f;
+          }
+        }
+    }
   };
 
   if (k_begin < p.K) {
@@ -320,7 +371,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     for (int c = 0; c < kChunk; ++c) {
       const int r = pass * kChunk + c;
       const int j = r % NV, mt = (r / NV) / 4, t = (r / NV) % 4;
-      float v = acc[j][mt][t];
+      float v = GF ? tot[j][mt][t] : acc[j][mt][t];
       lds[(wave * kChunk + c) * 64 + lane] = v;
     }
     __syncthreads();
@@ -433,6 +484,9 @@ int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const c
   const bool g32 = dp.group % 32 == 0;
   if constexpr (MODE == kFactored)  // the main loop never touches the scales
     kern = dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, true>;
+  else if constexpr (MODE == kGroupFactored)  // groups of whole steps only
+    kern = dp.scale_is_bf16 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, true>
+                            : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, true>;
   else if (dp.scale_is_bf16)
     kern = g32 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, true>
                : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, true, false>;
@@ -609,13 +663,17 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.ragged_chunks = ragged && p.M > 64 ? (int)((p.M + 63) / 64) : 1;
   if (ragged && (p.M + 63) / 64 > 65535)
     return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes at most 4194240 rows");
-  const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded : kFactored;
   const bool per_channel = p.group == p.K;
+  // f32-typed multiply: one scale per channel factors out of the whole sum, scales per group of whole
+  // 32-row steps out of each group's sum; anything else under an f32 multiply takes the generic kernel
+  const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded
+                   : per_channel || p.group % 32 != 0     ? kFactored
+                                                          : kGroupFactored;
 
   const int force = GetOption("dequant_dot_kernel");  // 0 auto, 1 generic, 2 decode, 3 prefill
   const bool aligned = p.K % 8 == 0 && p.group % 8 == 0 && ((uintptr_t)p.lhs % 16 == 0) &&
                        ((uintptr_t)p.weights % 16 == 0);
-  const bool mode_ok = mode == kRounded || per_channel;
+  const bool mode_ok = mode == kRounded || mode == kGroupFactored || per_channel;
 
   // A ragged dot takes the tiled kernel (a grouped GEMM: 256-row tiles per group) once the groups
   // average 96 rows; below that most tiles would be nearly empty and the 64-row chunks of the decode
@@ -650,8 +708,9 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // in a call of its own, so the chunks compose bit for bit; each pass streams the weights again,
   // which at 8192 x 28672 s4 still reaches 0.55 PFLOP/s against 2-3 TFLOP/s of the generic kernel.
   int mt64, vec64, nv64;
+  // (4-bit weights with group-factored sums stop at 32 tokens: two sets of accumulators per tile)
   if (force != 1 && force != 3 && aligned && mode_ok && p.M > 64 && p.K >= 32 && p.N % 2 == 0 && !ragged &&
-      decode_shape(64, &mt64, &vec64, &nv64)) {
+      !(mode == kGroupFactored && s4) && decode_shape(64, &mt64, &vec64, &nv64)) {
     const size_t wbytes = (size_t)p.K * p.N * (s4 ? 1 : 2) / 2;
     const size_t ssz = p.scale_dtype == XLA_FFI_DataType_BF16 ? 2 : 4;
     const size_t sbytes = p.scale_batch == p.batch && p.batch > 1 ? (size_t)(p.K / p.group) * p.N * ssz : 0;
@@ -738,6 +797,12 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
       XLA_AMD_DECODE(4, 4, 2, kFactored, "dequant_dot_decode_s4_v4_m32_factored")
       XLA_AMD_DECODE(4, 4, 3, kFactored, "dequant_dot_decode_s4_v4_m48_factored")
       XLA_AMD_DECODE(4, 4, 4, kFactored, "dequant_dot_decode_s4_v4_m64_factored")
+      XLA_AMD_DECODE(4, 4, 1, kGroupFactored, "dequant_dot_decode_s4_v4_m16_group_factored")
+      XLA_AMD_DECODE(4, 4, 2, kGroupFactored, "dequant_dot_decode_s4_v4_m32_group_factored")
+      XLA_AMD_DECODE(8, 8, 1, kGroupFactored, "dequant_dot_decode_s8_v8_m16_group_factored")
+      XLA_AMD_DECODE(8, 8, 2, kGroupFactored, "dequant_dot_decode_s8_v8_m32_group_factored")
+      XLA_AMD_DECODE(8, 4, 3, kGroupFactored, "dequant_dot_decode_s8_v4_m48_group_factored")
+      XLA_AMD_DECODE(8, 4, 4, kGroupFactored, "dequant_dot_decode_s8_v4_m64_group_factored")
       XLA_AMD_DECODE(8, 16, 1, kRounded, "dequant_dot_decode_s8_v16_m16_rounded")
       XLA_AMD_DECODE(8, 8, 1, kRounded, "dequant_dot_decode_s8_v8_m16_rounded")
       XLA_AMD_DECODE(8, 8, 2, kRounded, "dequant_dot_decode_s8_v8_m32_rounded")
