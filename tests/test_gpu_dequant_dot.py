@@ -822,7 +822,7 @@ def test_ragged_dot_grouped_gemm(oracle, kind, M, K, N, G, sizes):
 @pytest.mark.parametrize("bits,M,K,N,group,scale_ty,epilogue", [
     (8, 5, 1024, 256, 128, "f32", "BIAS_GELU"), (8, 24, 512, 128, 32, "bf16", "DEFAULT"), (8, 40, 2048, 512, 64, "f32", "BIAS"),
     (8, 64, 1024, 256, 256, "f32", "SILU"), (4, 8, 2048, 512, 128, "f32", "BIAS_SILU"), (4, 30, 1024, 256, 64, "bf16", "RELU"),
-    (8, 200, 512, 128, 64, "f32", "DEFAULT")])
+    (8, 200, 512, 128, 64, "f32", "DEFAULT"), (4, 50, 1024, 256, 128, "f32", "BIAS"), (4, 100, 512, 128, 64, "bf16", "DEFAULT")])
 def test_group_scales_under_f32_multiply(oracle, bits, M, K, N, group, scale_ty, epilogue):
     """convert(w) * scale[K/g,N] f32-typed: every product is an f32 in the reference; the kernel adds a
     group's integers exactly and multiplies the group's sum by its scale (2^-24 per term apart, inside
@@ -838,6 +838,8 @@ def test_group_scales_under_f32_multiply(oracle, bits, M, K, N, group, scale_ty,
              weight_dtype="s%d" % bits, weight_shape=(K, N), group=group, dequant_type="f32", epilogue=epilogue)
     got, kern = run_dot(w)
     assert "_group_factored" in kern, kern
+    if bits == 4 and M > 32:   # two sets of accumulators per tile: 4-bit weights go 32 tokens at a time
+        assert kern.endswith(":x32"), kern
     compare(oracle, w, got, "group-factored %s" % kern)
     generic, kern2 = run_dot(w, force_kernel=1)   # one thread per output, every product rounded to f32
     assert kern2 == "dequant_dot_generic", kern2

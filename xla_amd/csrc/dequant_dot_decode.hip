@@ -708,9 +708,10 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // in a call of its own, so the chunks compose bit for bit; each pass streams the weights again,
   // which at 8192 x 28672 s4 still reaches 0.55 PFLOP/s against 2-3 TFLOP/s of the generic kernel.
   int mt64, vec64, nv64;
-  // (4-bit weights with group-factored sums stop at 32 tokens: two sets of accumulators per tile)
-  if (force != 1 && force != 3 && aligned && mode_ok && p.M > 64 && p.K >= 32 && p.N % 2 == 0 && !ragged &&
-      !(mode == kGroupFactored && s4) && decode_shape(64, &mt64, &vec64, &nv64)) {
+  // (4-bit weights with group-factored sums hold two sets of accumulators per tile: chunks of 32 tokens)
+  const int64_t chunk = mode == kGroupFactored && s4 ? 32 : 64;
+  if (force != 1 && force != 3 && aligned && mode_ok && p.M > chunk && p.K >= 32 && p.N % 2 == 0 && !ragged &&
+      decode_shape(chunk, &mt64, &vec64, &nv64)) {
     const size_t wbytes = (size_t)p.K * p.N * (s4 ? 1 : 2) / 2;
     const size_t ssz = p.scale_dtype == XLA_FFI_DataType_BF16 ? 2 : 4;
     const size_t sbytes = p.scale_batch == p.batch && p.batch > 1 ? (size_t)(p.K / p.group) * p.N * ssz : 0;
@@ -725,24 +726,24 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
         sub.zero_points = (const char*)p.zero_points + (sbytes ? b * ((size_t)(p.K / p.group) * p.N / 2) : 0);
       // the whole 64-token chunks go out as one launch with the chunk index in the grid (the
       // workgroups of all chunks then pack onto the CUs together), the remainder as a second one
-      const int64_t whole = p.M / 64;
+      const int64_t whole = p.M / chunk;
       for (int part = 0; part < 2; ++part) {
-        const int64_t m0 = part == 0 ? 0 : whole * 64;
-        sub.M = part == 0 ? 64 : p.M - m0;
+        const int64_t m0 = part == 0 ? 0 : whole * chunk;
+        sub.M = part == 0 ? chunk : p.M - m0;
         sub.batch = part == 0 ? whole : 1;
         if (sub.M == 0 || sub.batch == 0) continue;
         sub.lhs = (const uint16_t*)p.lhs + ((size_t)b * p.M + m0) * p.K;
         sub.out = (uint16_t*)p.out + ((size_t)b * p.M + m0) * p.N;
         const int rc = LaunchDequantDotImpl(sub, stream, true);
         if (rc) return rc;
-        if (!name[0]) snprintf(name, sizeof(name), "%s:x64", xla_amd_last_kernel());
+        if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)chunk);
       }
     }
     SetLastKernel(name);
     return 0;
   }
 
-  if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= 64 || ragged) && p.K >= 32) {
+  if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= chunk || ragged) && p.K >= 32) {
     int mt, vec, nv;
     const bool shape_ok = decode_shape(p.M > 64 ? 64 : p.M, &mt, &vec, &nv);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
