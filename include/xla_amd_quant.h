@@ -215,6 +215,14 @@ XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, vo
 XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                                              int32_t rhs_contracting_dim);
 
+/* The same for a call whose dequantise multiply has the given type (XLA_FFI_DataType): under a BF16
+ * multiply every a * a_scale and b * b_scale is rounded to bf16, and unless both scales turn out to
+ * be powers of two the call runs on the bf16 matrix cores from operands a pre-pass writes into the
+ * scratch ((M + N) * K * 2 bytes more); without that scratch it runs on the slow exact kernel. */
+XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes_typed(int64_t M, int64_t K, int64_t N,
+                                                                   int32_t rhs_contracting_dim,
+                                                                   int32_t dequant_type);
+
 typedef struct XlaAmdRowwiseQuantize {
   const void* x;     /* bf16 [rows, cols] */
   const void* gamma; /* bf16 [cols] or NULL when rmsnorm == 0 */

@@ -111,11 +111,15 @@ def test_vector_scales(oracle, which, nk):
     assert kern.startswith("fp8_scaled_dot_tiled"), kern
     n_floor = check_dot(got, reference(oracle, w), floor_for(w), kern)
     assert n_floor <= got.size // 100
-    # the slow kernel takes the same vectors (and is the one a bf16-typed multiply gets)
+    # the slow kernel takes the same vectors
     got, kern = run(w, nk=nk, force=1)
     assert kern == "fp8_scaled_dot_exact", kern
     check_dot(got, reference(oracle, w), floor_for(w, exact_kernel=True), kern)
+    # a bf16-typed multiply rounds every scaled operand: the bf16-operand kernel (the exact one without scratch)
     got, kern = run(w, nk=nk, dequant_type="bf16")
+    assert kern == "fp8_scaled_dot_bf16_operands", kern
+    check_dot(got, reference(oracle, w, dequant_type="bf16"), floor_for(w, exact_kernel=True), kern)
+    got, kern = run(w, nk=nk, dequant_type="bf16", scratch=None)
     assert kern == "fp8_scaled_dot_exact", kern
     check_dot(got, reference(oracle, w, dequant_type="bf16"), floor_for(w, exact_kernel=True), kern)
 
@@ -382,14 +386,62 @@ def test_reference_pattern_bf16_typed_ops(oracle):
     check_dot(got, ref, fl, kern)
 
 
-def test_non_power_of_two_scales_take_exact_kernel(oracle):
-    say("fp8_scaled_dot bf16-typed multiply with scale 0.3")
-    w = workloads.c3_fp8(64, 128, 64)
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 520, 272), (130, 264, 200)])
+def test_bf16_typed_multiply_with_any_scale(oracle, M, K, N, nk):
+    """bf16-typed dequantise multiply with scales that are no powers of two: every a * a_scale and
+    b * b_scale is rounded to bf16, so the f8 kernel (which scales the sum) does not serve the call;
+    a pre-pass writes the rounded operands as bf16 and the bf16 matrix cores multiply them.  bf16
+    products are exact in f32: only the order of the sum differs from the oracle (the strict floor).
+    With power-of-two scales the same launches leave the f8 kernel's result untouched."""
+    say("fp8_scaled_dot bf16-typed multiply, scales 0.3 / 0.013, M=%d K=%d N=%d nk=%s" % (M, K, N, nk))
+    w = workloads.c3_fp8(M, K, N)
     w["a_scale"] = np.float32(0.3)
-    w["b_scale"] = np.float32(1 / 64)
+    w["b_scale"] = np.float32(0.013)
+    types = dict(dequant_type="bf16")
+    got, kern = run(w, nk=nk, **types)
+    # K % 16 != 0 keeps the f8 kernel out altogether; otherwise both are enqueued and the scales decide
+    assert kern == ("fp8_scaled_dot_bf16_operands" if K % 16 else kern) and kern.endswith("bf16_operands"), kern
+    n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
+    assert n_floor <= max(8, got.size // 50)
+    exact, kern2 = run(w, nk=nk, force=1, **types)
+    assert kern2 == "fp8_scaled_dot_exact", kern2
+    check_dot(exact, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern2)
+    w2 = dict(w, a_scale=np.float32(1 / 64), b_scale=np.float32(1 / 32))
+    got2, kern3 = run(w2, nk=nk, **types)
+    assert kern3.endswith("bf16_operands"), kern3
+    if K % 16 == 0:
+        plain, _ = run(w2, nk=nk)   # f32-typed: the f8 kernel alone; identical values for power-of-two scales
+        assert np.array_equal(got2, plain)
+    else:
+        check_dot(got2, reference(oracle, w2, **types), floor_for(w2, exact_kernel=True), kern3)
+
+
+@pytest.mark.parametrize("which", ["a", "b", "ab"])
+def test_bf16_typed_multiply_with_vector_scales(oracle, which):
+    say("fp8_scaled_dot bf16-typed multiply, vector scales on %s" % which)
+    M, K, N = 200, 256, 136
+    w = workloads.c3_fp8(M, K, N)
+    rng = np.random.default_rng(8)
+    if "a" in which:
+        w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+    if "b" in which:
+        w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
     types = dict(dequant_type="bf16")
     got, kern = run(w, **types)
-    n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w), kern)
+    assert kern == "fp8_scaled_dot_bf16_operands", kern
+    n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
+    assert n_floor <= got.size // 50
+
+
+def test_bf16_typed_multiply_without_scratch_takes_exact_kernel(oracle):
+    say("fp8_scaled_dot bf16-typed multiply with scale 0.3, no scratch")
+    w = workloads.c3_fp8(64, 128, 64)
+    w["a_scale"] = np.float32(0.3)
+    types = dict(dequant_type="bf16")
+    got, kern = run(w, scratch=None, **types)
+    assert kern == "fp8_scaled_dot_tiled_kn", kern   # followed by the exact kernel, which runs for this scale
+    n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
     assert n_floor <= got.size // 100
 
 

@@ -87,6 +87,23 @@ def test_c3_module_vector_scales():
     check_dot(host_bf16(out), ref, dot_floor(fa, fb, K) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "C3 vector scales")
 
 
+def test_c3_module_vector_scales_under_a_bf16_multiply():
+    say("module C3, every op bf16-typed, per-row / per-channel scales")
+    M, K, N = 128, 256, 144
+    w = workloads.c3_fp8(M, K, N)
+    text = hm.c3_fp8(M, K, N, typed="bf16", vector_scales=True)
+    rng = np.random.default_rng(9)
+    sa = dtypes.f32_to_bf16(rng.uniform(0.004, 0.04, M).astype(np.float32))
+    sb = dtypes.f32_to_bf16(rng.uniform(0.004, 0.04, N).astype(np.float32))
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(w["a"]), dev_u8(w["b"]), dev_bf16(sa), dev_bf16(sb), dev_bf16(w["bias"])])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"]
+    ref = reference(text, [w["a"], w["b"], sa, sb, w["bias"]])
+    fa = np.abs(dtypes.f8e4m3fn_to_f32(w["a"]).astype(np.float64)) * dtypes.bf16_to_f32(sa).astype(np.float64)[:, None]
+    fb = np.abs(dtypes.f8e4m3fn_to_f32(w["b"]).astype(np.float64)) * dtypes.bf16_to_f32(sb).astype(np.float64)[None, :]
+    check_dot(host_bf16(out), ref, dot_floor(fa, fb, K), "C3 bf16-typed vector scales")
+
+
 def test_c3_module_f8_result(oracle):
     say("module C3 with an f8 result")
     M, K, N = 128, 256, 144

@@ -109,9 +109,13 @@ def test_c3_fp8_bias_gelu(typed, code):
     check(new, r"custom-call\(%a, %b, %a_scale\S*, %b_scale\S*, %bias\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
           r'epilogue = \\"BIAS_GELU\\", dequant_type = %d : i32, dot_type = %d : i32, epilogue_type = %d : i32, '
           r'rhs_contracting_dim = 0 : i64' % (code, code, code))
-    assert "s8[" not in new                    # N % 16 == 0: the [K,N] rhs goes in as it is, no scratch
     ragged_n = hlo.rewrite(hm.c3_fp8(512, 4096, 1000, typed=typed))[0]
-    assert "s8[4096000]{0}" in ragged_n        # K*N bytes to re-lay a [K,N] rhs out with K minor when N % 16 != 0
+    if typed == "f32":
+        assert "s8[" not in new                # N % 16 == 0: the [K,N] rhs goes in as it is, no scratch
+        assert "s8[4096000]{0}" in ragged_n    # K*N bytes to re-lay a [K,N] rhs out with K minor when N % 16 != 0
+    else:   # a bf16-typed multiply: room for both operands as bf16, (M + N) * K * 2 bytes, behind the copy
+        assert "s8[%d]{0}" % (2 * 8192 * 8192 * 2) in new
+        assert "s8[%d]{0}" % (4096000 + (512 + 1000) * 4096 * 2) in ragged_n
     if typed == "bf16":                        # bf16 scalars are widened, as GemmRewriter does
         check(new, r"%a_scale.f32 = f32\[\] convert\(%a_scale\)", r"%b_scale.f32 = f32\[\] convert\(%b_scale\)")
 
@@ -294,7 +298,7 @@ def test_fp8_divide_by_scale_and_rhs_contracting_minor():
     new, rw, rf = hlo.rewrite(text)
     assert rw == ["out -> xla_amd.fp8_scaled_dot [DEFAULT]"], (rw, rf)
     check(new, r"%\S+ = f32\[\] divide\(%one\S*, %\S+\)", r"rhs_contracting_dim = 1 : i64")
-    assert "s8[" not in new                      # K-minor rhs needs no scratch
+    assert "s8[2048]{0}" in new                  # K-minor rhs needs no copy; bf16-typed multiply: both operands as bf16
 
 
 def test_unscaled_fp8_dot_gets_unit_scales():
@@ -544,3 +548,14 @@ def test_grouped_scales_behind_a_batch_or_expert_dimension():
     # scales of another expert count are not this pattern
     bad = text.replace("%scales = bf16[4,4,64] parameter(2)", "%scales = bf16[2,4,64] parameter(2)")
     assert hlo.rewrite(bad)[1] == []
+
+
+def test_c3_fp8_vector_scales_under_a_bf16_multiply():
+    """Per-row / per-channel scales with every op bf16-typed: taken (the rounded operands go to the bf16
+    matrix cores); the bf16 vectors are widened to the f32 the handler reads, and the scratch holds both
+    operands as bf16."""
+    new, rw, rf = hlo.rewrite(hm.c3_fp8(64, 128, 32, typed="bf16", vector_scales=True))
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU]"] and rf == []
+    check(new, r"%a_scale.f32 = f32\[64\]\{0\} convert\(%a_scale\)", r"%b_scale.f32 = f32\[32\]\{0\} convert\(%b_scale\)",
+          r"s8\[%d\]\{0\}\) custom-call\(%%a, %%b, %%a_scale.f32, %%b_scale.f32, %%bias\)" % ((64 + 32) * 128 * 2),
+          r"dequant_type = 16 : i32")

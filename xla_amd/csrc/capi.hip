@@ -51,7 +51,7 @@ int GetOption(const char* key) {
 }
 
 size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4);
-size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim);
+size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contracting_dim, int dequant_type);
 size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N);
 
 }  // namespace xla_amd
@@ -89,8 +89,12 @@ size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, 
 
 size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                               int32_t rhs_contracting_dim) {
-  (void)M;
-  return xla_amd::Fp8ScaledDotWorkspaceBytes(K, N, rhs_contracting_dim);
+  return xla_amd::Fp8ScaledDotWorkspaceBytes(M, K, N, rhs_contracting_dim, XLA_FFI_DataType_F32);
+}
+
+size_t xla_amd_fp8_scaled_dot_workspace_bytes_typed(int64_t M, int64_t K, int64_t N, int32_t rhs_contracting_dim,
+                                                    int32_t dequant_type) {
+  return xla_amd::Fp8ScaledDotWorkspaceBytes(M, K, N, rhs_contracting_dim, dequant_type);
 }
 
 const char* xla_amd_last_error(void) { return xla_amd::g_error; }

@@ -42,7 +42,7 @@ std::string ShapeJson(const xla_amd::hlo::Shape& s) {
 
 struct XlaAmdRewriteCallbacks {
   size_t (*dequant_workspace_bytes)(int64_t, int64_t, int64_t, int64_t, int32_t);
-  size_t (*fp8_workspace_bytes)(int64_t, int64_t, int64_t, int32_t);
+  size_t (*fp8_workspace_bytes)(int64_t, int64_t, int64_t, int32_t, int32_t);
 };
 
 // Returns the rewritten module text (malloc'd; free with xla_amd_host_free), or NULL with the

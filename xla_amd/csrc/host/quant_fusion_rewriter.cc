@@ -419,8 +419,6 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
   // of b): along K it does not factor out of the sum
   if (a.scale_dim == 1) return refuse("the lhs scales vary along the contracting dimension");
   if (b.scale_dim == rc[0]) return refuse("the rhs scales vary along the contracting dimension");
-  if ((a.scale_dim >= 0 || b.scale_dim >= 0) && a.type != "f32")
-    return refuse("per-row / per-channel scales are taken with an f32 multiply only");
   if ((a.scale_dim >= 0 && a.divide) || (b.scale_dim >= 0 && b.divide))
     return refuse("a division by a vector of scales is not taken");
   auto scale_of = [&](const F8Operand& o) -> Instr* {
@@ -449,7 +447,7 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
   if (ep.d_scale) ops.push_back(ep.d_scale);
   std::vector<Shape> results = {Shape::Array(ep.d_scale ? "f8e4m3fn" : "bf16", out_dims)};
   if (ep.amax) results.push_back(Shape::Array("f32", {}));
-  size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0]) : 0;
+  size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, (int32_t)rc[0], DTypeCode(a.type)) : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
   std::string cfg = CommonConfig(ep, a.type, dot->shape.dtype) + ", rhs_contracting_dim = " +
                     std::to_string(rc[0]) + " : i64";

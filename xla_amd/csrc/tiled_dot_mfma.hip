@@ -39,7 +39,9 @@ namespace {
 
 // kFp8KN: fp8 with the weights given [K,N]; kFp8MX: fp8 [M,K] x [N,K] with one f8e8m0fnu scale per
 // 32 elements of K on both operands (MXFP8), multiplied in by the matrix cores themselves
-enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4 };
+// kBf16: both operands bf16 with K minor, a [M,K] and b [N,K] -- the f8 operands of a dot whose
+// dequantise multiply is bf16-typed, already scaled and rounded by a pre-pass
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4, kBf16 = 5 };
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
@@ -66,6 +68,7 @@ struct TiledParams {
   const uint8_t* a_block_scales;  // kFp8MX: f8e8m0fnu [M, K/32]
   const uint8_t* b_block_scales;  // kFp8MX: f8e8m0fnu [N, K/32]
   int closed_form_epilogue;       // option "tiled_epilogue" = 1
+  int skip_if_pow2_scales;        // kBf16: both scales powers of two -> the f8 kernel has done the call, return
   // Integer-weight kinds: the tiles of the last, at most half-full round of 256 are each split over
   // two workgroups along K (grid: tail_first whole tiles, then tail_tiles second halves, then
   // tail_tiles first halves; one dimension, batches flattened).  A second half leaves its f32
@@ -230,17 +233,21 @@ __device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, 
 template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr bool WQ = KIND == kS8 || KIND == kS4;  // integer weights [K,N], dequantised on the way into LDS
-  constexpr bool F8 = !WQ;               // both operands f8e4m3fn
+  constexpr bool BB = KIND == kBf16;     // both operands bf16, K minor
+  constexpr bool F8 = !WQ && !BB;        // both operands f8e4m3fn
   constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
   constexpr bool MX = KIND == kFp8MX;    // block scales ride along with every stage
-  constexpr bool BNK = KIND == kFp8 || MX;  // f8 weights [N,K]: staged like the activations
+  constexpr bool BNK = KIND == kFp8 || MX || BB;  // weights [N,K]: staged like the activations
   constexpr int ESZ = F8 ? 1 : 2;  // bytes per activation element
   constexpr int KS = kRow / ESZ;             // K elements per stage
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [2][(kTM + kTN) * kRow]
   constexpr int kBufBytes = (kTM + kTN) * kRow;
 
   if (F8 && !MX && p.require_pow2_scales) {
-    if (!(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;  // the exact kernel runs
+    if (!(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;  // the bf16-operand (or the exact) kernel runs
+  }
+  if (BB && p.skip_if_pow2_scales) {
+    if (is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;
   }
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -318,7 +325,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const uint32_t a_pitch = (uint32_t)p.K * ESZ;
   const __amdgpu_buffer_rsrc_t ra =
       tile_rsrc(p.a + (size_t)a_batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
-  const uint32_t b_bytes = KIND == kS4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N;
+  const uint32_t b_bytes = KIND == kS4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N * (BB ? 2u : 1u);
   const __amdgpu_buffer_rsrc_t rb = tile_rsrc(p.b + (size_t)batch * b_bytes, b_bytes);  // bytes, either layout
 
   // kFp8MX: scales [rows, K/32]; lane l of wave w owns tile row (w & 3) * 64 + l of its operand
@@ -340,7 +347,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   for (int j = 0; j < 4; ++j) {
     const int r = wave * 32 + j * 8 + ld_row;
     voff_a[j] = (uint32_t)(m0 + r) * a_pitch + ld_chunk[j & 1] * 16;
-    if (BNK) voff_b[j] = (uint32_t)(n0 + r) * (uint32_t)p.K + ld_chunk[j & 1] * 16;
+    if (BNK) voff_b[j] = (uint32_t)(n0 + r) * a_pitch + ld_chunk[j & 1] * 16;  // K * ESZ bytes per row, as for a
     if (BKN) {
       // [K,N]: instruction j of this wave moves 4 rows of K x 256 channels; lane l fills slot l%16
       // of row l/16 with global chunk (l%16) ^ ((k & 7) << 1): eight consecutive rows then spread a
@@ -879,6 +886,41 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   }
 }
 
+// Pre-pass of the bf16-operand path: dst[r][c] = bf16(f32(src f8) * bf16(scale)), the dequantised operand
+// exactly as a bf16-typed multiply leaves it.  src is [rows, cols] (TRANSPOSE: [cols, rows], i.e. a [K,N]
+// rhs read so that dst is [N,K]); scale is one value or one per row of dst.  64 x 256 elements per
+// workgroup.  With skip_if_pow2 the call belongs to the f8 kernel when both scales are powers of two.
+template <bool TRANSPOSE>
+__global__ __launch_bounds__(256) void f8_to_scaled_bf16_kernel(const uint8_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                               int rows, int cols, const float* __restrict__ scale,
+                                                               int per_row, const float* __restrict__ other_scale,
+                                                               int skip_if_pow2) {
+  if (skip_if_pow2 && is_pow2_f32(*scale) && is_pow2_f32(*other_scale)) return;
+  __shared__ uint8_t tile[64][64 + 4];
+  const int r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int part = 0; part < 4; ++part) {   // four 64-column tiles per workgroup
+    const int c0 = (blockIdx.x * 4 + part) * 64;
+    if (c0 >= cols) break;
+    if (TRANSPOSE) {
+      // src row = c0 + i (a k of the rhs), src column = r0 + tx (a channel): read along the channels
+      for (int i = ty; i < 64; i += 4) {
+        const int c = c0 + i, r = r0 + tx;
+        tile[i][tx] = (c < cols && r < rows) ? src[(size_t)c * rows + r] : 0;
+      }
+      __syncthreads();
+    }
+    for (int i = ty; i < 64; i += 4) {
+      const int r = r0 + i, c = c0 + tx;
+      if (r >= rows || c >= cols) continue;
+      const uint8_t code = TRANSPOSE ? tile[tx][i] : src[(size_t)r * cols + c];
+      const float s = round_bf16(scale[per_row ? r : 0]);
+      dst[(size_t)r * cols + c] = f32_to_bf16(f8e4m3fn_to_f32(code) * s);
+    }
+    if (TRANSPOSE) __syncthreads();  // the tile is refilled by the next part
+  }
+}
+
 __global__ void store_u32_kernel(uint32_t* dst, uint32_t value) { *dst = value; }
 
 // Ragged dot: rows past the last group are a dot of nothing, epilogue(0).  Workgroup (x, y) takes 256
@@ -1014,9 +1056,27 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
 }
 
-// The transposed copy of a [K,N] rhs that cannot go in as it is: N no multiple of 16, or the pre-pass forced.
-size_t Fp8ScaledDotWorkspaceBytes(int64_t K, int64_t N, int rhs_contracting_dim) {
+namespace {
+size_t RoundUp256(size_t v) { return (v + 255) & ~(size_t)255; }
+// the transposed copy of a [K,N] rhs that cannot go in as it is: N no multiple of 16, or the pre-pass forced
+size_t TransposedCopyBytes(int64_t K, int64_t N, int rhs_contracting_dim) {
   return rhs_contracting_dim == 0 && (N % 16 != 0 || GetOption("fp8_dot_layout") == 1) ? (size_t)K * N : 0;
+}
+// both operands as bf16 with K minor (a dequantise multiply that is bf16-typed: see LaunchFp8ScaledDot);
+// 0 when the bf16-operand kernel does not take the shape
+size_t Bf16OperandBytes(int64_t M, int64_t K, int64_t N) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || (double)M * K * 2 >= 2147483000.0 || (double)N * K * 2 >= 2147483000.0)
+    return 0;
+  return RoundUp256((size_t)M * K * 2) + (size_t)N * K * 2;
+}
+}  // namespace
+
+// Scratch of an f8 scaled dot: [transposed copy of the rhs, if it needs one][a as bf16][b as bf16, K minor],
+// the last two only under a bf16-typed dequantise multiply.
+size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contracting_dim, int dequant_type) {
+  const size_t copy = TransposedCopyBytes(K, N, rhs_contracting_dim);
+  const size_t ops = dequant_type == XLA_FFI_DataType_BF16 ? Bf16OperandBytes(M, K, N) : 0;
+  return ops ? RoundUp256(copy) + ops : copy;
 }
 
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
@@ -1143,6 +1203,50 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
 
   const size_t eblocks = ((size_t)p.M * p.N + 255) / 256;
   dim3 egrid((unsigned)(eblocks < 8192 ? (eblocks ? eblocks : 1) : 8192), (unsigned)batch);
+
+  // A bf16-typed dequantise multiply rounds every a * a_scale and b * b_scale to bf16.  With scales
+  // that are powers of two that rounding changes nothing and the f8 kernel serves the call; otherwise
+  // the rounded operands are bf16 numbers, so a pre-pass writes them out (b with K minor) and the
+  // bf16 matrix cores multiply them -- decided on the device from the scale values, where both are
+  // single values; vectors of scales always go this way.  Without the scratch: the exact kernel.
+  const size_t ops_bytes = deq_bf16 && !mx && !out_f8 && batch == 1 && force != 1 ? Bf16OperandBytes(p.M, p.K, p.N) : 0;
+  const size_t ops_at = RoundUp256(TransposedCopyBytes(p.K, p.N, p.rhs_contracting_dim));
+  if (ops_bytes && p.workspace && ((uintptr_t)p.workspace % 256) == 0 && p.workspace_bytes >= ops_at + ops_bytes &&
+      ((uintptr_t)p.out % 8) == 0) {
+    int rc = 0;
+    const bool by_value = !vector_scales;  // the f8 kernel may serve the call: both decide from the scale values
+    if (by_value && tiled_ok) {
+      TiledParams tt = tp;
+      tt.b = b_nk;
+      rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn") : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
+      if (rc) return rc;
+    }
+    uint16_t* a16 = (uint16_t*)((char*)p.workspace + ops_at);
+    uint16_t* b16 = (uint16_t*)((char*)a16 + RoundUp256((size_t)p.M * p.K * 2));
+    const int skip = by_value && tiled_ok ? 1 : 0;
+    hipLaunchKernelGGL(f8_to_scaled_bf16_kernel<false>, dim3((unsigned)((p.K + 255) / 256), (unsigned)((p.M + 63) / 64)), dim3(256), 0,
+                       stream, (const uint8_t*)p.a, a16, (int)p.M, (int)p.K, p.a_scale, tp.a_per_row ? 1 : 0, p.b_scale, skip);
+    if (nk)
+      hipLaunchKernelGGL(f8_to_scaled_bf16_kernel<false>, dim3((unsigned)((p.K + 255) / 256), (unsigned)((p.N + 63) / 64)), dim3(256),
+                         0, stream, (const uint8_t*)p.b, b16, (int)p.N, (int)p.K, p.b_scale, tp.b_per_channel ? 1 : 0, p.a_scale, skip);
+    else
+      hipLaunchKernelGGL(f8_to_scaled_bf16_kernel<true>, dim3((unsigned)((p.K + 255) / 256), (unsigned)((p.N + 63) / 64)), dim3(256),
+                         0, stream, (const uint8_t*)p.b, b16, (int)p.N, (int)p.K, p.b_scale, tp.b_per_channel ? 1 : 0, p.a_scale, skip);
+    rc = CheckLaunch("fp8_scaled_dot_bf16_operands_prepass");
+    if (rc) return rc;
+    TiledParams tb = tp;
+    tb.a = (const uint8_t*)a16;
+    tb.b = (const uint8_t*)b16;
+    tb.require_pow2_scales = 0;
+    tb.skip_if_pow2_scales = skip;
+    tb.a_per_row = tb.b_per_channel = 0;  // already in the operands
+    rc = launch_tiled<kBf16>(tb, 1, stream, "fp8_scaled_dot_bf16_operands");
+    if (rc) return rc;
+    SetLastKernel(skip ? (kn_direct ? "fp8_scaled_dot_tiled_kn|bf16_operands" : nk ? "fp8_scaled_dot_tiled|bf16_operands"
+                                                                                    : "fp8_scaled_dot_tiled+transpose|bf16_operands")
+                       : "fp8_scaled_dot_bf16_operands");
+    return 0;
+  }
   if (tiled_ok) {
     TiledParams tt = tp;
     tt.b = b_nk;

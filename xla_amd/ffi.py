@@ -24,7 +24,8 @@ EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
     "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch",
     "xla_amd_launch_fp8_scaled_dot",
     "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
-    "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_last_error", "xla_amd_last_kernel",
+    "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_fp8_scaled_dot_workspace_bytes_typed", "xla_amd_last_error",
+    "xla_amd_last_kernel",
     "xla_amd_debug_set_option"]
 SELFCHECK_SYMBOLS = ["xla_amd_selfcheck_tanh_division_mismatches", "xla_amd_selfcheck_stream",
                      "xla_amd_selfcheck_launch_empty"]
@@ -274,6 +275,8 @@ def library():
             getattr(L, sym).argtypes = [C.POINTER(LaunchDequantDot), C.c_void_p]
         L.xla_amd_fp8_scaled_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_fp8_scaled_dot_workspace_bytes.argtypes = [C.c_int64] * 3 + [C.c_int32]
+        L.xla_amd_fp8_scaled_dot_workspace_bytes_typed.restype = C.c_size_t
+        L.xla_amd_fp8_scaled_dot_workspace_bytes_typed.argtypes = [C.c_int64] * 3 + [C.c_int32] * 2
         _lib = L
     return _lib
 

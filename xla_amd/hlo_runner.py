@@ -7,7 +7,7 @@ xla/backends/gpu/runtime/custom_call_thunk.cc:110-157).
 
 Only what a rewritten quantized-inference module contains is supported besides the custom
 calls: parameters, tuples, get-tuple-element, and scalar glue (constants, converts and
-divides of rank-0 values), which run as torch ops.  Anything else raises: this is not an HLO
+divides of rank-0 values, converts of rank-1 scale vectors), which run as torch ops.  Anything else raises: this is not an HLO
 interpreter, and a module the pass did not fully rewrite does not run here.
 """
 import re
@@ -88,8 +88,8 @@ class Executable:
                 v = x[0][int(ins["attrs"]["index"])]
             elif op == "tuple":
                 v = list(x)
-            elif not sh.get("tuple") and sh["dims"] == []:
-                v = self._scalar_glue(ins, x)
+            elif not sh.get("tuple") and (sh["dims"] == [] or (op == "convert" and len(sh["dims"]) == 1)):
+                v = self._scalar_glue(ins, x)   # scalars, and the widening convert of a vector of scales
             else:
                 raise NotImplementedError("instruction %s = %s(...) was not rewritten into a custom call; "
                                           "this runner only executes custom calls" % (ins["name"], op))

@@ -32,6 +32,7 @@ def cases():
         ("quant_fusion_rewriter_fp8_bias_gelu", hm.c3_fp8(64, 128, 32)),
         ("quant_fusion_rewriter_fp8_bf16_typed", hm.c3_fp8(64, 128, 32, typed="bf16")),
         ("quant_fusion_rewriter_fp8_vector_scales", hm.c3_fp8(64, 128, 32, vector_scales=True)),
+        ("quant_fusion_rewriter_fp8_bf16_typed_vector_scales", hm.c3_fp8(64, 128, 32, typed="bf16", vector_scales=True)),
         ("quant_fusion_rewriter_fp8_f8_result_amax", hm.c3_fp8_f8_result(64, 128, 32, amax=True)),
         ("quant_fusion_rewriter_rowwise_quantize_rmsnorm", hm.c4_quantize(8, 64)),
         ("quant_fusion_rewriter_rowwise_quantize_rsqrt", hm.c4_quantize(8, 64, rsqrt=True)),

@@ -131,7 +131,8 @@ def fp8_scaled_dot(a, b, a_scale, b_scale, bias=None, *, rhs_contracting_dim=0, 
         amax_t = torch.empty((), dtype=torch.float32, device=a.device)
         rets.append((dtypes.F32, amax_t.data_ptr(), []))
     if scratch == "auto":
-        nbytes = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(m, k, n, rhs_contracting_dim)
+        nbytes = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes_typed(
+            m, k, n, rhs_contracting_dim, dtypes.BF16 if dequant_type == "bf16" else dtypes.F32)
         scratch = _scratch(nbytes, a.device)
     if scratch is not None:
         rets.append((dtypes.U8, scratch.data_ptr(), [scratch.numel()]))
