@@ -150,6 +150,11 @@ typedef struct XlaAmdDequantDot {
    * are a dot of nothing (epilogue(0)).  Never read on the host. */
   const void* group_sizes;
   int32_t group_sizes_dtype;
+  /* 0: weights [batch,K,N] as above.  1: weights [batch,N,K], the contracting dimension minor
+   * (dot ... rhs_contracting_dims={1}, fusion_emitter_int4_device_test.cc:867-892): 4-bit values are
+   * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  Not with
+   * group_sizes. */
+  int32_t rhs_contracting_dim;
 } XlaAmdDequantDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);
@@ -161,6 +166,11 @@ XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* s
  * A call without (enough) scratch still works; it just cannot split K. */
 XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K,
                                                           int64_t N, int32_t weight_dtype);
+
+/* The same for weights [batch,N,K] (rhs_contracting_dim = 1): the f32 partial sums of the K-slices
+ * a call with few output channels is cut into. */
+XLA_AMD_EXPORT size_t xla_amd_dequant_dot_workspace_bytes_nk(int64_t batch, int64_t M, int64_t K,
+                                                             int64_t N, int32_t weight_dtype);
 
 /*
  * xla_amd_launch_dequant_dot for callers that cannot allocate device memory (code under HIP graph

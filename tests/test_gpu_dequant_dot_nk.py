@@ -1,0 +1,204 @@
+"""GPU parity of xla_amd.dequant_dot over weights stored [N,K] (rhs_contracting_dim = 1, the
+spelling of fusion_emitter_int4_device_test.cc:867-892).  The values of such a dot are those of
+the [K,N] call on the transposed arrays, so the reference is the oracle on the [K,N] workload the
+case was made from; the dequantised weights themselves are read back bit-exactly with one-hot
+activations."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import dev_bf16, dev_f32, dev_s8, dev_u8, host_bf16
+from tests.test_gpu_dequant_dot import compare
+from xla_amd import dtypes, ffi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+    sys.stdout.flush()
+
+
+def run_nk(w, force_kernel=0, slices=0, ct=0, scratch="auto"):
+    """w: a [K,N] workload; runs it with the weights re-laid out [N,K]."""
+    v = workloads.k_minor(w)
+    lhs = dev_bf16(v["lhs"])
+    wt = dev_u8(v["weights_packed"]) if v["weight_dtype"] in ("s4", "u4") else dev_s8(v["weights"])
+    zp = dev_u8(v["zero_points_packed"]) if v.get("zero_points_packed") is not None else None
+    sc = dev_bf16(v["scales"]) if v["scales"].dtype == np.uint16 else dev_f32(v["scales"])
+    bias = None
+    if v.get("bias") is not None:
+        bias = dev_bf16(v["bias"]) if v["bias"].dtype == np.uint16 else dev_f32(v["bias"])
+    ffi.set_option("dequant_dot_kernel", force_kernel)
+    ffi.set_option("dequant_dot_slices", slices)
+    ffi.set_option("dequant_dot_nk_ct", ct)
+    try:
+        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=v["weight_dtype"], weight_shape=v["weight_shape"],
+                              epilogue=v["epilogue"], dequant_type=v["dequant_type"], dot_type=v.get("dot_type", "f32"),
+                              epilogue_type=v.get("epilogue_type", "f32"), zero_points=zp,
+                              scale_group_size=0 if v["group"] == v["lhs"].shape[-1] else v["group"],
+                              rhs_contracting_dim=1, scratch=scratch)
+        torch.cuda.synchronize()
+    finally:
+        for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_nk_ct"):
+            ffi.set_option(k, 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 40, 64])
+def test_s4_group_scales_bf16_multiply(oracle, M):
+    say("dequant_dot [N,K] s4 group 128 bf16 multiply M=%d" % M)
+    w = workloads.c2_s4_group(M=M, K=4096, N=1024)
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_s4_m%d_rounded" % (16 if M <= 16 else 32 if M <= 32 else 64), kern
+    compare(oracle, w, got, "[N,K] s4 M=%d %s" % (M, kern))
+
+
+@pytest.mark.parametrize("M", [3, 16, 24, 33, 64])
+def test_s8_per_channel_f32_multiply(oracle, M):
+    say("dequant_dot [N,K] s8 per channel M=%d" % M)
+    w = workloads.c1_s8_channel(M=M, K=2048, N=1000)
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_s8_m%d_factored" % (16 if M <= 16 else 32 if M <= 32 else 64), kern
+    compare(oracle, w, got, "[N,K] s8 M=%d %s" % (M, kern))
+
+
+@pytest.mark.parametrize("ct", [1, 2, 4])
+@pytest.mark.parametrize("slices", [1, 2, 4])
+def test_channel_tiles_and_k_slices(oracle, ct, slices):
+    say("dequant_dot [N,K] s4 ct=%d slices=%d" % (ct, slices))
+    w = workloads.c2_s4_group(M=5, K=2048, N=328, group=64)
+    got, kern = run_nk(w, ct=ct, slices=slices)
+    assert kern.startswith("dequant_dot_nk_s4_m16") and kern.endswith("_rounded"), kern
+    compare(oracle, w, got, "[N,K] s4 %s slices=%d" % (kern, slices))
+    w = workloads.c1_s8_channel(M=9, K=1024, N=200)
+    got, kern = run_nk(w, ct=ct, slices=slices)
+    assert kern.startswith("dequant_dot_nk_s8_m16") and kern.endswith("_factored"), kern
+    compare(oracle, w, got, "[N,K] s8 %s slices=%d" % (kern, slices))
+
+
+def test_k_slices_without_scratch_run_as_one(oracle):
+    say("dequant_dot [N,K] s8 few channels, no scratch")
+    w = workloads.c1_s8_channel(M=4, K=4096, N=256)
+    got, kern = run_nk(w)
+    got2, kern2 = run_nk(w, scratch=None)
+    assert kern == kern2 == "dequant_dot_nk_s8_m16_factored"
+    compare(oracle, w, got, "[N,K] sliced")
+    compare(oracle, w, got2, "[N,K] unsliced")
+
+
+@pytest.mark.parametrize("kind,M", [("s8", 8), ("s8", 48), ("s4", 8), ("s4", 32), ("u4", 16)])
+def test_group_scales_f32_multiply(oracle, kind, M):
+    """f32-typed multiply with group scales: per-group integer sums folded with the scale."""
+    say("dequant_dot [N,K] %s group scales f32 multiply M=%d" % (kind, M))
+    if kind == "s8":
+        w = workloads.c1_s8_channel(M=M, K=2048, N=520)
+        w["scales"] = np.random.default_rng(5).uniform(1e-3, 1e-2, (2048 // 128, 520)).astype(np.float32)
+        w["group"] = 128
+    elif kind == "s4":
+        w = workloads.c2_s4_group(M=M, K=2048, N=520, group=256)
+        w["dequant_type"] = "f32"
+    else:
+        w = workloads.u4_zero_point_group(M=M, K=2048, N=520, group=128)
+        w["dequant_type"] = "f32"
+    got, kern = run_nk(w)
+    assert kern.endswith("_group_factored"), kern
+    compare(oracle, w, got, "[N,K] %s %s" % (kind, kern))
+
+
+@pytest.mark.parametrize("M", [2, 16, 30])
+def test_u4_zero_points(oracle, M):
+    say("dequant_dot [N,K] u4 + zero points M=%d" % M)
+    w = workloads.u4_zero_point_group(M=M, K=2048, N=776, group=64)
+    got, kern = run_nk(w)
+    assert kern.startswith("dequant_dot_nk_s4_m") and kern.endswith("_rounded"), kern
+    compare(oracle, w, got, "[N,K] u4 zp M=%d" % M)
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4", "u4"])
+def test_one_hot_reads_back_the_dequantised_weights(oracle, kind):
+    """Activation row m is the unit vector of k = (m * 37 + 5) % K: output [m, n] is weight (n, k)
+    dequantised, with no sum to hide behind."""
+    say("dequant_dot [N,K] one-hot %s" % kind)
+    K, N, M = 512, 264, 64
+    if kind == "s8":
+        w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    elif kind == "s4":
+        w = workloads.c2_s4_group(M=M, K=K, N=N, group=32)
+        w["epilogue"], w["bias"] = "DEFAULT", None
+    else:
+        w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=32)
+        w["epilogue"], w["bias"] = "DEFAULT", None
+    a = np.zeros((M, K), np.float32)
+    ks = (np.arange(M) * 37 + 5) % K
+    a[np.arange(M), ks] = 1.0
+    w["lhs"] = dtypes.f32_to_bf16(a)
+    got, kern = run_nk(w)
+    assert kern.startswith("dequant_dot_nk_"), kern
+    from tests.test_gpu_dequant_dot import oracle_dot
+    assert np.array_equal(got, oracle_dot(oracle, w)), kern
+
+
+def test_batched_with_per_batch_scales(oracle):
+    say("dequant_dot [B,N,K] s8 per batch scales, s4 group scales")
+    w = workloads.c5_s8_batched(B=3, M=20, K=1024, N=392)
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_s8_m32_factored", kern
+    compare(oracle, w, got, "[B,N,K] s8")
+    w = workloads.batched_s4_group(B=3, M=8, K=1024, N=264, group=128)
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_s4_m16_rounded", kern
+    compare(oracle, w, got, "[B,N,K] s4")
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4"])
+def test_more_than_64_tokens_run_in_token_chunks(oracle, kind):
+    say("dequant_dot [N,K] %s 200 tokens" % kind)
+    w = (workloads.c1_s8_channel(M=200, K=1024, N=392) if kind == "s8"
+         else workloads.c2_s4_group(M=200, K=1024, N=392, group=128))
+    got, kern = run_nk(w)
+    assert kern.startswith("dequant_dot_nk_" + kind), kern
+    compare(oracle, w, got, "[N,K] %s 200 tokens" % kind)
+
+
+@pytest.mark.parametrize("K,N,group", [(1000, 36, 1000), (1096, 50, 8), (72, 7, 24)])
+def test_unaligned_shapes_take_the_generic_kernel(oracle, K, N, group):
+    say("dequant_dot [N,K] generic K=%d N=%d group=%d" % (K, N, group))
+    w = workloads.c1_s8_channel(M=5, K=K, N=N)
+    if group != K:
+        w["scales"] = np.random.default_rng(6).uniform(1e-3, 1e-2, (K // group, N)).astype(np.float32)
+        w["group"] = group
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_generic", kern
+    compare(oracle, w, got, "[N,K] generic s8")
+    w = workloads.c2_s4_group(M=5, K=K, N=N + (N & 1), group=group)
+    got, kern = run_nk(w)
+    assert kern == "dequant_dot_nk_generic", kern
+    compare(oracle, w, got, "[N,K] generic s4")
+
+
+def test_forced_generic_equals_streaming_kernel_within_tolerance(oracle):
+    say("dequant_dot [N,K] forced generic")
+    w = workloads.c2_s4_group(M=12, K=1024, N=136, group=128)
+    got, kern = run_nk(w, force_kernel=1)
+    assert kern == "dequant_dot_nk_generic", kern
+    compare(oracle, w, got, "[N,K] forced generic")
+
+
+def test_bad_arguments():
+    say("dequant_dot [N,K] error paths")
+    lhs = torch.zeros((4, 64), dtype=torch.bfloat16, device="cuda")
+    wt = torch.zeros((32, 64), dtype=torch.int8, device="cuda")
+    sc = torch.ones((32,), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffi.FfiError, match="come with scale_group_size"):
+        ops.dequant_dot(lhs, wt, sc, rhs_contracting_dim=1)
+    with pytest.raises(ffi.FfiError, match="rhs_contracting_dim must be 0 or 1"):
+        ops.dequant_dot(lhs, wt, sc, rhs_contracting_dim=2, scale_group_size=0)
+    sc2 = torch.ones((2, 32), dtype=torch.float32, device="cuda")
+    with pytest.raises(ffi.FfiError, match=r"must be \[batch,\]N,K/scale_group_size"):
+        ops.dequant_dot(lhs, wt, sc2, rhs_contracting_dim=1, scale_group_size=32)
+    gs = torch.tensor([4], dtype=torch.int32, device="cuda")
+    with pytest.raises(ffi.FfiError, match="a ragged dot takes weights"):
+        ops.dequant_dot(lhs, wt.reshape(1, 32, 64), sc, group_sizes=gs, rhs_contracting_dim=1, scale_group_size=0)

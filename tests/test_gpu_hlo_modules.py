@@ -10,7 +10,7 @@ import torch
 
 from oracle import hlo_eval
 from tests.gpu_util import check_dot, check_f8_result, dev_bf16, dev_f32, dev_s8, dev_u8, dot_floor, host_bf16
-from xla_amd import dtypes, hlo, hlo_modules as hm, hlo_runner, workloads
+from xla_amd import dtypes, ffi, hlo, hlo_modules as hm, hlo_runner, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -261,6 +261,60 @@ def test_batched_s4_group_module():
     wd = np.abs(w["weights"].astype(np.float64)) * np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1)
     fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
     check_dot(host_bf16(out), ref, fl, "batched s4 group module")
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4", "s4_f32", "u4", "batched"])
+def test_k_minor_weight_modules(kind):
+    """Weights stored [N,K] (rhs_contracting_dims = {1}): module -> pass -> handler, against the
+    op-by-op evaluation of the same module."""
+    say("module with [N,K] weights: %s" % kind)
+    if kind == "s8":
+        M, K, N = 16, 1024, 520
+        v = workloads.k_minor(workloads.c1_s8_channel(M=M, K=K, N=N))
+        text = hm.k_minor_s8_channel(M, K, N)
+        host_args = [v["lhs"], v["weights"], v["scales"]]
+        dev_args = [dev_bf16(v["lhs"]), dev_s8(v["weights"]), dev_f32(v["scales"])]
+        want = "dot -> xla_amd.dequant_dot [DEFAULT, s8, weights [N,K]]"
+        sv = np.repeat(v["scales"].astype(np.float64)[:, None], K, axis=1)
+    elif kind in ("s4", "s4_f32"):
+        M, K, N, g = 24, 1024, 520, 128
+        w = workloads.c2_s4_group(M=M, K=K, N=N, group=g)
+        ty = "bf16" if kind == "s4" else "f32"
+        if ty == "f32":
+            w["scales"] = dtypes.bf16_to_f32(w["scales"])
+        v = workloads.k_minor(w)
+        text = hm.k_minor_s4_group(M, K, N, g, typed=ty)
+        host_args = [v["lhs"], v["weights"], v["scales"], v["bias"]]
+        dev_args = [dev_bf16(v["lhs"]), dev_u8(v["weights_packed"]),
+                    dev_bf16(v["scales"]) if ty == "bf16" else dev_f32(v["scales"]), dev_bf16(v["bias"])]
+        want = "dot -> xla_amd.dequant_dot [BIAS_SILU, s4, weights [N,K]]"
+        sc = dtypes.bf16_to_f32(v["scales"]) if ty == "bf16" else v["scales"]
+        sv = np.repeat(sc.astype(np.float64), g, axis=1)
+    elif kind == "u4":
+        M, K, N, g = 8, 512, 264, 64
+        v = workloads.k_minor(workloads.u4_zero_point_group(M=M, K=K, N=N, group=g))
+        text = hm.k_minor_u4_zero_point_group(M, K, N, g)
+        host_args = [v["lhs"], v["weights"], v["scales"], v["zero_points"].astype(np.int8), v["bias"]]
+        dev_args = [dev_bf16(v["lhs"]), dev_u8(v["weights_packed"]), dev_bf16(v["scales"]),
+                    dev_u8(v["zero_points_packed"]), dev_bf16(v["bias"])]
+        want = "dot -> xla_amd.dequant_dot [BIAS, u4 with zero points, weights [N,K]]"
+        sv = np.repeat(dtypes.bf16_to_f32(v["scales"]).astype(np.float64), g, axis=1) * 2.0   # |w - z| <= 15
+    else:
+        B, M, K, N = 3, 20, 1024, 392
+        v = workloads.k_minor(workloads.c5_s8_batched(B=B, M=M, K=K, N=N))
+        text = hm.k_minor_s8_batched(B, M, K, N)
+        host_args = [v["lhs"], v["weights"], v["scales"]]
+        dev_args = [dev_bf16(v["lhs"]), dev_s8(v["weights"]), dev_f32(v["scales"])]
+        want = "dot -> xla_amd.dequant_dot [DEFAULT, s8, weights [N,K]]"
+        sv = np.repeat(v["scales"].astype(np.float64)[:, :, None], K, axis=2)
+    out, rw, _ = hlo_runner.compile_and_run(text, dev_args)
+    torch.cuda.synchronize()
+    assert rw == [want]
+    assert ffi.last_kernel().startswith("dequant_dot_nk_"), ffi.last_kernel()
+    ref = reference(text, host_args)
+    wd = np.abs(v["weights"].astype(np.float64)) * sv          # [.., N, K]
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(v["lhs"]).astype(np.float64)), np.swapaxes(wd, -1, -2), K)
+    check_dot(host_bf16(out), ref, fl, "[N,K] %s module" % kind)
 
 
 def test_unrewritten_module_does_not_run():

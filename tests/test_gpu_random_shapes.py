@@ -56,6 +56,41 @@ def test_dequant_dot_random_shapes(oracle):
     assert len(kernels) >= 3, kernels    # decode, tiled and generic all took part
 
 
+def test_dequant_dot_k_minor_random_shapes(oracle):
+    """The same draw with the weights stored [N,K] (rhs_contracting_dim = 1)."""
+    from tests.test_gpu_dequant_dot_nk import run_nk
+    rng = np.random.default_rng(4048)
+    kernels = set()
+    for case in range(30):
+        bits = int(rng.choice([4, 8]))
+        M = int(rng.choice([1, 2, 5, 8, 13, 16, 17, 31, 32, 40, 64, 65, 100, 200]))
+        group = int(rng.choice([8, 16, 32, 64, 128, 256]))
+        K = group * int(rng.integers(1, 24))
+        N = int(rng.choice([8, 24, 64, 100, 128, 136, 256, 520, 1000]))
+        per_channel = bool(rng.integers(0, 2))
+        if per_channel:
+            group = K
+        if bits == 4 and K % 2:
+            K += 1; group = K; per_channel = True
+        epilogue = EPILOGUES[int(rng.integers(0, 8))]
+        typed = "bf16" if rng.integers(0, 2) else "f32"
+        say("dequant_dot [N,K] #%d s%d M=%d K=%d N=%d group=%d %s %s" % (case, bits, M, K, N, group, epilogue, typed))
+        lhs = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+        wq = rng.integers(-8 if bits == 4 else -127, 8 if bits == 4 else 128, size=(K, N)).astype(np.int8)
+        sc = rng.uniform(1e-3, 2e-2, size=(K // group, N)).astype(np.float32)
+        if per_channel:
+            sc = sc.reshape(N)
+        w = dict(lhs=lhs, weights=wq, scales=dtypes.f32_to_bf16(sc) if typed == "bf16" else sc,
+                 bias=dtypes.f32_to_bf16(rng.standard_normal(N).astype(np.float32)) if "BIAS" in epilogue else None,
+                 weight_dtype="s%d" % bits, weight_shape=(K, N), group=group, dequant_type=typed, epilogue=epilogue)
+        if bits == 4:
+            w["weights_packed"] = dtypes.pack_s4(wq)
+        got, kern = run_nk(w)
+        kernels.add("generic" if kern.endswith("generic") else kern.rsplit("_", 1)[-1])
+        compare(oracle, w, got, "[N,K] #%d %s" % (case, kern))
+    assert len(kernels) >= 3, kernels    # rounded, factored (or group-factored) and generic all took part
+
+
 def test_fp8_dot_random_shapes(oracle):
     rng = np.random.default_rng(77)
     for case in range(16):

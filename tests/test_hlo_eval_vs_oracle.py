@@ -167,3 +167,36 @@ def test_batched_s4_group_scales(oracle):
     ref = np.stack([oracle.dequant_dot(w["lhs"][b], dtypes.pack_s4(w["weights"][b]), 4, w["scales"][b], "bf16", "bf16",
                                        group=32) for b in range(3)])
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4", "s4_f32", "u4", "batched"])
+def test_weights_with_the_contracting_dimension_minor(oracle, kind):
+    """Weights stored [N,K] (rhs_contracting_dims = {1}): the module, op by op, on the re-laid-out
+    arrays gives the bits of the fused oracle function on the [K,N] arrays it was made from."""
+    if kind == "s8":
+        w = workloads.c1_s8_channel(M=5, K=96, N=40)
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_s8_channel(5, 96, 40), [v["lhs"], v["weights"], v["scales"]])
+        ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
+    elif kind in ("s4", "s4_f32"):
+        w = workloads.c2_s4_group(M=3, K=256, N=48, group=64)
+        ty = "bf16" if kind == "s4" else "f32"
+        if ty == "f32":
+            w["scales"] = dtypes.bf16_to_f32(w["scales"])
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_s4_group(3, 256, 48, 64, typed=ty), [v["lhs"], v["weights"], v["scales"], v["bias"]])
+        ref = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], ty, ty, bias=w["bias"],
+                                 group=64, epilogue="silu")
+    elif kind == "u4":
+        w = workloads.u4_zero_point_group(M=3, K=128, N=24, group=32)
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_u4_zero_point_group(3, 128, 24, 32),
+                         [v["lhs"], v["weights"], v["scales"], v["zero_points"].astype(np.int8), v["bias"]])
+        ref = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", bias=w["bias"],
+                                 group=32, unsigned=True, zero_points=w["zero_points_packed"])
+    else:
+        w = workloads.c5_s8_batched(B=2, M=4, K=64, N=24)
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_s8_batched(2, 4, 64, 24), [v["lhs"], v["weights"], v["scales"]])
+        ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
+    assert np.array_equal(got, ref)

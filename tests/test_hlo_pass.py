@@ -362,7 +362,7 @@ ENTRY main {
 }
 """
     assert hlo.rewrite(text)[1] == []
-    # weights as rhs but contracting their minor dimension: refused with the reason
+    # weights as rhs contracting their minor dimension ([N,K]): taken, with rhs_contracting_dim = 1
     text = """HloModule t
 ENTRY main {
   a = bf16[4,128] parameter(0)
@@ -375,7 +375,8 @@ ENTRY main {
 }
 """
     new, rw, rf = hlo.rewrite(text)
-    assert rw == [] and "custom-call" not in new
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8, weights [N,K]]"] and rf == []
+    check(new, r"dequant_type = 16 : i32", r"dot_type = 16 : i32", r"rhs_contracting_dim = 1 : i64")
 
 
 def test_dot_with_second_user_keeps_epilogue_outside():
@@ -559,3 +560,35 @@ def test_c3_fp8_vector_scales_under_a_bf16_multiply():
     check(new, r"%a_scale.f32 = f32\[64\]\{0\} convert\(%a_scale\)", r"%b_scale.f32 = f32\[32\]\{0\} convert\(%b_scale\)",
           r"s8\[%d\]\{0\}\) custom-call\(%%a, %%b, %%a_scale.f32, %%b_scale.f32, %%bias\)" % ((64 + 32) * 128 * 2),
           r"dequant_type = 16 : i32")
+
+
+def test_weights_with_the_contracting_dimension_minor():
+    """dot(lhs, dequantised [N,K] weights), rhs_contracting_dims = {1} (the spelling of
+    fusion_emitter_int4_device_test.cc:867-892): one call with rhs_contracting_dim = 1, the scales
+    [N] or [N,K/g] as they are, scratch sized by the [N,K] kernels' own query."""
+    new, rw, rf = hlo.rewrite(hm.k_minor_s8_channel(16, 4096, 4096))
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8, weights [N,K]]"] and rf == []
+    ws = ffi.library().xla_amd_dequant_dot_workspace_bytes_nk(1, 16, 4096, 4096, 2)
+    check(new, r"%w = s8\[4096,4096\] parameter\(1\)",
+          r"\(bf16\[16,4096\]\{1,0\}, s8\[%d\]\{0\}\) custom-call\(%%lhs, %%w, %%scale\)" % ws,
+          r"scale_group_size = 0 : i64, rhs_contracting_dim = 1 : i64")
+    assert ws > 0
+    new, rw, rf = hlo.rewrite(hm.k_minor_s4_group(8, 8192, 28672))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, weights [N,K]]"] and rf == []
+    check(new, r"%scales = bf16\[28672,64\] parameter\(2\)", r"custom-call\(%lhs, %w, %scales, %bias\)",
+          r"dequant_type = 16 : i32", r"scale_group_size = 128 : i64, rhs_contracting_dim = 1 : i64")
+    assert sorted(set(opcodes(new))) == ["custom-call", "get-tuple-element", "parameter"]
+    new, rw, rf = hlo.rewrite(hm.k_minor_s4_group(8, 2048, 512, 256, typed="f32"))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, weights [N,K]]"] and rf == []
+    check(new, r"dequant_type = 11 : i32", r"scale_group_size = 256 : i64, rhs_contracting_dim = 1 : i64")
+    new, rw, rf = hlo.rewrite(hm.k_minor_u4_zero_point_group(8, 256, 64, 64))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, u4 with zero points, weights [N,K]]"] and rf == []
+    check(new, r"%zero = u4\[64,4\] parameter\(3\)", r"custom-call\(%lhs, %w, %scales, %zero, %bias\)")
+    new, rw, rf = hlo.rewrite(hm.k_minor_s8_batched(3, 20, 1024, 392))
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8, weights [N,K]]"] and rf == []
+    check(new, r"%scale = f32\[3,392\] parameter\(2\)", r"custom-call\(%lhs, %w, %scale\)", r"rhs_contracting_dim = 1 : i64")
+    # scales broadcast along the wrong dimension of [N,K] weights are no dequantisation of them
+    bad = hm.k_minor_s8_channel(16, 64, 64).replace("broadcast(%scale), dimensions={0}", "broadcast(%scale), dimensions={1}")
+    assert hlo.rewrite(bad)[1] == []
+    # the [K,N] spelling keeps its attributes (no rhs_contracting_dim)
+    assert "rhs_contracting_dim" not in hlo.rewrite(hm.c1_s8_channel())[0]

@@ -20,7 +20,7 @@ struct Option {
   int value;
 };
 thread_local Option g_options[] = {{"dequant_dot_kernel", 0}, {"dequant_dot_vec", 0},
-                      {"dequant_dot_slices", 0}, {"dequant_dot_waves", 0}, {"dequant_dot_skew", 0}, {"dequant_dot_x", 0}, {"dequant_dot_pair", 0}, {"dequant_dot_share", 0}, {"dequant_dot_depth", 0}, {"dequant_dot_steps", 0},
+                      {"dequant_dot_slices", 0}, {"dequant_dot_waves", 0}, {"dequant_dot_skew", 0}, {"dequant_dot_x", 0}, {"dequant_dot_nk_ct", 0}, {"dequant_dot_pair", 0}, {"dequant_dot_share", 0}, {"dequant_dot_depth", 0}, {"dequant_dot_steps", 0},
                       {"fp8_dot_kernel", 0},
                       {"quantize_variant", 0}, {"fp8_dot_layout", 0}, {"tiled_epilogue", 0}, {"tiled_tail", 0}};
 }  // namespace
@@ -51,6 +51,7 @@ int GetOption(const char* key) {
 }
 
 size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4);
+size_t DequantDotNkWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit);
 size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contracting_dim, int dequant_type);
 size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N);
 
@@ -85,6 +86,12 @@ size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, 
   // more than 64 tokens may run on the tiled kernel, which splits the tiles of a short last round
   const size_t tail = weight_dtype == XLA_FFI_DataType_U4 ? 0 : xla_amd::TiledTailWorkspaceBytes(batch, M, K, N);
   return decode > tail ? decode : tail;
+}
+
+size_t xla_amd_dequant_dot_workspace_bytes_nk(int64_t batch, int64_t M, int64_t K, int64_t N,
+                                              int32_t weight_dtype) {
+  return xla_amd::DequantDotNkWorkspaceBytes(
+      batch, M, K, N, weight_dtype == XLA_FFI_DataType_S4 || weight_dtype == XLA_FFI_DataType_U4);
 }
 
 size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,

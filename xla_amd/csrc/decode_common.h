@@ -136,5 +136,10 @@ size_t S4xPairWorkspaceBytes(int64_t batch, int64_t M, int64_t N);
 int LaunchDequantDotDecodeS8x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream);
 size_t S8xWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N);
 
+// Weights stored [N,K] (the contracting dimension minor), scales [N] or [N, K/group], any number of
+// tokens (dequant_dot_nk.hip).  dp comes filled except for the strip / slice layout.
+int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream);
+size_t DequantDotNkWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit);
+
 }  // namespace xla_amd
 #endif  // XLA_AMD_CSRC_DECODE_COMMON_H_

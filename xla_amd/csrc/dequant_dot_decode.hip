@@ -663,6 +663,13 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.ragged_chunks = ragged && p.M > 64 ? (int)((p.M + 63) / 64) : 1;
   if (ragged && (p.M + 63) / 64 > 65535)
     return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes at most 4194240 rows");
+  if (p.rhs_contracting_dim != 0 && p.rhs_contracting_dim != 1)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: rhs_contracting_dim must be 0 or 1");
+  if (p.rhs_contracting_dim == 1) {  // weights [N,K]
+    if (ragged)
+      return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes weights [groups,K,N]");
+    return LaunchDequantDotNk(dp, p, stream);
+  }
   const bool per_channel = p.group == p.K;
   // f32-typed multiply: one scale per channel factors out of the whole sum, scales per group of whole
   // 32-row steps out of each group's sum; anything else under an f32 multiply takes the generic kernel
@@ -867,8 +874,10 @@ static int StaticScratchPointer(void** out) {
 }
 
 int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream) {
+  const bool four_bit = p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4;
   const size_t need = p.batch > 0 && p.M > 0 && p.K > 0 && p.N > 0
-                          ? DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4)
+                          ? p.rhs_contracting_dim == 1 ? DequantDotNkWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit) :
+                          DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4)
                           : 0;
   if (need > kStaticScratchBytes)
     return Fail(XLA_FFI_Error_Code_RESOURCE_EXHAUSTED,

@@ -1,0 +1,480 @@
+// Dequantize-dot over weights stored [N,K] -- the contracting dimension minor, as
+// `dot(lhs, convert(s4[N,K])), rhs_contracting_dims={1}` spells it
+// (xla/backends/gpu/codegen/triton/tests/fusion_emitter_int4_device_test.cc:867-892) and as a
+// checkpoint written for `y = x W^T` stores its matrices.  4-bit weights are packed two per byte
+// along K (low nibble = the even k, xla/packing.cc:142-170), scales are [N] or [N, K/group].
+//
+// K-minor rows are already the matrix instruction's operand: for v_mfma_f32_16x16x32_bf16 lane
+// (c, q) = (lane % 16, lane / 16) holds 8 consecutive k of row c, so a lane that fetches 16
+// contiguous bytes of channel c owns two (s8) or four (s4) operands with no transposition.
+// A wave walks K for CT tiles of 16 channels and MT tiles of 16 tokens; the waves of a workgroup
+// take neighbouring channels over the same k and share the activations through LDS.  Few
+// channels: K is cut into slices (grid.z) whose f32 partial sums the finalize kernel adds in
+// slice order.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "decode_common.h"
+
+namespace xla_amd {
+namespace {
+
+constexpr uint32_t kPastEnd = 0x80000000u;  // every buffer here is smaller than 2 GiB
+constexpr int kNkWaves = 4;
+
+struct NkParams {
+  DecodeParams d;        // operands, shapes, types, slices (strips: channel strips of kNkWaves*CT*16)
+  int k_per_slice;       // multiple of the step (and of the group for group-factored sums)
+  int group_shift;       // log2(group) or -1
+  int m_chunks;          // grid.y = batch * m_chunks, chunk c takes tokens [c*16*MT, +16*MT)
+};
+
+static __device__ __forceinline__ uint32_t group_of(const NkParams& p, uint32_t k) {
+  return p.group_shift >= 0 ? k >> p.group_shift : k / (uint32_t)p.d.group;
+}
+
+// Stage geometry shared by the kernel and its launch.
+template <int WBITS, int MT>
+struct NkStage {
+  static constexpr int KP = 128 / WBITS;                      // k per lane and step: 16 bytes of weights
+  static constexpr int STEP = 4 * KP;                         // k per step (one b128 load per lane and tile)
+  static constexpr int SPS = (WBITS == 4 && MT == 4) ? 2 : 4; // steps per stage
+  static constexpr int KS = SPS * STEP;                       // k per stage
+  static constexpr int ROWB = KS * 2 + 16;                    // LDS pitch of a token row: 16 tokens x 16 bytes
+                                                              // then cover all 64 banks once
+  static constexpr int TOK = 16 * MT;
+  static constexpr int STAGE_BYTES = TOK * ROWB;
+  static constexpr int CHUNKS = TOK * (KS / 8) / (kNkWaves * 64);  // 16-byte pieces a thread moves per stage
+};
+
+// WBITS 8 | 4; MT token tiles; CT channel tiles per wave; MODE as in the [K,N] kernels:
+// kRounded   bf16(w * s) per weight (bf16-typed multiply; group % KP == 0 or one scale per channel)
+// kFactored  integers through the matrix cores, one scale per channel applied to the sum
+// kGroupFactored  the same per scale group (group % (4*KP) == 0), folded with fma(sum, scale, total)
+//
+// K goes by in stages of SPS steps.  The workgroup's activations of a stage ([16 MT tokens][KS k])
+// are fetched once, cooperatively, into one of two LDS buffers, from where every wave reads its
+// matrix operands; a wave's weights (and scales) of the next stage are requested, all of them,
+// before it starts on the current one, so a whole stage of loads is in flight per wave.  One
+// barrier per stage.
+template <int WBITS, int MT, int CT, int MODE>
+__global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams q) {
+  const DecodeParams& p = q.d;
+  using S = NkStage<WBITS, MT>;
+  constexpr int KP = S::KP, NJ = KP / 8, STEP = S::STEP, SPS = S::SPS, KS = S::KS, ROWB = S::ROWB, CHUNKS = S::CHUNKS;
+  constexpr bool GF = MODE == kGroupFactored;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [2][STAGE_BYTES]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, kq = lane >> 4;
+  const int strip = blockIdx.x, slice = blockIdx.z;
+  const int batch = blockIdx.y / q.m_chunks, chunk = blockIdx.y % q.m_chunks;
+  const int m0 = chunk * 16 * MT;
+  const int rows_here = min(16 * MT, p.M - m0);
+  const int n_wave = (strip * kNkWaves + wave) * CT * 16;  // (a wave past N loads nothing and stores nothing)
+  const int G = p.K / p.group;  // scales per channel
+  const uint32_t row_bytes = (uint32_t)p.K * WBITS / 8;
+  const size_t sbatch = p.scale_batched ? batch : 0;
+
+  const __amdgpu_buffer_rsrc_t rw =
+      make_rsrc(p.w + (size_t)batch * p.N * row_bytes, (uint32_t)p.N * row_bytes);
+  const __amdgpu_buffer_rsrc_t ra =
+      make_rsrc(p.lhs + ((size_t)batch * p.M + m0) * p.K, (uint32_t)rows_here * (uint32_t)p.K * 2u);
+  uint32_t voff_w[CT];
+#pragma unroll
+  for (int t = 0; t < CT; ++t) {
+    const int n = n_wave + t * 16 + c;
+    voff_w[t] = n < p.N ? (uint32_t)n * row_bytes + kq * 16 : kPastEnd;
+  }
+
+  const int k_begin = slice * q.k_per_slice;
+  const int k_end = min(p.K, k_begin + q.k_per_slice);
+
+  floatx4 acc[CT][MT], tot[GF ? CT : 1][GF ? MT : 1];
+#pragma unroll
+  for (int t = 0; t < CT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (GF) tot[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  uintx4 wq[2][SPS][CT], areg[CHUNKS];
+  float sv[2][SPS][CT], zv[2][SPS][CT];  // kRounded (and zero points): the lane's scale / zero point of the step
+  const bool has_zp = WBITS == 4 && p.zero_points != nullptr;
+  const float z_default = WBITS == 4 ? (p.w_unsigned ? 0.0f : 8.0f) : 0.0f;
+
+  // ---- the stage's activations: piece id = i * 256 + tid -> token row id / (KS/8), 8 k at (id % (KS/8)) * 8
+  auto load_acts = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int id = i * (kNkWaves * 64) + tid;
+      const int row = id / (KS / 8), col = id % (KS / 8);
+      const uint32_t k = (uint32_t)(ks + col * 8);
+      // (K % 8 == 0: a piece lies inside its row or past it)
+      areg[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          ra, row < rows_here && k < (uint32_t)k_end ? (uint32_t)row * (uint32_t)p.K * 2u + k * 2u : kPastEnd, 0, 0);
+    }
+  };
+  auto store_acts = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS; ++i) {
+      const int id = i * (kNkWaves * 64) + tid;
+      const int row = id / (KS / 8), col = id % (KS / 8);
+      *reinterpret_cast<uintx4*>(lds + buf * S::STAGE_BYTES + row * ROWB + col * 16) = areg[i];
+    }
+  };
+  auto load_weights = [&](int set, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int st = 0; st < SPS; ++st) {
+      // a 16-byte piece lies inside its row or past it (the row pitch is a multiple of 16 bytes):
+      // past it the lane must not read on into the next row
+      const uint32_t kl = (uint32_t)(ks + st * STEP + kq * KP);
+      const bool live = kl < (uint32_t)k_end;
+      const uint32_t wb = (uint32_t)(ks + st * STEP) * WBITS / 8;
+#pragma unroll
+      for (int t = 0; t < CT; ++t)
+        wq[set][st][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, live ? voff_w[t] + wb : kPastEnd, 0, 0);
+      if (MODE == kRounded || has_zp) {
+        const uint32_t g = group_of(q, live ? kl : 0u);
+#pragma unroll
+        for (int t = 0; t < CT; ++t) {
+          const int n = n_wave + t * 16 + c;
+          const size_t e = (sbatch * p.N + (size_t)max(0, min(n, p.N - 1))) * G + g;
+          sv[set][st][t] = MODE == kRounded ? load_scale(p.scales, e, p.scale_is_bf16) : 1.0f;
+          zv[set][st][t] = has_zp ? (float)((p.zero_points[e >> 1] >> (4 * (e & 1))) & 0xfu) : z_default;
+        }
+      }
+    }
+  };
+
+  // whether the scale group ends with the step that starts at k0 (groups are whole steps)
+  auto closes_group = [&](int k0) __attribute__((always_inline)) {
+    const uint32_t e = (uint32_t)(k0 + STEP);
+    return q.group_shift >= 0 ? (e & ((uint32_t)p.group - 1u)) == 0u : e % (uint32_t)p.group == 0u;
+  };
+
+  auto compute = [&](int set, int st, int buf, int k0) __attribute__((always_inline)) {
+    float gs[CT][4] = {};
+    const bool closing = GF && k0 < k_end && closes_group(k0);
+    if (closing) {  // its scales, by output register
+      const uint32_t g = group_of(q, (uint32_t)k0);
+#pragma unroll
+      for (int t = 0; t < CT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n_wave + t * 16 + 4 * kq + i;
+          gs[t][i] = load_scale(p.scales, (sbatch * p.N + (size_t)max(0, min(n, p.N - 1))) * G + g, p.scale_is_bf16);
+        }
+    }
+    // the lane's operands of the step: token 16 mt + c, k = st * STEP + kq * KP + 8 j ...
+    uintx4 av[MT][NJ];
+    const uint8_t* abase = lds + buf * S::STAGE_BYTES + c * ROWB + (st * STEP + kq * KP) * 2;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+        av[mt][j] = *reinterpret_cast<const uintx4*>(abase + mt * 16 * ROWB + j * 16);
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+      // 4-bit: nibble e of a dword arrives as the f16 value 1024 + u (even e) or 1024 + 16 u (odd e);
+      // (u - z) * s = (1024 + u) * s - (1024 + z) * s = (1024 + 16 u) * (s / 16) - (64 + z) * s:
+      // one fma each, exact for a scale of 8 significant bits
+      const float s = (MODE == kRounded) ? sv[set][st][t] : 1.0f;
+      const float z = WBITS == 4 ? ((MODE == kRounded || has_zp) ? zv[set][st][t] : z_default) : 0.0f;
+      const float s_even = s, c_even = s * -(1024.0f + z), s_odd = s * 0.0625f, c_odd = s * -(64.0f + z);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        float f[8];
+        if constexpr (WBITS == 4) {
+          typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+          const uint32_t x = wq[set][st][t][j];
+          // nibble pairs (0,4), (1,5) of x and (2,6), (3,7) of x >> 8, offset binary for s4 (the
+          // sign bit flipped: u = w + 8), as they are for u4
+          const uint32_t ce = p.w_unsigned ? 0x64006400u : 0x64086408u, co = p.w_unsigned ? 0x64006400u : 0x64806480u;
+          const halfx2 p04 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, ce, 0x6a));
+          const halfx2 p15 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, co, 0x6a));
+          const halfx2 p26 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x >> 8, 0x000f000fu, ce, 0x6a));
+          const halfx2 p37 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x >> 8, 0x00f000f0u, co, 0x6a));
+          f[0] = __builtin_fmaf((float)p04[0], s_even, c_even);
+          f[1] = __builtin_fmaf((float)p15[0], s_odd, c_odd);
+          f[2] = __builtin_fmaf((float)p26[0], s_even, c_even);
+          f[3] = __builtin_fmaf((float)p37[0], s_odd, c_odd);
+          f[4] = __builtin_fmaf((float)p04[1], s_even, c_even);
+          f[5] = __builtin_fmaf((float)p15[1], s_odd, c_odd);
+          f[6] = __builtin_fmaf((float)p26[1], s_even, c_even);
+          f[7] = __builtin_fmaf((float)p37[1], s_odd, c_odd);
+        } else {
+          // 16 bytes are two operands: dwords (2j, 2j + 1)
+          const uint32_t x0 = wq[set][st][t][j * 2], x1 = wq[set][st][t][j * 2 + 1];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            f[e] = (float)(int8_t)((x0 >> (8 * e)) & 0xffu);
+            f[4 + e] = (float)(int8_t)((x1 >> (8 * e)) & 0xffu);
+          }
+          if (MODE == kRounded) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = f[e] * s;
+          }
+        }
+        const uintx4 a = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                          pack_bf16x2(f[6], f[7])};
+        const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, __builtin_bit_cast(bf16x8, av[mt][j]),
+                                                               acc[t][mt], 0, 0, 0);
+      }
+    }
+    if (closing) {
+#pragma unroll
+      for (int t = 0; t < CT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            tot[t][mt][i] = __builtin_fmaf(acc[t][mt][i], gs[t][i], tot[t][mt][i]);
+            acc[t][mt][i] = 0.0f;
+          }
+    }
+  };
+  // Steps past k_end run on zeros (their loads are masked) rather than being branched around: a
+  // branch between a stage's loads and their use lets the compiler move the loads down to the use.
+  auto compute_stage = [&](int set, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int st = 0; st < SPS; ++st) compute(set, st, set, ks + st * STEP);  // (buffer index = register set)
+  };
+
+  load_acts(k_begin);
+  load_weights(0, k_begin);
+  store_acts(0);
+  __syncthreads();
+  for (int ks = k_begin; ks < k_end; ks += 2 * KS) {  // two stages a round; the second may lie past k_end
+    load_acts(ks + KS);
+    load_weights(1, ks + KS);
+    __builtin_amdgcn_sched_barrier(0);  // (keeps the next stage's loads above this stage's arithmetic)
+    compute_stage(0, ks);
+    __builtin_amdgcn_sched_barrier(0);
+    store_acts(1);  // nobody reads buffer 1 any more: every wave passed the barrier that ended its stage
+    __syncthreads();
+    load_acts(ks + 2 * KS);
+    load_weights(0, ks + 2 * KS);
+    __builtin_amdgcn_sched_barrier(0);
+    compute_stage(1, ks + KS);
+    __builtin_amdgcn_sched_barrier(0);
+    store_acts(0);
+    __syncthreads();
+  }
+
+  // ---- lane (c, kq), register i of tile (t, mt): channel n_wave + 16 t + 4 kq + i, token m0 + 16 mt + c.
+  // One tile at a time (the fences keep the scheduler from interleaving the tiles' activations,
+  // which would hold every tile's temporaries in registers at once).
+  const bool quads = p.N % 4 == 0;
+#pragma unroll
+  for (int t = 0; t < CT; ++t) {
+    float fq[4], bq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = max(0, min(n_wave + t * 16 + 4 * kq + i, p.N - 1));
+      fq[i] = MODE == kFactored && p.slices == 1 ? load_scale(p.scales, sbatch * p.N + n, p.scale_is_bf16) : 1.0f;
+      bq[i] = p.bias && p.slices == 1 ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (GF ? tot[t][mt][i] : acc[t][mt][i]) * fq[i];
+      if (p.slices == 1) epilogue_all_dispatch<4>(v, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
+      const int n = n_wave + t * 16 + 4 * kq, m = mt * 16 + c;
+      if (m < rows_here && n < p.N) {
+        const size_t o = ((size_t)batch * p.M + m0 + m) * p.N + n;
+        if (p.slices > 1) {
+          float* dst = p.workspace + ((size_t)batch * p.slices + slice) * ((size_t)p.M * p.N) + (size_t)(m0 + m) * p.N + n;
+          if (quads) {
+            *reinterpret_cast<floatx4*>(dst) = floatx4{v[0], v[1], v[2], v[3]};
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (n + i < p.N) dst[i] = v[i];
+          }
+        } else if (quads) {
+          *reinterpret_cast<uintx2*>(p.out + o) = uintx2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < p.N) p.out[o + i] = f32_to_bf16(v[i]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+// Any shape and alignment: one thread per output, k in increasing order.
+__global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParams p, int wbits, int mode) {
+  const size_t total = (size_t)p.M * p.N;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int batch = blockIdx.y;
+  if (idx >= total) return;
+  const int n = (int)(idx % p.N), m = (int)(idx / p.N);
+  const int G = p.K / p.group;
+  const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
+  const size_t wrow = ((size_t)batch * p.N + n) * p.K;                     // in elements
+  const size_t srow = ((size_t)(p.scale_batched ? batch : 0) * p.N + n) * G;
+  float acc = 0.0f;
+  for (int k = 0; k < p.K; ++k) {
+    const size_t e = wrow + k;
+    int wi;
+    if (wbits == 8) {
+      wi = (int8_t)p.w[e];
+    } else {
+      const uint32_t nib = (p.w[e >> 1] >> (4 * (e & 1))) & 0xfu;
+      wi = p.w_unsigned ? (int)nib : (int)(nib ^ 8u) - 8;
+      if (p.zero_points) {
+        const size_t ze = srow + k / p.group;
+        wi -= (int)((p.zero_points[ze >> 1] >> (4 * (ze & 1))) & 0xfu);
+      }
+    }
+    float wv = (float)wi * load_scale(p.scales, srow + k / p.group, p.scale_is_bf16);
+    if (mode == kRounded) wv = round_bf16(wv);
+    acc = acc + bf16_to_f32(a[k]) * wv;
+  }
+  const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  p.out[(size_t)batch * total + idx] = f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+}
+
+template <int WBITS, int MT, int CT, int MODE>
+int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name) {
+  constexpr size_t kLds = 2 * (size_t)NkStage<WBITS, MT>::STAGE_BYTES;
+  // per kernel instantiation and device: one bit per device ordinal (two threads that race set the
+  // attribute to the same value)
+  static std::atomic<unsigned long long> configured{0};
+  int device = 0;
+  (void)hipGetDevice(&device);
+  const unsigned long long bit = 1ull << (device & 63);
+  if (kLds > 48 * 1024 && !(configured.load(std::memory_order_acquire) & bit)) {
+    hipError_t e = hipFuncSetAttribute((const void*)dequant_dot_nk_kernel<WBITS, MT, CT, MODE>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
+    if (e != hipSuccess)
+      return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", name, kLds, hipGetErrorString(e));
+    configured.fetch_or(bit, std::memory_order_release);
+  }
+  dim3 grid((unsigned)q.d.strips, (unsigned)(batch * q.m_chunks), (unsigned)q.d.slices);
+  hipLaunchKernelGGL((dequant_dot_nk_kernel<WBITS, MT, CT, MODE>), grid, dim3(kNkWaves * 64), kLds, stream, q);
+  int rc = CheckLaunch(name);
+  if (rc) return rc;
+  if (q.d.slices > 1) rc = LaunchDecodeFinalize(q.d, batch, stream, MODE);
+  SetLastKernel(name);
+  return rc;
+}
+
+struct NkShape {
+  int wbits, kp, step, mt, ct, strips, m_chunks, slices, k_per_slice;
+};
+
+// Token tiles, channel tiles and K-slices for a shape the streaming kernel takes.
+NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, int64_t slice_unit) {
+  NkShape s;
+  s.wbits = four_bit ? 4 : 8;
+  s.kp = 128 / s.wbits;
+  s.step = 4 * s.kp;
+  s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  // One token tile: a channel tile per wave and about four workgroups per CU measured fastest on
+  // 8192 x 28672 s4 (1 / 2 / 4 slices: 55.6 / 48.3 / 44.1 us with one tile per wave, 78.9 / 55.2 /
+  // 57.5 us with two); more token tiles: two channel tiles per wave, two workgroups per CU.
+  s.ct = s.mt == 1 ? 1 : 2;
+  if (int v = GetOption("dequant_dot_nk_ct")) s.ct = s.mt != 1 ? 2 : v == 1 ? 1 : v == 4 ? 4 : 2;  // (one token tile only)
+  s.strips = (int)((N + kNkWaves * s.ct * 16 - 1) / (kNkWaves * s.ct * 16));
+  s.m_chunks = (int)((M + 16 * s.mt - 1) / (16 * s.mt));
+  // few workgroups: cut K (at most four ways) while a slice keeps eight steps (or whole groups) and
+  // the partial sums stay below a quarter of the weight bytes
+  const int64_t unit = slice_unit > s.step ? slice_unit : s.step;
+  const int64_t want = s.mt == 1 ? 1024 : 448;
+  int slices = 1;
+  const double weight_bytes = (double)K * N * s.wbits / 8;
+  while (slices < 4 && (int64_t)s.strips * batch * s.m_chunks * slices < want && K / (slices * 2) >= 8 * s.step &&
+         (K / (slices * 2)) % unit == 0 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes)
+    slices *= 2;
+  if (int v = GetOption("dequant_dot_slices")) {
+    if (K % (v * unit) == 0) slices = v;
+  }
+  s.slices = slices;
+  s.k_per_slice = (int)((K / slices + unit - 1) / unit * unit);
+  return s;
+}
+
+}  // namespace
+
+size_t DequantDotNkWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit) {
+  if (batch <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
+  // (the group is not known here: a slice of whole 128-k steps holds whole groups only when the
+  // group divides it, which the launch checks again; sizing assumes the most slices)
+  const NkShape s = PlanNk(batch, M, K, N, four_bit, 0);
+  return DequantDotWorkspaceBytes(batch, M, N, s.slices);
+}
+
+int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream) {
+  const bool four_bit = p.weight_dtype != XLA_FFI_DataType_S8;
+  const int wbits = four_bit ? 4 : 8;
+  const int kp = 128 / wbits;
+  const bool per_channel = p.group == p.K;
+  // f32-typed multiply: one scale per channel factors out of the whole sum, scales per group of whole
+  // steps out of each group's sum; other groups under an f32 multiply take the one-thread-per-output kernel
+  const int mode = p.dequant_type == XLA_FFI_DataType_BF16 ? kRounded
+                   : per_channel || p.group % (4 * kp) != 0 ? kFactored
+                                                            : kGroupFactored;
+  const int64_t row_bytes = p.K * wbits / 8;
+  int group_shift = -1;
+  for (int s = 0; s < 31; ++s)
+    if ((int64_t)1 << s == p.group) group_shift = s;
+  bool fast = row_bytes % 16 == 0 && p.K >= 4 * kp && ((uintptr_t)p.lhs % 16 == 0) && ((uintptr_t)p.weights % 16 == 0) &&
+              (double)p.N * row_bytes < 2147483648.0 && (double)p.M * p.K * 2 < 2147483648.0 &&
+              p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1;
+  if (mode == kRounded && !per_channel && p.group % kp != 0) fast = false;
+  if (mode == kFactored && !per_channel) fast = false;  // an f32 multiply by scales that do not cover whole steps
+  if (p.zero_points && !per_channel && p.group % kp != 0) fast = false;
+  if (!fast) {
+    if (GetOption("dequant_dot_kernel") == 2 || GetOption("dequant_dot_kernel") == 3)
+      return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION, "dequant_dot: the requested kernel does not cover this shape");
+    dp.slices = 1;
+    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)p.batch);
+    hipLaunchKernelGGL(dequant_dot_nk_generic_kernel, grid, dim3(256), 0, stream, dp, wbits,
+                       mode == kGroupFactored ? (int)kFactored : mode);
+    SetLastKernel("dequant_dot_nk_generic");
+    return CheckLaunch("dequant_dot_nk_generic");
+  }
+  NkShape s = PlanNk(p.batch, p.M, p.K, p.N, four_bit, mode == kGroupFactored ? p.group : 0);
+  if (s.slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, s.slices))) {
+    s.slices = 1;
+    s.k_per_slice = (int)p.K;
+  }
+  NkParams q;
+  q.d = dp;
+  q.d.strips = s.strips;
+  q.d.slices = s.slices;
+  q.k_per_slice = s.k_per_slice;
+  q.group_shift = group_shift;
+  q.m_chunks = s.m_chunks;
+#define XLA_AMD_NK(WB, MT_, CT_, MODE_, NAME)                     \
+  if (wbits == WB && s.mt == MT_ && s.ct == CT_ && mode == MODE_) \
+    return launch_nk<WB, MT_, CT_, MODE_>(q, (int)p.batch, stream, NAME);
+#define XLA_AMD_NK_MODES(WB, MT_, CT_, TAG)                                         \
+  XLA_AMD_NK(WB, MT_, CT_, kRounded, "dequant_dot_nk_" TAG "_rounded")              \
+  XLA_AMD_NK(WB, MT_, CT_, kFactored, "dequant_dot_nk_" TAG "_factored")            \
+  XLA_AMD_NK(WB, MT_, CT_, kGroupFactored, "dequant_dot_nk_" TAG "_group_factored")
+  XLA_AMD_NK_MODES(4, 1, 1, "s4_m16")
+  XLA_AMD_NK_MODES(4, 2, 2, "s4_m32")
+  XLA_AMD_NK_MODES(4, 4, 2, "s4_m64")
+  XLA_AMD_NK_MODES(8, 1, 1, "s8_m16")
+  XLA_AMD_NK_MODES(8, 2, 2, "s8_m32")
+  XLA_AMD_NK_MODES(8, 4, 2, "s8_m64")
+  XLA_AMD_NK_MODES(4, 1, 2, "s4_m16_c2")
+  XLA_AMD_NK_MODES(4, 1, 4, "s4_m16_c4")
+  XLA_AMD_NK_MODES(8, 1, 2, "s8_m16_c2")
+  XLA_AMD_NK_MODES(8, 1, 4, "s8_m16_c4")
+#undef XLA_AMD_NK_MODES
+#undef XLA_AMD_NK
+  return Fail(XLA_FFI_Error_Code_INTERNAL, "dequant_dot: no [N,K] kernel for this shape");
+}
+
+}  // namespace xla_amd

@@ -387,7 +387,10 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   DecodeCommonAttrs(d, &a);
   int64_t group_size = 0;
   const bool has_group_size = d.Int("scale_group_size", &group_size);
+  int64_t rcd = 0;  // 1: weights [..,N,K], scales [N] | [B,N] | [N,K/g] | [B,N,K/g]
+  d.Int("rhs_contracting_dim", &rcd);
   if (!d.ok()) return d.Error();
+  const bool nk = rcd == 1;
 
   // ragged: lhs [M,K] (rows sorted by group), weights [groups,K,N], out [M,N]; the groups take the
   // place of the batch for weights and scales
@@ -397,17 +400,21 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   p.batch = ragged ? (w->rank == 3 ? w->dims[0] : 0) : batched ? lhs->dims[0] : 1;
   p.M = lhs->dims[lhs->rank - 2];
   p.K = lhs->dims[lhs->rank - 1];
-  p.N = w->dims[w->rank - 1];
+  p.N = w->dims[w->rank - (nk ? 2 : 1)];
+  p.rhs_contracting_dim = (int32_t)rcd;
   std::string why;
-  if (ragged && (lhs->rank != 2 || w->rank != 3)) why = "a ragged dot takes lhs [M,K] and weights [groups,K,N]";
+  if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
+  else if (nk && ragged) why = "a ragged dot takes weights [groups,K,N]";
+  else if (nk && !has_group_size) why = "weights [N,K] come with scale_group_size";
+  else if (ragged && (lhs->rank != 2 || w->rank != 3)) why = "a ragged dot takes lhs [M,K] and weights [groups,K,N]";
   else if (ragged && gs->dims[0] != p.batch) why = "group_sizes must have one entry per group of weights";
   else if (!ragged && w->rank != lhs->rank) why = "lhs and weights must have the same rank";
-  else if (w->dims[w->rank - 2] != p.K) why = "contracting dimensions differ";
+  else if (w->dims[w->rank - (nk ? 1 : 2)] != p.K) why = "contracting dimensions differ";
   else if (!ragged && batched && w->dims[0] != p.batch) why = "batch dimensions differ";
   else if (out->rank != lhs->rank || out->dims[out->rank - 1] != p.N ||
            out->dims[out->rank - 2] != p.M || (!ragged && batched && out->dims[0] != p.batch))
     why = "result shape must be [batch,]M,N";
-  else if (sc->dims[sc->rank - 1] != p.N) why = "scales must have N as their last dimension";
+  else if (!(nk && group_size > 0) && sc->dims[sc->rank - 1] != p.N) why = "scales must have N as their last dimension";
   else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
   else if (zp && w->dtype != XLA_FFI_DataType_U4) why = "zero points go with U4 weights";
   else if (zp && (zp->rank != sc->rank || memcmp(zp->dims, sc->dims, sizeof(int64_t) * sc->rank) != 0))
@@ -422,7 +429,12 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
     p.scale_batch = 1;
     if (has_group_size) {
       if (group_size < 0 || (group_size > 0 && p.K % group_size != 0)) why = "scale_group_size must divide K";
-      else {
+      else if (nk && group_size > 0) {
+        groups = p.K == 0 ? 1 : p.K / group_size;
+        if (sc->rank == 3) p.scale_batch = sc->dims[0];
+        if (sc->rank < 2 || sc->dims[sc->rank - 1] != groups || sc->dims[sc->rank - 2] != p.N)
+          why = "scales of weights [N,K] must be [batch,]N,K/scale_group_size";
+      } else {
         groups = group_size == 0 || p.K == 0 ? 1 : p.K / group_size;
         const bool per_channel = group_size == 0;
         if (sc->rank == 3) {

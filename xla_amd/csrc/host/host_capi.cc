@@ -43,6 +43,7 @@ std::string ShapeJson(const xla_amd::hlo::Shape& s) {
 struct XlaAmdRewriteCallbacks {
   size_t (*dequant_workspace_bytes)(int64_t, int64_t, int64_t, int64_t, int32_t);
   size_t (*fp8_workspace_bytes)(int64_t, int64_t, int64_t, int32_t, int32_t);
+  size_t (*dequant_nk_workspace_bytes)(int64_t, int64_t, int64_t, int64_t, int32_t);
 };
 
 // Returns the rewritten module text (malloc'd; free with xla_amd_host_free), or NULL with the
@@ -60,6 +61,7 @@ HOST_EXPORT char* xla_amd_hlo_rewrite(const char* text, const XlaAmdRewriteCallb
   if (cb) {
     opt.dequant_workspace_bytes = cb->dequant_workspace_bytes;
     opt.fp8_workspace_bytes = cb->fp8_workspace_bytes;
+    opt.dequant_nk_workspace_bytes = cb->dequant_nk_workspace_bytes;
   }
   xla_amd::hlo::RewriteLog rl;
   int n = xla_amd::hlo::RunQuantFusionRewriter(mod.get(), opt, &rl);

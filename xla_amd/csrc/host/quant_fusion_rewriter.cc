@@ -500,10 +500,11 @@ bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
 
 // ---------------------------------------------------------------- weight-only dequantize dot
 struct QWeights {
-  Instr* w = nullptr;       // s8, s4 or u4 tensor [B,]K,N
-  Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N], bf16 or f32
+  Instr* w = nullptr;       // s8, s4 or u4 tensor [B,]K,N -- or [B,]N,K (K minor)
+  Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N] -- K minor: [N] | [N,G] | [B,N] | [B,N,G]; bf16 or f32
   std::string type;         // element type of the multiply
   Instr* zero = nullptr;    // u4 zero points, shaped like the scales: (w - zero) * scale
+  int64_t groups = 0;       // scales along K, 0 = one per output channel
 };
 
 // convert(s4 -> s8) or convert(u4 -> u8): how 4-bit values are often widened before the float convert
@@ -540,20 +541,26 @@ Instr* LookThroughWidening(Instr* s, const std::string& to) {
   return s;
 }
 
-bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
+// k_minor: the weights are [B,]N,K (the dot contracts their minor dimension) instead of [B,]K,N.
+bool MatchQWeights(Instr* op, bool k_minor, QWeights* out, std::string* why) {
   const std::string ty = op->shape.dtype;
   if (!IsFloatTy(ty)) return false;
   const int64_t rank = op->shape.rank();
   // grouped: reshape([G,g,N] product) -> [K,N], or with a leading batch / expert dimension
-  // reshape([B,G,g,N] product) -> [B,K,N]
+  // reshape([B,G,g,N] product) -> [B,K,N]; K minor: reshape([B,]N,G,g product) -> [B,]N,K
   if (op->Is("reshape") && (rank == 2 || rank == 3) && op->operands[0]->shape.rank() == rank + 1 &&
       op->operands[0]->Is("multiply")) {
     Instr* mul = op->operands[0];
     const int64_t lead = rank - 2;  // 0, or 1 with a batch dimension in front
-    std::vector<int64_t> d3(mul->shape.dims.begin() + lead, mul->shape.dims.end());  // G, g, N
-    if (d3[0] * d3[1] != op->shape.dims[lead] || d3[2] != op->shape.dims[lead + 1]) return false;
+    std::vector<int64_t> d3(mul->shape.dims.begin() + lead, mul->shape.dims.end());  // G, g, N -- or N, G, g
+    if (k_minor) {
+      if (d3[0] != op->shape.dims[lead] || d3[1] * d3[2] != op->shape.dims[lead + 1]) return false;
+    } else if (d3[0] * d3[1] != op->shape.dims[lead] || d3[2] != op->shape.dims[lead + 1]) {
+      return false;
+    }
     if (lead && mul->shape.dims[0] != op->shape.dims[0]) return false;
-    const std::vector<int64_t> bdims = lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2};
+    const std::vector<int64_t> bdims = k_minor ? (lead ? std::vector<int64_t>{0, 1, 2} : std::vector<int64_t>{0, 1})
+                                               : (lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2});
     Instr *sc = nullptr, *cv = nullptr;
     if (!BinaryWith(mul, "multiply", [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
     Instr* zero = nullptr;
@@ -574,28 +581,35 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
       return false;
     }
     sc = LookThroughWidening(sc, ty);
-    if (sc->shape.rank() != rank || sc->shape.dims[lead] != d3[0] || sc->shape.dims[lead + 1] != d3[2]) return false;
+    if (sc->shape.rank() != rank || sc->shape.dims[lead] != d3[0] || sc->shape.dims[lead + 1] != d3[k_minor ? 1 : 2])
+      return false;
     if (lead && sc->shape.dims[0] != op->shape.dims[0]) return false;
-    *out = {w, sc, ty, zero};
+    *out = {w, sc, ty, zero, d3[k_minor ? 1 : 0]};
     return true;
   }
   if (!op->Is("multiply")) return false;
   Instr *sc = nullptr, *cv = nullptr;
-  const std::vector<int64_t> bdims = rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2};
+  const std::vector<int64_t> bdims = k_minor ? (rank == 2 ? std::vector<int64_t>{0} : std::vector<int64_t>{0, 1})
+                                             : (rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2});
   if (!BinaryWith(op, "multiply", [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
   Instr* zero = nullptr;
   PeelZeroPoint(cv, bdims, ty, &cv, &zero);
   Instr* w;
   if (!IntSource(cv, ty, &w) || w->shape.dims != op->shape.dims) return false;
   sc = LookThroughWidening(sc, ty);
-  *out = {w, sc, ty, zero};
+  *out = {w, sc, ty, zero, 0};
   return true;
 }
 
 bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->operands[1], &q, &why)) {
+  const int64_t rank = dot->shape.rank();
+  auto lb = dot->DimsAttr("lhs_batch_dims"), rb = dot->DimsAttr("rhs_batch_dims");
+  auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
+  // weights [..,N,K]: the dot contracts their minor dimension (fusion_emitter_int4_device_test.cc:867-892)
+  const bool k_minor = rc == std::vector<int64_t>{rank - 1};
+  if (!MatchQWeights(dot->operands[1], k_minor, &q, &why)) {
     if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
     return false;
   }
@@ -607,16 +621,13 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   Instr* inner;
   if (lhs->Is("convert") && ConvertFrom(lhs, "bf16", &inner) && lhs->shape.dtype == "f32") lhs = inner;
   if (lhs->shape.dtype != "bf16") return refuse("the activation must be bf16 (or its convert to f32)");
-  const int64_t rank = dot->shape.rank();
   if (rank != 2 && rank != 3) return refuse("rank " + std::to_string(rank));
-  auto lb = dot->DimsAttr("lhs_batch_dims"), rb = dot->DimsAttr("rhs_batch_dims");
-  auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
   if (rank == 3 && (lb != std::vector<int64_t>{0} || rb != std::vector<int64_t>{0}))
     return refuse("the batch dimension must be dimension 0 of both operands");
   if (rank == 2 && !lb.empty()) return refuse("unexpected batch dimensions");
-  if (lc != std::vector<int64_t>{rank - 1} || rc != std::vector<int64_t>{rank - 2})
-    return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] contracting K (N minor); s4 with a "
-                  "minor contracting or batch dimension is rejected as in gemm_fusion.cc:1572-1590");
+  if (lc != std::vector<int64_t>{rank - 1} || (rc != std::vector<int64_t>{rank - 2} && !k_minor))
+    return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] or [..,N,K]; s4 with a "
+                  "minor batch dimension is rejected as in gemm_fusion.cc:1572-1590");
   const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
   if (four_bit && q.w->shape.dims.back() % 2 != 0)
     return refuse("s4 rows must hold an even number of values");
@@ -628,25 +639,26 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
 
   const int64_t B = rank == 3 ? lhs->shape.dims[0] : 1;
-  const int64_t M = lhs->shape.dims[rank - 2], K = lhs->shape.dims[rank - 1], N = q.w->shape.dims[rank - 1];
+  const int64_t M = lhs->shape.dims[rank - 2], K = lhs->shape.dims[rank - 1], N = q.w->shape.dims[rank - (k_minor ? 2 : 1)];
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
   std::vector<Shape> results = {Shape::Array("bf16", dot->shape.dims)};
-  size_t ws = opt.dequant_workspace_bytes
-                  ? opt.dequant_workspace_bytes(B, M, K, N, q.w->shape.dtype == "s4" ? 21 : q.w->shape.dtype == "u4" ? 22 : 2)
-                  : 0;
+  const int32_t wdt = q.w->shape.dtype == "s4" ? 21 : q.w->shape.dtype == "u4" ? 22 : 2;
+  auto sizer = k_minor ? opt.dequant_nk_workspace_bytes : opt.dequant_workspace_bytes;
+  size_t ws = sizer ? sizer(B, M, K, N, wdt) : 0;
   if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
-  // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
-  const int64_t group_size = rank == 2 && q.scale->shape.rank() == 2 ? K / q.scale->shape.dims[0]
-                             : rank == 3 && q.scale->shape.rank() == 3 ? K / q.scale->shape.dims[1] : 0;
+  // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are
+  // [K/g,N], or [N,K/g] next to weights [N,K]
+  const int64_t group_size = q.groups ? K / q.groups : 0;
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results,
                          CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
-                             std::to_string(group_size) + " : i64");
+                             std::to_string(group_size) + " : i64" +
+                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
-                          (q.zero ? " with zero points" : "") + "]");
+                          (q.zero ? " with zero points" : "") + (k_minor ? ", weights [N,K]" : "") + "]");
   return true;
 }
 
@@ -656,7 +668,7 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
 bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->operands[1], &q, &why)) {
+  if (!MatchQWeights(dot->operands[1], /*k_minor=*/false, &q, &why)) {
     if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
     return false;
   }

@@ -18,6 +18,8 @@ namespace hlo {
 // "emit no scratch result".
 struct RewriteOptions {
   size_t (*dequant_workspace_bytes)(int64_t batch, int64_t M, int64_t K, int64_t N, int32_t weight_dtype) = nullptr;
+  // the same for weights [N,K] (xla_amd_dequant_dot_workspace_bytes_nk)
+  size_t (*dequant_nk_workspace_bytes)(int64_t batch, int64_t M, int64_t K, int64_t N, int32_t weight_dtype) = nullptr;
   size_t (*fp8_workspace_bytes)(int64_t M, int64_t K, int64_t N, int32_t rhs_contracting_dim,
                                 int32_t dequant_type) = nullptr;
 };

@@ -23,7 +23,7 @@ HANDLER_SYMBOLS = {
 EXPORTED_SYMBOLS = list(HANDLER_SYMBOLS.values()) + [
     "xla_amd_register_handlers", "xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch",
     "xla_amd_launch_fp8_scaled_dot",
-    "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes",
+    "xla_amd_launch_rowwise_quantize_fp8", "xla_amd_dequant_dot_workspace_bytes", "xla_amd_dequant_dot_workspace_bytes_nk",
     "xla_amd_fp8_scaled_dot_workspace_bytes", "xla_amd_fp8_scaled_dot_workspace_bytes_typed", "xla_amd_last_error",
     "xla_amd_last_kernel",
     "xla_amd_debug_set_option"]
@@ -270,6 +270,8 @@ def library():
         L.xla_amd_debug_set_option.argtypes = [C.c_char_p, C.c_int]
         L.xla_amd_dequant_dot_workspace_bytes.restype = C.c_size_t
         L.xla_amd_dequant_dot_workspace_bytes.argtypes = [C.c_int64] * 4 + [C.c_int32]
+        L.xla_amd_dequant_dot_workspace_bytes_nk.restype = C.c_size_t
+        L.xla_amd_dequant_dot_workspace_bytes_nk.argtypes = [C.c_int64] * 4 + [C.c_int32]
         for sym in ("xla_amd_launch_dequant_dot", "xla_amd_launch_dequant_dot_static_scratch"):
             getattr(L, sym).restype = C.c_int
             getattr(L, sym).argtypes = [C.POINTER(LaunchDequantDot), C.c_void_p]

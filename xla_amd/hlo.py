@@ -7,7 +7,8 @@ from . import ffi
 
 
 class _Callbacks(C.Structure):
-    _fields_ = [("dequant_workspace_bytes", C.c_void_p), ("fp8_workspace_bytes", C.c_void_p)]
+    _fields_ = [("dequant_workspace_bytes", C.c_void_p), ("fp8_workspace_bytes", C.c_void_p),
+                ("dequant_nk_workspace_bytes", C.c_void_p)]
 
 
 def _lib():
@@ -43,7 +44,8 @@ def rewrite(text, with_scratch=True):
     if with_scratch:
         q = ffi.library()
         cb = _Callbacks(C.cast(q.xla_amd_dequant_dot_workspace_bytes, C.c_void_p).value,
-                        C.cast(q.xla_amd_fp8_scaled_dot_workspace_bytes_typed, C.c_void_p).value)
+                        C.cast(q.xla_amd_fp8_scaled_dot_workspace_bytes_typed, C.c_void_p).value,
+                        C.cast(q.xla_amd_dequant_dot_workspace_bytes_nk, C.c_void_p).value)
     log = C.c_void_p()
     n = C.c_int(0)
     out = L.xla_amd_hlo_rewrite(text.encode(), C.byref(cb) if cb else None, C.byref(log), C.byref(n))

@@ -390,3 +390,102 @@ ENTRY %main {{
   ROOT %out = bf16[{B},{M},{N}] convert(%dot)
 }}
 """
+
+
+# ---- weights stored [N,K]: the dot contracts the minor dimension of its rhs, the layout of a
+# checkpoint written for y = x W^T (fusion_emitter_int4_device_test.cc:867-892)
+
+def k_minor_s8_channel(M=16, K=4096, N=4096):
+    """bf16 [M,K] . (convert(s8 [N,K]) * f32 scale[N])^T -> bf16; f32 multiply."""
+    return f"""HloModule k_minor_s8_channel_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s8[{N},{K}] parameter(1)
+  %scale = f32[{N}] parameter(2)
+  %lhs_f32 = f32[{M},{K}] convert(%lhs)
+  %w_f32 = f32[{N},{K}] convert(%w)
+  %scale_b = f32[{N},{K}] broadcast(%scale), dimensions={{0}}
+  %w_deq = f32[{N},{K}] multiply(%w_f32, %scale_b)
+  %dot = f32[{M},{N}] dot(%lhs_f32, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{1}}
+  ROOT %out = bf16[{M},{N}] convert(%dot)
+}}
+"""
+
+
+def k_minor_s4_group(M=1, K=8192, N=28672, group=128, typed="bf16"):
+    """bf16 [M,K] . typed(convert(s4 [N,K]) * scale[N,K/g])^T + bias, SiLU in f32 -> bf16."""
+    G, t = K // group, typed
+    return f"""HloModule k_minor_s4_group_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s4[{N},{K}] parameter(1)
+  %scales = {t}[{N},{G}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %w_s8 = s8[{N},{K}] convert(%w)
+  %w_g = s8[{N},{G},{group}] reshape(%w_s8)
+  %w_t = {t}[{N},{G},{group}] convert(%w_g)
+  %scales_b = {t}[{N},{G},{group}] broadcast(%scales), dimensions={{0,1}}
+  %w_deq_g = {t}[{N},{G},{group}] multiply(%w_t, %scales_b)
+  %w_deq = {t}[{N},{K}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] dot(%lhs, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{1}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  %neg = f32[{M},{N}] negate(%z)
+  %exp = f32[{M},{N}] exponential(%neg)
+  %one = f32[] constant(1)
+  %one_b = f32[{M},{N}] broadcast(%one), dimensions={{}}
+  %den = f32[{M},{N}] add(%one_b, %exp)
+  %sig = f32[{M},{N}] divide(%one_b, %den)
+  %silu = f32[{M},{N}] multiply(%z, %sig)
+  ROOT %out = bf16[{M},{N}] convert(%silu)
+}}
+"""
+
+
+def k_minor_u4_zero_point_group(M=8, K=4096, N=4096, group=128):
+    """bf16 [M,K] . bf16((convert(u4 [N,K]) - convert(u4 zero[N,K/g])) * bf16 scale[N,K/g])^T + bias -> bf16."""
+    G = K // group
+    return f"""HloModule k_minor_u4_zero_point_group_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = u4[{N},{K}] parameter(1)
+  %scales = bf16[{N},{G}] parameter(2)
+  %zero = u4[{N},{G}] parameter(3)
+  %bias = bf16[{N}] parameter(4)
+  %w_g = u4[{N},{G},{group}] reshape(%w)
+  %w_t = bf16[{N},{G},{group}] convert(%w_g)
+  %zero_t = bf16[{N},{G}] convert(%zero)
+  %zero_b = bf16[{N},{G},{group}] broadcast(%zero_t), dimensions={{0,1}}
+  %w_centered = bf16[{N},{G},{group}] subtract(%w_t, %zero_b)
+  %scales_b = bf16[{N},{G},{group}] broadcast(%scales), dimensions={{0,1}}
+  %w_deq_g = bf16[{N},{G},{group}] multiply(%w_centered, %scales_b)
+  %w_deq = bf16[{N},{K}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] dot(%lhs, %w_deq), lhs_contracting_dims={{1}}, rhs_contracting_dims={{1}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""
+
+
+def k_minor_s8_batched(B=8, M=512, K=4096, N=14336):
+    """bf16 [B,M,K] . (convert(s8 [B,N,K]) * f32 scale[B,N])^T, batch dimension 0 -> bf16 [B,M,N]."""
+    return f"""HloModule k_minor_s8_batched_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{B},{M},{K}] parameter(0)
+  %w = s8[{B},{N},{K}] parameter(1)
+  %scale = f32[{B},{N}] parameter(2)
+  %lhs_f32 = f32[{B},{M},{K}] convert(%lhs)
+  %w_f32 = f32[{B},{N},{K}] convert(%w)
+  %scale_b = f32[{B},{N},{K}] broadcast(%scale), dimensions={{0,1}}
+  %w_deq = f32[{B},{N},{K}] multiply(%w_f32, %scale_b)
+  %dot = f32[{B},{M},{N}] dot(%lhs_f32, %w_deq), lhs_batch_dims={{0}}, lhs_contracting_dims={{2}}, rhs_batch_dims={{0}}, rhs_contracting_dims={{2}}
+  ROOT %out = bf16[{B},{M},{N}] convert(%dot)
+}}
+"""

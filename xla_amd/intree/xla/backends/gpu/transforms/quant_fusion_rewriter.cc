@@ -36,6 +36,7 @@
 extern "C" {
 // libxla_amd_quant.so (include/xla_amd_quant.h)
 size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, int64_t N, int32_t weight_dtype);
+size_t xla_amd_dequant_dot_workspace_bytes_nk(int64_t batch, int64_t M, int64_t K, int64_t N, int32_t weight_dtype);
 size_t xla_amd_fp8_scaled_dot_workspace_bytes_typed(int64_t M, int64_t K, int64_t N, int32_t rhs_contracting_dim,
                                                     int32_t dequant_type);
 }
@@ -446,10 +447,11 @@ bool RewriteBlockScaledDot(HloComputation* comp, Instr* cc, const std::function<
 
 // ---------------------------------------------------------------- weight-only dequantize dot
 struct QWeights {
-  Instr* w = nullptr;       // s8, s4 or u4 tensor [B,]K,N
-  Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N], bf16 or f32
+  Instr* w = nullptr;       // s8, s4 or u4 tensor [B,]K,N -- or [B,]N,K (K minor)
+  Instr* scale = nullptr;   // [N] | [G,N] | [B,N] | [B,G,N] -- K minor: [N] | [N,G] | [B,N] | [B,N,G]; bf16 or f32
   PrimitiveType type = F32; // element type of the multiply
   Instr* zero = nullptr;    // u4 zero points, shaped like the scales: (w - zero) * scale
+  int64_t groups = 0;       // scales along K, 0 = one per output channel
 };
 
 bool IsQuantTy(PrimitiveType t) { return t == S8 || t == S4 || t == U4; }
@@ -484,21 +486,27 @@ Instr* LookThroughWidening(Instr* s, PrimitiveType to) {
   return s;
 }
 
-bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
+// k_minor: the weights are [B,]N,K (the dot contracts their minor dimension) instead of [B,]K,N.
+bool MatchQWeights(Instr* op, bool k_minor, QWeights* out, std::string* why) {
   const PrimitiveType ty = Ty(op);
   if (!IsFloatTy(ty)) return false;
   const int64_t rank = Rank(op);
   // grouped: reshape([G,g,N] product) -> [K,N], or with a leading batch / expert dimension
-  // reshape([B,G,g,N] product) -> [B,K,N]
+  // reshape([B,G,g,N] product) -> [B,K,N]; K minor: reshape([B,]N,G,g product) -> [B,]N,K
   if (op->opcode() == HloOpcode::kReshape && (rank == 2 || rank == 3) && Rank(op->operand(0)) == rank + 1 &&
       op->operand(0)->opcode() == HloOpcode::kMultiply) {
     Instr* mul = op->mutable_operand(0);
     const int64_t lead = rank - 2;  // 0, or 1 with a batch dimension in front
     const std::vector<int64_t> dm = Dims(mul);
-    const std::vector<int64_t> d3(dm.begin() + lead, dm.end());  // G, g, N
-    if (d3[0] * d3[1] != op->shape().dimensions(lead) || d3[2] != op->shape().dimensions(lead + 1)) return false;
+    const std::vector<int64_t> d3(dm.begin() + lead, dm.end());  // G, g, N -- or N, G, g
+    if (k_minor) {
+      if (d3[0] != op->shape().dimensions(lead) || d3[1] * d3[2] != op->shape().dimensions(lead + 1)) return false;
+    } else if (d3[0] * d3[1] != op->shape().dimensions(lead) || d3[2] != op->shape().dimensions(lead + 1)) {
+      return false;
+    }
     if (lead && dm[0] != op->shape().dimensions(0)) return false;
-    const std::vector<int64_t> gdims = lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2};
+    const std::vector<int64_t> gdims = k_minor ? (lead ? std::vector<int64_t>{0, 1, 2} : std::vector<int64_t>{0, 1})
+                                               : (lead ? std::vector<int64_t>{0, 1, 3} : std::vector<int64_t>{0, 2});
     Instr *sc = nullptr, *cv = nullptr;
     if (!BinaryWith(mul, HloOpcode::kMultiply, [&](Instr* s) { return BroadcastAlong(s, gdims, &sc); }, &cv))
       return false;
@@ -517,29 +525,35 @@ bool MatchQWeights(Instr* op, QWeights* out, std::string* why) {
       return false;
     }
     sc = LookThroughWidening(sc, ty);
-    if (Rank(sc) != rank || sc->shape().dimensions(lead) != d3[0] || sc->shape().dimensions(lead + 1) != d3[2])
+    if (Rank(sc) != rank || sc->shape().dimensions(lead) != d3[0] ||
+        sc->shape().dimensions(lead + 1) != d3[k_minor ? 1 : 2])
       return false;
     if (lead && sc->shape().dimensions(0) != op->shape().dimensions(0)) return false;
-    *out = {w, sc, ty, zero};
+    *out = {w, sc, ty, zero, d3[k_minor ? 1 : 0]};
     return true;
   }
   if (op->opcode() != HloOpcode::kMultiply) return false;
   Instr *sc = nullptr, *cv = nullptr;
-  const std::vector<int64_t> bdims = rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2};
+  const std::vector<int64_t> bdims = k_minor ? (rank == 2 ? std::vector<int64_t>{0} : std::vector<int64_t>{0, 1})
+                                             : (rank == 2 ? std::vector<int64_t>{1} : std::vector<int64_t>{0, 2});
   if (!BinaryWith(op, HloOpcode::kMultiply, [&](Instr* s) { return BroadcastAlong(s, bdims, &sc); }, &cv)) return false;
   Instr* zero = nullptr;
   PeelZeroPoint(cv, bdims, ty, &cv, &zero);
   Instr* w;
   if (!IntSource(cv, ty, &w) || Dims(w) != Dims(op)) return false;
   sc = LookThroughWidening(sc, ty);
-  *out = {w, sc, ty, zero};
+  *out = {w, sc, ty, zero, 0};
   return true;
 }
 
 bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<void(std::string)>& log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->mutable_operand(1), &q, &why)) {
+  const int64_t rank = Rank(dot);
+  const DotDimensionNumbers& dn = dot->dot_dimension_numbers();
+  // weights [..,N,K]: the dot contracts their minor dimension (fusion_emitter_int4_device_test.cc:867-892)
+  const bool k_minor = dn.rhs_contracting_dimensions_size() == 1 && dn.rhs_contracting_dimensions(0) == rank - 1;
+  if (!MatchQWeights(dot->mutable_operand(1), k_minor, &q, &why)) {
     if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
     return false;
   }
@@ -551,17 +565,15 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   Instr* inner;
   if (ConvertFrom(lhs, BF16, &inner) && Ty(lhs) == F32) lhs = inner;
   if (Ty(lhs) != BF16) return refuse("the activation must be bf16 (or its convert to f32)");
-  const int64_t rank = Rank(dot);
   if (rank != 2 && rank != 3) return refuse("rank " + std::to_string(rank));
-  const DotDimensionNumbers& dn = dot->dot_dimension_numbers();
   auto is0 = [](const auto& d) { return d.size() == 1 && d[0] == 0; };
   if (rank == 3 && (!is0(dn.lhs_batch_dimensions()) || !is0(dn.rhs_batch_dimensions())))
     return refuse("the batch dimension must be dimension 0 of both operands");
   if (rank == 2 && dn.lhs_batch_dimensions_size() != 0) return refuse("unexpected batch dimensions");
   if (dn.lhs_contracting_dimensions_size() != 1 || dn.rhs_contracting_dimensions_size() != 1 ||
-      dn.lhs_contracting_dimensions(0) != rank - 1 || dn.rhs_contracting_dimensions(0) != rank - 2)
-    return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] contracting K (N minor); s4 with a "
-                  "minor contracting or batch dimension is rejected as in gemm_fusion.cc:1572-1590");
+      dn.lhs_contracting_dimensions(0) != rank - 1 || (dn.rhs_contracting_dimensions(0) != rank - 2 && !k_minor))
+    return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] or [..,N,K]; s4 with a "
+                  "minor batch dimension is rejected as in gemm_fusion.cc:1572-1590");
   const bool four_bit = Ty(q.w) == S4 || Ty(q.w) == U4;
   if (four_bit && q.w->shape().dimensions(rank - 1) % 2 != 0)
     return refuse("s4 rows must hold an even number of values");
@@ -574,23 +586,24 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
 
   const int64_t B = rank == 3 ? lhs->shape().dimensions(0) : 1;
   const int64_t M = lhs->shape().dimensions(rank - 2), K = lhs->shape().dimensions(rank - 1);
-  const int64_t N = q.w->shape().dimensions(rank - 1);
+  const int64_t N = q.w->shape().dimensions(rank - (k_minor ? 2 : 1));
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
   std::vector<Shape> results = {ShapeUtil::MakeShape(BF16, Dims(dot))};
-  if (size_t ws = xla_amd_dequant_dot_workspace_bytes(B, M, K, N, (int32_t)Ty(q.w)))
+  if (size_t ws = k_minor ? xla_amd_dequant_dot_workspace_bytes_nk(B, M, K, N, (int32_t)Ty(q.w))
+                          : xla_amd_dequant_dot_workspace_bytes(B, M, K, N, (int32_t)Ty(q.w)))
     results.push_back(ShapeUtil::MakeShape(S8, {(int64_t)ws}));
-  // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are [K/g,N]
-  const int64_t group_size = rank == 2 && Rank(q.scale) == 2   ? K / q.scale->shape().dimensions(0)
-                             : rank == 3 && Rank(q.scale) == 3 ? K / q.scale->shape().dimensions(1)
-                                                               : 0;
+  // rows of K per scale: 0 = one scale per output channel ([N] or [B,N]); grouped scales are
+  // [K/g,N], or [N,K/g] next to weights [N,K]
+  const int64_t group_size = q.groups ? K / q.groups : 0;
   Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, results,
-                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64"));
+                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64") +
+                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0) : call;
   CHECK_OK(ep.tail->ReplaceAllUsesWith(value));
   VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
-          << (q.zero ? " with zero points" : "") << "]";
+          << (q.zero ? " with zero points" : "") << (k_minor ? ", weights [N,K]" : "") << "]";
   return true;
 }
 
@@ -600,7 +613,7 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
 bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::function<void(std::string)>& log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->mutable_operand(1), &q, &why)) {
+  if (!MatchQWeights(dot->mutable_operand(1), /*k_minor=*/false, &q, &why)) {
     if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
     return false;
   }

@@ -57,19 +57,21 @@ def _scratch(nbytes, device):
 
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
-                scale_group_size=None, zero_points=None, group_sizes=None, out=None, scratch="auto",
-                build_only=False):
+                scale_group_size=None, zero_points=None, group_sizes=None, rhs_contracting_dim=0, out=None,
+                scratch="auto", build_only=False):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
     scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
     the handler reads the grouping off the scales' shape.
     weight_dtype "u4": unsigned 4-bit weights, packed like s4; zero_points (uint8, packed u4, one per
     scale) then makes the dequantised weight (w - zero_point) * scale.
     group_sizes (int32 or int64 [G], on the device): ragged dot -- lhs [M,K] with its rows sorted by
-    group, weights [G,K,N]; group g multiplies rows [sum(sizes[:g]), +sizes[g]) with weights[g]."""
+    group, weights [G,K,N]; group g multiplies rows [sum(sizes[:g]), +sizes[g]) with weights[g].
+    rhs_contracting_dim=1: weights [N,K] or [B,N,K] (4-bit values packed along K), scales [N], [B,N],
+    [N,K/g] or [B,N,K/g]; scale_group_size is then required."""
     _check_cuda(lhs, weights, scales, bias, zero_points, group_sizes)
     wdt = {"s4": dtypes.S4, "u4": dtypes.U4}.get(weight_dtype, dtypes.S8)
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
-    n = wshape[-1]
+    n = wshape[-2] if rhs_contracting_dim == 1 else wshape[-1]
     oshape = list(lhs.shape[:-1]) + [n]
     if out is None:
         out = torch.empty(oshape, dtype=torch.bfloat16, device=lhs.device)
@@ -85,7 +87,9 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
                      group_sizes.shape))
     rets = [(dtypes.BF16, out.data_ptr(), oshape)]
     if scratch == "auto":
-        nbytes = ffi.library().xla_amd_dequant_dot_workspace_bytes(batch, lhs.shape[-2], lhs.shape[-1], n, wdt)
+        sizer = (ffi.library().xla_amd_dequant_dot_workspace_bytes_nk if rhs_contracting_dim == 1
+                 else ffi.library().xla_amd_dequant_dot_workspace_bytes)
+        nbytes = sizer(batch, lhs.shape[-2], lhs.shape[-1], n, wdt)
         scratch = _scratch(nbytes, lhs.device)
     if scratch is not None:
         rets.append((dtypes.U8, scratch.data_ptr(), [scratch.numel()]))
@@ -94,6 +98,8 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
              "epilogue_type": ffi.Attr.i32(_TYPE_ATTR[epilogue_type])}
     if scale_group_size is not None:
         attrs["scale_group_size"] = ffi.Attr.i64(scale_group_size)
+    if rhs_contracting_dim != 0:
+        attrs["rhs_contracting_dim"] = ffi.Attr.i64(rhs_contracting_dim)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
                 keep=(lhs, weights, scales, bias, scratch, zero_points, group_sizes))
     return call if build_only else call.run()

@@ -102,6 +102,29 @@ def batched_s4_group(B=4, M=8, K=1024, N=512, group=128):
                 algorithmic_flops=2 * B * M * K * N)
 
 
+def k_minor(w):
+    """The same dequantize-dot with its weights stored [N,K] (or [B,N,K]) -- the contracting dimension
+    minor -- and scales / zero points [N,K/group] (per-channel scales stay [N] / [B,N]).  4-bit values are
+    re-packed along K.  Returns a copy of the workload with `rhs_contracting_dim` = 1; the values of the
+    dot are those of `w`."""
+    v = dict(w)
+    wt = np.ascontiguousarray(np.swapaxes(w["weights"], -1, -2))
+    v["weights"] = wt
+    v["weight_shape"] = tuple(wt.shape)
+    K = w["lhs"].shape[-1]
+    pack = lambda x: (x.reshape(-1)[0::2] | (x.reshape(-1)[1::2] << 4)).astype(np.uint8)
+    if w["weight_dtype"] in ("s4", "u4"):
+        v["weights_packed"] = pack(wt.astype(np.int8).view(np.uint8) & 0xF)
+    if w["group"] != K:
+        v["scales"] = np.ascontiguousarray(np.swapaxes(w["scales"], -1, -2))
+        if w.get("zero_points") is not None:
+            z = np.ascontiguousarray(np.swapaxes(w["zero_points"], -1, -2))
+            v["zero_points"] = z
+            v["zero_points_packed"] = pack(z)
+    v["rhs_contracting_dim"] = 1
+    return v
+
+
 def c3_fp8(M=8192, K=8192, N=8192):
     """f8 A[M,K] . f8 B[K,N], per-tensor f32 scales 1/64, + bias, GELU(tanh) -> bf16."""
     def f8(seed, shape):
