@@ -202,3 +202,53 @@ def test_bad_arguments():
     gs = torch.tensor([4], dtype=torch.int32, device="cuda")
     with pytest.raises(ffi.FfiError, match="a ragged dot takes weights"):
         ops.dequant_dot(lhs, wt.reshape(1, 32, 64), sc, group_sizes=gs, rhs_contracting_dim=1, scale_group_size=0)
+
+
+# ---- more than 64 tokens: the tiled kernel with the [N,K] loaders ----------------------------
+
+@pytest.mark.parametrize("kind,M,K,N,group", [("s8", 300, 1024, 520, 0), ("s8", 65, 4096, 264, 0), ("s4", 300, 1024, 520, 128),
+                                              ("s4", 129, 2048, 1000, 32), ("s4", 256, 1024, 256, 1024)])
+def test_tiled_kernel_takes_k_minor_weights(oracle, kind, M, K, N, group):
+    say("dequant_dot [N,K] tiled %s M=%d K=%d N=%d group=%d" % (kind, M, K, N, group))
+    w = (workloads.c1_s8_channel(M=M, K=K, N=N) if kind == "s8" else workloads.c2_s4_group(M=M, K=K, N=N, group=group))
+    got, kern = run_nk(w, force_kernel=3)
+    assert kern.startswith("dequant_dot_tiled_nk_%s_" % kind), kern
+    compare(oracle, w, got, "[N,K] tiled %s" % kern)
+
+
+def test_tiled_k_minor_batched_and_split_last_round(oracle):
+    say("dequant_dot [B,N,K] tiled s8, tiles split along K")
+    w = workloads.c5_s8_batched(B=2, M=300, K=2048, N=520)
+    got, kern = run_nk(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_nk_s8_factored:tail2", kern   # 2 x 2 x 3 tiles: all of them as pairs
+    compare(oracle, w, got, "[B,N,K] tiled s8 split")
+    got2, kern2 = run_nk(w, force_kernel=3, scratch=None)
+    assert kern2 == "dequant_dot_tiled_nk_s8_factored", kern2
+    compare(oracle, w, got2, "[B,N,K] tiled s8 whole")
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4"])
+def test_tiled_k_minor_one_hot(oracle, kind):
+    say("dequant_dot [N,K] tiled one-hot %s" % kind)
+    K, N, M = 512, 264, 192
+    w = workloads.c1_s8_channel(M=M, K=K, N=N) if kind == "s8" else workloads.c2_s4_group(M=M, K=K, N=N, group=32)
+    w["epilogue"], w["bias"] = "DEFAULT", None
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), (np.arange(M) * 37 + 5) % K] = 1.0
+    w["lhs"] = dtypes.f32_to_bf16(a)
+    got, kern = run_nk(w, force_kernel=3)
+    assert kern.startswith("dequant_dot_tiled_nk_"), kern
+    from tests.test_gpu_dequant_dot import oracle_dot
+    assert np.array_equal(got, oracle_dot(oracle, w)), kern
+
+
+def test_large_prefill_picks_the_tiled_kernel_by_itself(oracle):
+    say("dequant_dot [N,K] s8 1024 tokens: routing")
+    w = workloads.c1_s8_channel(M=1024, K=1024, N=4096)
+    got, kern = run_nk(w)
+    assert kern.startswith("dequant_dot_tiled_nk_s8_factored"), kern
+    sub = dict(w, lhs=w["lhs"][:64], )
+    # the oracle on a block of rows and channels
+    rows, cols = slice(512, 560), slice(1000, 1256)
+    blk = dict(w, lhs=w["lhs"][rows], weights=w["weights"][:, cols], scales=w["scales"][cols], weight_shape=(1024, 256))
+    compare(oracle, blk, got[rows, cols], "[N,K] tiled s8 block")

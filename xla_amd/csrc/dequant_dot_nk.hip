@@ -405,8 +405,16 @@ NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, in
 
 }  // namespace
 
+int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream);  // tiled_dot_mfma.hip
+
 size_t DequantDotNkWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit) {
   if (batch <= 0 || M <= 0 || K <= 0 || N <= 0) return 0;
+  // more than 64 tokens may run on the tiled kernel, which splits the tiles of a short last round
+  if (M > 64) {
+    const size_t tail = TiledTailWorkspaceBytes(batch, M, K, N);
+    const size_t slices = DequantDotWorkspaceBytes(batch, M, N, PlanNk(batch, M, K, N, four_bit, 0).slices);
+    return tail > slices ? tail : slices;
+  }
   // (the group is not known here: a slice of whole 128-k steps holds whole groups only when the
   // group divides it, which the launch checks again; sizing assumes the most slices)
   const NkShape s = PlanNk(batch, M, K, N, four_bit, 0);
@@ -427,6 +435,10 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
   int group_shift = -1;
   for (int s = 0; s < 31; ++s)
     if ((int64_t)1 << s == p.group) group_shift = s;
+  if (p.M > 64 && GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
+    const int rc = LaunchDequantDotPrefillNk(p, stream);
+    if (rc >= 0) return rc;  // -1: the tiled kernel does not take it (or token chunks are cheaper)
+  }
   bool fast = row_bytes % 16 == 0 && p.K >= 4 * kp && ((uintptr_t)p.lhs % 16 == 0) && ((uintptr_t)p.weights % 16 == 0) &&
               (double)p.N * row_bytes < 2147483648.0 && (double)p.M * p.K * 2 < 2147483648.0 &&
               p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1;

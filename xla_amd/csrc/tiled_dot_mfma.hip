@@ -4,6 +4,7 @@
 //   kS8  : out[b,m,n] = epi( scale[b,n] * sum_k A[b,m,k] * W[b,k,n] )    bf16 x s8 (per channel)
 //   kS4  : out[b,m,n] = epi( sum_k A[b,m,k] * bf16(W[b,k,n] * scale[b,k/g,n]) )   bf16 x s4, bf16 scales per
 //          group of g rows, every dequantised weight rounded once (the bf16-typed multiply)
+//   kS8NK, kS4NK : the same two with the weights stored [b,n,k] (K minor; scales [b,n] / [b,n,k/g])
 //
 // A workgroup of 8 waves (2x4, two per SIMD) owns a 256x256 output tile, each wave a 128x64
 // part held in 128 accumulator registers, and walks K in stages of 128 bytes per activation
@@ -41,7 +42,9 @@ namespace {
 // 32 elements of K on both operands (MXFP8), multiplied in by the matrix cores themselves
 // kBf16: both operands bf16 with K minor, a [M,K] and b [N,K] -- the f8 operands of a dot whose
 // dequantise multiply is bf16-typed, already scaled and rounded by a pre-pass
-enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4, kBf16 = 5 };
+// kS8NK, kS4NK: integer weights stored [N,K]: a thread fetches 32 consecutive k of one channel and
+// writes them, dequantised, as four chunks of that channel's LDS row
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4, kBf16 = 5, kS8NK = 6, kS4NK = 7 };
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
@@ -232,7 +235,9 @@ __device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, 
 
 template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
-  constexpr bool WQ = KIND == kS8 || KIND == kS4;  // integer weights [K,N], dequantised on the way into LDS
+  constexpr bool WQ = KIND == kS8 || KIND == kS4 || KIND == kS8NK || KIND == kS4NK;  // integer weights, dequantised on the way into LDS
+  constexpr bool W4 = KIND == kS4 || KIND == kS4NK;   // two weights per byte, bf16 group scales
+  constexpr bool W8 = KIND == kS8 || KIND == kS8NK;   // one scale per channel, applied to the sums
   constexpr bool BB = KIND == kBf16;     // both operands bf16, K minor
   constexpr bool F8 = !WQ && !BB;        // both operands f8e4m3fn
   constexpr bool BKN = KIND == kFp8KN;   // weight tile staged K-major and transposed on the way out of LDS
@@ -325,7 +330,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const uint32_t a_pitch = (uint32_t)p.K * ESZ;
   const __amdgpu_buffer_rsrc_t ra =
       tile_rsrc(p.a + (size_t)a_batch * p.M * a_pitch, (uint32_t)p.M * a_pitch);
-  const uint32_t b_bytes = KIND == kS4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N * (BB ? 2u : 1u);
+  const uint32_t b_bytes = W4 ? (uint32_t)(((size_t)p.K * p.N) >> 1) : (uint32_t)p.K * (uint32_t)p.N * (BB ? 2u : 1u);
   const __amdgpu_buffer_rsrc_t rb = tile_rsrc(p.b + (size_t)batch * b_bytes, b_bytes);  // bytes, either layout
 
   // kFp8MX: scales [rows, K/32]; lane l of wave w owns tile row (w & 3) * 64 + l of its operand
@@ -395,9 +400,9 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const int q_kblk = lane >> 3, q_oct = (wave & 3) * 8 + (lane & 7), q_half = wave >> 2;
   const uint32_t s4_pitch = (uint32_t)p.N >> 1;
   const __amdgpu_buffer_rsrc_t rsc4 =
-      tile_rsrc(KIND == kS4 ? (const uint8_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * p.N * 2
-                            : p.a,
-                KIND == kS4 ? (uint32_t)(p.K >> p.group_shift) * (uint32_t)p.N * 2u : 0u);
+      tile_rsrc(W4 ? (const uint8_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * p.N * 2
+                   : p.a,
+                W4 ? (uint32_t)(p.K >> p.group_shift) * (uint32_t)p.N * 2u : 0u);
   auto s4_load = [&](int k0) {
     const uint32_t col = (uint32_t)(n0 + q_oct * 8);
     const uint32_t kfirst = (uint32_t)(k0 + q_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
@@ -439,9 +444,69 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
   };
+  // ---- weights stored [N,K]: thread t takes channel t >> 1 and the half t & 1 of the stage's 64 k:
+  // 32 bytes of s8 or 16 bytes of s4, both contiguous, that become chunks 4 * half ... + 3 of the
+  // channel's LDS row (K % 32 == 0 for s4 and % 16 for s8: a 16-byte piece lies inside its row or past it)
+  const int nk_n = tid >> 1, nk_half = tid & 1;
+  uint32_t nk_scale = 0;
+  auto nk_load = [&](int k0) {
+    const uint32_t ch = (uint32_t)(n0 + nk_n);
+    const uint32_t k = (uint32_t)(k0 + nk_half * 32);
+    if constexpr (KIND == kS8NK) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const bool live = ch < (uint32_t)p.N && k + 16 * j < (uint32_t)p.K;
+        const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? ch * (uint32_t)p.K + k + 16 * j : kOutOfRange, 0, 0);
+        wreg[4 * j] = v[0]; wreg[4 * j + 1] = v[1]; wreg[4 * j + 2] = v[2]; wreg[4 * j + 3] = v[3];
+      }
+    } else {
+      const bool live = ch < (uint32_t)p.N && k < (uint32_t)p.K;
+      const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? (ch * (uint32_t)p.K + k) >> 1 : kOutOfRange, 0, 0);
+      wreg[0] = v[0]; wreg[1] = v[1]; wreg[2] = v[2]; wreg[3] = v[3];
+      // the lane's 32 k share a scale (groups of at least 32, or one scale per channel: shift 31)
+      nk_scale = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(
+          rsc4, live ? (ch * (uint32_t)(p.K >> p.group_shift) + (k >> p.group_shift)) * 2u : kOutOfRange, 0, 0);
+    }
+  };
+  auto nk_store = [&](uint8_t* bt) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float f[8];
+      if constexpr (KIND == kS8NK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          f[e] = (float)(int8_t)((wreg[2 * c] >> (8 * e)) & 0xffu);
+          f[4 + e] = (float)(int8_t)((wreg[2 * c + 1] >> (8 * e)) & 0xffu);
+        }
+      } else {
+        typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+        // nibble pairs (0,4), (1,5) of x and (2,6), (3,7) of x >> 8 as f16 1024 + u or 1024 + 16 u,
+        // u = w + 8; one fma each takes the offset out and the scale in: see dequant_dot_decode.hip
+        const uint32_t x = wreg[c];
+        const float v = bf16lo_to_f32(nk_scale);
+        const float s_even = v, c_even = v * -1032.0f, s_odd = v * 0.0625f, c_odd = v * -72.0f;
+        const halfx2 p04 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+        const halfx2 p15 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a));
+        const halfx2 p26 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x >> 8, 0x000f000fu, 0x64086408u, 0x6a));
+        const halfx2 p37 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x >> 8, 0x00f000f0u, 0x64806480u, 0x6a));
+        f[0] = __builtin_fmaf((float)p04[0], s_even, c_even);
+        f[1] = __builtin_fmaf((float)p15[0], s_odd, c_odd);
+        f[2] = __builtin_fmaf((float)p26[0], s_even, c_even);
+        f[3] = __builtin_fmaf((float)p37[0], s_odd, c_odd);
+        f[4] = __builtin_fmaf((float)p04[1], s_even, c_even);
+        f[5] = __builtin_fmaf((float)p15[1], s_odd, c_odd);
+        f[6] = __builtin_fmaf((float)p26[1], s_even, c_even);
+        f[7] = __builtin_fmaf((float)p37[1], s_odd, c_odd);
+      }
+      const uintx4 o = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                        pack_bf16x2(f[6], f[7])};
+      *reinterpret_cast<uintx4*>(bt + nk_n * kRow + (((nk_half * 4 + c) ^ ((nk_n >> 1) & 7)) << 4)) = o;
+    }
+  };
   auto wq_store = [&](uint8_t* bt) {
     if constexpr (KIND == kS8) s8_store(bt);
     if constexpr (KIND == kS4) s4_store(bt);
+    if constexpr (KIND == kS8NK || KIND == kS4NK) nk_store(bt);
   };
 
   auto issue_loads = [&](int buf, int k0) {
@@ -462,6 +527,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     }
     if (KIND == kS8) s8_load(k0);
     if (KIND == kS4) s4_load(k0);
+    if (KIND == kS8NK || KIND == kS4NK) nk_load(k0);
     if (MX) {
       // the stage's four scale bytes of every tile row, one dword per row: waves 0-3 fetch the
       // 256 token rows, waves 4-7 the 256 channel rows (64 lanes x 4 bytes land contiguously)
@@ -681,7 +747,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const bool ok = n + t < p.N;
     d.sc[t] = alpha;
     if (F8 && !MX && p.b_per_channel) d.sc[t] = alpha * p.b_scale[ok ? n + t : 0];
-    if (KIND == kS8) {
+    if (W8) {
       const size_t si = (size_t)(p.scale_batched ? batch : 0) * p.N + (ok ? n + t : 0);
       d.sc[t] = p.scale_is_bf16 ? bf16_to_f32(((const uint16_t*)p.scales)[si]) : ((const float*)p.scales)[si];
     }
@@ -1054,6 +1120,62 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   }
   SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_s8_factored:tail2" : "dequant_dot_tiled_s8_factored");
   return launch_tiled<kS8>(tp, (int)p.batch, stream, "dequant_dot_tiled_s8");
+}
+
+// The same for weights stored [batch,N,K] (scales [batch,N] or [batch,N,K/group]): s8 with one scale per
+// channel under an f32-typed multiply, s4 with bf16 scales per power-of-two group of at least 32 under
+// a bf16-typed one.  -1: not taken (the token-chunked streaming kernel runs instead).
+int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream) {
+  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4 && p.dequant_type == XLA_FFI_DataType_BF16 &&
+                  p.scale_dtype == XLA_FFI_DataType_BF16 && p.group >= 32 && (p.group & (p.group - 1)) == 0 &&
+                  p.K % 32 == 0 && (double)(p.K / p.group) * p.N * 2 < 2147483000.0;
+  const bool s8 = p.weight_dtype == XLA_FFI_DataType_S8 && p.group == p.K && p.dequant_type == XLA_FFI_DataType_F32 &&
+                  p.K % 16 == 0;
+  if ((!s4 && !s8) || p.group_sizes || p.zero_points) return -1;
+  if (GetOption("dequant_dot_kernel") != 3) {
+    // token chunks of the streaming kernel against rounds of 256 tiles, in microseconds fitted on MI355X
+    // (s4 8192 x 28672: 75 per 64-token pass; s8 4096 x 14336: 25)
+    const double passes = (double)p.batch * (double)((p.M + 63) / 64);
+    const double decode_us = passes * (6.0 + (double)p.K * (double)p.N * (s4 ? 3.0e-7 : 3.3e-7));
+    const double tiles = (double)p.batch * (double)((p.M + kTM - 1) / kTM) * (double)((p.N + kTN - 1) / kTN);
+    const double rounds = (double)(int64_t)((tiles + 255.0) / 256.0);
+    if (decode_us <= rounds * (10.0 + (double)p.K * 0.035)) return -1;
+  }
+  if (p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 16) || ((uintptr_t)p.scales % 2)) return -1;
+  if ((double)p.M * p.K * 2 >= 2147483000.0 || (double)p.K * p.N >= 2147483000.0) return -1;
+  TiledParams tp{};
+  tp.a = (const uint8_t*)p.lhs;
+  tp.b = (const uint8_t*)p.weights;
+  tp.scales = p.scales;
+  tp.bias = (p.epilogue & 1) ? p.bias : nullptr;
+  tp.out = (uint16_t*)p.out;
+  tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
+  tp.scale_is_bf16 = p.scale_dtype == XLA_FFI_DataType_BF16;
+  tp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
+  tp.scale_batched = p.scale_batch == p.batch && p.batch > 1;
+  tp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
+  tp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
+  tp.epilogue = p.epilogue;
+  tp.tiles_m = (tp.M + kTM - 1) / kTM;
+  tp.tiles_n = (tp.N + kTN - 1) / kTN;
+  tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
+  if (s4) tp.group_shift = __builtin_ctzll((unsigned long long)p.group);  // sizes the scales' descriptor
+  const size_t need = TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
+  if (need && GetOption("tiled_tail") != 1 && p.workspace && ((uintptr_t)p.workspace % 16) == 0 &&
+      p.workspace_bytes >= need) {
+    const int64_t tiles = p.batch * (int64_t)tp.tiles_m * tp.tiles_n;
+    tp.tail_tiles = (int)(tiles % 256);
+    tp.tail_first = (int)(tiles - tp.tail_tiles);
+    tp.tail_sums = (float*)p.workspace;
+    tp.tail_flags = (unsigned long long*)((char*)p.workspace + (size_t)tp.tail_tiles * kTailSumsBytes);
+    tp.epoch = NextHandOverEpoch();
+  }
+  if (s4) {
+    SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_nk_s4_rounded:tail2" : "dequant_dot_tiled_nk_s4_rounded");
+    return launch_tiled<kS4NK>(tp, (int)p.batch, stream, "dequant_dot_tiled_nk_s4");
+  }
+  SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_nk_s8_factored:tail2" : "dequant_dot_tiled_nk_s8_factored");
+  return launch_tiled<kS8NK>(tp, (int)p.batch, stream, "dequant_dot_tiled_nk_s8");
 }
 
 namespace {
