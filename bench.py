@@ -276,7 +276,24 @@ def main():
               ops.dequant_dot(a5r, w5, s5, scale_group_size=0, group_sizes=gsz5, build_only=True),
               8 * (4096 * 14336 + 14336 * 4) + 4096 * 4096 * 2 + 4096 * 14336 * 2,
               2 * 4096 * 4096 * 14336, "mfma", "bf16")
-        del a5, w5, a5r
+        # weights stored [N,K] (the contracting dimension minor, rhs_contracting_dim = 1; informational):
+        # C5's experts through the tiled kernel's [N,K] loader, C2's matrix at 8 tokens through the
+        # streaming kernel that takes K-minor rows as matrix operands
+        w5t = w5.transpose(1, 2).contiguous()
+        del w5, a5r
+        entry("C5 k-minor", "C5 with the weights stored [8,14336,4096]",
+              ops.dequant_dot(a5, w5t, s5, scale_group_size=0, rhs_contracting_dim=1, build_only=True),
+              8 * (4096 * 14336 + 512 * 4096 * 2 + 14336 * 4 + 512 * 14336 * 2),
+              2 * 8 * 512 * 4096 * 14336, "mfma", "bf16")
+        del a5, w5t
+        w2t = torch.randint(0, 256, (N2, K2 // 2), dtype=torch.uint8, device=dev)
+        s2t = torch.empty((N2, K2 // GROUP2), device=dev).uniform_(1e-3, 2e-2).to(torch.bfloat16)
+        lhs8 = torch.randn((8, K2), device=dev).to(torch.bfloat16)
+        entry("C2 k-minor", "C2 at 8 tokens with the weights stored [28672,8192], scales [28672,64]",
+              ops.dequant_dot(lhs8, w2t, s2t, bias, weight_dtype="s4", weight_shape=(N2, K2), epilogue="BIAS_SILU",
+                              dequant_type="bf16", scale_group_size=GROUP2, rhs_contracting_dim=1, build_only=True),
+              c2_bytes(8), 2 * 8 * K2 * N2, "hbm")
+        del w2t, s2t, lhs8
 
     # ---- CPU baselines: the oracle on the same workload, or on a stated sample of it ------------
     cpu = None
@@ -309,6 +326,8 @@ def main():
             return {"value": value, "unit": unit, "cores": cores, "kind": "port", "sample": sample}
 
         by_key = {e["key"]: e for e in other}
+        if "C2 k-minor" in by_key:   # the same arithmetic on re-laid-out weights
+            by_key["C2 k-minor"]["cpu_baseline"] = base(cpu["value"], "GB/s", "as C2 (the oracle reads the weights [K,N]): " + cpu["sample"])
         if "C1" in by_key:
             w = workloads.c1_s8_channel()
             t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))
@@ -344,6 +363,9 @@ def main():
             t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))
             by_key["C5"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
                                                 "1 of 8 batches, 64 of 512 tokens (full K and N), %.2f s" % t)
+            if "C5 k-minor" in by_key:   # the same arithmetic on re-laid-out weights
+                by_key["C5 k-minor"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
+                                                            "as C5 (the oracle reads the weights [K,N]), %.2f s" % t)
             if "ragged prefill" in by_key:   # the same arithmetic per row and expert
                 by_key["ragged prefill"]["cpu_baseline"] = base(round(2 * 64 * 4096 * 14336 / t / 1e12, 4), "TFLOP/s",
                                                                 "64 rows of one expert (full K and N), %.2f s" % t)
