@@ -91,3 +91,23 @@ def test_static_scratch_refuses_oversized_partial_sums():
     p = _params(t, t, t, None, t, M, K, N, 128, dtypes.S4, dtypes.BF16, dtypes.BF16, "DEFAULT")
     rc = L.xla_amd_launch_dequant_dot_static_scratch(C.byref(p), torch.cuda.current_stream().cuda_stream)
     assert rc == 8 and b"static scratch holds" in L.xla_amd_last_error()
+
+
+def test_static_scratch_with_weights_stored_k_minor(oracle):
+    """Weights [N,K] (rhs_contracting_dim = 1): the K-slices of the [N,K] kernel go through the static
+    array as well, bit-identical to the workspace launcher."""
+    L = ffi.library()
+    M, K, N = 8, 4096, 512
+    c1 = workloads.c1_s8_channel(M=M, K=K, N=N)
+    v = workloads.k_minor(c1)
+    need = L.xla_amd_dequant_dot_workspace_bytes_nk(1, M, K, N, dtypes.S8)
+    assert need > 0, "few channels: K is expected to be cut into slices"
+    lhs, w, sc = dev_bf16(v["lhs"]), dev_s8(v["weights"]), dev_f32(v["scales"])
+    p = _params(lhs, w, sc, None, lhs, M, K, N, K, dtypes.S8, dtypes.F32, dtypes.F32, "DEFAULT")
+    p.rhs_contracting_dim = 1
+    got_ws, got_st = _both(p, need)
+    assert np.array_equal(got_ws, got_st)
+    ref = oracle.dequant_dot(c1["lhs"], c1["weights"], 8, c1["scales"], "f32", "f32")
+    a = np.abs(dtypes.bf16_to_f32(c1["lhs"]).astype(np.float64))
+    wd = np.abs(c1["weights"].astype(np.float64)) * c1["scales"].astype(np.float64)[None, :]
+    check_dot(got_st.reshape(M, N), ref, dot_floor(a, wd, K), "static scratch, weights [N,K]")
