@@ -104,7 +104,7 @@ def test_group_scales_f32_multiply(oracle, kind, M):
         w = workloads.u4_zero_point_group(M=M, K=2048, N=520, group=128)
         w["dequant_type"] = "f32"
     got, kern = run_nk(w)
-    assert kern.endswith("_group_factored"), kern
+    assert kern.endswith("_group_factored_zp" if kind == "u4" else "_group_factored"), kern
     compare(oracle, w, got, "[N,K] %s %s" % (kind, kern))
 
 
@@ -113,7 +113,7 @@ def test_u4_zero_points(oracle, M):
     say("dequant_dot [N,K] u4 + zero points M=%d" % M)
     w = workloads.u4_zero_point_group(M=M, K=2048, N=776, group=64)
     got, kern = run_nk(w)
-    assert kern.startswith("dequant_dot_nk_s4_m") and kern.endswith("_rounded"), kern
+    assert kern.startswith("dequant_dot_nk_s4_m") and kern.endswith("_rounded_zp"), kern
     compare(oracle, w, got, "[N,K] u4 zp M=%d" % M)
 
 

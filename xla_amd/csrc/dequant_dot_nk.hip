@@ -26,13 +26,12 @@ constexpr int kNkWaves = 4;
 struct NkParams {
   DecodeParams d;        // operands, shapes, types, slices (strips: channel strips of kNkWaves*CT*16)
   int k_per_slice;       // multiple of the step (and of the group for group-factored sums)
-  int group_shift;       // log2(group) or -1
+  int group_shift;       // log2(group); 31 for one scale per channel
   int m_chunks;          // grid.y = batch * m_chunks, chunk c takes tokens [c*16*MT, +16*MT)
 };
 
-static __device__ __forceinline__ uint32_t group_of(const NkParams& p, uint32_t k) {
-  return p.group_shift >= 0 ? k >> p.group_shift : k / (uint32_t)p.d.group;
-}
+// (scale groups are powers of two, or one per channel: shift 31)
+static __device__ __forceinline__ uint32_t group_of(const NkParams& p, uint32_t k) { return k >> p.group_shift; }
 
 // Stage geometry shared by the kernel and its launch.
 template <int WBITS, int MT>
@@ -58,7 +57,9 @@ struct NkStage {
 // matrix operands; a wave's weights (and scales) of the next stage are requested, all of them,
 // before it starts on the current one, so a whole stage of loads is in flight per wave.  One
 // barrier per stage.
-template <int WBITS, int MT, int CT, int MODE>
+// ZP: u4 weights with zero points.  The main loop has no branch: the scales of a bf16-typed multiply
+// are bf16, and scales and zero points come through buffer descriptors with 32-bit offsets.
+template <int WBITS, int MT, int CT, int MODE, bool ZP>
 __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams q) {
   const DecodeParams& p = q.d;
   using S = NkStage<WBITS, MT>;
@@ -80,11 +81,17 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
       make_rsrc(p.w + (size_t)batch * p.N * row_bytes, (uint32_t)p.N * row_bytes);
   const __amdgpu_buffer_rsrc_t ra =
       make_rsrc(p.lhs + ((size_t)batch * p.M + m0) * p.K, (uint32_t)rows_here * (uint32_t)p.K * 2u);
-  uint32_t voff_w[CT];
+  // scales of a bf16-typed multiply: bf16 [N,G]; zero points: one nibble each, same shape
+  const uint32_t sc_elems = (uint32_t)p.N * (uint32_t)G;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc((const uint16_t*)p.scales + sbatch * sc_elems, sc_elems * 2u);
+  const uint32_t zp_first = (uint32_t)(sbatch * sc_elems);  // element index of this batch's first zero point
+  const __amdgpu_buffer_rsrc_t rz = make_rsrc(ZP ? p.zero_points : p.w, ZP ? (uint32_t)(((size_t)(p.scale_batched ? gridDim.y / q.m_chunks : 1) * sc_elems + 1) >> 1) : 0u);
+  uint32_t voff_w[CT], elem_s[CT];
 #pragma unroll
   for (int t = 0; t < CT; ++t) {
     const int n = n_wave + t * 16 + c;
     voff_w[t] = n < p.N ? (uint32_t)n * row_bytes + kq * 16 : kPastEnd;
+    elem_s[t] = (uint32_t)max(0, min(n, p.N - 1)) * (uint32_t)G;
   }
 
   const int k_begin = slice * q.k_per_slice;
@@ -100,8 +107,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
     }
 
   uintx4 wq[2][SPS][CT], areg[CHUNKS];
-  float sv[2][SPS][CT], zv[2][SPS][CT];  // kRounded (and zero points): the lane's scale / zero point of the step
-  const bool has_zp = WBITS == 4 && p.zero_points != nullptr;
+  uint32_t sraw[2][SPS][CT], zraw[2][SPS][CT];  // kRounded / ZP: the lane's scale (bf16 bits) / zero point of the step
   const float z_default = WBITS == 4 ? (p.w_unsigned ? 0.0f : 8.0f) : 0.0f;
 
   // ---- the stage's activations: piece id = i * 256 + tid -> token row id / (KS/8), 8 k at (id % (KS/8)) * 8
@@ -135,14 +141,17 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
 #pragma unroll
       for (int t = 0; t < CT; ++t)
         wq[set][st][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, live ? voff_w[t] + wb : kPastEnd, 0, 0);
-      if (MODE == kRounded || has_zp) {
+      if constexpr (MODE == kRounded || ZP) {
         const uint32_t g = group_of(q, live ? kl : 0u);
 #pragma unroll
         for (int t = 0; t < CT; ++t) {
-          const int n = n_wave + t * 16 + c;
-          const size_t e = (sbatch * p.N + (size_t)max(0, min(n, p.N - 1))) * G + g;
-          sv[set][st][t] = MODE == kRounded ? load_scale(p.scales, e, p.scale_is_bf16) : 1.0f;
-          zv[set][st][t] = has_zp ? (float)((p.zero_points[e >> 1] >> (4 * (e & 1))) & 0xfu) : z_default;
+          const uint32_t e = elem_s[t] + g;
+          if constexpr (MODE == kRounded)
+            sraw[set][st][t] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, e * 2u, 0, 0);
+          if constexpr (ZP) {
+            const uint32_t ez = zp_first + e;  // nibble ez & 1 of byte ez >> 1
+            zraw[set][st][t] = ((uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(rz, ez >> 1, 0, 0)) | ((ez & 1u) << 8);
+          }
         }
       }
     }
@@ -150,8 +159,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
 
   // whether the scale group ends with the step that starts at k0 (groups are whole steps)
   auto closes_group = [&](int k0) __attribute__((always_inline)) {
-    const uint32_t e = (uint32_t)(k0 + STEP);
-    return q.group_shift >= 0 ? (e & ((uint32_t)p.group - 1u)) == 0u : e % (uint32_t)p.group == 0u;
+    return ((uint32_t)(k0 + STEP) & ((uint32_t)p.group - 1u)) == 0u;
   };
 
   auto compute = [&](int set, int st, int buf, int k0) __attribute__((always_inline)) {
@@ -180,8 +188,9 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
       // 4-bit: nibble e of a dword arrives as the f16 value 1024 + u (even e) or 1024 + 16 u (odd e);
       // (u - z) * s = (1024 + u) * s - (1024 + z) * s = (1024 + 16 u) * (s / 16) - (64 + z) * s:
       // one fma each, exact for a scale of 8 significant bits
-      const float s = (MODE == kRounded) ? sv[set][st][t] : 1.0f;
-      const float z = WBITS == 4 ? ((MODE == kRounded || has_zp) ? zv[set][st][t] : z_default) : 0.0f;
+      float s = 1.0f, z = z_default;
+      if constexpr (MODE == kRounded) s = bf16lo_to_f32(sraw[set][st][t]);
+      if constexpr (ZP) z = (float)((zraw[set][st][t] >> ((zraw[set][st][t] >> 6) & 4u)) & 0xfu);  // bit 8: the high nibble
       const float s_even = s, c_even = s * -(1024.0f + z), s_odd = s * 0.0625f, c_odd = s * -(64.0f + z);
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
@@ -343,7 +352,7 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
   p.out[(size_t)batch * total + idx] = f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
-template <int WBITS, int MT, int CT, int MODE>
+template <int WBITS, int MT, int CT, int MODE, bool ZP>
 int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name) {
   constexpr size_t kLds = 2 * (size_t)NkStage<WBITS, MT>::STAGE_BYTES;
   // per kernel instantiation and device: one bit per device ordinal (two threads that race set the
@@ -353,14 +362,14 @@ int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name
   (void)hipGetDevice(&device);
   const unsigned long long bit = 1ull << (device & 63);
   if (kLds > 48 * 1024 && !(configured.load(std::memory_order_acquire) & bit)) {
-    hipError_t e = hipFuncSetAttribute((const void*)dequant_dot_nk_kernel<WBITS, MT, CT, MODE>,
+    hipError_t e = hipFuncSetAttribute((const void*)dequant_dot_nk_kernel<WBITS, MT, CT, MODE, ZP>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
     if (e != hipSuccess)
       return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", name, kLds, hipGetErrorString(e));
     configured.fetch_or(bit, std::memory_order_release);
   }
   dim3 grid((unsigned)q.d.strips, (unsigned)(batch * q.m_chunks), (unsigned)q.d.slices);
-  hipLaunchKernelGGL((dequant_dot_nk_kernel<WBITS, MT, CT, MODE>), grid, dim3(kNkWaves * 64), kLds, stream, q);
+  hipLaunchKernelGGL((dequant_dot_nk_kernel<WBITS, MT, CT, MODE, ZP>), grid, dim3(kNkWaves * 64), kLds, stream, q);
   int rc = CheckLaunch(name);
   if (rc) return rc;
   if (q.d.slices > 1) rc = LaunchDecodeFinalize(q.d, batch, stream, MODE);
@@ -373,7 +382,7 @@ struct NkShape {
 };
 
 // Token tiles, channel tiles and K-slices for a shape the streaming kernel takes.
-NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, int64_t slice_unit) {
+NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, int64_t slice_unit, bool tuned_ct = true) {
   NkShape s;
   s.wbits = four_bit ? 4 : 8;
   s.kp = 128 / s.wbits;
@@ -383,7 +392,7 @@ NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, in
   // 8192 x 28672 s4 (1 / 2 / 4 slices: 55.6 / 48.3 / 44.1 us with one tile per wave, 78.9 / 55.2 /
   // 57.5 us with two); more token tiles: two channel tiles per wave, two workgroups per CU.
   s.ct = s.mt == 1 ? 1 : 2;
-  if (int v = GetOption("dequant_dot_nk_ct")) s.ct = s.mt != 1 ? 2 : v == 1 ? 1 : v == 4 ? 4 : 2;  // (one token tile only)
+  if (int v = tuned_ct ? GetOption("dequant_dot_nk_ct") : 0) s.ct = s.mt != 1 ? 2 : v == 1 ? 1 : v == 4 ? 4 : 2;  // (one token tile only)
   s.strips = (int)((N + kNkWaves * s.ct * 16 - 1) / (kNkWaves * s.ct * 16));
   s.m_chunks = (int)((M + 16 * s.mt - 1) / (16 * s.mt));
   // few workgroups: cut K (at most four ways) while a slice keeps eight steps (or whole groups) and
@@ -432,8 +441,8 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
                    : per_channel || p.group % (4 * kp) != 0 ? kFactored
                                                             : kGroupFactored;
   const int64_t row_bytes = p.K * wbits / 8;
-  int group_shift = -1;
-  for (int s = 0; s < 31; ++s)
+  int group_shift = per_channel ? 31 : -1;  // (k >> 31 == 0: the one scale of the channel)
+  for (int s = 0; s < 31 && !per_channel; ++s)
     if ((int64_t)1 << s == p.group) group_shift = s;
   if (p.M > 64 && GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
     const int rc = LaunchDequantDotPrefillNk(p, stream);
@@ -442,6 +451,8 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
   bool fast = row_bytes % 16 == 0 && p.K >= 4 * kp && ((uintptr_t)p.lhs % 16 == 0) && ((uintptr_t)p.weights % 16 == 0) &&
               (double)p.N * row_bytes < 2147483648.0 && (double)p.M * p.K * 2 < 2147483648.0 &&
               p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1;
+  if (group_shift < 0) fast = false;  // groups are powers of two, or one scale per channel
+  if ((double)p.scale_batch * p.N * (p.K / p.group) * 4 >= 2147483648.0) fast = false;  // 32-bit offsets into the scales
   if (mode == kRounded && !per_channel && p.group % kp != 0) fast = false;
   if (mode == kFactored && !per_channel) fast = false;  // an f32 multiply by scales that do not cover whole steps
   if (p.zero_points && !per_channel && p.group % kp != 0) fast = false;
@@ -455,7 +466,8 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
     SetLastKernel("dequant_dot_nk_generic");
     return CheckLaunch("dequant_dot_nk_generic");
   }
-  NkShape s = PlanNk(p.batch, p.M, p.K, p.N, four_bit, mode == kGroupFactored ? p.group : 0);
+  const bool zp = p.zero_points != nullptr;
+  NkShape s = PlanNk(p.batch, p.M, p.K, p.N, four_bit, mode == kGroupFactored ? p.group : 0, /*tuned_ct=*/!zp);
   if (s.slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, s.slices))) {
     s.slices = 1;
     s.k_per_slice = (int)p.K;
@@ -467,9 +479,12 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
   q.k_per_slice = s.k_per_slice;
   q.group_shift = group_shift;
   q.m_chunks = s.m_chunks;
-#define XLA_AMD_NK(WB, MT_, CT_, MODE_, NAME)                     \
-  if (wbits == WB && s.mt == MT_ && s.ct == CT_ && mode == MODE_) \
-    return launch_nk<WB, MT_, CT_, MODE_>(q, (int)p.batch, stream, NAME);
+#define XLA_AMD_NK(WB, MT_, CT_, MODE_, NAME)                                             \
+  if (wbits == WB && s.mt == MT_ && s.ct == CT_ && mode == MODE_) {                       \
+    if constexpr (WB == 4 && CT_ == (MT_ == 1 ? 1 : 2))                                   \
+      if (zp) return launch_nk<WB, MT_, CT_, MODE_, true>(q, (int)p.batch, stream, NAME "_zp"); \
+    return launch_nk<WB, MT_, CT_, MODE_, false>(q, (int)p.batch, stream, NAME);          \
+  }
 #define XLA_AMD_NK_MODES(WB, MT_, CT_, TAG)                                         \
   XLA_AMD_NK(WB, MT_, CT_, kRounded, "dequant_dot_nk_" TAG "_rounded")              \
   XLA_AMD_NK(WB, MT_, CT_, kFactored, "dequant_dot_nk_" TAG "_factored")            \
