@@ -152,8 +152,8 @@ typedef struct XlaAmdDequantDot {
   int32_t group_sizes_dtype;
   /* 0: weights [batch,K,N] as above.  1: weights [batch,N,K], the contracting dimension minor
    * (dot ... rhs_contracting_dims={1}, fusion_emitter_int4_device_test.cc:867-892): 4-bit values are
-   * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  Not with
-   * group_sizes. */
+   * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  With
+   * group_sizes the experts are [groups,N,K]. */
   int32_t rhs_contracting_dim;
 } XlaAmdDequantDot;
 

@@ -148,15 +148,16 @@ def evaluate(module_json, args):
             b_ = np.asarray(x[1], np.float32)
             sizes = [int(v) for v in np.asarray(x[2]).reshape(-1)]
             assert _dims(ins["attrs"].get("lhs_contracting_dims", "")) == [1]
-            assert _dims(ins["attrs"].get("rhs_contracting_dims", "")) == [1]
+            rc = _dims(ins["attrs"].get("rhs_contracting_dims", ""))
+            assert rc in ([1], [2])          # rhs [G,K,N], or [G,N,K] with the contracting dimension minor
             assert _dims(ins["attrs"].get("lhs_ragged_dims", "")) == [0]
             assert _dims(ins["attrs"].get("rhs_group_dims", "")) == [0]
-            r = np.zeros((a_.shape[0], b_.shape[2]), np.float32)
+            r = np.zeros((a_.shape[0], b_.shape[3 - rc[0]]), np.float32)
             start = 0
             for g, n in enumerate(sizes):
                 n = max(0, min(n, a_.shape[0] - start))
                 if n:
-                    r[start:start + n] = _dot(a_[start:start + n], b_[g], [1], [0], [], [])
+                    r[start:start + n] = _dot(a_[start:start + n], b_[g], [1], [rc[0] - 1], [], [])
                 start += n
             v = _round(r, ty)
         elif op == "negate":

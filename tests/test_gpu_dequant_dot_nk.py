@@ -199,9 +199,6 @@ def test_bad_arguments():
     sc2 = torch.ones((2, 32), dtype=torch.float32, device="cuda")
     with pytest.raises(ffi.FfiError, match=r"must be \[batch,\]N,K/scale_group_size"):
         ops.dequant_dot(lhs, wt, sc2, rhs_contracting_dim=1, scale_group_size=32)
-    gs = torch.tensor([4], dtype=torch.int32, device="cuda")
-    with pytest.raises(ffi.FfiError, match="a ragged dot takes weights"):
-        ops.dequant_dot(lhs, wt.reshape(1, 32, 64), sc, group_sizes=gs, rhs_contracting_dim=1, scale_group_size=0)
 
 
 # ---- more than 64 tokens: the tiled kernel with the [N,K] loaders ----------------------------
@@ -252,3 +249,81 @@ def test_large_prefill_picks_the_tiled_kernel_by_itself(oracle):
     rows, cols = slice(512, 560), slice(1000, 1256)
     blk = dict(w, lhs=w["lhs"][rows], weights=w["weights"][:, cols], scales=w["scales"][cols], weight_shape=(1024, 256))
     compare(oracle, blk, got[rows, cols], "[N,K] tiled s8 block")
+
+
+# ---- ragged dot over experts stored [G,N,K] ------------------------------------------------------
+
+def run_ragged_nk(w, sizes_dtype=torch.int32, force_kernel=0):
+    v = workloads.k_minor(w)
+    lhs = dev_bf16(v["lhs"])
+    wt = dev_u8(v["weights_packed"]) if v["weight_dtype"] in ("s4", "u4") else dev_s8(v["weights"])
+    sc = dev_bf16(v["scales"]) if v["scales"].dtype == np.uint16 else dev_f32(v["scales"])
+    bias = dev_bf16(v["bias"]) if v.get("bias") is not None else None
+    gs = torch.from_numpy(np.asarray(v["group_sizes"], np.int64)).to(sizes_dtype).cuda()
+    ffi.set_option("dequant_dot_kernel", force_kernel)
+    try:
+        out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=v["weight_dtype"], weight_shape=v["weight_shape"],
+                              epilogue=v["epilogue"], dequant_type=v["dequant_type"],
+                              scale_group_size=0 if v["group"] == v["lhs"].shape[-1] else v["group"], group_sizes=gs,
+                              rhs_contracting_dim=1)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("dequant_dot_kernel", 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+@pytest.mark.parametrize("M,K,N,G,sizes,sizes_dtype", [
+    (32, 1024, 512, 8, None, torch.int32), (64, 512, 384, 4, [10, 0, 50, 4], torch.int64),
+    (12, 256, 136, 3, [5, 0, 2], torch.int32), (7, 512, 128, 2, [9, 9], torch.int32),
+    (40, 512, 256, 5, [0, 0, 0, 0, 0], torch.int64), (200, 512, 264, 3, [150, 0, 30], torch.int32)])
+def test_ragged_dot_over_k_minor_experts(oracle, M, K, N, G, sizes, sizes_dtype):
+    """Rows sorted by expert, experts stored [G,N,K]: random splits with empty groups, rows that no
+    group owns (epilogue(0) = the bias), sizes that overrun M, a call whose groups are all empty, a
+    group of more rows than a token chunk."""
+    from tests.test_gpu_dequant_dot import ragged_floor
+    from tests.gpu_util import check_dot
+    say("dequant_dot ragged [G,N,K] M=%d K=%d N=%d G=%d sizes=%s" % (M, K, N, G, sizes))
+    w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+    got, kern = run_ragged_nk(w, sizes_dtype)
+    assert kern.startswith("dequant_dot_nk_s8_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged [G,N,K] %s" % kern)
+    got_g, kern_g = run_ragged_nk(w, sizes_dtype, force_kernel=1)
+    assert kern_g == "dequant_dot_nk_generic", kern_g
+    check_dot(got_g, ref, ragged_floor(w), "ragged [G,N,K] generic")
+
+
+def test_ragged_dot_k_minor_s4_group_scales(oracle):
+    from tests.gpu_util import check_dot, dot_floor
+    say("dequant_dot ragged [G,N,K] s4 group scales")
+    w = workloads.ragged_s4_group_experts(M=48, K=1024, N=264, groups=4, group=128, sizes=[20, 0, 17, 5])
+    got, kern = run_ragged_nk(w)
+    assert kern.startswith("dequant_dot_nk_s4_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                    bias=w.get("bias"), group=128)
+    a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
+    wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+    check_dot(got, ref, dot_floor(a, wd, 1024), "ragged [G,N,K] s4 %s" % kern)
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4"])
+def test_ragged_dot_k_minor_grouped_gemm(oracle, kind):
+    """Groups of hundreds of rows: the tiled kernel as a grouped GEMM over [G,N,K] experts."""
+    from tests.gpu_util import check_dot, dot_floor
+    say("dequant_dot ragged [G,N,K] tiled %s" % kind)
+    sizes = [300, 0, 257, 100]
+    if kind == "s8":
+        w = workloads.ragged_s8_experts(M=700, K=512, N=264, groups=4, sizes=sizes)
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+        wd = np.max(np.abs(w["weights"].astype(np.float64)) * w["scales"].astype(np.float64)[:, None, :], axis=0)
+    else:
+        w = workloads.ragged_s4_group_experts(M=700, K=512, N=264, groups=4, group=128, sizes=sizes)
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                        bias=w.get("bias"), group=128)
+        wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                    np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+    got, kern = run_ragged_nk(w)
+    assert kern.startswith("dequant_dot_tiled_nk_%s_" % kind) and kern.endswith(":ragged"), kern
+    a = np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64))
+    check_dot(got, ref, dot_floor(a, wd, 512), "ragged [G,N,K] tiled %s" % kind)

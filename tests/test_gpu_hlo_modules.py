@@ -249,6 +249,32 @@ def test_ragged_experts_modules(M):
         check_dot(host_bf16(out), ref, fl, "ragged %s module M=%d" % (kind, M))
 
 
+@pytest.mark.parametrize("kind", ["s8", "s4"])
+def test_k_minor_ragged_experts_modules(kind):
+    """ragged-dot modules over experts stored [G,N,K] through the pass and the registry."""
+    say("module ragged experts stored [G,N,K]: %s" % kind)
+    M, K, N, G = 40, 512, 264, 4
+    if kind == "s8":
+        v = workloads.k_minor(workloads.ragged_s8_experts(M, K, N, G))
+        text = hm.k_minor_ragged_s8_experts(M, K, N, G)
+        ops_in = [dev_bf16(v["lhs"]), dev_s8(v["weights"]), dev_f32(v["scales"]), dev_bf16(v["bias"])]
+        wd = np.max(np.abs(v["weights"].astype(np.float64)) * v["scales"].astype(np.float64)[:, :, None], axis=0)
+    else:
+        v = workloads.k_minor(workloads.ragged_s4_group_experts(M, K, N, G, 128))
+        text = hm.k_minor_ragged_s4_group_experts(M, K, N, G, 128)
+        ops_in = [dev_bf16(v["lhs"]), dev_u8(v["weights_packed"]), dev_bf16(v["scales"]), dev_bf16(v["bias"])]
+        wd = np.max(np.abs(v["weights"].astype(np.float64)) *
+                    np.repeat(dtypes.bf16_to_f32(v["scales"]).astype(np.float64), 128, axis=2), axis=0)
+    sizes = torch.from_numpy(v["group_sizes"].astype(np.int32)).cuda()
+    out, rw, _ = hlo_runner.compile_and_run(text, ops_in + [sizes])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, %s, ragged over 4 groups, weights [G,N,K]]" % kind], rw
+    assert ffi.last_kernel().startswith("dequant_dot_nk_"), ffi.last_kernel()
+    ref = reference(text, [v["lhs"], v["weights"], v["scales"], v["bias"], v["group_sizes"]])
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(v["lhs"]).astype(np.float64)), wd.T, K)
+    check_dot(host_bf16(out), ref, fl, "ragged [G,N,K] %s module" % kind)
+
+
 def test_batched_s4_group_module():
     say("module batched s4 group scales")
     B, M, K, N = 3, 8, 512, 256

@@ -200,3 +200,24 @@ def test_weights_with_the_contracting_dimension_minor(oracle, kind):
         got = run_module(hm.k_minor_s8_batched(2, 4, 64, 24), [v["lhs"], v["weights"], v["scales"]])
         ref = oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32")
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("kind", ["s8", "s4"])
+def test_ragged_dot_over_k_minor_experts(oracle, kind):
+    """Experts stored [G,N,K] (rhs_contracting_dims = {2}): the module op by op on the re-laid-out arrays
+    gives the bits of the oracle's composition of per-group calls on the [G,K,N] arrays."""
+    sizes = [5, 0, 6, 1]
+    if kind == "s8":
+        w = workloads.ragged_s8_experts(M=12, K=64, N=24, groups=4, sizes=sizes)
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_ragged_s8_experts(12, 64, 24, 4),
+                         [v["lhs"], v["weights"], v["scales"], v["bias"], v["group_sizes"]])
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    else:
+        w = workloads.ragged_s4_group_experts(M=12, K=64, N=24, groups=4, group=32, sizes=sizes)
+        v = workloads.k_minor(w)
+        got = run_module(hm.k_minor_ragged_s4_group_experts(12, 64, 24, 4, 32),
+                         [v["lhs"], v["weights"], v["scales"], v["bias"], v["group_sizes"]])
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                        bias=w["bias"], group=32)
+    assert np.array_equal(got, ref)

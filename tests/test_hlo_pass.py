@@ -592,3 +592,20 @@ def test_weights_with_the_contracting_dimension_minor():
     assert hlo.rewrite(bad)[1] == []
     # the [K,N] spelling keeps its attributes (no rhs_contracting_dim)
     assert "rhs_contracting_dim" not in hlo.rewrite(hm.c1_s8_channel())[0]
+
+
+def test_ragged_dot_over_k_minor_experts():
+    """ragged-dot whose experts are stored [G,N,K] (rhs_contracting_dims = {2}): the same call with
+    rhs_contracting_dim = 1; scales [G,N] or [G,N,K/g]."""
+    new, rw, rf = hlo.rewrite(hm.k_minor_ragged_s8_experts(32, 512, 256, 4))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, s8, ragged over 4 groups, weights [G,N,K]]"] and rf == []
+    check(new, r"%w = s8\[4,256,512\] parameter\(1\)", r"custom-call\(%lhs, %w, %scale, %bias, %sizes\)",
+          r"scale_group_size = 0 : i64, rhs_contracting_dim = 1 : i64")
+    new, rw, rf = hlo.rewrite(hm.k_minor_ragged_s4_group_experts(32, 512, 256, 4, 128))
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS, s4, ragged over 4 groups, weights [G,N,K]]"] and rf == []
+    check(new, r"%scales = bf16\[4,256,4\] parameter\(2\)", r"custom-call\(%lhs, %w, %scales, %bias, %sizes\)",
+          r"scale_group_size = 128 : i64, rhs_contracting_dim = 1 : i64")
+    # the group dimension anywhere but in front is left alone, as for [G,K,N]
+    bad = hm.k_minor_ragged_s8_experts(32, 512, 256, 4).replace("rhs_group_dims={0}", "rhs_group_dims={1}")
+    _, rw, rf = hlo.rewrite(bad)
+    assert rw == [] and any("group dimension leading the weights" in r for r in rf)

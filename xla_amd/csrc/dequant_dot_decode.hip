@@ -666,8 +666,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   if (p.rhs_contracting_dim != 0 && p.rhs_contracting_dim != 1)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: rhs_contracting_dim must be 0 or 1");
   if (p.rhs_contracting_dim == 1) {  // weights [N,K]
-    if (ragged)
-      return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes weights [groups,K,N]");
+    if (ragged) dp.scale_batched = p.scale_batch == p.batch;  // one set of scales per group, also for a single group
     return LaunchDequantDotNk(dp, p, stream);
   }
   const bool per_channel = p.group == p.K;

@@ -13,6 +13,7 @@
 // slice order.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 
 #include "decode_common.h"
@@ -70,8 +71,14 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   const int c = lane & 15, kq = lane >> 4;
   const int strip = blockIdx.x, slice = blockIdx.z;
   const int batch = blockIdx.y / q.m_chunks, chunk = blockIdx.y % q.m_chunks;
+  // ragged dot: `batch` is the group, whose rows [m_first, m_first + m_rows) of the one [M,K] activation
+  // matrix are read on the device; a chunk past the end of its group has nothing to do
+  int m_first = 0, m_rows = p.M;
+  if (p.group_sizes) ragged_rows(p, batch, &m_first, &m_rows);
+  const int a_batch = p.group_sizes ? 0 : batch;
   const int m0 = chunk * 16 * MT;
-  const int rows_here = min(16 * MT, p.M - m0);
+  const int rows_here = min(16 * MT, m_rows - m0);
+  if (rows_here <= 0) return;  // (the whole workgroup, before any barrier)
   const int n_wave = (strip * kNkWaves + wave) * CT * 16;  // (a wave past N loads nothing and stores nothing)
   const int G = p.K / p.group;  // scales per channel
   const uint32_t row_bytes = (uint32_t)p.K * WBITS / 8;
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   const __amdgpu_buffer_rsrc_t rw =
       make_rsrc(p.w + (size_t)batch * p.N * row_bytes, (uint32_t)p.N * row_bytes);
   const __amdgpu_buffer_rsrc_t ra =
-      make_rsrc(p.lhs + ((size_t)batch * p.M + m0) * p.K, (uint32_t)rows_here * (uint32_t)p.K * 2u);
+      make_rsrc(p.lhs + ((size_t)a_batch * p.M + m_first + m0) * p.K, (uint32_t)rows_here * (uint32_t)p.K * 2u);
   // scales of a bf16-typed multiply: bf16 [N,G]; zero points: one nibble each, same shape
   const uint32_t sc_elems = (uint32_t)p.N * (uint32_t)G;
   const __amdgpu_buffer_rsrc_t rs = make_rsrc((const uint16_t*)p.scales + sbatch * sc_elems, sc_elems * 2u);
@@ -296,7 +303,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
       if (p.slices == 1) epilogue_all_dispatch<4>(v, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
       const int n = n_wave + t * 16 + 4 * kq, m = mt * 16 + c;
       if (m < rows_here && n < p.N) {
-        const size_t o = ((size_t)batch * p.M + m0 + m) * p.N + n;
+        const size_t o = ((size_t)a_batch * p.M + m_first + m0 + m) * p.N + n;
         if (p.slices > 1) {
           float* dst = p.workspace + ((size_t)batch * p.slices + slice) * ((size_t)p.M * p.N) + (size_t)(m0 + m) * p.N + n;
           if (quads) {
@@ -327,11 +334,21 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
   if (idx >= total) return;
   const int n = (int)(idx % p.N), m = (int)(idx / p.N);
   const int G = p.K / p.group;
+  // ragged dot (launched with one batch): the row's group picks the weights; rows no group owns add nothing
+  int wbatch = batch, k_end = p.K;
+  if (p.group_sizes) {
+    k_end = 0;
+    for (int g = 0; g < p.ragged_groups; ++g) {
+      int b0, rows;
+      ragged_rows(p, g, &b0, &rows);
+      if (m >= b0 && m < b0 + rows) { wbatch = g; k_end = p.K; break; }
+    }
+  }
   const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
-  const size_t wrow = ((size_t)batch * p.N + n) * p.K;                     // in elements
-  const size_t srow = ((size_t)(p.scale_batched ? batch : 0) * p.N + n) * G;
+  const size_t wrow = ((size_t)wbatch * p.N + n) * p.K;                     // in elements
+  const size_t srow = ((size_t)(p.scale_batched ? wbatch : 0) * p.N + n) * G;
   float acc = 0.0f;
-  for (int k = 0; k < p.K; ++k) {
+  for (int k = 0; k < k_end; ++k) {
     const size_t e = wrow + k;
     int wi;
     if (wbits == 8) {
@@ -350,6 +367,18 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
   }
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
   p.out[(size_t)batch * total + idx] = f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+}
+
+// Ragged dot: rows past the last group are a dot of nothing, epilogue(0).  Workgroup (x, y) takes 256
+// channels and every gridDim.y-th of those rows; usually there are none and it returns at once.
+__global__ __launch_bounds__(256) void nk_ragged_tail_rows_kernel(DecodeParams p) {
+  int begin, rows;
+  ragged_rows(p, p.ragged_groups - 1, &begin, &rows);
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= p.N) return;
+  const float bias = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  const uint16_t v = f32_to_bf16(epilogue_dispatch(0.0f, bias, p.epilogue, p.bf16_dot, p.bf16_ops));
+  for (int m = begin + rows + blockIdx.y; m < p.M; m += gridDim.y) p.out[(size_t)m * p.N + n] = v;
 }
 
 template <int WBITS, int MT, int CT, int MODE, bool ZP>
@@ -373,6 +402,10 @@ int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name
   int rc = CheckLaunch(name);
   if (rc) return rc;
   if (q.d.slices > 1) rc = LaunchDecodeFinalize(q.d, batch, stream, MODE);
+  if (q.d.group_sizes && rc == 0) {
+    hipLaunchKernelGGL(nk_ragged_tail_rows_kernel, dim3((unsigned)((q.d.N + 255) / 256), 16u), dim3(256), 0, stream, q.d);
+    rc = CheckLaunch("dequant_dot_nk_ragged_tail_rows");
+  }
   SetLastKernel(name);
   return rc;
 }
@@ -382,12 +415,15 @@ struct NkShape {
 };
 
 // Token tiles, channel tiles and K-slices for a shape the streaming kernel takes.
-NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, int64_t slice_unit, bool tuned_ct = true) {
+// tile_rows: the rows that decide the number of token tiles (a ragged dot: about what a group owns), 0 = M.
+NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, int64_t slice_unit, bool tuned_ct = true,
+               int64_t tile_rows = 0) {
   NkShape s;
   s.wbits = four_bit ? 4 : 8;
   s.kp = 128 / s.wbits;
   s.step = 4 * s.kp;
-  s.mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  if (tile_rows <= 0) tile_rows = M;
+  s.mt = tile_rows <= 16 ? 1 : tile_rows <= 32 ? 2 : 4;
   // One token tile: a channel tile per wave and about four workgroups per CU measured fastest on
   // 8192 x 28672 s4 (1 / 2 / 4 slices: 55.6 / 48.3 / 44.1 us with one tile per wave, 78.9 / 55.2 /
   // 57.5 us with two); more token tiles: two channel tiles per wave, two workgroups per CU.
@@ -444,13 +480,17 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
   int group_shift = per_channel ? 31 : -1;  // (k >> 31 == 0: the one scale of the channel)
   for (int s = 0; s < 31 && !per_channel; ++s)
     if ((int64_t)1 << s == p.group) group_shift = s;
-  if (p.M > 64 && GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
+  const bool ragged = p.group_sizes != nullptr;
+  // (a ragged dot takes the tiled kernel -- 256-row tiles per group -- once the groups average 96 rows)
+  if (p.M > 64 && (!ragged || GetOption("dequant_dot_kernel") == 3 || p.M / p.batch >= 96) &&
+      GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
     const int rc = LaunchDequantDotPrefillNk(p, stream);
     if (rc >= 0) return rc;  // -1: the tiled kernel does not take it (or token chunks are cheaper)
   }
   bool fast = row_bytes % 16 == 0 && p.K >= 4 * kp && ((uintptr_t)p.lhs % 16 == 0) && ((uintptr_t)p.weights % 16 == 0) &&
               (double)p.N * row_bytes < 2147483648.0 && (double)p.M * p.K * 2 < 2147483648.0 &&
-              p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1;
+              p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1 &&
+              (!ragged || (double)p.M * p.N * 2 < 2147483648.0);
   if (group_shift < 0) fast = false;  // groups are powers of two, or one scale per channel
   if ((double)p.scale_batch * p.N * (p.K / p.group) * 4 >= 2147483648.0) fast = false;  // 32-bit offsets into the scales
   if (mode == kRounded && !per_channel && p.group % kp != 0) fast = false;
@@ -460,15 +500,18 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
     if (GetOption("dequant_dot_kernel") == 2 || GetOption("dequant_dot_kernel") == 3)
       return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION, "dequant_dot: the requested kernel does not cover this shape");
     dp.slices = 1;
-    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)p.batch);
+    dim3 grid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)(ragged ? 1 : p.batch));
     hipLaunchKernelGGL(dequant_dot_nk_generic_kernel, grid, dim3(256), 0, stream, dp, wbits,
                        mode == kGroupFactored ? (int)kFactored : mode);
     SetLastKernel("dequant_dot_nk_generic");
     return CheckLaunch("dequant_dot_nk_generic");
   }
   const bool zp = p.zero_points != nullptr;
-  NkShape s = PlanNk(p.batch, p.M, p.K, p.N, four_bit, mode == kGroupFactored ? p.group : 0, /*tuned_ct=*/!zp);
-  if (s.slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, s.slices))) {
+  // (a ragged dot: any group may own any number of the rows; token tiles for twice the average)
+  const int64_t tile_rows = ragged ? std::min<int64_t>(p.M, 2 * ((p.M + p.batch - 1) / p.batch)) : 0;
+  NkShape s = PlanNk(p.batch, p.M, p.K, p.N, four_bit, mode == kGroupFactored ? p.group : 0, /*tuned_ct=*/!zp, tile_rows);
+  if (ragged || (s.slices > 1 && (!p.workspace || p.workspace_bytes < DequantDotWorkspaceBytes(p.batch, p.M, p.N, s.slices)))) {
+    // (a group's rows are only known on the device: every group is one workgroup per strip and token chunk)
     s.slices = 1;
     s.k_per_slice = (int)p.K;
   }

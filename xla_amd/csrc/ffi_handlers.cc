@@ -404,7 +404,6 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   p.rhs_contracting_dim = (int32_t)rcd;
   std::string why;
   if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
-  else if (nk && ragged) why = "a ragged dot takes weights [groups,K,N]";
   else if (nk && !has_group_size) why = "weights [N,K] come with scale_group_size";
   else if (ragged && (lhs->rank != 2 || w->rank != 3)) why = "a ragged dot takes lhs [M,K] and weights [groups,K,N]";
   else if (ragged && gs->dims[0] != p.batch) why = "group_sizes must have one entry per group of weights";

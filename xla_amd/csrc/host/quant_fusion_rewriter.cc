@@ -662,13 +662,14 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   return true;
 }
 
-// ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N], group_sizes [G]) with the ragged dimension
-// on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call whose
-// kernels read the group sizes on the device, for any number of rows.
+// ragged-dot(lhs bf16 [M,K], dequantised weights [G,K,N] or [G,N,K], group_sizes [G]) with the ragged
+// dimension on the rows of lhs (what gemm_rewriter.cc:781-863 hands to a grouped matmul): one call
+// whose kernels read the group sizes on the device, for any number of rows.
 bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->operands[1], /*k_minor=*/false, &q, &why)) {
+  const bool k_minor = dot->DimsAttr("rhs_contracting_dims") == std::vector<int64_t>{2};  // experts stored [G,N,K]
+  if (!MatchQWeights(dot->operands[1], k_minor, &q, &why)) {
     if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
     return false;
   }
@@ -682,29 +683,31 @@ bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   if (lhs->Is("convert") && ConvertFrom(lhs, "bf16", &inner) && lhs->shape.dtype == "f32") lhs = inner;
   if (lhs->shape.dtype != "bf16") return refuse("the activation must be bf16 (or its convert to f32)");
   if (lhs->shape.rank() != 2 || q.w->shape.rank() != 3 || dot->shape.rank() != 2)
-    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] and a result [M,N]");
+    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] or [groups,N,K] and a result [M,N]");
   if (dot->DimsAttr("lhs_contracting_dims") != std::vector<int64_t>{1} ||
-      dot->DimsAttr("rhs_contracting_dims") != std::vector<int64_t>{1} ||
+      (dot->DimsAttr("rhs_contracting_dims") != std::vector<int64_t>{1} && !k_minor) ||
       dot->DimsAttr("lhs_ragged_dims") != std::vector<int64_t>{0} ||
       dot->DimsAttr("rhs_group_dims") != std::vector<int64_t>{0} || !dot->DimsAttr("lhs_batch_dims").empty())
     return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
                   "leading the weights");
-  const int64_t G = q.w->shape.dims[0], K = lhs->shape.dims[1], N = q.w->shape.dims[2];  // any number of rows
-  if (q.w->shape.dims[1] != K) return refuse("contracting dimensions differ");
+  const int64_t G = q.w->shape.dims[0], K = lhs->shape.dims[1], N = q.w->shape.dims[k_minor ? 1 : 2];  // any number of rows
+  if (q.w->shape.dims[k_minor ? 2 : 1] != K) return refuse("contracting dimensions differ");
   if ((sizes->shape.dtype != "s32" && sizes->shape.dtype != "s64") || sizes->shape.dims != std::vector<int64_t>{G})
     return refuse("group sizes must be s32 or s64, one per group of weights");
   const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
-  if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
+  if (four_bit && q.w->shape.dims[2] % 2 != 0) return refuse("s4 rows must hold an even number of values");
   if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");
   if (q.zero && q.zero->shape.dims != q.scale->shape.dims)
     return refuse("zero points must have the shape of the scales (one per scale)");
-  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well)
+  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well; [G,N,K/g]
+  // next to experts stored [G,N,K])
   const bool grouped = q.scale->shape.rank() == 3;
+  const int sn = k_minor ? 1 : 2, sg = k_minor ? 2 : 1;  // where N and the groups sit in rank-3 scales
   if (!(q.scale->shape.dims == std::vector<int64_t>{G, N}) &&
-      !(grouped && q.scale->shape.dims[0] == G && q.scale->shape.dims[2] == N && q.scale->shape.dims[1] > 0 &&
-        K % q.scale->shape.dims[1] == 0))
+      !(grouped && q.scale->shape.dims[0] == G && q.scale->shape.dims[sn] == N && q.scale->shape.dims[sg] > 0 &&
+        K % q.scale->shape.dims[sg] == 0))
     return refuse("a ragged dot takes scales [groups,N] or [groups,K/g,N]");
-  const int64_t group_size = grouped ? K / q.scale->shape.dims[1] : 0;
+  const int64_t group_size = grouped ? K / q.scale->shape.dims[sg] : 0;
   if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
   if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
@@ -714,10 +717,11 @@ bool RewriteRaggedDequantDot(Computation* comp, Instr* dot, RewriteLog* log) {
   ops.push_back(sizes);
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, {Shape::Array("bf16", dot->shape.dims)},
                          CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
-                             std::to_string(group_size) + " : i64");
+                             std::to_string(group_size) + " : i64" + (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
   comp->ReplaceAllUses(ep.tail, call);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
-                          (q.zero ? " with zero points" : "") + ", ragged over " + std::to_string(G) + " groups]");
+                          (q.zero ? " with zero points" : "") + ", ragged over " + std::to_string(G) + " groups" +
+                          (k_minor ? ", weights [G,N,K]" : "") + "]");
   return true;
 }
 

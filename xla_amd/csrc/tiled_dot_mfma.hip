@@ -1131,8 +1131,9 @@ int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream) {
                   p.K % 32 == 0 && (double)(p.K / p.group) * p.N * 2 < 2147483000.0;
   const bool s8 = p.weight_dtype == XLA_FFI_DataType_S8 && p.group == p.K && p.dequant_type == XLA_FFI_DataType_F32 &&
                   p.K % 16 == 0;
-  if ((!s4 && !s8) || p.group_sizes || p.zero_points) return -1;
-  if (GetOption("dequant_dot_kernel") != 3) {
+  if ((!s4 && !s8) || p.zero_points) return -1;
+  const bool ragged = p.group_sizes != nullptr;  // the caller has decided that the rows per group make tiles worth it
+  if (!ragged && GetOption("dequant_dot_kernel") != 3) {
     // token chunks of the streaming kernel against rounds of 256 tiles, in microseconds fitted on MI355X
     // (s4 8192 x 28672: 75 per 64-token pass; s8 4096 x 14336: 25)
     const double passes = (double)p.batch * (double)((p.M + 63) / 64);
@@ -1160,6 +1161,22 @@ int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
   if (s4) tp.group_shift = __builtin_ctzll((unsigned long long)p.group);  // sizes the scales' descriptor
+  if (ragged) {
+    // at most floor(M / 256) + groups tiles of rows, whatever the sizes turn out to be
+    if ((double)p.M * p.N * 2 >= 2147483000.0) return -1;
+    tp.group_sizes = p.group_sizes;
+    tp.group_sizes_64 = p.group_sizes_dtype == XLA_FFI_DataType_S64;
+    tp.ragged_groups = (int)p.batch;
+    tp.ragged_slots = (int)(p.M / kTM + p.batch);
+    if ((double)tp.ragged_slots * tp.tiles_n > 2147483000.0) return -1;
+    tp.tiles_m = tp.ragged_slots;
+    tp.scale_batched = p.scale_batch == p.batch;  // one set of scales per group, also for a single group
+    const int rc = s4 ? launch_tiled<kS4NK>(tp, 1, stream, "dequant_dot_tiled_nk_s4") : launch_tiled<kS8NK>(tp, 1, stream, "dequant_dot_tiled_nk_s8");
+    if (rc) return rc;
+    hipLaunchKernelGGL(ragged_tail_rows_kernel, dim3((unsigned)((p.N + 255) / 256), 64u), dim3(256), 0, stream, tp);
+    SetLastKernel(s4 ? "dequant_dot_tiled_nk_s4_rounded:ragged" : "dequant_dot_tiled_nk_s8_factored:ragged");
+    return CheckLaunch("dequant_dot_ragged_tail_rows");
+  }
   const size_t need = TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
   if (need && GetOption("tiled_tail") != 1 && p.workspace && ((uintptr_t)p.workspace % 16) == 0 &&
       p.workspace_bytes >= need) {

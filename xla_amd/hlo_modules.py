@@ -489,3 +489,54 @@ ENTRY %main {{
   ROOT %out = bf16[{B},{M},{N}] convert(%dot)
 }}
 """
+
+
+def k_minor_ragged_s8_experts(M=32, K=4096, N=4096, groups=8, sizes_ty="s32"):
+    """ragged-dot(bf16 [M,K], convert(s8 [G,N,K]) * f32 scale[G,N], group sizes [G]) + bias -> bf16:
+    experts stored with the contracting dimension minor."""
+    G = groups
+    return f"""HloModule k_minor_ragged_s8_experts_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s8[{G},{N},{K}] parameter(1)
+  %scale = f32[{G},{N}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %sizes = {sizes_ty}[{G}] parameter(4)
+  %lhs_f32 = f32[{M},{K}] convert(%lhs)
+  %w_f32 = f32[{G},{N},{K}] convert(%w)
+  %scale_b = f32[{G},{N},{K}] broadcast(%scale), dimensions={{0,1}}
+  %w_deq = f32[{G},{N},{K}] multiply(%w_f32, %scale_b)
+  %dot = f32[{M},{N}] ragged-dot(%lhs_f32, %w_deq, %sizes), lhs_contracting_dims={{1}}, rhs_contracting_dims={{2}}, lhs_ragged_dims={{0}}, rhs_group_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""
+
+
+def k_minor_ragged_s4_group_experts(M=32, K=4096, N=4096, groups=8, group=128):
+    """ragged-dot(bf16 [M,K], bf16(convert(s4 [G,N,K]) * bf16 scale[G,N,K/g]), group sizes [G]) + bias -> bf16."""
+    G, Kg = groups, K // group
+    return f"""HloModule k_minor_ragged_s4_group_experts_dequant_dot
+
+ENTRY %main {{
+  %lhs = bf16[{M},{K}] parameter(0)
+  %w = s4[{G},{N},{K}] parameter(1)
+  %scales = bf16[{G},{N},{Kg}] parameter(2)
+  %bias = bf16[{N}] parameter(3)
+  %sizes = s32[{G}] parameter(4)
+  %w_s8 = s8[{G},{N},{K}] convert(%w)
+  %w_g = s8[{G},{N},{Kg},{group}] reshape(%w_s8)
+  %w_bf16 = bf16[{G},{N},{Kg},{group}] convert(%w_g)
+  %scales_b = bf16[{G},{N},{Kg},{group}] broadcast(%scales), dimensions={{0,1,2}}
+  %w_deq_g = bf16[{G},{N},{Kg},{group}] multiply(%w_bf16, %scales_b)
+  %w_deq = bf16[{G},{N},{K}] reshape(%w_deq_g)
+  %dot = f32[{M},{N}] ragged-dot(%lhs, %w_deq, %sizes), lhs_contracting_dims={{1}}, rhs_contracting_dims={{2}}, lhs_ragged_dims={{0}}, rhs_group_dims={{0}}
+  %bias_f32 = f32[{N}] convert(%bias)
+  %bias_b = f32[{M},{N}] broadcast(%bias_f32), dimensions={{1}}
+  %z = f32[{M},{N}] add(%dot, %bias_b)
+  ROOT %out = bf16[{M},{N}] convert(%z)
+}}
+"""

@@ -33,6 +33,7 @@ def cases():
         ("quant_fusion_rewriter_fp8_bf16_typed", hm.c3_fp8(64, 128, 32, typed="bf16")),
         ("quant_fusion_rewriter_k_minor_s8_channel", hm.k_minor_s8_channel(16, 4096, 4096)),
         ("quant_fusion_rewriter_k_minor_s4_group", hm.k_minor_s4_group(8, 8192, 28672)),
+        ("quant_fusion_rewriter_k_minor_ragged_s8_experts", hm.k_minor_ragged_s8_experts(32, 512, 256, 4)),
         ("quant_fusion_rewriter_k_minor_u4_zero_points", hm.k_minor_u4_zero_point_group(8, 256, 64, 64)),
         ("quant_fusion_rewriter_fp8_vector_scales", hm.c3_fp8(64, 128, 32, vector_scales=True)),
         ("quant_fusion_rewriter_fp8_bf16_typed_vector_scales", hm.c3_fp8(64, 128, 32, typed="bf16", vector_scales=True)),

@@ -613,7 +613,11 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
 bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::function<void(std::string)>& log) {
   QWeights q;
   std::string why;
-  if (!MatchQWeights(dot->mutable_operand(1), /*k_minor=*/false, &q, &why)) {
+  const RaggedDotDimensionNumbers& rd = Cast<HloRaggedDotInstruction>(dot)->ragged_dot_dimension_numbers();
+  const DotDimensionNumbers& dn = rd.dot_dimension_numbers();
+  auto is = [](const auto& d, int64_t v) { return d.size() == 1 && d[0] == v; };
+  const bool k_minor = is(dn.rhs_contracting_dimensions(), 2);  // experts stored [G,N,K]
+  if (!MatchQWeights(dot->mutable_operand(1), k_minor, &q, &why)) {
     if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
     return false;
   }
@@ -627,31 +631,30 @@ bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::functi
   if (ConvertFrom(lhs, BF16, &inner) && Ty(lhs) == F32) lhs = inner;
   if (Ty(lhs) != BF16) return refuse("the activation must be bf16 (or its convert to f32)");
   if (Rank(lhs) != 2 || Rank(q.w) != 3 || Rank(dot) != 2)
-    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] and a result [M,N]");
-  const RaggedDotDimensionNumbers& rd = Cast<HloRaggedDotInstruction>(dot)->ragged_dot_dimension_numbers();
-  const DotDimensionNumbers& dn = rd.dot_dimension_numbers();
-  auto is = [](const auto& d, int64_t v) { return d.size() == 1 && d[0] == v; };
-  if (!is(dn.lhs_contracting_dimensions(), 1) || !is(dn.rhs_contracting_dimensions(), 1) ||
+    return refuse("a ragged dot is taken with lhs [M,K], weights [groups,K,N] or [groups,N,K] and a result [M,N]");
+  if (!is(dn.lhs_contracting_dimensions(), 1) || (!is(dn.rhs_contracting_dimensions(), 1) && !k_minor) ||
       !is(rd.lhs_ragged_dimensions(), 0) || !is(rd.rhs_group_dimensions(), 0) || dn.lhs_batch_dimensions_size() != 0)
     return refuse("a ragged dot is taken with the ragged dimension on the rows of lhs and the group dimension "
                   "leading the weights");
   const int64_t G = q.w->shape().dimensions(0), K = lhs->shape().dimensions(1),  // any number of rows
-                N = q.w->shape().dimensions(2);
-  if (q.w->shape().dimensions(1) != K) return refuse("contracting dimensions differ");
+                N = q.w->shape().dimensions(k_minor ? 1 : 2);
+  if (q.w->shape().dimensions(k_minor ? 2 : 1) != K) return refuse("contracting dimensions differ");
   if ((Ty(sizes) != S32 && Ty(sizes) != S64) || Dims(sizes) != std::vector<int64_t>{G})
     return refuse("group sizes must be s32 or s64, one per group of weights");
   const bool four_bit = Ty(q.w) == S4 || Ty(q.w) == U4;
-  if (four_bit && N % 2 != 0) return refuse("s4 rows must hold an even number of values");
+  if (four_bit && q.w->shape().dimensions(2) % 2 != 0) return refuse("s4 rows must hold an even number of values");
   if (q.zero && Ty(q.w) != U4) return refuse("zero points are taken with u4 weights only");
   if (q.zero && Dims(q.zero) != Dims(q.scale))
     return refuse("zero points must have the shape of the scales (one per scale)");
-  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well)
+  // scales [G,N] (one per expert and channel) or [G,K/g,N] (one per g rows of K as well; [G,N,K/g]
+  // next to experts stored [G,N,K])
   const bool grouped = Rank(q.scale) == 3;
+  const int sn = k_minor ? 1 : 2, sg = k_minor ? 2 : 1;  // where N and the groups sit in rank-3 scales
   if (!(Dims(q.scale) == std::vector<int64_t>{G, N}) &&
-      !(grouped && q.scale->shape().dimensions(0) == G && q.scale->shape().dimensions(2) == N &&
-        q.scale->shape().dimensions(1) > 0 && K % q.scale->shape().dimensions(1) == 0))
+      !(grouped && q.scale->shape().dimensions(0) == G && q.scale->shape().dimensions(sn) == N &&
+        q.scale->shape().dimensions(sg) > 0 && K % q.scale->shape().dimensions(sg) == 0))
     return refuse("a ragged dot takes scales [groups,N] or [groups,K/g,N]");
-  const int64_t group_size = grouped ? K / q.scale->shape().dimensions(1) : 0;
+  const int64_t group_size = grouped ? K / q.scale->shape().dimensions(sg) : 0;
   if (q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
   if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false)) return refuse(why);
@@ -660,10 +663,12 @@ bool RewriteRaggedDequantDot(HloComputation* comp, Instr* dot, const std::functi
   if (ep.bias) ops.push_back(ep.bias);
   ops.push_back(sizes);
   Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, {ShapeUtil::MakeShape(BF16, Dims(dot))},
-                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64"));
+                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64") +
+                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
   CHECK_OK(ep.tail->ReplaceAllUsesWith(call));
   VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
-          << (q.zero ? " with zero points" : "") << ", ragged over " << G << " groups]";
+          << (q.zero ? " with zero points" : "") << ", ragged over " << G << " groups"
+          << (k_minor ? ", weights [G,N,K]" : "") << "]";
   return true;
 }
 
