@@ -7,6 +7,8 @@
 // K-minor rows are already the matrix instruction's operand: for v_mfma_f32_16x16x32_bf16 lane
 // (c, q) = (lane % 16, lane / 16) holds 8 consecutive k of row c, so a lane that fetches 16
 // contiguous bytes of channel c owns two (s8) or four (s4) operands with no transposition.
+// (The bytes are fetched quad-wise, 64 contiguous bytes per four lanes, and re-dealt to those
+// lanes through a small wave-private LDS buffer: see NkStage::VIA_LDS.)
 // A wave walks K for CT tiles of 16 channels and MT tiles of 16 tokens; the waves of a workgroup
 // take neighbouring channels over the same k and share the activations through LDS.  Few
 // channels: K is cut into slices (grid.z) whose f32 partial sums the finalize kernel adds in
@@ -46,6 +48,12 @@ struct NkStage {
   static constexpr int TOK = 16 * MT;
   static constexpr int STAGE_BYTES = TOK * ROWB;
   static constexpr int CHUNKS = TOK * (KS / 8) / (kNkWaves * 64);  // 16-byte pieces a thread moves per stage
+  // Whether a lane fetches the very bytes it multiplies (the four lanes of a quad then read four different
+  // 64-byte segments, which the address unit serves at a quarter of its rate: its FIFO was full 59 % of
+  // the time) or the wave fetches whole segments per quad and re-deals them through 1 KiB of LDS per
+  // channel tile.  Measured on 8192 x 28672 s4: 41 -> 35 us up to 8 tokens, 41 -> 38 at 16, 52 -> 50 at
+  // 32, but 58 -> 61 at 64, where the activation reads already keep LDS busy; s8 gains at every size.
+  static constexpr bool VIA_LDS = !(WBITS == 4 && MT == 4);
 };
 
 // WBITS 8 | 4; MT token tiles; CT channel tiles per wave; MODE as in the [K,N] kernels:
@@ -66,7 +74,8 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   using S = NkStage<WBITS, MT>;
   constexpr int KP = S::KP, NJ = KP / 8, STEP = S::STEP, SPS = S::SPS, KS = S::KS, ROWB = S::ROWB, CHUNKS = S::CHUNKS;
   constexpr bool GF = MODE == kGroupFactored;
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [2][STAGE_BYTES]
+  constexpr bool VIA_LDS = S::VIA_LDS;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [2][STAGE_BYTES], then [waves][CT][1024]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 15, kq = lane >> 4;
   const int strip = blockIdx.x, slice = blockIdx.z;
@@ -97,7 +106,9 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
 #pragma unroll
   for (int t = 0; t < CT; ++t) {
     const int n = n_wave + t * 16 + c;
-    voff_w[t] = n < p.N ? (uint32_t)n * row_bytes + kq * 16 : kPastEnd;
+    // VIA_LDS: fetched by lane (channel lane / 4, piece lane % 4), a quad reading 64 contiguous bytes
+    const int nf = VIA_LDS ? n_wave + t * 16 + (lane >> 2) : n;
+    voff_w[t] = nf < p.N ? (uint32_t)nf * row_bytes + (VIA_LDS ? lane & 3 : kq) * 16 : kPastEnd;
     elem_s[t] = (uint32_t)max(0, min(n, p.N - 1)) * (uint32_t)G;
   }
 
@@ -144,10 +155,11 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
       // past it the lane must not read on into the next row
       const uint32_t kl = (uint32_t)(ks + st * STEP + kq * KP);
       const bool live = kl < (uint32_t)k_end;
+      const bool live_f = (uint32_t)(ks + st * STEP + (VIA_LDS ? lane & 3 : kq) * KP) < (uint32_t)k_end;  // the piece this lane fetches
       const uint32_t wb = (uint32_t)(ks + st * STEP) * WBITS / 8;
 #pragma unroll
       for (int t = 0; t < CT; ++t)
-        wq[set][st][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, live ? voff_w[t] + wb : kPastEnd, 0, 0);
+        wq[set][st][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, live_f ? voff_w[t] + wb : kPastEnd, 0, 0);
       if constexpr (MODE == kRounded || ZP) {
         const uint32_t g = group_of(q, live ? kl : 0u);
 #pragma unroll
@@ -165,11 +177,32 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   };
 
   // whether the scale group ends with the step that starts at k0 (groups are whole steps)
+  // ---- fetched pieces -> matrix operands, through 1 KiB of LDS that only this wave touches (LDS serves a
+  // wave's instructions in order: no wait between the write and the read).  Lane (r, p) = (lane / 4,
+  // lane % 4) holds piece p of channel r and writes it to slot p ^ (r / 4) of row r; lane (c, kq) reads
+  // slot kq ^ (c / 4) of row c.  Both ways 16 lanes cover all 64 banks once.
+  uint8_t* stage_w = lds + 2 * S::STAGE_BYTES + wave * (CT * 1024);
+  const uint32_t st_wr = (uint32_t)(lane >> 2) * 64u + (uint32_t)(((lane & 3) ^ (lane >> 4)) << 4);
+  const uint32_t st_rd = (uint32_t)c * 64u + (uint32_t)((kq ^ (c >> 2)) << 4);
+  auto transpose = [&](int set, int st, uintx4* x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < CT; ++t) {
+      if constexpr (VIA_LDS) {
+        uint8_t* b = stage_w + t * 1024;  // (one buffer: the read of the step before was issued first)
+        *reinterpret_cast<uintx4*>(b + st_wr) = wq[set][st][t];
+        __builtin_amdgcn_wave_barrier();  // (no instruction: keeps the compiler from moving the read up)
+        x[t] = *reinterpret_cast<const uintx4*>(b + st_rd);
+      } else {
+        x[t] = wq[set][st][t];
+      }
+    }
+  };
+
   auto closes_group = [&](int k0) __attribute__((always_inline)) {
     return ((uint32_t)(k0 + STEP) & ((uint32_t)p.group - 1u)) == 0u;
   };
 
-  auto compute = [&](int set, int st, int buf, int k0) __attribute__((always_inline)) {
+  auto compute = [&](int set, int st, int buf, int k0, const uintx4* xw) __attribute__((always_inline)) {
     float gs[CT][4] = {};
     const bool closing = GF && k0 < k_end && closes_group(k0);
     if (closing) {  // its scales, by output register
@@ -204,7 +237,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
         float f[8];
         if constexpr (WBITS == 4) {
           typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
-          const uint32_t x = wq[set][st][t][j];
+          const uint32_t x = xw[t][j];
           // nibble pairs (0,4), (1,5) of x and (2,6), (3,7) of x >> 8, offset binary for s4 (the
           // sign bit flipped: u = w + 8), as they are for u4
           const uint32_t ce = p.w_unsigned ? 0x64006400u : 0x64086408u, co = p.w_unsigned ? 0x64006400u : 0x64806480u;
@@ -222,7 +255,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
           f[7] = __builtin_fmaf((float)p37[1], s_odd, c_odd);
         } else {
           // 16 bytes are two operands: dwords (2j, 2j + 1)
-          const uint32_t x0 = wq[set][st][t][j * 2], x1 = wq[set][st][t][j * 2 + 1];
+          const uint32_t x0 = xw[t][j * 2], x1 = xw[t][j * 2 + 1];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             f[e] = (float)(int8_t)((x0 >> (8 * e)) & 0xffu);
@@ -257,8 +290,13 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   // Steps past k_end run on zeros (their loads are masked) rather than being branched around: a
   // branch between a stage's loads and their use lets the compiler move the loads down to the use.
   auto compute_stage = [&](int set, int ks) __attribute__((always_inline)) {
+    uintx4 xw[2][CT];  // the operands of this step and, requested one step ahead, of the next
+    transpose(set, 0, xw[0]);
 #pragma unroll
-    for (int st = 0; st < SPS; ++st) compute(set, st, set, ks + st * STEP);  // (buffer index = register set)
+    for (int st = 0; st < SPS; ++st) {
+      if (st + 1 < SPS) transpose(set, st + 1, xw[(st + 1) & 1]);
+      compute(set, st, set, ks + st * STEP, xw[st & 1]);  // (buffer index = register set)
+    }
   };
 
   load_acts(k_begin);
@@ -383,7 +421,8 @@ __global__ __launch_bounds__(256) void nk_ragged_tail_rows_kernel(DecodeParams p
 
 template <int WBITS, int MT, int CT, int MODE, bool ZP>
 int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name) {
-  constexpr size_t kLds = 2 * (size_t)NkStage<WBITS, MT>::STAGE_BYTES;
+  constexpr size_t kLds = 2 * (size_t)NkStage<WBITS, MT>::STAGE_BYTES +
+                          (NkStage<WBITS, MT>::VIA_LDS ? (size_t)kNkWaves * CT * 1024 : 0);
   // per kernel instantiation and device: one bit per device ordinal (two threads that race set the
   // attribute to the same value)
   static std::atomic<unsigned long long> configured{0};
