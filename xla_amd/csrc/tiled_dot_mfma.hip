@@ -369,13 +369,14 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const int w_nq = tid & 63, w_kblk = tid >> 6;
   auto s8_load = [&](int k0) {
     const uint32_t col = (uint32_t)(n0 + w_nq * 4);
+    const uint32_t kfirst = (uint32_t)(k0 + w_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
+    // (one select for the block, not a branch per row: the loads sit between the matrix instructions)
+    const bool live = col < (uint32_t)p.N && kfirst < (uint32_t)p.K;  // else it would alias other rows
+    // the top bit puts an offset past the end of every buffer (all are smaller than 2 GiB)
+    const uint32_t first = (kfirst * (uint32_t)p.N + col) | (live ? 0u : kOutOfRange);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const uint32_t k = (uint32_t)(k0 + w_kblk * 8 + r);
-      uint32_t voff = k * (uint32_t)p.N + col;
-      if (col >= (uint32_t)p.N || k >= (uint32_t)p.K) voff = kOutOfRange;  // would alias other rows
-      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, voff, 0, 0);
-    }
+    for (int r = 0; r < 8; ++r)
+      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * (uint32_t)p.N, 0, 0);
   };
   auto s8_store = [&](uint8_t* bt) {
 #pragma unroll
@@ -407,9 +408,11 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const uint32_t col = (uint32_t)(n0 + q_oct * 8);
     const uint32_t kfirst = (uint32_t)(k0 + q_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
     const bool live = col < (uint32_t)p.N && kfirst < (uint32_t)p.K;  // N % 8 == 0
+    // (the top bit puts an offset past the end of the buffer: one select for the block, no branch per row)
+    const uint32_t first = (kfirst * s4_pitch + (col >> 1)) | (live ? 0u : kOutOfRange);
 #pragma unroll
     for (int r = 0; r < 8; ++r)
-      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, live ? (kfirst + r) * s4_pitch + (col >> 1) : kOutOfRange, 0, 0);
+      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * s4_pitch, 0, 0);
     s4_scales = __builtin_amdgcn_raw_buffer_load_b128(
         rsc4, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) * 2u : kOutOfRange, 0, 0);
   };
