@@ -447,19 +447,23 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
   };
-  // ---- weights stored [N,K]: thread t takes channel t >> 1 and the half t & 1 of the stage's 64 k:
-  // 32 bytes of s8 or 16 bytes of s4, both contiguous, that become chunks 4 * half ... + 3 of the
-  // channel's LDS row (K % 32 == 0 for s4 and % 16 for s8: a 16-byte piece lies inside its row or past it)
-  const int nk_n = tid >> 1, nk_half = tid & 1;
+  // ---- weights stored [N,K].  s4: thread t takes channel t >> 1 and the half t & 1 of the stage's 64 k,
+  // 16 contiguous bytes that become chunks 4 * half ... + 3 of the channel's LDS row.  s8: thread t
+  // takes the 16-byte piece t & 3 of channels t >> 2 and (t >> 2) + 128 -- the four lanes of a quad
+  // read the 64 contiguous bytes of one channel -- and each piece becomes chunks 2 * piece, + 1.
+  // (K % 32 == 0 for s4 and % 16 for s8: a 16-byte piece lies inside its row or past it.)
+  const int nk_n = KIND == kS8NK ? tid >> 2 : tid >> 1, nk_half = tid & 1, nk_piece = tid & 3;
   uint32_t nk_scale = 0;
   auto nk_load = [&](int k0) {
     const uint32_t ch = (uint32_t)(n0 + nk_n);
     const uint32_t k = (uint32_t)(k0 + nk_half * 32);
     if constexpr (KIND == kS8NK) {
+      const uint32_t kp = (uint32_t)(k0 + nk_piece * 16);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const bool live = ch < (uint32_t)p.N && k + 16 * j < (uint32_t)p.K;
-        const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? ch * (uint32_t)p.K + k + 16 * j : kOutOfRange, 0, 0);
+        const uint32_t cj = ch + 128u * j;
+        const bool live = cj < (uint32_t)p.N && kp < (uint32_t)p.K;
+        const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? cj * (uint32_t)p.K + kp : kOutOfRange, 0, 0);
         wreg[4 * j] = v[0]; wreg[4 * j + 1] = v[1]; wreg[4 * j + 2] = v[2]; wreg[4 * j + 3] = v[3];
       }
     } else {
@@ -503,7 +507,10 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
       const uintx4 o = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
                         pack_bf16x2(f[6], f[7])};
-      *reinterpret_cast<uintx4*>(bt + nk_n * kRow + (((nk_half * 4 + c) ^ ((nk_n >> 1) & 7)) << 4)) = o;
+      // s8: dwords (2c, 2c + 1) are half c & 1 of the piece of channel nk_n + 128 * (c >> 1)
+      const int row = KIND == kS8NK ? nk_n + 128 * (c >> 1) : nk_n;
+      const int chunk = KIND == kS8NK ? nk_piece * 2 + (c & 1) : nk_half * 4 + c;
+      *reinterpret_cast<uintx4*>(bt + row * kRow + ((chunk ^ ((row >> 1) & 7)) << 4)) = o;
     }
   };
   auto wq_store = [&](uint8_t* bt) {
