@@ -38,18 +38,21 @@ def test_handlers_replay_from_a_hip_graph(oracle):
                     (workloads.c2_s4_group(M=20, K=2048, N=768, group=64), {"dequant_dot_slices": 2}),  # finalize launch
                     (workloads.c2_s4_group(M=70, K=1024, N=512), {}),                     # 64 + 6 tokens
                     (workloads.c1_s8_channel(M=16, K=2048, N=1024), {}),                  # slices inside the kernel
-                    (workloads.c5_s8_batched(B=1, M=300, K=2048, N=700), {})):            # tiles split along K
-        lhs = dev_bf16(w["lhs"])
-        wt = dev_u8(w["weights_packed"]) if w["weight_dtype"] == "s4" else dev_s8(w["weights"])
-        sc = dev_bf16(w["scales"]) if w["scales"].dtype == np.uint16 else dev_f32(w["scales"])
-        bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
-        for k, v in opts.items():
-            ffi.set_option(k, v)
+                    (workloads.c5_s8_batched(B=1, M=300, K=2048, N=700), {}),             # tiles split along K
+                    (workloads.c2_s4_group(M=8, K=2048, N=512), {"nk": 1})):              # weights stored [N,K], K-slices
+        nk = opts.pop("nk", 0)
+        v = workloads.k_minor(w) if nk else w   # (the oracle keeps reading the [K,N] arrays)
+        lhs = dev_bf16(v["lhs"])
+        wt = dev_u8(v["weights_packed"]) if v["weight_dtype"] == "s4" else dev_s8(v["weights"])
+        sc = dev_bf16(v["scales"]) if v["scales"].dtype == np.uint16 else dev_f32(v["scales"])
+        bias = dev_bf16(v["bias"]) if v.get("bias") is not None else None
+        for k, val in opts.items():
+            ffi.set_option(k, val)
         try:
-            call = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"], weight_shape=w["weight_shape"],
-                                   epilogue=w["epilogue"], dequant_type=w["dequant_type"],
-                                   scale_group_size=0 if w["group"] == w["lhs"].shape[-1] else w["group"],
-                                   build_only=True)
+            call = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=v["weight_dtype"], weight_shape=v["weight_shape"],
+                                   epilogue=v["epilogue"], dequant_type=v["dequant_type"],
+                                   scale_group_size=0 if v["group"] == v["lhs"].shape[-1] else v["group"],
+                                   rhs_contracting_dim=nk, build_only=True)
             call.run()   # eager warm-up with the options that pick the kernel; the frame keeps its scratch
             torch.cuda.synchronize()
             kern = ffi.last_kernel()
@@ -61,6 +64,7 @@ def test_handlers_replay_from_a_hip_graph(oracle):
     assert dots[2][4].endswith(":x64"), dots[2][4]
     assert dots[3][4].startswith("dequant_dot_decode_s8x_"), dots[3][4]
     assert dots[4][4] == "dequant_dot_tiled_s8_factored:tail2", dots[4][4]
+    assert dots[5][4] == "dequant_dot_nk_s4_m16_rounded", dots[5][4]
 
     q4 = workloads.c4_quantize(rows=256, cols=1024)
     x, gamma = dev_bf16(q4["x"]), dev_bf16(q4["gamma"])
