@@ -31,6 +31,7 @@ struct NkParams {
   int k_per_slice;       // multiple of the step (and of the group for group-factored sums)
   int group_shift;       // log2(group); 31 for one scale per channel
   int m_chunks;          // grid.y = batch * m_chunks, chunk c takes tokens [c*16*MT, +16*MT)
+  int scale_batches;     // sets of scales (and zero points): the batch count, or 1 when all batches share one
 };
 
 // (scale groups are powers of two, or one per channel: shift 31)
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   const uint32_t sc_elems = (uint32_t)p.N * (uint32_t)G;
   const __amdgpu_buffer_rsrc_t rs = make_rsrc((const uint16_t*)p.scales + sbatch * sc_elems, sc_elems * 2u);
   const uint32_t zp_first = (uint32_t)(sbatch * sc_elems);  // element index of this batch's first zero point
-  const __amdgpu_buffer_rsrc_t rz = make_rsrc(ZP ? p.zero_points : p.w, ZP ? (uint32_t)(((size_t)(p.scale_batched ? gridDim.y / q.m_chunks : 1) * sc_elems + 1) >> 1) : 0u);
+  const __amdgpu_buffer_rsrc_t rz =
+      make_rsrc(ZP ? p.zero_points : p.w, ZP ? (uint32_t)(((size_t)q.scale_batches * sc_elems + 1) >> 1) : 0u);
   uint32_t voff_w[CT], elem_s[CT];
 #pragma unroll
   for (int t = 0; t < CT; ++t) {
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
     for (int t = 0; t < CT; ++t) {
       // 4-bit: nibble e of a dword arrives as the f16 value 1024 + u (even e) or 1024 + 16 u (odd e);
       // (u - z) * s = (1024 + u) * s - (1024 + z) * s = (1024 + 16 u) * (s / 16) - (64 + z) * s:
-      // one fma each, exact for a scale of 8 significant bits
+      // one fma each, exact for a scale of 8 significant bits with |1040 s| finite (an infinite scale
+      // gives NaN where the product would be an infinity)
       float s = 1.0f, z = z_default;
       if constexpr (MODE == kRounded) s = bf16lo_to_f32(sraw[set][st][t]);
       if constexpr (ZP) z = (float)((zraw[set][st][t] >> ((zraw[set][st][t] >> 6) & 4u)) & 0xfu);  // bit 8: the high nibble
@@ -561,6 +564,7 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
   q.k_per_slice = s.k_per_slice;
   q.group_shift = group_shift;
   q.m_chunks = s.m_chunks;
+  q.scale_batches = dp.scale_batched ? (int)p.batch : 1;
 #define XLA_AMD_NK(WB, MT_, CT_, MODE_, NAME)                                             \
   if (wbits == WB && s.mt == MT_ && s.ct == CT_ && mode == MODE_) {                       \
     if constexpr (WB == 4 && CT_ == (MT_ == 1 ? 1 : 2))                                   \
