@@ -244,7 +244,6 @@ def test_large_prefill_picks_the_tiled_kernel_by_itself(oracle):
     w = workloads.c1_s8_channel(M=1024, K=1024, N=4096)
     got, kern = run_nk(w)
     assert kern.startswith("dequant_dot_tiled_nk_s8_factored"), kern
-    sub = dict(w, lhs=w["lhs"][:64], )
     # the oracle on a block of rows and channels
     rows, cols = slice(512, 560), slice(1000, 1256)
     blk = dict(w, lhs=w["lhs"][rows], weights=w["weights"][:, cols], scales=w["scales"][cols], weight_shape=(1024, 256))
