@@ -147,9 +147,11 @@ typedef struct XlaAmdDequantDot {
    * dot.  Otherwise `batch` row counts in device memory, S32 or S64 (group_sizes_dtype): lhs is
    * [M,K] with its rows sorted by group, weights [batch,K,N] hold one matrix per group, out is
    * [M,N]; group g takes rows [sum of the sizes before it, + its size), rows past the last group
-   * are a dot of nothing (epilogue(0)).  Never read on the host. */
+   * are a dot of nothing (epilogue(0)).  Never read on the host.  A ragged dot over zero groups
+   * (batch = 0, where the pointer of the empty array may be NULL) is told by group_sizes_dtype
+   * being S32 or S64: every row of out is then epilogue(0). */
   const void* group_sizes;
-  int32_t group_sizes_dtype;
+  int32_t group_sizes_dtype; /* S32 or S64; 0 for an ordinary dot */
   /* 0: weights [batch,K,N] as above.  1: weights [batch,N,K], the contracting dimension minor
    * (dot ... rhs_contracting_dims={1}, fusion_emitter_int4_device_test.cc:867-892): 4-bit values are
    * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  With

@@ -320,3 +320,17 @@ def test_batched_rank2_scales_need_scale_group_size_when_both_readings_fit():
         a1 = [(dtypes.BF16, FAKE, (2, 64)), (dtypes.S8, FAKE, (64, 8)), (dtypes.F32, FAKE, (8,))]
         ffi.invoke("xla_amd.dequant_dot", ffi.Frame(host, a1, [(dtypes.BF16, FAKE, (2, 8))],
                                                     {"scale_group_size": ffi.Attr.i64(16)}))
+
+
+def test_workspace_sizer_covers_token_chunks():
+    """More than 64 tokens of 4-bit weights run as 64-token chunks with the chunk index as the batch
+    of one launch: the sizer must report what that launch can use (narrow N wants K-slices), not what
+    a single 64-token call would."""
+    L = ffi.library()
+    s4 = 21
+    one = L.xla_amd_dequant_dot_workspace_bytes(1, 64, 8192, 1024, s4)
+    two = L.xla_amd_dequant_dot_workspace_bytes(2, 64, 8192, 1024, s4)
+    chunked = L.xla_amd_dequant_dot_workspace_bytes(1, 128, 8192, 1024, s4)
+    assert two > 0 and chunked >= two, (one, two, chunked)
+    # the remainder launch is covered as well
+    assert L.xla_amd_dequant_dot_workspace_bytes(1, 64 + 8, 8192, 1024, s4) >= L.xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 1024, s4)

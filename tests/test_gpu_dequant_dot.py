@@ -743,6 +743,26 @@ def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
     check_dot(got_generic, ref, ragged_floor(w), "ragged generic")
 
 
+@pytest.mark.parametrize("nk", [False, True])
+def test_ragged_dot_without_any_group(nk):
+    """A ragged dot over zero groups (weights [0,K,N], group_sizes [0]): no row has a group, so every
+    row is epilogue(0 + bias) -- the result must be written, not left as it was."""
+    say("dequant_dot ragged, zero groups, nk=%s" % nk)
+    M, K, N = 9, 256, 136
+    lhs = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda")
+    wt = torch.zeros((0, N, K) if nk else (0, K, N), dtype=torch.int8, device="cuda")
+    sc = torch.zeros((0, N), dtype=torch.float32, device="cuda")
+    bias_h = dtypes.f32_to_bf16(np.linspace(-3.0, 3.0, N).astype(np.float32))
+    gs = torch.zeros((0,), dtype=torch.int32, device="cuda")
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.dequant_dot(lhs, wt, sc, dev_bf16(bias_h), weight_dtype="s8", epilogue="BIAS_RELU", dequant_type="f32", scale_group_size=0,
+                    group_sizes=gs, rhs_contracting_dim=1 if nk else 0, out=out)
+    torch.cuda.synchronize()
+    assert ffi.last_kernel() == "dequant_dot:ragged_no_groups"
+    want = np.where(dtypes.bf16_to_f32(bias_h) > 0, bias_h, 0).astype(np.uint16)
+    assert np.array_equal(host_bf16(out), np.broadcast_to(want, (M, N)))
+
+
 @pytest.mark.parametrize("M,K,N,G,sizes", [
     (200, 512, 256, 4, [70, 0, 129, 1]), (640, 1024, 512, 8, None), (130, 512, 128, 2, [130, 0]),
     (100, 256, 128, 3, [10, 20, 30]), (300, 512, 256, 4, [0, 400, 7, 0])])

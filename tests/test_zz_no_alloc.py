@@ -111,3 +111,34 @@ def test_static_scratch_with_weights_stored_k_minor(oracle):
     a = np.abs(dtypes.bf16_to_f32(c1["lhs"]).astype(np.float64))
     wd = np.abs(c1["weights"].astype(np.float64)) * c1["scales"].astype(np.float64)[None, :]
     check_dot(got_st.reshape(M, N), ref, dot_floor(a, wd, K), "static scratch, weights [N,K]")
+
+
+def test_static_scratch_with_more_than_64_tokens(oracle):
+    """More than 64 tokens of s8 weights run on the tiled kernel, whose short last round is split along
+    K through the scratch: the static array must be sized for that too.  A shape whose split fits is
+    bit-identical to the workspace launcher (same split, same order of the two halves); one whose
+    split needs more than the array is refused, as the [N,K] spelling of it is."""
+    L = ffi.library()
+    M, K, N = 128, 2048, 2048      # 8 tiles, all split in two: 8 x (256 KiB + 8)
+    need = L.xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S8)
+    assert 0 < need <= 8 << 20, need
+    c = workloads.c1_s8_channel(M=M, K=K, N=N)
+    lhs, w, sc = dev_bf16(c["lhs"]), dev_s8(c["weights"]), dev_f32(c["scales"])
+    p = _params(lhs, w, sc, None, lhs, M, K, N, K, dtypes.S8, dtypes.F32, dtypes.F32, "DEFAULT")
+    got_ws, got_st = _both(p, need)
+    assert L.xla_amd_last_kernel().endswith(b":tail2"), L.xla_amd_last_kernel()
+    assert np.array_equal(got_ws, got_st)
+    ref = oracle.dequant_dot(c["lhs"], c["weights"], 8, c["scales"], "f32", "f32")
+    a = np.abs(dtypes.bf16_to_f32(c["lhs"]).astype(np.float64))
+    wd = np.abs(c["weights"].astype(np.float64)) * c["scales"].astype(np.float64)[None, :]
+    check_dot(got_st.reshape(M, N), ref, dot_floor(a, wd, K), "static scratch, split last round")
+
+    M2, N2 = 1024, 4096            # 64 tiles split in two: 16 MiB
+    need2 = L.xla_amd_dequant_dot_workspace_bytes(1, M2, K, N2, dtypes.S8)
+    assert need2 > 8 << 20, need2
+    t = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    for rcd in (0, 1):
+        p2 = _params(t, t, t, None, t, M2, K, N2, K, dtypes.S8, dtypes.F32, dtypes.F32, "DEFAULT")
+        p2.rhs_contracting_dim = rcd
+        rc = L.xla_amd_launch_dequant_dot_static_scratch(C.byref(p2), torch.cuda.current_stream().cuda_stream)
+        assert rc == 8 and b"static scratch holds" in L.xla_amd_last_error(), (rcd, rc, L.xla_amd_last_error())

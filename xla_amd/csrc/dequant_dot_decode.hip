@@ -576,11 +576,7 @@ int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int
 
 // What xla_amd_dequant_dot_workspace_bytes reports: the scratch the launch below will use for
 // this shape (the narrowest strips give the most slices), or what a forced slice count needs.
-size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4) {
-  if (M > 64 && s4) {  // runs as one batch-1 launch per 64 tokens, all sharing the scratch
-    M = 64;
-    batch = 1;
-  }
+static size_t DecodeWorkspaceBytesUpTo64(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4) {
   if (M <= 0 || M > 64 || K < 32 || N <= 0 || batch <= 0) return 0;
   const int mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 48 ? 3 : 4;
   int vec = s4 ? 4 : (mt >= 3 ? 4 : 8);
@@ -595,6 +591,31 @@ size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64
   // small s8 matrices up to 16 tokens: the slices of a strip hand over inside the kernel
   if (!s4 && S8xWorkspaceBytes(batch, M, K, N) > bytes) bytes = S8xWorkspaceBytes(batch, M, K, N);
   return bytes;
+}
+
+size_t DequantDotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, bool s4) {
+  if (M <= 64) return DecodeWorkspaceBytesUpTo64(batch, M, K, N, s4);
+  // More than 64 tokens on the decode kernels: per batch, all whole chunks of 64 tokens (32 for
+  // 4-bit weights under group-factored sums: the mode is not known here, the larger need decides)
+  // as one launch with the chunk index as its batch, then the remaining tokens as a second launch;
+  // the launches follow each other on the stream and share the scratch.
+  size_t bytes = 0;
+  for (int64_t chunk = 64; chunk >= (s4 ? 32 : 64); chunk /= 2) {
+    const size_t whole = DecodeWorkspaceBytesUpTo64(M / chunk, chunk, K, N, s4);
+    const size_t rest = DecodeWorkspaceBytesUpTo64(1, M % chunk, K, N, s4);
+    bytes = bytes > whole ? bytes : whole;
+    bytes = bytes > rest ? bytes : rest;
+  }
+  return bytes;
+}
+
+// Ragged dot without a single group: every row is a dot of nothing, epilogue(0 [+ bias]).
+__global__ __launch_bounds__(256) void ragged_no_groups_kernel(DecodeParams p) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= p.N) return;
+  const float bias = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  const uint16_t v = f32_to_bf16(epilogue_dispatch(0.0f, bias, p.epilogue, p.bf16_dot, p.bf16_ops));
+  for (int m = blockIdx.y; m < p.M; m += gridDim.y) p.out[(size_t)m * p.N + n] = v;
 }
 
 // weights_shared: `batch` counts 64-token chunks of one [batch * M, K] activation matrix that all
@@ -625,6 +646,23 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   if (p.dequant_type == XLA_FFI_DataType_BF16 && p.scale_dtype != XLA_FFI_DataType_BF16)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT,
                 "dequant_dot: a bf16-typed dequantise multiply needs bf16 scales");
+  if (p.batch == 0 && (p.group_sizes || p.group_sizes_dtype != 0) && p.M > 0 && p.N > 0) {
+    // a ragged dot over no groups: no row has a group, so every row is epilogue(0 [+ bias])
+    if (!p.out || ((p.epilogue & 1) && !p.bias))
+      return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: null buffer");
+    DecodeParams fp = {};
+    fp.out = (uint16_t*)p.out;
+    fp.bias = (p.epilogue & 1) ? p.bias : nullptr;
+    fp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
+    fp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
+    fp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
+    fp.epilogue = p.epilogue;
+    fp.M = (int)p.M; fp.N = (int)p.N;
+    const unsigned rows = (unsigned)(p.M < 64 ? p.M : 64);
+    hipLaunchKernelGGL(ragged_no_groups_kernel, dim3((unsigned)((p.N + 255) / 256), rows), dim3(256), 0, stream, fp);
+    SetLastKernel("dequant_dot:ragged_no_groups");
+    return CheckLaunch("dequant_dot_ragged_no_groups");
+  }
   if (p.batch == 0 || p.M == 0 || p.N == 0) {
     SetLastKernel("dequant_dot:empty");
     return 0;
@@ -874,10 +912,19 @@ static int StaticScratchPointer(void** out) {
 
 int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream) {
   const bool four_bit = p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4;
-  const size_t need = p.batch > 0 && p.M > 0 && p.K > 0 && p.N > 0
-                          ? p.rhs_contracting_dim == 1 ? DequantDotNkWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit) :
-                          DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, p.weight_dtype == XLA_FFI_DataType_S4 || p.weight_dtype == XLA_FFI_DataType_U4)
-                          : 0;
+  // exactly what the public sizers report: the decode kernels' partial sums, or the split last round
+  // of the tiled kernel when more than 64 tokens go there (it adds the halves of a tile in a fixed
+  // order only when the whole of that scratch is there, so a shape needing more is refused as well)
+  size_t need = 0;
+  if (p.batch > 0 && p.M > 0 && p.K > 0 && p.N > 0) {
+    if (p.rhs_contracting_dim == 1) {
+      need = DequantDotNkWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit);
+    } else {
+      need = DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit);
+      const size_t tail = p.weight_dtype == XLA_FFI_DataType_U4 ? 0 : TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
+      if (tail > need) need = tail;
+    }
+  }
   if (need > kStaticScratchBytes)
     return Fail(XLA_FFI_Error_Code_RESOURCE_EXHAUSTED,
                 "dequant_dot_static_scratch: this shape splits K through %zu bytes of partial sums, the static "
