@@ -64,12 +64,19 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // [16 tokens][64 bytes] of activations.  The same memory later carries the waves' partial tiles.
   constexpr int kWBytes = 32 * WROW;
   constexpr int kSlot = kWBytes + MT * 1024;
-  constexpr int kRingBytes = WAVES * DEPTH * kSlot, kSumBytes = WAVES * kChunk * 64 * 4;
+  constexpr int kRingBytes = WAVES * DEPTH * kSlot, kSumBytes = 2 * WAVES * kChunk * 64 * 4;
   __shared__ __attribute__((aligned(16))) uint8_t smem[kRingBytes > kSumBytes ? kRingBytes : kSumBytes];
   float* const lds = (float*)smem;
   __shared__ uint32_t lds_bad[4 * COLS];
   __shared__ int lds_partner;
 
+#ifdef XLA_AMD_STAMPS
+  long long stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define STAMP(i) stamps[i] = wall_clock64()
+#else
+#define STAMP(i)
+#endif
+  STAMP(0);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4, q = (lane >> 2) & 3, i = lane & 3;
@@ -104,16 +111,27 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // rows of WROW contiguous bytes; lane l deposits at slot + 16 * l: the slot is a row-major
   // [32 rows][WROW bytes] tile.  32-channel pieces beyond N (N % 32 == 0) read as zeros.
   constexpr int LPR = 4 * COLS, RPI = 64 / LPR, NLD = 32 / RPI;
-  const uint32_t voff_w = strip * TN + 32 * (lane % LPR) < p.N
-                              ? (uint32_t)(lane / LPR) * pitch + (uint32_t)((strip * TN + 32 * (lane % LPR)) >> 1)
+  // LDS serves a 16-byte read 16 lanes at a time, and those 16 pieces must fall into 16 different
+  // 16-byte bank groups (address / 16 mod 16).  The loads deposit lane l's piece at 16 * l whatever it
+  // fetched, so the layout is swizzled by choosing WHICH piece of its row (weights) or token
+  // (activations) a lane fetches -- the lanes of a row still cover the same contiguous bytes.
+  // Weights, two columns: rows i and i + 2 of a lane group would meet in the same bank groups (rows
+  // are 128 bytes apart); rows with bit 1 set keep their two 64-byte halves exchanged.
+  const int wpiece = COLS == 2 ? (lane % LPR) ^ ((((lane / LPR) >> 1) & 1) << 2) : lane % LPR;
+  const uint32_t voff_w = strip * TN + 32 * wpiece < p.N
+                              ? (uint32_t)(lane / LPR) * pitch + (uint32_t)((strip * TN + 32 * wpiece) >> 1)
                               : kNowhere;
   uint8_t* const my_ring = smem + wave * (DEPTH * kSlot);
   // Consuming side: rows 8 * kb + i and 8 * kb + i + 4, column c, piece q
-  const uint32_t rd_off = (uint32_t)(WROW * (8 * kb + i) + 16 * q);
-  // activations, loading side: lane l fetches 16 bytes (8 rows) of token l >> 2 for the block l & 3
-  // and deposits them at 16 * l; consuming side: token li, block kb
-  const uint32_t voff_a = ((uint32_t)(lane >> 2) * p.K + (uint32_t)((lane & 3) * 8)) * 2u;
-  const uint32_t rd_off_a = (uint32_t)(64 * li + 16 * kb);
+  uint32_t rd_off[COLS];
+#pragma unroll
+  for (int c = 0; c < COLS; ++c)
+    rd_off[c] = (uint32_t)(WROW * (8 * kb + i) + 16 * q + 64 * (COLS == 2 ? c ^ ((i >> 1) & 1) : c));
+  // activations, loading side: lane l fetches 16 bytes (8 rows) of token l >> 2 and deposits them at
+  // 16 * l; consuming side: token li, block kb.  Tokens are 64 bytes apart, so tokens t, t + 4, t + 8,
+  // t + 12 would meet: token t keeps its four blocks in the order block ^ ((t >> 2) & 3).
+  const uint32_t voff_a = ((uint32_t)(lane >> 2) * p.K + (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2u;
+  const uint32_t rd_off_a = (uint32_t)(64 * li + 16 * (kb ^ ((li >> 2) & 3)));
   // as column j = i of B and D the lane stands for channels 128c + 32q + 8d + sm + h of the strip,
   // sm = (0,4,2,6)[i]; one dword of a scales row holds the pair h = 0, 1
   const int sm = (i & 1) * 4 + (i >> 1) * 2;
@@ -237,14 +255,25 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
         for (int h = 0; h < 2; ++h)
           Cm[c][d][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(h ? off1 : off0, Bm[c][d][h], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
   };
+  // One 32-row step.  The work of consecutive operands (16 channels x 32 rows each: 2 small MFMAs,
+  // 4 conversions, MT large MFMAs) is overlapped by hand: while operand o goes through the large
+  // MFMAs, operand o + 1 is in the small ones and the nibbles of operand o + 2 are being unpacked,
+  // so that no instruction waits for the one just before it.  A SIMD issues one VALU or matrix
+  // instruction per four cycles and a matrix instruction then occupies the matrix pipe for 8 (small)
+  // or 16 (large) cycles: VALU instructions placed between them ride along for free, instructions
+  // that wait for a result do not.  sched_barrier pins the order; the compiler still places waits.
   auto compute = [&](int buf, int row) {
-    // the step's data has landed once at most the loads of the DEPTH - 1 later steps are outstanding
-    // (loads complete in order; the scale loads in between only make this wait longer)
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (MT + NLD)) : "memory");
     const uint8_t* const slot = my_ring + buf * kSlot;
     uintx4 av[MT];
+    uintx4 wq[COLS][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) av[mt] = *(const uintx4*)(slot + kWBytes + mt * 1024 + rd_off_a);
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+      wq[c][0] = *(const uintx4*)(slot + rd_off[c]);
+      wq[c][1] = *(const uintx4*)(slot + rd_off[c] + 4 * WROW);
+    }
     if (row + 32 > p.K) {  // scalar: only a step that reaches the end of K
       asm volatile("");
       const bool ok = row + 8 * kb < p.K;
@@ -255,39 +284,58 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     bf16x8 bop[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) bop[mt] = __builtin_bit_cast(bf16x8, av[mt]);
+    constexpr int NO = COLS * 8;   // operands of the step: o = (c, d, h)
+    uint32_t ysh[2] = {0u, 0u};    // x >> 8 of the two rows of the current (c, d)
+    halfx4 A[3][2];                // unpacked nibbles of operand o % 3, rows rho = 0, 1
+    floatx4 Dq[2][2];              // scaled products of operand o % 2
+    auto unpack = [&](int o, int rho) {
+      const int c = o / 8, d = (o / 2) % 4, h = o % 2;
+      const uint32_t x = wq[c][rho][d];
+      if (h == 0) ysh[rho] = x >> 8;
+      const uint32_t m = h ? 0x00f000f0u : 0x000f000fu, k = h ? 0x64806480u : 0x64086408u;
+      A[o % 3][rho] = __builtin_bit_cast(halfx4, uintx2{(uint32_t)__builtin_amdgcn_bitop3_b32(x, m, k, 0x6a),
+                                                        (uint32_t)__builtin_amdgcn_bitop3_b32(ysh[rho], m, k, 0x6a)});
+    };
+    auto small = [&](int o, int rho) {
+      const int c = o / 8, d = (o / 2) % 4, h = o % 2;
+      Dq[o % 2][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[o % 3][rho], Bm[c][d][h], Cm[c][d][h], 0, 0, 0);
+    };
+    uintx4 aw;
+    auto convert = [&](int o, int rho) {
+      aw[2 * rho] = pack_bf16x2(Dq[o % 2][rho][0], Dq[o % 2][rho][1]);
+      aw[2 * rho + 1] = pack_bf16x2(Dq[o % 2][rho][2], Dq[o % 2][rho][3]);
+    };
+    auto large = [&](int o, int mt) {
+      const int c = o / 8, d = (o / 2) % 4, h = o % 2;
+      acc[c][d][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, aw), bop[mt], acc[c][d][h][mt], 0, 0, 0);
+    };
+    // fill: operands 0 and 1 unpacked, operand 0 through the small MFMAs
+    unpack(0, 0); unpack(0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    small(0, 0); unpack(1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    small(0, 1); unpack(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int c = 0; c < COLS; ++c) {
-      uintx4 wq[2];
-      wq[0] = *(const uintx4*)(slot + rd_off + 64 * c);
-      wq[1] = *(const uintx4*)(slot + rd_off + 64 * c + 4 * WROW);
+    for (int o = 0; o < NO; ++o) {
+      if (o + 1 < NO) small(o + 1, 0);
+      convert(o, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (o + 1 < NO) small(o + 1, 1);
+      convert(o, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (o + 2 < NO) unpack(o + 2, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      large(o, 0);
+      if (o + 2 < NO) unpack(o + 2, 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        floatx4 D[2][2];
-#pragma unroll
-        for (int rho = 0; rho < 2; ++rho) {
-          const uint32_t x = wq[rho][d];
-          const uint32_t y = x >> 8;
-          // nibbles (0,4), (2,6) as 1024 + u; (1,5), (3,7) as 1024 + 16u
-          const uint32_t p0 = __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a);
-          const uint32_t p1 = __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a);
-          const uint32_t p2 = __builtin_amdgcn_bitop3_b32(y, 0x000f000fu, 0x64086408u, 0x6a);
-          const uint32_t p3 = __builtin_amdgcn_bitop3_b32(y, 0x00f000f0u, 0x64806480u, 0x6a);
-          D[0][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p0, p2}), Bm[c][d][0], Cm[c][d][0], 0, 0, 0);
-          D[1][rho] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(halfx4, uintx2{p1, p3}), Bm[c][d][1], Cm[c][d][1], 0, 0, 0);
-        }
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const uintx4 a = {pack_bf16x2(D[h][0][0], D[h][0][1]), pack_bf16x2(D[h][0][2], D[h][0][3]),
-                            pack_bf16x2(D[h][1][0], D[h][1][1]), pack_bf16x2(D[h][1][2], D[h][1][3])};
-          const bf16x8 aop = __builtin_bit_cast(bf16x8, a);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[c][d][h][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop[mt], acc[c][d][h][mt], 0, 0, 0);
-        }
-      }
+      for (int mt = 1; mt < MT; ++mt) large(o, mt);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
+  STAMP(1);
   if (cnt > 0) {
     load_scales(k_begin);
 #pragma unroll
@@ -322,9 +370,11 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
           }
   }
 
+  STAMP(2);
   // loads for steps past the wave's last may still be on their way into the ring
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();  // every wave is done with its ring: the memory now carries the partial tiles
+  STAMP(3);
   // ---- add the waves' tiles through LDS.  Register r = (c * MT + mt) * 32 + e32 holds channel
   // strip * TN + 128 * c + 32 * (lane >> 4) + e32, token 16 * mt + (lane & 15): a lane owns 32
   // consecutive channels per column.  In the MFMA tiles e32 = 8d + e sits in
@@ -343,22 +393,38 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     for (int u = 0; u < RPW; ++u)
       bq[pass * RPW + u] = live && p.bias ? load_scale(p.bias, n0 + u, p.bias_is_bf16) : 0.0f;
   }
+  // Two buffers of kChunk registers per wave: a wave deposits pass + 1 (16 bytes per lane and
+  // instruction) before it collects pass, so the passes overlap and need one barrier each.  The sums
+  // over the waves run in wave order.
+  static_assert(RPW == 4, "a lane collects one 16-byte piece per wave and pass");
+  floatx4* const lds4 = (floatx4*)smem;
+  auto deposit = [&](int pass) {
+#pragma unroll
+    for (int q4 = 0; q4 < kChunk / 4; ++q4) {
+      floatx4 v;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int r = pass * kChunk + 4 * q4 + u;
+        const int c = r / (32 * MT), mt = (r / 32) % MT, ch = r % 32, d = ch / 8, e = ch % 8;
+        v[u] = acc[c][d][e & 1][mt][2 * ((e >> 1) & 1) + (e >> 2)];
+      }
+      lds4[(((pass & 1) * WAVES + wave) * (kChunk / 4) + q4) * 64 + lane] = v;
+    }
+  };
+  deposit(0);
+  __syncthreads();
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
+    if (pass + 1 < PASSES) deposit(pass + 1);
+    floatx4 s = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int cc = 0; cc < kChunk; ++cc) {
-      const int r = pass * kChunk + cc;
-      const int c = r / (32 * MT), mt = (r / 32) % MT, ch = r % 32, d = ch / 8, e = ch % 8;
-      lds[(wave * kChunk + cc) * 64 + lane] = acc[c][d][e & 1][mt][2 * ((e >> 1) & 1) + (e >> 2)];
+    for (int w2 = 0; w2 < WAVES; ++w2) {
+      const floatx4 v = lds4[(((pass & 1) * WAVES + w2) * (kChunk / 4) + wave) * 64 + lane];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s[u] = s[u] + v[u];
     }
-    __syncthreads();
 #pragma unroll
-    for (int u = 0; u < RPW; ++u) {
-      float s = 0.0f;
-#pragma unroll
-      for (int w2 = 0; w2 < WAVES; ++w2) s = s + lds[(w2 * kChunk + wave * RPW + u) * 64 + lane];
-      res[pass * RPW + u] = s * kUnscale;
-    }
+    for (int u = 0; u < RPW; ++u) res[pass * RPW + u] = s[u] * kUnscale;
     if (pass + 1 < PASSES) __syncthreads();
   }
 
@@ -369,6 +435,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // the whole strip by the plain loop below instead.
   // The sums travel in the threads' own order -- [pass][wave][lane][RPW floats], 64 KiB... per strip
   // R * 64 floats -- so that every wave stores and loads 64 x 16 contiguous bytes.
+  STAMP(4);
   static_assert(RPW == 4 || COLS == 1, "the hand-over moves 16 bytes per lane and pass");
   const __amdgpu_buffer_rsrc_t rh = make_rsrc(p.workspace + ((size_t)batch * p.strips + strip) * (R * 64), R * 64 * 4);
   constexpr int kDeviceScope = 16;  // sc1: the access is performed where every XCD sees it
@@ -396,7 +463,12 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
         for (int u = 0; u < RPW; ++u) res[pass * RPW + u] = bits_to_f32(other[pass][u]) + res[pass * RPW + u];
     }
   }
+  STAMP(5);
   if (finishes) epilogue_all_dispatch<PASSES * RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
+#ifdef XLA_AMD_STAMPS
+  asm volatile("" : "+v"(res[0]));
+#endif
+  STAMP(6);
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
     const int r0 = pass * kChunk + wave * RPW;
@@ -423,6 +495,13 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // each (token, channel) over the rows with ordinary arithmetic, in a fixed order, and overwrites
   // what the loop above produced for it.  The stores above must have landed first.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  STAMP(7);
+#ifdef XLA_AMD_STAMPS
+  if (lane == 0 && p.workspace) {
+    long long* st = (long long*)((char*)p.workspace + (8u << 20)) + ((size_t)blockIdx.x * WAVES + wave) * 8;
+    for (int z = 0; z < 8; ++z) st[z] = stamps[z];
+  }
+#endif
   __syncthreads();
   uint32_t any_bad = partner_ok ? 0u : 1u;
 #pragma unroll
@@ -522,7 +601,8 @@ int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
   const int waves = 8;
   const int b = (int)p.batch;
   // a SIMD serves its older wave first: the older class takes the larger share of the rows
-  int w0 = 7, w1 = 5;
+  // (7:5 measured best up to 32 tokens, 5:3 from there on, where the matrix pipe is the busier one)
+  int w0 = mt <= 2 ? 7 : 5, w1 = mt <= 2 ? 5 : 3;
   if (int v = GetOption("dequant_dot_skew")) { w0 = v / 10 % 10; w1 = v % 10; }
   if (w0 + w1 <= 0) { w0 = 1; w1 = 1; }
   auto split_rows = [&](int slices) {
