@@ -78,7 +78,7 @@ def test_c2_grouped_s4_with_bias_silu():
     new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=1))
     assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
     want_ws = ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 1, 8192, 28672, 21)
-    assert want_ws >= 112 * (16 * 256 * 4 + 8)   # a 16-token tile of sums and a flag per 256-channel strip
+    assert want_ws >= 112 * (16 * 256 * 4 + 16)   # a 16-token tile of sums and a flag per 256-channel strip
     check(new, r"custom-call\(%lhs, %w, %scales, %bias\)",
           r'epilogue = \\"BIAS_SILU\\", dequant_type = 16 : i32, dot_type = 11 : i32, epilogue_type = 11 : i32, '
           r'scale_group_size = 128 : i64')
@@ -87,8 +87,8 @@ def test_c2_grouped_s4_with_bias_silu():
     # eight tokens: two workgroups per 256-channel strip hand over through the scratch
     new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=8))
     assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4]"] and rf == []
-    assert ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 28672, 21) == 112 * (16 * 256 * 4 + 8)
-    check(new, r"\(bf16\[8,28672\]\{1,0\}, s8\[1835904\]\{0\}\) custom-call\(%lhs, %w, %scales, %bias\)")
+    assert ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 8, 8192, 28672, 21) == 112 * (16 * 256 * 4 + 16)
+    check(new, r"\(bf16\[8,28672\]\{1,0\}, s8\[1836800\]\{0\}\) custom-call\(%lhs, %w, %scales, %bias\)")
     # 64 tokens: the 224 strips fill the machine, no split, no scratch, a plain array result
     new, rw, rf = hlo.rewrite(hm.c2_s4_group(M=64))
     assert ffi.library().xla_amd_dequant_dot_workspace_bytes(1, 64, 8192, 28672, 21) == 0

@@ -119,7 +119,7 @@ def test_static_scratch_with_more_than_64_tokens(oracle):
     bit-identical to the workspace launcher (same split, same order of the two halves); one whose
     split needs more than the array is refused, as the [N,K] spelling of it is."""
     L = ffi.library()
-    M, K, N = 128, 2048, 2048      # 8 tiles, all split in two: 8 x (256 KiB + 8)
+    M, K, N = 128, 2048, 2048      # 8 tiles, all split in two: 8 x (256 KiB + 16)
     need = L.xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S8)
     assert 0 < need <= 8 << 20, need
     c = workloads.c1_s8_channel(M=M, K=K, N=N)

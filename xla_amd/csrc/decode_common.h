@@ -34,13 +34,18 @@ struct DecodeParams {
   int units_per_simd;
   int class_units[4];
   // s4x kernels, two workgroups per strip handing over inside the kernel: the producer's sums go to
-  // workspace[batch * strips + strip][16 x 256 floats], then flags[batch * strips + strip] is set
-  // to epoch (never 0).  s8x kernels: slices - 1 producers per strip, each with sums and a flag.
+  // workspace[batch * strips + strip][16 x 256 floats], then its flag is raised to
+  // HandOverTarget(epoch, generation of the strip): flags[2 * (batch * strips + strip)] is the flag,
+  // the word after it the generation.  s8x kernels: slices - 1 producers per strip, each with sums
+  // and a flag, then the strip's generation word.
   int pair;
   int rows_first;       // rows the producer takes; the finisher takes rows_per_slice from there on
   int units_per_simd2;  // the finisher's units per SIMD; its class split is class_units[2..3]
   unsigned long long* flags;
   unsigned long long epoch;
+  // Test aid (option "handover_test" = 1): producers never raise their flags and the waiting
+  // workgroup gives up after a few polls, so that its own fallback computes the result.
+  int handover_test;
   // 4-bit weights are unsigned (u4, 0..15) and zero_points, if not null, holds one u4 value per
   // scale ([scale_batch, K/group, N], packed like the weights): W' = (w - z) * scale
   int w_unsigned;
@@ -98,9 +103,26 @@ static __device__ __forceinline__ void buffer_load_words(__amdgpu_buffer_rsrc_t 
 }
 
 
+// What a raised hand-over flag holds: the launch's epoch in the upper half and the slot's
+// generation in the lower.  The generation is a word in the workspace next to the flag(s) that the
+// workgroup which waits on the slot increments as the last thing it does, whether the flags showed
+// or it gave up waiting: a flag raised late in one run (after the waiting side gave up) can then
+// not be taken for the flag of the next run, also when that run is a replay of the same captured
+// launch with the same epoch.  Every workgroup reads the generation as it starts (the one that
+// increments it does so after its bounded wait, by when every producer has long started).
+static __device__ __forceinline__ unsigned long long HandOverTarget(unsigned long long epoch,
+                                                                    const unsigned long long* generation) {
+  return (epoch << 32) | (__hip_atomic_load(generation, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffffffffull);
+}
+static __device__ __forceinline__ void HandOverNextGeneration(unsigned long long* generation, unsigned long long target) {
+  __hip_atomic_store(generation, (target + 1) & 0xffffffffull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+constexpr int kHandOverSpins = 1 << 22;  // polls before the waiting side computes everything itself
+constexpr int kHandOverTestSpins = 16;
+
 // A value no earlier launch of this process used and never 0: what the workgroups of one launch
-// write into their hand-over flags, so that whatever an earlier call (or nobody) left in the
-// workspace cannot be mistaken for it.
+// write into their hand-over flags (HandOverTarget), so that whatever an earlier call (or nobody)
+// left in the workspace cannot be mistaken for it.
 inline unsigned long long NextHandOverEpoch() {
   static std::atomic<unsigned long long> counter{0};
   static const unsigned long long nonce =

@@ -687,6 +687,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.epilogue = p.epilogue;
   dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
   dp.weights_shared = weights_shared;
+  dp.handover_test = GetOption("handover_test");
   dp.w_unsigned = u4;
   dp.zero_points = (const uint8_t*)p.zero_points;
   const bool ragged = p.group_sizes != nullptr;

@@ -97,6 +97,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   const int groups = p.K / group;
   // two workgroups per strip that hand over inside the kernel: slice 0 produces, slice 1 finishes
   const bool producer = p.pair && slice == 0, finisher = p.pair && slice == 1;
+  unsigned long long* const flag = p.flags + 2 * ((size_t)blockIdx.y * p.strips + strip);  // then the generation
+  unsigned long long target = 0;  // what the raised flag holds in this run (thread 0 raises or polls)
+  if (p.pair && threadIdx.x == 0) target = HandOverTarget(p.epoch, flag + 1);
 
   const uint32_t pitch = (uint32_t)p.N >> 1;
   const __amdgpu_buffer_rsrc_t rw =
@@ -439,13 +442,13 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   static_assert(RPW == 4 || COLS == 1, "the hand-over moves 16 bytes per lane and pass");
   const __amdgpu_buffer_rsrc_t rh = make_rsrc(p.workspace + ((size_t)batch * p.strips + strip) * (R * 64), R * 64 * 4);
   constexpr int kDeviceScope = 16;  // sc1: the access is performed where every XCD sees it
-  unsigned long long* const flag = p.flags + (size_t)batch * p.strips + strip;
   bool partner_ok = true;
   if (finisher) {
     if (threadIdx.x == 0) {
       int ok = 0;
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) { ok = 1; break; }
+      const int spins = p.handover_test ? kHandOverTestSpins : kHandOverSpins;
+      for (int spin = 0; spin < spins; ++spin) {
+        if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target) { ok = 1; break; }
         __builtin_amdgcn_s_sleep(8);
       }
       lds_partner = ok;
@@ -543,12 +546,15 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     }
   }
   if (p.pair) {
-    // the producer raises the flag once all its sums have landed; the finisher lowers it again so
-    // that a replay of the same launch (a captured graph) waits for the producer's new sums
+    // the producer raises the flag once all its sums have landed; the finisher, done with the slot
+    // whether the flag showed or not, moves the strip on to its next generation so that the next
+    // run (also a replay of this same launch from a captured graph) waits for new sums
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0)
-      __hip_atomic_store(flag, producer ? p.epoch : 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) {
+      if (finisher) HandOverNextGeneration(flag + 1, target);
+      else if (!p.handover_test) __hip_atomic_store(flag, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
@@ -566,10 +572,10 @@ int launch_s4x(const DecodeParams& dp, int batch, hipStream_t stream, const char
 }  // namespace
 
 // Bytes of workspace the in-kernel hand-over between the two workgroups of a 256-channel strip
-// needs: the producer's f32 sums, 16 KiB per (batch, strip), and one 8-byte flag each.
+// needs: the producer's f32 sums, 16 KiB per (batch, strip), and an 8-byte flag and generation each.
 size_t S4xPairWorkspaceBytes(int64_t batch, int64_t M, int64_t N) {
   (void)M;  // the producer's sums travel as whole 16-token tiles: 16 x 256 floats per strip
-  return (size_t)batch * ((N + 255) / 256) * (16 * 256 * 4 + 8);
+  return (size_t)batch * ((N + 255) / 256) * (16 * 256 * 4 + 16);  // sums, flag, generation
 }
 
 // Whole 128-byte lines per load and two workgroups per 256-channel strip: up to 16 tokens (the

@@ -130,7 +130,10 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
   constexpr int kDeviceScope = 16;  // sc1: the access is performed where every XCD sees it
   const int others = p.slices - 1;
   const size_t strip_index = (size_t)batch * p.strips + strip;
-  unsigned long long* const flags = p.flags + strip_index * (size_t)(others > 0 ? others : 1);
+  // per strip: one flag per producing slice, then the strip's generation
+  unsigned long long* const flags = p.flags + strip_index * (size_t)(others + 1);
+  unsigned long long target = 0;  // only read where it is used: thread 0 of a producer, the watching lanes
+  if (others > 0 && (finisher ? (wave == 0 && lane < others) : tid == 0)) target = HandOverTarget(p.epoch, flags + others);
   bool all_here = true;
   if (others > 0) {
     const __amdgpu_buffer_rsrc_t rh =
@@ -141,15 +144,16 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
           (uint32_t)((slice * (kWaves * 64) + tid) * 16), 0, kDeviceScope);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (tid == 0) __hip_atomic_store(flags + slice, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0 && !p.handover_test) __hip_atomic_store(flags + slice, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
     }
     if (wave == 0) {  // lane s < others watches slice s (at most 15 of them)
       int ok = 1;
       if (lane < others) {
         ok = 0;
-        for (int spin = 0; spin < (1 << 22); ++spin) {
-          if (__hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) { ok = 1; break; }
+        const int spins = p.handover_test ? kHandOverTestSpins : kHandOverSpins;
+        for (int spin = 0; spin < spins; ++spin) {
+          if (__hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target) { ok = 1; break; }
           __builtin_amdgcn_s_sleep(4);
         }
       }
@@ -176,8 +180,9 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
       }
 #pragma unroll
       for (int u = 0; u < RPW; ++u) res[u] = v[u] + res[u];
-      // lowered again so that a replay of the same launch (a captured graph) waits for new sums
-      if (tid < others) __hip_atomic_store(flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // the strip moves on to its next generation: the next run (also a replay of this launch from a
+      // captured graph) waits for new sums
+      if (tid == 0) HandOverNextGeneration(flags + others, target);
     }
   }
   if (all_here) {
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
       p.out[((size_t)batch * p.M + m) * p.N + n] = f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
     }
   }
-  if (tid < others) __hip_atomic_store(flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) HandOverNextGeneration(flags + others, target);  // a flag raised late belongs to the old generation
 }
 
 template <int STEPS>
@@ -259,7 +264,8 @@ size_t S8xWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
   if (!steps) return 0;
   const int64_t others = K / (256 * steps) - 1;
   const int64_t strips = (N + kStripChannels - 1) / kStripChannels;
-  return others > 0 ? (size_t)(batch * strips * others) * (kSumsPerStrip * 4 + 8) : 0;
+  // per strip: the producers' sums and flags, and one generation word
+  return others > 0 ? (size_t)(batch * strips) * ((size_t)others * (kSumsPerStrip * 4 + 8) + 8) : 0;
 }
 
 int LaunchDequantDotDecodeS8x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream) {

@@ -79,8 +79,9 @@ struct TiledParams {
   // to its own (first half + second half) and finishes the tile.
   int tail_first, tail_tiles;
   float* tail_sums;                 // [tail_tiles][32][512] x 16 bytes
-  unsigned long long* tail_flags;   // [tail_tiles]
-  unsigned long long epoch;         // value a raised flag holds for this launch
+  unsigned long long* tail_flags;   // [tail_tiles] x {flag, generation}
+  unsigned long long epoch;         // a raised flag holds HandOverTarget(epoch, the slot's generation)
+  int handover_test;                // test aid: second halves never raise their flag, first halves give up at once
   // Integer-weight kinds, ragged dot: a is [M,K] with rows sorted by group, b [groups,K,N], out [M,N].
   // Group g owns rows [sum of the sizes before it, + its size), read on the device.  The grid holds
   // tiles_n x ragged_slots workgroups; slot s is the s-th 256-row tile counted over all groups (a
@@ -278,6 +279,9 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     batch = t / tiles_per_batch;
     bid = t % tiles_per_batch;
   }
+  const bool waited_for_tail = role == 2;  // (the role changes if the wait gives up)
+  unsigned long long tail_target = 0;      // what the slot's raised flag holds in this run
+  if (WQ && role != 0 && threadIdx.x == 0) tail_target = HandOverTarget(p.epoch, p.tail_flags + 2 * tail_slot + 1);
   const bool ragged = WQ && p.group_sizes != nullptr;
   int m0r = 0, m_limit = p.M;  // ragged: first row of the tile and the end of its group's rows
   if (ragged) {
@@ -702,8 +706,9 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     // so it was dispatched before this one and is running or done.
     if (tid == 0) {
       int ok = 0;
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        if (__hip_atomic_load(p.tail_flags + tail_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.epoch) { ok = 1; break; }
+      const int spins = p.handover_test ? kHandOverTestSpins : kHandOverSpins;
+      for (int spin = 0; spin < spins; ++spin) {
+        if (__hip_atomic_load(p.tail_flags + 2 * tail_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tail_target) { ok = 1; break; }
         __builtin_amdgcn_s_sleep(4);
       }
       tail_arrived = ok;
@@ -733,7 +738,8 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
           }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (tid == 0) __hip_atomic_store(p.tail_flags + tail_slot, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0 && !p.handover_test)
+        __hip_atomic_store(p.tail_flags + 2 * tail_slot, tail_target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
   }
 
@@ -848,9 +854,9 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     d.m_base = m0 + wm * 128 + pass * 64;
     amax_bits = max(amax_bits, drain_dispatch<OUT_F8>(d, p.epilogue & ~1, p.bf16_dot, p.bf16_ops));
   }
-  // lowered again so that a replay of the same launch (a captured graph) waits for new sums
-  if (WQ && add_sums && tid == 0)
-    __hip_atomic_store(p.tail_flags + tail_slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the slot moves on to its next generation, whether the flag showed or not: the next run (also a
+  // replay of this launch from a captured graph) waits for new sums
+  if (WQ && waited_for_tail && tid == 0) HandOverNextGeneration(p.tail_flags + 2 * tail_slot + 1, tail_target);
   if (OUT_F8 && p.amax) {  // one atomic per wave into the result a fill kernel zeroed
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, off));
@@ -1049,7 +1055,7 @@ size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
   const int64_t tiles = batch * ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
   const int64_t tail = tiles % 256;
   if (tail == 0 || tail > 128 || tiles + tail > 0x7fffffff) return 0;
-  return (size_t)tail * (kTailSumsBytes + sizeof(unsigned long long));
+  return (size_t)tail * (kTailSumsBytes + 2 * sizeof(unsigned long long));  // sums, flag, generation
 }
 
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
@@ -1122,6 +1128,7 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
       tp.tail_sums = (float*)p.workspace;
       tp.tail_flags = (unsigned long long*)((char*)p.workspace + (size_t)tp.tail_tiles * kTailSumsBytes);
       tp.epoch = NextHandOverEpoch();
+      tp.handover_test = GetOption("handover_test");
     }
   }
   if (s4) {
@@ -1196,6 +1203,7 @@ int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream) {
     tp.tail_sums = (float*)p.workspace;
     tp.tail_flags = (unsigned long long*)((char*)p.workspace + (size_t)tp.tail_tiles * kTailSumsBytes);
     tp.epoch = NextHandOverEpoch();
+    tp.handover_test = GetOption("handover_test");
   }
   if (s4) {
     SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_nk_s4_rounded:tail2" : "dequant_dot_tiled_nk_s4_rounded");
