@@ -10,7 +10,8 @@ the benchmark's shapes and distributions, and resident in HBM before the timed r
 
 Prints ONE JSON line: `value` = algorithmic bytes of a step / wall time per step (GB/s);
 `roofline` = the step's slowest kernel against the 8 TB/s HBM peak, timed with events on the
-launch stream; `cpu_baseline` = the CPU oracle on the same workload; `kernels` = every kernel of
+launch stream (every per-kernel `ms` is the median over 21 event-bracketed batches of back-to-back
+launches, `ms_best` the fastest batch); `cpu_baseline` = the CPU oracle on the same workload; `kernels` = every kernel of
 the step; `other_configs` = the four other configurations, each with a `roofline` and a
 `cpu_baseline` of its own (the oracle on a stated sample of the same shape); `launch_floor_us` =
 what a kernel that does nothing costs per launch in the same back-to-back measurement.
@@ -97,30 +98,33 @@ def main():
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
+    BATCHES = 21
+
     def ev_time(fn, reps, warm=1):
-        """Average device time of fn() over `reps` back-to-back launches, events on the stream."""
+        """Device time of fn() per launch: `BATCHES` batches of `reps` back-to-back launches, each batch
+        bracketed by events on the launch stream.  Returns (median, best) of the batch means in ms."""
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        best = None
-        for _ in range(3):
+        ts = []
+        for _ in range(BATCHES):
             e0.record()
             for _ in range(reps):
                 fn()
             e1.record()
             e1.synchronize()
-            t = e0.elapsed_time(e1) / reps
-            best = t if best is None else min(best, t)
-        return best  # ms
+            ts.append(e0.elapsed_time(e1) / reps)
+        ts.sort()
+        return ts[len(ts) // 2], ts[0]  # ms
 
     # ---- what a plain copy reaches on this machine (context for every HBM fraction below) ------
     ca = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     cb = torch.empty_like(ca)
     st = torch.cuda.current_stream().cuda_stream
-    copy_ms = ev_time(lambda: ffi.debug_stream(cb.data_ptr(), ca.data_ptr(), ca.numel(), st), 10, warm=3)
+    copy_ms, _ = ev_time(lambda: ffi.debug_stream(cb.data_ptr(), ca.data_ptr(), ca.numel(), st), 4, warm=3)
     copy_gbs = 2 * ca.numel() / (copy_ms * 1e-3) / 1e9
-    read_ms = ev_time(lambda: ffi.debug_stream(None, ca.data_ptr(), ca.numel(), st), 10, warm=3)
+    read_ms, _ = ev_time(lambda: ffi.debug_stream(None, ca.data_ptr(), ca.numel(), st), 4, warm=3)
     read_gbs = ca.numel() / (read_ms * 1e-3) / 1e9
     if args.calibrate_copy:
         for _ in range(3):
@@ -155,10 +159,10 @@ def main():
     kernels = []
     for m, c in zip(MS2, calls):
         one = ffi.Replay([(c.target, c.frame)])
-        ms = ev_time(lambda: one.run(1), args.reps)
+        ms, ms_best = ev_time(lambda: one.run(1), args.reps)
         c.run()
         gbs = c2_bytes(m) / (ms * 1e-3) / 1e9
-        kernels.append({"workload": "C2 M=%d" % m, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
+        kernels.append({"workload": "C2 M=%d" % m, "kernel": ffi.last_kernel(), "ms": round(ms, 5), "ms_best": round(ms_best, 5),
                         "bytes": c2_bytes(m), "GB/s": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
                         "TFLOP/s": round(2 * m * K2 * N2 / (ms * 1e-3) / 1e12, 2),
                         "traffic": traffic.get("C2 M=%d" % m)})
@@ -166,14 +170,15 @@ def main():
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "workload": dom["workload"],
                 "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
                 "frac_of_xla_device_file_peak": round(dom["GB/s"] / HBM_PEAK_XLA_GBS, 4),
-                "traffic": dom["traffic"], "launch_ms": dom["ms"],
+                "traffic": dom["traffic"], "launch_ms": dom["ms"], "launch_ms_best": dom["ms_best"],
+                "timing": "median of %d event-bracketed batches of %d launches" % (BATCHES, args.reps),
                 "algorithmic_bytes": dom["bytes"],
                 "device_copy_GB/s": round(copy_gbs, 1), "device_read_GB/s": round(read_gbs, 1),
                 "frac_of_device_read_rate": round(dom["GB/s"] / read_gbs, 4)}
 
     # ---- the floor under every one-kernel figure: a kernel that does nothing, launched the same way
     st = torch.cuda.current_stream().cuda_stream
-    floor_ms = ev_time(lambda: ffi.launch_empty(st, 50, 256), 4, warm=2) / 50
+    floor_ms = ev_time(lambda: ffi.launch_empty(st, 50, 256), 4, warm=2)[0] / 50
 
     # ---- the other four configurations, each with its own roofline and CPU baseline ---------------
     import numpy as np
@@ -182,8 +187,8 @@ def main():
     if not args.skip_other:
         def entry(key, name, call, bytes_, flops, bound, dtype=None):
             # the half-millisecond kernels get 20 ms of launches to settle the clocks before timing
-            ms = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=40 if bound == "mfma" else 2)
-            e = {"workload": name, "key": key, "kernel": ffi.last_kernel(), "ms": round(ms, 5),
+            ms, ms_best = ev_time(lambda: call.run(), max(3, args.reps // 4), warm=40 if bound == "mfma" else 2)
+            e = {"workload": name, "key": key, "kernel": ffi.last_kernel(), "ms": round(ms, 5), "ms_best": round(ms_best, 5),
                  "GB/s": round(bytes_ / (ms * 1e-3) / 1e9, 1)}
             e["frac_hbm"] = round(e["GB/s"] / HBM_PEAK_GBS, 4)
             if flops:

@@ -348,7 +348,8 @@ def test_closed_form_activations_opt_in(oracle, epilogue):
         ffi.set_option("tiled_epilogue", 0)
     assert kern.startswith("fp8_scaled_dot_tiled")
     assert not np.array_equal(got, strict)                      # it did take the other path
-    n_floor = check_dot(got, reference(oracle, w), floor_for(w) + 2e-5, kern)
+    n_floor = check_dot(got, reference(oracle, w), floor_for(w) + 2e-5,
+                        "OPT-IN closed-form %s (floor + 2e-5), not the default path: %s" % (epilogue, kern))
     big = np.abs(dtypes.bf16_to_f32(strict)) > 1e-3
     from tests.gpu_util import bf16_ordinal
     assert np.all(np.abs(bf16_ordinal(got[big]) - bf16_ordinal(strict[big])) <= 2)

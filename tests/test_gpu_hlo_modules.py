@@ -195,12 +195,14 @@ def test_quantize_then_fp8_dot_module(oracle):
     check_dot(host_bf16(out), ref, dot_floor(fa, fb, C) + 1.2 * 2.0 ** -12 * np.sqrt((fa * fa) @ (fb * fb)), "quantize -> dot")
 
 
-@pytest.mark.parametrize("rmsnorm", [True, False])
-def test_c4_module_bit_exact(rmsnorm):
-    say("module C4 rmsnorm=%s" % rmsnorm)
+@pytest.mark.parametrize("rmsnorm,rsqrt", [(True, False), (False, False), (True, True)])
+def test_c4_module_bit_exact(rmsnorm, rsqrt):
+    """rsqrt: the reciprocal root written as one `rsqrt` op (evaluated as 1 / sqrt by the reference
+    evaluator, rsqrt.cc:178-193) rewrites to the same call and the same bits."""
+    say("module C4 rmsnorm=%s rsqrt=%s" % (rmsnorm, rsqrt))
     rows, cols = 24, 2048
     w = workloads.c4_quantize(rows, cols)
-    text = hm.c4_quantize(rows, cols, rmsnorm=rmsnorm)
+    text = hm.c4_quantize(rows, cols, rmsnorm=rmsnorm, rsqrt=rsqrt)
     args_dev = [dev_bf16(w["x"])] + ([dev_bf16(w["gamma"])] if rmsnorm else [])
     (q, s), rw, _ = hlo_runner.compile_and_run(text, args_dev)
     torch.cuda.synchronize()
