@@ -157,6 +157,15 @@ typedef struct XlaAmdDequantDot {
    * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  With
    * group_sizes the experts are [groups,N,K]. */
   int32_t rhs_contracting_dim;
+  /* Element type of out: BF16 (also 0) or F32 -- a dot whose f32 value is the result
+   * (fusion_emitter_int4_device_test.cc:101,205,320,508). */
+  int32_t out_dtype;
+  /* 1: out is [batch,N,M]: the dequantised weights were the lhs of the dot
+   * (Int4WeightsOnTheLhs, fusion_emitter_int4_device_test.cc:495-523); the epilogue must be DEFAULT. */
+  int32_t out_transposed;
+  /* 1: lhs (the activations) is stored [batch,K,M]: the dot contracts their major dimension
+   * (the "128,16" x "128,256" cases of fusion_emitter_int4_device_test.cc:609-645). */
+  int32_t lhs_k_major;
 } XlaAmdDequantDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);

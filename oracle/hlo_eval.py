@@ -47,14 +47,16 @@ def _tree32_sum_last(x):
 
 
 def _dot(a, b, lc, rc, lb, rb):
-    """f32 dot, accumulating over increasing k.  Supports [M,K]x[K,N], [M,K]x[N,K] and a leading
-    batch dimension."""
+    """f32 dot, accumulating over increasing k: result [lhs free, rhs free].  Either operand may
+    contract its minor or its major non-batch dimension; one leading batch dimension at most."""
     a = np.ascontiguousarray(a, np.float32)
     b = np.ascontiguousarray(b, np.float32)
     if lb:
-        assert lb == [0] and rb == [0] and lc == [2]
-        return np.stack([_dot(a[i], b[i], [1], [rc[0] - 1], [], []) for i in range(a.shape[0])])
-    assert lc == [1] and a.ndim == 2 and b.ndim == 2
+        assert lb == [0] and rb == [0] and a.ndim == 3 and b.ndim == 3
+        return np.stack([_dot(a[i], b[i], [lc[0] - 1], [rc[0] - 1], [], []) for i in range(a.shape[0])])
+    assert a.ndim == 2 and b.ndim == 2 and lc in ([0], [1]) and rc in ([0], [1])
+    if lc == [0]:
+        a = np.ascontiguousarray(a.T)
     if rc == [1]:
         b = np.ascontiguousarray(b.T)
     acc = np.zeros((a.shape[0], b.shape[1]), np.float32)

@@ -81,6 +81,8 @@ def lib():
         L.xo_dequant_dot_zp.restype = i32
         L.xo_dequant_dot_zp.argtypes = [vp, vp, i32, i32, vp, vp, i32, i32, vp, i32, i64, i64, i64, i64,
                                         i64, i32, i32, i32, vp]
+        L.xo_dequant_dot_f32.restype = i32
+        L.xo_dequant_dot_f32.argtypes = L.xo_dequant_dot_zp.argtypes
         L.xo_fp8_scaled_dot.restype = i32
         L.xo_fp8_scaled_dot.argtypes = [vp, vp, i32, vp, i32, vp, i32, i32, vp, i32, i64, i64, i64,
                                         i32, i32, i32, vp, vp, i32, vp, vp]
@@ -204,10 +206,12 @@ def tree32_sum(v):
 # ---- the three fused paths -------------------------------------------------
 
 def dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, bias=None, bias_ty="bf16",
-                group=None, dot_ty="f32", ep_ty="f32", epilogue="none", unsigned=False, zero_points=None):
+                group=None, dot_ty="f32", ep_ty="f32", epilogue="none", unsigned=False, zero_points=None,
+                f32_result=False):
     """a_bf16: uint16 [B,M,K] or [M,K]; w: int8 [..,K,N] (w_bits=8) or packed uint8 (w_bits=4,
     with logical shape given by scale/N); scale: [..,K/group,N].  Returns uint16 bf16 [..,M,N].
-    unsigned: the 4-bit weights are u4; zero_points: packed u4, one per scale: (w - z) * scale."""
+    unsigned: the 4-bit weights are u4; zero_points: packed u4, one per scale: (w - z) * scale.
+    f32_result: returns float32, the value before the final convert to bf16."""
     a = _c(a_bf16, np.uint16)
     batched = a.ndim == 3
     if not batched:
@@ -231,15 +235,16 @@ def dequant_dot(a_bf16, w, w_bits, scale, scale_ty, mul_ty, bias=None, bias_ty="
         bias = _c(bias, np.uint16 if bias_ty == "bf16" else np.float32)
         assert bias.size == N
         bp = _ptr(bias)
-    out = np.empty((B, M, N), np.uint16)
+    out = np.empty((B, M, N), np.float32 if f32_result else np.uint16)
     zp = None
     if zero_points is not None:
         zero_points = _c(zero_points, np.uint8)
         assert zero_points.size == (B * G * N + 1) // 2
         zp = _ptr(zero_points)
-    rc = lib().xo_dequant_dot_zp(_ptr(a), _ptr(w), w_bits, int(bool(unsigned)), zp, _ptr(s), TYPES[scale_ty],
-                                 TYPES[mul_ty], bp, TYPES[bias_ty], B, M, K, N, group, TYPES[dot_ty],
-                                 TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
+    fn = lib().xo_dequant_dot_f32 if f32_result else lib().xo_dequant_dot_zp
+    rc = fn(_ptr(a), _ptr(w), w_bits, int(bool(unsigned)), zp, _ptr(s), TYPES[scale_ty],
+            TYPES[mul_ty], bp, TYPES[bias_ty], B, M, K, N, group, TYPES[dot_ty],
+            TYPES[ep_ty], EPILOGUES[epilogue], _ptr(out))
     assert rc == 0
     return out if batched else out[0]
 

@@ -381,11 +381,14 @@ XO_API int xo_dequant_dot(const uint16_t* A, const void* w, int w_bits,
                            group, dot_ty, ep_ty, epi, out);
 }
 
-XO_API int xo_dequant_dot_zp(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
-                             const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
-                             const void* bias, int bias_ty, int64_t batch, int64_t M,
-                             int64_t K, int64_t N, int64_t group, int dot_ty,
-                             int ep_ty, int epi, uint16_t* out) {
+/* out32, when given, receives the value before the final convert to bf16: the result of a module
+ * whose root is the f32 dot (or f32-typed epilogue op) itself, as in
+ * fusion_emitter_int4_device_test.cc:101,205,320,508; out may then be NULL. */
+static int dequant_dot_impl(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
+                            const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
+                            const void* bias, int bias_ty, int64_t batch, int64_t M,
+                            int64_t K, int64_t N, int64_t group, int dot_ty,
+                            int ep_ty, int epi, uint16_t* out, float* out32) {
   if (!(w_bits == 8 || w_bits == 4) || group <= 0 || K % group != 0) return -1;
   if ((w_unsigned || zero_points) && w_bits != 4) return -1;
   const int64_t G = K / group;
@@ -436,15 +439,35 @@ XO_API int xo_dequant_dot_zp(const uint16_t* A, const void* w, int w_bits, int w
         if (bias)
           bv = bias_ty == XO_BF16 ? xo_bf16_to_f32(((const uint16_t*)bias)[n])
                                   : ((const float*)bias)[n];
-        for (int64_t m = 0; m < M; ++m)
-          out[((size_t)b * M + m) * N + n] =
-              epilogue(accs[m], dot_ty, ep_ty, bias != NULL, bv, epi);
+        for (int64_t m = 0; m < M; ++m) {
+          const float v = epilogue_value(accs[m], dot_ty, ep_ty, bias != NULL, bv, epi);
+          if (out) out[((size_t)b * M + m) * N + n] = xo_f32_to_bf16(v);
+          if (out32) out32[((size_t)b * M + m) * N + n] = v;
+        }
       }
     }
     free(col);
     free(accs);
   }
   return rc;
+}
+
+XO_API int xo_dequant_dot_zp(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
+                             const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
+                             const void* bias, int bias_ty, int64_t batch, int64_t M,
+                             int64_t K, int64_t N, int64_t group, int dot_ty,
+                             int ep_ty, int epi, uint16_t* out) {
+  return dequant_dot_impl(A, w, w_bits, w_unsigned, zero_points, scale, scale_ty, mul_ty, bias, bias_ty, batch, M,
+                          K, N, group, dot_ty, ep_ty, epi, out, NULL);
+}
+
+XO_API int xo_dequant_dot_f32(const uint16_t* A, const void* w, int w_bits, int w_unsigned,
+                              const uint8_t* zero_points, const void* scale, int scale_ty, int mul_ty,
+                              const void* bias, int bias_ty, int64_t batch, int64_t M,
+                              int64_t K, int64_t N, int64_t group, int dot_ty,
+                              int ep_ty, int epi, float* out32) {
+  return dequant_dot_impl(A, w, w_bits, w_unsigned, zero_points, scale, scale_ty, mul_ty, bias, bias_ty, batch, M,
+                          K, N, group, dot_ty, ep_ty, epi, NULL, out32);
 }
 
 /* --------------------------------------------------------- fp8 scaled dot */

@@ -98,3 +98,22 @@ def check_f8_result(got_codes, ref_codes, ref_value, d_scale, divides, abs_floor
     differ = int((got_codes != ref_codes).sum())
     FLOOR_LOG.append((what or "f8 result", "codes other than the oracle's (inside the window)", differ, int(bad.size)))
     return differ
+
+
+def check_dot_f32(got_f32, ref_f32, abs_floor, what=""):
+    """The same rule for a dot whose f32 value is the result itself: within 2 bf16 ulp of the oracle's
+    value (2**-7 of its magnitude bounds that from below), or within `abs_floor`."""
+    g = np.asarray(got_f32, np.float64)
+    r = np.asarray(ref_f32, np.float64)
+    assert g.shape == r.shape, (g.shape, r.shape)
+    ok = np.abs(g - r) <= np.abs(r) * 2.0 ** -7
+    near = np.abs(g - r) <= abs_floor
+    both_nan = np.isnan(g) & np.isnan(r)
+    bad = ~(ok | near | both_nan)
+    if bad.any():
+        idx = np.argwhere(bad)[:8]
+        raise AssertionError("%s: %d of %d f32 outputs differ by more than 2 bf16 ulp (and the floor): %s"
+                             % (what, int(bad.sum()), bad.size, [(tuple(i), float(g[tuple(i)]), float(r[tuple(i)])) for i in idx]))
+    n_floor = int((~ok & near).sum())
+    FLOOR_LOG.append((what or "dot (f32 result)", "within the floor only", n_floor, int(bad.size)))
+    return n_floor

@@ -350,3 +350,39 @@ def test_unrewritten_module_does_not_run():
     text = "HloModule m\nENTRY e {\n  a = f32[4] parameter(0)\n  ROOT b = f32[4] add(a, a)\n}\n"
     with pytest.raises(NotImplementedError, match="was not rewritten into a custom call"):
         hlo_runner.compile_and_run(text, [torch.zeros(4, device="cuda")])
+
+
+@pytest.mark.parametrize("case", hm.INT4_DOT_CASES, ids=[c[0] for c in hm.INT4_DOT_CASES])
+@pytest.mark.parametrize("weights_on_lhs", [False, True])
+def test_reference_int4_shape_table(case, weights_on_lhs):
+    """The modules of Int4WeightsOnTheLhs[WithBatchDim] / Int4WeightsOnTheRhs over Int4TestCases
+    (fusion_emitter_int4_device_test.cc:495-645): f32 dot of unscaled s4 weights on either side, both
+    contracting dimensions on both operands, with and without a batch dimension.  Integer weights
+    and bf16 activations: compared with the op-by-op evaluation of the unrewritten module (the
+    reference compares at 1e-5 .. 1e-2, :603-604, :557-558)."""
+    from tests.gpu_util import check_dot_f32
+    name, lhs, rhs, lc, rc, out_dims = case
+    say("module %s %s" % ("lhs" if weights_on_lhs else "rhs", name))
+    import zlib
+    rng = np.random.default_rng(zlib.crc32(name.encode()) + int(weights_on_lhs))
+    w_dims, a_dims = (lhs, rhs) if weights_on_lhs else (rhs, lhs)
+    w = rng.integers(-8, 8, size=w_dims).astype(np.int8)
+    a = dtypes.f32_to_bf16(rng.standard_normal(a_dims).astype(np.float32))
+    text = hm.int4_weights_dot(case, weights_on_lhs)
+    wd, ad = dev_u8(dtypes.pack_s4(w)), dev_bf16(a)
+    out, rw, rf = hlo_runner.compile_and_run(text, [wd, ad] if weights_on_lhs else [ad, wd])
+    torch.cuda.synchronize()
+    assert len(rw) == 1 and "f32 result" in rw[0] and rf == [], (rw, rf)
+    assert list(out.shape) == list(out_dims) and out.dtype == torch.float32
+    ref = reference(text, [w, a] if weights_on_lhs else [a, w])
+    # floor from sum |a| |w| over k, laid out like the result
+    rank = len(lhs)
+    w_c, a_c = (lc, rc) if weights_on_lhs else (rc, lc)
+    wa = np.abs(w.astype(np.float64))
+    aa = np.abs(dtypes.bf16_to_f32(a).astype(np.float64))
+    wkn = wa if w_c == rank - 2 else np.swapaxes(wa, -1, -2)        # [..,K,N]
+    amk = aa if a_c == rank - 1 else np.swapaxes(aa, -1, -2)        # [..,M,K]
+    s = amk @ wkn                                                   # [..,M,N]
+    if weights_on_lhs:
+        s = np.swapaxes(s, -1, -2)
+    check_dot_f32(out.cpu().numpy(), ref, 8 * 2.0 ** -24 * s, "int4 table %s %s" % (name, ffi.last_kernel()))

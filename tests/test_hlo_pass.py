@@ -336,8 +336,9 @@ ENTRY main {
     check(new, r"custom-call\(%a, %w.s4, %s\)", r"dequant_type = 16 : i32, dot_type = 16 : i32")
 
 
-def test_weights_on_the_lhs_and_minor_batch_dim_are_left_alone():
-    # weights as lhs (fusion_emitter_int4_device_test.cc:93-104 orientation): not this kernel's layout
+def test_weights_on_the_lhs_are_taken_and_a_minor_batch_dim_is_left_alone():
+    # weights as lhs (fusion_emitter_int4_device_test.cc:93-104 orientation), activations [K,M]: one call
+    # whose result is [N,M]
     text = """HloModule t
 ENTRY main {
   w = s4[128,256] parameter(0)
@@ -351,7 +352,9 @@ ENTRY main {
 }
 """
     new, rw, _ = hlo.rewrite(text)
-    assert rw == [] and "custom-call" not in new
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s4, weights as lhs, activations [K,M]]"], rw
+    check(new, r"ROOT %\S+ = bf16\[256,4\]\{1,0\} custom-call\(%a, %w, %s\)",
+          r"scale_group_size = 0 : i64, lhs_contracting_dim = 0 : i64, result_transposed = true")
     # RejectTritonFusionForWithMinorBatchDim (fusion_emitter_int4_device_test.cc:698-716)
     text = """HloModule t
 ENTRY main {
@@ -383,7 +386,9 @@ def test_dot_with_second_user_keeps_epilogue_outside():
     text = hm.c1_s8_channel(4, 64, 32).replace("ROOT %out = bf16[4,32] convert(%dot)",
                                                "%out = bf16[4,32] convert(%dot)\n  ROOT %t = (bf16[4,32], f32[4,32]) tuple(%out, %dot)")
     new, rw, rf = hlo.rewrite(text)
-    assert rw == [] and any("is f32" in r for r in rf)
+    # the f32 dot itself is a value the module keeps: the call returns it, the convert stays outside
+    assert rw == ["dot -> xla_amd.dequant_dot [DEFAULT, s8, f32 result]"] and rf == []
+    check(new, r"f32\[4,32\]\{1,0\}(, s8\[\d+\]\{0\}\))? custom-call\(", r"%out = bf16\[4,32\](\{1,0\})? convert\(%dot\S*\)")
 
 
 def test_quantize_near_misses_are_refused_with_reasons():
@@ -609,3 +614,46 @@ def test_ragged_dot_over_k_minor_experts():
     bad = hm.k_minor_ragged_s8_experts(32, 512, 256, 4).replace("rhs_group_dims={0}", "rhs_group_dims={1}")
     _, rw, rf = hlo.rewrite(bad)
     assert rw == [] and any("group dimension leading the weights" in r for r in rf)
+
+
+@pytest.mark.parametrize("case", hm.INT4_DOT_CASES, ids=[c[0] for c in hm.INT4_DOT_CASES])
+@pytest.mark.parametrize("weights_on_lhs", [False, True])
+def test_reference_int4_shape_table_is_taken(case, weights_on_lhs):
+    """Every shape of Int4TestCases (fusion_emitter_int4_device_test.cc:609-645), weights on either
+    side: an f32 dot of unscaled converted s4 weights becomes one call with unit scales, the
+    contracting dimensions as attributes and -- weights on the lhs -- a transposed result."""
+    name, lhs, rhs, lc, rc, out = case
+    text = hm.int4_weights_dot(case, weights_on_lhs)
+    new, rw, rf = hlo.rewrite(text)
+    assert len(rw) == 1 and rf == [], (rw, rf)
+    rank = len(lhs)
+    w_c, a_c = (lc, rc) if weights_on_lhs else (rc, lc)
+    tags = ["DEFAULT", "s4"]
+    if w_c == rank - 1:
+        tags.append("weights [N,K]")
+    if weights_on_lhs:
+        tags.append("weights as lhs")
+    if a_c == rank - 2:
+        tags.append("activations [K,M]")
+    tags.append("f32 result")
+    assert rw == ["dot -> xla_amd.dequant_dot [%s]" % ", ".join(tags)], rw
+    n = (lhs if weights_on_lhs else rhs)[rank - (2 if w_c == rank - 1 else 1)]
+    check(new, r"f32\[\] constant\(1\)", r"f32\[%d\]\{0\} broadcast\(%%\S+\), dimensions=\{\}" % n,
+          r"f32\[%s\]\{[0-9,]+\}(, s8\[\d+\]\{0\}\))? custom-call\(%%a, %%w, %%\S+unit_scales\)" % ",".join(str(v) for v in out),
+          r"dequant_type = 11 : i32, dot_type = 11 : i32")
+    assert ("result_transposed = true" in new) == weights_on_lhs
+    assert ("lhs_contracting_dim = 0" in new) == (a_c == rank - 2)
+    assert ("rhs_contracting_dim = 1" in new) == (w_c == rank - 1)
+    assert sorted(set(opcodes(new)) - {"get-tuple-element"}) == ["broadcast", "constant", "custom-call", "parameter"]
+
+
+def test_f32_result_with_scales_and_epilogue():
+    """The value leaving the pattern may be f32: C2's module without its final convert keeps the f32
+    SiLU value as the result (epilogue ops f32-typed, dequantise multiply bf16-typed)."""
+    text = hm.c2_s4_group(M=8, K=256, N=64, group=64)
+    assert "ROOT %out = bf16[8,64] convert(" in text
+    root = re.search(r"ROOT %out = bf16\[8,64\] convert\((%\w+)\)", text).group(1)
+    text = re.sub(r"  ROOT %out = bf16\[8,64\] convert\(%\w+\)\n", "", text).replace("  %s = " % root, "  ROOT %s = " % root)
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, f32 result]"], (rw, rf)
+    check(new, r"f32\[8,64\]\{1,0\}")

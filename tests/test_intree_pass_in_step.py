@@ -36,7 +36,8 @@ def test_refusal_reasons_are_the_same_in_both_files():
 def test_custom_call_targets_and_attributes_are_the_same():
     a, b = open(OFFLINE_CC).read(), open(INTREE_CC).read()
     for needle in ('"xla_amd.fp8_scaled_dot"', '"xla_amd.dequant_dot"', '"xla_amd.rowwise_quantize_fp8"',
-                   "scale_group_size = ", "rhs_contracting_dim = ", "d_scale_multiplies = ", "rmsnorm = ",
+                   "scale_group_size = ", "rhs_contracting_dim = ", "lhs_contracting_dim = 0", "result_transposed = true",
+                   "d_scale_multiplies = ", "rmsnorm = ",
                    "dequant_type = ", "dot_type = ", "epilogue_type = ", "0.7978845608028654", "0.044715",
                    "-448.0", "448.0", "__op$block_scaled_dot"):
         assert needle in a and needle in b, needle

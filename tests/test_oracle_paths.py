@@ -419,3 +419,39 @@ def test_ragged_dot_composition_is_pinned(oracle):
     over = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", [10, 10, 0, 0], bias=w["bias"])
     assert np.array_equal(over[:10], oracle.dequant_dot(w["lhs"][:10], w["weights"][0], 8, w["scales"][0], "f32", "f32", bias=w["bias"]))
     assert np.array_equal(over[10:], oracle.dequant_dot(w["lhs"][10:], w["weights"][1], 8, w["scales"][1], "f32", "f32", bias=w["bias"]))
+
+
+# ---- f32 result of the dequantize-dot (the dot's own value is the module's result) ----------------
+
+def test_dequant_dot_f32_result_is_the_value_before_the_final_convert(oracle):
+    """fusion_emitter_int4_device_test.cc:101,205,320,508 end in an f32 dot.  The f32 result is pinned
+    three ways: rounding it gives the bf16 result bit for bit (every epilogue); one-hot activations
+    read single dequantised weights back exactly; and float64 on a small dot bounds it to f32
+    summation noise -- with the rows of the weights reversed it must not."""
+    rng = np.random.default_rng(5)
+    M, K, N, g = 5, 256, 48, 64
+    a = dtypes.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    sc = dtypes.f32_to_bf16(rng.uniform(1e-3, 2e-2, size=(K // g, N)).astype(np.float32))
+    bias = dtypes.f32_to_bf16(rng.standard_normal((N,)).astype(np.float32))
+    wp = dtypes.pack_s4(w)
+    for epi in ("none", "relu", "gelu_tanh", "silu"):
+        v32 = oracle.dequant_dot(a, wp, 4, sc, "bf16", "bf16", bias=bias, group=g, epilogue=epi, f32_result=True)
+        v16 = oracle.dequant_dot(a, wp, 4, sc, "bf16", "bf16", bias=bias, group=g, epilogue=epi)
+        assert v32.dtype == np.float32 and np.array_equal(dtypes.f32_to_bf16(v32), v16), epi
+    # one-hot rows: out[m, n] = bf16(w[k_m, n] * s) exactly, as an f32
+    hot = np.zeros((M, K), np.float32)
+    ks = [0, 63, 64, 200, 255]
+    hot[np.arange(M), ks] = 1.0
+    got = oracle.dequant_dot(dtypes.f32_to_bf16(hot), wp, 4, sc, "bf16", "bf16", group=g, f32_result=True)
+    s32 = dtypes.bf16_to_f32(sc)
+    want = np.stack([dtypes.bf16_to_f32(dtypes.f32_to_bf16(w[k].astype(np.float32) * s32[k // g])) for k in ks])
+    assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # float64 on the rounded weights
+    wd = dtypes.bf16_to_f32(dtypes.f32_to_bf16(w.astype(np.float32) * np.repeat(s32, g, axis=0))).astype(np.float64)
+    a64 = dtypes.bf16_to_f32(a).astype(np.float64)
+    ref = a64 @ wd
+    v32 = oracle.dequant_dot(a, wp, 4, sc, "bf16", "bf16", group=g, f32_result=True)
+    tol = 2.0 ** -22 * (np.abs(a64) @ np.abs(wd))
+    assert np.all(np.abs(v32 - ref) <= tol)
+    assert not np.all(np.abs(v32 - a64 @ wd[::-1]) <= tol)

@@ -58,7 +58,20 @@ struct DecodeParams {
   int group_sizes_64;
   int ragged_groups;  // number of groups (the kernels that do not carry it in grid.y)
   int ragged_chunks;  // grid.z of a ragged launch: 64-row chunks any one group may need (1 up to 64 rows)
+  // Result and activation layouts beyond bf16 [batch,M,N] / [batch,M,K] (the kernels that honour them
+  // store through StoreResult; the launcher keeps every other kernel away from such calls):
+  int out_f32;         // out holds f32, not bf16
+  int out_transposed;  // out is [batch,N,M]: the dequantised weights were the lhs of the dot
+  int lhs_k_major;     // lhs is [batch,K,M] (one-thread-per-output kernels only)
 };
+
+// One result element; row = batch * M + m over the flattened [batch * M, N] result.
+static __device__ __forceinline__ void StoreResult(const DecodeParams& p, size_t row, int n, float v) {
+  size_t idx = row * (size_t)p.N + (size_t)n;
+  if (p.out_transposed) idx = ((row / (size_t)p.M) * (size_t)p.N + (size_t)n) * (size_t)p.M + row % (size_t)p.M;
+  if (p.out_f32) reinterpret_cast<float*>(p.out)[idx] = v;
+  else p.out[idx] = f32_to_bf16(v);
+}
 
 // Rows of a ragged dot that group g covers, read on the device: [*begin, *begin + *rows), clamped to
 // [0, M] so that sizes that do not add up cannot reach outside the operands.

@@ -398,6 +398,11 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = res[pass * RPW + u];
     } else {
+      if (p.out_f32 | p.out_transposed) {
+#pragma unroll
+        for (int u = 0; u < RPW; ++u) StoreResult(p, (size_t)m_begin + m, n0 + u, res[pass * RPW + u]);
+        continue;
+      }
       uint16_t* dst = p.out + ((size_t)m_begin + m) * p.N + n0;
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = f32_to_bf16(res[pass * RPW + u]);
@@ -428,8 +433,7 @@ __global__ __launch_bounds__(256) void dequant_dot_finalize_kernel(DecodeParams 
   if (mode == kFactored)
     v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n, p.scale_is_bf16);
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  p.out[(size_t)batch * total + idx] =
-      f32_to_bf16(epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, (size_t)batch * p.M + idx / p.N, n, epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 // Any shape, any alignment: one thread per output, k in increasing order.  Correct for every
@@ -451,7 +455,9 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
       if (m >= b0 && m < b0 + rows) { wbatch = g; k_end = p.K; break; }
     }
   }
-  const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
+  // activations [batch,M,K], or [batch,K,M] when the dot contracts their major dimension
+  const uint16_t* a = p.lhs + (p.lhs_k_major ? (size_t)batch * p.M * p.K + m : ((size_t)batch * p.M + m) * p.K);
+  const size_t a_step = p.lhs_k_major ? (size_t)p.M : 1;
   const size_t wbase = (size_t)wbatch * p.K * p.N;
   const size_t sbase = (size_t)(p.scale_batched ? wbatch : 0) * (p.K / p.group) * p.N;
   float acc = 0.0f;
@@ -471,11 +477,10 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
     float s = load_scale(p.scales, sbase + (size_t)(k / p.group) * p.N + n, p.scale_is_bf16);
     float wv = (float)wi * s;
     if (mode == kRounded) wv = round_bf16(wv);
-    acc = acc + bf16_to_f32(a[k]) * wv;
+    acc = acc + bf16_to_f32(a[(size_t)k * a_step]) * wv;
   }
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  p.out[(size_t)batch * total + idx] =
-      f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, (size_t)batch * p.M + m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 template <int WBITS, int VEC, int MT, int WAVES, int MODE>
@@ -688,6 +693,17 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
   dp.weights_shared = weights_shared;
   dp.handover_test = GetOption("handover_test");
+  if (p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16 && p.out_dtype != XLA_FFI_DataType_F32)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: out must be BF16 or F32");
+  dp.out_f32 = p.out_dtype == XLA_FFI_DataType_F32;
+  dp.out_transposed = p.out_transposed != 0;
+  dp.lhs_k_major = p.lhs_k_major != 0;
+  // A result other than bf16 [batch,M,N], or activations stored [batch,K,M], keep the call on the
+  // kernels that store through StoreResult / read lhs with a stride: the first-generation decode
+  // kernel (and its token chunks), the [N,K] streaming kernel and the one-thread-per-output kernels.
+  const bool plain = !dp.out_f32 && !dp.out_transposed && !dp.lhs_k_major;
+  if (!plain && p.group_sizes)
+    return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot writes bf16 [M,N] from lhs [M,K]");
   dp.w_unsigned = u4;
   dp.zero_points = (const uint8_t*)p.zero_points;
   const bool ragged = p.group_sizes != nullptr;
@@ -724,7 +740,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // average 96 rows; below that most tiles would be nearly empty and the 64-row chunks of the decode
   // kernel do less work.  The sizes themselves are only known on the device.
   const bool ragged_tiles = ragged && (force == 3 || (p.batch > 0 && p.M / p.batch >= 96));
-  if (force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && (!ragged || ragged_tiles)) {
+  if (plain && force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && (!ragged || ragged_tiles)) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
@@ -756,7 +772,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // (4-bit weights with group-factored sums hold two sets of accumulators per tile: chunks of 32 tokens)
   const int64_t chunk = mode == kGroupFactored && s4 ? 32 : 64;
   if (force != 1 && force != 3 && aligned && mode_ok && p.M > chunk && p.K >= 32 && p.N % 2 == 0 && !ragged &&
-      decode_shape(chunk, &mt64, &vec64, &nv64)) {
+      !dp.out_transposed && !dp.lhs_k_major && decode_shape(chunk, &mt64, &vec64, &nv64)) {
     const size_t wbytes = (size_t)p.K * p.N * (s4 ? 1 : 2) / 2;
     const size_t ssz = p.scale_dtype == XLA_FFI_DataType_BF16 ? 2 : 4;
     const size_t sbytes = p.scale_batch == p.batch && p.batch > 1 ? (size_t)(p.K / p.group) * p.N * ssz : 0;
@@ -778,7 +794,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
         sub.batch = part == 0 ? whole : 1;
         if (sub.M == 0 || sub.batch == 0) continue;
         sub.lhs = (const uint16_t*)p.lhs + ((size_t)b * p.M + m0) * p.K;
-        sub.out = (uint16_t*)p.out + ((size_t)b * p.M + m0) * p.N;
+        sub.out = (char*)p.out + ((size_t)b * p.M + m0) * p.N * (dp.out_f32 ? 4 : 2);
         const int rc = LaunchDequantDotImpl(sub, stream, true);
         if (rc) return rc;
         if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)chunk);
@@ -788,18 +804,18 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     return 0;
   }
 
-  if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= chunk || ragged) && p.K >= 32) {
+  if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= chunk || ragged) && p.K >= 32 && !dp.lhs_k_major) {
     int mt, vec, nv;
     const bool shape_ok = decode_shape(p.M > 64 ? 64 : p.M, &mt, &vec, &nv);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // s4 with bf16 group scales and a bf16-typed multiply: the kernels that dequantise through the
     // 4x4x4 matrix instruction
-    if (shape_ok && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1 && !ragged) {
+    if (shape_ok && plain && s4 && mode == kRounded && GetOption("dequant_dot_x") != 1 && !ragged) {
       const int rc = LaunchDequantDotDecodeS4x(dp, p, stream);
       if (rc >= 0) return rc;
     }
     // small s8 matrices with per-channel scales under an f32-typed multiply: one launch
-    if (shape_ok && !s4 && mode == kFactored && per_channel && !weights_shared && !ragged) {
+    if (shape_ok && plain && !s4 && mode == kFactored && per_channel && !weights_shared && !ragged) {
       const int rc = LaunchDequantDotDecodeS8x(dp, p, stream);
       if (rc >= 0) return rc;
     }

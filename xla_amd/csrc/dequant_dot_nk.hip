@@ -354,6 +354,10 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
             for (int i = 0; i < 4; ++i)
               if (n + i < p.N) dst[i] = v[i];
           }
+        } else if (p.out_f32 | p.out_transposed) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < p.N) StoreResult(p, (size_t)a_batch * p.M + m_first + m0 + m, n + i, v[i]);
         } else if (quads) {
           *reinterpret_cast<uintx2*>(p.out + o) = uintx2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         } else {
@@ -385,7 +389,9 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
       if (m >= b0 && m < b0 + rows) { wbatch = g; k_end = p.K; break; }
     }
   }
-  const uint16_t* a = p.lhs + ((size_t)batch * p.M + m) * p.K;
+  // activations [batch,M,K], or [batch,K,M] when the dot contracts their major dimension
+  const uint16_t* a = p.lhs + (p.lhs_k_major ? (size_t)batch * p.M * p.K + m : ((size_t)batch * p.M + m) * p.K);
+  const size_t a_step = p.lhs_k_major ? (size_t)p.M : 1;
   const size_t wrow = ((size_t)wbatch * p.N + n) * p.K;                     // in elements
   const size_t srow = ((size_t)(p.scale_batched ? wbatch : 0) * p.N + n) * G;
   float acc = 0.0f;
@@ -404,10 +410,10 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
     }
     float wv = (float)wi * load_scale(p.scales, srow + k / p.group, p.scale_is_bf16);
     if (mode == kRounded) wv = round_bf16(wv);
-    acc = acc + bf16_to_f32(a[k]) * wv;
+    acc = acc + bf16_to_f32(a[(size_t)k * a_step]) * wv;
   }
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  p.out[(size_t)batch * total + idx] = f32_to_bf16(epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, (size_t)batch * p.M + m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 // Ragged dot: rows past the last group are a dot of nothing, epilogue(0).  Workgroup (x, y) takes 256
@@ -524,7 +530,8 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
     if ((int64_t)1 << s == p.group) group_shift = s;
   const bool ragged = p.group_sizes != nullptr;
   // (a ragged dot takes the tiled kernel -- 256-row tiles per group -- once the groups average 96 rows)
-  if (p.M > 64 && (!ragged || GetOption("dequant_dot_kernel") == 3 || p.M / p.batch >= 96) &&
+  const bool plain = !dp.out_f32 && !dp.out_transposed && !dp.lhs_k_major;  // else: no tiled kernel
+  if (plain && p.M > 64 && (!ragged || GetOption("dequant_dot_kernel") == 3 || p.M / p.batch >= 96) &&
       GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
     const int rc = LaunchDequantDotPrefillNk(p, stream);
     if (rc >= 0) return rc;  // -1: the tiled kernel does not take it (or token chunks are cheaper)
@@ -534,6 +541,7 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
               p.batch * ((p.M + 15) / 16) <= 65535 && GetOption("dequant_dot_kernel") != 1 &&
               (!ragged || (double)p.M * p.N * 2 < 2147483648.0);
   if (group_shift < 0) fast = false;  // groups are powers of two, or one scale per channel
+  if (dp.lhs_k_major) fast = false;   // the streaming kernel reads activations [M,K]
   if ((double)p.scale_batch * p.N * (p.K / p.group) * 4 >= 2147483648.0) fast = false;  // 32-bit offsets into the scales
   if (mode == kRounded && !per_channel && p.group % kp != 0) fast = false;
   if (mode == kFactored && !per_channel) fast = false;  // an f32 multiply by scales that do not cover whole steps

@@ -381,7 +381,7 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Buffer* bias = nargs > bias_at ? d.Arg(bias_at, kFloatMask, 1, 1, "bias") : nullptr;
   if (((!has_zp && nargs > 4) || nargs > 5) && d.ok())
     return InvalidArgument(f->api, "xla_amd.dequant_dot: five operands are lhs, weights, scales, zero_points (U4), bias");
-  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16), 2, 3, "out");
+  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F32), 2, 3, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
   CommonAttrs a;
   DecodeCommonAttrs(d, &a);
@@ -389,8 +389,14 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   const bool has_group_size = d.Int("scale_group_size", &group_size);
   int64_t rcd = 0;  // 1: weights [..,N,K], scales [N] | [B,N] | [N,K/g] | [B,N,K/g]
   d.Int("rhs_contracting_dim", &rcd);
+  int64_t lcd = -1;  // which of lhs's last two dimensions the dot contracts: 1 (default) = the minor one, lhs [..,M,K]
+  const bool has_lcd = d.Int("lhs_contracting_dim", &lcd);
+  uint8_t transposed_attr = 0;  // the dequantised weights were the dot's lhs: out is [..,N,M]
+  d.Scalar("result_transposed", XLA_FFI_DataType_PRED, &transposed_attr, 1);
+  const bool transposed = transposed_attr != 0;
   if (!d.ok()) return d.Error();
   const bool nk = rcd == 1;
+  const bool lhs_k_major = has_lcd && lcd == 0;
 
   // ragged: lhs [M,K] (rows sorted by group), weights [groups,K,N], out [M,N]; the groups take the
   // place of the batch for weights and scales
@@ -398,21 +404,25 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   const bool batched = lhs->rank == 3 || ragged;
   XlaAmdDequantDot p{};
   p.batch = ragged ? (w->rank == 3 ? w->dims[0] : 0) : batched ? lhs->dims[0] : 1;
-  p.M = lhs->dims[lhs->rank - 2];
-  p.K = lhs->dims[lhs->rank - 1];
+  p.M = lhs->dims[lhs->rank - (lhs_k_major ? 1 : 2)];
+  p.K = lhs->dims[lhs->rank - (lhs_k_major ? 2 : 1)];
   p.N = w->dims[w->rank - (nk ? 2 : 1)];
   p.rhs_contracting_dim = (int32_t)rcd;
   std::string why;
   if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
+  else if (has_lcd && lcd != 0 && lcd != 1) why = "lhs_contracting_dim must be 0 (lhs [..,K,M]) or 1 (lhs [..,M,K])";
+  else if (ragged && (transposed || lhs_k_major || out->dtype != XLA_FFI_DataType_BF16))
+    why = "a ragged dot writes bf16 [M,N] from lhs [M,K]";
+  else if (transposed && a.epilogue != 0) why = "a transposed result takes the DEFAULT epilogue only";
   else if (nk && !has_group_size) why = "weights [N,K] come with scale_group_size";
   else if (ragged && (lhs->rank != 2 || w->rank != 3)) why = "a ragged dot takes lhs [M,K] and weights [groups,K,N]";
   else if (ragged && gs->dims[0] != p.batch) why = "group_sizes must have one entry per group of weights";
   else if (!ragged && w->rank != lhs->rank) why = "lhs and weights must have the same rank";
   else if (w->dims[w->rank - (nk ? 1 : 2)] != p.K) why = "contracting dimensions differ";
   else if (!ragged && batched && w->dims[0] != p.batch) why = "batch dimensions differ";
-  else if (out->rank != lhs->rank || out->dims[out->rank - 1] != p.N ||
-           out->dims[out->rank - 2] != p.M || (!ragged && batched && out->dims[0] != p.batch))
-    why = "result shape must be [batch,]M,N";
+  else if (out->rank != lhs->rank || out->dims[out->rank - (transposed ? 2 : 1)] != p.N ||
+           out->dims[out->rank - (transposed ? 1 : 2)] != p.M || (!ragged && batched && out->dims[0] != p.batch))
+    why = transposed ? "result shape must be [batch,]N,M" : "result shape must be [batch,]M,N";
   else if (!(nk && group_size > 0) && sc->dims[sc->rank - 1] != p.N) why = "scales must have N as their last dimension";
   else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
   else if (zp && w->dtype != XLA_FFI_DataType_U4) why = "zero points go with U4 weights";
@@ -476,6 +486,9 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   p.bias_dtype = bias ? bias->dtype : XLA_FFI_DataType_F32;
   p.dequant_type = a.dequant_type; p.dot_type = a.dot_type; p.epilogue_type = a.epilogue_type;
   p.epilogue = a.epilogue;
+  p.out_dtype = out->dtype;
+  p.out_transposed = transposed ? 1 : 0;
+  p.lhs_k_major = lhs_k_major ? 1 : 0;
   void* stream;
   if (XLA_FFI_Error* e = GetStream(f, &stream)) return e;
   return LaunchStatus(f, xla_amd_launch_dequant_dot(&p, stream));

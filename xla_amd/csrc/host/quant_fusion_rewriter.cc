@@ -16,8 +16,8 @@
 //                                           codegen/emitters/reduction.cc:840-991)
 //
 // Every refusal is recorded with a reason (the reference logs them with VLOG(1),
-// gemm_rewriter.cc:295,316,1248).  The kernels produce bf16 (f8 for the quantizer), so a
-// pattern is only taken when the value leaving it has that type.
+// gemm_rewriter.cc:295,316,1248).  The kernels produce bf16 (f8 for the quantizer; the dequantize-dot
+// also the f32 value itself), so a pattern is only taken when the value leaving it has such a type.
 #include "quant_fusion_rewriter.h"
 
 #include <math.h>
@@ -174,7 +174,10 @@ bool MatchSilu(Instr* out, Instr* x) {
 // Walks forward from the dot: optional convert, optional + broadcast(bias) along the minor
 // dimension, optional activation, optional final convert to bf16.  Returns false when what
 // leaves the chain is not bf16.
-bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_result_in = nullptr) {
+// allow_f32_result: the kernels behind the call can write the f32 value itself (the dequantize-dot);
+// otherwise the value leaving the pattern must be bf16.
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_result_in = nullptr,
+                   bool allow_f32_result = false) {
   const bool allow_f8_result = f8_result_in != nullptr;
   Instr* cur = dot;
   const int64_t rank = dot->shape.rank();
@@ -300,7 +303,7 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_
     }
   }
   step_convert();
-  if (cur->shape.dtype != "bf16") {
+  if (cur->shape.dtype != "bf16" && !(allow_f32_result && cur->shape.dtype == "f32")) {
     *why = "the value leaving the dot pattern is " + cur->shape.dtype + ", the kernels produce bf16";
     return false;
   }
@@ -587,6 +590,14 @@ bool MatchQWeights(Instr* op, bool k_minor, QWeights* out, std::string* why) {
     *out = {w, sc, ty, zero, d3[k_minor ? 1 : 0]};
     return true;
   }
+  if (op->Is("convert")) {
+    // convert(s4|s8|u4 -> float) straight into the dot: no scale at all (Int4WeightsOnTheRhs / OnTheLhs,
+    // fusion_emitter_int4_device_test.cc:495-606); the caller supplies scales of one
+    Instr* w;
+    if (!IntSource(op, ty, &w) || w->shape.dims != op->shape.dims) return false;
+    *out = {w, nullptr, ty, nullptr, 0};
+    return true;
+  }
   if (!op->Is("multiply")) return false;
   Instr *sc = nullptr, *cv = nullptr;
   const std::vector<int64_t> bdims = k_minor ? (rank == 2 ? std::vector<int64_t>{0} : std::vector<int64_t>{0, 1})
@@ -607,17 +618,31 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   const int64_t rank = dot->shape.rank();
   auto lb = dot->DimsAttr("lhs_batch_dims"), rb = dot->DimsAttr("rhs_batch_dims");
   auto lc = dot->DimsAttr("lhs_contracting_dims"), rc = dot->DimsAttr("rhs_contracting_dims");
-  // weights [..,N,K]: the dot contracts their minor dimension (fusion_emitter_int4_device_test.cc:867-892)
-  const bool k_minor = rc == std::vector<int64_t>{rank - 1};
+  // The dequantised weights are usually the rhs of the dot; they may be its lhs as well
+  // (Int4WeightsOnTheLhs, fusion_emitter_int4_device_test.cc:495-523): the result is then [..,N,M].
+  // Either operand may contract its minor or its major (non-batch) dimension: weights [..,K,N] or
+  // [..,N,K] (:867-892), activations [..,M,K] or [..,K,M] (the shape table :609-645).
+  bool weights_lhs = false;
+  bool k_minor = rc == std::vector<int64_t>{rank - 1};
   if (!MatchQWeights(dot->operands[1], k_minor, &q, &why)) {
-    if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
-    return false;
+    std::string why_lhs;
+    const bool lhs_k_minor = lc == std::vector<int64_t>{rank - 1};
+    if (dot->operands.size() == 2 && MatchQWeights(dot->operands[0], lhs_k_minor, &q, &why_lhs)) {
+      weights_lhs = true;
+      k_minor = lhs_k_minor;
+    } else {
+      if (!why.empty()) log->refusals.push_back(dot->name + ": " + why);
+      else if (!why_lhs.empty()) log->refusals.push_back(dot->name + ": " + why_lhs);
+      return false;
+    }
   }
   auto refuse = [&](const std::string& w) {
     log->refusals.push_back(dot->name + ": quantized weights found but not rewritten: " + w);
     return false;
   };
-  Instr* lhs = dot->operands[0];
+  Instr* lhs = dot->operands[weights_lhs ? 1 : 0];  // the activations
+  const auto& ac = weights_lhs ? rc : lc;           // their contracting dimension, and the weights'
+  const auto& wc = weights_lhs ? lc : rc;
   Instr* inner;
   if (lhs->Is("convert") && ConvertFrom(lhs, "bf16", &inner) && lhs->shape.dtype == "f32") lhs = inner;
   if (lhs->shape.dtype != "bf16") return refuse("the activation must be bf16 (or its convert to f32)");
@@ -625,25 +650,39 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   if (rank == 3 && (lb != std::vector<int64_t>{0} || rb != std::vector<int64_t>{0}))
     return refuse("the batch dimension must be dimension 0 of both operands");
   if (rank == 2 && !lb.empty()) return refuse("unexpected batch dimensions");
-  if (lc != std::vector<int64_t>{rank - 1} || (rc != std::vector<int64_t>{rank - 2} && !k_minor))
+  const bool lhs_k_major = ac == std::vector<int64_t>{rank - 2};
+  if ((ac != std::vector<int64_t>{rank - 1} && !lhs_k_major) || (wc != std::vector<int64_t>{rank - 2} && !k_minor))
     return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] or [..,N,K]; s4 with a "
                   "minor batch dimension is rejected as in gemm_fusion.cc:1572-1590");
-  const bool four_bit = q.w->shape.dtype == "s4" || q.w->shape.dtype == "u4";
-  if (four_bit && q.w->shape.dims.back() % 2 != 0)
-    return refuse("s4 rows must hold an even number of values");
+  // (4-bit rows of an odd number of values are packed across row ends, xla/packing.cc:142-170: the
+  // one-thread-per-output kernel reads them by flat index)
   if (q.zero && q.w->shape.dtype != "u4") return refuse("zero points are taken with u4 weights only");
   if (q.zero && q.zero->shape.dims != q.scale->shape.dims)
     return refuse("zero points must have the shape of the scales (one per scale)");
-  if (q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
+  if (q.scale && q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
-  if (!MatchEpilogue(dot, &ep, &why)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, nullptr, /*allow_f32_result=*/true)) return refuse(why);
+  if (weights_lhs && (ep.bias || !ep.act.empty()))
+    return refuse("with the weights as the lhs of the dot only the plain dot is taken (a bias would run along the other dimension)");
 
   const int64_t B = rank == 3 ? lhs->shape.dims[0] : 1;
-  const int64_t M = lhs->shape.dims[rank - 2], K = lhs->shape.dims[rank - 1], N = q.w->shape.dims[rank - (k_minor ? 2 : 1)];
+  const int64_t M = lhs->shape.dims[rank - (lhs_k_major ? 1 : 2)], K = lhs->shape.dims[rank - (lhs_k_major ? 2 : 1)];
+  const int64_t N = q.w->shape.dims[rank - (k_minor ? 2 : 1)];
+  std::string dequant_ty = q.type;
+  if (!q.scale) {
+    // no multiply in the module: the integers themselves are the weights.  One scale per channel, all
+    // ones, under an f32-typed multiply gives exactly those values (convert(int -> bf16) is exact).
+    Instr* one = comp->Insert(Make(comp->UniqueName(dot->name + ".one"), "constant", Shape::Array("f32", {}), {}), dot);
+    one->literal = "1";
+    auto bc = Make(comp->UniqueName(dot->name + ".unit_scales"), "broadcast", Shape::Array("f32", {N}), {one});
+    bc->attrs.emplace_back("dimensions", "{}");
+    q.scale = comp->Insert(std::move(bc), dot);
+    dequant_ty = "f32";
+  }
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
-  std::vector<Shape> results = {Shape::Array("bf16", dot->shape.dims)};
+  std::vector<Shape> results = {Shape::Array(ep.tail->shape.dtype, dot->shape.dims)};
   const int32_t wdt = q.w->shape.dtype == "s4" ? 21 : q.w->shape.dtype == "u4" ? 22 : 2;
   auto sizer = k_minor ? opt.dequant_nk_workspace_bytes : opt.dequant_workspace_bytes;
   size_t ws = sizer ? sizer(B, M, K, N, wdt) : 0;
@@ -652,13 +691,17 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   // [K/g,N], or [N,K/g] next to weights [N,K]
   const int64_t group_size = q.groups ? K / q.groups : 0;
   Instr* call = EmitCall(comp, ep.tail, "xla_amd.dequant_dot", ops, results,
-                         CommonConfig(ep, q.type, dot->shape.dtype) + ", scale_group_size = " +
+                         CommonConfig(ep, dequant_ty, dot->shape.dtype) + ", scale_group_size = " +
                              std::to_string(group_size) + " : i64" +
-                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
+                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : "") +
+                             (lhs_k_major ? ", lhs_contracting_dim = 0 : i64" : "") +
+                             (weights_lhs ? ", result_transposed = true" : ""));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
-                          (q.zero ? " with zero points" : "") + (k_minor ? ", weights [N,K]" : "") + "]");
+                          (q.zero ? " with zero points" : "") + (k_minor ? ", weights [N,K]" : "") +
+                          (weights_lhs ? ", weights as lhs" : "") + (lhs_k_major ? ", activations [K,M]" : "") +
+                          (ep.tail->shape.dtype == "f32" ? ", f32 result" : "") + "]");
   return true;
 }
 

@@ -246,7 +246,8 @@ class LaunchDequantDot(C.Structure):
                 ("scale_dtype", C.c_int32), ("bias_dtype", C.c_int32), ("dequant_type", C.c_int32),
                 ("dot_type", C.c_int32), ("epilogue_type", C.c_int32), ("epilogue", C.c_int32),
                 ("zero_points", C.c_void_p), ("group_sizes", C.c_void_p), ("group_sizes_dtype", C.c_int32),
-                ("rhs_contracting_dim", C.c_int32)]
+                ("rhs_contracting_dim", C.c_int32), ("out_dtype", C.c_int32), ("out_transposed", C.c_int32),
+                ("lhs_k_major", C.c_int32)]
 
 
 _lib = None

@@ -540,3 +540,56 @@ ENTRY %main {{
   ROOT %out = bf16[{M},{N}] convert(%z)
 }}
 """
+
+
+# The shape table of the reference's parametrised int4 tests (Int4TestCases,
+# fusion_emitter_int4_device_test.cc:609-645): name, lhs dims, rhs dims, lhs and rhs contracting
+# dimension, result dims.  The 3-d cases carry a batch dimension 0 on both operands.
+INT4_DOT_CASES = [
+    ("int4_dot_128_16_x_128_256", (128, 16), (128, 256), 0, 0, (16, 256)),
+    ("int4_dot_128_16_x_256_128", (128, 16), (256, 128), 0, 1, (16, 256)),
+    ("int4_dot_16_128_x_256_128", (16, 128), (256, 128), 1, 1, (16, 256)),
+    ("int4_dot_16_128_x_128_256", (16, 128), (128, 256), 1, 0, (16, 256)),
+    ("int4_dot_1_128_x_256_128", (1, 128), (256, 128), 1, 1, (1, 256)),
+    ("int4_dot_128_1_x_256_128", (128, 1), (256, 128), 0, 1, (1, 256)),
+    ("int4_dot_16_128_x_128_1", (16, 128), (128, 1), 1, 0, (16, 1)),
+    ("int4_dot_16_128_x_1_128", (16, 128), (1, 128), 1, 1, (16, 1)),
+    ("dot_8_128_16_x_8_128_256", (8, 128, 16), (8, 128, 256), 1, 1, (8, 16, 256)),
+    ("dot_8_128_16_x_8_256_128", (8, 128, 16), (8, 256, 128), 1, 2, (8, 16, 256)),
+    ("dot_8_16_128_x_8_256_128", (8, 16, 128), (8, 256, 128), 2, 2, (8, 16, 256)),
+    ("dot_8_16_128_x_8_128_256", (8, 16, 128), (8, 128, 256), 2, 1, (8, 16, 256)),
+    ("dot_8_1_128_x_8_256_128", (8, 1, 128), (8, 256, 128), 2, 2, (8, 1, 256)),
+    ("dot_8_128_1_x_8_256_128", (8, 128, 1), (8, 256, 128), 1, 2, (8, 1, 256)),
+    ("dot_8_16_128_x_8_128_1", (8, 16, 128), (8, 128, 1), 2, 1, (8, 16, 1)),
+    ("dot_8_16_128_x_8_1_128", (8, 16, 128), (8, 1, 128), 2, 2, (8, 16, 1)),
+]
+
+
+def int4_weights_dot(case, weights_on_lhs):
+    """The dot of Int4WeightsOnTheLhs[WithBatchDim] / Int4WeightsOnTheRhs
+    (fusion_emitter_int4_device_test.cc:495-606) as the module reads before GemmFusion wraps it into a
+    fusion: convert(s4 -> s8 -> bf16) of one operand straight into an f32 dot, no scale."""
+    name, lhs, rhs, lc, rc, out = case
+    d = lambda t: ",".join(str(v) for v in t)
+    batch = "lhs_batch_dims={0}, rhs_batch_dims={0}, " if len(lhs) == 3 else ""
+    if weights_on_lhs:
+        return f"""HloModule lhs_{name}
+
+ENTRY %entry_computation {{
+  %w = s4[{d(lhs)}] parameter(0)
+  %w.s8 = s8[{d(lhs)}] convert(%w)
+  %w.b16 = bf16[{d(lhs)}] convert(%w.s8)
+  %a = bf16[{d(rhs)}] parameter(1)
+  ROOT %dot = f32[{d(out)}] dot(%w.b16, %a), {batch}lhs_contracting_dims={{{lc}}}, rhs_contracting_dims={{{rc}}}
+}}
+"""
+    return f"""HloModule rhs_{name}
+
+ENTRY %entry_computation {{
+  %a = bf16[{d(lhs)}] parameter(0)
+  %w = s4[{d(rhs)}] parameter(1)
+  %w.s8 = s8[{d(rhs)}] convert(%w)
+  %w.b16 = bf16[{d(rhs)}] convert(%w.s8)
+  ROOT %dot = f32[{d(out)}] dot(%a, %w.b16), {batch}lhs_contracting_dims={{{lc}}}, rhs_contracting_dims={{{rc}}}
+}}
+"""

@@ -7,7 +7,8 @@ xla/backends/gpu/runtime/custom_call_thunk.cc:110-157).
 
 Only what a rewritten quantized-inference module contains is supported besides the custom
 calls: parameters, tuples, get-tuple-element, and scalar glue (constants, converts and
-divides of rank-0 values, converts of rank-1 scale vectors), which run as torch ops.  Anything else raises: this is not an HLO
+divides of rank-0 values, converts of rank-1 scale vectors, a rank-1 broadcast of a scalar), which
+run as torch ops.  Anything else raises: this is not an HLO
 interpreter, and a module the pass did not fully rewrite does not run here.
 """
 import re
@@ -88,8 +89,9 @@ class Executable:
                 v = x[0][int(ins["attrs"]["index"])]
             elif op == "tuple":
                 v = list(x)
-            elif not sh.get("tuple") and (sh["dims"] == [] or (op == "convert" and len(sh["dims"]) == 1)):
-                v = self._scalar_glue(ins, x)   # scalars, and the widening convert of a vector of scales
+            elif not sh.get("tuple") and (sh["dims"] == [] or (op in ("convert", "broadcast") and len(sh["dims"]) == 1)):
+                # scalars, the widening convert of a vector of scales, a vector of one repeated scalar
+                v = self._scalar_glue(ins, x)
             else:
                 raise NotImplementedError("instruction %s = %s(...) was not rewritten into a custom call; "
                                           "this runner only executes custom calls" % (ins["name"], op))
@@ -104,6 +106,8 @@ class Executable:
             return torch.tensor(float(ins["literal"].strip("{} ")), dtype=ty, device="cuda")
         if op == "convert":
             return x[0].to(ty)
+        if op == "broadcast" and x[0].dim() == 0:
+            return x[0].to(ty).expand(ins["shape"]["dims"]).contiguous()
         if op == "divide":
             return (x[0] / x[1]).to(ty)
         if op == "multiply":

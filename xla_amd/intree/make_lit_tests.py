@@ -42,6 +42,9 @@ def cases():
         ("quant_fusion_rewriter_rowwise_quantize_rsqrt", hm.c4_quantize(8, 64, rsqrt=True)),
         ("quant_fusion_rewriter_rowwise_quantize_plain", hm.c4_quantize(8, 64, rmsnorm=False)),
         ("quant_fusion_rewriter_quantize_then_dot", hm.quantize_then_fp8_dot(8, 64, 32)),
+        ("quant_fusion_rewriter_int4_weights_on_the_rhs_f32", hm.int4_weights_dot(hm.INT4_DOT_CASES[1], False)),
+        ("quant_fusion_rewriter_int4_weights_on_the_lhs_f32", hm.int4_weights_dot(hm.INT4_DOT_CASES[3], True)),
+        ("quant_fusion_rewriter_int4_weights_on_the_lhs_batched", hm.int4_weights_dot(hm.INT4_DOT_CASES[9], True)),
         ("quant_fusion_rewriter_refuses_far_gelu_constant", gelu_far),
     ]
 
@@ -63,7 +66,7 @@ def expectations(text):
         lines.append("// CHECK-SAME: api_version=API_VERSION_TYPED_FFI")
         for attr in cfg.split(", "):
             key = attr.split(" = ")[0]
-            if key in ("epilogue", "rmsnorm", "scale_group_size", "rhs_contracting_dim", "d_scale_multiplies",
+            if key in ("epilogue", "rmsnorm", "scale_group_size", "rhs_contracting_dim", "lhs_contracting_dim", "result_transposed", "d_scale_multiplies",
                        "dequant_type", "dot_type", "epilogue_type"):
                 lines.append("// CHECK-SAME: %s" % attr.replace("\\", ""))
     if not lines:

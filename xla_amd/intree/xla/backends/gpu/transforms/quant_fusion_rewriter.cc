@@ -157,7 +157,9 @@ bool MatchSilu(Instr* out, Instr* x) {
 // Walks forward from the dot: optional convert, optional + broadcast(bias) along the minor
 // dimension, optional activation, optional final convert to bf16 -- or, for f32-typed f8 dots, the
 // f8 result tail convert(clamp(-448, v / z | v * z, 448)) with its optional amax.
-bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result) {
+// allow_f32_result: the kernels behind the call can write the f32 value itself (the dequantize-dot);
+// otherwise the value leaving the pattern must be bf16.
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result, bool allow_f32_result = false) {
   Instr* cur = dot;
   const int64_t rank = Rank(dot);
   ep->ops_type = Ty(dot);
@@ -271,7 +273,7 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_res
     }
   }
   step_convert();
-  if (Ty(cur) != BF16) {
+  if (Ty(cur) != BF16 && !(allow_f32_result && Ty(cur) == F32)) {
     *why = "the value leaving the dot pattern is " + TyName(Ty(cur)) + ", the kernels produce bf16";
     return false;
   }
@@ -532,6 +534,14 @@ bool MatchQWeights(Instr* op, bool k_minor, QWeights* out, std::string* why) {
     *out = {w, sc, ty, zero, d3[k_minor ? 1 : 0]};
     return true;
   }
+  if (op->opcode() == HloOpcode::kConvert) {
+    // convert(s4|s8|u4 -> float) straight into the dot: no scale at all (Int4WeightsOnTheRhs / OnTheLhs,
+    // fusion_emitter_int4_device_test.cc:495-606); the caller supplies scales of one
+    Instr* w;
+    if (!IntSource(op, ty, &w) || Dims(w) != Dims(op)) return false;
+    *out = {w, nullptr, ty, nullptr, 0};
+    return true;
+  }
   if (op->opcode() != HloOpcode::kMultiply) return false;
   Instr *sc = nullptr, *cv = nullptr;
   const std::vector<int64_t> bdims = k_minor ? (rank == 2 ? std::vector<int64_t>{0} : std::vector<int64_t>{0, 1})
@@ -551,17 +561,32 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   std::string why;
   const int64_t rank = Rank(dot);
   const DotDimensionNumbers& dn = dot->dot_dimension_numbers();
-  // weights [..,N,K]: the dot contracts their minor dimension (fusion_emitter_int4_device_test.cc:867-892)
-  const bool k_minor = dn.rhs_contracting_dimensions_size() == 1 && dn.rhs_contracting_dimensions(0) == rank - 1;
+  auto contracts = [](const auto& dims, int64_t d) { return dims.size() == 1 && dims[0] == d; };
+  // The dequantised weights are usually the rhs of the dot; they may be its lhs as well
+  // (Int4WeightsOnTheLhs, fusion_emitter_int4_device_test.cc:495-523): the result is then [..,N,M].
+  // Either operand may contract its minor or its major (non-batch) dimension: weights [..,K,N] or
+  // [..,N,K] (:867-892), activations [..,M,K] or [..,K,M] (the shape table :609-645).
+  bool weights_lhs = false;
+  bool k_minor = contracts(dn.rhs_contracting_dimensions(), rank - 1);
   if (!MatchQWeights(dot->mutable_operand(1), k_minor, &q, &why)) {
-    if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
-    return false;
+    std::string why_lhs;
+    const bool lhs_k_minor = contracts(dn.lhs_contracting_dimensions(), rank - 1);
+    if (dot->operand_count() == 2 && MatchQWeights(dot->mutable_operand(0), lhs_k_minor, &q, &why_lhs)) {
+      weights_lhs = true;
+      k_minor = lhs_k_minor;
+    } else {
+      if (!why.empty()) log(absl::StrCat(dot->name(), ": ", why));
+      else if (!why_lhs.empty()) log(absl::StrCat(dot->name(), ": ", why_lhs));
+      return false;
+    }
   }
   auto refuse = [&](const std::string& w) {
     log(absl::StrCat(dot->name(), ": quantized weights found but not rewritten: ", w));
     return false;
   };
-  Instr* lhs = dot->mutable_operand(0);
+  Instr* lhs = dot->mutable_operand(weights_lhs ? 1 : 0);  // the activations
+  const auto& ac = weights_lhs ? dn.rhs_contracting_dimensions() : dn.lhs_contracting_dimensions();
+  const auto& wc = weights_lhs ? dn.lhs_contracting_dimensions() : dn.rhs_contracting_dimensions();
   Instr* inner;
   if (ConvertFrom(lhs, BF16, &inner) && Ty(lhs) == F32) lhs = inner;
   if (Ty(lhs) != BF16) return refuse("the activation must be bf16 (or its convert to f32)");
@@ -570,27 +595,36 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   if (rank == 3 && (!is0(dn.lhs_batch_dimensions()) || !is0(dn.rhs_batch_dimensions())))
     return refuse("the batch dimension must be dimension 0 of both operands");
   if (rank == 2 && dn.lhs_batch_dimensions_size() != 0) return refuse("unexpected batch dimensions");
-  if (dn.lhs_contracting_dimensions_size() != 1 || dn.rhs_contracting_dimensions_size() != 1 ||
-      dn.lhs_contracting_dimensions(0) != rank - 1 || (dn.rhs_contracting_dimensions(0) != rank - 2 && !k_minor))
+  const bool lhs_k_major = contracts(ac, rank - 2);
+  if ((!contracts(ac, rank - 1) && !lhs_k_major) || (!contracts(wc, rank - 2) && !k_minor))
     return refuse("needs lhs [..,M,K] contracting K and weights [..,K,N] or [..,N,K]; s4 with a "
                   "minor batch dimension is rejected as in gemm_fusion.cc:1572-1590");
-  const bool four_bit = Ty(q.w) == S4 || Ty(q.w) == U4;
-  if (four_bit && q.w->shape().dimensions(rank - 1) % 2 != 0)
-    return refuse("s4 rows must hold an even number of values");
+  // (4-bit rows of an odd number of values are packed across row ends, xla/packing.cc:142-170: the
+  // one-thread-per-output kernel reads them by flat index)
   if (q.zero && Ty(q.w) != U4) return refuse("zero points are taken with u4 weights only");
   if (q.zero && Dims(q.zero) != Dims(q.scale))
     return refuse("zero points must have the shape of the scales (one per scale)");
-  if (q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
+  if (q.scale && q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
-  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false, /*allow_f32_result=*/true)) return refuse(why);
+  if (weights_lhs && (ep.bias || !ep.act.empty()))
+    return refuse("with the weights as the lhs of the dot only the plain dot is taken (a bias would run along the other dimension)");
 
   const int64_t B = rank == 3 ? lhs->shape().dimensions(0) : 1;
-  const int64_t M = lhs->shape().dimensions(rank - 2), K = lhs->shape().dimensions(rank - 1);
+  const int64_t M = lhs->shape().dimensions(rank - (lhs_k_major ? 1 : 2)), K = lhs->shape().dimensions(rank - (lhs_k_major ? 2 : 1));
   const int64_t N = q.w->shape().dimensions(rank - (k_minor ? 2 : 1));
+  PrimitiveType dequant_ty = q.type;
+  if (!q.scale) {
+    // no multiply in the module: the integers themselves are the weights.  One scale per channel, all
+    // ones, under an f32-typed multiply gives exactly those values (convert(int -> bf16) is exact).
+    Instr* one = comp->AddInstruction(HloInstruction::CreateConstant(LiteralUtil::CreateR0<float>(1.0f)));
+    q.scale = comp->AddInstruction(HloInstruction::CreateBroadcast(ShapeUtil::MakeShape(F32, {N}), one, {}));
+    dequant_ty = F32;
+  }
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
-  std::vector<Shape> results = {ShapeUtil::MakeShape(BF16, Dims(dot))};
+  std::vector<Shape> results = {ShapeUtil::MakeShape(Ty(ep.tail), Dims(dot))};
   if (size_t ws = k_minor ? xla_amd_dequant_dot_workspace_bytes_nk(B, M, K, N, (int32_t)Ty(q.w))
                           : xla_amd_dequant_dot_workspace_bytes(B, M, K, N, (int32_t)Ty(q.w)))
     results.push_back(ShapeUtil::MakeShape(S8, {(int64_t)ws}));
@@ -598,12 +632,16 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   // [K/g,N], or [N,K/g] next to weights [N,K]
   const int64_t group_size = q.groups ? K / q.groups : 0;
   Instr* call = EmitCall(comp, "xla_amd.dequant_dot", ops, results,
-                         CommonConfig(ep, q.type, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64") +
-                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : ""));
+                         CommonConfig(ep, dequant_ty, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64") +
+                             (k_minor ? ", rhs_contracting_dim = 1 : i64" : "") +
+                             (lhs_k_major ? ", lhs_contracting_dim = 0 : i64" : "") +
+                             (weights_lhs ? ", result_transposed = true" : ""));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0) : call;
   CHECK_OK(ep.tail->ReplaceAllUsesWith(value));
   VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
-          << (q.zero ? " with zero points" : "") << (k_minor ? ", weights [N,K]" : "") << "]";
+          << (q.zero ? " with zero points" : "") << (k_minor ? ", weights [N,K]" : "")
+          << (weights_lhs ? ", weights as lhs" : "") << (lhs_k_major ? ", activations [K,M]" : "")
+          << (Ty(ep.tail) == F32 ? ", f32 result" : "") << "]";
   return true;
 }
 

@@ -58,7 +58,7 @@ def _scratch(nbytes, device):
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
                 scale_group_size=None, zero_points=None, group_sizes=None, rhs_contracting_dim=0, out=None,
-                scratch="auto", build_only=False):
+                scratch="auto", build_only=False, out_dtype="bf16", result_transposed=False, lhs_contracting_dim=1):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
     scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
     the handler reads the grouping off the scales' shape.
@@ -67,14 +67,18 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     group_sizes (int32 or int64 [G], on the device): ragged dot -- lhs [M,K] with its rows sorted by
     group, weights [G,K,N]; group g multiplies rows [sum(sizes[:g]), +sizes[g]) with weights[g].
     rhs_contracting_dim=1: weights [N,K] or [B,N,K] (4-bit values packed along K), scales [N], [B,N],
-    [N,K/g] or [B,N,K/g]; scale_group_size is then required."""
+    [N,K/g] or [B,N,K/g]; scale_group_size is then required.
+    out_dtype "f32": the dot's f32 value is the result.  result_transposed: the result is [..,N,M] (the
+    dequantised weights were the lhs of the dot; DEFAULT epilogue only).  lhs_contracting_dim=0: lhs is
+    stored [..,K,M]."""
     _check_cuda(lhs, weights, scales, bias, zero_points, group_sizes)
     wdt = {"s4": dtypes.S4, "u4": dtypes.U4}.get(weight_dtype, dtypes.S8)
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
     n = wshape[-2] if rhs_contracting_dim == 1 else wshape[-1]
-    oshape = list(lhs.shape[:-1]) + [n]
+    m, k = (lhs.shape[-1], lhs.shape[-2]) if lhs_contracting_dim == 0 else (lhs.shape[-2], lhs.shape[-1])
+    oshape = list(lhs.shape[:-2]) + ([n, m] if result_transposed else [m, n])
     if out is None:
-        out = torch.empty(oshape, dtype=torch.bfloat16, device=lhs.device)
+        out = torch.empty(oshape, dtype=torch.float32 if out_dtype == "f32" else torch.bfloat16, device=lhs.device)
     batch = lhs.shape[0] if lhs.dim() == 3 else (wshape[0] if group_sizes is not None else 1)
     args = [(dtypes.BF16, lhs.data_ptr(), lhs.shape), (wdt, weights.data_ptr(), wshape),
             (_FLOAT[scales.dtype], scales.data_ptr(), scales.shape)]
@@ -85,11 +89,11 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     if group_sizes is not None:
         args.append((dtypes.S64 if group_sizes.dtype == torch.int64 else dtypes.S32, group_sizes.data_ptr(),
                      group_sizes.shape))
-    rets = [(dtypes.BF16, out.data_ptr(), oshape)]
+    rets = [(dtypes.F32 if out.dtype == torch.float32 else dtypes.BF16, out.data_ptr(), oshape)]
     if scratch == "auto":
         sizer = (ffi.library().xla_amd_dequant_dot_workspace_bytes_nk if rhs_contracting_dim == 1
                  else ffi.library().xla_amd_dequant_dot_workspace_bytes)
-        nbytes = sizer(batch, lhs.shape[-2], lhs.shape[-1], n, wdt)
+        nbytes = sizer(batch, m, k, n, wdt)
         scratch = _scratch(nbytes, lhs.device)
     if scratch is not None:
         rets.append((dtypes.U8, scratch.data_ptr(), [scratch.numel()]))
@@ -100,6 +104,10 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
         attrs["scale_group_size"] = ffi.Attr.i64(scale_group_size)
     if rhs_contracting_dim != 0:
         attrs["rhs_contracting_dim"] = ffi.Attr.i64(rhs_contracting_dim)
+    if lhs_contracting_dim != 1:
+        attrs["lhs_contracting_dim"] = ffi.Attr.i64(lhs_contracting_dim)
+    if result_transposed:
+        attrs["result_transposed"] = ffi.Attr.pred(True)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
                 keep=(lhs, weights, scales, bias, scratch, zero_points, group_sizes))
     return call if build_only else call.run()
