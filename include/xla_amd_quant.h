@@ -46,12 +46,25 @@ extern "C" {
  * (xla/backends/gpu/transforms/gemm_fusion.cc:1629-1702) together with the
  * bias/activation epilogue that GemmRewriter folds into a library matmul
  * (xla/backends/gpu/transforms/gemm_rewriter.cc:888-1007,1987-2304).
- *   args: lhs     BF16 [M,K] or [B,M,K]
- *         weights S8 or S4 [K,N] or [B,K,N]   (S4: two per byte, low nibble first over the
- *                                              row-major index, ir_array.cc:588-603)
- *         scales  F32 or BF16 [N] | [K/g,N] | [B,N] | [B,K/g,N]
- *         bias    BF16 or F32 [N]             (only with a BIAS* epilogue)
- *   rets: out     BF16 [M,N] or [B,M,N]
+ *   args, in this order (optional ones are told apart by their element type):
+ *         lhs         BF16 [M,K] or [B,M,K]     ([..,K,M] with lhs_contracting_dim = 0)
+ *         weights     S8, S4 or U4 [K,N] or [B,K,N]; [N,K] or [B,N,K] with rhs_contracting_dim = 1
+ *                     (4-bit: two per byte, low nibble first over the row-major index,
+ *                     ir_array.cc:588-603; U4 is unsigned, 0..15)
+ *         scales      F32 or BF16 [N] | [K/g,N] | [B,N] | [B,K/g,N]; next to weights [..,N,K]:
+ *                     [N] | [B,N] | [N,K/g] | [B,N,K/g]
+ *         zero_points U4, shaped like the scales (optional; U4 weights only): the dequantised
+ *                     weight is (w - zero_point) * scale
+ *         bias        BF16 or F32 [N]            (optional; exactly with a BIAS* epilogue)
+ *         group_sizes S32 or S64 [G], last       (optional): a ragged dot -- lhs [M,K] with its rows
+ *                     sorted by group, weights [G,K,N] (or [G,N,K]), out [M,N]; group g multiplies rows
+ *                     [sum of the sizes before it, + its size), rows past the last group are epilogue(0)
+ *                     (xla ragged-dot, ragged_dot_rewriter.cc:110-210; gemm_rewriter.cc:781-863)
+ *   rets: out     BF16 or F32 [M,N] or [B,M,N] (F32: the value before the final convert, the root of
+ *                 fusion_emitter_int4_device_test.cc:101,205,320,508); [..,N,M] with result_transposed
+ *         scratch S8 or U8 [bytes]             (optional second result: what
+ *                 xla_amd_dequant_dot_workspace_bytes[_nk] reports for the shape; without it the
+ *                 kernels that need none run)
  *   attrs (all optional, looked up by name):
  *     epilogue      string: DEFAULT|BIAS|RELU|BIAS_RELU|GELU|BIAS_GELU|SILU|BIAS_SILU
  *                   (GemmBackendConfig.Epilogue, xla/service/gpu/backend_configs.proto:105-119)
@@ -64,6 +77,12 @@ extern "C" {
  *                   channel: scales [N] or [B,N]), g > 0: scales [K/g,N] or [B,K/g,N].  The rewrite
  *                   pass always sets it.  Without it the grouping is read off the scales' shape,
  *                   and a batched call whose rank-2 scales fit both readings is refused.
+ *     rhs_contracting_dim i64: 0 (default) weights [..,K,N]; 1 weights [..,N,K], 4-bit values packed
+ *                   along K (fusion_emitter_int4_device_test.cc:867-892); needs scale_group_size
+ *     lhs_contracting_dim i64: 1 (default) lhs [..,M,K]; 0 lhs [..,K,M] (the dot contracts the
+ *                   activations' major dimension, shape table :609-645)
+ *     result_transposed pred (default false): the dequantised weights were the lhs of the dot
+ *                   (Int4WeightsOnTheLhs, :495-523), so out is [..,N,M]; DEFAULT epilogue only
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame);
 
