@@ -69,14 +69,6 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   float* const lds = (float*)smem;
   __shared__ uint32_t lds_bad[4 * COLS];
   __shared__ int lds_partner;
-
-#ifdef XLA_AMD_STAMPS
-  long long stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#define STAMP(i) stamps[i] = wall_clock64()
-#else
-#define STAMP(i)
-#endif
-  STAMP(0);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4, q = (lane >> 2) & 3, i = lane & 3;
@@ -337,8 +329,6 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-
-  STAMP(1);
   if (cnt > 0) {
     load_scales(k_begin);
 #pragma unroll
@@ -372,12 +362,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
             atomicOr(&lds_bad[ch >> 5], 1u << (ch & 31));
           }
   }
-
-  STAMP(2);
   // loads for steps past the wave's last may still be on their way into the ring
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();  // every wave is done with its ring: the memory now carries the partial tiles
-  STAMP(3);
   // ---- add the waves' tiles through LDS.  Register r = (c * MT + mt) * 32 + e32 holds channel
   // strip * TN + 128 * c + 32 * (lane >> 4) + e32, token 16 * mt + (lane & 15): a lane owns 32
   // consecutive channels per column.  In the MFMA tiles e32 = 8d + e sits in
@@ -438,7 +425,6 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // the whole strip by the plain loop below instead.
   // The sums travel in the threads' own order -- [pass][wave][lane][RPW floats], 64 KiB... per strip
   // R * 64 floats -- so that every wave stores and loads 64 x 16 contiguous bytes.
-  STAMP(4);
   static_assert(RPW == 4 || COLS == 1, "the hand-over moves 16 bytes per lane and pass");
   const __amdgpu_buffer_rsrc_t rh = make_rsrc(p.workspace + ((size_t)batch * p.strips + strip) * (R * 64), R * 64 * 4);
   constexpr int kDeviceScope = 16;  // sc1: the access is performed where every XCD sees it
@@ -466,12 +452,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
         for (int u = 0; u < RPW; ++u) res[pass * RPW + u] = bits_to_f32(other[pass][u]) + res[pass * RPW + u];
     }
   }
-  STAMP(5);
   if (finishes) epilogue_all_dispatch<PASSES * RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
-#ifdef XLA_AMD_STAMPS
-  asm volatile("" : "+v"(res[0]));
-#endif
-  STAMP(6);
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
     const int r0 = pass * kChunk + wave * RPW;
@@ -498,13 +479,6 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // each (token, channel) over the rows with ordinary arithmetic, in a fixed order, and overwrites
   // what the loop above produced for it.  The stores above must have landed first.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  STAMP(7);
-#ifdef XLA_AMD_STAMPS
-  if (lane == 0 && p.workspace) {
-    long long* st = (long long*)((char*)p.workspace + (8u << 20)) + ((size_t)blockIdx.x * WAVES + wave) * 8;
-    for (int z = 0; z < 8; ++z) st[z] = stamps[z];
-  }
-#endif
   __syncthreads();
   uint32_t any_bad = partner_ok ? 0u : 1u;
 #pragma unroll
