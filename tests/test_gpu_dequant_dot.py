@@ -19,11 +19,12 @@ def say(msg):
     sys.stdout.flush()
 
 
-def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0, tail=0):
+def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0, tail=0, strip=0):
     """x: 1 keeps s4 weights off the kernels that dequantise through the 4x4x4 matrix instruction
     (default: off whenever a strip width `vec` of the other kernels is asked for); pair: 1 takes the
     two-workgroups-per-strip form of those kernels wherever the shape allows, 2 never; tail: 1 keeps
-    the tiled kernel from splitting the tiles of its last round along K."""
+    the tiled kernel from splitting the tiles of its last round along K; strip: 64 or 128 channels per
+    strip of the single-launch s8 kernel (0: its own choice)."""
     lhs = dev_bf16(w["lhs"])
     if w["weight_dtype"] in ("s4", "u4"):
         wt = dev_u8(w["weights_packed"] if "weights_packed" in w else dtypes.pack_s4(w["weights"]))
@@ -41,6 +42,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
     ffi.set_option("dequant_dot_pair", pair)
     ffi.set_option("dequant_dot_depth", depth)
     ffi.set_option("dequant_dot_steps", steps)
+    ffi.set_option("dequant_dot_strip", strip)
     ffi.set_option("tiled_tail", tail)
     try:
         out = ops.dequant_dot(lhs, wt, sc, bias, weight_dtype=w["weight_dtype"],
@@ -51,7 +53,7 @@ def run_dot(w, force_kernel=0, slices=0, vec=0, x=None, pair=0, depth=0, steps=0
         torch.cuda.synchronize()
     finally:
         for k in ("dequant_dot_kernel", "dequant_dot_slices", "dequant_dot_vec", "dequant_dot_x", "dequant_dot_pair",
-                  "dequant_dot_depth", "dequant_dot_steps", "tiled_tail"):
+                  "dequant_dot_depth", "dequant_dot_steps", "dequant_dot_strip", "tiled_tail"):
             ffi.set_option(k, 0)
     return host_bf16(out), ffi.last_kernel()
 
@@ -225,14 +227,20 @@ def test_s4x_pair_same_call_frame_replayed(oracle):
         ffi.set_option("dequant_dot_pair", 0)
 
 
+def s8x_name(steps, strip):
+    return "dequant_dot_decode_s8x_m16_%ss%d" % ("n64_" if strip == 64 else "", steps)
+
+
+@pytest.mark.parametrize("strip", [128, 64])
 @pytest.mark.parametrize("M,steps,K,N,epilogue,bf16_vectors", [
     (16, 0, 4096, 4096, "DEFAULT", False), (1, 1, 1024, 640, "BIAS_GELU", False), (5, 2, 1024, 648, "BIAS_SILU", True),
     (16, 4, 4096, 200, "RELU", True), (8, 1, 4096, 384, "BIAS", False), (3, 4, 1024, 128, "DEFAULT", False),
     (12, 2, 512, 1000, "BIAS_RELU", False), (16, 1, 256, 136, "SILU", True)])
-def test_s8x_variants(oracle, M, steps, K, N, epilogue, bf16_vectors):
+def test_s8x_variants(oracle, M, steps, K, N, epilogue, bf16_vectors, strip):
     """The single-launch s8 kernel for small matrices: 1 to 16 K-slices per strip adding up inside the
-    kernel, a ragged last strip, every epilogue, f32 and bf16 scale and bias vectors."""
-    say("dequant_dot s8x M=%d steps=%d K=%d N=%d %s bf16_vectors=%s" % (M, steps, K, N, epilogue, bf16_vectors))
+    kernel, strips of 128 and of 64 channels, a ragged last strip, every epilogue, f32 and bf16 scale
+    and bias vectors."""
+    say("dequant_dot s8x M=%d steps=%d K=%d N=%d %s bf16_vectors=%s strip=%d" % (M, steps, K, N, epilogue, bf16_vectors, strip))
     w = workloads.c1_s8_channel(M=M, K=K, N=N)
     w["epilogue"] = epilogue
     rng = np.random.default_rng(11)
@@ -242,8 +250,8 @@ def test_s8x_variants(oracle, M, steps, K, N, epilogue, bf16_vectors):
             w["bias"] = dtypes.f32_to_bf16(w["bias"])
     if bf16_vectors:
         w["scales"] = dtypes.f32_to_bf16(w["scales"])
-    got, kern = run_dot(w, force_kernel=2, steps=steps)
-    assert kern.startswith("dequant_dot_decode_s8x_m16_s") and (steps == 0 or kern.endswith("s%d" % steps)), kern
+    got, kern = run_dot(w, force_kernel=2, steps=steps, strip=strip)
+    assert kern == s8x_name(steps or 4, strip), kern
     compare(oracle, w, got, kern)
 
 
@@ -261,14 +269,16 @@ def test_s8x_one_hot_integer_exact_and_batched(oracle):
         a[np.arange(16), m0 + np.arange(16)] = 1.0
         w = dict(lhs=dtypes.f32_to_bf16(a), weights=wv, scales=sc, bias=None, weight_dtype="s8",
                  weight_shape=(K, N), group=K, dequant_type="f32", epilogue="DEFAULT")
-        got, kern = run_dot(w, force_kernel=2, steps=1)
-        assert kern == "dequant_dot_decode_s8x_m16_s1", kern
-        want = dtypes.f32_to_bf16(wv[m0:m0 + 16].astype(np.float32) * sc[None, :])
-        assert np.array_equal(got, want), (kern, m0)
+        for strip in (128, 64):
+            got, kern = run_dot(w, force_kernel=2, steps=1, strip=strip)
+            assert kern == s8x_name(1, strip), kern
+            want = dtypes.f32_to_bf16(wv[m0:m0 + 16].astype(np.float32) * sc[None, :])
+            assert np.array_equal(got, want), (kern, m0)
     w = workloads.c5_s8_batched(B=2, M=7, K=1024, N=392)
-    got, kern = run_dot(w, force_kernel=2, steps=2)
-    assert kern == "dequant_dot_decode_s8x_m16_s2", kern
-    compare(oracle, w, got, kern)
+    for strip in (128, 64):
+        got, kern = run_dot(w, force_kernel=2, steps=2, strip=strip)
+        assert kern == s8x_name(2, strip), kern
+        compare(oracle, w, got, kern)
 
 
 def test_s8x_same_call_frame_replayed(oracle):
@@ -290,7 +300,7 @@ def test_s8x_same_call_frame_replayed(oracle):
         lhs.copy_(dev_bf16(a))
         out = call.run()
         torch.cuda.synchronize()
-        assert ffi.last_kernel().startswith("dequant_dot_decode_s8x_m16_s"), ffi.last_kernel()
+        assert ffi.last_kernel().startswith("dequant_dot_decode_s8x_m16_"), ffi.last_kernel()
         compare(oracle, dict(w, lhs=a), host_bf16(out), "s8x replay %d" % it)
 
 

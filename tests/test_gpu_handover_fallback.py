@@ -37,17 +37,19 @@ def test_s4_pair_finisher_recomputes_its_strip(oracle, M, K, N, group):
     assert np.array_equal(again, normal)
 
 
+@pytest.mark.parametrize("strip", [128, 64])
 @pytest.mark.parametrize("M,K,N,steps", [(16, 1024, 256, 1), (5, 2048, 136, 2), (16, 4096, 384, 4)])
-def test_s8_last_slice_recomputes_its_strip(oracle, M, K, N, steps):
-    say("hand-over give-up, s8 slices M=%d K=%d N=%d steps=%d" % (M, K, N, steps))
+def test_s8_last_slice_recomputes_its_strip(oracle, M, K, N, steps, strip):
+    say("hand-over give-up, s8 slices M=%d K=%d N=%d steps=%d strip=%d" % (M, K, N, steps, strip))
     w = workloads.c1_s8_channel(M=M, K=K, N=N)
-    normal, kern = run_dot(w, steps=steps)
-    assert kern == "dequant_dot_decode_s8x_m16_s%d" % steps, kern
+    name = "dequant_dot_decode_s8x_m16_%ss%d" % ("n64_" if strip == 64 else "", steps)
+    normal, kern = run_dot(w, steps=steps, strip=strip)
+    assert kern == name, kern
     compare(oracle, w, normal, "s8 slices, ordinary run")
-    alone, kern = run_with_dropped_flags(w, steps=steps)
-    assert kern == "dequant_dot_decode_s8x_m16_s%d" % steps, kern
+    alone, kern = run_with_dropped_flags(w, steps=steps, strip=strip)
+    assert kern == name, kern
     compare(oracle, w, alone, "s8 slices, last slice gave up")
-    again, _ = run_dot(w, steps=steps)
+    again, _ = run_dot(w, steps=steps, strip=strip)
     assert np.array_equal(again, normal)
 
 

@@ -5,9 +5,11 @@
 //
 // A matrix of a few MB is over in a couple of microseconds of HBM time, so the kernel is all
 // latency: nothing may wait for anything it could have asked for earlier.  A workgroup of 8 waves
-// owns 128 channels (one 128-byte line per row of s8) and 256 * STEPS rows; every wave requests ALL
-// its weights (STEPS steps of 32 rows, 8 bytes per lane and row) and activations before it touches
-// the first, so one round trip to memory covers the whole matrix.  The integers go through
+// owns 128 channels (one 128-byte line per row of s8) and 256 * STEPS rows -- or 64 channels where
+// the wide strips would be fewer workgroups than the chip has CUs: half the bytes per workgroup
+// for the same number of slices to wait for ([16,4096]x[4096,4096]: 8.2 -> 7.1 us).  Every wave
+// requests ALL its weights (STEPS steps of 32 rows, 8 or 4 bytes per lane and row) and activations
+// before it touches the first, so one round trip to memory covers the whole matrix.  The integers go through
 // v_mfma_f32_16x16x32_bf16 exactly (an s8 value is a bf16 value), the waves add their tiles
 // through LDS, and the K-slices of a strip add up inside the kernel: every slice but the last
 // stores its f32 sums with device-scope stores and raises a flag; the last slice -- dispatched
@@ -27,15 +29,16 @@ namespace xla_amd {
 namespace {
 
 constexpr int kWaves = 8;
-constexpr int kStripChannels = 128;
-constexpr int kSumsPerStrip = 16 * kStripChannels;  // f32 sums of one 16-token tile
 
-template <int STEPS>
+// NV: channels per lane, 8 (strips of 128 channels, one 128-byte line per row) or 4 (strips of 64:
+// half the bytes per workgroup, for matrices whose wide strips would leave CUs without one)
+template <int STEPS, int NV>
 __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(DecodeParams p) {
-  constexpr int NV = 8;   // channels per lane
-  constexpr int R = 32;   // accumulator registers per lane
+  constexpr int kStripChannels = 16 * NV;
+  constexpr int kSumsPerStrip = 16 * kStripChannels;  // f32 sums of one 16-token tile
+  constexpr int R = 4 * NV;   // accumulator registers per lane
   constexpr int RPW = R / kWaves;
-  __shared__ float lds[kWaves * R * 64];  // 64 KiB
+  __shared__ float lds[kWaves * R * 64];  // 64 or 32 KiB
   __shared__ int lds_all_here;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -58,24 +61,25 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
   const int k_begin = slice * p.rows_per_slice + wave * (32 * STEPS);  // rows_per_slice = 256 * STEPS
 
   // ---- every load of this wave, at once
-  uint32_t wq[STEPS][8][2];
+  uint32_t wq[STEPS][8][NV / 4];
   uintx4 aq[STEPS];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     const int k0 = k_begin + 32 * s;
     aq[s] = __builtin_amdgcn_raw_buffer_load_b128(ra, voff_a + (uint32_t)k0 * 2u, 0, 0);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) buffer_load_words<2>(rw, voff_w + (uint32_t)k0 * pitch, (uint32_t)r * pitch, wq[s][r]);
+    for (int r = 0; r < 8; ++r) buffer_load_words<NV / 4>(rw, voff_w + (uint32_t)k0 * pitch, (uint32_t)r * pitch, wq[s][r]);
   }
   // what the finisher's epilogue needs, requested now as well: the lane ends up with channels
-  // n0 .. n0+3 of token li (see the reduction below)
+  // n0 .. n0+RPW-1 of token li (see the reduction below)
   const int n0 = strip * kStripChannels + (4 * kb + (wave >> 1)) * NV + (wave & 1) * RPW;
   // (raw bits now, converted after the arithmetic: a conversion here would wait for every load above)
   const int bias_esz = p.bias_is_bf16 ? 2 : 4, scale_esz = p.scale_is_bf16 ? 2 : 4;
   const __amdgpu_buffer_rsrc_t rbias = make_rsrc(p.bias, p.bias ? (uint32_t)p.N * bias_esz : 0u);
   const __amdgpu_buffer_rsrc_t rscale = make_rsrc(
       (const char*)p.scales + (size_t)(p.scale_batched ? batch : 0) * p.N * scale_esz, (uint32_t)p.N * scale_esz);
-  // N % 8 == 0 and n0 % 4 == 0: the four values are inside the vector or not at all
+  // N % 8 == 0 and n0 % RPW == 0: the lane's RPW values are inside the vector or not at all (with
+  // RPW = 2 the loads reach two values further, past the end at most: those read as zeros)
   const bool ep_live = finisher && n0 < p.N;
   // two 8-byte loads whatever the type (bf16: the second one goes nowhere): no branch for the
   // compiler to put a wait in front of
@@ -99,7 +103,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
   for (int s = 0; s < STEPS; ++s) {
     const bf16x8 bop = __builtin_bit_cast(bf16x8, aq[s]);
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
+    for (int q = 0; q < NV / 4; ++q)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float f[8];
@@ -139,9 +143,13 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
     const __amdgpu_buffer_rsrc_t rh =
         make_rsrc(p.workspace + strip_index * (size_t)others * kSumsPerStrip, (uint32_t)others * kSumsPerStrip * 4u);
     if (!finisher) {
-      __builtin_amdgcn_raw_buffer_store_b128(
-          uintx4{f32_to_bits(res[0]), f32_to_bits(res[1]), f32_to_bits(res[2]), f32_to_bits(res[3])}, rh,
-          (uint32_t)((slice * (kWaves * 64) + tid) * 16), 0, kDeviceScope);
+      if constexpr (RPW == 4)
+        __builtin_amdgcn_raw_buffer_store_b128(
+            uintx4{f32_to_bits(res[0]), f32_to_bits(res[1]), f32_to_bits(res[2]), f32_to_bits(res[3])}, rh,
+            (uint32_t)((slice * (kWaves * 64) + tid) * 16), 0, kDeviceScope);
+      else
+        __builtin_amdgcn_raw_buffer_store_b64(uintx2{f32_to_bits(res[0]), f32_to_bits(res[1])}, rh,
+                                              (uint32_t)((slice * (kWaves * 64) + tid) * 8), 0, kDeviceScope);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0 && !p.handover_test) __hip_atomic_store(flags + slice, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -164,13 +172,21 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
     all_here = lds_all_here != 0;
     if (all_here) {
       // slice 0 first, this workgroup's own sums last
-      float v[RPW] = {0.0f, 0.0f, 0.0f, 0.0f};
+      float v[RPW];
+#pragma unroll
+      for (int u = 0; u < RPW; ++u) v[u] = 0.0f;
       for (int s0 = 0; s0 < others; s0 += 4) {
         uintx4 o[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          o[i] = __builtin_amdgcn_raw_buffer_load_b128(
-              rh, s0 + i < others ? (uint32_t)(((s0 + i) * (kWaves * 64) + tid) * 16) : kNowhere, 0, kDeviceScope);
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t at = s0 + i < others ? (uint32_t)(((s0 + i) * (kWaves * 64) + tid) * (4 * RPW)) : kNowhere;
+          if constexpr (RPW == 4) {
+            o[i] = __builtin_amdgcn_raw_buffer_load_b128(rh, at, 0, kDeviceScope);
+          } else {
+            const uintx2 h = __builtin_amdgcn_raw_buffer_load_b64(rh, at, 0, kDeviceScope);
+            o[i] = uintx4{h[0], h[1], 0u, 0u};
+          }
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (s0 + i < others) {
@@ -195,8 +211,11 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
     epilogue_all_dispatch<RPW>(res, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
     if (li < p.M && n0 < p.N) {
       uint16_t* dst = p.out + ((size_t)batch * p.M + li) * p.N + n0;
-      if (n0 + RPW <= p.N) {  // N % 4 == 0 and n0 % 4 == 0: whole and 8-byte aligned
-        *reinterpret_cast<uintx2*>(dst) = uintx2{pack_bf16x2(res[0], res[1]), pack_bf16x2(res[2], res[3])};
+      if (n0 + RPW <= p.N) {  // N % 4 == 0 and n0 % RPW == 0: whole and aligned
+        if constexpr (RPW == 4)
+          *reinterpret_cast<uintx2*>(dst) = uintx2{pack_bf16x2(res[0], res[1]), pack_bf16x2(res[2], res[3])};
+        else
+          *reinterpret_cast<uint32_t*>(dst) = pack_bf16x2(res[0], res[1]);
       } else {
 #pragma unroll
         for (int u = 0; u < RPW; ++u)
@@ -225,21 +244,28 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
   if (tid == 0) HandOverNextGeneration(flags + others, target);  // a flag raised late belongs to the old generation
 }
 
-template <int STEPS>
+template <int STEPS, int NV>
 int launch_s8x(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
-  hipLaunchKernelGGL((dequant_dot_decode_s8x_kernel<STEPS>), grid, dim3(kWaves * 64), 0, stream, dp);
+  hipLaunchKernelGGL((dequant_dot_decode_s8x_kernel<STEPS, NV>), grid, dim3(kWaves * 64), 0, stream, dp);
   const int rc = CheckLaunch(name);
   SetLastKernel(name);
   return rc;
 }
 
-// Steps of 32 rows per wave, or 0 when the shape is not one for this kernel.
-int S8xSteps(int64_t batch, int64_t M, int64_t K, int64_t N) {
-  if (GetOption("dequant_dot_x") == 1) return 0;
-  if (M < 1 || M > 16 || K < 256 || K % 256 != 0 || N % 8 != 0) return 0;
+struct S8xShape {
+  int steps;    // steps of 32 rows per wave; 0: the shape is not one for this kernel
+  int channels; // per strip: 128 or 64
+  int64_t strips, slices;
+  size_t sums_bytes() const { return (size_t)16 * channels * 4; }  // one producer's 16-token tile
+};
+
+S8xShape S8xShapeFor(int64_t batch, int64_t M, int64_t K, int64_t N) {
+  S8xShape none = {0, 0, 0, 0};
+  if (GetOption("dequant_dot_x") == 1) return none;
+  if (M < 1 || M > 16 || K < 256 || K % 256 != 0 || N % 8 != 0) return none;
   const int64_t units = K / 256;  // one step of every wave each
-  const int64_t strips = (N + kStripChannels - 1) / kStripChannels;
+  const int64_t wide = (N + 127) / 128;
   int steps = 0;
   if (int v = GetOption("dequant_dot_steps")) {
     steps = v;
@@ -249,47 +275,58 @@ int S8xSteps(int64_t batch, int64_t M, int64_t K, int64_t N) {
     // 8.2 / 9.1 / 10.0 us; the same bytes with no slices at all 4.8 - 6.2 us).  So: the most steps
     // per wave that still leave 64 workgroups.
     for (int s : {4, 2, 1})
-      if (units % s == 0 && (steps == 0 || strips * batch * (units / steps) < 64)) steps = s;
+      if (units % s == 0 && (steps == 0 || wide * batch * (units / steps) < 64)) steps = s;
   }
-  if ((steps != 1 && steps != 2 && steps != 4) || units % steps != 0) return 0;
-  const int64_t slices = units / steps;
-  if (slices > 16 || strips * batch * slices > 1024) return 0;
-  return steps;
+  if ((steps != 1 && steps != 2 && steps != 4) || units % steps != 0) return none;
+  S8xShape shape = {steps, 128, wide, units / steps};
+  // strips of 64 channels where the wide ones would leave CUs without a workgroup: the same number
+  // of slices to wait for, half the bytes per workgroup
+  const int forced = GetOption("dequant_dot_strip");
+  if (forced == 64 || (forced == 0 && shape.strips * batch * shape.slices < 256)) {
+    shape.channels = 64;
+    shape.strips = (N + 63) / 64;
+  }
+  if (shape.slices > 16 || shape.strips * batch * shape.slices > 1024) return none;
+  return shape;
 }
 
 }  // namespace
 
 size_t S8xWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
-  const int steps = S8xSteps(batch, M, K, N);
-  if (!steps) return 0;
-  const int64_t others = K / (256 * steps) - 1;
-  const int64_t strips = (N + kStripChannels - 1) / kStripChannels;
+  const S8xShape shape = S8xShapeFor(batch, M, K, N);
+  if (!shape.steps) return 0;
+  const int64_t others = shape.slices - 1;
   // per strip: the producers' sums and flags, and one generation word
-  return others > 0 ? (size_t)(batch * strips) * ((size_t)others * (kSumsPerStrip * 4 + 8) + 8) : 0;
+  return others > 0 ? (size_t)(batch * shape.strips) * ((size_t)others * (shape.sums_bytes() + 8) + 8) : 0;
 }
 
 int LaunchDequantDotDecodeS8x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream) {
   if (p.weight_dtype != XLA_FFI_DataType_S8 || p.dequant_type == XLA_FFI_DataType_BF16 || p.group != p.K) return -1;
-  const int steps = S8xSteps(p.batch, p.M, p.K, p.N);
+  const S8xShape shape = S8xShapeFor(p.batch, p.M, p.K, p.N);
+  const int steps = shape.steps;
   if (!steps) return -1;
   if ((double)p.K * p.N >= 2147483648.0 || (double)p.M * p.K * 2 >= 2147483648.0) return -1;
-  dp.strips = (int)((p.N + kStripChannels - 1) / kStripChannels);
-  dp.slices = (int)(p.K / (256 * steps));
+  dp.strips = (int)shape.strips;
+  dp.slices = (int)shape.slices;
   dp.rows_per_slice = 256 * steps;
   dp.flags = nullptr;
   dp.epoch = 0;
   if (dp.slices > 1) {
     const size_t need = S8xWorkspaceBytes(p.batch, p.M, p.K, p.N);
     if (!p.workspace || ((uintptr_t)p.workspace % 16) != 0 || p.workspace_bytes < need) return -1;
-    const size_t sums = (size_t)p.batch * dp.strips * (dp.slices - 1) * (kSumsPerStrip * 4);
-    if ((double)(dp.slices - 1) * kSumsPerStrip * 4 >= 2147483648.0) return -1;
+    const size_t sums = (size_t)p.batch * dp.strips * (dp.slices - 1) * shape.sums_bytes();
     dp.flags = (unsigned long long*)((char*)p.workspace + sums);
     dp.epoch = NextHandOverEpoch();
   }
   const int b = (int)p.batch;
-  if (steps == 1) return launch_s8x<1>(dp, b, stream, "dequant_dot_decode_s8x_m16_s1");
-  if (steps == 2) return launch_s8x<2>(dp, b, stream, "dequant_dot_decode_s8x_m16_s2");
-  return launch_s8x<4>(dp, b, stream, "dequant_dot_decode_s8x_m16_s4");
+  if (shape.channels == 64) {
+    if (steps == 1) return launch_s8x<1, 4>(dp, b, stream, "dequant_dot_decode_s8x_m16_n64_s1");
+    if (steps == 2) return launch_s8x<2, 4>(dp, b, stream, "dequant_dot_decode_s8x_m16_n64_s2");
+    return launch_s8x<4, 4>(dp, b, stream, "dequant_dot_decode_s8x_m16_n64_s4");
+  }
+  if (steps == 1) return launch_s8x<1, 8>(dp, b, stream, "dequant_dot_decode_s8x_m16_s1");
+  if (steps == 2) return launch_s8x<2, 8>(dp, b, stream, "dequant_dot_decode_s8x_m16_s2");
+  return launch_s8x<4, 8>(dp, b, stream, "dequant_dot_decode_s8x_m16_s4");
 }
 
 }  // namespace xla_amd
