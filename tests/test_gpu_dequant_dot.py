@@ -450,6 +450,41 @@ def test_s4_group_scales_tiled(oracle, M, K, N, group):
     compare(oracle, w, got, "s4 tiled M=%d" % M)
 
 
+@pytest.mark.parametrize("zero_points", [True, False])
+@pytest.mark.parametrize("M,K,N,group", [(200, 1024, 512, 128), (65, 264, 264, 8), (300, 2048, 1000, 64), (130, 1000, 72, 8)])
+def test_u4_group_scales_tiled(oracle, M, K, N, group, zero_points):
+    """Prefill-sized M on u4 weights: the tiled MFMA kernel with the zero point folded into the
+    constant of the dequantising fma, with zero points and without."""
+    say("dequant_dot u4 tiled M=%d K=%d N=%d group=%d zero_points=%s" % (M, K, N, group, zero_points))
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=group)
+    if not zero_points:
+        w["zero_points"] = w["zero_points_packed"] = None
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == ("dequant_dot_tiled_u4_rounded:tail2" if K >= 2048 else "dequant_dot_tiled_u4_rounded"), kern
+    compare(oracle, w, got, "u4 tiled M=%d" % M)
+
+
+def test_u4_tiled_dequantised_weights_bit_exact(oracle):
+    """One-hot activations pick single dequantised weights out of the tiled kernel: bf16((u - z) * s)
+    exactly, every (u, z) pair among them."""
+    say("dequant_dot u4 tiled one-hot")
+    M, K, N, g = 128, 128, 256, 32
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=g)
+    w["weights"][:16, :16] = np.arange(16, dtype=np.int8)[:, None]
+    w["zero_points"][0, :16] = np.arange(16, dtype=np.uint8)
+    pack = lambda v: (v.reshape(-1)[0::2] | (v.reshape(-1)[1::2] << 4)).astype(np.uint8)
+    w["weights_packed"] = pack(w["weights"].astype(np.uint8))
+    w["zero_points_packed"] = pack(w["zero_points"])
+    lhs = np.zeros((M, K), np.float32)
+    lhs[np.arange(M), np.arange(M) % K] = 1.0
+    w = dict(w, lhs=dtypes.f32_to_bf16(lhs), bias=None, epilogue="DEFAULT")
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_u4_rounded", kern
+    diff = w["weights"].astype(np.float32) - np.repeat(w["zero_points"], g, axis=0).astype(np.float32)
+    want = dtypes.f32_to_bf16(diff * np.repeat(dtypes.bf16_to_f32(w["scales"]), g, axis=0))[np.arange(M) % K]
+    assert np.array_equal(got, want)
+
+
 def test_s4_more_than_64_tokens_picks_the_cheaper_kernel():
     """8192 x 28672 s4 weights: decode passes up to a few hundred tokens, the tiled kernel beyond."""
     say("dequant_dot s4 kernel choice at the C2 weight shape")
@@ -649,8 +684,76 @@ def test_u4_zero_point_decode(oracle, M, K, N, group, vec, slices):
     if (K, N) == (100, 42):
         assert kern == "dequant_dot_generic", kern
     else:
-        assert kern.startswith("dequant_dot_decode_s4_") and (M <= 64 or kern.endswith(":x64")), kern
+        # a forced strip width keeps the call on the first-generation kernels
+        family = "dequant_dot_decode_s4_" if vec or group % 64 else "dequant_dot_decode_u4x_"
+        assert kern.startswith(family) and (M <= 64 or kern.endswith(":x64")), kern
     compare(oracle, w, got, "u4+zp %s" % kern)
+
+
+@pytest.mark.parametrize("zero_points", [True, False])
+@pytest.mark.parametrize("M,pair,slices,K,N,group", [
+    (1, 2, 1, 2048, 768, 128), (8, 1, 0, 2048 + 256, 800, 128), (16, 1, 0, 4096, 256, 64), (3, 2, 2, 2048, 768, 64),
+    (20, 2, 2, 2048 + 128, 736, 64), (33, 2, 1, 1536, 512, 128), (64, 2, 1, 2048, 768, 128), (5, 1, 0, 1024 + 64, 1120, 64)])
+def test_u4x_variants(oracle, M, pair, slices, K, N, group, zero_points):
+    """Unsigned nibbles through the matrix-instruction dequantisation, the zero point riding in the
+    scaling MFMA's operand C: one or two workgroups per strip, K-slices, every token-tile count, a
+    ragged last strip, with zero points and without (then the nibble itself is the weight)."""
+    say("dequant_dot u4x M=%d pair=%d slices=%d K=%d N=%d group=%d zero_points=%s" % (M, pair, slices, K, N, group, zero_points))
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=group)
+    if not zero_points:
+        w["zero_points"] = w["zero_points_packed"] = None
+    got, kern = run_dot(w, force_kernel=2, slices=slices, pair=pair)
+    assert kern.startswith("dequant_dot_decode_u4x_") and kern.endswith("_pair") == (pair == 1), kern
+    compare(oracle, w, got, "%s slices=%d" % (kern, slices))
+
+
+@pytest.mark.parametrize("pair", [2, 1])
+def test_u4x_unpack_and_zero_points_bit_exact(oracle, pair):
+    """One-hot activations: every output is one dequantised weight bf16((u - z) * s), exactly -- the
+    nibble order of weights and zero points, every (u, z) pair, scales across the f16 window."""
+    say("dequant_dot u4x one-hot pair=%d" % pair)
+    K, N, group = 512, 512, 64
+    rng = np.random.default_rng(15)
+    wu = rng.integers(0, 16, size=(K, N)).astype(np.uint8)
+    zero = rng.integers(0, 16, size=(K // group, N)).astype(np.uint8)
+    wu[:16, :16] = np.arange(16, dtype=np.uint8)[:, None]
+    zero[0, :16] = np.arange(16, dtype=np.uint8)
+    mant = rng.integers(128, 256, size=(K // group, N)).astype(np.float32) / 128.0
+    expo = rng.integers(-22, 3, size=(K // group, N)).astype(np.float32)
+    sign = rng.choice([-1.0, 1.0], size=(K // group, N)).astype(np.float32)
+    sc = dtypes.f32_to_bf16(sign * mant * np.exp2(expo))
+    pack = lambda v: (v.reshape(-1)[0::2] | (v.reshape(-1)[1::2] << 4)).astype(np.uint8)
+    diff = wu.astype(np.float32) - np.repeat(zero, group, axis=0).astype(np.float32)
+    want_all = dtypes.f32_to_bf16(diff * np.repeat(dtypes.bf16_to_f32(sc), group, axis=0))
+    for m0 in range(0, K, 16):
+        a = np.zeros((16, K), np.float32)
+        a[np.arange(16), m0 + np.arange(16)] = 1.0
+        w = dict(lhs=dtypes.f32_to_bf16(a), weights=wu.astype(np.int8), weights_packed=pack(wu), scales=sc,
+                 zero_points=zero, zero_points_packed=pack(zero), bias=None, weight_dtype="u4",
+                 weight_shape=(K, N), group=group, dequant_type="bf16", epilogue="DEFAULT")
+        got, kern = run_dot(w, force_kernel=2, pair=pair)
+        assert kern.startswith("dequant_dot_decode_u4x_") and kern.endswith("_pair") == (pair == 1), kern
+        assert np.array_equal(dtypes.bf16_to_f32(got), dtypes.bf16_to_f32(want_all[m0:m0 + 16])), (kern, m0)
+
+
+@pytest.mark.parametrize("M,pair", [(4, 1), (24, 2)])
+def test_u4x_scales_outside_the_f16_window(oracle, M, pair):
+    """Channels whose scale cannot be an f16 operand are recomputed by the plain loop, which must
+    subtract the zero points as well."""
+    say("dequant_dot u4x odd scales M=%d pair=%d" % (M, pair))
+    K, N, group = 1024, 512, 128
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=group)
+    sc = dtypes.bf16_to_f32(w["scales"]).copy()
+    sc[0, 3] = 0.0
+    sc[1, 40] = 16.0
+    sc[2, 41] = 2.0 ** -30
+    sc[7, 255] = -3.0e4
+    sc[0, 300] = 64.0
+    sc[7, 301] = 2.0 ** -25
+    w["scales"] = dtypes.f32_to_bf16(sc)
+    got, kern = run_dot(w, force_kernel=2, pair=pair)
+    assert kern.startswith("dequant_dot_decode_u4x_") and kern.endswith("_pair") == (pair == 1), kern
+    compare(oracle, w, got, kern)
 
 
 def test_u4_zero_point_one_hot_bit_exact(oracle):

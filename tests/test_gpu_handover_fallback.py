@@ -37,6 +37,17 @@ def test_s4_pair_finisher_recomputes_its_strip(oracle, M, K, N, group):
     assert np.array_equal(again, normal)
 
 
+def test_u4_pair_finisher_recomputes_its_strip(oracle):
+    say("hand-over give-up, u4 pair with zero points")
+    w = workloads.u4_zero_point_group(M=8, K=2048, N=512, group=128)
+    normal, kern = run_dot(w, pair=1)
+    assert kern == "dequant_dot_decode_u4x_m16_pair", kern
+    compare(oracle, w, normal, "u4 pair, ordinary run")
+    alone, kern = run_with_dropped_flags(w, pair=1)
+    assert kern == "dequant_dot_decode_u4x_m16_pair", kern
+    compare(oracle, w, alone, "u4 pair, finisher gave up")
+
+
 @pytest.mark.parametrize("strip", [128, 64])
 @pytest.mark.parametrize("M,K,N,steps", [(16, 1024, 256, 1), (5, 2048, 136, 2), (16, 4096, 384, 4)])
 def test_s8_last_slice_recomputes_its_strip(oracle, M, K, N, steps, strip):

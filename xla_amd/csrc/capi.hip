@@ -84,7 +84,7 @@ size_t xla_amd_dequant_dot_workspace_bytes(int64_t batch, int64_t M, int64_t K, 
   const size_t decode = xla_amd::DequantDotDecodeWorkspaceBytes(
       batch, M, K, N, weight_dtype == XLA_FFI_DataType_S4 || weight_dtype == XLA_FFI_DataType_U4);
   // more than 64 tokens may run on the tiled kernel, which splits the tiles of a short last round
-  const size_t tail = weight_dtype == XLA_FFI_DataType_U4 ? 0 : xla_amd::TiledTailWorkspaceBytes(batch, M, K, N);
+  const size_t tail = xla_amd::TiledTailWorkspaceBytes(batch, M, K, N);
   return decode > tail ? decode : tail;
 }
 

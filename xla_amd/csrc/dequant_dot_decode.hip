@@ -740,7 +740,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   // average 96 rows; below that most tiles would be nearly empty and the 64-row chunks of the decode
   // kernel do less work.  The sizes themselves are only known on the device.
   const bool ragged_tiles = ragged && (force == 3 || (p.batch > 0 && p.M / p.batch >= 96));
-  if (plain && force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && !u4 && (!ragged || ragged_tiles)) {
+  if (plain && force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && (!ragged || ragged_tiles)) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
   }
@@ -938,7 +938,7 @@ int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream)
       need = DequantDotNkWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit);
     } else {
       need = DequantDotDecodeWorkspaceBytes(p.batch, p.M, p.K, p.N, four_bit);
-      const size_t tail = p.weight_dtype == XLA_FFI_DataType_U4 ? 0 : TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
+      const size_t tail = TiledTailWorkspaceBytes(p.batch, p.M, p.K, p.N);
       if (tail > need) need = tail;
     }
   }

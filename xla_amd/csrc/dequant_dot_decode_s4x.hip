@@ -53,7 +53,10 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // MT: 16-token tiles.  WAVES: waves per workgroup (they split the rows).  COLS: 128-channel columns
 // a wave covers (1 or 2).  DEPTH: steps whose loads are in flight or in use (>= 2).
-template <int MT, int WAVES, int COLS, int DEPTH>
+// U4: the nibbles are unsigned (0..15) and every scale may come with a zero point (one u4 value per
+// scale, packed like the weights; none: zero).  The zero point takes the place of the 8 that is
+// subtracted from a biased s4 nibble: it goes into operand C of the scaling MFMA, per channel.
+template <int MT, int WAVES, int COLS, int DEPTH, bool U4 = false>
 __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(DecodeParams p) {
   constexpr int R = 32 * MT * COLS;  // accumulator registers per lane: 32 channels x MT token tiles per column
   constexpr int kChunk = (WAVES <= 8) ? 32 : 16;
@@ -100,6 +103,11 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.lhs + (size_t)batch * p.M * p.K, (uint32_t)p.M * p.K * 2u);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(
       (const char*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N * 2, (uint32_t)groups * p.N * 2u);
+  // zero points [groups, N / 2]; without them the descriptor is empty and every load returns zero
+  const bool has_zp = U4 && p.zero_points != nullptr;
+  const __amdgpu_buffer_rsrc_t rz =
+      make_rsrc(has_zp ? p.zero_points + (size_t)(p.scale_batched ? batch : 0) * groups * pitch : p.w,
+                has_zp ? (uint32_t)groups * pitch : 0u);
 
   constexpr uint32_t kNowhere = 0x80000000u;
   // Loading side: LPR lanes cover one row (16 bytes each), so a load instruction takes 64 / LPR whole
@@ -130,11 +138,12 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   // as column j = i of B and D the lane stands for channels 128c + 32q + 8d + sm + h of the strip,
   // sm = (0,4,2,6)[i]; one dword of a scales row holds the pair h = 0, 1
   const int sm = (i & 1) * 4 + (i >> 1) * 2;
-  uint32_t voff_s[COLS];
+  uint32_t voff_s[COLS], voff_z[COLS];
 #pragma unroll
   for (int c = 0; c < COLS; ++c) {
     const int n = strip * TN + 128 * c + 32 * q;
     voff_s[c] = n < p.N ? (uint32_t)(n + sm) * 2u : kNowhere;
+    voff_z[c] = n < p.N ? (uint32_t)n >> 1 : kNowhere;  // 4 bytes per d: the 8 channels of one weight dword
   }
   // byte selectors that put a 16-bit scale where s_j sits in column j = i of B (0x0c selects zero):
   // sel[h][r]: register r of the column, taking the low (h = 0) or high (h = 1) half of the source
@@ -170,6 +179,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   if (k_begin >= p.K) cnt = 0;
 
   uint32_t sraw[COLS][4];
+  uint32_t zraw[COLS][4];  // U4: the zero points of the dword's 8 channels, one nibble each
   halfx4 Bm[COLS][4][2];
   floatx4 Cm[COLS][4][2];
   uint32_t bad = 0;
@@ -180,6 +190,13 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     for (int c = 0; c < COLS; ++c)
 #pragma unroll
       for (int d = 0; d < 4; ++d) sraw[c][d] = __builtin_amdgcn_raw_buffer_load_b32(rs, voff_s[c] + vs + 16u * d, 0, 0);
+    if constexpr (U4) {
+      const uint32_t vz = (uint32_t)(km / group) * pitch;  // a row of zero points is as long as a row of weights
+#pragma unroll
+      for (int c = 0; c < COLS; ++c)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) zraw[c][d] = __builtin_amdgcn_raw_buffer_load_b32(rz, voff_z[c] + vz + 4u * d, 0, 0);
+    }
   };
   auto load_step = [&](int buf, int row) {  // row: first row of the step
     uint8_t* const slot = my_ring + buf * kSlot;
@@ -247,8 +264,17 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
 #pragma unroll
       for (int d = 0; d < 4; ++d)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-          Cm[c][d][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(h ? off1 : off0, Bm[c][d][h], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        for (int h = 0; h < 2; ++h) {
+          halfx4 off = h ? off1 : off0;
+          if constexpr (U4) {
+            // -(1024 + z) | -(1024 + 16 z) of the four channels the block's columns stand for, in the
+            // order the nibbles of a weight dword are unpacked in: f16 bits 0xe400 | z, 0xe400 | z << 4
+            const uint32_t z = zraw[c][d], m = h ? 0x00f000f0u : 0x000f000fu;
+            off = __builtin_bit_cast(halfx4, uintx2{(uint32_t)__builtin_amdgcn_bitop3_b32(z, m, 0xe400e400u, 0x6a),
+                                                    (uint32_t)__builtin_amdgcn_bitop3_b32(z >> 8, m, 0xe400e400u, 0x6a)});
+          }
+          Cm[c][d][h] = __builtin_amdgcn_mfma_f32_4x4x4f16(off, Bm[c][d][h], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        }
   };
   // One 32-row step.  The work of consecutive operands (16 channels x 32 rows each: 2 small MFMAs,
   // 4 conversions, MT large MFMAs) is overlapped by hand: while operand o goes through the large
@@ -287,7 +313,8 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
       const int c = o / 8, d = (o / 2) % 4, h = o % 2;
       const uint32_t x = wq[c][rho][d];
       if (h == 0) ysh[rho] = x >> 8;
-      const uint32_t m = h ? 0x00f000f0u : 0x000f000fu, k = h ? 0x64806480u : 0x64086408u;
+      // f16 1024 + u | 1024 + 16 u; an s4 nibble is biased on the way (u = w + 8: its top bit flipped)
+      const uint32_t m = h ? 0x00f000f0u : 0x000f000fu, k = U4 ? 0x64006400u : h ? 0x64806480u : 0x64086408u;
       A[o % 3][rho] = __builtin_bit_cast(halfx4, uintx2{(uint32_t)__builtin_amdgcn_bitop3_b32(x, m, k, 0x6a),
                                                         (uint32_t)__builtin_amdgcn_bitop3_b32(ysh[rho], m, k, 0x6a)});
     };
@@ -488,6 +515,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
     const int ke = partner_ok ? min(ks + slice_rows, p.K) : p.K;
     const uint16_t* sc16 = (const uint16_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * groups * p.N;
     const uint8_t* wb = p.w + (p.weights_shared ? (size_t)0 : (size_t)batch * p.K * pitch);
+    const uint8_t* zb = p.zero_points ? p.zero_points + (size_t)(p.scale_batched ? batch : 0) * groups * pitch : nullptr;
     for (int ch = wave; ch < TN; ch += WAVES) {
       const int n = strip * TN + ch;
       if ((partner_ok && !((lds_bad[ch >> 5] >> (ch & 31)) & 1u)) || n >= p.N) continue;
@@ -496,7 +524,12 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
         float v = 0.0f;
         for (int k = ks + lane; k < ke; k += 64) {
           const uint32_t nib = (wb[(size_t)k * pitch + (n >> 1)] >> (4 * (n & 1))) & 0xfu;
-          const float wv = round_bf16((float)((int)(nib ^ 8u) - 8) * bf16_to_f32(sc16[(size_t)(k / group) * p.N + n]));
+          int wi = (int)(nib ^ 8u) - 8;
+          if constexpr (U4) {
+            wi = (int)nib;
+            if (p.zero_points) wi -= (int)((zb[(size_t)(k / group) * pitch + (n >> 1)] >> (4 * (n & 1))) & 0xfu);
+          }
+          const float wv = round_bf16((float)wi * bf16_to_f32(sc16[(size_t)(k / group) * p.N + n]));
           v = v + bf16_to_f32(arow[k]) * wv;
         }
 #pragma unroll
@@ -532,10 +565,10 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_s4x_kernel(Deco
   }
 }
 
-template <int MT, int WAVES, int COLS, int DEPTH>
+template <int MT, int WAVES, int COLS, int DEPTH, bool U4 = false>
 int launch_s4x(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
-  hipLaunchKernelGGL((dequant_dot_decode_s4x_kernel<MT, WAVES, COLS, DEPTH>), grid, dim3(WAVES * 64), 0, stream, dp);
+  hipLaunchKernelGGL((dequant_dot_decode_s4x_kernel<MT, WAVES, COLS, DEPTH, U4>), grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
   if (rc) return rc;
   if (dp.slices > 1 && !dp.pair) rc = LaunchDecodeFinalize(dp, batch, stream, kRounded);
@@ -565,8 +598,10 @@ bool S4xPairShape(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t group)
 }
 
 int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t stream) {
-  if (p.weight_dtype != XLA_FFI_DataType_S4 || !dp.scale_is_bf16 || p.M > 64 || p.N % 32 != 0 || p.group % 64 != 0)
+  const bool u4 = p.weight_dtype == XLA_FFI_DataType_U4;
+  if ((p.weight_dtype != XLA_FFI_DataType_S4 && !u4) || !dp.scale_is_bf16 || p.M > 64 || p.N % 32 != 0 || p.group % 64 != 0)
     return -1;
+  if (u4 && p.zero_points && ((uintptr_t)p.zero_points % 4) != 0) return -1;  // read a dword (8 channels) at a time
   const int mt = p.M <= 16 ? 1 : p.M <= 32 ? 2 : p.M <= 48 ? 3 : 4;
   const int group = (int)p.group;
   const int spg = group / 32;   // steps per unit
@@ -630,6 +665,7 @@ int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
     dp.rows_per_slice = (groups_total - g0) * group;   // the finisher's rows (to the end of K, rounded up to a group)
     class_split(g0, &dp.units_per_simd, &dp.class_units[0], &dp.class_units[1]);
     class_split(groups_total - g0, &dp.units_per_simd2, &dp.class_units[2], &dp.class_units[3]);
+    if (u4) return launch_s4x<1, 8, 2, 2, true>(dp, b, stream, "dequant_dot_decode_u4x_m16_pair");
     return launch_s4x<1, 8, 2, 2>(dp, b, stream, "dequant_dot_decode_s4x_m16_pair");
   }
   dp.strips = (int)((p.N + 127) / 128);
@@ -640,6 +676,13 @@ int LaunchDequantDotDecodeS4x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
     slices = 1;
   while (slices > 1 && p.K / slices < group) slices /= 2;
   split_rows(slices);
+  if (u4) {
+    if (depth != 2) return -1;
+    if (mt == 1) return launch_s4x<1, 8, 1, 2, true>(dp, b, stream, "dequant_dot_decode_u4x_m16_d2");
+    if (mt == 2) return launch_s4x<2, 8, 1, 2, true>(dp, b, stream, "dequant_dot_decode_u4x_m32_d2");
+    if (mt == 3) return launch_s4x<3, 8, 1, 2, true>(dp, b, stream, "dequant_dot_decode_u4x_m48_d2");
+    return launch_s4x<4, 8, 1, 2, true>(dp, b, stream, "dequant_dot_decode_u4x_m64_d2");
+  }
 #define XLA_AMD_S4X(MT_, DEPTH_, NAME) \
   if (mt == MT_ && depth == DEPTH_) return launch_s4x<MT_, 8, 1, DEPTH_>(dp, b, stream, NAME);
   XLA_AMD_S4X(1, 2, "dequant_dot_decode_s4x_m16_d2")

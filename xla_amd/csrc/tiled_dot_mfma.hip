@@ -42,9 +42,10 @@ namespace {
 // 32 elements of K on both operands (MXFP8), multiplied in by the matrix cores themselves
 // kBf16: both operands bf16 with K minor, a [M,K] and b [N,K] -- the f8 operands of a dot whose
 // dequantise multiply is bf16-typed, already scaled and rounded by a pre-pass
+// kU4: kS4 with unsigned nibbles and, optionally, one u4 zero point per scale (packed like the weights).
 // kS8NK, kS4NK: integer weights stored [N,K]: a thread fetches 32 consecutive k of one channel and
 // writes them, dequantised, as four chunks of that channel's LDS row
-enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4, kBf16 = 5, kS8NK = 6, kS4NK = 7 };
+enum : int { kFp8 = 0, kS8 = 1, kFp8KN = 2, kFp8MX = 3, kS4 = 4, kBf16 = 5, kS8NK = 6, kS4NK = 7, kU4 = 8 };
 
 constexpr int kTM = 256, kTN = 256;  // output tile (tokens x channels)
 constexpr int kRow = 128;            // bytes of K per LDS row per stage
@@ -56,6 +57,7 @@ struct TiledParams {
   const float* b_scale; // kFp8: one value, or N (b_per_channel)
   const void* scales;   // kS8: [scale_batch, N]; kS4: bf16 [scale_batch, K/group, N]
   int group_shift;      // kS4: log2 of the scale group (rows of K)
+  const uint8_t* zero_points;  // kU4: u4 [scale_batch, K/group, N], two per byte, or null (all zero)
   const void* bias;
   uint16_t* out;        // [batch, M, N]
   int M, K, N;
@@ -236,8 +238,9 @@ __device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, 
 
 template <int KIND, bool OUT_F8>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
-  constexpr bool WQ = KIND == kS8 || KIND == kS4 || KIND == kS8NK || KIND == kS4NK;  // integer weights, dequantised on the way into LDS
-  constexpr bool W4 = KIND == kS4 || KIND == kS4NK;   // two weights per byte, bf16 group scales
+  constexpr bool WQ = KIND == kS8 || KIND == kS4 || KIND == kU4 || KIND == kS8NK || KIND == kS4NK;  // integer weights, dequantised on the way into LDS
+  constexpr bool W4 = KIND == kS4 || KIND == kU4 || KIND == kS4NK;   // two weights per byte, bf16 group scales
+  constexpr bool U4 = KIND == kU4;
   constexpr bool W8 = KIND == kS8 || KIND == kS8NK;   // one scale per channel, applied to the sums
   constexpr bool BB = KIND == kBf16;     // both operands bf16, K minor
   constexpr bool F8 = !WQ && !BB;        // both operands f8e4m3fn
@@ -408,6 +411,13 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       tile_rsrc(W4 ? (const uint8_t*)p.scales + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * p.N * 2
                    : p.a,
                 W4 ? (uint32_t)(p.K >> p.group_shift) * (uint32_t)p.N * 2u : 0u);
+  // kU4: the zero points of the lane's 8 channels, one dword per group of rows; without zero points
+  // the descriptor is empty and the loads return zero
+  uint32_t u4_zeros = 0u;
+  const bool has_zp = U4 && p.zero_points != nullptr;
+  const __amdgpu_buffer_rsrc_t rzp =
+      tile_rsrc(has_zp ? p.zero_points + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * (p.N >> 1) : p.a,
+                has_zp ? (uint32_t)(p.K >> p.group_shift) * ((uint32_t)p.N >> 1) : 0u);
   auto s4_load = [&](int k0) {
     const uint32_t col = (uint32_t)(n0 + q_oct * 8);
     const uint32_t kfirst = (uint32_t)(k0 + q_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
@@ -419,19 +429,21 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * s4_pitch, 0, 0);
     s4_scales = __builtin_amdgcn_raw_buffer_load_b128(
         rsc4, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) * 2u : kOutOfRange, 0, 0);
+    if constexpr (U4)
+      u4_zeros = __builtin_amdgcn_raw_buffer_load_b32(rzp, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) >> 1 : kOutOfRange, 0, 0);
   };
   auto s4_store = [&](uint8_t* bt) {
     typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int sl = 0; sl < 2; ++sl) {
       // nibbles (e, e + 4), e = 2 * q_half + sl, as the f16 pair (1024 + u, 1024 + u) or, for odd
-      // e, (1024 + 16 u, 1024 + 16 u), u = w + 8: see dequant_dot_decode.hip
+      // e, (1024 + 16 u, 1024 + 16 u), u = w + 8 (kU4: the nibble itself): see dequant_dot_decode.hip
       halfx2 pr[8];
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const uint32_t x = q_half ? wreg[r] >> 8 : wreg[r];
-        pr[r] = __builtin_bit_cast(halfx2, sl ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a)
-                                              : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
+        pr[r] = __builtin_bit_cast(halfx2, sl ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, U4 ? 0x64006400u : 0x64806480u, 0x6a)
+                                              : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, U4 ? 0x64006400u : 0x64086408u, 0x6a));
       }
 #pragma unroll
       for (int hi = 0; hi < 2; ++hi) {
@@ -440,7 +452,12 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
         const uint32_t sw = q_half ? sw1 : sw0;  // e and e + 2 have the same parity: same half of the dword
         const float v = (e_lo & 1) ? bf16hi_to_f32(sw) : bf16lo_to_f32(sw);
         const float sj = sl ? v * 0.0625f : v;
-        const float cj = sl ? v * -72.0f : v * -1032.0f;
+        float cj = sl ? v * -72.0f : v * -1032.0f;
+        if constexpr (U4) {
+          // the zero point in place of the 8: -(1024 + z) s, or -(64 + z) s next to 1024 + 16 u (exact in f32)
+          const float z = (float)((u4_zeros >> (4 * (e_lo + 2 * q_half))) & 0xfu);
+          cj = v * (sl ? -64.0f - z : -1024.0f - z);
+        }
         float f[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) f[r] = __builtin_fmaf((float)pr[r][hi], sj, cj);
@@ -519,7 +536,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   };
   auto wq_store = [&](uint8_t* bt) {
     if constexpr (KIND == kS8) s8_store(bt);
-    if constexpr (KIND == kS4) s4_store(bt);
+    if constexpr (KIND == kS4 || KIND == kU4) s4_store(bt);
     if constexpr (KIND == kS8NK || KIND == kS4NK) nk_store(bt);
   };
 
@@ -540,7 +557,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       }
     }
     if (KIND == kS8) s8_load(k0);
-    if (KIND == kS4) s4_load(k0);
+    if (KIND == kS4 || KIND == kU4) s4_load(k0);
     if (KIND == kS8NK || KIND == kS4NK) nk_load(k0);
     if (MX) {
       // the stage's four scale bytes of every tile row, one dword per row: waves 0-3 fetch the
@@ -1062,14 +1079,17 @@ size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
 // (the caller then falls back), 0 on success, or an error code.
 int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   // s4 with bf16 scales per power-of-two group of rows and a bf16-typed dequantise multiply, or
-  // s8 with per-channel scales and an f32-typed one
-  const bool s4 = p.weight_dtype == XLA_FFI_DataType_S4 && p.dequant_type == XLA_FFI_DataType_BF16 &&
+  // s8 with per-channel scales and an f32-typed one; u4 (with or without zero points) as s4
+  const bool u4 = p.weight_dtype == XLA_FFI_DataType_U4;
+  if (u4 && p.zero_points && ((uintptr_t)p.zero_points % 4) != 0) return -1;  // a dword (8 channels) per load
+  const bool s4 = (p.weight_dtype == XLA_FFI_DataType_S4 || u4) && p.dequant_type == XLA_FFI_DataType_BF16 &&
                   p.scale_dtype == XLA_FFI_DataType_BF16 && p.group >= 8 && (p.group & (p.group - 1)) == 0 &&
                   p.N % 8 == 0 && ((uintptr_t)p.scales % 16) == 0 &&
                   (double)(p.K / p.group) * p.N * 2 < 2147483000.0;
   const bool s8 = p.weight_dtype == XLA_FFI_DataType_S8 && p.group == p.K && p.dequant_type == XLA_FFI_DataType_F32;
   if (!s4 && !s8) return -1;
   const bool ragged = p.group_sizes != nullptr;  // the caller has decided that the rows per group make tiles worth it
+  if (u4 && ragged) return -1;  // a ragged dot over u4 weights stays with the 64-row chunks of the decode kernel
   if (s4 && !ragged && GetOption("dequant_dot_kernel") != 3) {
     // The decode kernel, run once per 64 tokens, streams and dequantises the weights on every
     // pass but fills the machine at any M; the tiled kernel dequantises once per 256 tokens but
@@ -1102,6 +1122,7 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   tp.tiles_n = (tp.N + kTN - 1) / kTN;
   tp.closed_form_epilogue = GetOption("tiled_epilogue") == 1;
   if (s4) tp.group_shift = __builtin_ctzll((unsigned long long)p.group);  // sizes the scales' descriptor: set before any launch
+  tp.zero_points = u4 ? (const uint8_t*)p.zero_points : nullptr;
   if (ragged) {
     // at most floor(M / 256) + groups tiles of rows, whatever the sizes turn out to be
     tp.group_sizes = p.group_sizes;
@@ -1111,10 +1132,12 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
     if ((double)tp.ragged_slots * tp.tiles_n > 2147483000.0) return -1;
     tp.tiles_m = tp.ragged_slots;
     tp.scale_batched = p.scale_batch == p.batch;  // one set of scales per group, also for a single group
-    const int rc = s4 ? launch_tiled<kS4>(tp, 1, stream, "dequant_dot_tiled_s4") : launch_tiled<kS8>(tp, 1, stream, "dequant_dot_tiled_s8");
+    const int rc = u4   ? launch_tiled<kU4>(tp, 1, stream, "dequant_dot_tiled_u4")
+                   : s4 ? launch_tiled<kS4>(tp, 1, stream, "dequant_dot_tiled_s4")
+                        : launch_tiled<kS8>(tp, 1, stream, "dequant_dot_tiled_s8");
     if (rc) return rc;
     hipLaunchKernelGGL(ragged_tail_rows_kernel, dim3((unsigned)((p.N + 255) / 256), 64u), dim3(256), 0, stream, tp);
-    SetLastKernel(s4 ? "dequant_dot_tiled_s4_rounded:ragged" : "dequant_dot_tiled_s8_factored:ragged");
+    SetLastKernel(u4 ? "dequant_dot_tiled_u4_rounded:ragged" : s4 ? "dequant_dot_tiled_s4_rounded:ragged" : "dequant_dot_tiled_s8_factored:ragged");
     return CheckLaunch("dequant_dot_ragged_tail_rows");
   }
   // the last round of 256 workgroups, when at most half full, runs as two workgroups per tile
@@ -1130,6 +1153,10 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
       tp.epoch = NextHandOverEpoch();
       tp.handover_test = GetOption("handover_test");
     }
+  }
+  if (u4) {
+    SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_u4_rounded:tail2" : "dequant_dot_tiled_u4_rounded");
+    return launch_tiled<kU4>(tp, (int)p.batch, stream, "dequant_dot_tiled_u4");
   }
   if (s4) {
     SetLastKernel(tp.tail_tiles ? "dequant_dot_tiled_s4_rounded:tail2" : "dequant_dot_tiled_s4_rounded");
