@@ -210,7 +210,8 @@ def evaluate(module_json, args):
             blk = a8.shape[-1] // sa.shape[-1]
             ad = _round(O.f8e4m3fn_to_f32(a8) * np.repeat(O.f8e8m0fnu_to_f32(sa), blk, axis=-1), ty)
             bd = _round(O.f8e4m3fn_to_f32(b8) * np.repeat(O.f8e8m0fnu_to_f32(sb), blk, axis=-1), ty)
-            v = _round(_dot(ad, bd, [ad.ndim - 1], [bd.ndim - 1], [], []), ty)
+            lead = list(range(ad.ndim - 2))  # a batch dimension, if present, is the major one (block_scaling_rewriter.h:53)
+            v = _round(_dot(ad, bd, [ad.ndim - 1], [bd.ndim - 1], lead, lead), ty)
         elif op == "tuple":
             v = list(x)
         elif op == "get-tuple-element":

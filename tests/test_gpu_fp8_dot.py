@@ -282,6 +282,48 @@ def test_mxfp8_block_scales(oracle, M, K, N):
     assert np.array_equal(host_bf16(out), ref)
 
 
+@pytest.mark.parametrize("epilogue,dot_ty,ep_ty", [("BIAS_GELU", "f32", "f32"), ("BIAS_SILU", "bf16", "bf16"), ("RELU", "f32", "f32"),
+                                                  ("BIAS", "f32", "f32")])
+def test_mxfp8_with_an_epilogue(oracle, epilogue, dot_ty, ep_ty):
+    """Block scales with a bias and an activation behind the dot, on the tiled and on the exact kernel."""
+    say("fp8_scaled_dot MXFP8 %s dot %s epilogue %s" % (epilogue, dot_ty, ep_ty))
+    names = {"BIAS_GELU": "gelu_tanh", "BIAS_SILU": "silu", "RELU": "relu", "BIAS": "none"}
+    for (M, K, N) in ((300, 512, 272), (70, 96, 40)):
+        a, b, sa, sb = mx_case(M, K, N, 11)
+        rng = np.random.default_rng(3)
+        bias = dtypes.f32_to_bf16(rng.standard_normal(N).astype(np.float32)) if "BIAS" in epilogue else None
+        ref = oracle.block_scaled_dot(a, b, sa, sb, bias=bias, dot_ty=dot_ty, ep_ty=ep_ty, epilogue=names[epilogue])
+        out = ops.fp8_scaled_dot(dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), dev_bf16(bias) if bias is not None else None,
+                                 rhs_contracting_dim=1, epilogue=epilogue, dot_type=dot_ty, epilogue_type=ep_ty)
+        torch.cuda.synchronize()
+        kern = ffi.last_kernel()
+        assert kern == ("fp8_scaled_dot_tiled_mx" if K % 128 == 0 else "fp8_scaled_dot_exact"), kern
+        if "exact" in kern:
+            assert np.array_equal(host_bf16(out), ref)
+        else:
+            # the floor is that of the value entering the activation; both activations have slope <= 1.13
+            check_dot(host_bf16(out), ref, 1.2 * mx_floor(a, b, sa, sb, False), kern + " " + epilogue)
+
+
+def test_mxfp8_batched(oracle):
+    """One leading batch dimension on the operands, their block scales and the result."""
+    say("fp8_scaled_dot MXFP8 batched")
+    for (B, M, K, N) in ((3, 130, 256, 264), (2, 40, 64, 72)):
+        cases = [mx_case(M, K, N, 20 + i) for i in range(B)]
+        a, b, sa, sb = (np.stack([c[j] for c in cases]) for j in range(4))
+        out = ops.fp8_scaled_dot(dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), rhs_contracting_dim=1)
+        torch.cuda.synchronize()
+        kern = ffi.last_kernel()
+        assert kern == ("fp8_scaled_dot_tiled_mx" if K % 128 == 0 else "fp8_scaled_dot_exact"), kern
+        got = host_bf16(out)
+        for i in range(B):
+            ref = oracle.block_scaled_dot(a[i], b[i], sa[i], sb[i])
+            if "exact" in kern:
+                assert np.array_equal(got[i], ref), i
+            else:
+                check_dot(got[i], ref, mx_floor(a[i], b[i], sa[i], sb[i], False), "%s batch %d" % (kern, i))
+
+
 def test_mxfp8_one_block_at_a_time(oracle):
     """Data in a single 32-element block of K, a different scale on every block: each block must
     come out multiplied by its own two scales exactly (products of small integers, exact sums)."""

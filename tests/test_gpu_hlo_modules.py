@@ -176,6 +176,35 @@ def test_mxfp8_module(oracle):
     check_dot(host_bf16(out), ref, dot_floor(ad, bd.T, K) + 1.2 * 2.0 ** -12 * np.sqrt((ad * ad) @ (bd * bd).T), "MXFP8 module")
 
 
+@pytest.mark.parametrize("batch", [0, 3])
+def test_mxfp8_module_with_bias_gelu(oracle, batch):
+    """The block-scaled custom call yielding f32, a bias add, GELU and the convert to bf16 behind it,
+    with and without a leading batch dimension: one call after the pass, against the op-by-op
+    evaluation of the original module."""
+    say("module MXFP8 block-scaled dot + bias + GELU, batch=%d" % batch)
+    M, K, N = 128, 256, 96
+    rng = np.random.default_rng(16)
+    lead = (batch,) if batch else ()
+    a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal(lead + (M, K)) * 4, -448, 448).astype(np.float32))
+    b = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal(lead + (N, K)) * 4, -448, 448).astype(np.float32))
+    sa = rng.integers(120, 128, lead + (M, K // 32)).astype(np.uint8)
+    sb = rng.integers(120, 128, lead + (N, K // 32)).astype(np.uint8)
+    bias = dtypes.f32_to_bf16(rng.standard_normal(N).astype(np.float32))
+    text = hm.mxfp8_block_scaled_dot(M, K, N, batch=batch, bias_gelu=True)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), dev_bf16(bias)])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, block scales%s]" % (", batched" if batch else "")]
+    assert ffi.last_kernel() == "fp8_scaled_dot_tiled_mx"
+    ref = reference(text, [a, b, sa, sb, bias])
+    got = host_bf16(out)
+    for i in range(max(batch, 1)):
+        ai, bi, sai, sbi = (v[i] if batch else v for v in (a, b, sa, sb))
+        ad = np.abs(dtypes.f8e4m3fn_to_f32(ai).astype(np.float64)) * np.repeat(2.0 ** (sai.astype(np.float64) - 127), 32, axis=1)
+        bd = np.abs(dtypes.f8e4m3fn_to_f32(bi).astype(np.float64)) * np.repeat(2.0 ** (sbi.astype(np.float64) - 127), 32, axis=1)
+        floor = 1.2 * (dot_floor(ad, bd.T, K) + 1.2 * 2.0 ** -12 * np.sqrt((ad * ad) @ (bd * bd).T))
+        check_dot(got[i] if batch else got, ref[i] if batch else ref, floor, "MXFP8 module + bias + GELU, batch %d" % i)
+
+
 def test_quantize_then_fp8_dot_module(oracle):
     """RMSNorm + quantize feeding an f8 dot: two custom calls after the pass, against the op-by-op
     evaluation of the original module."""

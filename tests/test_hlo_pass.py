@@ -180,17 +180,28 @@ def test_batched_fp8_dot():
 
 def test_mxfp8_block_scaled_dot():
     """"__op$block_scaled_dot" with f8e4m3fn operands and f8e8m0fnu scales per 32 of K keeps its
-    operands and becomes the library's call (block_scaling_rewriter.h:48-69); other scale types
-    or an f32 result stay for BlockScalingRewriter, with the reason."""
+    operands and becomes the library's call (block_scaling_rewriter.h:48-69), with a leading batch
+    dimension and with what follows an f32-typed call (bias, GELU, convert to bf16) taken along;
+    other scale types or an f32 value leaving the pattern stay for BlockScalingRewriter, with the reason."""
     text = hm.mxfp8_block_scaled_dot(64, 256, 32)
     new, rw, rf = hlo.rewrite(text)
     assert rw == ["result -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]"] and rf == []
     check(new, r"bf16\[64,32\]\{1,0\} custom-call\(%lhs, %rhs, %lhs_scale, %rhs_scale\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
           r"rhs_contracting_dim = 1 : i64")
+    new, rw, rf = hlo.rewrite(hm.mxfp8_block_scaled_dot(64, 256, 32, batch=3))
+    assert rw == ["result -> xla_amd.fp8_scaled_dot [DEFAULT, block scales, batched]"] and rf == []
+    check(new, r"bf16\[3,64,32\]\{2,1,0\} custom-call\(%lhs, %rhs, %lhs_scale, %rhs_scale\), custom_call_target=\"xla_amd.fp8_scaled_dot\"")
+    new, rw, rf = hlo.rewrite(hm.mxfp8_block_scaled_dot(64, 256, 32, batch=2, bias_gelu=True))
+    assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, block scales, batched]"] and rf == []
+    check(new, r"bf16\[2,64,32\]\{2,1,0\} custom-call\(%lhs, %rhs, %lhs_scale, %rhs_scale, %bias\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
+          r"epilogue = \\\"BIAS_GELU\\\"")
+    assert "tanh" not in new and "__op$block_scaled_dot" not in new
     new, rw, rf = hlo.rewrite(text.replace("f8e8m0fnu", "f8e5m2"))
     assert rw == [] and "__op$block_scaled_dot" in new and "f8e8m0fnu scales" in rf[0]
     new, rw, rf = hlo.rewrite(text.replace("%result = bf16[64,32]", "%result = f32[64,32]"))
-    assert rw == [] and "the result is f32" in rf[0]
+    assert rw == [] and "the value leaving the dot pattern is f32" in rf[0]
+    new, rw, rf = hlo.rewrite(text.replace("%rhs = f8e4m3fn[32,256]", "%rhs = f8e4m3fn[2,32,256]"))
+    assert rw == [] and "must all be rank 2, or rank 3" in rf[0]
 
 
 def test_quantizer_feeding_a_dot_becomes_two_calls():

@@ -504,9 +504,9 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   // per-tensor / per-row / per-channel f32 scales, or f8e8m0fnu block scales [rows, K/32] on both
   const bool mx = f->args.size > 3 && f->args.types[2] == XLA_FFI_ArgType_BUFFER &&
                   static_cast<XLA_FFI_Buffer*>(f->args.args[2])->dtype == XLA_FFI_DataType_F8E8M0FNU;
-  XLA_FFI_Buffer* sa = mx ? d.Arg(2, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 2, "a_scale")
+  XLA_FFI_Buffer* sa = mx ? d.Arg(2, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 3, "a_scale")
                           : d.Arg(2, Bit(XLA_FFI_DataType_F32), 0, 1, "a_scale");
-  XLA_FFI_Buffer* sb = mx ? d.Arg(3, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 2, "b_scale")
+  XLA_FFI_Buffer* sb = mx ? d.Arg(3, Bit(XLA_FFI_DataType_F8E8M0FNU), 2, 3, "b_scale")
                           : d.Arg(3, Bit(XLA_FFI_DataType_F32), 0, 1, "b_scale");
   // an F8E4M3FN result brings its scale as the last operand; a bias, if any, sits before it
   const bool out_f8 = f->rets.types[0] == XLA_FFI_RetType_BUFFER &&
@@ -544,10 +544,12 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
   p.batch = lead ? (a->dims[0] > 0 ? a->dims[0] : -1) : 1;  // -1: an empty batch, nothing to do
   std::string why;
   if (rcd != 0 && rcd != 1) why = "rhs_contracting_dim must be 0 or 1";
-  else if (mx && (lead || rcd != 1)) why = "block scales go with unbatched a [M,K] and b [N,K]";
+  else if (mx && rcd != 1) why = "block scales go with a [M,K] and b [N,K]";
+  else if (mx && (sa->rank != a->rank || sb->rank != a->rank)) why = "block scales have the rank of their operand";
   else if (b->rank != a->rank || out->rank != a->rank) why = "a, b and out must have the same rank";
   else if (lead && (b->dims[0] != p.batch || out->dims[0] != p.batch)) why = "batch dimensions differ";
-  else if (lead && (sa->rank != 0 || sb->rank != 0)) why = "a batched dot takes per-tensor scales";
+  else if (lead && !mx && (sa->rank != 0 || sb->rank != 0)) why = "a batched dot takes per-tensor scales";
+  else if (lead && mx && (sa->dims[0] != p.batch || sb->dims[0] != p.batch)) why = "batch dimensions differ";
   else {
     p.N = b->dims[lead + 1 - rcd];
     if (b->dims[lead + rcd] != p.K) why = "contracting dimensions differ";
@@ -555,8 +557,8 @@ XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* f) {
     else if (bias && bias->dims[0] != p.N) why = "bias must have N elements";
 
     else if (((at.epilogue & 1) != 0) != (bias != nullptr)) why = "a bias operand goes with a BIAS* epilogue, and only with one";
-    else if (mx && (p.K % 32 != 0 || sa->dims[0] != p.M || sb->dims[0] != p.N || sa->dims[1] != p.K / 32 ||
-                    sb->dims[1] != p.K / 32))
+    else if (mx && (p.K % 32 != 0 || sa->dims[lead] != p.M || sb->dims[lead] != p.N || sa->dims[lead + 1] != p.K / 32 ||
+                    sb->dims[lead + 1] != p.K / 32))
       why = "block scales must be [M,K/32] and [N,K/32]";
     else if (!mx && sa->rank == 1 && sa->dims[0] != p.M) why = "a rank-1 a_scale must have M elements";
     else if (!mx && sb->rank == 1 && sb->dims[0] != p.N) why = "a rank-1 b_scale must have N elements";

@@ -482,22 +482,37 @@ bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
   if (a->shape.dtype != "f8e4m3fn" || b->shape.dtype != "f8e4m3fn" || sa->shape.dtype != "f8e8m0fnu" ||
       sb->shape.dtype != "f8e8m0fnu")
     return refuse("operands must be f8e4m3fn with f8e8m0fnu scales");
-  if (a->shape.rank() != 2 || b->shape.rank() != 2 || sa->shape.rank() != 2 || sb->shape.rank() != 2 ||
-      cc->shape.is_tuple || cc->shape.rank() != 2)
-    return refuse("only unbatched rank-2 operands are supported");
-  const int64_t M = a->shape.dims[0], K = a->shape.dims[1], N = b->shape.dims[0];
-  if (b->shape.dims[1] != K || K % 32 != 0 || sa->shape.dims != std::vector<int64_t>{M, K / 32} ||
-      sb->shape.dims != std::vector<int64_t>{N, K / 32})
+  // one leading batch dimension, on all of them or on none (block_scaling_rewriter.h:53: the batch
+  // dimension, if present, is the major one)
+  const int64_t rank = a->shape.rank();
+  if ((rank != 2 && rank != 3) || b->shape.rank() != rank || sa->shape.rank() != rank || sb->shape.rank() != rank ||
+      cc->shape.is_tuple || cc->shape.rank() != rank)
+    return refuse("operands, scales and result must all be rank 2, or rank 3 with the batch dimension first");
+  const int64_t lead = rank - 2;
+  const int64_t M = a->shape.dims[lead], K = a->shape.dims[lead + 1], N = b->shape.dims[lead];
+  std::vector<int64_t> sa_dims = {M, K / 32}, sb_dims = {N, K / 32}, out_dims = {M, N};
+  if (lead) {
+    const int64_t B = a->shape.dims[0];
+    if (b->shape.dims[0] != B) return refuse("batch dimensions differ");
+    for (auto* d : {&sa_dims, &sb_dims, &out_dims}) d->insert(d->begin(), B);
+  }
+  if (b->shape.dims[lead + 1] != K || K % 32 != 0 || sa->shape.dims != sa_dims || sb->shape.dims != sb_dims)
     return refuse("scales must be one per 32 elements of the contracting (minor) dimension");
   if (cc->Attr("backend_config")) return refuse("a backend_config (explicit block size, global scale) is not taken");
-  if (cc->shape.dtype != "bf16" || cc->shape.dims != std::vector<int64_t>{M, N})
-    return refuse("the result is " + cc->shape.dtype + ", the kernels produce bf16 [M,N]");
+  if (!IsFloatTy(cc->shape.dtype) || cc->shape.dims != out_dims)
+    return refuse("the result is " + cc->shape.dtype + ", the kernels produce bf16 [M,N] from a bf16 or f32 dot");
+  // what follows the dot (bias, activation, the convert to bf16) goes into the call like behind an
+  // ordinary dot; the value that leaves must be bf16
   Epilogue ep;
-  ep.ops_type = "f32";
-  std::string cfg = CommonConfig(ep, "f32", "f32") + ", rhs_contracting_dim = 1 : i64";
-  Instr* call = EmitCall(comp, cc, "xla_amd.fp8_scaled_dot", {a, b, sa, sb}, {Shape::Array("bf16", {M, N})}, cfg);
-  comp->ReplaceAllUses(cc, call);
-  log->rewrites.push_back(cc->name + " -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]");
+  std::string why;
+  if (!MatchEpilogue(cc, &ep, &why)) return refuse(why);
+  std::vector<Instr*> ops = {a, b, sa, sb};
+  if (ep.bias) ops.push_back(ep.bias);
+  std::string cfg = CommonConfig(ep, "f32", cc->shape.dtype) + ", rhs_contracting_dim = 1 : i64";
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, {Shape::Array("bf16", out_dims)}, cfg);
+  comp->ReplaceAllUses(ep.tail, call);
+  log->rewrites.push_back(cc->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + ", block scales" +
+                          (lead ? ", batched" : "") + "]");
   return true;
 }
 

@@ -342,8 +342,10 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
 
   // kFp8MX: scales [rows, K/32]; lane l of wave w owns tile row (w & 3) * 64 + l of its operand
   const int nblk = p.K >> 5;
-  const __amdgpu_buffer_rsrc_t rsa = tile_rsrc(MX ? p.a_block_scales : p.a, MX ? (uint32_t)p.M * (uint32_t)nblk : 0u);
-  const __amdgpu_buffer_rsrc_t rsb = tile_rsrc(MX ? p.b_block_scales : p.a, MX ? (uint32_t)p.N * (uint32_t)nblk : 0u);
+  const __amdgpu_buffer_rsrc_t rsa =
+      tile_rsrc(MX ? p.a_block_scales + (size_t)batch * p.M * nblk : p.a, MX ? (uint32_t)p.M * (uint32_t)nblk : 0u);
+  const __amdgpu_buffer_rsrc_t rsb =
+      tile_rsrc(MX ? p.b_block_scales + (size_t)batch * p.N * nblk : p.a, MX ? (uint32_t)p.N * (uint32_t)nblk : 0u);
   const uint32_t sc_voff = (uint32_t)((wave < 4 ? m0 : n0) + (wave & 3) * 64 + lane) * (uint32_t)nblk;
 
   // ---- direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fills slot l%8
@@ -953,6 +955,10 @@ __global__ __launch_bounds__(256) void fp8_dot_exact_kernel(TiledParams p, int b
   if (p.out8) p.out8 += (size_t)blockIdx.y * total;
   const bool mx = p.a_block_scales != nullptr;
   const int nblk = p.K >> 5;
+  if (mx) {
+    p.a_block_scales += (size_t)blockIdx.y * p.M * nblk;
+    p.b_block_scales += (size_t)blockIdx.y * p.N * nblk;
+  }
   // the grid is bounded (a call that returns at the first line costs a few workgroups, not one
   // per 256 outputs): each workgroup strides over the outputs
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
@@ -1291,10 +1297,10 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
                   "fp8_scaled_dot: block scales come for both operands, one per 32 elements of K");
     if (p.rhs_contracting_dim != 1)
       return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: a block-scaled rhs is [N,K]");
-    if (p.a_scale_per_row || p.b_scale_per_channel || p.batch > 1 || p.out_dtype == XLA_FFI_DataType_F8E4M3FN ||
+    if (p.a_scale_per_row || p.b_scale_per_channel || p.out_dtype == XLA_FFI_DataType_F8E4M3FN ||
         p.dequant_type != XLA_FFI_DataType_F32)
       return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED,
-                  "fp8_scaled_dot: block scales go with an unbatched bf16 result and no other scales");
+                  "fp8_scaled_dot: block scales go with a bf16 result and no other scales");
   }
   if (!p.a || !p.b || (!mx && (!p.a_scale || !p.b_scale)) || !p.out)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: null buffer");
@@ -1436,7 +1442,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     tt.b = b_nk;
     int rc;
     if (mx)
-      rc = launch_tiled<kFp8MX>(tt, 1, stream, "fp8_scaled_dot_tiled_mx");
+      rc = launch_tiled<kFp8MX>(tt, batch, stream, "fp8_scaled_dot_tiled_mx");
     else if (out_f8)
       rc = kn_direct ? launch_tiled<kFp8KN, true>(tt, batch, stream, "fp8_scaled_dot_tiled_kn_f8")
                      : launch_tiled<kFp8, true>(tt, batch, stream, "fp8_scaled_dot_tiled_f8");

@@ -254,17 +254,49 @@ ENTRY %main {{
 """
 
 
-def mxfp8_block_scaled_dot(M=8192, K=8192, N=8192):
+def mxfp8_block_scaled_dot(M=8192, K=8192, N=8192, batch=0, bias_gelu=False):
     """MXFP8: f8e4m3fn operands [M,K] and [N,K] with one f8e8m0fnu scale per 32 elements of K, as
-    the "__op$block_scaled_dot" custom call of block_scaling_rewriter.h:48-69 -> bf16 [M,N]."""
-    return f"""HloModule mxfp8_block_scaled_dot
+    the "__op$block_scaled_dot" custom call of block_scaling_rewriter.h:48-69 -> bf16 [M,N].
+    batch: a leading batch dimension on every operand and the result (the header's second example).
+    bias_gelu: the custom call yields f32 and a bias add and GELU(tanh) follow before the convert
+    to bf16, as behind the dot of c3_fp8."""
+    lead = f"{batch}," if batch else ""
+    o = f"{lead}{M},{N}"
+    head = f"""HloModule mxfp8_block_scaled_dot
 
 ENTRY %main {{
-  %lhs = f8e4m3fn[{M},{K}] parameter(0)
-  %rhs = f8e4m3fn[{N},{K}] parameter(1)
-  %lhs_scale = f8e8m0fnu[{M},{K // 32}] parameter(2)
-  %rhs_scale = f8e8m0fnu[{N},{K // 32}] parameter(3)
-  ROOT %result = bf16[{M},{N}] custom-call(%lhs, %rhs, %lhs_scale, %rhs_scale), custom_call_target="__op$block_scaled_dot"
+  %lhs = f8e4m3fn[{lead}{M},{K}] parameter(0)
+  %rhs = f8e4m3fn[{lead}{N},{K}] parameter(1)
+  %lhs_scale = f8e8m0fnu[{lead}{M},{K // 32}] parameter(2)
+  %rhs_scale = f8e8m0fnu[{lead}{N},{K // 32}] parameter(3)
+"""
+    if not bias_gelu:
+        return head + f"""  ROOT %result = bf16[{o}] custom-call(%lhs, %rhs, %lhs_scale, %rhs_scale), custom_call_target="__op$block_scaled_dot"
+}}
+"""
+    return head + f"""  %bias = bf16[{N}] parameter(4)
+  %dot = f32[{o}] custom-call(%lhs, %rhs, %lhs_scale, %rhs_scale), custom_call_target="__op$block_scaled_dot"
+  %bias_t = f32[{N}] convert(%bias)
+  %bias_b = f32[{o}] broadcast(%bias_t), dimensions={{{2 if batch else 1}}}
+  %z = f32[{o}] add(%dot, %bias_b)
+  %z2 = f32[{o}] multiply(%z, %z)
+  %z3 = f32[{o}] multiply(%z, %z2)
+  %c0 = f32[] constant(0.044715)
+  %c0_b = f32[{o}] broadcast(%c0), dimensions={{}}
+  %z3c = f32[{o}] multiply(%z3, %c0_b)
+  %inner = f32[{o}] add(%z, %z3c)
+  %c1 = f32[] constant(0.797884583)
+  %c1_b = f32[{o}] broadcast(%c1), dimensions={{}}
+  %arg = f32[{o}] multiply(%inner, %c1_b)
+  %tanh = f32[{o}] tanh(%arg)
+  %one = f32[] constant(1)
+  %one_b = f32[{o}] broadcast(%one), dimensions={{}}
+  %onep = f32[{o}] add(%tanh, %one_b)
+  %half = f32[] constant(0.5)
+  %half_b = f32[{o}] broadcast(%half), dimensions={{}}
+  %cdf = f32[{o}] multiply(%onep, %half_b)
+  %gelu = f32[{o}] multiply(%z, %cdf)
+  ROOT %out = bf16[{o}] convert(%gelu)
 }}
 """
 

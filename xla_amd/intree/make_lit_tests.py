@@ -45,6 +45,8 @@ def cases():
         ("quant_fusion_rewriter_int4_weights_on_the_rhs_f32", hm.int4_weights_dot(hm.INT4_DOT_CASES[1], False)),
         ("quant_fusion_rewriter_int4_weights_on_the_lhs_f32", hm.int4_weights_dot(hm.INT4_DOT_CASES[3], True)),
         ("quant_fusion_rewriter_int4_weights_on_the_lhs_batched", hm.int4_weights_dot(hm.INT4_DOT_CASES[9], True)),
+        ("quant_fusion_rewriter_mxfp8_block_scaled_dot", hm.mxfp8_block_scaled_dot(64, 256, 32)),
+        ("quant_fusion_rewriter_mxfp8_batched_bias_gelu", hm.mxfp8_block_scaled_dot(64, 256, 32, batch=2, bias_gelu=True)),
         ("quant_fusion_rewriter_refuses_far_gelu_constant", gelu_far),
     ]
 

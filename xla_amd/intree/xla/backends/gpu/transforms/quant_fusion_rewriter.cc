@@ -428,22 +428,38 @@ bool RewriteBlockScaledDot(HloComputation* comp, Instr* cc, const std::function<
         *sb = cc->mutable_operand(3);
   if (Ty(a) != F8E4M3FN || Ty(b) != F8E4M3FN || Ty(sa) != F8E8M0FNU || Ty(sb) != F8E8M0FNU)
     return refuse("operands must be f8e4m3fn with f8e8m0fnu scales");
-  if (Rank(a) != 2 || Rank(b) != 2 || Rank(sa) != 2 || Rank(sb) != 2 || cc->shape().IsTuple() || Rank(cc) != 2)
-    return refuse("only unbatched rank-2 operands are supported");
-  const int64_t M = a->shape().dimensions(0), K = a->shape().dimensions(1), N = b->shape().dimensions(0);
-  if (b->shape().dimensions(1) != K || K % 32 != 0 || Dims(sa) != std::vector<int64_t>{M, K / 32} ||
-      Dims(sb) != std::vector<int64_t>{N, K / 32})
+  // one leading batch dimension, on all of them or on none (block_scaling_rewriter.h:53: the batch
+  // dimension, if present, is the major one)
+  const int64_t rank = Rank(a);
+  if ((rank != 2 && rank != 3) || Rank(b) != rank || Rank(sa) != rank || Rank(sb) != rank || cc->shape().IsTuple() ||
+      Rank(cc) != rank)
+    return refuse("operands, scales and result must all be rank 2, or rank 3 with the batch dimension first");
+  const int64_t lead = rank - 2;
+  const int64_t M = a->shape().dimensions(lead), K = a->shape().dimensions(lead + 1), N = b->shape().dimensions(lead);
+  std::vector<int64_t> sa_dims = {M, K / 32}, sb_dims = {N, K / 32}, out_dims = {M, N};
+  if (lead) {
+    const int64_t B = a->shape().dimensions(0);
+    if (b->shape().dimensions(0) != B) return refuse("batch dimensions differ");
+    for (auto* d : {&sa_dims, &sb_dims, &out_dims}) d->insert(d->begin(), B);
+  }
+  if (b->shape().dimensions(lead + 1) != K || K % 32 != 0 || Dims(sa) != sa_dims || Dims(sb) != sb_dims)
     return refuse("scales must be one per 32 elements of the contracting (minor) dimension");
   if (!cc->raw_backend_config_string().empty())
     return refuse("a backend_config (explicit block size, global scale) is not taken");
-  if (Ty(cc) != BF16 || Dims(cc) != std::vector<int64_t>{M, N})
-    return refuse("the result is " + TyName(Ty(cc)) + ", the kernels produce bf16 [M,N]");
+  if (!IsFloatTy(Ty(cc)) || Dims(cc) != out_dims)
+    return refuse("the result is " + TyName(Ty(cc)) + ", the kernels produce bf16 [M,N] from a bf16 or f32 dot");
+  // what follows the dot (bias, activation, the convert to bf16) goes into the call like behind an
+  // ordinary dot; the value that leaves must be bf16
   Epilogue ep;
-  ep.ops_type = F32;
-  std::string cfg = CommonConfig(ep, F32, F32) + ", rhs_contracting_dim = 1 : i64";
-  Instr* call = EmitCall(comp, "xla_amd.fp8_scaled_dot", {a, b, sa, sb}, {ShapeUtil::MakeShape(BF16, {M, N})}, cfg);
-  CHECK_OK(cc->ReplaceAllUsesWith(call));
-  VLOG(1) << cc->name() << " -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]";
+  std::string why;
+  if (!MatchEpilogue(cc, &ep, &why, /*allow_f8_result=*/false)) return refuse(why);
+  std::vector<Instr*> ops = {a, b, sa, sb};
+  if (ep.bias) ops.push_back(ep.bias);
+  std::string cfg = CommonConfig(ep, F32, Ty(cc)) + ", rhs_contracting_dim = 1 : i64";
+  Instr* call = EmitCall(comp, "xla_amd.fp8_scaled_dot", ops, {ShapeUtil::MakeShape(BF16, out_dims)}, cfg);
+  CHECK_OK(ep.tail->ReplaceAllUsesWith(call));
+  VLOG(1) << cc->name() << " -> xla_amd.fp8_scaled_dot [" << ep.Name() << ", block scales" << (lead ? ", batched" : "")
+          << "]";
   return true;
 }
 
