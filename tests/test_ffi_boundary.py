@@ -143,7 +143,7 @@ def test_shape_validation_happens_before_any_launch():
     # block scales: f8e8m0fnu [rows, K/32] on both operands, rhs [N,K]
     mx = [(dtypes.F8E4M3FN, FAKE, (4, 64)), (dtypes.F8E4M3FN, FAKE, (8, 64)), (dtypes.F8E8M0FNU, FAKE, (4, 2)),
           (dtypes.F8E8M0FNU, FAKE, (8, 2))]
-    with pytest.raises(ffi.FfiError, match="block scales go with unbatched a \\[M,K\\] and b \\[N,K\\]"):
+    with pytest.raises(ffi.FfiError, match="block scales go with a \\[M,K\\] and b \\[N,K\\]"):
         ffi.invoke("xla_amd.fp8_scaled_dot", ffi.Frame(host, mx, [(dtypes.BF16, FAKE, (4, 64))]))
     with pytest.raises(ffi.FfiError, match="block scales must be \\[M,K/32\\] and \\[N,K/32\\]"):
         bad = list(mx)
