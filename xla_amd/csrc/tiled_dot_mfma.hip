@@ -373,10 +373,19 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     }
   }
 
+  // ---- integer weights travel global -> registers -> (dequantised) LDS.  Two sets of registers: the
+  // loads run three stages ahead of the MFMAs, the conversion one stage ahead, cut into four parts
+  // that issue in the shadow of the current stage's matrix instructions (see the main loop).
+  struct WSet {
+    uint32_t w[8];   // the thread's weights of one stage
+    uintx4 sc;       // kS4, kU4: the bf16 scales of its 8 channels
+    uint32_t z;      // kU4: their zero points, one nibble each
+    uint32_t nks;    // kS4NK: the scale of its 32 k
+  };
+  WSet ws0, ws1;
   // ---- s8 weights: a thread takes 4 channels (quad nq) of the 8 rows of block kblk
-  uint32_t wreg[8];
   const int w_nq = tid & 63, w_kblk = tid >> 6;
-  auto s8_load = [&](int k0) {
+  auto s8_load = [&](int k0, WSet& w) {
     const uint32_t col = (uint32_t)(n0 + w_nq * 4);
     const uint32_t kfirst = (uint32_t)(k0 + w_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
     // (one select for the block, not a branch per row: the loads sit between the matrix instructions)
@@ -385,14 +394,14 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const uint32_t first = (kfirst * (uint32_t)p.N + col) | (live ? 0u : kOutOfRange);
 #pragma unroll
     for (int r = 0; r < 8; ++r)
-      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * (uint32_t)p.N, 0, 0);
+      w.w[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * (uint32_t)p.N, 0, 0);
   };
-  auto s8_store = [&](uint8_t* bt) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
+  auto s8_store = [&](uint8_t* bt, const WSet& w, int part) {  // part: the byte of each dword, one channel
+    {
+      const int e = part;
       float f[8];
 #pragma unroll
-      for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((wreg[r] >> (8 * e)) & 0xffu);
+      for (int r = 0; r < 8; ++r) f[r] = (float)(int8_t)((w.w[r] >> (8 * e)) & 0xffu);
       const uintx4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
                         pack_bf16x2(f[6], f[7])};
       const int n = w_nq * 4 + e;
@@ -406,7 +415,6 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // four rows and the kernel was 11 % slower), and the 8 lanes of a row block write 8 different
   // 16-byte chunks.  Waves 0-3 / 4-7 dequantise nibble pairs (0,4),(1,5) / (2,6),(3,7) of the same
   // dwords.  The group's 8 bf16 scales ride along.
-  uintx4 s4_scales = {0u, 0u, 0u, 0u};
   const int q_kblk = lane >> 3, q_oct = (wave & 3) * 8 + (lane & 7), q_half = wave >> 2;
   const uint32_t s4_pitch = (uint32_t)p.N >> 1;
   const __amdgpu_buffer_rsrc_t rsc4 =
@@ -415,12 +423,11 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
                 W4 ? (uint32_t)(p.K >> p.group_shift) * (uint32_t)p.N * 2u : 0u);
   // kU4: the zero points of the lane's 8 channels, one dword per group of rows; without zero points
   // the descriptor is empty and the loads return zero
-  uint32_t u4_zeros = 0u;
   const bool has_zp = U4 && p.zero_points != nullptr;
   const __amdgpu_buffer_rsrc_t rzp =
       tile_rsrc(has_zp ? p.zero_points + (size_t)(p.scale_batched ? batch : 0) * (size_t)(p.K >> p.group_shift) * (p.N >> 1) : p.a,
                 has_zp ? (uint32_t)(p.K >> p.group_shift) * ((uint32_t)p.N >> 1) : 0u);
-  auto s4_load = [&](int k0) {
+  auto s4_load = [&](int k0, WSet& w) {
     const uint32_t col = (uint32_t)(n0 + q_oct * 8);
     const uint32_t kfirst = (uint32_t)(k0 + q_kblk * 8);       // K % 8 == 0: the block is inside K or not at all
     const bool live = col < (uint32_t)p.N && kfirst < (uint32_t)p.K;  // N % 8 == 0
@@ -428,36 +435,36 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     const uint32_t first = (kfirst * s4_pitch + (col >> 1)) | (live ? 0u : kOutOfRange);
 #pragma unroll
     for (int r = 0; r < 8; ++r)
-      wreg[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * s4_pitch, 0, 0);
-    s4_scales = __builtin_amdgcn_raw_buffer_load_b128(
+      w.w[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, first + (uint32_t)r * s4_pitch, 0, 0);
+    w.sc = __builtin_amdgcn_raw_buffer_load_b128(
         rsc4, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) * 2u : kOutOfRange, 0, 0);
     if constexpr (U4)
-      u4_zeros = __builtin_amdgcn_raw_buffer_load_b32(rzp, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) >> 1 : kOutOfRange, 0, 0);
+      w.z = __builtin_amdgcn_raw_buffer_load_b32(rzp, live ? ((kfirst >> p.group_shift) * (uint32_t)p.N + col) >> 1 : kOutOfRange, 0, 0);
   };
-  auto s4_store = [&](uint8_t* bt) {
+  auto s4_store = [&](uint8_t* bt, const WSet& w, int part) {  // part: (sl, hi), one channel
     typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
-#pragma unroll
-    for (int sl = 0; sl < 2; ++sl) {
+    {
+      const int sl = part >> 1;
       // nibbles (e, e + 4), e = 2 * q_half + sl, as the f16 pair (1024 + u, 1024 + u) or, for odd
       // e, (1024 + 16 u, 1024 + 16 u), u = w + 8 (kU4: the nibble itself): see dequant_dot_decode.hip
       halfx2 pr[8];
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
-        const uint32_t x = q_half ? wreg[r] >> 8 : wreg[r];
+        const uint32_t x = q_half ? w.w[r] >> 8 : w.w[r];
         pr[r] = __builtin_bit_cast(halfx2, sl ? __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, U4 ? 0x64006400u : 0x64806480u, 0x6a)
                                               : __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, U4 ? 0x64006400u : 0x64086408u, 0x6a));
       }
-#pragma unroll
-      for (int hi = 0; hi < 2; ++hi) {
+      {
+        const int hi = part & 1;
         const int e_lo = sl + 4 * hi;  // nibble index when q_half == 0; + 2 otherwise
-        const uint32_t sw0 = s4_scales[(e_lo) >> 1], sw1 = s4_scales[(e_lo + 2) >> 1];
+        const uint32_t sw0 = w.sc[(e_lo) >> 1], sw1 = w.sc[(e_lo + 2) >> 1];
         const uint32_t sw = q_half ? sw1 : sw0;  // e and e + 2 have the same parity: same half of the dword
         const float v = (e_lo & 1) ? bf16hi_to_f32(sw) : bf16lo_to_f32(sw);
         const float sj = sl ? v * 0.0625f : v;
         float cj = sl ? v * -72.0f : v * -1032.0f;
         if constexpr (U4) {
           // the zero point in place of the 8: -(1024 + z) s, or -(64 + z) s next to 1024 + 16 u (exact in f32)
-          const float z = (float)((u4_zeros >> (4 * (e_lo + 2 * q_half))) & 0xfu);
+          const float z = (float)((w.z >> (4 * (e_lo + 2 * q_half))) & 0xfu);
           cj = v * (sl ? -64.0f - z : -1024.0f - z);
         }
         float f[8];
@@ -476,8 +483,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   // read the 64 contiguous bytes of one channel -- and each piece becomes chunks 2 * piece, + 1.
   // (K % 32 == 0 for s4 and % 16 for s8: a 16-byte piece lies inside its row or past it.)
   const int nk_n = KIND == kS8NK ? tid >> 2 : tid >> 1, nk_half = tid & 1, nk_piece = tid & 3;
-  uint32_t nk_scale = 0;
-  auto nk_load = [&](int k0) {
+  auto nk_load = [&](int k0, WSet& w) {
     const uint32_t ch = (uint32_t)(n0 + nk_n);
     const uint32_t k = (uint32_t)(k0 + nk_half * 32);
     if constexpr (KIND == kS8NK) {
@@ -487,33 +493,33 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
         const uint32_t cj = ch + 128u * j;
         const bool live = cj < (uint32_t)p.N && kp < (uint32_t)p.K;
         const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? cj * (uint32_t)p.K + kp : kOutOfRange, 0, 0);
-        wreg[4 * j] = v[0]; wreg[4 * j + 1] = v[1]; wreg[4 * j + 2] = v[2]; wreg[4 * j + 3] = v[3];
+        w.w[4 * j] = v[0]; w.w[4 * j + 1] = v[1]; w.w[4 * j + 2] = v[2]; w.w[4 * j + 3] = v[3];
       }
     } else {
       const bool live = ch < (uint32_t)p.N && k < (uint32_t)p.K;
       const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(rb, live ? (ch * (uint32_t)p.K + k) >> 1 : kOutOfRange, 0, 0);
-      wreg[0] = v[0]; wreg[1] = v[1]; wreg[2] = v[2]; wreg[3] = v[3];
+      w.w[0] = v[0]; w.w[1] = v[1]; w.w[2] = v[2]; w.w[3] = v[3];
       // the lane's 32 k share a scale (groups of at least 32, or one scale per channel: shift 31)
-      nk_scale = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(
+      w.nks = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(
           rsc4, live ? (ch * (uint32_t)(p.K >> p.group_shift) + (k >> p.group_shift)) * 2u : kOutOfRange, 0, 0);
     }
   };
-  auto nk_store = [&](uint8_t* bt) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
+  auto nk_store = [&](uint8_t* bt, const WSet& w, int part) {  // part: one 16-byte chunk of the row
+    {
+      const int c = part;
       float f[8];
       if constexpr (KIND == kS8NK) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          f[e] = (float)(int8_t)((wreg[2 * c] >> (8 * e)) & 0xffu);
-          f[4 + e] = (float)(int8_t)((wreg[2 * c + 1] >> (8 * e)) & 0xffu);
+          f[e] = (float)(int8_t)((w.w[2 * c] >> (8 * e)) & 0xffu);
+          f[4 + e] = (float)(int8_t)((w.w[2 * c + 1] >> (8 * e)) & 0xffu);
         }
       } else {
         typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
         // nibble pairs (0,4), (1,5) of x and (2,6), (3,7) of x >> 8 as f16 1024 + u or 1024 + 16 u,
         // u = w + 8; one fma each takes the offset out and the scale in: see dequant_dot_decode.hip
-        const uint32_t x = wreg[c];
-        const float v = bf16lo_to_f32(nk_scale);
+        const uint32_t x = w.w[c];
+        const float v = bf16lo_to_f32(w.nks);
         const float s_even = v, c_even = v * -1032.0f, s_odd = v * 0.0625f, c_odd = v * -72.0f;
         const halfx2 p04 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x000f000fu, 0x64086408u, 0x6a));
         const halfx2 p15 = __builtin_bit_cast(halfx2, __builtin_amdgcn_bitop3_b32(x, 0x00f000f0u, 0x64806480u, 0x6a));
@@ -536,10 +542,15 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
       *reinterpret_cast<uintx4*>(bt + row * kRow + ((chunk ^ ((row >> 1) & 7)) << 4)) = o;
     }
   };
-  auto wq_store = [&](uint8_t* bt) {
-    if constexpr (KIND == kS8) s8_store(bt);
-    if constexpr (KIND == kS4 || KIND == kU4) s4_store(bt);
-    if constexpr (KIND == kS8NK || KIND == kS4NK) nk_store(bt);
+  auto wq_store = [&](uint8_t* bt, const WSet& w, int part) {
+    if constexpr (KIND == kS8) s8_store(bt, w, part);
+    if constexpr (KIND == kS4 || KIND == kU4) s4_store(bt, w, part);
+    if constexpr (KIND == kS8NK || KIND == kS4NK) nk_store(bt, w, part);
+  };
+  auto wq_load = [&](int k0, WSet& w) {  // k0 past K: every load lands as zeros without touching memory
+    if constexpr (KIND == kS8) s8_load(k0, w);
+    if constexpr (KIND == kS4 || KIND == kU4) s4_load(k0, w);
+    if constexpr (KIND == kS8NK || KIND == kS4NK) nk_load(k0, w);
   };
 
   auto issue_loads = [&](int buf, int k0) {
@@ -558,9 +569,6 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
         load_to_lds(rb, bt + (wave * 16 + j * 4) * 256, v);
       }
     }
-    if (KIND == kS8) s8_load(k0);
-    if (KIND == kS4 || KIND == kU4) s4_load(k0);
-    if (KIND == kS8NK || KIND == kS4NK) nk_load(k0);
     if (MX) {
       // the stage's four scale bytes of every tile row, one dword per row: waves 0-3 fetch the
       // 256 token rows, waves 4-7 the 256 channel rows (64 lanes x 4 bytes land contiguously)
@@ -683,39 +691,98 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   int s_begin = role == 1 ? half : 0, s_end = role == 2 ? half : stages;
   bool add_sums = false;
   __shared__ int tail_arrived;
+  // Integer-weight kinds: VMEM instructions of one stage's weight loads (the wait in front of the
+  // stage barrier lets exactly those stay in flight)
+  constexpr int kWLoads = KIND == kS8 ? 8 : KIND == kS4 ? 9 : KIND == kU4 ? 10 : 2;
+  constexpr int kPastK = 0x40000000;  // a k0 no matrix reaches: the weight loads of such a stage fetch nothing
   for (;;) {
-    issue_loads(0, s_begin * KS);
-    if (WQ) wq_store(lds + kTM * kRow);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
-    issue_loads(1, (s_begin + 1) * KS);  // past K: lands as zeros, never read
-    for (int s = s_begin; s + 1 < s_end; ++s) {
-      const int buf = (s - s_begin) & 1;
+    if constexpr (WQ) {
+      // Weights: loaded three stages ahead into one of two register sets, dequantised into the other
+      // stage buffer one stage ahead, a quarter of the conversion behind each of the current stage's
+      // first three MFMA steps (the last quarter rides with the third), where its VALU instructions
+      // issue while the matrix pipe works.  Activations: DMA two stages ahead, as for the f8 kinds.
+      uint8_t* const wt0 = lds + kTM * kRow;
+      uint8_t* const wt1 = lds + kBufBytes + kTM * kRow;
+      issue_loads(0, s_begin * KS);
+      wq_load(s_begin * KS, ws0);
 #pragma unroll
-      for (int ks = 0; ks + 1 < NKS; ++ks) {
-        read_frags(buf, ks);
-        mfma_all(ks);
-      }
-      read_frags(buf, NKS - 1);
-      if (WQ) wq_store(lds + (buf ^ 1) * kBufBytes + kTM * kRow);
+      for (int part = 0; part < 4; ++part) wq_store(wt0, ws0, part);
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();
-      issue_loads(buf, (s + 2) * KS);  // past this workgroup's stages in the last rounds: into a buffer nobody reads
-      mfma_all(NKS - 1);
-      if (F8) {
+      issue_loads(1, (s_begin + 1) * KS);  // past K: lands as zeros, never read
+      __builtin_amdgcn_sched_barrier(0);   // the activation loads stay older than the weight loads
+      wq_load(s_begin + 1 < s_end ? (s_begin + 1) * KS : kPastK, ws1);
+      wq_load(s_begin + 2 < s_end ? (s_begin + 2) * KS : kPastK, ws0);
+      auto stage = [&](int buf, uint8_t* wt_next, WSet& set, int s) __attribute__((always_inline)) {
+        read_frags(buf, 0);
+        mfma_all(0);
+        wq_store(wt_next, set, 0);
+        read_frags(buf, 1);
+        mfma_all(1);
+        wq_store(wt_next, set, 1);
+        read_frags(buf, 2);
+        mfma_all(2);
+        wq_store(wt_next, set, 2);
+        wq_store(wt_next, set, 3);
+        read_frags(buf, 3);
+        // the next stage's activations have landed (the weight loads issued after them may still fly),
+        // this wave's LDS reads and writes are done
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kWLoads) : "memory");
+        __syncthreads();
+        issue_loads(buf, (s + 2) * KS);  // past this workgroup's stages in the last rounds: into a buffer nobody reads
+        __builtin_amdgcn_sched_barrier(0);
+        wq_load(s + 3 < s_end ? (s + 3) * KS : kPastK, set);
+        mfma_all(3);
+      };
+      int s = s_begin;
+      for (; s + 2 < s_end; s += 2) {
+        stage(0, wt1, ws1, s);
+        stage(1, wt0, ws0, s + 1);
+      }
+      if (s + 1 < s_end) {
+        stage(0, wt1, ws1, s);
+        ++s;
+      }
+      {  // last stage: nothing left to fetch or convert
+        const int buf = (s - s_begin) & 1;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+        for (int ks = 0; ks < NKS; ++ks) {
+          read_frags(buf, ks);
+          mfma_all(ks);
         }
       }
-    }
-    {  // last stage: nothing left to fetch
-      const int buf = (s_end - 1 - s_begin) & 1;
+    } else {
+      issue_loads(0, s_begin * KS);
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+      issue_loads(1, (s_begin + 1) * KS);  // past K: lands as zeros, never read
+      for (int s = s_begin; s + 1 < s_end; ++s) {
+        const int buf = (s - s_begin) & 1;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        read_frags(buf, ks);
-        mfma_all(ks);
+        for (int ks = 0; ks + 1 < NKS; ++ks) {
+          read_frags(buf, ks);
+          mfma_all(ks);
+        }
+        read_frags(buf, NKS - 1);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        issue_loads(buf, (s + 2) * KS);  // past this workgroup's stages in the last rounds: into a buffer nobody reads
+        mfma_all(NKS - 1);
+        if (F8) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // one buffer load
+          }
+        }
+      }
+      {  // last stage: nothing left to fetch
+        const int buf = (s_end - 1 - s_begin) & 1;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          read_frags(buf, ks);
+          mfma_all(ks);
+        }
       }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads issued past the end have landed
