@@ -43,6 +43,11 @@ struct DecodeParams {
   int units_per_simd2;  // the finisher's units per SIMD; its class split is class_units[2..3]
   unsigned long long* flags;
   unsigned long long epoch;
+  // s8x kernels with 64-channel strips and 1, 2 or 4 slices: workgroup ids are laid out so that the
+  // two strips that share a 128-byte line of every weight row lie 8 ids apart (the same XCD and L2
+  // when workgroups go round the XCDs in turn): id = 16 * G + 8 * half + pair_in_group * slices + slice,
+  // strip = 2 * (G * pairs_per_group + pair_in_group) + half.  0: strip = id / slices as usual.
+  int pairs_per_group;
   // Test aid (option "handover_test" = 1): producers never raise their flags and the waiting
   // workgroup gives up after a few polls, so that its own fallback computes the result.
   int handover_test;

@@ -45,8 +45,14 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 15, kb = lane >> 4;
   // workgroup ids in dispatch order: the slices of a strip follow each other, the finisher last
-  const int slice = blockIdx.x % p.slices;
-  const int strip = blockIdx.x / p.slices;
+  int slice = blockIdx.x % p.slices;
+  int strip = blockIdx.x / p.slices;
+  if (NV == 4 && p.pairs_per_group) {
+    const int low = blockIdx.x & 7;
+    slice = low % p.slices;
+    strip = 2 * ((blockIdx.x >> 4) * p.pairs_per_group + low / p.slices) + ((blockIdx.x >> 3) & 1);
+    if (strip >= p.strips) return;  // the grid is padded to whole groups of 16
+  }
   const int batch = blockIdx.y;
   const bool finisher = slice == p.slices - 1;
 
@@ -247,6 +253,10 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_dot_decode_s8x_kernel(Dec
 template <int STEPS, int NV>
 int launch_s8x(const DecodeParams& dp, int batch, hipStream_t stream, const char* name) {
   dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch);
+  if (NV == 4 && dp.pairs_per_group) {
+    const int pairs = (dp.strips + 1) / 2;
+    grid.x = (unsigned)((pairs + dp.pairs_per_group - 1) / dp.pairs_per_group * 16);
+  }
   hipLaunchKernelGGL((dequant_dot_decode_s8x_kernel<STEPS, NV>), grid, dim3(kWaves * 64), 0, stream, dp);
   const int rc = CheckLaunch(name);
   SetLastKernel(name);
@@ -311,6 +321,7 @@ int LaunchDequantDotDecodeS8x(DecodeParams dp, const XlaAmdDequantDot& p, hipStr
   dp.rows_per_slice = 256 * steps;
   dp.flags = nullptr;
   dp.epoch = 0;
+  dp.pairs_per_group = shape.channels == 64 && (dp.slices == 1 || dp.slices == 2 || dp.slices == 4) ? 8 / dp.slices : 0;
   if (dp.slices > 1) {
     const size_t need = S8xWorkspaceBytes(p.batch, p.M, p.K, p.N);
     if (!p.workspace || ((uintptr_t)p.workspace % 16) != 0 || p.workspace_bytes < need) return -1;
