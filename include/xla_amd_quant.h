@@ -92,9 +92,10 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  * CublasLtMatmulThunk -> hipBLASLt, xla/stream_executor/rocm/hip_blas_lt.cc:468-484).
  *   args: a F8E4M3FN [M,K]; b F8E4M3FN [K,N] (rhs_contracting_dim=0) or [N,K] (=1); or both
  *         with one leading batch dimension ([B,M,K], [B,K,N]|[B,N,K], out [B,M,N]: the batched
- *         dot of gemm_rewriter_fp8_test.cc:941-957), then with per-tensor scales only;
+ *         dot of gemm_rewriter_fp8_test.cc:941-957), then with per-tensor or block scales only;
  *         a_scale, b_scale F8E8M0FNU [M,K/32], [N,K/32] with b = [N,K]: block-scaled (MXFP8)
- *         operands, "__op$block_scaled_dot" of block_scaling_rewriter.h:48-69; otherwise
+ *         operands, "__op$block_scaled_dot" of block_scaling_rewriter.h:48-69 (a leading batch
+ *         dimension goes on the scales as well: [B,M,K/32], [B,N,K/32]); otherwise
  *         a_scale F32 [] or [M] (one per row of a, as a row-wise quantizer produces them);
  *         b_scale F32 [] or [N] (one per output channel); bias BF16|F32 [N] (only with BIAS*)
  *         d_scale F32 [] (last; only when out is F8E4M3FN)
@@ -238,8 +239,8 @@ typedef struct XlaAmdFp8ScaledDot {
   const float* d_scale;        /* device scalar, only with an F8E4M3FN result */
   float* amax;                 /* optional device scalar result with an F8E4M3FN result:
                                   max |v| over all outputs, NaN if any v is NaN */
-  const void* a_block_scales;  /* MXFP8: f8e8m0fnu [M, K/32], one scale per 32 elements of K of a;   */
-  const void* b_block_scales;  /* f8e8m0fnu [N, K/32] for b = [N,K]; both or neither; a_scale and   */
+  const void* a_block_scales;  /* MXFP8: f8e8m0fnu [batch, M, K/32], one per 32 elements of K of a;  */
+  const void* b_block_scales;  /* f8e8m0fnu [batch, N, K/32] for b = [N,K]; both or neither; a_scale and */
   int32_t block;               /* b_scale are unused then; block must be 32                          */
   int32_t reserved0;
   int64_t batch;               /* 0 or 1: a [M,K], b [K,N]|[N,K]; B > 1: a [B,M,K], b [B,K,N]|[B,N,K],
@@ -290,7 +291,10 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * off the matrix-instruction-dequantising and the single-launch kernels), "dequant_dot_pair" (1: two
  * workgroups per 256-channel strip wherever the shape allows, 2: never), "dequant_dot_share" (the
  * first workgroup's sixteenths of K), "dequant_dot_depth" (ring depth 2 or 4), "dequant_dot_steps"
- * (steps per wave of the single-launch s8 kernel: 1, 2, 4), "fp8_dot_kernel" (1 exact, 2 tiled),
+ * (steps per wave of the single-launch s8 kernel: 1, 2, 4), "dequant_dot_strip" (channels per strip of
+ * that kernel: 64 or 128), "handover_test" (1: workgroups that hand partial sums over never raise their
+ * flags and the waiting side gives up after 16 polls, so that its own fallback computes the result --
+ * for tests of that fallback only), "fp8_dot_kernel" (1 exact, 2 tiled),
  * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1:
  * the tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the
