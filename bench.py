@@ -8,7 +8,9 @@ the benchmark's shapes and distributions, and resident in HBM before the timed r
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-other] [--skip-cpu]
 
-Prints ONE JSON line: `value` = algorithmic bytes of a step / wall time per step (GB/s);
+Prints ONE JSON line: `value` = algorithmic bytes of a step / wall time per step (GB/s), over exactly
+K steps between two synchronisations, after the W warm-up steps and `settle_steps` further untimed
+steps that bring the clocks of a GPU that has idled back up;
 `roofline` = the step's slowest kernel against the 8 TB/s HBM peak, timed with events on the
 launch stream (every per-kernel `ms` is the median over 21 event-bracketed batches of back-to-back
 launches, `ms_best` the fastest batch); `cpu_baseline` = the CPU oracle on the same workload; `kernels` = every kernel of
