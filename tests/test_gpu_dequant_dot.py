@@ -438,6 +438,26 @@ def test_batched_decode(oracle):
     compare(oracle, w, got, "batched decode")
 
 
+@pytest.mark.parametrize("K", [8, 40, 64, 72, 128, 136, 192, 200, 256, 320])
+def test_tiled_kernels_with_few_stages(oracle, K):
+    """One to five stages of 64 rows, whole and ragged: the prologue that loads three stages of weights
+    ahead, the loop that runs stages in pairs, a lone stage after the pairs and the last stage."""
+    say("dequant_dot tiled kernels, K=%d" % K)
+    M, N = 130, 264
+    w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_s8_factored", kern
+    compare(oracle, w, got, "s8 tiled K=%d" % K)
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=8)
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_s4_rounded", kern
+    compare(oracle, w, got, "s4 tiled K=%d" % K)
+    w = workloads.u4_zero_point_group(M=M, K=K, N=N, group=8)
+    got, kern = run_dot(w, force_kernel=3)
+    assert kern == "dequant_dot_tiled_u4_rounded", kern
+    compare(oracle, w, got, "u4 tiled K=%d" % K)
+
+
 @pytest.mark.parametrize("M,K,N,group", [(200, 1024, 512, 128), (65, 264, 264, 8), (300, 2048, 1000, 64),
                                          (512, 512, 256, 512), (130, 1000, 72, 8)])
 def test_s4_group_scales_tiled(oracle, M, K, N, group):

@@ -213,6 +213,21 @@ def test_tiled_kernel_takes_k_minor_weights(oracle, kind, M, K, N, group):
     compare(oracle, w, got, "[N,K] tiled %s" % kern)
 
 
+@pytest.mark.parametrize("K", [32, 64, 96, 128, 160, 192, 256, 288])
+def test_tiled_k_minor_with_few_stages(oracle, K):
+    """One to five stages of 64 k through the [N,K] loaders of the tiled kernel."""
+    say("dequant_dot [N,K] tiled, K=%d" % K)
+    M, N = 130, 264
+    w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    got, kern = run_nk(w, force_kernel=3)
+    assert kern.startswith("dequant_dot_tiled_nk_s8_"), kern
+    compare(oracle, w, got, "[N,K] s8 tiled K=%d" % K)
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=32)
+    got, kern = run_nk(w, force_kernel=3)
+    assert kern.startswith("dequant_dot_tiled_nk_s4_"), kern
+    compare(oracle, w, got, "[N,K] s4 tiled K=%d" % K)
+
+
 def test_tiled_k_minor_batched_and_split_last_round(oracle):
     say("dequant_dot [B,N,K] tiled s8, tiles split along K")
     w = workloads.c5_s8_batched(B=2, M=300, K=2048, N=520)
