@@ -56,12 +56,17 @@ extern "C" {
  *         zero_points U4, shaped like the scales (optional; U4 weights only): the dequantised
  *                     weight is (w - zero_point) * scale
  *         bias        BF16 or F32 [N]            (optional; exactly with a BIAS* epilogue)
+ *         d_scale     F32 []                     (exactly with an F8E4M3FN out, after the bias): out is
+ *                     convert(clamp(-448, v / d_scale, 448)) of the f32 value v after the epilogue, the D
+ *                     scaling of gemm_rewriter_fp8_test.cc:1665-1690 (v * d_scale with d_scale_multiplies,
+ *                     :1730-1748) -- the next fp8 dot's activations made in this dot's store
  *         group_sizes S32 or S64 [G], last       (optional): a ragged dot -- lhs [M,K] with its rows
  *                     sorted by group, weights [G,K,N] (or [G,N,K]), out [M,N]; group g multiplies rows
  *                     [sum of the sizes before it, + its size), rows past the last group are epilogue(0)
  *                     (xla ragged-dot, ragged_dot_rewriter.cc:110-210; gemm_rewriter.cc:781-863)
- *   rets: out     BF16 or F32 [M,N] or [B,M,N] (F32: the value before the final convert, the root of
- *                 fusion_emitter_int4_device_test.cc:101,205,320,508); [..,N,M] with result_transposed
+ *   rets: out     BF16, F32 or F8E4M3FN [M,N] or [B,M,N] (F32: the value before the final convert, the
+ *                 root of fusion_emitter_int4_device_test.cc:101,205,320,508; F8E4M3FN: with d_scale);
+ *                 [..,N,M] with result_transposed
  *         scratch S8 or U8 [bytes]             (optional second result: what
  *                 xla_amd_dequant_dot_workspace_bytes[_nk] reports for the shape; without it the
  *                 kernels that need none run)
@@ -83,6 +88,7 @@ extern "C" {
  *                   activations' major dimension, shape table :609-645)
  *     result_transposed pred (default false): the dequantised weights were the lhs of the dot
  *                   (Int4WeightsOnTheLhs, :495-523), so out is [..,N,M]; DEFAULT epilogue only
+ *     d_scale_multiplies pred (default false): an F8E4M3FN out is v * d_scale, not v / d_scale
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame);
 
@@ -177,8 +183,8 @@ typedef struct XlaAmdDequantDot {
    * packed two per byte along K, scales and zero points are [batch or 1, N, K/group].  With
    * group_sizes the experts are [groups,N,K]. */
   int32_t rhs_contracting_dim;
-  /* Element type of out: BF16 (also 0) or F32 -- a dot whose f32 value is the result
-   * (fusion_emitter_int4_device_test.cc:101,205,320,508). */
+  /* Element type of out: BF16 (also 0), F32 -- a dot whose f32 value is the result
+   * (fusion_emitter_int4_device_test.cc:101,205,320,508) -- or F8E4M3FN with d_scale below. */
   int32_t out_dtype;
   /* 1: out is [batch,N,M]: the dequantised weights were the lhs of the dot
    * (Int4WeightsOnTheLhs, fusion_emitter_int4_device_test.cc:495-523); the epilogue must be DEFAULT. */
@@ -186,6 +192,11 @@ typedef struct XlaAmdDequantDot {
   /* 1: lhs (the activations) is stored [batch,K,M]: the dot contracts their major dimension
    * (the "128,16" x "128,256" cases of fusion_emitter_int4_device_test.cc:609-645). */
   int32_t lhs_k_major;
+  /* out_dtype F8E4M3FN: out holds convert(clamp(-448, v / d_scale, 448)) of the f32 value v after the
+   * epilogue (v * d_scale with d_scale_multiplies), as for xla_amd_fp8_scaled_dot: d_scale is one f32
+   * in device memory.  Such calls run on the general kernels (bf16 [M,N] results have the tuned ones). */
+  const float* d_scale;
+  int32_t d_scale_multiplies;
 } XlaAmdDequantDot;
 
 XLA_AMD_EXPORT int xla_amd_launch_dequant_dot(const XlaAmdDequantDot* p, void* stream);

@@ -1,19 +1,21 @@
 """Result and operand layouts of xla_amd.dequant_dot beyond bf16 [M,N] = lhs [M,K] . W: an f32 result
 (the dot's own value, fusion_emitter_int4_device_test.cc:101,205,320,508), the dequantised weights as
-the lhs of the dot (result [N,M], :495-523) and activations stored [K,M] (the dot contracts their
-major dimension, the shape table :609-645) -- against the CPU oracle, through the FFI handler."""
+the lhs of the dot (result [N,M], :495-523), activations stored [K,M] (the dot contracts their major dimension, the shape
+table :609-645) and an f8e4m3fn result (the D scaling of gemm_rewriter_fp8_test.cc:1665-1690, :1730-1748
+on the dot's f32 value) -- against the CPU oracle, through the FFI handler."""
 import numpy as np
 import pytest
 import torch
 
-from tests.gpu_util import check_dot, check_dot_f32, dev_bf16, dev_f32, dev_s8, dev_u8, host_bf16
+from tests.gpu_util import check_dot, check_dot_f32, check_f8_result, dev_bf16, dev_f32, dev_s8, dev_u8, host_bf16
 from tests.test_gpu_dequant_dot import floor_for, oracle_dot, say
 from xla_amd import dtypes, ffi, ops, workloads
 
 pytestmark = pytest.mark.gpu
 
 
-def run(w, nk=False, out_dtype="bf16", transposed=False, lhs_k_major=False, force_kernel=0):
+def run(w, nk=False, out_dtype="bf16", transposed=False, lhs_k_major=False, force_kernel=0, d_scale=None,
+        d_scale_multiplies=False):
     v = workloads.k_minor(w) if nk else w
     lhs_h = v["lhs"]
     if lhs_k_major:
@@ -34,11 +36,13 @@ def run(w, nk=False, out_dtype="bf16", transposed=False, lhs_k_major=False, forc
                               epilogue=v["epilogue"], dequant_type=v["dequant_type"],
                               scale_group_size=0 if w["group"] == K else w["group"],
                               rhs_contracting_dim=1 if nk else 0, out_dtype=out_dtype, result_transposed=transposed,
-                              lhs_contracting_dim=0 if lhs_k_major else 1)
+                              lhs_contracting_dim=0 if lhs_k_major else 1,
+                              d_scale=None if d_scale is None else dev_f32(np.array(d_scale, np.float32)),
+                              d_scale_multiplies=d_scale_multiplies)
         torch.cuda.synchronize()
     finally:
         ffi.set_option("dequant_dot_kernel", 0)
-    got = out.cpu().numpy() if out_dtype == "f32" else host_bf16(out)
+    got = out.cpu().numpy() if (out_dtype == "f32" or d_scale is not None) else host_bf16(out)
     if transposed:
         got = np.swapaxes(got, -1, -2)
     return got, ffi.last_kernel()
@@ -118,6 +122,82 @@ def test_one_hot_activations_read_single_weights_back_in_every_layout(oracle):
             for lhs_k_major in (False, True):
                 got, kern = run(w, nk=nk, out_dtype="f32", transposed=transposed, lhs_k_major=lhs_k_major)
                 assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32)), (nk, transposed, lhs_k_major, kern)
+
+
+def f8_codes(v, z, divides):
+    """convert(clamp(-448, v / z | v * z, 448)) op by op on f32, as the HLO evaluates it."""
+    v = np.asarray(v, np.float32)
+    t = (v / np.float32(z) if divides else v * np.float32(z)).astype(np.float32)
+    return dtypes.f32_to_f8e4m3fn(np.clip(t, -448, 448))
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("divides", [True, False])
+@pytest.mark.parametrize("kind,kw", CASES)
+def test_f8_result(oracle, kind, kw, nk, divides):
+    """An f8e4m3fn result: the codes of the oracle's f32 value scaled, clamped and cast, up to the window
+    the dot itself is matched to (the rule of the fp8 dot's f8 result)."""
+    say("dequant_dot f8 result %s %s nk=%s divides=%s" % (kind, kw, nk, divides))
+    w = make(kind, kw)
+    val = reference(oracle, w, True)
+    amax = float(np.nanmax(np.abs(val)))
+    # the largest value lands at 600: some codes saturate at 448, most use the format's whole range
+    z = np.float32(amax / 600.0) if divides else np.float32(600.0 / amax)
+    got, kern = run(w, nk=nk, d_scale=z, d_scale_multiplies=not divides)
+    assert got.dtype == np.uint8 and got.shape == val.shape
+    ref = f8_codes(val, z, divides)
+    assert (np.abs(dtypes.f8e4m3fn_to_f32(ref)) == 448).any()
+    differ = check_f8_result(got, ref, val, z, divides, floor_for(w), "f8 result %s" % kern)
+    assert differ <= max(8, got.size // 8), (differ, got.size)
+
+
+@pytest.mark.parametrize("divides", [True, False])
+def test_f8_result_of_single_weights_bit_exact(oracle, divides):
+    """One-hot activations make the dot's value a single dequantised weight, exact in f32: the codes
+    must then be exactly convert(clamp(v / z)) with an IEEE quotient (z is chosen so that v * (1/z)
+    rounds differently for many v), in every layout, saturating beyond +-448."""
+    say("dequant_dot f8 result, one-hot, divides=%s" % divides)
+    M, K, N, g = 6, 256, 64, 64
+    w = workloads.c2_s4_group(M=M, K=K, N=N, group=g)
+    hot = np.zeros((M, K), np.float32)
+    ks = [0, 1, 63, 64, 129, 255]
+    hot[np.arange(M), ks] = 1.0
+    w = dict(w, lhs=dtypes.f32_to_bf16(hot), epilogue="DEFAULT", bias=None)
+    s32 = dtypes.bf16_to_f32(w["scales"])
+    v = np.stack([dtypes.bf16_to_f32(dtypes.f32_to_bf16(w["weights"][k].astype(np.float32) * s32[k // g])) for k in ks])
+    amax = float(np.abs(v).max())
+    odd = np.frombuffer(np.uint32(0x3c7fffff).tobytes(), np.float32)[0]   # 0.0156249991: not a power of two
+    z = np.float32(odd * amax / 8.0) if divides else np.float32(500.0 / amax)
+    want = f8_codes(v, z, divides)
+    assert (np.abs(dtypes.f8e4m3fn_to_f32(want)) == 448).any()
+    for nk in (False, True):
+        for transposed in (False, True):
+            for lhs_k_major in (False, True):
+                got, kern = run(w, nk=nk, transposed=transposed, lhs_k_major=lhs_k_major, d_scale=z,
+                                d_scale_multiplies=not divides)
+                assert np.array_equal(got, want), (nk, transposed, lhs_k_major, kern, int((got != want).sum()))
+
+
+def test_f8_result_special_values(oracle):
+    """A NaN stays one through the clamp and +-inf saturates at +-448: a NaN scale in one channel, and
+    single products that overflow f32 (one-hot activations of +-3e38 on weights of magnitude >= 1)."""
+    say("dequant_dot f8 result, special values")
+    M, K, N = 4, 64, 32
+    w = workloads.c1_s8_channel(M=M, K=K, N=N)
+    hot = np.zeros((M, K), np.float32)
+    hot[np.arange(M), [0, 5, 17, 63]] = [1.0, 3e38, -3e38, 1.0]
+    sc = np.full(N, 4.0, np.float32)
+    sc[5] = np.nan
+    wt = w["weights"].copy()
+    wt[wt == 0] = 1
+    w = dict(w, lhs=dtypes.f32_to_bf16(hot), scales=sc, weights=wt, epilogue="DEFAULT", bias=None)
+    v = reference(oracle, w, True)
+    assert np.isinf(v[1:3, :5]).all() and np.isnan(v[:, 5]).all()
+    z = np.float32(0.25)
+    want = f8_codes(v, z, True)
+    got, kern = run(w, d_scale=z)
+    assert np.array_equal(got, want), (kern, int((got != want).sum()))
+    assert (want[:, 5] & 0x7f == 0x7f).all() and (want[1:3, :5] & 0x7f == 0x7e).all()
 
 
 def test_refusals():

@@ -55,6 +55,27 @@ def test_c2_module(M):
     check_dot(host_bf16(out), ref, fl, "C2 module")
 
 
+@pytest.mark.parametrize("multiply", [False, True])
+def test_c2_module_f8_result(oracle, multiply):
+    say("module C2 with an f8 result, multiply=%s" % multiply)
+    M, K, N = 8, 1024, 512
+    w = workloads.c2_s4_group(M, K, N)
+    text = hm.c2_s4_group_f8_result(M, K, N, multiply=multiply)
+    z = np.array(1 / 0.37 if multiply else 0.37, np.float32)
+    out, rw, _ = hlo_runner.compile_and_run(text, [dev_bf16(w["lhs"]), dev_u8(w["weights_packed"]),
+                                                   dev_bf16(w["scales"]), dev_bf16(w["bias"]), dev_f32(z)])
+    torch.cuda.synchronize()
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, f8 result]"]
+    ref = reference(text, [w["lhs"], w["weights"], w["scales"], w["bias"], z])
+    val = oracle.dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", bias=w["bias"], bias_ty="bf16",
+                             group=128, epilogue="silu", f32_result=True)
+    wd = np.abs(w["weights"].astype(np.float64)) * np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=0)
+    fl = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+    got = out.cpu().numpy().view(np.uint8)
+    assert list(got.shape) == [M, N]
+    assert check_f8_result(got, ref, val, z, not multiply, fl, "C2 f8 result") <= got.size // 8
+
+
 def test_c3_module():
     say("module C3")
     M, K, N = 128, 256, 128

@@ -658,6 +658,35 @@ def test_reference_int4_shape_table_is_taken(case, weights_on_lhs):
     assert sorted(set(opcodes(new)) - {"get-tuple-element"}) == ["broadcast", "constant", "custom-call", "parameter"]
 
 
+def test_dequant_dot_with_f8_result():
+    """The D scaling of gemm_rewriter_fp8_test.cc:1665-1690 / :1730-1748 behind a weight-only dot: the
+    scale is the call's last operand and the result is f8e4m3fn.  A value that also feeds its own amax
+    keeps its f32 result and leaves scaling, clamp, convert and the reduce to the ops after the call."""
+    for mul in (False, True):
+        new, rw, rf = hlo.rewrite(hm.c2_s4_group_f8_result(8, 256, 64, 64, multiply=mul))
+        assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, f8 result]"] and rf == [], (rw, rf)
+        check(new, r"f8e4m3fn\[8,64\]\{1,0\}(, s8\[\d+\]\{0\}\))? custom-call\(%lhs, %w, %scales, %bias, %d_scale\)",
+              r"d_scale_multiplies = %s" % ("true" if mul else "false"))
+        assert sorted(set(opcodes(new)) - {"get-tuple-element"}) == ["custom-call", "parameter"]
+    text = hm.c2_s4_group_f8_result(8, 256, 64, 64)
+    text = text.replace("ENTRY %main {", "%max_f32 {\n  %a = f32[] parameter(0)\n  %b = f32[] parameter(1)\n"
+                        "  ROOT %m = f32[] maximum(%a, %b)\n}\n\nENTRY %main {")
+    text = text.replace("  ROOT %out = f8e4m3fn[8,64] convert(%clamped)\n", """  %out = f8e4m3fn[8,64] convert(%clamped)
+  %abs_v = f32[8,64] abs(%silu)
+  %ninf = f32[] constant(-inf)
+  %amax = f32[] reduce(%abs_v, %ninf), dimensions={0,1}, to_apply=%max_f32
+  ROOT %result = (f8e4m3fn[8,64], f32[]) tuple(%out, %amax)
+""")
+    new, rw, rf = hlo.rewrite(text)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, f32 result]"], (rw, rf)
+    assert all("clamp/convert to f8e4m3fn found but not rewritten" in r for r in rf), rf   # the quantizer's matcher looked too
+    assert {"clamp", "reduce", "divide", "abs"} <= set(opcodes(new))
+    # a clamp to anything but +-448 is not the f8 saturation: the f32 value is the call's result
+    bad = hm.c2_s4_group_f8_result(8, 256, 64, 64).replace("constant(448)", "constant(240)")
+    new, rw, rf = hlo.rewrite(bad)
+    assert rw == ["dot -> xla_amd.dequant_dot [BIAS_SILU, s4, f32 result]"] and "clamp" in opcodes(new)
+
+
 def test_f32_result_with_scales_and_epilogue():
     """The value leaving the pattern may be f32: C2's module without its final convert keeps the f32
     SiLU value as the result (epilogue ops f32-typed, dequantise multiply bf16-typed)."""

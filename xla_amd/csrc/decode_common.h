@@ -68,14 +68,26 @@ struct DecodeParams {
   int out_f32;         // out holds f32, not bf16
   int out_transposed;  // out is [batch,N,M]: the dequantised weights were the lhs of the dot
   int lhs_k_major;     // lhs is [batch,K,M] (one-thread-per-output kernels only)
+  // out holds f8e4m3fn codes: convert(clamp(-448, v / *d_scale, 448)), or v * *d_scale with d_multiplies
+  int out_f8;
+  const float* d_scale;
+  int d_multiplies;
 };
 
 // One result element; row = batch * M + m over the flattened [batch * M, N] result.
 static __device__ __forceinline__ void StoreResult(const DecodeParams& p, size_t row, int n, float v) {
   size_t idx = row * (size_t)p.N + (size_t)n;
   if (p.out_transposed) idx = ((row / (size_t)p.M) * (size_t)p.N + (size_t)n) * (size_t)p.M + row % (size_t)p.M;
-  if (p.out_f32) reinterpret_cast<float*>(p.out)[idx] = v;
-  else p.out[idx] = f32_to_bf16(v);
+  if (p.out_f8) {
+    // op by op as the HLO does: an IEEE quotient (or product), clamp (a NaN stays one), cast
+    float c = p.d_multiplies ? v * *p.d_scale : v / *p.d_scale;
+    if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+    reinterpret_cast<uint8_t*>(p.out)[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
+  } else if (p.out_f32) {
+    reinterpret_cast<float*>(p.out)[idx] = v;
+  } else {
+    p.out[idx] = f32_to_bf16(v);
+  }
 }
 
 // Rows of a ragged dot that group g covers, read on the device: [*begin, *begin + *rows), clamped to

@@ -398,7 +398,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
 #pragma unroll
       for (int u = 0; u < RPW; ++u) dst[u] = res[pass * RPW + u];
     } else {
-      if (p.out_f32 | p.out_transposed) {
+      if (p.out_f32 | p.out_transposed | p.out_f8) {
 #pragma unroll
         for (int u = 0; u < RPW; ++u) StoreResult(p, (size_t)m_begin + m, n0 + u, res[pass * RPW + u]);
         continue;
@@ -655,6 +655,8 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     // a ragged dot over no groups: no row has a group, so every row is epilogue(0 [+ bias])
     if (!p.out || ((p.epilogue & 1) && !p.bias))
       return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: null buffer");
+    if (p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16)
+      return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot writes bf16 [M,N] from lhs [M,K]");
     DecodeParams fp = {};
     fp.out = (uint16_t*)p.out;
     fp.bias = (p.epilogue & 1) ? p.bias : nullptr;
@@ -693,15 +695,21 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.strips = 1; dp.slices = 1; dp.rows_per_slice = 0;
   dp.weights_shared = weights_shared;
   dp.handover_test = GetOption("handover_test");
-  if (p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16 && p.out_dtype != XLA_FFI_DataType_F32)
-    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: out must be BF16 or F32");
+  if (p.out_dtype != 0 && p.out_dtype != XLA_FFI_DataType_BF16 && p.out_dtype != XLA_FFI_DataType_F32 &&
+      p.out_dtype != XLA_FFI_DataType_F8E4M3FN)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: out must be BF16, F32 or F8E4M3FN");
   dp.out_f32 = p.out_dtype == XLA_FFI_DataType_F32;
+  dp.out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
+  dp.d_scale = p.d_scale;
+  dp.d_multiplies = p.d_scale_multiplies != 0;
+  if (dp.out_f8 && !p.d_scale)
+    return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: an F8E4M3FN result needs d_scale");
   dp.out_transposed = p.out_transposed != 0;
   dp.lhs_k_major = p.lhs_k_major != 0;
   // A result other than bf16 [batch,M,N], or activations stored [batch,K,M], keep the call on the
   // kernels that store through StoreResult / read lhs with a stride: the first-generation decode
   // kernel (and its token chunks), the [N,K] streaming kernel and the one-thread-per-output kernels.
-  const bool plain = !dp.out_f32 && !dp.out_transposed && !dp.lhs_k_major;
+  const bool plain = !dp.out_f32 && !dp.out_f8 && !dp.out_transposed && !dp.lhs_k_major;
   if (!plain && p.group_sizes)
     return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot writes bf16 [M,N] from lhs [M,K]");
   dp.w_unsigned = u4;
@@ -794,7 +802,7 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
         sub.batch = part == 0 ? whole : 1;
         if (sub.M == 0 || sub.batch == 0) continue;
         sub.lhs = (const uint16_t*)p.lhs + ((size_t)b * p.M + m0) * p.K;
-        sub.out = (char*)p.out + ((size_t)b * p.M + m0) * p.N * (dp.out_f32 ? 4 : 2);
+        sub.out = (char*)p.out + ((size_t)b * p.M + m0) * p.N * (dp.out_f32 ? 4 : dp.out_f8 ? 1 : 2);
         const int rc = LaunchDequantDotImpl(sub, stream, true);
         if (rc) return rc;
         if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)chunk);

@@ -354,7 +354,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
             for (int i = 0; i < 4; ++i)
               if (n + i < p.N) dst[i] = v[i];
           }
-        } else if (p.out_f32 | p.out_transposed) {
+        } else if (p.out_f32 | p.out_transposed | p.out_f8) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (n + i < p.N) StoreResult(p, (size_t)a_batch * p.M + m_first + m0 + m, n + i, v[i]);
@@ -530,7 +530,7 @@ int LaunchDequantDotNk(DecodeParams dp, const XlaAmdDequantDot& p, hipStream_t s
     if ((int64_t)1 << s == p.group) group_shift = s;
   const bool ragged = p.group_sizes != nullptr;
   // (a ragged dot takes the tiled kernel -- 256-row tiles per group -- once the groups average 96 rows)
-  const bool plain = !dp.out_f32 && !dp.out_transposed && !dp.lhs_k_major;  // else: no tiled kernel
+  const bool plain = !dp.out_f32 && !dp.out_f8 && !dp.out_transposed && !dp.lhs_k_major;  // else: no tiled kernel
   if (plain && p.M > 64 && (!ragged || GetOption("dequant_dot_kernel") == 3 || p.M / p.batch >= 96) &&
       GetOption("dequant_dot_kernel") != 1 && GetOption("dequant_dot_kernel") != 2) {
     const int rc = LaunchDequantDotPrefillNk(p, stream);

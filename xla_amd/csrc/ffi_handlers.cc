@@ -356,11 +356,21 @@ extern "C" {
 
 XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Error* err;
-  if (Preamble(f, 3, 6, 1, 2, &err)) return err;
+  if (Preamble(f, 3, 7, 1, 2, &err)) return err;
   Decoder d{f};
   // a ragged dot brings its group sizes (S32 or S64 [groups]) as the last operand
   int64_t nargs = f->args.size;
   XLA_FFI_Buffer* gs = nullptr;
+  // an F8E4M3FN result brings its scale (one F32) as the last operand
+  const bool out_f8 = f->rets.types[0] == XLA_FFI_RetType_BUFFER &&
+                      static_cast<XLA_FFI_Buffer*>(f->rets.rets[0])->dtype == XLA_FFI_DataType_F8E4M3FN;
+  XLA_FFI_Buffer* sd = nullptr;
+  if (out_f8) {
+    if (nargs < 4)
+      return InvalidArgument(f->api, "xla_amd.dequant_dot: an F8E4M3FN result takes d_scale as the last operand");
+    sd = d.Arg((int)nargs - 1, Bit(XLA_FFI_DataType_F32), 0, 0, "d_scale");
+    --nargs;
+  }
   if (nargs > 3 && f->args.types[nargs - 1] == XLA_FFI_ArgType_BUFFER) {
     XLA_FFI_Buffer* last = static_cast<XLA_FFI_Buffer*>(f->args.args[nargs - 1]);
     if (last->dtype == XLA_FFI_DataType_S32 || last->dtype == XLA_FFI_DataType_S64) {
@@ -381,10 +391,13 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   XLA_FFI_Buffer* bias = nargs > bias_at ? d.Arg(bias_at, kFloatMask, 1, 1, "bias") : nullptr;
   if (((!has_zp && nargs > 4) || nargs > 5) && d.ok())
     return InvalidArgument(f->api, "xla_amd.dequant_dot: five operands are lhs, weights, scales, zero_points (U4), bias");
-  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F32), 2, 3, "out");
+  XLA_FFI_Buffer* out = d.Ret(0, Bit(XLA_FFI_DataType_BF16) | Bit(XLA_FFI_DataType_F32) | Bit(XLA_FFI_DataType_F8E4M3FN),
+                              2, 3, "out");
   XLA_FFI_Buffer* ws = f->rets.size > 1 ? d.Ret(1, kBytesMask, 1, 1, "scratch") : nullptr;
   CommonAttrs a;
   DecodeCommonAttrs(d, &a);
+  bool d_mul = false;
+  d.Scalar("d_scale_multiplies", XLA_FFI_DataType_PRED, &d_mul, 1);
   int64_t group_size = 0;
   const bool has_group_size = d.Int("scale_group_size", &group_size);
   int64_t rcd = 0;  // 1: weights [..,N,K], scales [N] | [B,N] | [N,K/g] | [B,N,K/g]
@@ -487,6 +500,8 @@ XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* f) {
   p.dequant_type = a.dequant_type; p.dot_type = a.dot_type; p.epilogue_type = a.epilogue_type;
   p.epilogue = a.epilogue;
   p.out_dtype = out->dtype;
+  p.d_scale = sd ? (const float*)sd->data : nullptr;
+  p.d_scale_multiplies = d_mul;
   p.out_transposed = transposed ? 1 : 0;
   p.lhs_k_major = lhs_k_major ? 1 : 0;
   void* stream;

@@ -175,9 +175,10 @@ bool MatchSilu(Instr* out, Instr* x) {
 // dimension, optional activation, optional final convert to bf16.  Returns false when what
 // leaves the chain is not bf16.
 // allow_f32_result: the kernels behind the call can write the f32 value itself (the dequantize-dot);
-// otherwise the value leaving the pattern must be bf16.
+// otherwise the value leaving the pattern must be bf16.  allow_amax: the handler can also return the
+// amax of an f8 result; without it a value that feeds its own amax is left to the ops after the call.
 bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_result_in = nullptr,
-                   bool allow_f32_result = false) {
+                   bool allow_f32_result = false, bool allow_amax = true) {
   const bool allow_f8_result = f8_result_in != nullptr;
   Instr* cur = dot;
   const int64_t rank = dot->shape.rank();
@@ -263,7 +264,7 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, const Module* f8_
     // maximum (gemm_rewriter_fp8_test.cc:2559-2600)
     Instr* sc = SoleUser(cur);
     Instr* amax = nullptr;
-    if (!sc && cur->users.size() == 2) {
+    if (!sc && allow_amax && cur->users.size() == 2) {
       for (int which = 0; which < 2 && !amax; ++which) {
         Instr* ab = cur->users[which];
         Instr* rd = ab->Is("abs") ? SoleUser(ab) : nullptr;
@@ -627,7 +628,7 @@ bool MatchQWeights(Instr* op, bool k_minor, QWeights* out, std::string* why) {
   return true;
 }
 
-bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
+bool RewriteDequantDot(const Module& mod, Computation* comp, Instr* dot, const RewriteOptions& opt, RewriteLog* log) {
   QWeights q;
   std::string why;
   const int64_t rank = dot->shape.rank();
@@ -676,7 +677,8 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
     return refuse("zero points must have the shape of the scales (one per scale)");
   if (q.scale && q.type == "bf16" && q.scale->shape.dtype != "bf16") return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
-  if (!MatchEpilogue(dot, &ep, &why, nullptr, /*allow_f32_result=*/true)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, /*f8_result_in=*/&mod, /*allow_f32_result=*/true, /*allow_amax=*/false))
+    return refuse(why);
   if (weights_lhs && (ep.bias || !ep.act.empty()))
     return refuse("with the weights as the lhs of the dot only the plain dot is taken (a bias would run along the other dimension)");
 
@@ -697,6 +699,7 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
+  if (ep.d_scale) ops.push_back(ep.d_scale);  // an f8e4m3fn result: its scale goes last
   std::vector<Shape> results = {Shape::Array(ep.tail->shape.dtype, dot->shape.dims)};
   const int32_t wdt = q.w->shape.dtype == "s4" ? 21 : q.w->shape.dtype == "u4" ? 22 : 2;
   auto sizer = k_minor ? opt.dequant_nk_workspace_bytes : opt.dequant_workspace_bytes;
@@ -710,13 +713,15 @@ bool RewriteDequantDot(Computation* comp, Instr* dot, const RewriteOptions& opt,
                              std::to_string(group_size) + " : i64" +
                              (k_minor ? ", rhs_contracting_dim = 1 : i64" : "") +
                              (lhs_k_major ? ", lhs_contracting_dim = 0 : i64" : "") +
-                             (weights_lhs ? ", result_transposed = true" : ""));
+                             (weights_lhs ? ", result_transposed = true" : "") +
+                             (ep.d_scale ? std::string(", d_scale_multiplies = ") + (ep.d_multiplies ? "true" : "false")
+                                         : std::string()));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
   comp->ReplaceAllUses(ep.tail, value);
   log->rewrites.push_back(dot->name + " -> xla_amd.dequant_dot [" + ep.Name() + ", " + q.w->shape.dtype +
                           (q.zero ? " with zero points" : "") + (k_minor ? ", weights [N,K]" : "") +
                           (weights_lhs ? ", weights as lhs" : "") + (lhs_k_major ? ", activations [K,M]" : "") +
-                          (ep.tail->shape.dtype == "f32" ? ", f32 result" : "") + "]");
+                          (ep.tail->shape.dtype == "f32" ? ", f32 result" : "") + (ep.d_scale ? ", f8 result" : "") + "]");
   return true;
 }
 
@@ -901,7 +906,7 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         Instr* i = up.get();
         bool did = false;
         if (i->Is("dot") && i->operands.size() == 2) {
-          did = RewriteF8Dot(*mod, comp.get(), i, opt, log) || RewriteDequantDot(comp.get(), i, opt, log);
+          did = RewriteF8Dot(*mod, comp.get(), i, opt, log) || RewriteDequantDot(*mod, comp.get(), i, opt, log);
         } else if (i->Is("ragged-dot") && i->operands.size() == 3) {
           did = RewriteRaggedDequantDot(comp.get(), i, log);
         } else if (i->Is("custom-call")) {

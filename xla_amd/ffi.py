@@ -247,7 +247,7 @@ class LaunchDequantDot(C.Structure):
                 ("dot_type", C.c_int32), ("epilogue_type", C.c_int32), ("epilogue", C.c_int32),
                 ("zero_points", C.c_void_p), ("group_sizes", C.c_void_p), ("group_sizes_dtype", C.c_int32),
                 ("rhs_contracting_dim", C.c_int32), ("out_dtype", C.c_int32), ("out_transposed", C.c_int32),
-                ("lhs_k_major", C.c_int32)]
+                ("lhs_k_major", C.c_int32), ("d_scale", C.c_void_p), ("d_scale_multiplies", C.c_int32)]
 
 
 _lib = None

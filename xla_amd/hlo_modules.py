@@ -71,6 +71,26 @@ ENTRY %main {{
 """
 
 
+def c2_s4_group_f8_result(M=8, K=8192, N=28672, group=128, multiply=False):
+    """c2_s4_group whose SiLU value leaves as f8e4m3fn: divided (or multiplied) by a per-tensor scale,
+    clamped to +-448 and converted -- the D scaling of gemm_rewriter_fp8_test.cc:1665-1690 / :1730-1748
+    behind a weight-only dot, i.e. the activations of the next fp8 dot made in this dot's store."""
+    text = c2_s4_group(M, K, N, group)
+    head, _ = text.split(f"  ROOT %out = bf16[{M},{N}] convert(%silu)")
+    op = "multiply" if multiply else "divide"
+    return head + f"""  %d_scale = f32[] parameter(4)
+  %d_scale_b = f32[{M},{N}] broadcast(%d_scale), dimensions={{}}
+  %scaled = f32[{M},{N}] {op}(%silu, %d_scale_b)
+  %lo = f32[] constant(-448)
+  %lo_b = f32[{M},{N}] broadcast(%lo), dimensions={{}}
+  %hi = f32[] constant(448)
+  %hi_b = f32[{M},{N}] broadcast(%hi), dimensions={{}}
+  %clamped = f32[{M},{N}] clamp(%lo_b, %scaled, %hi_b)
+  ROOT %out = f8e4m3fn[{M},{N}] convert(%clamped)
+}}
+"""
+
+
 def u4_zero_point_group(M=8, K=4096, N=4096, group=128, typed="bf16"):
     """bf16 [M,K] . ((convert(u4 [K,N]) - convert(u4 zero[K/g,N])) * scale[K/g,N]) + bias -> bf16: the
     asymmetric 4-bit weight-only form (one zero point and one scale per group and channel).

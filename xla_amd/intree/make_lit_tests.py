@@ -23,6 +23,7 @@ def cases():
     return [
         ("quant_fusion_rewriter_s8_per_channel", hm.c1_s8_channel(16, 256, 128)),
         ("quant_fusion_rewriter_s4_grouped_silu", hm.c2_s4_group(8, 256, 64, 64)),
+        ("quant_fusion_rewriter_s4_grouped_silu_f8_result", hm.c2_s4_group_f8_result(8, 256, 64, 64)),
         ("quant_fusion_rewriter_u4_zero_points", hm.u4_zero_point_group(8, 256, 64, 64)),
         ("quant_fusion_rewriter_s8_batched", hm.c5_s8_batched(2, 8, 32, 16)),
         ("quant_fusion_rewriter_s8_ragged_experts", hm.ragged_s8_experts(16, 256, 64, 4)),

@@ -159,7 +159,8 @@ bool MatchSilu(Instr* out, Instr* x) {
 // f8 result tail convert(clamp(-448, v / z | v * z, 448)) with its optional amax.
 // allow_f32_result: the kernels behind the call can write the f32 value itself (the dequantize-dot);
 // otherwise the value leaving the pattern must be bf16.
-bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result, bool allow_f32_result = false) {
+bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_result, bool allow_f32_result = false,
+                   bool allow_amax = true) {
   Instr* cur = dot;
   const int64_t rank = Rank(dot);
   ep->ops_type = Ty(dot);
@@ -234,7 +235,7 @@ bool MatchEpilogue(Instr* dot, Epilogue* ep, std::string* why, bool allow_f8_res
   if (allow_f8_result && Ty(cur) == F32 && Ty(dot) == F32 && ep->ops_type == F32) {
     Instr* sc = SoleUser(cur);
     Instr* amax = nullptr;
-    if (!sc && cur->user_count() == 2) {
+    if (!sc && allow_amax && cur->user_count() == 2) {
       for (int which = 0; which < 2 && !amax; ++which) {
         Instr* ab = cur->users()[which];
         Instr* rd = ab->opcode() == HloOpcode::kAbs ? SoleUser(ab) : nullptr;
@@ -622,7 +623,8 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
     return refuse("zero points must have the shape of the scales (one per scale)");
   if (q.scale && q.type == BF16 && Ty(q.scale) != BF16) return refuse("bf16 multiply with non-bf16 scales");
   Epilogue ep;
-  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/false, /*allow_f32_result=*/true)) return refuse(why);
+  if (!MatchEpilogue(dot, &ep, &why, /*allow_f8_result=*/true, /*allow_f32_result=*/true, /*allow_amax=*/false))
+    return refuse(why);
   if (weights_lhs && (ep.bias || !ep.act.empty()))
     return refuse("with the weights as the lhs of the dot only the plain dot is taken (a bias would run along the other dimension)");
 
@@ -640,6 +642,7 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
   std::vector<Instr*> ops = {lhs, q.w, q.scale};
   if (q.zero) ops.push_back(q.zero);
   if (ep.bias) ops.push_back(ep.bias);
+  if (ep.d_scale) ops.push_back(ep.d_scale);  // an f8e4m3fn result: its scale goes last
   std::vector<Shape> results = {ShapeUtil::MakeShape(Ty(ep.tail), Dims(dot))};
   if (size_t ws = k_minor ? xla_amd_dequant_dot_workspace_bytes_nk(B, M, K, N, (int32_t)Ty(q.w))
                           : xla_amd_dequant_dot_workspace_bytes(B, M, K, N, (int32_t)Ty(q.w)))
@@ -651,13 +654,15 @@ bool RewriteDequantDot(HloComputation* comp, Instr* dot, const std::function<voi
                          CommonConfig(ep, dequant_ty, Ty(dot)) + absl::StrCat(", scale_group_size = ", group_size, " : i64") +
                              (k_minor ? ", rhs_contracting_dim = 1 : i64" : "") +
                              (lhs_k_major ? ", lhs_contracting_dim = 0 : i64" : "") +
-                             (weights_lhs ? ", result_transposed = true" : ""));
+                             (weights_lhs ? ", result_transposed = true" : "") +
+                             (ep.d_scale ? absl::StrCat(", d_scale_multiplies = ", ep.d_multiplies ? "true" : "false")
+                                         : std::string()));
   Instr* value = results.size() > 1 ? EmitGte(comp, call, 0) : call;
   CHECK_OK(ep.tail->ReplaceAllUsesWith(value));
   VLOG(1) << dot->name() << " -> xla_amd.dequant_dot [" << ep.Name() << ", " << TyName(Ty(q.w))
           << (q.zero ? " with zero points" : "") << (k_minor ? ", weights [N,K]" : "")
           << (weights_lhs ? ", weights as lhs" : "") << (lhs_k_major ? ", activations [K,M]" : "")
-          << (Ty(ep.tail) == F32 ? ", f32 result" : "") << "]";
+          << (Ty(ep.tail) == F32 ? ", f32 result" : "") << (ep.d_scale ? ", f8 result" : "") << "]";
   return true;
 }
 

@@ -58,7 +58,8 @@ def _scratch(nbytes, device):
 def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_shape=None,
                 epilogue="DEFAULT", dequant_type="f32", dot_type="f32", epilogue_type="f32",
                 scale_group_size=None, zero_points=None, group_sizes=None, rhs_contracting_dim=0, out=None,
-                scratch="auto", build_only=False, out_dtype="bf16", result_transposed=False, lhs_contracting_dim=1):
+                scratch="auto", build_only=False, out_dtype="bf16", result_transposed=False, lhs_contracting_dim=1,
+                d_scale=None, d_scale_multiplies=False):
     """out = epilogue(lhs . (convert(weights) * scales)).  lhs bf16 [M,K] or [B,M,K].
     scale_group_size: rows of K per scale (0 = per output channel); None leaves the attribute out and
     the handler reads the grouping off the scales' shape.
@@ -70,15 +71,17 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
     [N,K/g] or [B,N,K/g]; scale_group_size is then required.
     out_dtype "f32": the dot's f32 value is the result.  result_transposed: the result is [..,N,M] (the
     dequantised weights were the lhs of the dot; DEFAULT epilogue only).  lhs_contracting_dim=0: lhs is
-    stored [..,K,M]."""
-    _check_cuda(lhs, weights, scales, bias, zero_points, group_sizes)
+    stored [..,K,M].  With d_scale (f32 []) the result is f8e4m3fn codes (uint8):
+    convert(clamp(out / d_scale)), or out * d_scale with d_scale_multiplies."""
+    _check_cuda(lhs, weights, scales, bias, zero_points, group_sizes, d_scale)
     wdt = {"s4": dtypes.S4, "u4": dtypes.U4}.get(weight_dtype, dtypes.S8)
     wshape = list(weight_shape) if weight_shape is not None else list(weights.shape)
     n = wshape[-2] if rhs_contracting_dim == 1 else wshape[-1]
     m, k = (lhs.shape[-1], lhs.shape[-2]) if lhs_contracting_dim == 0 else (lhs.shape[-2], lhs.shape[-1])
     oshape = list(lhs.shape[:-2]) + ([n, m] if result_transposed else [m, n])
     if out is None:
-        out = torch.empty(oshape, dtype=torch.float32 if out_dtype == "f32" else torch.bfloat16, device=lhs.device)
+        odt = torch.uint8 if d_scale is not None else torch.float32 if out_dtype == "f32" else torch.bfloat16
+        out = torch.empty(oshape, dtype=odt, device=lhs.device)
     batch = lhs.shape[0] if lhs.dim() == 3 else (wshape[0] if group_sizes is not None else 1)
     args = [(dtypes.BF16, lhs.data_ptr(), lhs.shape), (wdt, weights.data_ptr(), wshape),
             (_FLOAT[scales.dtype], scales.data_ptr(), scales.shape)]
@@ -86,10 +89,13 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
         args.append((dtypes.U4, zero_points.data_ptr(), scales.shape))
     if bias is not None:
         args.append((_FLOAT[bias.dtype], bias.data_ptr(), bias.shape))
+    if d_scale is not None:
+        args.append((dtypes.F32, d_scale.data_ptr(), []))
     if group_sizes is not None:
         args.append((dtypes.S64 if group_sizes.dtype == torch.int64 else dtypes.S32, group_sizes.data_ptr(),
                      group_sizes.shape))
-    rets = [(dtypes.F32 if out.dtype == torch.float32 else dtypes.BF16, out.data_ptr(), oshape)]
+    rets = [(dtypes.F8E4M3FN if d_scale is not None else dtypes.F32 if out.dtype == torch.float32 else dtypes.BF16,
+             out.data_ptr(), oshape)]
     if scratch == "auto":
         sizer = (ffi.library().xla_amd_dequant_dot_workspace_bytes_nk if rhs_contracting_dim == 1
                  else ffi.library().xla_amd_dequant_dot_workspace_bytes)
@@ -108,8 +114,10 @@ def dequant_dot(lhs, weights, scales, bias=None, *, weight_dtype="s8", weight_sh
         attrs["lhs_contracting_dim"] = ffi.Attr.i64(lhs_contracting_dim)
     if result_transposed:
         attrs["result_transposed"] = ffi.Attr.pred(True)
+    if d_scale_multiplies:
+        attrs["d_scale_multiplies"] = ffi.Attr.pred(True)
     call = Call("xla_amd.dequant_dot", ffi.Frame(host(), args, rets, attrs), out,
-                keep=(lhs, weights, scales, bias, scratch, zero_points, group_sizes))
+                keep=(lhs, weights, scales, bias, scratch, zero_points, group_sizes, d_scale))
     return call if build_only else call.run()
 
 
