@@ -1,0 +1,213 @@
+"""The weight-streaming kernels of xla_amd.fp8_scaled_dot (up to 64 rows of a; rhs [K,N] or [N,K]) against
+the CPU oracle, through the FFI handler: every token-tile count, ragged K and N, K-slices with and without
+scratch, vector scales, f8 results with amax, batches, one-hot exactness and special values."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_dot, check_f8_result, dev_bf16, dev_f32, dev_u8, host_bf16
+from tests.test_gpu_fp8_dot import EPI, floor_for, reference, say
+from xla_amd import dtypes, ffi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def run(w, nk=False, slices=0, scratch="auto", force=3, batch=None, **kw):
+    """force=3: the streaming kernels or an error; slices: K-slices (0: the launcher's choice)."""
+    b = w["b"]
+    if nk:
+        b = np.ascontiguousarray(np.swapaxes(b, -1, -2))
+    a, b = dev_u8(w["a"]), dev_u8(b)
+    sa = dev_f32(np.array(w["a_scale"], np.float32))
+    sb = dev_f32(np.array(w["b_scale"], np.float32))
+    bias = dev_bf16(w["bias"]) if w.get("bias") is not None else None
+    ffi.set_option("fp8_dot_kernel", force)
+    ffi.set_option("fp8_decode_slices", slices)
+    try:
+        if scratch == "auto" and slices:   # the sizer is asked under the same option
+            n = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(w["a"].shape[-2], w["a"].shape[-1], w["b"].shape[-1], 1 if nk else 0)
+            scratch = torch.empty(max(n * (batch or 1), 16), dtype=torch.uint8, device="cuda")
+        out = ops.fp8_scaled_dot(a, b, sa, sb, bias, rhs_contracting_dim=1 if nk else 0, epilogue=w["epilogue"],
+                                 scratch=scratch, **kw)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+        ffi.set_option("fp8_decode_slices", 0)
+    return out, ffi.last_kernel()
+
+
+def tile_name(nk, M):
+    return "fp8_dot_decode_%s_m%d" % ("nk" if nk else "kn", 16 * ((M + 15) // 16))
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 48, 64])
+@pytest.mark.parametrize("K,N", [(1024, 256), (528, 136), (4096, 72)])
+def test_every_tile_count_ragged_k_and_n(oracle, M, K, N, nk):
+    """528 is no multiple of a step (32 rows, or 128 of the [N,K] kernel), 136 and 72 none of a strip."""
+    if nk and M > 32:
+        pytest.skip("the [N,K] streaming kernel takes up to 32 rows of a")
+    say("fp8 streaming M=%d K=%d N=%d nk=%s" % (M, K, N, nk))
+    w = workloads.c3_fp8(M, K, N)
+    out, kern = run(w, nk=nk)
+    assert kern == tile_name(nk, M), kern
+    n_floor = check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    assert n_floor <= max(4, out.numel() // 50)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("slices", [2, 4, 8])
+def test_k_slices(oracle, slices, nk):
+    """K split over workgroups: sums through the scratch and the second kernel; without the scratch one
+    slice.  The last slices of K = 2176 are short or empty."""
+    say("fp8 streaming, %d K-slices, nk=%s" % (slices, nk))
+    w = workloads.c3_fp8(24, 2176, 264)
+    ref = reference(oracle, w)
+    out, kern = run(w, nk=nk, slices=slices)
+    assert kern == tile_name(nk, 24)
+    check_dot(host_bf16(out), ref, floor_for(w), "%s, %d slices" % (kern, slices))
+    out1, _ = run(w, nk=nk, slices=slices, scratch=None)
+    check_dot(host_bf16(out1), ref, floor_for(w), "%s, no scratch" % kern)
+    # two runs give the same bits: the slices are added in slice order
+    out2, _ = run(w, nk=nk, slices=slices)
+    assert torch.equal(out, out2)
+
+
+def test_the_launcher_splits_k_for_narrow_results(oracle):
+    say("fp8 streaming, the launcher's own slices")
+    M, K, N = 16, 4096, 512
+    assert ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(M, K, N, 0) >= 2 * M * N * 4
+    w = workloads.c3_fp8(M, K, N)
+    out, kern = run(w, force=0)
+    assert kern == tile_name(False, M)
+    check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("which", ["a", "b", "ab"])
+@pytest.mark.parametrize("slices", [0, 2])
+def test_vector_scales(oracle, which, nk, slices):
+    say("fp8 streaming, vector scales %s, nk=%s, slices=%d" % (which, nk, slices))
+    M, K, N = 20, 1024, 200
+    w = workloads.c3_fp8(M, K, N)
+    rng = np.random.default_rng(5)
+    if "a" in which:
+        w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+    if "b" in which:
+        w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    out, kern = run(w, nk=nk, slices=slices)
+    assert kern == tile_name(nk, M)
+    check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+
+
+@pytest.mark.parametrize("epilogue,dot_ty,ep_ty", [("DEFAULT", "f32", "f32"), ("BIAS", "f32", "f32"), ("RELU", "f32", "f32"),
+                                                  ("BIAS_SILU", "f32", "f32"), ("GELU", "f32", "bf16"), ("BIAS_RELU", "bf16", "bf16")])
+def test_epilogues_and_rounding_points(oracle, epilogue, dot_ty, ep_ty):
+    say("fp8 streaming, %s dot %s ops %s" % (epilogue, dot_ty, ep_ty))
+    w = dict(workloads.c3_fp8(40, 512, 128), epilogue=epilogue)
+    if "BIAS" not in epilogue:
+        w["bias"] = None
+    types = dict(dot_type=dot_ty, epilogue_type=ep_ty)
+    out, kern = run(w, **types)
+    ref = reference(oracle, w, **types)
+    fl = floor_for(w)
+    if "bf16" in (dot_ty, ep_ty):   # a difference far below one ulp can flip a bf16 rounding on the way
+        fl = fl * 12 + np.abs(dtypes.bf16_to_f32(ref)) * 6 * 2.0 ** -8
+    check_dot(host_bf16(out), ref, fl, kern)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("divides", [True, False])
+@pytest.mark.parametrize("slices", [0, 4])
+def test_f8_result_with_amax(oracle, divides, nk, slices):
+    say("fp8 streaming, f8 result, divides=%s nk=%s slices=%d" % (divides, nk, slices))
+    M, K, N = 32, 1024, 136
+    w = workloads.c3_fp8(M, K, N)
+    s = np.float32(1 / 64)
+    w["a_scale"] = w["b_scale"] = s
+    z = np.float32(0.0171 if divides else 1 / 0.0171)
+    (out, amax), kern = run(w, nk=nk, slices=slices, d_scale=dev_f32(np.array(z, np.float32)), d_scale_multiplies=not divides,
+                            amax=True)
+    assert kern == tile_name(nk, M)
+    ref, val = oracle.fp8_scaled_dot(w["a"], w["b"], s, s, bias=w["bias"], epilogue=EPI[w["epilogue"]], d_scale=z,
+                                     d_scale_divides=divides)
+    check_f8_result(out.cpu().numpy(), ref, val, z, divides, floor_for(w), kern)
+    want = float(np.max(np.abs(val)))
+    got = float(amax.cpu())
+    assert abs(got - want) <= 2.0 ** -7 * want + float(np.max(floor_for(w))), (got, want)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+def test_batched(oracle, nk):
+    say("fp8 streaming, batched, nk=%s" % nk)
+    B, M, K, N = 3, 12, 640, 264
+    ws = [workloads.c3_fp8(M, K, N) for _ in range(B)]
+    for i, x in enumerate(ws):   # different data per batch
+        x["a"] = np.roll(x["a"], 3 * i, axis=0)
+        x["b"] = np.roll(x["b"], 5 * i, axis=1)
+    w = dict(ws[0], a=np.stack([x["a"] for x in ws]), b=np.stack([x["b"] for x in ws]))
+    for slices in (0, 2):
+        out, kern = run(w, nk=nk, slices=slices, batch=B)
+        assert kern == tile_name(nk, M)
+        got = host_bf16(out)
+        for i in range(B):
+            check_dot(got[i], reference(oracle, ws[i]), floor_for(ws[i]), "%s batch %d" % (kern, i))
+
+
+@pytest.mark.parametrize("nk", [False, True])
+def test_one_hot_rows_read_single_values_back_exactly(oracle, nk):
+    """a = selector rows of 1.0: every output is one rhs value times the scales, exactly -- every f8 code
+    at every position of a 128-value step, so a transposed byte or a permuted k shows as a wrong value."""
+    say("fp8 streaming, one-hot, nk=%s" % nk)
+    M, K, N = 32, 384, 256
+    ks = (np.arange(M) * 37 + 5) % K
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), ks] = 1.0
+    b8 = ((np.arange(K)[:, None] * 7 + np.arange(N)[None, :]) % 256).astype(np.uint8)
+    b8[(b8 & 0x7F) == 0x7F] = 0x3A
+    w = dict(a=dtypes.f32_to_f8e4m3fn(a), b=b8, a_scale=np.float32(0.5), b_scale=np.float32(0.25), bias=None,
+             epilogue="DEFAULT")
+    want = dtypes.f32_to_bf16(dtypes.f8e4m3fn_to_f32(b8[ks]) * np.float32(0.125))
+    for slices in (0, 2):
+        out, kern = run(w, nk=nk, slices=slices)
+        assert kern == tile_name(nk, M)
+        assert np.array_equal(dtypes.bf16_to_f32(host_bf16(out)), dtypes.bf16_to_f32(want)), (kern, slices)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+def test_nan_codes_and_the_end_of_k(oracle, nk):
+    """A NaN code makes its row or channel NaN and nothing else.  K = 144 ends inside a step, and what
+    lies behind a row's end in memory (the start of the next row of a, or of the next channel of an
+    [N,K] rhs) must not leak in even when it holds NaN codes."""
+    say("fp8 streaming, NaN codes, nk=%s" % nk)
+    M, K, N = 5, 144, 64
+    w = dict(workloads.c3_fp8(M, K, N), epilogue="DEFAULT", bias=None)
+    a8, b8 = w["a"].copy(), w["b"].copy()
+    a8[1, :16] = 0x7F         # right behind row 0's end: row 1 is NaN, row 0 stays finite
+    a8[3, 17] = 0xFF
+    b8[:16, 1] = 0x7F         # right behind channel 0's end in an [N,K] rhs
+    b8[100, 9] = 0x7F
+    w["a"], w["b"] = a8, b8
+    out, kern = run(w, nk=nk)
+    got = dtypes.bf16_to_f32(host_bf16(out))
+    ref = dtypes.bf16_to_f32(reference(oracle, w))
+    assert np.array_equal(np.isnan(got), np.isnan(ref)), kern
+    finite = np.ones((M, N), bool)
+    finite[[1, 3], :] = False
+    finite[:, [1, 9]] = False
+    assert np.array_equal(~np.isnan(got), finite), kern
+    assert np.allclose(got[finite], ref[finite], rtol=2.0 ** -7, atol=float(np.max(floor_for(w)[finite]))), kern
+
+
+def test_what_the_streaming_kernels_do_not_take():
+    a = torch.zeros((80, 64), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((64, 64), dtype=torch.uint8, device="cuda")
+    one = torch.ones((), dtype=torch.float32, device="cuda")
+    ffi.set_option("fp8_dot_kernel", 3)
+    try:
+        with pytest.raises(ffi.FfiError, match="streaming kernels take up to 64 rows"):
+            ops.fp8_scaled_dot(a, b, one, one)
+        with pytest.raises(ffi.FfiError, match="streaming kernels take"):
+            ops.fp8_scaled_dot(a[:8], b, one, one, dequant_type="bf16")
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)

@@ -16,7 +16,7 @@ CSRC = os.path.join(ROOT, "xla_amd", "csrc")
 LIB = os.path.join(ROOT, "xla_amd", "lib")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-KERNEL_SOURCES = ["capi.hip", "rowwise_quantize.hip", "dequant_dot_decode.hip", "dequant_dot_decode_s4x.hip", "dequant_dot_decode_s8x.hip", "dequant_dot_nk.hip", "tiled_dot_mfma.hip",
+KERNEL_SOURCES = ["capi.hip", "rowwise_quantize.hip", "dequant_dot_decode.hip", "dequant_dot_decode_s4x.hip", "dequant_dot_decode_s8x.hip", "dequant_dot_nk.hip", "tiled_dot_mfma.hip", "fp8_dot_decode.hip",
                   "ffi_handlers.cc"]
 SELFCHECK_SOURCES = ["self_check.hip"]
 HOST_SOURCES = ["host/ffi_host.cc", "host/hlo_ir.cc", "host/quant_fusion_rewriter.cc",

@@ -1,0 +1,458 @@
+// Weight-streaming f8e4m3fn scaled dot for decode shapes (M <= 64):
+//   out[b,m,n] = epilogue( a_scale[m] * b_scale[n] * sum_k A8[b,m,k] * B8[b,k,n] )
+// -- the small-M end of the f8 matmul that GemmRewriter hands to the library
+// (xla/backends/gpu/transforms/gemm_rewriter.cc:1178-1540; the dequantising multiplies by the
+// scales are f32-typed, so factoring them out of the sum moves no rounding: every product of
+// two f8e4m3fn numbers is exact in f32).
+//
+// At these sizes the rhs is the only large operand and the kernel is a stream over it, built
+// like the integer-weight decode kernels next to it but with nothing to dequantise:
+//  * rhs [K,N] (N minor): a lane pulls 8 bytes (8 channels) of 8 consecutive rows into
+//    registers, so 16 lanes take one whole 128-byte line per row.  Four 4x4 byte transposes
+//    (v_perm_b32) turn the 8 x 8 block into 8 operands of 8 consecutive k for
+//    v_mfma_f32_16x16x32_fp8_fp8, whose 16 rows are 16 *output channels*; the activations are
+//    the other operand (8 bytes per lane straight from memory), so an instruction yields a
+//    [16 channels x 16 tokens] tile.
+//  * rhs [N,K] (K minor): a load instruction takes whole 128-byte lines of 8 channels (8 lanes per
+//    line, 16 bytes each); ds_bpermute_b32 then deals the pieces to the lanes that stand for
+//    their channel in the matrix operand (lane (channel, kb) gets bytes 32 kb .. 32 kb + 31 of
+//    the channel's line).  Which k a slot of the matrix instruction stands for is free as long
+//    as both operands agree, so the activations are read 32 contiguous bytes per lane and
+//    nothing is transposed.
+// The waves of a workgroup split its rows of K and add their tiles through LDS in wave order;
+// K may also be split over workgroups, whose f32 sums go through the workspace and a second
+// small kernel, in slice order: results do not depend on scheduling.
+//
+// Bound: HBM.  Algorithmic bytes: K*N (rhs) + a, scales, bias and out once each.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "decode_common.h"
+#include "device_numerics.h"
+#include "launch.h"
+
+namespace xla_amd {
+namespace {
+
+struct Fp8DecodeParams {
+  const uint8_t* a;      // [batch, M, K]
+  const uint8_t* b;      // [batch, K, N], or [batch, N, K]
+  const float* a_scale;  // one value, or M (a_per_row)
+  const float* b_scale;  // one value, or N (b_per_channel)
+  const void* bias;      // [N] or null
+  uint16_t* out;         // [batch, M, N] bf16, or
+  uint8_t* out8;         // f8e4m3fn codes: convert(clamp(v / *d_scale)) (v * *d_scale unless d_divides)
+  const float* d_scale;
+  float* amax;           // optional: max |v| over an f8 result, folded in with atomics
+  float* partial;        // slices > 1: [batch, slices, M, N] f32 sums
+  int M, K, N;
+  int a_per_row, b_per_channel, bias_is_bf16, d_divides;
+  int bf16_dot, bf16_ops, epilogue;
+  int slices, rows_per_slice, rows_per_wave;  // rows_per_wave: a multiple of the kernel's step
+};
+
+constexpr int kWaves = 8;
+constexpr uint32_t kNowhere = 0x80000000u;  // a lane offset no buffer reaches: the load returns zeros
+
+// One result value: the scales, the epilogue, and the store (bf16, or an f8 code with its amax).
+__device__ __forceinline__ void finish_value(const Fp8DecodeParams& p, int batch, int m, int n, float sum, float alpha,
+                                             uint32_t* amax_bits) {
+  float v = sum;
+  if (p.a_per_row) v = v * p.a_scale[m];
+  v = v * (p.b_per_channel ? alpha * p.b_scale[n] : alpha);
+  const float bias = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
+  v = epilogue_dispatch(v, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
+  const size_t idx = ((size_t)batch * p.M + m) * p.N + n;
+  if (p.out8) {
+    *amax_bits = max(*amax_bits, f32_to_bits(v) & 0x7fffffffu);  // a NaN pattern exceeds every number
+    // op by op as the HLO does: an IEEE quotient (or product), clamp (a NaN stays one), cast
+    float c = p.d_divides ? v / *p.d_scale : v * *p.d_scale;
+    if (c == c) c = __builtin_fminf(__builtin_fmaxf(c, -448.0f), 448.0f);
+    p.out8[idx] = (uint8_t)f32_to_f8e4m3fn_any(c);
+  } else {
+    p.out[idx] = f32_to_bf16(v);
+  }
+}
+
+// One atomic per wave into the amax result, which a fill kernel zeroed before the launch.
+__device__ __forceinline__ void fold_amax(const Fp8DecodeParams& p, uint32_t amax_bits) {
+  if (!p.out8 || !p.amax) return;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, off));
+  if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned*>(p.amax), amax_bits);
+}
+
+// Adds the waves' accumulator tiles through LDS, 32 registers (one 16-token tile) per pass, and
+// finishes them.  rhs [K,N]: register r = t * 8 + j (acc[j][mt][t]) in lane (li, kb) is channel
+// strip * 128 + (4 * kb + t) * 8 + j; rhs [N,K]: register r = 4 * g + t (acc[g][mt][t]) is channel
+// strip * 128 + 16 * g + 4 * kb + t; token 16 * mt + li in both.  Wave w finishes registers
+// 4w .. 4w+3 of every pass, four consecutive channels of one token.
+template <int MT, bool NK>
+__device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float* lds, const floatx4 (&acc)[8][MT],
+                                                 int strip, int slice, int batch) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, kb = lane >> 4;
+  const float alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+  uint32_t amax_bits = 0u;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (mt) __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 32; ++r) lds[(wave * 32 + r) * 64 + lane] = NK ? acc[r >> 2][mt][r & 3] : acc[r & 7][mt][r >> 3];
+    __syncthreads();
+    float res[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float s = 0.0f;
+#pragma unroll
+      for (int w2 = 0; w2 < kWaves; ++w2) s = s + lds[(w2 * 32 + wave * 4 + u) * 64 + lane];
+      res[u] = s;
+    }
+    const int m = 16 * mt + li;
+    const int n0 = strip * 128 + (NK ? 16 * wave + 4 * kb : (4 * kb + (wave >> 1)) * 8 + 4 * (wave & 1));
+    if (m >= p.M || n0 >= p.N) continue;  // N % 8 == 0: a run of four is inside N or not at all
+    if (p.slices > 1) {
+      float* dst = p.partial + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
+      *reinterpret_cast<floatx4*>(dst) = floatx4{res[0], res[1], res[2], res[3]};
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) finish_value(p, batch, m, n0 + u, res[u], alpha, &amax_bits);
+    }
+  }
+  if (p.slices == 1) fold_amax(p, amax_bits);
+}
+
+// rhs [K,N].  MT: 16-token tiles.  A workgroup owns 128 channels (one 128-byte line per row) and
+// rows_per_slice rows, its waves rows_per_wave consecutive rows each, in steps of 32.
+template <int MT>
+__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
+  __shared__ float lds[kWaves * 32 * 64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, kb = lane >> 4;
+  const int slice = blockIdx.x % p.slices;
+  const int strip = blockIdx.x / p.slices;
+  const int batch = blockIdx.y;
+  const int n_lane = strip * 128 + li * 8;
+  const uint32_t pitch = (uint32_t)p.N;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * pitch);
+  // one descriptor per 16-token tile, each ending where the activations end: the lane offset is
+  // then the same for every tile and still range-checks tokens >= M
+  __amdgpu_buffer_rsrc_t ra[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int rows = max(p.M - 16 * mt, 0);
+    ra[mt] = make_rsrc(p.a + ((size_t)batch * p.M + (rows ? 16 * mt : 0)) * p.K, (uint32_t)rows * p.K);
+  }
+  const uint32_t voff_w = n_lane < p.N ? (uint32_t)(8 * kb) * pitch + (uint32_t)n_lane : kNowhere;
+  const uint32_t voff_a = (uint32_t)li * p.K + 8 * kb;
+  // rows 1..7 of a lane's block of 8 are reached through the scalar offset: K % 8 == 0, so the
+  // block is inside the rhs exactly when its first row is, which the lane offset checks
+  uint32_t soff_w[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) soff_w[r] = (uint32_t)r * pitch;
+
+  floatx4 acc[8][MT];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int slice_end = min((slice + 1) * p.rows_per_slice, p.K);
+  const int k_begin = slice * p.rows_per_slice + wave * p.rows_per_wave;
+  const int k_stop = min(k_begin + p.rows_per_wave, slice_end);
+
+  uintx2 wq[2][8];
+  uintx2 aq[2][MT];
+  auto load_step = [&](int buf, int k0) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) aq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b64(ra[mt], voff_a + (uint32_t)k0, 0, 0);
+    const uint32_t vw = voff_w + (uint32_t)k0 * pitch;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) wq[buf][r] = __builtin_amdgcn_raw_buffer_load_b64(rw, vw, soff_w[r], 0);
+  };
+  auto compute = [&](int buf, int k0) {
+    uintx2 av[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) av[mt] = aq[buf][mt];
+    if (k0 + 32 > p.K) {  // scalar: only a step that crosses the end of K (its rhs rows read as zeros)
+      asm volatile("");
+      const bool ok = k0 + 8 * kb < p.K;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) av[mt] = uintx2{ok ? av[mt][0] : 0u, ok ? av[mt][1] : 0u};
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      // 4x4 byte transposes: t[h][e] = byte e of rows 4h .. 4h+3 of dword q
+      uint32_t t[2][4];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t x0 = wq[buf][4 * h][q], x1 = wq[buf][4 * h + 1][q], x2 = wq[buf][4 * h + 2][q], x3 = wq[buf][4 * h + 3][q];
+        const uint32_t p0 = __builtin_amdgcn_perm(x1, x0, 0x05010400u), p1 = __builtin_amdgcn_perm(x1, x0, 0x07030602u);
+        const uint32_t q0 = __builtin_amdgcn_perm(x3, x2, 0x05010400u), q1 = __builtin_amdgcn_perm(x3, x2, 0x07030602u);
+        t[h][0] = __builtin_amdgcn_perm(q0, p0, 0x05040100u);
+        t[h][1] = __builtin_amdgcn_perm(q0, p0, 0x07060302u);
+        t[h][2] = __builtin_amdgcn_perm(q1, p1, 0x05040100u);
+        t[h][3] = __builtin_amdgcn_perm(q1, p1, 0x07060302u);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const long wop = __builtin_bit_cast(long, uintx2{t[0][e], t[1][e]});
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[4 * q + e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wop, __builtin_bit_cast(long, av[mt]),
+                                                                          acc[4 * q + e][mt], 0, 0, 0);
+      }
+    }
+  };
+  if (k_begin < k_stop) {
+    load_step(0, k_begin);
+    for (int k0 = k_begin; k0 < k_stop; k0 += 64) {
+      if (k0 + 32 < k_stop) load_step(1, k0 + 32);
+      compute(0, k0);
+      if (k0 + 64 < k_stop) load_step(0, k0 + 64);
+      if (k0 + 32 < k_stop) compute(1, k0 + 32);
+    }
+  }
+  reduce_and_store<MT, false>(p, lds, acc, strip, slice, batch);
+}
+
+// rhs [N,K].  A workgroup owns 128 channels (8 groups of 16) and rows_per_slice values of k, its
+// waves rows_per_wave consecutive ones each, in steps of 128 (one line per channel), a step in two
+// halves of four channel groups.
+template <int MT>
+__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
+  __shared__ float lds[kWaves * 32 * 64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int li = lane & 15, kb = lane >> 4;
+  const int slice = blockIdx.x % p.slices;
+  const int strip = blockIdx.x / p.slices;
+  const int batch = blockIdx.y;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
+  __amdgpu_buffer_rsrc_t ra[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int rows = max(p.M - 16 * mt, 0);
+    ra[mt] = make_rsrc(p.a + ((size_t)batch * p.M + (rows ? 16 * mt : 0)) * p.K, (uint32_t)rows * p.K);
+  }
+  // loading side: instruction (g, hh) takes channels 16 g + 8 hh + (lane >> 3), piece lane & 7 of
+  // their lines; N % 8 == 0, so its 8 channels are inside N or not at all
+  uint32_t voff_w[8][2];
+#pragma unroll
+  for (int g = 0; g < 8; ++g)
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int n = strip * 128 + 16 * g + 8 * hh + (lane >> 3);
+      voff_w[g][hh] = n < p.N ? (uint32_t)n * p.K + 16u * (lane & 7) : kNowhere;
+    }
+  const uint32_t voff_a = (uint32_t)li * p.K + 32 * kb;
+  // consuming side: lane (li, kb) stands for channel 16 g + li and wants pieces 2 kb and 2 kb + 1,
+  // which lanes 8 (li & 7) + 2 kb (+ 1) of instruction (g, li >> 3) hold
+  const int src0 = 4 * (8 * (li & 7) + 2 * kb);
+  const bool upper = li >= 8;
+
+  floatx4 acc[8][MT];
+#pragma unroll
+  for (int g = 0; g < 8; ++g)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[g][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int slice_end = min((slice + 1) * p.rows_per_slice, p.K);
+  const int k_begin = slice * p.rows_per_slice + wave * p.rows_per_wave;
+  const int k_stop = min(k_begin + p.rows_per_wave, slice_end);
+
+  uintx4 wq[2][4][2];   // [buffer][group of the half][hh]
+  uintx4 aq[2][MT][2];  // [buffer][tile][16-byte half]
+  auto load_a = [&](int buf, int k0) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      aq[buf][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], voff_a + (uint32_t)k0, 0, 0);
+      aq[buf][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], voff_a + (uint32_t)k0 + 16u, 0, 0);
+    }
+  };
+  auto load_w = [&](int buf, int half, int k0) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+        wq[buf][g][hh] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w[4 * half + g][hh] + (uint32_t)k0, 0, 0);
+  };
+  auto compute = [&](int buf, int abuf, int half, int k0) {
+    uintx4 av[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      av[mt][0] = aq[abuf][mt][0];
+      av[mt][1] = aq[abuf][mt][1];
+    }
+    uintx4 wv[4][2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      wv[g][0] = wq[buf][g][0];
+      wv[g][1] = wq[buf][g][1];
+    }
+    if (k0 + 128 > p.K) {  // scalar: only a step that crosses the end of K (K % 16 == 0: whole pieces)
+      asm volatile("");
+      const bool wok = k0 + 16 * (lane & 7) < p.K;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) wv[g][hh][d] = wok ? wv[g][hh][d] : 0u;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+          const bool aok = k0 + 32 * kb + 16 * x < p.K;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) av[mt][x][d] = aok ? av[mt][x][d] : 0u;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint32_t tg[8];
+#pragma unroll
+      for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + 4 * x, (int)wv[g][0][d]);
+          const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + 4 * x, (int)wv[g][1][d]);
+          tg[4 * x + d] = upper ? hi : lo;
+        }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const long wop = __builtin_bit_cast(long, uintx2{tg[2 * i], tg[2 * i + 1]});
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const uintx2 a2 = {av[mt][i >> 1][2 * (i & 1)], av[mt][i >> 1][2 * (i & 1) + 1]};
+          acc[4 * half + g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wop, __builtin_bit_cast(long, a2),
+                                                                             acc[4 * half + g][mt], 0, 0, 0);
+        }
+      }
+    }
+  };
+  if (k_begin < k_stop) {
+    load_a(0, k_begin);
+    load_w(0, 0, k_begin);
+    for (int k0 = k_begin; k0 < k_stop; k0 += 256) {
+      load_w(1, 1, k0);
+      compute(0, 0, 0, k0);
+      if (k0 + 128 < k_stop) { load_a(1, k0 + 128); load_w(0, 0, k0 + 128); }
+      compute(1, 0, 1, k0);
+      if (k0 + 128 < k_stop) {
+        load_w(1, 1, k0 + 128);
+        compute(0, 1, 0, k0 + 128);
+        if (k0 + 256 < k_stop) { load_a(0, k0 + 256); load_w(0, 0, k0 + 256); }
+        compute(1, 1, 1, k0 + 128);
+      }
+    }
+  }
+  reduce_and_store<MT, true>(p, lds, acc, strip, slice, batch);
+}
+
+// Sums the K-slices in slice order and finishes the values.
+__global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeParams p) {
+  const size_t total = (size_t)p.M * p.N;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int batch = blockIdx.y;
+  uint32_t amax_bits = 0u;
+  if (idx < total) {
+    const float* ws = p.partial + (size_t)batch * p.slices * total + idx;
+    float v = 0.0f;
+    for (int s = 0; s < p.slices; ++s) v = v + ws[(size_t)s * total];
+    const float alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+    finish_value(p, batch, (int)(idx / p.N), (int)(idx % p.N), v, alpha, &amax_bits);
+  }
+  fold_amax(p, amax_bits);
+}
+
+// K-slices for the shape: more workgroups until every CU has one, as long as a wave keeps at
+// least 128 values of k (256 for the [N,K] kernel, two of its steps) and the sums written and read
+// again stay under a quarter of the rhs bytes.
+int Slices(int64_t batch, int64_t M, int64_t K, int64_t N, bool nk) {
+  if (int s = GetOption("fp8_decode_slices")) return s;
+  const int64_t strips = (N + 127) / 128;
+  int slices = 1;
+  while (strips * batch * slices < 192 && slices < 16 && K / (slices * 2) >= (nk ? 256 : 128) * kWaves &&
+         2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * (double)K * N)
+    slices *= 2;
+  return slices;
+}
+
+}  // namespace
+
+size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
+  if (M <= 0 || M > (rhs_contracting_dim == 1 ? 32 : 64) || K <= 0 || N <= 0 || batch <= 0) return 0;
+  const int slices = Slices(batch, M, K, N, rhs_contracting_dim == 1);
+  return slices > 1 ? (size_t)batch * slices * M * N * 4 : 0;
+}
+
+// Returns -1 when the shape is not covered, else the launch status.
+int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
+  const int64_t batch = p.batch > 1 ? p.batch : 1;
+  const bool nk = p.rhs_contracting_dim == 1;
+  const int align = nk ? 16 : 8;  // bytes a lane loads at once
+  if (p.M <= 0 || p.M > (nk ? 32 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
+  if (p.a_block_scales || p.b_block_scales || p.dequant_type != XLA_FFI_DataType_F32) return -1;
+  if (((uintptr_t)p.a % align) || ((uintptr_t)p.b % align) || (double)p.K * p.N >= 2147483000.0 || batch > 65535) return -1;
+  const bool out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
+  Fp8DecodeParams dp{};
+  dp.a = (const uint8_t*)p.a;
+  dp.b = (const uint8_t*)p.b;
+  dp.a_scale = p.a_scale;
+  dp.b_scale = p.b_scale;
+  dp.a_per_row = p.a_scale_per_row != 0;
+  dp.b_per_channel = p.b_scale_per_channel != 0;
+  dp.bias = (p.epilogue & 1) ? p.bias : nullptr;
+  dp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
+  dp.out = out_f8 ? nullptr : (uint16_t*)p.out;
+  dp.out8 = out_f8 ? (uint8_t*)p.out : nullptr;
+  dp.d_scale = p.d_scale;
+  dp.d_divides = p.d_scale_multiplies ? 0 : 1;
+  dp.amax = out_f8 ? p.amax : nullptr;
+  dp.M = (int)p.M; dp.K = (int)p.K; dp.N = (int)p.N;
+  dp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
+  dp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
+  dp.epilogue = p.epilogue;
+  const int kStep = nk ? 128 : 32;
+  int slices = Slices(batch, p.M, p.K, p.N, nk);
+  const size_t need = (size_t)batch * slices * p.M * p.N * 4;
+  if (slices > 1 && (!p.workspace || p.workspace_bytes < need || ((uintptr_t)p.workspace % 16))) slices = 1;
+  dp.slices = slices;
+  dp.partial = (float*)p.workspace;
+  const int per = (int)((p.K + slices - 1) / slices);
+  dp.rows_per_wave = ((per + kWaves - 1) / kWaves + kStep - 1) / kStep * kStep;
+  dp.rows_per_slice = dp.rows_per_wave * kWaves;
+  const int strips = (int)((p.N + 127) / 128);
+  dim3 grid((unsigned)(strips * slices), (unsigned)batch);
+  const int mt = (int)((p.M + 15) / 16);
+  if (nk) {
+    switch (mt) {
+      case 1: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<1>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      default: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+    }
+  } else {
+    switch (mt) {
+      case 1: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<1>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      case 2: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      case 3: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<3>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      default: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<4>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+    }
+  }
+  int rc = CheckLaunch("fp8_dot_decode");
+  if (rc) return rc;
+  if (slices > 1) {
+    dim3 fgrid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(fp8_dot_decode_finalize_kernel, fgrid, dim3(256), 0, stream, dp);
+    rc = CheckLaunch("fp8_dot_decode_finalize");
+    if (rc) return rc;
+  }
+  static const char* names[2][4] = {{"fp8_dot_decode_kn_m16", "fp8_dot_decode_kn_m32", "fp8_dot_decode_kn_m48", "fp8_dot_decode_kn_m64"},
+                                    {"fp8_dot_decode_nk_m16", "fp8_dot_decode_nk_m32", "fp8_dot_decode_nk_m48", "fp8_dot_decode_nk_m64"}};
+  SetLastKernel(names[nk ? 1 : 0][mt - 1]);
+  return 0;
+}
+
+}  // namespace xla_amd

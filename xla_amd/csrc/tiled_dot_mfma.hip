@@ -1333,7 +1333,10 @@ size_t Bf16OperandBytes(int64_t M, int64_t K, int64_t N) {
 size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contracting_dim, int dequant_type) {
   const size_t copy = TransposedCopyBytes(K, N, rhs_contracting_dim);
   const size_t ops = dequant_type == XLA_FFI_DataType_BF16 ? Bf16OperandBytes(M, K, N) : 0;
-  return ops ? RoundUp256(copy) + ops : copy;
+  const size_t tiled = ops ? RoundUp256(copy) + ops : copy;
+  // up to 64 rows of a under f32-typed multiplies: the streaming kernels' K-slices instead
+  const size_t decode = dequant_type == XLA_FFI_DataType_BF16 ? 0 : Fp8DotDecodeWorkspaceBytes(1, M, K, N, rhs_contracting_dim);
+  return tiled > decode ? tiled : decode;
 }
 
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
@@ -1400,6 +1403,15 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     int rc = CheckLaunch("fp8_scaled_dot_amax_init");
     if (rc) return rc;
   }
+  const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled, 3 streaming (up to 64 rows of a)
+  if (force == 0 || force == 3) {
+    const int rc = LaunchFp8DotDecode(p, stream);
+    if (rc >= 0) return rc;
+    if (force == 3)
+      return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
+                  "fp8_scaled_dot: the streaming kernels take up to 64 rows of a, K %% 8 == 0 and N %% 8 == 0, "
+                  "8-byte aligned operands, f32-typed multiplies and no block scales");
+  }
   tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
   tp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
   tp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
@@ -1414,7 +1426,6 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   // multiply it takes the exact kernel
   const bool vector_scales = tp.a_per_row || tp.b_per_channel;
 
-  const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled
   const bool nk = p.rhs_contracting_dim == 1;
   const int batch = p.batch > 1 ? (int)p.batch : 1;
   if (p.batch > 65535) return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: more than 65535 batches");
