@@ -281,6 +281,21 @@ def main():
         finally:
             ffi.set_option("tiled_epilogue", 0)
         del a8, b8
+        # the decode end of the same call: 16 rows of a against an f8 matrix of C2's shape, streamed once
+        # (informational -- not one of the five configurations)
+        a8d = (torch.randn((16, K2), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+        b8d = (torch.randn((K2, N2), device=dev) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+        b3d = torch.randn((N2,), device=dev).to(torch.bfloat16)
+        f8d_bytes = K2 * N2 + 16 * K2 + 16 * N2 * 2 + N2 * 2
+        entry("fp8 decode", "fp8 [16,8192]x[8192,28672] + bias + GELU (rhs [K,N])",
+              ops.fp8_scaled_dot(a8d, b8d, s64, s64, b3d, epilogue="BIAS_GELU", build_only=True),
+              f8d_bytes, 2 * 16 * K2 * N2, "hbm")
+        b8dt = b8d.view(torch.uint8).t().contiguous()
+        del b8d
+        entry("fp8 decode nk", "fp8 [16,8192]x[28672,8192] + bias + GELU (rhs [N,K])",
+              ops.fp8_scaled_dot(a8d, b8dt, s64, s64, b3d, epilogue="BIAS_GELU", rhs_contracting_dim=1, build_only=True),
+              f8d_bytes, 2 * 16 * K2 * N2, "hbm")
+        del a8d, b8dt
         # C5: batched s8 per-channel prefill
         a5 = torch.randn((8, 512, 4096), device=dev).to(torch.bfloat16)
         w5 = torch.randint(-127, 128, (8, 4096, 14336), dtype=torch.int8, device=dev)
@@ -378,6 +393,14 @@ def main():
             for k in c3_keys:
                 by_key[k]["cpu_baseline"] = base(round(2 * 1024 * 8192 * 2048 / t / 1e12, 4), "TFLOP/s",
                                                  "1024 of 8192 rows x 2048 of 8192 channels (full K), f32-typed ops, %.2f s" % t)
+        f8d_keys = [k for k in ("fp8 decode", "fp8 decode nk") if k in by_key]
+        if f8d_keys:
+            w = workloads.c3_fp8(16, K2, 4096)
+            t = timed(lambda: oracle.fp8_scaled_dot(w["a"], w["b"], w["a_scale"], w["b_scale"], bias=w["bias"],
+                                                    epilogue="gelu_tanh"))
+            for k in f8d_keys:
+                by_key[k]["cpu_baseline"] = base(round(w["algorithmic_bytes"] / t / 1e9, 3), "GB/s",
+                                                 "4096 of %d channels (16 rows, full K; the oracle reads the rhs [K,N]), %.2f s" % (N2, t))
         if "C5" in by_key:
             w = workloads.c5_s8_batched(B=1, M=64, K=4096, N=14336)
             t = timed(lambda: oracle.dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32"))

@@ -66,7 +66,7 @@ def test_c3_shape_reduced(oracle, M, K, N, nk):
     say("fp8_scaled_dot M=%d K=%d N=%d nk=%s" % (M, K, N, nk))
     w = workloads.c3_fp8(M, K, N)
     got, kern = run(w, nk=nk)
-    assert kern.startswith("fp8_dot_decode" if M <= 32 else "fp8_scaled_dot_tiled"), kern
+    assert kern.startswith("fp8_dot_decode" if M <= 48 else "fp8_scaled_dot_tiled"), kern
     n_floor = check_dot(got, reference(oracle, w), floor_for(w), kern)
     assert n_floor <= got.size // 100
 

@@ -101,23 +101,26 @@ __device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float
 #pragma unroll
     for (int r = 0; r < 32; ++r) lds[(wave * 32 + r) * 64 + lane] = NK ? acc[r >> 2][mt][r & 3] : acc[r & 7][mt][r >> 3];
     __syncthreads();
-    float res[4];
+    constexpr int RPW = 32 / kWaves;
+    float res[RPW];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < RPW; ++u) {
       float s = 0.0f;
 #pragma unroll
-      for (int w2 = 0; w2 < kWaves; ++w2) s = s + lds[(w2 * 32 + wave * 4 + u) * 64 + lane];
+      for (int w2 = 0; w2 < kWaves; ++w2) s = s + lds[(w2 * 32 + wave * RPW + u) * 64 + lane];
       res[u] = s;
     }
     const int m = 16 * mt + li;
-    const int n0 = strip * 128 + (NK ? 16 * wave + 4 * kb : (4 * kb + (wave >> 1)) * 8 + 4 * (wave & 1));
-    if (m >= p.M || n0 >= p.N) continue;  // N % 8 == 0: a run of four is inside N or not at all
+    const int r0 = wave * RPW;  // the wave's first register of the pass
+    const int n0 = strip * 128 + (NK ? 16 * (r0 >> 2) + 4 * kb + (r0 & 3) : (4 * kb + (r0 >> 3)) * 8 + (r0 & 7));
+    if (m >= p.M || n0 >= p.N) continue;  // N % 8 == 0: an aligned run of four is inside N or not at all
     if (p.slices > 1) {
       float* dst = p.partial + (((size_t)batch * p.slices + slice) * p.M + m) * p.N + n0;
-      *reinterpret_cast<floatx4*>(dst) = floatx4{res[0], res[1], res[2], res[3]};
+#pragma unroll
+      for (int u = 0; u < RPW; ++u) dst[u] = res[u];
     } else {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) finish_value(p, batch, m, n0 + u, res[u], alpha, &amax_bits);
+      for (int u = 0; u < RPW; ++u) finish_value(p, batch, m, n0 + u, res[u], alpha, &amax_bits);
     }
   }
   if (p.slices == 1) fold_amax(p, amax_bits);
@@ -265,21 +268,26 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 
   uintx4 wq[2][4][2];   // [buffer][group of the half][hh]
   uintx4 aq[2][MT][2];  // [buffer][tile][16-byte half]
+  // A piece past the end of K (K % 16 == 0: pieces are whole) lies in the next row of its operand, not
+  // past the buffer: such a load gets the offset no buffer reaches instead and returns zeros.
   auto load_a = [&](int buf, int k0) {
+    const uint32_t o0 = k0 + 32 * kb < p.K ? voff_a + (uint32_t)k0 : kNowhere;
+    const uint32_t o1 = k0 + 32 * kb + 16 < p.K ? voff_a + (uint32_t)k0 + 16u : kNowhere;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      aq[buf][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], voff_a + (uint32_t)k0, 0, 0);
-      aq[buf][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], voff_a + (uint32_t)k0 + 16u, 0, 0);
+      aq[buf][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], o0, 0, 0);
+      aq[buf][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], o1, 0, 0);
     }
   };
   auto load_w = [&](int buf, int half, int k0) {
+    const bool ok = k0 + 16 * (lane & 7) < p.K;
 #pragma unroll
     for (int g = 0; g < 4; ++g)
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh)
-        wq[buf][g][hh] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff_w[4 * half + g][hh] + (uint32_t)k0, 0, 0);
+        wq[buf][g][hh] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? voff_w[4 * half + g][hh] + (uint32_t)k0 : kNowhere, 0, 0);
   };
-  auto compute = [&](int buf, int abuf, int half, int k0) {
+  auto compute = [&](int buf, int abuf, int half) {
     uintx4 av[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -292,24 +300,6 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
       wv[g][0] = wq[buf][g][0];
       wv[g][1] = wq[buf][g][1];
     }
-    if (k0 + 128 > p.K) {  // scalar: only a step that crosses the end of K (K % 16 == 0: whole pieces)
-      asm volatile("");
-      const bool wok = k0 + 16 * (lane & 7) < p.K;
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-          for (int d = 0; d < 4; ++d) wv[g][hh][d] = wok ? wv[g][hh][d] : 0u;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int x = 0; x < 2; ++x) {
-          const bool aok = k0 + 32 * kb + 16 * x < p.K;
-#pragma unroll
-          for (int d = 0; d < 4; ++d) av[mt][x][d] = aok ? av[mt][x][d] : 0u;
-        }
-    }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       uint32_t tg[8];
@@ -321,16 +311,16 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
           const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + 4 * x, (int)wv[g][1][d]);
           tg[4 * x + d] = upper ? hi : lo;
         }
+      // 32 bytes of k per lane and operand: one v_mfma_f32_16x16x128_f8f6f4 (both formats e4m3, no block scales)
+      const intx8 wop = {(int)tg[0], (int)tg[1], (int)tg[2], (int)tg[3], (int)tg[4], (int)tg[5], (int)tg[6], (int)tg[7]};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const long wop = __builtin_bit_cast(long, uintx2{tg[2 * i], tg[2 * i + 1]});
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const uintx2 a2 = {av[mt][i >> 1][2 * (i & 1)], av[mt][i >> 1][2 * (i & 1) + 1]};
-          acc[4 * half + g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wop, __builtin_bit_cast(long, a2),
-                                                                             acc[4 * half + g][mt], 0, 0, 0);
-        }
+      for (int mt = 0; mt < MT; ++mt) {
+        const intx8 aop = {(int)av[mt][0][0], (int)av[mt][0][1], (int)av[mt][0][2], (int)av[mt][0][3],
+                           (int)av[mt][1][0], (int)av[mt][1][1], (int)av[mt][1][2], (int)av[mt][1][3]};
+        acc[4 * half + g][mt] =
+            __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc[4 * half + g][mt], 0, 0, 0, 0, 0, 0);
       }
+      if (g & 1) __builtin_amdgcn_sched_barrier(0);  // two groups' pieces on their way at a time, not all four
     }
   };
   if (k_begin < k_stop) {
@@ -338,14 +328,14 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
     load_w(0, 0, k_begin);
     for (int k0 = k_begin; k0 < k_stop; k0 += 256) {
       load_w(1, 1, k0);
-      compute(0, 0, 0, k0);
+      compute(0, 0, 0);
       if (k0 + 128 < k_stop) { load_a(1, k0 + 128); load_w(0, 0, k0 + 128); }
-      compute(1, 0, 1, k0);
+      compute(1, 0, 1);
       if (k0 + 128 < k_stop) {
         load_w(1, 1, k0 + 128);
-        compute(0, 1, 0, k0 + 128);
+        compute(0, 1, 0);
         if (k0 + 256 < k_stop) { load_a(0, k0 + 256); load_w(0, 0, k0 + 256); }
-        compute(1, 1, 1, k0 + 128);
+        compute(1, 1, 1);
       }
     }
   }
@@ -384,7 +374,7 @@ int Slices(int64_t batch, int64_t M, int64_t K, int64_t N, bool nk) {
 }  // namespace
 
 size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
-  if (M <= 0 || M > (rhs_contracting_dim == 1 ? 32 : 64) || K <= 0 || N <= 0 || batch <= 0) return 0;
+  if (M <= 0 || M > (rhs_contracting_dim == 1 ? 48 : 64) || K <= 0 || N <= 0 || batch <= 0) return 0;
   const int slices = Slices(batch, M, K, N, rhs_contracting_dim == 1);
   return slices > 1 ? (size_t)batch * slices * M * N * 4 : 0;
 }
@@ -394,7 +384,8 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const int64_t batch = p.batch > 1 ? p.batch : 1;
   const bool nk = p.rhs_contracting_dim == 1;
   const int align = nk ? 16 : 8;  // bytes a lane loads at once
-  if (p.M <= 0 || p.M > (nk ? 32 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
+  // (four token tiles of the [N,K] kernel do not fit the registers of two waves per SIMD: 48 rows there)
+  if (p.M <= 0 || p.M > (nk ? 48 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
   if (p.a_block_scales || p.b_block_scales || p.dequant_type != XLA_FFI_DataType_F32) return -1;
   if (((uintptr_t)p.a % align) || ((uintptr_t)p.b % align) || (double)p.K * p.N >= 2147483000.0 || batch > 65535) return -1;
   const bool out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
@@ -422,16 +413,18 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   if (slices > 1 && (!p.workspace || p.workspace_bytes < need || ((uintptr_t)p.workspace % 16))) slices = 1;
   dp.slices = slices;
   dp.partial = (float*)p.workspace;
+  const int mt = (int)((p.M + 15) / 16);
+  const int waves = kWaves;
   const int per = (int)((p.K + slices - 1) / slices);
-  dp.rows_per_wave = ((per + kWaves - 1) / kWaves + kStep - 1) / kStep * kStep;
-  dp.rows_per_slice = dp.rows_per_wave * kWaves;
+  dp.rows_per_wave = ((per + waves - 1) / waves + kStep - 1) / kStep * kStep;
+  dp.rows_per_slice = dp.rows_per_wave * waves;
   const int strips = (int)((p.N + 127) / 128);
   dim3 grid((unsigned)(strips * slices), (unsigned)batch);
-  const int mt = (int)((p.M + 15) / 16);
   if (nk) {
     switch (mt) {
       case 1: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<1>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      default: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      case 2: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+      default: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<3>, grid, dim3(kWaves * 64), 0, stream, dp); break;
     }
   } else {
     switch (mt) {
