@@ -113,6 +113,8 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
  *          rhs_contracting_dim i64 (default 0);
  *          d_scale_multiplies pred (default false): v * d_scale instead (:1730-1748)
+ * One handler for every size: up to 64 rows of a take kernels that stream the rhs once (HBM-bound),
+ * more rows the tiled kernel (MFMA-bound).
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* call_frame);
 
@@ -263,7 +265,9 @@ XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, vo
 /* Scratch the call can use (0 = none).  A [K,N] rhs whose N is a multiple of 16 goes in as it is;
  * any other [K,N] rhs is re-laid out with K minor first (the transpose GemmRewriter inserts at
  * gemm_rewriter.cc:1235-1591), which takes K*N bytes -- without them such a rhs runs on the slow
- * exact kernel. */
+ * exact kernel.  Up to 64 rows of a (48 with an [N,K] rhs; K and N multiples of 8, resp. 16 and 8)
+ * stream the rhs once instead and, where the channels alone leave CUs idle, split K over workgroups:
+ * slices * M * N * 4 bytes of f32 sums, per batch -- without them one slice. */
 XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                                              int32_t rhs_contracting_dim);
 
@@ -305,7 +309,7 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * (steps per wave of the single-launch s8 kernel: 1, 2, 4), "dequant_dot_strip" (channels per strip of
  * that kernel: 64 or 128), "handover_test" (1: workgroups that hand partial sums over never raise their
  * flags and the waiting side gives up after 16 polls, so that its own fallback computes the result --
- * for tests of that fallback only), "fp8_dot_kernel" (1 exact, 2 tiled),
+ * for tests of that fallback only), "fp8_dot_kernel" (1 exact, 2 tiled, 3 streaming), "fp8_decode_slices" (K-slices of the streaming kernels),
  * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1:
  * the tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the
