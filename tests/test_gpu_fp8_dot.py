@@ -333,7 +333,7 @@ def test_mxfp8_one_block_at_a_time(oracle):
     ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
     bi = rng.integers(-3, 4, (N, K)).astype(np.float32)
     sa = np.repeat((121 + np.arange(K // 32)).astype(np.uint8)[None, :], M, axis=0)
-    sb = np.repeat((130 - np.arange(K // 32)).astype(np.uint8)[None, :], N, axis=0)
+    sb = np.repeat((134 - 2 * np.arange(K // 32)).astype(np.uint8)[None, :], N, axis=0)   # sa + sb differs from block to block
     sb[:, :] += (np.arange(N) % 3).astype(np.uint8)[:, None]
     for j in range(K // 32):
         a1 = np.zeros_like(ai)

@@ -211,3 +211,76 @@ def test_what_the_streaming_kernels_do_not_take():
             ops.fp8_scaled_dot(a[:8], b, one, one, dequant_type="bf16")
     finally:
         ffi.set_option("fp8_dot_kernel", 0)
+
+
+# ---- block scales (MXFP8) on the [N,K] streaming kernel: up to 32 rows of a, K % 128 == 0 ---------------
+
+def run_mx(a, b, sa, sb, bias=None, slices=0, batch=None, **kw):
+    ffi.set_option("fp8_dot_kernel", 3)
+    ffi.set_option("fp8_decode_slices", slices)
+    try:
+        scratch = "auto"
+        if slices:
+            n = ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(a.shape[-2], a.shape[-1], b.shape[-2], 1)
+            scratch = torch.empty(max(n * (batch or 1), 16), dtype=torch.uint8, device="cuda")
+        out = ops.fp8_scaled_dot(dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), dev_bf16(bias) if bias is not None else None,
+                                 rhs_contracting_dim=1, scratch=scratch, **kw)
+        torch.cuda.synchronize()
+    finally:
+        ffi.set_option("fp8_dot_kernel", 0)
+        ffi.set_option("fp8_decode_slices", 0)
+    return host_bf16(out), ffi.last_kernel()
+
+
+@pytest.mark.parametrize("M", [1, 16, 17, 32])
+@pytest.mark.parametrize("K,N", [(512, 272), (1024, 136), (128, 64)])
+@pytest.mark.parametrize("slices", [0, 2])
+def test_mxfp8_block_scales(oracle, M, K, N, slices):
+    from tests.test_gpu_fp8_dot import mx_case, mx_floor
+    say("fp8 streaming MXFP8 M=%d K=%d N=%d slices=%d" % (M, K, N, slices))
+    a, b, sa, sb = mx_case(M, K, N, 7)
+    got, kern = run_mx(a, b, sa, sb, slices=slices)
+    assert kern == "fp8_dot_decode_mx_m%d" % (16 * ((M + 15) // 16)), kern
+    n_floor = check_dot(got, oracle.block_scaled_dot(a, b, sa, sb), mx_floor(a, b, sa, sb, False), kern)
+    assert n_floor <= max(4, got.size // 50)
+
+
+@pytest.mark.parametrize("epilogue,dot_ty,ep_ty", [("BIAS_GELU", "f32", "f32"), ("BIAS_SILU", "bf16", "bf16"), ("RELU", "f32", "f32")])
+def test_mxfp8_with_an_epilogue_and_batched(oracle, epilogue, dot_ty, ep_ty):
+    from tests.test_gpu_fp8_dot import mx_case, mx_floor
+    say("fp8 streaming MXFP8 %s dot %s ops %s, batched" % (epilogue, dot_ty, ep_ty))
+    names = {"BIAS_GELU": "gelu_tanh", "BIAS_SILU": "silu", "RELU": "relu"}
+    B, M, K, N = 2, 24, 384, 200
+    cases = [mx_case(M, K, N, 30 + i) for i in range(B)]
+    a, b, sa, sb = (np.stack([c[j] for c in cases]) for j in range(4))
+    bias = dtypes.f32_to_bf16(np.random.default_rng(3).standard_normal(N).astype(np.float32)) if "BIAS" in epilogue else None
+    got, kern = run_mx(a, b, sa, sb, bias, batch=B, epilogue=epilogue, dot_type=dot_ty, epilogue_type=ep_ty)
+    assert kern == "fp8_dot_decode_mx_m32", kern
+    for i in range(B):
+        ref = oracle.block_scaled_dot(a[i], b[i], sa[i], sb[i], bias=bias, dot_ty=dot_ty, ep_ty=ep_ty, epilogue=names[epilogue])
+        fl = 1.2 * mx_floor(a[i], b[i], sa[i], sb[i], False)
+        if "bf16" in (dot_ty, ep_ty):
+            fl = fl * 12 + np.abs(dtypes.bf16_to_f32(ref)) * 6 * 2.0 ** -8
+        check_dot(got[i], ref, fl, "%s %s batch %d" % (kern, epilogue, i))
+
+
+def test_mxfp8_one_block_at_a_time(oracle):
+    """Data in a single 32-element block of K, a different scale on every block and channel: each block must
+    come out multiplied by its own two scales exactly (products of small integers, exact sums) -- a scale
+    byte taken from the wrong block, row or channel shows as a wrong power of two."""
+    say("fp8 streaming MXFP8 block by block")
+    M, K, N = 20, 256, 144
+    rng = np.random.default_rng(2)
+    ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    bi = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    sa = np.repeat((121 + np.arange(K // 32)).astype(np.uint8)[None, :], M, axis=0)
+    sa[:, :] += (np.arange(M) % 5).astype(np.uint8)[:, None]
+    sb = np.repeat((134 - 2 * np.arange(K // 32)).astype(np.uint8)[None, :], N, axis=0)   # sa + sb differs from block to block
+    sb[:, :] += (np.arange(N) % 3).astype(np.uint8)[:, None]
+    for j in range(K // 32):
+        a1 = np.zeros_like(ai)
+        a1[:, 32 * j:32 * j + 32] = ai[:, 32 * j:32 * j + 32]
+        a8, b8 = dtypes.f32_to_f8e4m3fn(a1), dtypes.f32_to_f8e4m3fn(bi)
+        got, kern = run_mx(a8, b8, sa, sb)
+        assert kern == "fp8_dot_decode_mx_m32"
+        assert np.array_equal(got, oracle.block_scaled_dot(a8, b8, sa, sb)), j

@@ -39,6 +39,10 @@ struct Fp8DecodeParams {
   const uint8_t* b;      // [batch, K, N], or [batch, N, K]
   const float* a_scale;  // one value, or M (a_per_row)
   const float* b_scale;  // one value, or N (b_per_channel)
+  // block scales instead (rhs [N,K] only): one f8e8m0fnu byte per 32 values of k,
+  // [batch, M, K / 32] and [batch, N, K / 32]; K % 128 == 0
+  const uint8_t* a_block_scales;
+  const uint8_t* b_block_scales;
   const void* bias;      // [N] or null
   uint16_t* out;         // [batch, M, N] bf16, or
   uint8_t* out8;         // f8e4m3fn codes: convert(clamp(v / *d_scale)) (v * *d_scale unless d_divides)
@@ -93,7 +97,8 @@ __device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4;
-  const float alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+  // (block scales went in with the matrix instructions)
+  const float alpha = p.a_block_scales ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
   uint32_t amax_bits = 0u;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -223,8 +228,14 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8Decod
 
 // rhs [N,K].  A workgroup owns 128 channels (8 groups of 16) and rows_per_slice values of k, its
 // waves rows_per_wave consecutive ones each, in steps of 128 (one line per channel), a step in two
-// halves of four channel groups.
-template <int MT>
+// halves of four channel groups.  MX: block scales.  The matrix instruction takes the scale of the
+// step's block j (32 values of k) from the lanes with kb = j and applies it to the first 16 bytes of
+// the lanes kb = 2 (j & 1), 2 (j & 1) + 1 for j < 2 and to their second 16 bytes for j >= 2 (as
+// measured on the 32x32x64 form: the first 16 bytes of all lanes of a row are k 0..63 in lane order,
+// the second 16 bytes k 64..127).  So with block scales lane (., kb) holds pieces kb and kb + 4 of the
+// line instead of 2 kb and 2 kb + 1; a step's four scales of a channel (or row of a) are one dword,
+// of which lane (., kb) hands in byte kb.
+template <int MT, bool MX>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
   const int lane = threadIdx.x & 63;
@@ -250,10 +261,26 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
       const int n = strip * 128 + 16 * g + 8 * hh + (lane >> 3);
       voff_w[g][hh] = n < p.N ? (uint32_t)n * p.K + 16u * (lane & 7) : kNowhere;
     }
-  const uint32_t voff_a = (uint32_t)li * p.K + 32 * kb;
+  const uint32_t voff_a = (uint32_t)li * p.K + (MX ? 16 : 32) * kb;
+  constexpr uint32_t kSecond = MX ? 64u : 16u;  // from a lane's first piece to its second
+  // block scales: the dword of row li of a's tile, and of channel 16 g + li
+  const uint32_t kblocks = (uint32_t)p.K >> 5;
+  __amdgpu_buffer_rsrc_t rsa[MX ? MT : 1];
+  const __amdgpu_buffer_rsrc_t rsb =
+      make_rsrc(MX ? p.b_block_scales + (size_t)batch * p.N * kblocks : p.b, MX ? (uint32_t)p.N * kblocks : 0u);
+  if (MX) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int rows = max(p.M - 16 * mt, 0);
+      rsa[mt] = make_rsrc(p.a_block_scales + ((size_t)batch * p.M + (rows ? 16 * mt : 0)) * kblocks, (uint32_t)rows * kblocks);
+    }
+  }
+  const uint32_t voff_sa = (uint32_t)li * kblocks;
+  const int n_li = strip * 128 + li;
   // consuming side: lane (li, kb) stands for channel 16 g + li and wants pieces 2 kb and 2 kb + 1,
   // which lanes 8 (li & 7) + 2 kb (+ 1) of instruction (g, li >> 3) hold
-  const int src0 = 4 * (8 * (li & 7) + 2 * kb);
+  const int src0 = 4 * (8 * (li & 7) + (MX ? kb : 2 * kb));
+  constexpr int kSrcStep = MX ? 16 : 4;  // four lanes on, or the next one
   const bool upper = li >= 8;
 
   floatx4 acc[8][MT];
@@ -268,15 +295,18 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 
   uintx4 wq[2][4][2];   // [buffer][group of the half][hh]
   uintx4 aq[2][MT][2];  // [buffer][tile][16-byte half]
+  uint32_t sbq[2][MX ? 4 : 1], saq[2][MX ? MT : 1];  // the step's block scales
   // A piece past the end of K (K % 16 == 0: pieces are whole) lies in the next row of its operand, not
   // past the buffer: such a load gets the offset no buffer reaches instead and returns zeros.
   auto load_a = [&](int buf, int k0) {
-    const uint32_t o0 = k0 + 32 * kb < p.K ? voff_a + (uint32_t)k0 : kNowhere;
-    const uint32_t o1 = k0 + 32 * kb + 16 < p.K ? voff_a + (uint32_t)k0 + 16u : kNowhere;
+    const int piece = MX ? 16 * kb : 32 * kb;
+    const uint32_t o0 = k0 + piece < p.K ? voff_a + (uint32_t)k0 : kNowhere;
+    const uint32_t o1 = k0 + piece + (int)kSecond < p.K ? voff_a + (uint32_t)k0 + kSecond : kNowhere;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       aq[buf][mt][0] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], o0, 0, 0);
       aq[buf][mt][1] = __builtin_amdgcn_raw_buffer_load_b128(ra[mt], o1, 0, 0);
+      if (MX) saq[buf][mt] = __builtin_amdgcn_raw_buffer_load_b32(rsa[mt], voff_sa + ((uint32_t)k0 >> 5), 0, 0);
     }
   };
   auto load_w = [&](int buf, int half, int k0) {
@@ -286,6 +316,13 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 #pragma unroll
       for (int hh = 0; hh < 2; ++hh)
         wq[buf][g][hh] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? voff_w[4 * half + g][hh] + (uint32_t)k0 : kNowhere, 0, 0);
+    if (MX) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n_li + 16 * (4 * half + g);
+        sbq[buf][g] = __builtin_amdgcn_raw_buffer_load_b32(rsb, n < p.N ? (uint32_t)n * kblocks + ((uint32_t)k0 >> 5) : kNowhere, 0, 0);
+      }
+    }
   };
   auto compute = [&](int buf, int abuf, int half) {
     uintx4 av[MT][2];
@@ -307,8 +344,8 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
       for (int x = 0; x < 2; ++x)
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + 4 * x, (int)wv[g][0][d]);
-          const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + 4 * x, (int)wv[g][1][d]);
+          const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + kSrcStep * x, (int)wv[g][0][d]);
+          const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + kSrcStep * x, (int)wv[g][1][d]);
           tg[4 * x + d] = upper ? hi : lo;
         }
       // 32 bytes of k per lane and operand: one v_mfma_f32_16x16x128_f8f6f4 (both formats e4m3, no block scales)
@@ -317,8 +354,16 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
       for (int mt = 0; mt < MT; ++mt) {
         const intx8 aop = {(int)av[mt][0][0], (int)av[mt][0][1], (int)av[mt][0][2], (int)av[mt][0][3],
                            (int)av[mt][1][0], (int)av[mt][1][1], (int)av[mt][1][2], (int)av[mt][1][3]};
-        acc[4 * half + g][mt] =
-            __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc[4 * half + g][mt], 0, 0, 0, 0, 0, 0);
+        if (MX)
+          acc[4 * half + g][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+              wop, aop, acc[4 * half + g][mt], 0, 0, 0, (int)(sbq[buf][g] >> (8 * kb)), 0, (int)(saq[abuf][mt] >> (8 * kb)));
+        else
+          acc[4 * half + g][mt] =
+              __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc[4 * half + g][mt], 0, 0, 0, 0, 0, 0);
+      }
+      if (MX) {  // (with scale operands the compiler otherwise sinks all four groups' MFMAs below their permutes)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(acc[4 * half + g][mt]));
       }
       if (g & 1) __builtin_amdgcn_sched_barrier(0);  // two groups' pieces on their way at a time, not all four
     }
@@ -352,7 +397,7 @@ __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeP
     const float* ws = p.partial + (size_t)batch * p.slices * total + idx;
     float v = 0.0f;
     for (int s = 0; s < p.slices; ++s) v = v + ws[(size_t)s * total];
-    const float alpha = (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+    const float alpha = p.a_block_scales ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
     finish_value(p, batch, (int)(idx / p.N), (int)(idx % p.N), v, alpha, &amax_bits);
   }
   fold_amax(p, amax_bits);
@@ -383,10 +428,16 @@ size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N
 int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const int64_t batch = p.batch > 1 ? p.batch : 1;
   const bool nk = p.rhs_contracting_dim == 1;
+  const bool mx = p.a_block_scales != nullptr;
   const int align = nk ? 16 : 8;  // bytes a lane loads at once
-  // (four token tiles of the [N,K] kernel do not fit the registers of two waves per SIMD: 48 rows there)
-  if (p.M <= 0 || p.M > (nk ? 48 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
-  if (p.a_block_scales || p.b_block_scales || p.dequant_type != XLA_FFI_DataType_F32) return -1;
+  // (four token tiles of the [N,K] kernel do not fit the registers of two waves per SIMD: 48 rows there,
+  // 32 with block scales)
+  if (p.M <= 0 || p.M > (mx ? 32 : nk ? 48 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
+  if (p.dequant_type != XLA_FFI_DataType_F32) return -1;
+  // block scales: a step's four scales of a row move as one dword
+  if (mx && (!nk || p.K % 128 != 0 || ((uintptr_t)p.a_block_scales % 4) || ((uintptr_t)p.b_block_scales % 4) ||
+             (double)p.N * (p.K / 32) >= 2147483000.0))
+    return -1;
   if (((uintptr_t)p.a % align) || ((uintptr_t)p.b % align) || (double)p.K * p.N >= 2147483000.0 || batch > 65535) return -1;
   const bool out_f8 = p.out_dtype == XLA_FFI_DataType_F8E4M3FN;
   Fp8DecodeParams dp{};
@@ -394,6 +445,8 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   dp.b = (const uint8_t*)p.b;
   dp.a_scale = p.a_scale;
   dp.b_scale = p.b_scale;
+  dp.a_block_scales = (const uint8_t*)p.a_block_scales;
+  dp.b_block_scales = (const uint8_t*)p.b_block_scales;
   dp.a_per_row = p.a_scale_per_row != 0;
   dp.b_per_channel = p.b_scale_per_channel != 0;
   dp.bias = (p.epilogue & 1) ? p.bias : nullptr;
@@ -421,10 +474,15 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const int strips = (int)((p.N + 127) / 128);
   dim3 grid((unsigned)(strips * slices), (unsigned)batch);
   if (nk) {
-    switch (mt) {
-      case 1: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<1>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      case 2: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      default: hipLaunchKernelGGL(fp8_dot_decode_nk_kernel<3>, grid, dim3(kWaves * 64), 0, stream, dp); break;
+    if (mx) {
+      if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<1, true>), grid, dim3(kWaves * 64), 0, stream, dp);
+      else hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<2, true>), grid, dim3(kWaves * 64), 0, stream, dp);
+    } else {
+      switch (mt) {
+        case 1: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<1, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
+        case 2: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<2, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
+        default: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<3, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
+      }
     }
   } else {
     switch (mt) {
@@ -444,7 +502,8 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   }
   static const char* names[2][4] = {{"fp8_dot_decode_kn_m16", "fp8_dot_decode_kn_m32", "fp8_dot_decode_kn_m48", "fp8_dot_decode_kn_m64"},
                                     {"fp8_dot_decode_nk_m16", "fp8_dot_decode_nk_m32", "fp8_dot_decode_nk_m48", "fp8_dot_decode_nk_m64"}};
-  SetLastKernel(names[nk ? 1 : 0][mt - 1]);
+  static const char* mx_names[2] = {"fp8_dot_decode_mx_m16", "fp8_dot_decode_mx_m32"};
+  SetLastKernel(mx ? mx_names[mt - 1] : names[nk ? 1 : 0][mt - 1]);
   return 0;
 }
 
