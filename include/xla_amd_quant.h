@@ -265,8 +265,8 @@ XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, vo
 /* Scratch the call can use (0 = none).  A [K,N] rhs whose N is a multiple of 16 goes in as it is;
  * any other [K,N] rhs is re-laid out with K minor first (the transpose GemmRewriter inserts at
  * gemm_rewriter.cc:1235-1591), which takes K*N bytes -- without them such a rhs runs on the slow
- * exact kernel.  Up to 64 rows of a (48 with an [N,K] rhs; K and N multiples of 8, resp. 16 and 8)
- * stream the rhs once instead and, where the channels alone leave CUs idle, split K over workgroups:
+ * exact kernel.  Up to 64 rows of a (48 with an [N,K] rhs, 32 with block scales; K and N multiples
+ * of 8, resp. 16 and 8, K of 128 with block scales) stream the rhs once instead and, where the channels alone leave CUs idle, split K over workgroups:
  * slices * M * N * 4 bytes of f32 sums, per batch -- without them one slice. */
 XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                                              int32_t rhs_contracting_dim);

@@ -197,13 +197,15 @@ def test_mxfp8_module(oracle):
     check_dot(host_bf16(out), ref, dot_floor(ad, bd.T, K) + 1.2 * 2.0 ** -12 * np.sqrt((ad * ad) @ (bd * bd).T), "MXFP8 module")
 
 
+@pytest.mark.parametrize("M,K", [(128, 256), (16, 8192)])
 @pytest.mark.parametrize("batch", [0, 3])
-def test_mxfp8_module_with_bias_gelu(oracle, batch):
+def test_mxfp8_module_with_bias_gelu(oracle, batch, M, K):
     """The block-scaled custom call yielding f32, a bias add, GELU and the convert to bf16 behind it,
     with and without a leading batch dimension: one call after the pass, against the op-by-op
-    evaluation of the original module."""
-    say("module MXFP8 block-scaled dot + bias + GELU, batch=%d" % batch)
-    M, K, N = 128, 256, 96
+    evaluation of the original module.  16 rows take the streaming kernel, K split over workgroups
+    through the scratch the pass asked for."""
+    say("module MXFP8 block-scaled dot + bias + GELU, batch=%d M=%d K=%d" % (batch, M, K))
+    N = 96
     rng = np.random.default_rng(16)
     lead = (batch,) if batch else ()
     a = dtypes.f32_to_f8e4m3fn(np.clip(rng.standard_normal(lead + (M, K)) * 4, -448, 448).astype(np.float32))
@@ -215,7 +217,9 @@ def test_mxfp8_module_with_bias_gelu(oracle, batch):
     out, rw, _ = hlo_runner.compile_and_run(text, [dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), dev_bf16(bias)])
     torch.cuda.synchronize()
     assert rw == ["dot -> xla_amd.fp8_scaled_dot [BIAS_GELU, block scales%s]" % (", batched" if batch else "")]
-    assert ffi.last_kernel() == "fp8_scaled_dot_tiled_mx"
+    assert ffi.last_kernel() == ("fp8_scaled_dot_tiled_mx" if M > 32 else "fp8_dot_decode_mx_m16")
+    if M <= 32:
+        assert ffi.library().xla_amd_fp8_scaled_dot_workspace_bytes(M, K, N, 1) > 0 and "s8[" in hlo.rewrite(text)[0]
     ref = reference(text, [a, b, sa, sb, bias])
     got = host_bf16(out)
     for i in range(max(batch, 1)):

@@ -188,6 +188,12 @@ def test_mxfp8_block_scaled_dot():
     assert rw == ["result -> xla_amd.fp8_scaled_dot [DEFAULT, block scales]"] and rf == []
     check(new, r"bf16\[64,32\]\{1,0\} custom-call\(%lhs, %rhs, %lhs_scale, %rhs_scale\), custom_call_target=\"xla_amd.fp8_scaled_dot\"",
           r"rhs_contracting_dim = 1 : i64")
+    # few rows of lhs: the streaming kernel's K-slices get their scratch (f32 sums, per batch)
+    for batch in (0, 3):
+        new, rw, rf = hlo.rewrite(hm.mxfp8_block_scaled_dot(16, 4096, 512, batch=batch))
+        assert len(rw) == 1 and rf == []
+        m = re.search(r"\(bf16\[(?:3,)?16,512\]\{[0-9,]+\}, s8\[(\d+)\]\{0\}\) custom-call\(", new)
+        assert m and int(m.group(1)) % (16 * 512 * 4 * max(batch, 1)) == 0 and int(m.group(1)) > 0, new
     new, rw, rf = hlo.rewrite(hm.mxfp8_block_scaled_dot(64, 256, 32, batch=3))
     assert rw == ["result -> xla_amd.fp8_scaled_dot [DEFAULT, block scales, batched]"] and rf == []
     check(new, r"bf16\[3,64,32\]\{2,1,0\} custom-call\(%lhs, %rhs, %lhs_scale, %rhs_scale\), custom_call_target=\"xla_amd.fp8_scaled_dot\"")

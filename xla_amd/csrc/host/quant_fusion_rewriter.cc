@@ -471,7 +471,7 @@ bool RewriteF8Dot(const Module& mod, Computation* comp, Instr* dot, const Rewrit
 // (block_scaling_rewriter.h:48-69) becomes xla_amd.fp8_scaled_dot with the scales as they are:
 // the matrix cores multiply them in.  BlockScalingRewriter would expand it into converts,
 // multiplies and a dot on anything but cuDNN (block_scaling_rewriter.cc:548-571).
-bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
+bool RewriteBlockScaledDot(Computation* comp, Instr* cc, const RewriteOptions& opt, RewriteLog* log) {
   const std::string* target = cc->Attr("custom_call_target");
   if (!target || *target != "\"__op$block_scaled_dot\"") return false;
   auto refuse = [&](const std::string& why) {
@@ -510,8 +510,14 @@ bool RewriteBlockScaledDot(Computation* comp, Instr* cc, RewriteLog* log) {
   std::vector<Instr*> ops = {a, b, sa, sb};
   if (ep.bias) ops.push_back(ep.bias);
   std::string cfg = CommonConfig(ep, "f32", cc->shape.dtype) + ", rhs_contracting_dim = 1 : i64";
-  Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, {Shape::Array("bf16", out_dims)}, cfg);
-  comp->ReplaceAllUses(ep.tail, call);
+  std::vector<Shape> results = {Shape::Array("bf16", out_dims)};
+  // scratch: the f32 sums of the K-slices of the kernels that take few rows of lhs, per batch
+  size_t ws = opt.fp8_workspace_bytes ? opt.fp8_workspace_bytes(M, K, N, 1, DTypeCode("f32")) : 0;
+  if (lead) ws *= (size_t)a->shape.dims[0];
+  if (ws) results.push_back(Shape::Array("s8", {(int64_t)ws}));
+  Instr* call = EmitCall(comp, ep.tail, "xla_amd.fp8_scaled_dot", ops, results, cfg);
+  Instr* value = results.size() > 1 ? EmitGte(comp, call, 0, ep.tail, ep.tail->name + ".out") : call;
+  comp->ReplaceAllUses(ep.tail, value);
   log->rewrites.push_back(cc->name + " -> xla_amd.fp8_scaled_dot [" + ep.Name() + ", block scales" +
                           (lead ? ", batched" : "") + "]");
   return true;
@@ -910,7 +916,7 @@ int RunQuantFusionRewriter(Module* mod, const RewriteOptions& opt, RewriteLog* l
         } else if (i->Is("ragged-dot") && i->operands.size() == 3) {
           did = RewriteRaggedDequantDot(comp.get(), i, log);
         } else if (i->Is("custom-call")) {
-          did = RewriteBlockScaledDot(comp.get(), i, log);
+          did = RewriteBlockScaledDot(comp.get(), i, opt, log);
         } else if (i->Is("convert") && i->shape.dtype == "f8e4m3fn") {
           did = RewriteQuantize(*mod, comp.get(), i, log);
         }

@@ -457,8 +457,14 @@ bool RewriteBlockScaledDot(HloComputation* comp, Instr* cc, const std::function<
   std::vector<Instr*> ops = {a, b, sa, sb};
   if (ep.bias) ops.push_back(ep.bias);
   std::string cfg = CommonConfig(ep, F32, Ty(cc)) + ", rhs_contracting_dim = 1 : i64";
-  Instr* call = EmitCall(comp, "xla_amd.fp8_scaled_dot", ops, {ShapeUtil::MakeShape(BF16, out_dims)}, cfg);
-  CHECK_OK(ep.tail->ReplaceAllUsesWith(call));
+  std::vector<Shape> results = {ShapeUtil::MakeShape(BF16, out_dims)};
+  // scratch: the f32 sums of the K-slices of the kernels that take few rows of lhs, per batch
+  size_t ws = xla_amd_fp8_scaled_dot_workspace_bytes_typed(M, K, N, 1, (int32_t)F32);
+  if (lead) ws *= (size_t)a->shape().dimensions(0);
+  if (ws) results.push_back(ShapeUtil::MakeShape(S8, {(int64_t)ws}));
+  Instr* call = EmitCall(comp, "xla_amd.fp8_scaled_dot", ops, results, cfg);
+  Instr* value = results.size() > 1 ? EmitGte(comp, call, 0) : call;
+  CHECK_OK(ep.tail->ReplaceAllUsesWith(value));
   VLOG(1) << cc->name() << " -> xla_amd.fp8_scaled_dot [" << ep.Name() << ", block scales" << (lead ? ", batched" : "")
           << "]";
   return true;
