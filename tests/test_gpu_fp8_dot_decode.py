@@ -73,6 +73,32 @@ def test_k_slices(oracle, slices, nk):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("mode", ["kn", "nk", "mx"])
+@pytest.mark.parametrize("cols", [2, 3])
+def test_workgroups_that_walk_several_strips(oracle, mode, cols):
+    """More strips than CUs: a workgroup takes `cols` strips in turn (forced here on five strips, the
+    last one short and, with three per workgroup, the second workgroup's walk ending early); with
+    K-slices beside it."""
+    from tests.test_gpu_fp8_dot import mx_case, mx_floor
+    say("fp8 streaming, %d strips per workgroup, %s" % (cols, mode))
+    M, K, N = 24, 1024, 584
+    ffi.set_option("fp8_decode_cols", cols)
+    try:
+        for slices in (0, 2):
+            if mode == "mx":
+                a, b, sa, sb = mx_case(M, K, N, 9)
+                got, kern = run_mx(a, b, sa, sb, slices=slices)
+                assert kern == "fp8_dot_decode_mx_m32:walk", kern
+                check_dot(got, oracle.block_scaled_dot(a, b, sa, sb), mx_floor(a, b, sa, sb, False), kern)
+            else:
+                w = workloads.c3_fp8(M, K, N)
+                out, kern = run(w, nk=mode == "nk", slices=slices)
+                assert kern == tile_name(mode == "nk", M) + ":walk", kern
+                check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    finally:
+        ffi.set_option("fp8_decode_cols", 0)
+
+
 def test_the_launcher_splits_k_for_narrow_results(oracle):
     say("fp8 streaming, the launcher's own slices")
     M, K, N = 16, 4096, 512

@@ -26,6 +26,7 @@
 // Bound: HBM.  Algorithmic bytes: K*N (rhs) + a, scales, bias and out once each.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include "decode_common.h"
 #include "device_numerics.h"
@@ -53,6 +54,7 @@ struct Fp8DecodeParams {
   int a_per_row, b_per_channel, bias_is_bf16, d_divides;
   int bf16_dot, bf16_ops, epilogue;
   int slices, rows_per_slice, rows_per_wave;  // rows_per_wave: a multiple of the kernel's step
+  int cols;                                   // consecutive strips a workgroup takes, one after the other
 };
 
 constexpr int kWaves = 8;
@@ -134,14 +136,13 @@ __device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float
 // rhs [K,N].  MT: 16-token tiles.  A workgroup owns 128 channels (one 128-byte line per row) and
 // rows_per_slice rows, its waves rows_per_wave consecutive rows each, in steps of 32.
 template <int MT>
-__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
-  __shared__ float lds[kWaves * 32 * 64];
-  const int lane = threadIdx.x & 63;
+__device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, int strip, int slice, int batch) {
+  int lane = threadIdx.x & 63;
+  // (opaque to the compiler, so that a strip's descriptors and offsets are made anew for every strip of
+  // a caller's loop instead of staying in registers through the other strips' sums)
+  asm volatile("" : "+v"(lane), "+s"(batch));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4;
-  const int slice = blockIdx.x % p.slices;
-  const int strip = blockIdx.x / p.slices;
-  const int batch = blockIdx.y;
   const int n_lane = strip * 128 + li * 8;
   const uint32_t pitch = (uint32_t)p.N;
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * pitch);
@@ -226,6 +227,24 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8Decod
   reduce_and_store<MT, false>(p, lds, acc, strip, slice, batch);
 }
 
+// WALK: a workgroup takes p.cols consecutive strips one after the other (more strips than CUs: one
+// resident workgroup per CU that walks several strips finishes sooner than workgroups queueing for CUs;
+// a kernel of its own, because the loop costs the one-strip form registers).
+template <int MT, bool WALK>
+__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
+  __shared__ float lds[kWaves * 32 * 64];
+  const int slice = blockIdx.x % p.slices;
+  if constexpr (!WALK) {
+    kn_strip<MT>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
+  } else {
+    const int first = (blockIdx.x / p.slices) * p.cols;
+    for (int c = 0; c < p.cols && (first + c) * 128 < p.N; ++c) {
+      if (c) __syncthreads();  // the sums of the strip before have left LDS
+      kn_strip<MT>(p, lds, first + c, slice, blockIdx.y);
+    }
+  }
+}
+
 // rhs [N,K].  A workgroup owns 128 channels (8 groups of 16) and rows_per_slice values of k, its
 // waves rows_per_wave consecutive ones each, in steps of 128 (one line per channel), a step in two
 // halves of four channel groups.  MX: block scales.  The matrix instruction takes the scale of the
@@ -236,14 +255,11 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8Decod
 // line instead of 2 kb and 2 kb + 1; a step's four scales of a channel (or row of a) are one dword,
 // of which lane (., kb) hands in byte kb.
 template <int MT, bool MX>
-__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
-  __shared__ float lds[kWaves * 32 * 64];
-  const int lane = threadIdx.x & 63;
+__device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, int strip, int slice, int batch) {
+  int lane = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane), "+s"(batch));  // as in kn_strip
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4;
-  const int slice = blockIdx.x % p.slices;
-  const int strip = blockIdx.x / p.slices;
-  const int batch = blockIdx.y;
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(p.b + (size_t)batch * p.K * p.N, (uint32_t)p.K * (uint32_t)p.N);
   __amdgpu_buffer_rsrc_t ra[MT];
 #pragma unroll
@@ -387,6 +403,21 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
   reduce_and_store<MT, true>(p, lds, acc, strip, slice, batch);
 }
 
+template <int MT, bool MX, bool WALK>
+__global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
+  __shared__ float lds[kWaves * 32 * 64];
+  const int slice = blockIdx.x % p.slices;
+  if constexpr (!WALK) {
+    nk_strip<MT, MX>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
+  } else {
+    const int first = (blockIdx.x / p.slices) * p.cols;
+    for (int c = 0; c < p.cols && (first + c) * 128 < p.N; ++c) {
+      if (c) __syncthreads();
+      nk_strip<MT, MX>(p, lds, first + c, slice, blockIdx.y);
+    }
+  }
+}
+
 // Sums the K-slices in slice order and finishes the values.
 __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeParams p) {
   const size_t total = (size_t)p.M * p.N;
@@ -404,15 +435,17 @@ __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeP
 }
 
 // K-slices for the shape: more workgroups until every CU has one, as long as a wave keeps at
-// least 128 values of k (256 for the [N,K] kernel, two of its steps) and the sums written and read
-// again stay under a quarter of the rhs bytes.
+// least 128 values of k (four steps, or one of the [N,K] kernel) and the sums written and read
+// again stay under a quarter of the rhs bytes.  A few workgroups more than CUs are worse than half
+// as many (a second round for a quarter of the work: 80 strips take 19.8 us in 2 slices, 22.1 in 4).
 int Slices(int64_t batch, int64_t M, int64_t K, int64_t N, bool nk) {
   if (int s = GetOption("fp8_decode_slices")) return s;
   const int64_t strips = (N + 127) / 128;
   int slices = 1;
-  while (strips * batch * slices < 192 && slices < 16 && K / (slices * 2) >= (nk ? 256 : 128) * kWaves &&
+  while (strips * batch * slices < 192 && slices < 16 && K / (slices * 2) >= 128 * kWaves &&
          2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * (double)K * N)
     slices *= 2;
+  if (slices > 1 && strips * batch * slices > 256 && strips * batch * slices < 400) slices /= 2;
   return slices;
 }
 
@@ -472,26 +505,38 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   dp.rows_per_wave = ((per + waves - 1) / waves + kStep - 1) / kStep * kStep;
   dp.rows_per_slice = dp.rows_per_wave * waves;
   const int strips = (int)((p.N + 127) / 128);
-  dim3 grid((unsigned)(strips * slices), (unsigned)batch);
-  if (nk) {
-    if (mx) {
-      if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<1, true>), grid, dim3(kWaves * 64), 0, stream, dp);
-      else hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<2, true>), grid, dim3(kWaves * 64), 0, stream, dp);
-    } else {
-      switch (mt) {
-        case 1: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<1, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
-        case 2: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<2, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
-        default: hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<3, false>), grid, dim3(kWaves * 64), 0, stream, dp); break;
-      }
-    }
-  } else {
-    switch (mt) {
-      case 1: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<1>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      case 2: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<2>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      case 3: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<3>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-      default: hipLaunchKernelGGL(fp8_dot_decode_kn_kernel<4>, grid, dim3(kWaves * 64), 0, stream, dp); break;
-    }
+  // more work items than CUs: a workgroup walks `cols` strips, as long as that leaves about 200 workgroups
+  int cols = 1;
+  const int64_t items = (int64_t)strips * slices * batch;
+  if (items > 256) {
+    const int c = (int)((items + 255) / 256);
+    if ((strips + c - 1) / c * slices * batch >= 192) cols = c;
   }
+  // (three token tiles of the walking [N,K] kernel spill: one strip per workgroup there)
+  if (nk && !mx && mt >= 3) cols = 1;
+  if (int c = GetOption("fp8_decode_cols")) cols = c;
+  dp.cols = cols;
+  const dim3 grid((unsigned)((strips + cols - 1) / cols * slices), (unsigned)batch);
+  const dim3 block(kWaves * 64);
+#define XLA_AMD_LAUNCH_FP8_DECODE(KERNEL, ...)                                                      \
+  do {                                                                                              \
+    if (cols > 1) hipLaunchKernelGGL((KERNEL<__VA_ARGS__, true>), grid, block, 0, stream, dp);      \
+    else hipLaunchKernelGGL((KERNEL<__VA_ARGS__, false>), grid, block, 0, stream, dp);              \
+  } while (0)
+  if (nk && mx) {
+    if (mt == 1) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 1, true);
+    else XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 2, true);
+  } else if (nk) {
+    if (mt == 1) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 1, false);
+    else if (mt == 2) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 2, false);
+    else XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 3, false);
+  } else {
+    if (mt == 1) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_kn_kernel, 1);
+    else if (mt == 2) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_kn_kernel, 2);
+    else if (mt == 3) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_kn_kernel, 3);
+    else XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_kn_kernel, 4);
+  }
+#undef XLA_AMD_LAUNCH_FP8_DECODE
   int rc = CheckLaunch("fp8_dot_decode");
   if (rc) return rc;
   if (slices > 1) {
@@ -503,7 +548,9 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   static const char* names[2][4] = {{"fp8_dot_decode_kn_m16", "fp8_dot_decode_kn_m32", "fp8_dot_decode_kn_m48", "fp8_dot_decode_kn_m64"},
                                     {"fp8_dot_decode_nk_m16", "fp8_dot_decode_nk_m32", "fp8_dot_decode_nk_m48", "fp8_dot_decode_nk_m64"}};
   static const char* mx_names[2] = {"fp8_dot_decode_mx_m16", "fp8_dot_decode_mx_m32"};
-  SetLastKernel(mx ? mx_names[mt - 1] : names[nk ? 1 : 0][mt - 1]);
+  char name[48];
+  snprintf(name, sizeof(name), "%s%s", mx ? mx_names[mt - 1] : names[nk ? 1 : 0][mt - 1], cols > 1 ? ":walk" : "");
+  SetLastKernel(name);
   return 0;
 }
 
