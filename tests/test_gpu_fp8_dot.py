@@ -525,3 +525,83 @@ def test_fp8_error_paths():
     with pytest.raises(ffi.FfiError, match="rhs_contracting_dim"):
         ops.fp8_scaled_dot(a, torch.zeros((32, 16), dtype=torch.uint8, device="cuda"), one, one,
                            rhs_contracting_dim=2)
+
+
+# ---- tiles of a last round that is at most a quarter full run as two workgroups along K ------------------
+
+def _split_case(mode):
+    M, K, N = 300, 2304, 272        # 2 x 2 tiles, 18 stages of 128: halves of 9 stages each
+    if mode == "mx":
+        return mx_case(M, K, N, 17)
+    w = workloads.c3_fp8(M, K, N)
+    if mode == "vector_scales":
+        rng = np.random.default_rng(8)
+        w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+        w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    return w
+
+
+@pytest.mark.parametrize("mode", ["kn", "nk", "vector_scales", "mx", "f8_result"])
+@pytest.mark.parametrize("drop_flags", [False, True])
+def test_last_round_split_along_k(oracle, mode, drop_flags):
+    """Few tiles and a long K: every tile is two workgroups, the one on the second half of K hands its sums
+    over.  drop_flags: that workgroup never raises its flag, the other gives up after a few polls and does
+    the second half itself (every kernel exits normally); the next ordinary call on the same scratch
+    must give the ordinary result bit for bit.  Unsplit tiles (option "tiled_tail" = 1) sum K in the order
+    the give-up path uses."""
+    say("fp8_scaled_dot split last round, %s, drop_flags=%s" % (mode, drop_flags))
+    scratch = torch.empty(4 << 20, dtype=torch.uint8, device="cuda")
+    case = _split_case(mode)
+
+    def once(drop=False, whole=False):
+        ffi.set_option("handover_test", 1 if drop else 0)
+        ffi.set_option("tiled_tail", 1 if whole else 0)
+        try:
+            if mode == "mx":
+                a, b, sa, sb = case
+                out = ops.fp8_scaled_dot(dev_u8(a), dev_u8(b), dev_u8(sa), dev_u8(sb), rhs_contracting_dim=1, scratch=scratch)
+            elif mode == "f8_result":
+                out, amax = ops.fp8_scaled_dot(dev_u8(case["a"]), dev_u8(case["b"]), s64, s64, dev_bf16(case["bias"]),
+                                               epilogue="BIAS_GELU", d_scale=dev_f32(np.array(z, np.float32)), amax=True,
+                                               scratch=scratch)
+                torch.cuda.synchronize()
+                return (out.cpu().numpy(), float(amax)), ffi.last_kernel()
+            else:
+                nk = mode == "nk"
+                out = ops.fp8_scaled_dot(dev_u8(case["a"]), dev_u8(np.ascontiguousarray(case["b"].T) if nk else case["b"]),
+                                         dev_f32(np.array(case["a_scale"], np.float32)), dev_f32(np.array(case["b_scale"], np.float32)),
+                                         dev_bf16(case["bias"]), rhs_contracting_dim=1 if nk else 0, epilogue="BIAS_GELU",
+                                         scratch=scratch)
+            torch.cuda.synchronize()
+            return host_bf16(out), ffi.last_kernel()
+        finally:
+            ffi.set_option("handover_test", 0)
+            ffi.set_option("tiled_tail", 0)
+
+    s64, z = dev_f32(np.array(1 / 64, np.float32)), np.float32(0.0117)
+    normal, kern = once()
+    assert kern.endswith(":tail2"), kern
+    got, kern = once(drop=drop_flags)
+    assert kern.endswith(":tail2"), kern
+    if mode == "mx":
+        a, b, sa, sb = case
+        check_dot(got, oracle.block_scaled_dot(a, b, sa, sb), mx_floor(a, b, sa, sb, False), kern)
+    elif mode == "f8_result":
+        ref, val = oracle.fp8_scaled_dot(case["a"], case["b"], 1 / 64, 1 / 64, bias=case["bias"], epilogue="gelu_tanh", d_scale=z)
+        check_f8_result(got[0], ref, val, z, True, floor_for(case), kern)
+        want = float(np.max(np.abs(val)))
+        assert abs(got[1] - want) <= want * 2.0 ** -7
+    else:
+        check_dot(got, reference(oracle, case), floor_for(case), kern)
+    if drop_flags:
+        whole, kern = once(whole=True)
+        assert not kern.endswith(":tail2"), kern
+        if mode == "f8_result":
+            assert np.array_equal(got[0], whole[0]) and got[1] == whole[1]
+        else:
+            assert np.array_equal(got, whole)
+    again, _ = once()
+    if mode == "f8_result":
+        assert np.array_equal(again[0], normal[0]) and again[1] == normal[1]
+    else:
+        assert np.array_equal(again, normal)

@@ -27,6 +27,7 @@
 // Algorithmic flops: 2*M*N*K per batch.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdio.h>
 
 #include <atomic>
 #include <type_traits>
@@ -236,7 +237,10 @@ __device__ __forceinline__ uint32_t drain_dispatch(const DrainArgs& d, int act, 
   return 0u;
 }
 
-template <int KIND, bool OUT_F8>
+// SPLIT: the kernel can run tiles as two workgroups along K (tail_tiles > 0).  The integer-weight
+// kinds always can; for the f8 kinds that is an instantiation of its own, because the one-workgroup
+// form has no register to spare (254) for it.
+template <int KIND, bool OUT_F8, bool SPLIT>
 __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr bool WQ = KIND == kS8 || KIND == kS4 || KIND == kU4 || KIND == kS8NK || KIND == kS4NK;  // integer weights, dequantised on the way into LDS
   constexpr bool W4 = KIND == kS4 || KIND == kU4 || KIND == kS4NK;   // two weights per byte, bf16 group scales
@@ -271,7 +275,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   int role = 0;       // 0: all of K; 1: second half of K, hands over; 2: first half of K, finishes
   int tail_slot = 0;
   const int tiles_per_batch = p.tiles_m * p.tiles_n;  // == gridDim.x unless the tail is split
-  if (WQ && p.tail_tiles > 0) {
+  if (SPLIT && p.tail_tiles > 0) {
     int t = blockIdx.x;
     if (t >= p.tail_first) {
       t -= p.tail_first;
@@ -284,7 +288,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   }
   const bool waited_for_tail = role == 2;  // (the role changes if the wait gives up)
   unsigned long long tail_target = 0;      // what the slot's raised flag holds in this run
-  if (WQ && role != 0 && threadIdx.x == 0) tail_target = HandOverTarget(p.epoch, p.tail_flags + 2 * tail_slot + 1);
+  if (SPLIT && role != 0 && threadIdx.x == 0) tail_target = HandOverTarget(p.epoch, p.tail_flags + 2 * tail_slot + 1);
   const bool ragged = WQ && p.group_sizes != nullptr;
   int m0r = 0, m_limit = p.M;  // ragged: first row of the tile and the end of its group's rows
   if (ragged) {
@@ -787,7 +791,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads issued past the end have landed
     __syncthreads();  // the epilogue (or another pass of this loop) reuses the stage buffers
-    if (!WQ || role != 2) break;
+    if (!SPLIT || role != 2) break;
     // first half done: wait (bounded) for the second half's flag.  That workgroup has a lower id,
     // so it was dispatched before this one and is running or done.
     if (tid == 0) {
@@ -809,8 +813,8 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   constexpr int kDeviceScope = 16;  // sc1: performed where every XCD sees it
   const __amdgpu_buffer_rsrc_t rt =
       tile_rsrc(reinterpret_cast<const uint8_t*>(p.tail_sums) + (size_t)tail_slot * kTailSumsBytes,
-                WQ && (role == 1 || add_sums) ? (uint32_t)kTailSumsBytes : 0u);
-  if (WQ && role == 1) {
+                SPLIT && (role == 1 || add_sums) ? (uint32_t)kTailSumsBytes : 0u);
+  if (SPLIT && role == 1) {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -881,45 +885,62 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   }
   d.n_vec = n_vec;
   d.has_bias = p.bias != nullptr;
+  float row_scale[4] = {1.0f, 1.0f, 1.0f, 1.0f};
   if (F8 && !MX && p.a_per_row) {
     // one scale per token row: all 16 registers of a tile belong to the lane's one token
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       const int m = m0 + wm * 128 + mt * 32 + l32;
       const float rs = p.a_scale[m < p.M ? m : p.M - 1];
+      row_scale[mt] = rs;
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) acc[nt][mt] *= rs;
     }
   }
 #pragma unroll
   for (int pass = 0; pass < 2; ++pass) {
-    if (WQ && add_sums) {
-      // the other half of K: this pass's 16 chunks are fetched together and added on the way into LDS
-      // (first half + second half), so the accumulators themselves are never rewritten
-      uintx4 o[2][2][4];
-#pragma unroll
-      for (int mtl = 0; mtl < 2; ++mtl)
+    if (SPLIT && add_sums) {
+      // the other half of K: a pass's 16 chunks are fetched together (8 and 8 by the f8 kinds, which
+      // have fewer registers free) and added on the way into LDS (first half + second half), so the
+      // accumulators themselves are never rewritten (with one scale per row of a the accumulators
+      // already carry it and the fetched sums take it here)
+      auto fetch = [&](int mtl, uintx4 (&o)[2][4]) {
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
           for (int vq = 0; vq < 4; ++vq)
-            o[mtl][nt][vq] = __builtin_amdgcn_raw_buffer_load_b128(
+            o[nt][vq] = __builtin_amdgcn_raw_buffer_load_b128(
                 rt, (uint32_t)((((nt * 4 + pass * 2 + mtl) * 4 + vq) * 512 + tid) * 16), 0, kDeviceScope);
-#pragma unroll
-      for (int mtl = 0; mtl < 2; ++mtl) {
+      };
+      auto add_and_stage = [&](int mtl, const uintx4 (&o)[2][4]) {
         const int m = mtl * 32 + l32;
+        const float rs = F8 && !MX ? row_scale[pass * 2 + mtl] : 1.0f;
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
           for (int vq = 0; vq < 4; ++vq) {
             const int c = nt * 8 + vq * 2 + kb;
             const floatx16& a = acc[nt][pass * 2 + mtl];
-            const uintx4& q = o[mtl][nt][vq];
-            const floatx4 v = {a[vq * 4] + bits_to_f32(q[0]), a[vq * 4 + 1] + bits_to_f32(q[1]),
-                               a[vq * 4 + 2] + bits_to_f32(q[2]), a[vq * 4 + 3] + bits_to_f32(q[3])};
+            const uintx4& q = o[nt][vq];
+            const floatx4 v = {a[vq * 4] + bits_to_f32(q[0]) * rs, a[vq * 4 + 1] + bits_to_f32(q[1]) * rs,
+                               a[vq * 4 + 2] + bits_to_f32(q[2]) * rs, a[vq * 4 + 3] + bits_to_f32(q[3]) * rs};
             *reinterpret_cast<floatx4*>(stage + m * 64 + ((c ^ (m & 15)) << 2)) = v;
           }
         }
+      };
+      if constexpr (WQ) {
+        uintx4 o0[2][4], o1[2][4];
+        fetch(0, o0);
+        fetch(1, o1);
+        add_and_stage(0, o0);
+        add_and_stage(1, o1);
+      } else {
+        uintx4 o[2][4];
+        fetch(0, o);
+        add_and_stage(0, o);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(1, o);
+        add_and_stage(1, o);
       }
     } else {
 #pragma unroll
@@ -942,7 +963,7 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   }
   // the slot moves on to its next generation, whether the flag showed or not: the next run (also a
   // replay of this launch from a captured graph) waits for new sums
-  if (WQ && waited_for_tail && tid == 0) HandOverNextGeneration(p.tail_flags + 2 * tail_slot + 1, tail_target);
+  if (SPLIT && waited_for_tail && tid == 0) HandOverNextGeneration(p.tail_flags + 2 * tail_slot + 1, tail_target);
   if (OUT_F8 && p.amax) {  // one atomic per wave into the result a fill kernel zeroed
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, off));
@@ -1112,8 +1133,8 @@ __global__ __launch_bounds__(256) void ragged_tail_rows_kernel(TiledParams p) {
   for (long long m = start + blockIdx.y; m < p.M; m += gridDim.y) p.out[(size_t)m * p.N + n] = v;
 }
 
-template <int KIND, bool OUT_F8 = false>
-int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
+template <int KIND, bool OUT_F8, bool SPLIT>
+int launch_tiled_form(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
   constexpr size_t kLds = 2 * (size_t)(kTM + kTN) * kRow + (KIND == kFp8MX ? 4096 : 0);  // 128 KiB (+ scales)
   // per kernel instantiation and device: one bit per device ordinal; two threads that race both set
   // the attribute to the same value, which is harmless, and neither launches before it is set
@@ -1122,7 +1143,7 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
   (void)hipGetDevice(&device);
   const unsigned long long bit = 1ull << (device & 63);
   if (!(configured.load(std::memory_order_acquire) & bit)) {
-    hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND, OUT_F8>,
+    hipError_t e = hipFuncSetAttribute((const void*)tiled_dot_kernel<KIND, OUT_F8, SPLIT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLds);
     if (e != hipSuccess)
       return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", what, kLds,
@@ -1131,8 +1152,19 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
   }
   dim3 grid((unsigned)(tp.tiles_m * tp.tiles_n), (unsigned)batch);
   if (tp.tail_tiles > 0) grid = dim3((unsigned)(tp.tail_first + 2 * tp.tail_tiles), 1u);
-  hipLaunchKernelGGL((tiled_dot_kernel<KIND, OUT_F8>), grid, dim3(512), kLds, stream, tp);
+  hipLaunchKernelGGL((tiled_dot_kernel<KIND, OUT_F8, SPLIT>), grid, dim3(512), kLds, stream, tp);
   return CheckLaunch(what);
+}
+
+// The integer-weight kinds have one form, which can split tiles along K; the others a form for each.
+template <int KIND, bool OUT_F8 = false>
+int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const char* what) {
+  constexpr bool WQ = KIND == kS8 || KIND == kS4 || KIND == kU4 || KIND == kS8NK || KIND == kS4NK;
+  if constexpr (WQ) return launch_tiled_form<KIND, OUT_F8, true>(tp, batch, stream, what);
+  else if constexpr (KIND == kBf16) return launch_tiled_form<KIND, OUT_F8, false>(tp, batch, stream, what);
+  else
+    return tp.tail_tiles > 0 ? launch_tiled_form<KIND, OUT_F8, true>(tp, batch, stream, what)
+                             : launch_tiled_form<KIND, OUT_F8, false>(tp, batch, stream, what);
 }
 
 }  // namespace
@@ -1140,13 +1172,19 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
 // Scratch for splitting the tiles of the last round along K: worth it when that round is at most
 // half full and K is long enough for half of it to outweigh the hand-over (256 KiB per tile,
 // written and read once).  0: no split for this shape.
-size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
-  if (batch <= 0 || M <= 64 || K < 2048 || N <= 0) return 0;
+static size_t TailBytesFor(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t min_rows, int64_t max_tail = 128) {
+  if (batch <= 0 || M < min_rows || K < 2048 || N <= 0) return 0;
   const int64_t tiles = batch * ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
   const int64_t tail = tiles % 256;
-  if (tail == 0 || tail > 128 || tiles + tail > 0x7fffffff) return 0;
+  if (tail == 0 || tail > max_tail || tiles + tail > 0x7fffffff) return 0;
   return (size_t)tail * (kTailSumsBytes + 2 * sizeof(unsigned long long));  // sums, flag, generation
 }
+// The f8 kinds' form that can split spills registers in its main loop (the one-workgroup form sits at
+// 254): two spilling workgroups per tile still beat one when a quarter of the CUs or fewer have a
+// tile at all (64 tiles: 88 -> 70 us at K = 8192), not when 112 have one (92 -> 95 us).
+constexpr int64_t kF8MaxTail = 64;
+// (up to 64 rows the integer-weight dots run on the decode kernels)
+size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) { return TailBytesFor(batch, M, K, N, 65); }
 
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
 // (the caller then falls back), 0 on success, or an error code.
@@ -1333,7 +1371,9 @@ size_t Bf16OperandBytes(int64_t M, int64_t K, int64_t N) {
 size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contracting_dim, int dequant_type) {
   const size_t copy = TransposedCopyBytes(K, N, rhs_contracting_dim);
   const size_t ops = dequant_type == XLA_FFI_DataType_BF16 ? Bf16OperandBytes(M, K, N) : 0;
-  const size_t tiled = ops ? RoundUp256(copy) + ops : copy;
+  size_t tiled = ops ? RoundUp256(copy) + ops : copy;
+  // nothing else in the scratch: the tiles of a last round at most half full split along K (f32 sums)
+  if (!tiled) tiled = TailBytesFor(1, M, K, N, 1, kF8MaxTail);
   // up to 64 rows of a under f32-typed multiplies: the streaming kernels' K-slices instead
   const size_t decode = dequant_type == XLA_FFI_DataType_BF16 ? 0 : Fp8DotDecodeWorkspaceBytes(1, M, K, N, rhs_contracting_dim);
   return tiled > decode ? tiled : decode;
@@ -1519,6 +1559,20 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     TiledParams tt = tp;
     tt.b = b_nk;
     int rc;
+    // the last round of 256 workgroups, when at most half full, runs as two workgroups per tile (the
+    // scratch then holds nothing else: no transposed copy, no bf16 operands)
+    const size_t tail_need = (nk || kn_direct) && !deq_bf16 ? TailBytesFor(batch, p.M, p.K, p.N, 1, kF8MaxTail) : 0;
+    if (tail_need && GetOption("tiled_tail") != 1 && p.workspace && ((uintptr_t)p.workspace % 16) == 0 &&
+        p.workspace_bytes >= tail_need) {
+      const int64_t tiles = (int64_t)batch * tt.tiles_m * tt.tiles_n;
+      tt.tail_tiles = (int)(tiles % 256);
+      tt.tail_first = (int)(tiles - tt.tail_tiles);
+      tt.tail_sums = (float*)p.workspace;
+      tt.tail_flags = (unsigned long long*)((char*)p.workspace + (size_t)tt.tail_tiles * kTailSumsBytes);
+      tt.epoch = NextHandOverEpoch();
+      tt.handover_test = GetOption("handover_test");
+    }
+    const char* const split = tt.tail_tiles ? ":tail2" : "";
     if (mx)
       rc = launch_tiled<kFp8MX>(tt, batch, stream, "fp8_scaled_dot_tiled_mx");
     else if (out_f8)
@@ -1534,12 +1588,13 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       rc = CheckLaunch("fp8_scaled_dot_exact");
       if (rc) return rc;
     }
-    if (mx)
-      SetLastKernel("fp8_scaled_dot_tiled_mx");
-    else if (out_f8)
-      SetLastKernel(nk ? "fp8_scaled_dot_tiled_f8" : kn_direct ? "fp8_scaled_dot_tiled_kn_f8" : "fp8_scaled_dot_tiled+transpose_f8");
-    else
-      SetLastKernel(nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose");
+    char name[64];
+    snprintf(name, sizeof(name), "%s%s",
+             mx       ? "fp8_scaled_dot_tiled_mx"
+             : out_f8 ? (nk ? "fp8_scaled_dot_tiled_f8" : kn_direct ? "fp8_scaled_dot_tiled_kn_f8" : "fp8_scaled_dot_tiled+transpose_f8")
+                      : (nk ? "fp8_scaled_dot_tiled" : kn_direct ? "fp8_scaled_dot_tiled_kn" : "fp8_scaled_dot_tiled+transpose"),
+             split);
+    SetLastKernel(name);
     return 0;
   }
   hipLaunchKernelGGL(fp8_dot_exact_kernel, egrid, dim3(256), 0, stream, tp, nk ? 1 : 0, deq_bf16 ? 1 : 0, 0);
