@@ -1373,7 +1373,8 @@ size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contr
   const size_t ops = dequant_type == XLA_FFI_DataType_BF16 ? Bf16OperandBytes(M, K, N) : 0;
   size_t tiled = ops ? RoundUp256(copy) + ops : copy;
   // nothing else in the scratch: the tiles of a last round at most half full split along K (f32 sums)
-  if (!tiled) tiled = TailBytesFor(1, M, K, N, 1, kF8MaxTail);
+  // (up to 64 rows the streaming kernels take the call, with the few exceptions that stay unsplit)
+  if (!tiled) tiled = TailBytesFor(1, M, K, N, 65, kF8MaxTail);
   // up to 64 rows of a under f32-typed multiplies: the streaming kernels' K-slices instead
   const size_t decode = dequant_type == XLA_FFI_DataType_BF16 ? 0 : Fp8DotDecodeWorkspaceBytes(1, M, K, N, rhs_contracting_dim);
   return tiled > decode ? tiled : decode;
@@ -1561,7 +1562,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     int rc;
     // the last round of 256 workgroups, when at most half full, runs as two workgroups per tile (the
     // scratch then holds nothing else: no transposed copy, no bf16 operands)
-    const size_t tail_need = (nk || kn_direct) && !deq_bf16 ? TailBytesFor(batch, p.M, p.K, p.N, 1, kF8MaxTail) : 0;
+    const size_t tail_need = (nk || kn_direct) && !deq_bf16 ? TailBytesFor(batch, p.M, p.K, p.N, 65, kF8MaxTail) : 0;
     if (tail_need && GetOption("tiled_tail") != 1 && p.workspace && ((uintptr_t)p.workspace % 16) == 0 &&
         p.workspace_bytes >= tail_need) {
       const int64_t tiles = (int64_t)batch * tt.tiles_m * tt.tiles_n;
