@@ -1172,16 +1172,18 @@ int launch_tiled(const TiledParams& tp, int batch, hipStream_t stream, const cha
 // Scratch for splitting the tiles of the last round along K: worth it when that round is at most
 // half full and K is long enough for half of it to outweigh the hand-over (256 KiB per tile,
 // written and read once).  0: no split for this shape.
-static size_t TailBytesFor(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t min_rows, int64_t max_tail = 128) {
+// max_tiles: the most tiles the whole call may have (the f8 kinds split only calls that are all tail)
+static size_t TailBytesFor(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t min_rows, int64_t max_tiles = 0x7fffffff) {
   if (batch <= 0 || M < min_rows || K < 2048 || N <= 0) return 0;
   const int64_t tiles = batch * ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
   const int64_t tail = tiles % 256;
-  if (tail == 0 || tail > max_tail || tiles + tail > 0x7fffffff) return 0;
+  if (tail == 0 || tail > 128 || tiles > max_tiles || tiles + tail > 0x7fffffff) return 0;
   return (size_t)tail * (kTailSumsBytes + 2 * sizeof(unsigned long long));  // sums, flag, generation
 }
-// The f8 kinds' form that can split spills registers in its main loop (the one-workgroup form sits at
-// 254): two spilling workgroups per tile still beat one when a quarter of the CUs or fewer have a
-// tile at all (64 tiles: 88 -> 70 us at K = 8192), not when 112 have one (92 -> 95 us).
+// The f8 kinds' form that can split spills registers (the one-workgroup form sits at 254), which costs
+// every tile of a launch: two spilling workgroups per tile still beat one when a quarter of the CUs or
+// fewer have a tile at all (64 tiles: 88 -> 70 us at K = 8192), not when 112 have one (92 -> 95 us),
+// and never when whole tiles run in the same launch.
 constexpr int64_t kF8MaxTail = 64;
 // (up to 64 rows the integer-weight dots run on the decode kernels)
 size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) { return TailBytesFor(batch, M, K, N, 65); }
