@@ -352,7 +352,8 @@ def test_c1_full_size(oracle):
 
 
 @pytest.mark.parametrize("M,vec,slices,deq", [(5, 16, 2, "f32"), (16, 8, 1, "f32"), (24, 8, 2, "f32"),
-                                              (64, 4, 1, "f32"), (7, 16, 1, "bf16"), (40, 4, 2, "bf16")])
+                                              (64, 4, 1, "f32"), (7, 16, 1, "bf16"), (40, 4, 2, "bf16"),
+                                              (48, 8, 1, "f32"), (64, 8, 2, "f32"), (40, 0, 0, "f32"), (64, 0, 0, "f32")])
 def test_s8_decode_variants(oracle, M, vec, slices, deq):
     say("dequant_dot s8 variants M=%d vec=%d slices=%d deq=%s" % (M, vec, slices, deq))
     w = workloads.c1_s8_channel(M=M, K=1024, N=640)
@@ -906,7 +907,7 @@ def test_ragged_dot_more_than_64_rows(oracle, M, K, N, G, sizes):
     say("dequant_dot ragged prefill M=%d K=%d N=%d G=%d sizes=%s" % (M, K, N, G, sizes))
     w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
     got, kern = run_ragged(w)
-    assert kern == "dequant_dot_decode_s8_v4_m64_factored", kern
+    assert kern == "dequant_dot_decode_s8_v8_m64_factored", kern
     ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
     check_dot(got, ref, ragged_floor(w), "ragged prefill %s" % kern)
     start = 0

@@ -83,14 +83,18 @@ def test_static_scratch_matches_workspace_launcher(oracle):
 
 def test_static_scratch_refuses_oversized_partial_sums():
     L = ffi.library()
-    # 64 tokens on 40 strips of a long K: eight K-slices of f32 partial sums, 10 MiB
+    # 64 tokens on 40 strips of a long K, cut into eight K-slices: 10 MiB of f32 partial sums
     M, K, N = 64, 32768, 5120
-    need = L.xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S4)
-    assert need > 8 << 20, need
-    t = torch.zeros(16, dtype=torch.uint8, device="cuda")
-    p = _params(t, t, t, None, t, M, K, N, 128, dtypes.S4, dtypes.BF16, dtypes.BF16, "DEFAULT")
-    rc = L.xla_amd_launch_dequant_dot_static_scratch(C.byref(p), torch.cuda.current_stream().cuda_stream)
-    assert rc == 8 and b"static scratch holds" in L.xla_amd_last_error()
+    ffi.set_option("dequant_dot_slices", 8)
+    try:
+        need = L.xla_amd_dequant_dot_workspace_bytes(1, M, K, N, dtypes.S4)
+        assert need > 8 << 20, need
+        t = torch.zeros(16, dtype=torch.uint8, device="cuda")
+        p = _params(t, t, t, None, t, M, K, N, 128, dtypes.S4, dtypes.BF16, dtypes.BF16, "DEFAULT")
+        rc = L.xla_amd_launch_dequant_dot_static_scratch(C.byref(p), torch.cuda.current_stream().cuda_stream)
+        assert rc == 8 and b"static scratch holds" in L.xla_amd_last_error()
+    finally:
+        ffi.set_option("dequant_dot_slices", 0)
 
 
 def test_static_scratch_with_weights_stored_k_minor(oracle):

@@ -566,16 +566,17 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
 // and a second launch); up to four tokens a second slice still pays.  Fewer strips are split
 // until there are, as long as a wave keeps at least four 32-row steps and the partial sums
 // (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or a quarter
-// of the weight bytes when the strips would leave three quarters of the CUs idle.
+// of the weight bytes (s8 [64,8192] x [8192,8192]: 44 us in one slice, 30 in two; K = 28672: 140 -> 80).
 int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
   if (int s = GetOption("dequant_dot_slices")) return s;
   const int64_t want = M <= 4 ? 448 : 192;
   const double weight_bytes = (double)K * row_bytes;
   int slices = 1;
   while (strips * slices * batch < want && K / (slices * 2) >= 128 * waves &&
-         (slices * 2 * M <= 32 ||
-          (strips * batch <= 64 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes)))
+         (slices * 2 * M <= 32 || 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes))
     slices *= 2;
+  // a few workgroups more than CUs are worse than half as many: a second round for a quarter of the work
+  if (want == 192 && slices > 1 && strips * batch * slices > 256 && strips * batch * slices < 400) slices /= 2;
   return slices;
 }
 
@@ -590,6 +591,12 @@ static size_t DecodeWorkspaceBytesUpTo64(int64_t batch, int64_t M, int64_t K, in
   const int64_t row_bytes = N * (s4 ? 1 : 2) / 2;
   const int strips = (int)((N + 16 * nv - 1) / (16 * nv));
   size_t bytes = DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, strips, row_bytes, 8));
+  // (s8 from 33 tokens on: per-channel scales under an f32 multiply take 128-channel strips, whose
+  // fewer workgroups may be split further; the mode is not known here, the larger need decides)
+  if (!s4 && mt >= 3 && !GetOption("dequant_dot_vec")) {
+    const size_t wide = DequantDotWorkspaceBytes(batch, M, N, DecodeSlices(batch, M, K, N, (int)((N + 127) / 128), row_bytes, 8));
+    if (wide > bytes) bytes = wide;
+  }
   // s4 up to 16 tokens may run as two workgroups per 256-channel strip that hand over through the
   // workspace (the group size is not known here: the smallest one that path takes decides)
   if (s4 && S4xPairShape(batch, M, K, N, 64)) bytes = bytes > S4xPairWorkspaceBytes(batch, M, N) ? bytes : S4xPairWorkspaceBytes(batch, M, N);
@@ -759,8 +766,10 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : M <= 48 ? 3 : 4;  // 16-token tiles
     // Narrow strips (4 bytes of s4 = 8 channels, 8 bytes of s8 per lane) measured fastest on
     // MI355X: the loop is bound by the dequantising VALU work, not by load width, and narrow
-    // strips give more workgroups to spread over the 256 CUs.
-    int vec = s4 ? 4 : (mt >= 3 ? 4 : 8);
+    // strips give more workgroups to spread over the 256 CUs.  s8 from 33 tokens on took 4 bytes
+    // per lane (64-byte pieces of every row) until the factored mode got its 8-byte forms:
+    // [64,8192] x [8192,28672] 87.5 -> 58.5 us, 48 tokens 76 -> 49.
+    int vec = s4 ? 4 : (mt >= 3 && (mode != kFactored || p.N % 8 != 0) ? 4 : 8);
     if (int v = GetOption("dequant_dot_vec")) vec = v;
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
@@ -881,6 +890,8 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
       XLA_AMD_DECODE(8, 16, 1, kFactored, "dequant_dot_decode_s8_v16_m16_factored")
       XLA_AMD_DECODE(8, 8, 1, kFactored, "dequant_dot_decode_s8_v8_m16_factored")
       XLA_AMD_DECODE(8, 8, 2, kFactored, "dequant_dot_decode_s8_v8_m32_factored")
+      XLA_AMD_DECODE(8, 8, 3, kFactored, "dequant_dot_decode_s8_v8_m48_factored")
+      XLA_AMD_DECODE(8, 8, 4, kFactored, "dequant_dot_decode_s8_v8_m64_factored")
       XLA_AMD_DECODE(8, 4, 3, kFactored, "dequant_dot_decode_s8_v4_m48_factored")
       XLA_AMD_DECODE(8, 4, 4, kFactored, "dequant_dot_decode_s8_v4_m64_factored")
 #undef XLA_AMD_DECODE
