@@ -907,7 +907,7 @@ def test_ragged_dot_more_than_64_rows(oracle, M, K, N, G, sizes):
     say("dequant_dot ragged prefill M=%d K=%d N=%d G=%d sizes=%s" % (M, K, N, G, sizes))
     w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
     got, kern = run_ragged(w)
-    assert kern == "dequant_dot_decode_s8_v8_m64_factored", kern
+    assert kern == "dequant_dot_decode_s8_v4_m64_factored", kern   # few strips: the narrow ones
     ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
     check_dot(got, ref, ragged_floor(w), "ragged prefill %s" % kern)
     start = 0

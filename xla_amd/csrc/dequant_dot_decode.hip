@@ -563,20 +563,22 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
 
 // K-slices for a decode launch.  One workgroup per CU is enough once the strips alone give about
 // that many (the kernel is bound by its own arithmetic, and every extra slice costs partial sums
-// and a second launch); up to four tokens a second slice still pays.  Fewer strips are split
+// and a second launch).  Fewer strips are split
 // until there are, as long as a wave keeps at least four 32-row steps and the partial sums
 // (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or a quarter
 // of the weight bytes (s8 [64,8192] x [8192,8192]: 44 us in one slice, 30 in two; K = 28672: 140 -> 80).
 int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
   if (int s = GetOption("dequant_dot_slices")) return s;
-  const int64_t want = M <= 4 ? 448 : 192;
+  // (two workgroups per CU up to four tokens, the rule of an earlier kernel generation, costs the
+  // current ones 15-30 % on mid-sized matrices: s4 8192 x 8192 at one token 16.6 us in 8 slices, 12.5 in 4)
+  const int64_t want = 192;
   const double weight_bytes = (double)K * row_bytes;
   int slices = 1;
   while (strips * slices * batch < want && K / (slices * 2) >= 128 * waves &&
          (slices * 2 * M <= 32 || 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes))
     slices *= 2;
   // a few workgroups more than CUs are worse than half as many: a second round for a quarter of the work
-  if (want == 192 && slices > 1 && strips * batch * slices > 256 && strips * batch * slices < 400) slices /= 2;
+  if (slices > 1 && strips * batch * slices > 256 && strips * batch * slices < 400) slices /= 2;
   return slices;
 }
 
@@ -769,7 +771,9 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     // strips give more workgroups to spread over the 256 CUs.  s8 from 33 tokens on took 4 bytes
     // per lane (64-byte pieces of every row) until the factored mode got its 8-byte forms:
     // [64,8192] x [8192,28672] 87.5 -> 58.5 us, 48 tokens 76 -> 49.
-    int vec = s4 ? 4 : (mt >= 3 && (mode != kFactored || p.N % 8 != 0) ? 4 : 8);
+    // (fewer than 64 such strips leave the narrow ones ahead: more workgroups; 4096 x 4096 at 64 tokens
+    // 17.5 us against 22.6)
+    int vec = s4 ? 4 : (mt >= 3 && (mode != kFactored || p.N % 8 != 0 || (p.N + 127) / 128 * p.batch < 64) ? 4 : 8);
     if (int v = GetOption("dequant_dot_vec")) vec = v;
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
