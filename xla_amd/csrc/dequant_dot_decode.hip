@@ -565,17 +565,20 @@ size_t DequantDotWorkspaceBytes(int64_t batch, int64_t M, int64_t N, int slices)
 // that many (the kernel is bound by its own arithmetic, and every extra slice costs partial sums
 // and a second launch).  Fewer strips are split
 // until there are, as long as a wave keeps at least four 32-row steps and the partial sums
-// (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or a quarter
-// of the weight bytes (s8 [64,8192] x [8192,8192]: 44 us in one slice, 30 in two; K = 28672: 140 -> 80).
+// (slices*M*N*4 bytes written and read again) stay small: at most 32 rows of them, or half a byte
+// per weight whatever the weights' width -- above 16 tokens the kernels are bound by their arithmetic,
+// which 4-bit weights do not halve (s8 [64,8192] x [8192,8192]: 44 us in one slice, 30 in two;
+// s4 [64,14336] x [14336,4096]: 36 us in two slices, 24 in eight; [64,4096] x [4096,4096]: 23 -> 17).
 int DecodeSlices(int64_t batch, int64_t M, int64_t K, int64_t N, int strips, int64_t row_bytes, int waves) {
   if (int s = GetOption("dequant_dot_slices")) return s;
   // (two workgroups per CU up to four tokens, the rule of an earlier kernel generation, costs the
   // current ones 15-30 % on mid-sized matrices: s4 8192 x 8192 at one token 16.6 us in 8 slices, 12.5 in 4)
   const int64_t want = 192;
-  const double weight_bytes = (double)K * row_bytes;
+  (void)row_bytes;
+  const double budget = 0.5 * (double)K * (double)N;
   int slices = 1;
   while (strips * slices * batch < want && K / (slices * 2) >= 128 * waves &&
-         (slices * 2 * M <= 32 || 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes))
+         (slices * 2 * M <= 32 || 2.0 * (slices * 2) * M * N * 4.0 <= budget))
     slices *= 2;
   // a few workgroups more than CUs are worse than half as many: a second round for a quarter of the work
   if (slices > 1 && strips * batch * slices > 256 && strips * batch * slices < 400) slices /= 2;
