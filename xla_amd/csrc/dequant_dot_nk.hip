@@ -479,15 +479,20 @@ NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, in
   if (int v = tuned_ct ? GetOption("dequant_dot_nk_ct") : 0) s.ct = s.mt != 1 ? 2 : v == 1 ? 1 : v == 4 ? 4 : 2;  // (one token tile only)
   s.strips = (int)((N + kNkWaves * s.ct * 16 - 1) / (kNkWaves * s.ct * 16));
   s.m_chunks = (int)((M + 16 * s.mt - 1) / (16 * s.mt));
-  // few workgroups: cut K (at most four ways) while a slice keeps eight steps (or whole groups) and
-  // the partial sums stay below a quarter of the weight bytes
+  // few workgroups: cut K while a slice keeps eight steps (or whole groups) and the partial sums
+  // (written and read again) stay below half a byte per weight.  One token tile: up to four ways,
+  // towards four workgroups per CU.  Two: up to eight ways, towards two per CU.  Four (33-64 tokens,
+  // where the arithmetic binds): one workgroup per CU and never a few more than CUs
+  // (s4 [64,14336] x [4096,14336]^T: 68 us in two slices, 31 in eight; [64,8192] x [8192,8192]^T 44 -> 31).
   const int64_t unit = slice_unit > s.step ? slice_unit : s.step;
-  const int64_t want = s.mt == 1 ? 1024 : 448;
+  const int64_t want = s.mt == 1 ? 1024 : s.mt == 2 ? 448 : 192;
+  const int most = s.mt == 1 ? 4 : 8;
   int slices = 1;
-  const double weight_bytes = (double)K * N * s.wbits / 8;
-  while (slices < 4 && (int64_t)s.strips * batch * s.m_chunks * slices < want && K / (slices * 2) >= 8 * s.step &&
-         (K / (slices * 2)) % unit == 0 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.25 * weight_bytes)
+  const int64_t wgs = (int64_t)s.strips * batch * s.m_chunks;
+  while (slices < most && wgs * slices < want && K / (slices * 2) >= 8 * s.step &&
+         (K / (slices * 2)) % unit == 0 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.5 * (double)K * N)
     slices *= 2;
+  if (s.mt == 4 && slices > 1 && wgs * slices > 256 && wgs * slices < 400) slices /= 2;
   if (int v = GetOption("dequant_dot_slices")) {
     if (K % (v * unit) == 0) slices = v;
   }
