@@ -255,13 +255,13 @@ def test_tiled_k_minor_one_hot(oracle, kind):
 
 
 def test_large_prefill_picks_the_tiled_kernel_by_itself(oracle):
-    say("dequant_dot [N,K] s8 1024 tokens: routing")
-    w = workloads.c1_s8_channel(M=1024, K=1024, N=4096)
+    say("dequant_dot [N,K] s8 2048 tokens: routing")
+    w = workloads.c1_s8_channel(M=2048, K=2048, N=8192)   # a full round of tiles (fewer tokens on a matrix this small stream)
     got, kern = run_nk(w)
     assert kern.startswith("dequant_dot_tiled_nk_s8_factored"), kern
     # the oracle on a block of rows and channels
     rows, cols = slice(512, 560), slice(1000, 1256)
-    blk = dict(w, lhs=w["lhs"][rows], weights=w["weights"][:, cols], scales=w["scales"][cols], weight_shape=(1024, 256))
+    blk = dict(w, lhs=w["lhs"][rows], weights=w["weights"][:, cols], scales=w["scales"][cols], weight_shape=(2048, 256))
     compare(oracle, blk, got[rows, cols], "[N,K] tiled s8 block")
 
 

@@ -38,7 +38,7 @@ def test_handlers_replay_from_a_hip_graph(oracle):
                     (workloads.c2_s4_group(M=20, K=2048, N=768, group=64), {"dequant_dot_slices": 2}),  # finalize launch
                     (workloads.c2_s4_group(M=70, K=1024, N=512), {}),                     # 64 + 6 tokens
                     (workloads.c1_s8_channel(M=16, K=2048, N=1024), {}),                  # slices inside the kernel
-                    (workloads.c5_s8_batched(B=1, M=300, K=2048, N=700), {}),             # tiles split along K
+                    (workloads.c5_s8_batched(B=1, M=300, K=2048, N=700), {"dequant_dot_kernel": 3}),   # tiles split along K
                     (workloads.c2_s4_group(M=8, K=2048, N=512), {"nk": 1})):              # weights stored [N,K], K-slices
         nk = opts.pop("nk", 0)
         v = workloads.k_minor(w) if nk else w   # (the oracle keeps reading the [K,N] arrays)

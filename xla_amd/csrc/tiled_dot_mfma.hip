@@ -1188,6 +1188,39 @@ constexpr int64_t kF8MaxTail = 64;
 // (up to 64 rows the integer-weight dots run on the decode kernels)
 size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) { return TailBytesFor(batch, M, K, N, 65); }
 
+// More than 64 tokens of integer weights: the decode kernel, run once per 64 tokens, streams and
+// dequantises the weights on every pass but fills the machine at any M; the tiled kernel dequantises
+// once per 256 tokens but gives a CU nothing to do unless there are 256 tiles.  Estimates in
+// microseconds fitted on MI355X over matrices from 4096 x 4096 to 8192 x 28672 and 80 to 1024 tokens:
+//   decode, weights [K,N]: the first pass 14 + 1.4e-7 K N (s4; s8 2.0e-7), every further one of the
+//     same launch 1 + 1.6e-7 K N (2.05e-7), a last pass of fewer than 64 tokens three quarters of a
+//     first one, all of it once per batch (8192 x 28672 s4: 47 / 86 / 168 us at 64 / 128 / 256 tokens);
+//   decode, weights [N,K]: one launch, 14 + 2.7e-7 K N per 64 tokens (s8: 2.8e-7, 3.5e-7 when the
+//     matrix is too large to stay in the last-level cache between passes), passes counted in pairs;
+//   tiled: 25 + 0.025 K per round of 256 tiles, a last round of at most 128 tiles (split along K)
+//     25 + 0.0125 K (K = 8192: 230 and 127); weights [N,K]: 25 + 0.0245 K and 20 + 0.01025 K.
+static bool DecodePassesAreCheaper(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, bool k_minor) {
+  const double kn = (double)K * (double)N;
+  double decode_us;
+  if (k_minor) {
+    int64_t passes = (M + 63) / 64;
+    if (passes > 1) passes = (passes + 1) / 2 * 2;
+    const double per_pass = kn * (four_bit ? 2.7e-7 : kn > 1.5e8 ? 3.5e-7 : 2.8e-7);
+    decode_us = 14.0 + (double)batch * (double)passes * per_pass;
+  } else {
+    const double first = 14.0 + kn * (four_bit ? 1.4e-7 : 2.0e-7);
+    const double next = 1.0 + kn * (four_bit ? 1.6e-7 : 2.05e-7);
+    const int64_t whole = M / 64, rest = M % 64;
+    decode_us = (double)batch * ((whole > 0 ? first + (double)(whole - 1) * next : 0.0) + (rest > 0 ? 0.75 * first : 0.0));
+  }
+  const int64_t tiles = batch * ((M + kTM - 1) / kTM) * ((N + kTN - 1) / kTN);
+  const int64_t tail = tiles % 256;
+  const double round_us = k_minor ? 25.0 + 0.0245 * (double)K : 25.0 + 0.025 * (double)K;
+  const double half_us = k_minor ? 20.0 + 0.01025 * (double)K : 25.0 + 0.0125 * (double)K;
+  const double tiled_us = (double)(tiles / 256) * round_us + (tail == 0 ? 0.0 : tail <= 128 && K >= 2048 ? half_us : round_us);
+  return decode_us <= tiled_us;
+}
+
 // bf16 x s8 per-channel prefill.  Returns -1 when the tiled kernel does not cover the shape
 // (the caller then falls back), 0 on success, or an error code.
 int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
@@ -1203,18 +1236,8 @@ int LaunchDequantDotPrefill(const XlaAmdDequantDot& p, hipStream_t stream) {
   if (!s4 && !s8) return -1;
   const bool ragged = p.group_sizes != nullptr;  // the caller has decided that the rows per group make tiles worth it
   if (u4 && ragged) return -1;  // a ragged dot over u4 weights stays with the 64-row chunks of the decode kernel
-  if (s4 && !ragged && GetOption("dequant_dot_kernel") != 3) {
-    // The decode kernel, run once per 64 tokens, streams and dequantises the weights on every
-    // pass but fills the machine at any M; the tiled kernel dequantises once per 256 tokens but
-    // needs 256 tiles per round.  Estimates in microseconds fitted on MI355X (8192 x 28672:
-    // 53 per decode pass, 287 per round of tiles); the cheaper one runs.
-    const double passes = (double)p.batch * (double)((p.M + 63) / 64);
-    const double decode_us = passes * (6.0 + (double)p.K * (double)p.N * 2.0e-7);
-    const double tiles = (double)p.batch * (double)((p.M + kTM - 1) / kTM) * (double)((p.N + kTN - 1) / kTN);
-    const double rounds = (double)(int64_t)((tiles + 255.0) / 256.0);
-    const double tiled_us = rounds * (10.0 + (double)p.K * 0.0338);
-    if (decode_us <= tiled_us) return -1;
-  }
+  if (!ragged && GetOption("dequant_dot_kernel") != 3 && DecodePassesAreCheaper(p.batch, p.M, p.K, p.N, s4, false))
+    return -1;
   if (p.K % 8 != 0 || p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 4)) return -1;
   // 32-bit buffer offsets per batch
   if ((double)p.M * p.K * 2 >= 2147483000.0 || (double)p.K * p.N >= 2147483000.0) return -1;
@@ -1290,15 +1313,8 @@ int LaunchDequantDotPrefillNk(const XlaAmdDequantDot& p, hipStream_t stream) {
                   p.K % 16 == 0;
   if ((!s4 && !s8) || p.zero_points) return -1;
   const bool ragged = p.group_sizes != nullptr;  // the caller has decided that the rows per group make tiles worth it
-  if (!ragged && GetOption("dequant_dot_kernel") != 3) {
-    // token chunks of the streaming kernel against rounds of 256 tiles, in microseconds fitted on MI355X
-    // (s4 8192 x 28672: 75 per 64-token pass; s8 4096 x 14336: 25)
-    const double passes = (double)p.batch * (double)((p.M + 63) / 64);
-    const double decode_us = passes * (6.0 + (double)p.K * (double)p.N * (s4 ? 3.0e-7 : 3.3e-7));
-    const double tiles = (double)p.batch * (double)((p.M + kTM - 1) / kTM) * (double)((p.N + kTN - 1) / kTN);
-    const double rounds = (double)(int64_t)((tiles + 255.0) / 256.0);
-    if (decode_us <= rounds * (10.0 + (double)p.K * 0.035)) return -1;
-  }
+  if (!ragged && GetOption("dequant_dot_kernel") != 3 && DecodePassesAreCheaper(p.batch, p.M, p.K, p.N, s4, true))
+    return -1;
   if (p.N % 4 != 0 || ((uintptr_t)p.lhs % 16) || ((uintptr_t)p.weights % 16) || ((uintptr_t)p.scales % 2)) return -1;
   if ((double)p.M * p.K * 2 >= 2147483000.0 || (double)p.K * p.N >= 2147483000.0) return -1;
   TiledParams tp{};
