@@ -113,8 +113,9 @@ XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_dequant_dot(XLA_FFI_CallFrame* call_frame)
  *   attrs: epilogue, dequant_type, dot_type, epilogue_type as above;
  *          rhs_contracting_dim i64 (default 0);
  *          d_scale_multiplies pred (default false): v * d_scale instead (:1730-1748)
- * One handler for every size: up to 64 rows of a take kernels that stream the rhs once (HBM-bound),
- * more rows the tiled kernel (MFMA-bound).
+ * One handler for every size: up to 64 rows of a take kernels that stream the rhs once (HBM-bound), as do
+ * a few hundred rows of a matrix with few 256 x 256 tiles (in passes of up to 64 rows); more rows the
+ * tiled kernel (MFMA-bound).
  */
 XLA_AMD_EXPORT XLA_FFI_Error* xla_amd_fp8_scaled_dot(XLA_FFI_CallFrame* call_frame);
 
@@ -267,7 +268,8 @@ XLA_AMD_EXPORT int xla_amd_launch_fp8_scaled_dot(const XlaAmdFp8ScaledDot* p, vo
  * gemm_rewriter.cc:1235-1591), which takes K*N bytes -- without them such a rhs runs on the slow
  * exact kernel.  Up to 64 rows of a (48 with an [N,K] rhs, 32 with block scales; K and N multiples
  * of 8, resp. 16 and 8, K of 128 with block scales) stream the rhs once instead and, where the channels alone leave CUs idle, split K over workgroups:
- * slices * M * N * 4 bytes of f32 sums, per batch -- without them one slice. */
+ * slices * M * N * 4 bytes of f32 sums, per batch -- without them one slice.  More rows that go through
+ * those kernels in passes (no batch, no block scales) need the sums of one pass. */
 XLA_AMD_EXPORT size_t xla_amd_fp8_scaled_dot_workspace_bytes(int64_t M, int64_t K, int64_t N,
                                                              int32_t rhs_contracting_dim);
 

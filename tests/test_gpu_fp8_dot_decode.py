@@ -1,4 +1,4 @@
-"""The weight-streaming kernels of xla_amd.fp8_scaled_dot (up to 64 rows of a; rhs [K,N] or [N,K]) against
+"""The weight-streaming kernels of xla_amd.fp8_scaled_dot (up to 64 rows of a per launch; rhs [K,N] or [N,K]) against
 the CPU oracle, through the FFI handler: every token-tile count, ragged K and N, K-slices with and without
 scratch, vector scales, f8 results with amax, batches, one-hot exactness and special values."""
 import numpy as np
@@ -226,17 +226,68 @@ def test_nan_codes_and_the_end_of_k(oracle, nk):
 
 
 def test_what_the_streaming_kernels_do_not_take():
-    a = torch.zeros((80, 64), dtype=torch.uint8, device="cuda")
-    b = torch.zeros((64, 64), dtype=torch.uint8, device="cuda")
+    a = torch.zeros((2, 80, 64), dtype=torch.uint8, device="cuda")
+    b = torch.zeros((2, 64, 64), dtype=torch.uint8, device="cuda")
     one = torch.ones((), dtype=torch.float32, device="cuda")
     ffi.set_option("fp8_dot_kernel", 3)
     try:
-        with pytest.raises(ffi.FfiError, match="streaming kernels take up to 64 rows"):
-            ops.fp8_scaled_dot(a, b, one, one)
+        with pytest.raises(ffi.FfiError, match="only without a batch dimension"):
+            ops.fp8_scaled_dot(a, b, one, one)      # 80 rows per batch
         with pytest.raises(ffi.FfiError, match="streaming kernels take"):
-            ops.fp8_scaled_dot(a[:8], b, one, one, dequant_type="bf16")
+            ops.fp8_scaled_dot(a[0, :8], b[0], one, one, dequant_type="bf16")
     finally:
         ffi.set_option("fp8_dot_kernel", 0)
+
+
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("M", [65, 100, 130, 200])
+def test_more_rows_go_through_in_equal_passes(oracle, M, nk):
+    """More rows of a than one launch takes (64, or 48 with the rhs [N,K]): passes of equal row counts
+    (multiples of 16), the last one with what is left; per-row scales and the bias follow the rows."""
+    say("fp8 streaming, %d rows in passes, nk=%s" % (M, nk))
+    K, N = 1024, 264
+    w = workloads.c3_fp8(M, K, N)
+    w["a_scale"] = np.random.default_rng(M).uniform(0.004, 0.04, M).astype(np.float32)
+    most = 48 if nk else 64
+    passes = -(-M // most)
+    rows = -(-(-(-M // passes)) // 16) * 16
+    for slices in (0, 2):
+        out, kern = run(w, nk=nk, slices=slices)
+        assert kern == "%s:x%d" % (tile_name(nk, rows), rows), kern
+        check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+
+
+def test_passes_with_an_f8_result_fold_one_amax(oracle):
+    say("fp8 streaming, 150 rows in passes, f8 result + amax")
+    M, K, N = 150, 512, 136
+    w = workloads.c3_fp8(M, K, N)
+    s = np.float32(1 / 64)
+    w["a_scale"] = w["b_scale"] = s
+    z = np.float32(0.0171)
+    (out, amax), kern = run(w, d_scale=dev_f32(np.array(z, np.float32)), amax=True)
+    assert kern == "fp8_dot_decode_kn_m64:x64", kern
+    ref, val = oracle.fp8_scaled_dot(w["a"], w["b"], s, s, bias=w["bias"], epilogue=EPI[w["epilogue"]], d_scale=z,
+                                     d_scale_divides=True)
+    check_f8_result(out.cpu().numpy(), ref, val, z, True, floor_for(w), kern)
+    want = float(np.max(np.abs(val)))
+    got = float(amax.cpu())
+    assert abs(got - want) <= 2.0 ** -7 * want + float(np.max(floor_for(w))), (got, want)
+
+
+def test_the_launcher_takes_passes_where_they_are_cheaper(oracle):
+    """Few tiles of a long K: two passes of the streaming kernel instead of a handful of 256 x 256 tiles;
+    many tiles: the tiled kernel."""
+    say("fp8 streaming passes, the launcher's own choice")
+    w = workloads.c3_fp8(96, 4096, 512)
+    out, kern = run(w, force=0)
+    assert kern == "fp8_dot_decode_kn_m48:x48", kern
+    check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    out, kern = run(w, nk=True, force=0)
+    assert kern == "fp8_dot_decode_nk_m48:x48", kern
+    check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    big = workloads.c3_fp8(512, 256, 512)   # four passes of a short K against one round of tiles
+    out, kern = run(big, force=0)
+    assert kern.startswith("fp8_scaled_dot_tiled"), kern
 
 
 # ---- block scales (MXFP8) on the [N,K] streaming kernel: up to 32 rows of a, K % 128 == 0 ---------------

@@ -451,14 +451,77 @@ int Slices(int64_t batch, int64_t M, int64_t K, int64_t N, bool nk) {
 
 }  // namespace
 
-size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
-  if (M <= 0 || M > (rhs_contracting_dim == 1 ? 48 : 64) || K <= 0 || N <= 0 || batch <= 0) return 0;
-  const int slices = Slices(batch, M, K, N, rhs_contracting_dim == 1);
-  return slices > 1 ? (size_t)batch * slices * M * N * 4 : 0;
+// More rows of a than one launch takes: the rows go through the streaming kernel in equal passes
+// (every row of the result depends on its own row of a only).  rows: rows per pass, a multiple of 16.
+static int Passes(int64_t M, bool nk, bool mx, int64_t* rows) {
+  const int64_t most = mx ? 32 : nk ? 48 : 64;
+  const int64_t passes = (M + most - 1) / most;
+  *rows = passes > 0 ? ((M + passes - 1) / passes + 15) / 16 * 16 : 0;
+  return (int)passes;
 }
+
+// Passes of the streaming kernel against the tiled kernel, in microseconds fitted on MI355X over
+// matrices from 4096 x 4096 to 8192 x 28672: a pass 15 + 1.95e-7 K N (rhs [K,N], up to 64 rows) or
+// 13 + 1.35e-7 K N (rhs [N,K], up to 48); the tiled kernel with at most one round of tiles
+// 32 + 0.0071 K, 27 + 0.0052 K when it splits its tiles along K (at most 64 of them, 65 rows on).
+// ([128,8192] x [8192,8192]: 69 us tiled, 46 in two passes; [64,14336] x [4096,14336]^T: 135 and 38.)
+static bool PassesAreCheaper(int64_t M, int64_t K, int64_t N, bool nk, int passes, int64_t rows) {
+  const int64_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (tiles > 256 || passes > 6) return false;
+  const double kn = (double)K * (double)N;
+  // (a [K,N] pass of 48 rows takes about 0.85 of one of 64)
+  const double pass_us = nk ? 13.0 + 1.35e-7 * kn : (15.0 + 1.95e-7 * kn) * (0.4 + 0.6 * (double)rows / 64.0);
+  const double tiled_us = tiles <= 64 && M >= 65 && K >= 2048 ? 27.0 + 0.0052 * (double)K : 32.0 + 0.0071 * (double)K;
+  return (double)passes * pass_us <= tiled_us;
+}
+
+size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
+  if (M <= 0 || K <= 0 || N <= 0 || batch <= 0) return 0;
+  const bool nk = rhs_contracting_dim == 1;
+  int64_t rows = M;
+  if (M > (nk ? 48 : 64)) {  // passes follow each other on the stream and share the scratch
+    if (batch > 1) return 0;
+    const int passes = Passes(M, nk, false, &rows);
+    if (GetOption("fp8_dot_kernel") != 3 && !PassesAreCheaper(M, K, N, nk, passes, rows)) return 0;
+  }
+  size_t bytes = 0;
+  for (const int64_t m : {rows, M % rows}) {  // (the last pass may have fewer rows and more slices)
+    if (m <= 0) continue;
+    const int slices = Slices(batch, m, K, N, nk);
+    const size_t need = slices > 1 ? (size_t)batch * slices * m * N * 4 : 0;
+    bytes = bytes > need ? bytes : need;
+  }
+  return bytes;
+}
+
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
 
 // Returns -1 when the shape is not covered, else the launch status.
 int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
+  const bool nk = p.rhs_contracting_dim == 1;
+  const bool mx = p.a_block_scales != nullptr;
+  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream);
+  if (p.batch > 1 || mx) return -1;
+  int64_t rows = 0;
+  const int passes = Passes(p.M, nk, mx, &rows);
+  if (GetOption("fp8_dot_kernel") != 3 && !PassesAreCheaper(p.M, p.K, p.N, nk, passes, rows)) return -1;
+  const size_t out_bytes = p.out_dtype == XLA_FFI_DataType_F8E4M3FN ? 1 : 2;
+  char name[64] = "";
+  for (int64_t m0 = 0; m0 < p.M; m0 += rows) {
+    XlaAmdFp8ScaledDot sub = p;
+    sub.M = p.M - m0 < rows ? p.M - m0 : rows;
+    sub.a = (const char*)p.a + (size_t)m0 * p.K;
+    sub.out = (char*)p.out + (size_t)m0 * p.N * out_bytes;
+    if (p.a_scale_per_row) sub.a_scale = p.a_scale + m0;
+    const int rc = LaunchFp8DotDecodeRows(sub, stream);
+    if (rc != 0) return rc;  // (-1 on the first pass: not covered; the passes differ in their row count only)
+    if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)rows);
+  }
+  SetLastKernel(name);
+  return 0;
+}
+
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const int64_t batch = p.batch > 1 ? p.batch : 1;
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;

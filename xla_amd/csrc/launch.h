@@ -25,8 +25,9 @@ int LaunchDequantDot(const XlaAmdDequantDot& p, hipStream_t stream);
 // Same, with the split-K partial sums in the library's static device array (allocates nothing).
 int LaunchDequantDotStaticScratch(const XlaAmdDequantDot& p, hipStream_t stream);
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
-// Up to 64 rows of a (48 with the rhs [N,K]), per-tensor / per-row / per-channel scales under f32-typed multiplies: the rhs
-// streamed once (fp8_dot_decode.hip).  Returns -1 when the shape is not covered, else the launch
+// Up to 64 rows of a per launch (48 with the rhs [N,K]), per-tensor / per-row / per-channel scales under
+// f32-typed multiplies: the rhs streamed once (fp8_dot_decode.hip); more rows in passes where that is
+// cheaper than tiles.  Returns -1 when the shape is not covered (or tiles are cheaper), else the launch
 // status; p comes validated and an amax result already zeroed.  The scratch is the f32 sums of its
 // K-slices (0: one slice).
 int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
