@@ -322,6 +322,22 @@ def test_mxfp8_block_scales(oracle, M, K, N, slices):
     assert n_floor <= max(4, got.size // 50)
 
 
+@pytest.mark.parametrize("M", [33, 64, 70])
+@pytest.mark.parametrize("slices", [0, 2])
+def test_mxfp8_more_rows_in_passes(oracle, M, slices):
+    """More than 32 rows with block scales: passes of up to 32 rows, each with its rows' scales."""
+    from tests.test_gpu_fp8_dot import mx_case, mx_floor
+    say("fp8 streaming MXFP8 M=%d in passes, slices=%d" % (M, slices))
+    K, N = 1024, 136
+    a, b, sa, sb = mx_case(M, K, N, 11)
+    sa[:] = ((np.arange(M)[:, None] * 3 + np.arange(K // 32)[None, :]) % 13 + 121).astype(np.uint8)   # scales that tell rows apart
+    got, kern = run_mx(a, b, sa, sb, slices=slices)
+    rows = -(-(-(-M // -(-M // 32))) // 16) * 16
+    assert kern == "fp8_dot_decode_mx_m%d:x%d" % (rows, rows), kern
+    n_floor = check_dot(got, oracle.block_scaled_dot(a, b, sa, sb), mx_floor(a, b, sa, sb, False), kern)
+    assert n_floor <= max(4, got.size // 50)
+
+
 @pytest.mark.parametrize("epilogue,dot_ty,ep_ty", [("BIAS_GELU", "f32", "f32"), ("BIAS_SILU", "bf16", "bf16"), ("RELU", "f32", "f32")])
 def test_mxfp8_with_an_epilogue_and_batched(oracle, epilogue, dot_ty, ep_ty):
     from tests.test_gpu_fp8_dot import mx_case, mx_floor

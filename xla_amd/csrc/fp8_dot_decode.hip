@@ -475,13 +475,11 @@ static bool PassesAreCheaper(int64_t M, int64_t K, int64_t N, bool nk, int passe
   return (double)passes * pass_us <= tiled_us;
 }
 
-size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
-  if (M <= 0 || K <= 0 || N <= 0 || batch <= 0) return 0;
-  const bool nk = rhs_contracting_dim == 1;
+static size_t WorkspaceBytesFor(int64_t batch, int64_t M, int64_t K, int64_t N, bool nk, bool mx) {
   int64_t rows = M;
-  if (M > (nk ? 48 : 64)) {  // passes follow each other on the stream and share the scratch
+  if (M > (mx ? 32 : nk ? 48 : 64)) {  // passes follow each other on the stream and share the scratch
     if (batch > 1) return 0;
-    const int passes = Passes(M, nk, false, &rows);
+    const int passes = Passes(M, nk, mx, &rows);
     if (GetOption("fp8_dot_kernel") != 3 && !PassesAreCheaper(M, K, N, nk, passes, rows)) return 0;
   }
   size_t bytes = 0;
@@ -494,6 +492,17 @@ size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N
   return bytes;
 }
 
+size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim) {
+  if (M <= 0 || K <= 0 || N <= 0 || batch <= 0) return 0;
+  const bool nk = rhs_contracting_dim == 1;
+  size_t bytes = WorkspaceBytesFor(batch, M, K, N, nk, false);
+  if (nk && K % 128 == 0) {  // the call may come with block scales (not known here): passes of 32 rows
+    const size_t mx = WorkspaceBytesFor(batch, M, K, N, true, true);
+    bytes = bytes > mx ? bytes : mx;
+  }
+  return bytes;
+}
+
 static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
 
 // Returns -1 when the shape is not covered, else the launch status.
@@ -501,7 +510,7 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;
   if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream);
-  if (p.batch > 1 || mx) return -1;
+  if (p.batch > 1) return -1;
   int64_t rows = 0;
   const int passes = Passes(p.M, nk, mx, &rows);
   if (GetOption("fp8_dot_kernel") != 3 && !PassesAreCheaper(p.M, p.K, p.N, nk, passes, rows)) return -1;
@@ -513,6 +522,7 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     sub.a = (const char*)p.a + (size_t)m0 * p.K;
     sub.out = (char*)p.out + (size_t)m0 * p.N * out_bytes;
     if (p.a_scale_per_row) sub.a_scale = p.a_scale + m0;
+    if (mx) sub.a_block_scales = (const char*)p.a_block_scales + (size_t)m0 * (size_t)(p.K / 32);
     const int rc = LaunchFp8DotDecodeRows(sub, stream);
     if (rc != 0) return rc;  // (-1 on the first pass: not covered; the passes differ in their row count only)
     if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)rows);

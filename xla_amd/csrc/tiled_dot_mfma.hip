@@ -1470,7 +1470,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
                   "fp8_scaled_dot: the streaming kernels take K %% 8 == 0 and N %% 8 == 0, 8-byte aligned operands "
                   "and f32-typed multiplies; more than 64 rows of a (48 with the rhs [N,K], 32 with block scales) "
-                  "only without a batch dimension and block scales");
+                  "only without a batch dimension");
   }
   tp.M = (int)p.M; tp.K = (int)p.K; tp.N = (int)p.N;
   tp.bias_is_bf16 = p.bias_dtype == XLA_FFI_DataType_BF16;
