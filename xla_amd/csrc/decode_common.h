@@ -74,10 +74,10 @@ struct DecodeParams {
   int d_multiplies;
 };
 
-// One result element; row = batch * M + m over the flattened [batch * M, N] result.
-static __device__ __forceinline__ void StoreResult(const DecodeParams& p, size_t row, int n, float v) {
-  size_t idx = row * (size_t)p.N + (size_t)n;
-  if (p.out_transposed) idx = ((row / (size_t)p.M) * (size_t)p.N + (size_t)n) * (size_t)p.M + row % (size_t)p.M;
+// One result element: row m of batch `batch` (a ragged dot: batch 0, m over all rows), channel n.
+static __device__ __forceinline__ void StoreResult(const DecodeParams& p, int batch, int m, int n, float v) {
+  size_t idx = ((size_t)batch * (size_t)p.M + (size_t)m) * (size_t)p.N + (size_t)n;
+  if (p.out_transposed) idx = ((size_t)batch * (size_t)p.N + (size_t)n) * (size_t)p.M + (size_t)m;
   if (p.out_f8) {
     // op by op as the HLO does: an IEEE quotient (or product), clamp (a NaN stays one), cast
     float c = p.d_multiplies ? v * *p.d_scale : v / *p.d_scale;

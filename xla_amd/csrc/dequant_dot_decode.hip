@@ -400,7 +400,7 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     } else {
       if (p.out_f32 | p.out_transposed | p.out_f8) {
 #pragma unroll
-        for (int u = 0; u < RPW; ++u) StoreResult(p, (size_t)m_begin + m, n0 + u, res[pass * RPW + u]);
+        for (int u = 0; u < RPW; ++u) StoreResult(p, p.group_sizes ? 0 : batch, p.group_sizes ? m_begin + m : m, n0 + u, res[pass * RPW + u]);
         continue;
       }
       uint16_t* dst = p.out + ((size_t)m_begin + m) * p.N + n0;
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256) void dequant_dot_finalize_kernel(DecodeParams 
   if (mode == kFactored)
     v = v * load_scale(p.scales, (size_t)(p.scale_batched ? batch : 0) * p.N + n, p.scale_is_bf16);
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  StoreResult(p, (size_t)batch * p.M + idx / p.N, n, epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, batch, (int)(idx / p.N), n, epilogue_dispatch(v, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 // Any shape, any alignment: one thread per output, k in increasing order.  Correct for every
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(256) void dequant_dot_generic_kernel(DecodeParams p
     acc = acc + bf16_to_f32(a[(size_t)k * a_step]) * wv;
   }
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  StoreResult(p, (size_t)batch * p.M + m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, batch, m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 template <int WBITS, int VEC, int MT, int WAVES, int MODE>

@@ -326,9 +326,11 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   // ---- lane (c, kq), register i of tile (t, mt): channel n_wave + 16 t + 4 kq + i, token m0 + 16 mt + c.
   // One tile at a time (the fences keep the scheduler from interleaving the tiles' activations,
   // which would hold every tile's temporaries in registers at once).
+  // (expanded, not unrolled: with the general stores in its body the compiler left the tile loop
+  // rolled, and accumulators indexed by a run-time t live in scratch memory -- also in the main loop)
   const bool quads = p.N % 4 == 0;
-#pragma unroll
-  for (int t = 0; t < CT; ++t) {
+  static_for<0, CT>([&](auto tile_index) {
+    constexpr int t = decltype(tile_index)::value;
     float fq[4], bq[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -336,11 +338,14 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
       fq[i] = MODE == kFactored && p.slices == 1 ? load_scale(p.scales, sbatch * p.N + n, p.scale_is_bf16) : 1.0f;
       bq[i] = p.bias && p.slices == 1 ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
     }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    static_for<0, MT>([&](auto token_tile) {
+      constexpr int mt = decltype(token_tile)::value;
       float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (GF ? tot[t][mt][i] : acc[t][mt][i]) * fq[i];
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (GF) v[i] = tot[t][mt][i] * fq[i];
+        else v[i] = acc[t][mt][i] * fq[i];
+      }
       if (p.slices == 1) epilogue_all_dispatch<4>(v, bq, p.epilogue, p.bf16_dot, p.bf16_ops);
       const int n = n_wave + t * 16 + 4 * kq, m = mt * 16 + c;
       if (m < rows_here && n < p.N) {
@@ -357,7 +362,7 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
         } else if (p.out_f32 | p.out_transposed | p.out_f8) {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (n + i < p.N) StoreResult(p, (size_t)a_batch * p.M + m_first + m0 + m, n + i, v[i]);
+            if (n + i < p.N) StoreResult(p, a_batch, m_first + m0 + m, n + i, v[i]);
         } else if (quads) {
           *reinterpret_cast<uintx2*>(p.out + o) = uintx2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         } else {
@@ -367,8 +372,8 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
         }
       }
       __builtin_amdgcn_sched_barrier(0);
-    }
-  }
+    });
+  });
 }
 
 // Any shape and alignment: one thread per output, k in increasing order.
@@ -413,7 +418,7 @@ __global__ __launch_bounds__(256) void dequant_dot_nk_generic_kernel(DecodeParam
     acc = acc + bf16_to_f32(a[(size_t)k * a_step]) * wv;
   }
   const float b = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
-  StoreResult(p, (size_t)batch * p.M + m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
+  StoreResult(p, batch, m, n, epilogue_dispatch(acc, b, p.epilogue, p.bf16_dot, p.bf16_ops));
 }
 
 // Ragged dot: rows past the last group are a dot of nothing, epilogue(0).  Workgroup (x, y) takes 256
@@ -481,18 +486,16 @@ NkShape PlanNk(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, in
   s.m_chunks = (int)((M + 16 * s.mt - 1) / (16 * s.mt));
   // few workgroups: cut K while a slice keeps eight steps (or whole groups) and the partial sums
   // (written and read again) stay below half a byte per weight.  One token tile: up to four ways,
-  // towards four workgroups per CU.  Two: up to eight ways, towards two per CU.  Four (33-64 tokens,
-  // where the arithmetic binds): one workgroup per CU and never a few more than CUs
-  // (s4 [64,14336] x [4096,14336]^T: 68 us in two slices, 31 in eight; [64,8192] x [8192,8192]^T 44 -> 31).
+  // towards four workgroups per CU; more: up to eight ways, towards two per CU
+  // (s4 [64,14336] x [4096,14336]^T: 60 us in two slices, 26 in eight; [64,28672] x [8192,28672]^T 64 -> 54).
   const int64_t unit = slice_unit > s.step ? slice_unit : s.step;
-  const int64_t want = s.mt == 1 ? 1024 : s.mt == 2 ? 448 : 192;
+  const int64_t want = s.mt == 1 ? 1024 : 448;
   const int most = s.mt == 1 ? 4 : 8;
   int slices = 1;
   const int64_t wgs = (int64_t)s.strips * batch * s.m_chunks;
   while (slices < most && wgs * slices < want && K / (slices * 2) >= 8 * s.step &&
          (K / (slices * 2)) % unit == 0 && 2.0 * (slices * 2) * M * N * 4.0 <= 0.5 * (double)K * N)
     slices *= 2;
-  if (s.mt == 4 && slices > 1 && wgs * slices > 256 && wgs * slices < 400) slices /= 2;
   if (int v = GetOption("dequant_dot_slices")) {
     if (K % (v * unit) == 0) slices = v;
   }

@@ -12,6 +12,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace xla_amd {
 
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -289,6 +291,17 @@ __device__ __forceinline__ void epilogue_all_dispatch(float* v, const float* bia
   } else {
     if (bf16_dot) epilogue_all_act<true, false, COUNT>(v, bias, epi);
     else epilogue_all_act<false, false, COUNT>(v, bias, epi);
+  }
+}
+
+// f(std::integral_constant<int, I>) for I = 0 .. N-1, expanded at compile time: unlike a loop under
+// `#pragma unroll`, which the compiler may decline for a large body, the index is a constant in
+// every copy, so arrays indexed by it stay in registers.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
   }
 }
 

@@ -1195,18 +1195,14 @@ size_t TiledTailWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N) {
 //   decode, weights [K,N]: the first pass 14 + 1.4e-7 K N (s4; s8 2.0e-7), every further one of the
 //     same launch 1 + 1.6e-7 K N (2.05e-7), a last pass of fewer than 64 tokens three quarters of a
 //     first one, all of it once per batch (8192 x 28672 s4: 47 / 86 / 168 us at 64 / 128 / 256 tokens);
-//   decode, weights [N,K]: one launch, 14 + 2.7e-7 K N per 64 tokens (s8: 2.8e-7, 3.5e-7 when the
-//     matrix is too large to stay in the last-level cache between passes), passes counted in pairs;
+//   decode, weights [N,K]: one launch, 14 + 1.85e-7 K N per 64 tokens (s4 and s8 alike);
 //   tiled: 25 + 0.025 K per round of 256 tiles, a last round of at most 128 tiles (split along K)
 //     25 + 0.0125 K (K = 8192: 230 and 127); weights [N,K]: 25 + 0.0245 K and 20 + 0.01025 K.
 static bool DecodePassesAreCheaper(int64_t batch, int64_t M, int64_t K, int64_t N, bool four_bit, bool k_minor) {
   const double kn = (double)K * (double)N;
   double decode_us;
   if (k_minor) {
-    int64_t passes = (M + 63) / 64;
-    if (passes > 1) passes = (passes + 1) / 2 * 2;
-    const double per_pass = kn * (four_bit ? 2.7e-7 : kn > 1.5e8 ? 3.5e-7 : 2.8e-7);
-    decode_us = 14.0 + (double)batch * (double)passes * per_pass;
+    decode_us = (14.0 + (double)batch * (double)((M + 63) / 64) * 1.85e-7 * kn) / 1.05;  // (ties go to the passes)
   } else {
     const double first = 14.0 + kn * (four_bit ? 1.4e-7 : 2.0e-7);
     const double next = 1.0 + kn * (four_bit ? 1.6e-7 : 2.05e-7);
