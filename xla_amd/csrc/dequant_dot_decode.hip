@@ -772,11 +772,12 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
     // Narrow strips (4 bytes of s4 = 8 channels, 8 bytes of s8 per lane) measured fastest on
     // MI355X: the loop is bound by the dequantising VALU work, not by load width, and narrow
     // strips give more workgroups to spread over the 256 CUs.  s8 from 33 tokens on took 4 bytes
-    // per lane (64-byte pieces of every row) until the factored mode got its 8-byte forms:
+    // per lane (64-byte pieces of every row) until the factored and rounded modes got their 8-byte forms:
     // [64,8192] x [8192,28672] 87.5 -> 58.5 us, 48 tokens 76 -> 49.
     // (fewer than 64 such strips leave the narrow ones ahead: more workgroups; 4096 x 4096 at 64 tokens
     // 17.5 us against 22.6)
-    int vec = s4 ? 4 : (mt >= 3 && (mode != kFactored || p.N % 8 != 0 || (p.N + 127) / 128 * p.batch < 64) ? 4 : 8);
+    // (the group-factored form of 8 bytes per lane at three or four token tiles spills 61-329 registers)
+    int vec = s4 ? 4 : (mt >= 3 && (mode == kGroupFactored || p.N % 8 != 0 || (p.N + 127) / 128 * p.batch < 64) ? 4 : 8);
     if (int v = GetOption("dequant_dot_vec")) vec = v;
     const int nv = vec * (s4 ? 2 : 1);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
@@ -892,6 +893,8 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
       XLA_AMD_DECODE(8, 16, 1, kRounded, "dequant_dot_decode_s8_v16_m16_rounded")
       XLA_AMD_DECODE(8, 8, 1, kRounded, "dequant_dot_decode_s8_v8_m16_rounded")
       XLA_AMD_DECODE(8, 8, 2, kRounded, "dequant_dot_decode_s8_v8_m32_rounded")
+      XLA_AMD_DECODE(8, 8, 3, kRounded, "dequant_dot_decode_s8_v8_m48_rounded")
+      XLA_AMD_DECODE(8, 8, 4, kRounded, "dequant_dot_decode_s8_v8_m64_rounded")
       XLA_AMD_DECODE(8, 4, 3, kRounded, "dequant_dot_decode_s8_v4_m48_rounded")
       XLA_AMD_DECODE(8, 4, 4, kRounded, "dequant_dot_decode_s8_v4_m64_rounded")
       XLA_AMD_DECODE(8, 16, 1, kFactored, "dequant_dot_decode_s8_v16_m16_factored")
