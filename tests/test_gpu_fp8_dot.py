@@ -491,7 +491,7 @@ def test_bf16_typed_multiply_without_scratch_takes_exact_kernel(oracle):
     w["a_scale"] = np.float32(0.3)
     types = dict(dequant_type="bf16")
     got, kern = run(w, scratch=None, **types)
-    assert kern == "fp8_scaled_dot_tiled_kn", kern   # followed by the exact kernel, which runs for this scale
+    assert kern == "fp8_dot_decode_kn_m64", kern   # followed by the exact kernel, which runs for this scale
     n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
     assert n_floor <= got.size // 100
 

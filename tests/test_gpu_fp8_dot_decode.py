@@ -225,6 +225,35 @@ def test_nan_codes_and_the_end_of_k(oracle, nk):
     assert np.allclose(got[finite], ref[finite], rtol=2.0 ** -7, atol=float(np.max(floor_for(w)[finite]))), kern
 
 
+@pytest.mark.parametrize("nk", [False, True])
+@pytest.mark.parametrize("M", [16, 48, 100])
+def test_bf16_typed_multiply(oracle, M, nk):
+    """A bf16-typed dequantise multiply with per-tensor scales: powers of two round nothing, the streaming
+    kernels serve the call and the result is that of the f32-typed call bit for bit; any other scale makes
+    them return at once and the bf16-operand kernels launched behind them (or, without their scratch,
+    the exact kernel) produce the result."""
+    say("fp8 streaming, bf16-typed multiply, M=%d nk=%s" % (M, nk))
+    K, N = 1024, 264
+    w = dict(workloads.c3_fp8(M, K, N), a_scale=np.float32(1 / 64), b_scale=np.float32(1 / 32))
+    types = dict(dequant_type="bf16")
+    out, kern = run(w, nk=nk, force=0, **types)
+    assert kern.startswith("fp8_dot_decode_%s_m" % ("nk" if nk else "kn")) and kern.endswith("|bf16_operands"), kern
+    plain, kern_plain = run(w, nk=nk, force=0)
+    assert kern == kern_plain + "|bf16_operands", (kern, kern_plain)
+    assert torch.equal(out, plain)
+    w2 = dict(w, a_scale=np.float32(0.3), b_scale=np.float32(0.013))
+    ref2 = reference(oracle, w2, **types)
+    out2, kern2 = run(w2, nk=nk, force=0, **types)
+    assert kern2 == kern, kern2
+    n_floor = check_dot(host_bf16(out2), ref2, floor_for(w2, exact_kernel=True), kern2)
+    assert n_floor <= max(8, out2.numel() // 50)
+    out3, kern3 = run(w2, nk=nk, force=0, scratch=None, **types)     # no scratch: one K-slice, then the exact kernel
+    assert kern3 == kern_plain.split(":")[0] or kern3 == kern_plain, kern3
+    check_dot(host_bf16(out3), ref2, floor_for(w2, exact_kernel=True), kern3)
+    out4, _ = run(w, nk=nk, force=0, scratch=None, **types)
+    check_dot(host_bf16(out4), reference(oracle, w, **types), floor_for(w), "pow2 scales, no scratch")
+
+
 def test_what_the_streaming_kernels_do_not_take():
     a = torch.zeros((2, 80, 64), dtype=torch.uint8, device="cuda")
     b = torch.zeros((2, 64, 64), dtype=torch.uint8, device="cuda")
@@ -234,7 +263,7 @@ def test_what_the_streaming_kernels_do_not_take():
         with pytest.raises(ffi.FfiError, match="only without a batch dimension"):
             ops.fp8_scaled_dot(a, b, one, one)      # 80 rows per batch
         with pytest.raises(ffi.FfiError, match="streaming kernels take"):
-            ops.fp8_scaled_dot(a[0, :8], b[0], one, one, dequant_type="bf16")
+            ops.fp8_scaled_dot(a[0, :8], b[0, :, :60].contiguous(), one, one)   # N % 8 != 0
     finally:
         ffi.set_option("fp8_dot_kernel", 0)
 

@@ -294,6 +294,14 @@ __device__ __forceinline__ void epilogue_all_dispatch(float* v, const float* bia
   }
 }
 
+// A normal power of two whose product with any finite f8e4m3fn value stays a normal bf16: scaling by it
+// is exact, so a bf16-typed dequantise multiply rounds nothing.
+__device__ __forceinline__ bool is_pow2_f32(float s) {
+  const uint32_t u = f32_to_bits(s);
+  const uint32_t e = (u >> 23) & 0xffu;
+  return (u & 0x807fffffu) == 0u && e > 24u && e < 230u;
+}
+
 // f(std::integral_constant<int, I>) for I = 0 .. N-1, expanded at compile time: unlike a loop under
 // `#pragma unroll`, which the compiler may decline for a large body, the index is a constant in
 // every copy, so arrays indexed by it stay in registers.

@@ -55,6 +55,10 @@ struct Fp8DecodeParams {
   int bf16_dot, bf16_ops, epilogue;
   int slices, rows_per_slice, rows_per_wave;  // rows_per_wave: a multiple of the kernel's step
   int cols;                                   // consecutive strips a workgroup takes, one after the other
+  // A bf16-typed dequantise multiply (per-tensor scales): with scales that are powers of two it rounds
+  // nothing and these kernels serve the call; otherwise every workgroup returns at once and the kernels
+  // launched behind them, which test the same condition the other way round, do.
+  int require_pow2_scales;
 };
 
 constexpr int kWaves = 8;
@@ -233,6 +237,7 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
 template <int MT, bool WALK>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
+  if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
   const int slice = blockIdx.x % p.slices;
   if constexpr (!WALK) {
     kn_strip<MT>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
@@ -406,6 +411,7 @@ __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, i
 template <int MT, bool MX, bool WALK>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
+  if (!MX && p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
   const int slice = blockIdx.x % p.slices;
   if constexpr (!WALK) {
     nk_strip<MT, MX>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
@@ -420,6 +426,7 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 
 // Sums the K-slices in slice order and finishes the values.
 __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeParams p) {
+  if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
   const size_t total = (size_t)p.M * p.N;
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   const int batch = blockIdx.y;
@@ -503,13 +510,13 @@ size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N
   return bytes;
 }
 
-static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply);
 
 // Returns -1 when the shape is not covered, else the launch status.
-int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
+int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply) {
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;
-  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream);
+  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream, bf16_multiply);
   if (p.batch > 1) return -1;
   int64_t rows = 0;
   const int passes = Passes(p.M, nk, mx, &rows);
@@ -523,7 +530,7 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     sub.out = (char*)p.out + (size_t)m0 * p.N * out_bytes;
     if (p.a_scale_per_row) sub.a_scale = p.a_scale + m0;
     if (mx) sub.a_block_scales = (const char*)p.a_block_scales + (size_t)m0 * (size_t)(p.K / 32);
-    const int rc = LaunchFp8DotDecodeRows(sub, stream);
+    const int rc = LaunchFp8DotDecodeRows(sub, stream, bf16_multiply);
     if (rc != 0) return rc;  // (-1 on the first pass: not covered; the passes differ in their row count only)
     if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)rows);
   }
@@ -531,7 +538,7 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   return 0;
 }
 
-static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply) {
   const int64_t batch = p.batch > 1 ? p.batch : 1;
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;
@@ -539,7 +546,11 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
   // (four token tiles of the [N,K] kernel do not fit the registers of two waves per SIMD: 48 rows there,
   // 32 with block scales)
   if (p.M <= 0 || p.M > (mx ? 32 : nk ? 48 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
-  if (p.dequant_type != XLA_FFI_DataType_F32) return -1;
+  // a bf16-typed dequantise multiply: only with per-tensor scales, and only as the caller says (it
+  // launches the kernels that take over when a scale is no power of two)
+  if (p.dequant_type != XLA_FFI_DataType_F32 &&
+      !(bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16 && !mx && !p.a_scale_per_row && !p.b_scale_per_channel))
+    return -1;
   // block scales: a step's four scales of a row move as one dword
   if (mx && (!nk || p.K % 128 != 0 || ((uintptr_t)p.a_block_scales % 4) || ((uintptr_t)p.b_block_scales % 4) ||
              (double)p.N * (p.K / 32) >= 2147483000.0))
@@ -566,6 +577,7 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
   dp.bf16_dot = p.dot_type == XLA_FFI_DataType_BF16;
   dp.bf16_ops = p.epilogue_type == XLA_FFI_DataType_BF16;
   dp.epilogue = p.epilogue;
+  dp.require_pow2_scales = p.dequant_type == XLA_FFI_DataType_BF16 ? 1 : 0;
   const int kStep = nk ? 128 : 32;
   int slices = Slices(batch, p.M, p.K, p.N, nk);
   const size_t need = (size_t)batch * slices * p.M * p.N * 4;

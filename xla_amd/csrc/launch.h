@@ -30,7 +30,9 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
 // cheaper than tiles.  Returns -1 when the shape is not covered (or tiles are cheaper), else the launch
 // status; p comes validated and an amax result already zeroed.  The scratch is the f32 sums of its
 // K-slices (0: one slice).
-int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
+// bf16_multiply: the caller takes care of a bf16-typed dequantise multiply whose per-tensor scales are no
+// powers of two (the kernels here then return at once); without it such calls are not covered.
+int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply = false);
 size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim);
 
 inline bool IsF32OrBf16(int32_t t) {

@@ -99,13 +99,6 @@ __device__ __forceinline__ float e8m0_to_f32(uint32_t e) {
   return e == 0xffu ? bits_to_f32(0x7fc00000u) : e == 0u ? bits_to_f32(0x00400000u) : bits_to_f32(e << 23);
 }
 
-__device__ __forceinline__ bool is_pow2_f32(float s) {
-  const uint32_t u = f32_to_bits(s);
-  const uint32_t e = (u >> 23) & 0xffu;
-  // normal power of two whose product with any finite f8 value stays a normal bf16
-  return (u & 0x807fffffu) == 0u && e > 24u && e < 230u;
-}
-
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
@@ -1390,7 +1383,7 @@ size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contr
   // (up to 64 rows the streaming kernels take the call, with the few exceptions that stay unsplit)
   if (!tiled) tiled = TailBytesFor(1, M, K, N, 65, kF8MaxTail);
   // up to 64 rows of a under f32-typed multiplies: the streaming kernels' K-slices instead
-  const size_t decode = dequant_type == XLA_FFI_DataType_BF16 ? 0 : Fp8DotDecodeWorkspaceBytes(1, M, K, N, rhs_contracting_dim);
+  const size_t decode = Fp8DotDecodeWorkspaceBytes(1, M, K, N, rhs_contracting_dim);
   return tiled > decode ? tiled : decode;
 }
 
@@ -1459,10 +1452,18 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     if (rc) return rc;
   }
   const int force = GetOption("fp8_dot_kernel");  // 0 auto, 1 exact (slow), 2 tiled, 3 streaming (up to 64 rows of a)
+  // A call with a bf16-typed multiply that the streaming kernels took: they have served it if both
+  // scales are powers of two; the kernels below that serve it otherwise are launched behind them.
+  bool streamed_if_pow2 = false;
+  char streamed_name[64] = "";
   if (force == 0 || force == 3) {
-    const int rc = LaunchFp8DotDecode(p, stream);
-    if (rc >= 0) return rc;
-    if (force == 3)
+    const bool bf16_multiply = p.dequant_type == XLA_FFI_DataType_BF16;
+    const int rc = LaunchFp8DotDecode(p, stream, bf16_multiply);
+    if (rc > 0 || (rc == 0 && !bf16_multiply)) return rc;
+    if (rc == 0) {
+      streamed_if_pow2 = true;
+      snprintf(streamed_name, sizeof(streamed_name), "%s", xla_amd_last_kernel());
+    } else if (force == 3)
       return Fail(XLA_FFI_Error_Code_FAILED_PRECONDITION,
                   "fp8_scaled_dot: the streaming kernels take K %% 8 == 0 and N %% 8 == 0, 8-byte aligned operands "
                   "and f32-typed multiplies; more than 64 rows of a (48 with the rhs [N,K], 32 with block scales) "
@@ -1495,7 +1496,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   // transposes on the way out of LDS (fp8_dot_layout = 1 forces the transposing pre-pass instead)
   const bool kn_direct = tiled_ok && !nk && p.N % 16 == 0 && ((uintptr_t)p.b % 16 == 0) &&
                          GetOption("fp8_dot_layout") != 1;
-  if (tiled_ok && !nk && !kn_direct) {
+  if (tiled_ok && !nk && !kn_direct && !streamed_if_pow2) {  // (streamed: no f8 tiled kernel will run)
     // (the pre-pass handles one matrix: a batched [K,N] rhs with ragged N takes the exact kernel)
     if (batch == 1 && p.workspace && p.workspace_bytes >= (size_t)p.K * p.N && ((uintptr_t)p.workspace % 16 == 0)) {
       if (p.N % 4 == 0 && ((uintptr_t)p.b % 4 == 0)) {
@@ -1539,7 +1540,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
       ((uintptr_t)p.out % 8) == 0) {
     int rc = 0;
     const bool by_value = !vector_scales;  // the f8 kernel may serve the call: both decide from the scale values
-    if (by_value && tiled_ok) {
+    if (by_value && tiled_ok && !streamed_if_pow2) {
       TiledParams tt = tp;
       tt.b = b_nk;
       rc = kn_direct ? launch_tiled<kFp8KN>(tt, 1, stream, "fp8_scaled_dot_tiled_kn") : launch_tiled<kFp8>(tt, 1, stream, "fp8_scaled_dot_tiled");
@@ -1547,7 +1548,7 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     }
     uint16_t* a16 = (uint16_t*)((char*)p.workspace + ops_at);
     uint16_t* b16 = (uint16_t*)((char*)a16 + RoundUp256((size_t)p.M * p.K * 2));
-    const int skip = by_value && tiled_ok ? 1 : 0;
+    const int skip = (by_value && tiled_ok) || streamed_if_pow2 ? 1 : 0;
     hipLaunchKernelGGL(f8_to_scaled_bf16_kernel<false>, dim3((unsigned)((p.K + 255) / 256), (unsigned)((p.M + 63) / 64)), dim3(256), 0,
                        stream, (const uint8_t*)p.a, a16, (int)p.M, (int)p.K, p.a_scale, tp.a_per_row ? 1 : 0, p.b_scale, skip);
     if (nk)
@@ -1566,9 +1567,22 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
     tb.a_per_row = tb.b_per_channel = 0;  // already in the operands
     rc = launch_tiled<kBf16>(tb, 1, stream, "fp8_scaled_dot_bf16_operands");
     if (rc) return rc;
+    if (streamed_if_pow2) {
+      char name[96];
+      snprintf(name, sizeof(name), "%s|bf16_operands", streamed_name);
+      SetLastKernel(name);
+      return 0;
+    }
     SetLastKernel(skip ? (kn_direct ? "fp8_scaled_dot_tiled_kn|bf16_operands" : nk ? "fp8_scaled_dot_tiled|bf16_operands"
                                                                                     : "fp8_scaled_dot_tiled+transpose|bf16_operands")
                        : "fp8_scaled_dot_bf16_operands");
+    return 0;
+  }
+  if (streamed_if_pow2) {  // (no scratch for the bf16 operands: the exact kernel, if a scale is no power of two)
+    hipLaunchKernelGGL(fp8_dot_exact_kernel, egrid, dim3(256), 0, stream, tp, nk ? 1 : 0, 1, 1);
+    const int rc = CheckLaunch("fp8_scaled_dot_exact");
+    if (rc) return rc;
+    SetLastKernel(streamed_name);
     return 0;
   }
   if (tiled_ok) {
