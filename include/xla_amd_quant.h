@@ -312,6 +312,10 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * that kernel: 64 or 128), "handover_test" (1: workgroups that hand partial sums over never raise their
  * flags and the waiting side gives up after 16 polls, so that its own fallback computes the result --
  * for tests of that fallback only), "fp8_dot_kernel" (1 exact, 2 tiled, 3 streaming), "fp8_decode_slices" (K-slices of the streaming kernels),
+ * "fp8_scales_on_sum" (1: a bf16-typed dequantise multiply of xla_amd.fp8_scaled_dot is computed as the
+ * reference's GPU pipeline computes that HLO -- scales on the f32 sum, gemm_rewriter.cc:1235-1591 -- not
+ * op by op: no rounding of a * a_scale and b * b_scale to bf16, so scales that are no powers of two keep
+ * the fp8 kernels; differs from the op-by-op value by up to the bf16 rounding of the operands),
  * "quantize_variant", "fp8_dot_layout" (1: transpose a [K,N] rhs in a pre-pass), "tiled_epilogue" (1:
  * the tiled kernels compute f32-typed GELU / SiLU from x * sigmoid(.) with the hardware exponential
  * instead of op by op as the HLO does; faster, but the far negative tail no longer matches the

@@ -254,6 +254,26 @@ def test_bf16_typed_multiply(oracle, M, nk):
     check_dot(host_bf16(out4), reference(oracle, w, **types), floor_for(w), "pow2 scales, no scratch")
 
 
+def test_scales_on_the_sum_option(oracle):
+    """fp8_scales_on_sum = 1: a bf16-typed multiply with any scale is the f32-typed call (what the reference's
+    GPU pipeline computes for that HLO), at decode size on the streaming kernels."""
+    say("fp8 bf16-typed multiply computed with the scales on the sum")
+    # (scales that are bf16 numbers, as the parameters of a bf16-typed module are, and no powers of two)
+    w = dict(workloads.c3_fp8(16, 1024, 264), a_scale=np.float32(77 / 256), b_scale=np.float32(213 / 16384))
+    plain, kern_plain = run(w, force=0)
+    ffi.set_option("fp8_scales_on_sum", 1)
+    try:
+        out, kern = run(w, force=0, dequant_type="bf16")
+    finally:
+        ffi.set_option("fp8_scales_on_sum", 0)
+    assert kern == kern_plain == "fp8_dot_decode_kn_m16", (kern, kern_plain)
+    assert torch.equal(out, plain)
+    # and close to the op-by-op value as a whole (that value rounds every a * a_scale and b * b_scale to bf16)
+    ref = dtypes.bf16_to_f32(reference(oracle, w, dequant_type="bf16")).astype(np.float64)
+    got = dtypes.bf16_to_f32(host_bf16(out)).astype(np.float64)
+    assert np.linalg.norm(got - ref) <= 1e-2 * np.linalg.norm(ref), np.linalg.norm(got - ref) / np.linalg.norm(ref)
+
+
 def test_what_the_streaming_kernels_do_not_take():
     a = torch.zeros((2, 80, 64), dtype=torch.uint8, device="cuda")
     b = torch.zeros((2, 64, 64), dtype=torch.uint8, device="cuda")

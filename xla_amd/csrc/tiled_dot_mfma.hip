@@ -1388,6 +1388,14 @@ size_t Fp8ScaledDotWorkspaceBytes(int64_t M, int64_t K, int64_t N, int rhs_contr
 }
 
 int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
+  // Opt-in: a bf16-typed dequantise multiply computed the way the reference's GPU pipeline computes the
+  // same HLO (GemmRewriter turns it into an FP8 matmul whose scales multiply the f32 sum,
+  // gemm_rewriter.cc:1235-1591), not op by op: the f32-typed call.
+  if (p.dequant_type == XLA_FFI_DataType_BF16 && GetOption("fp8_scales_on_sum") == 1) {
+    XlaAmdFp8ScaledDot q = p;
+    q.dequant_type = XLA_FFI_DataType_F32;
+    return LaunchFp8ScaledDot(q, stream);
+  }
   if (p.M < 0 || p.K < 0 || p.N < 0 || p.M > 0x7fffffff || p.K > 0x7fffffff || p.N > 0x7fffffff)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "fp8_scaled_dot: bad shape");
   if (p.rhs_contracting_dim != 0 && p.rhs_contracting_dim != 1)
