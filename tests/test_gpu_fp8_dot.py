@@ -452,7 +452,8 @@ def test_bf16_typed_multiply_with_any_scale(oracle, M, K, N, nk):
     types = dict(dequant_type="bf16")
     got, kern = run(w, nk=nk, **types)
     # K % 16 != 0 keeps the f8 kernel out altogether; otherwise both are enqueued and the scales decide
-    assert kern == ("fp8_scaled_dot_bf16_operands" if K % 16 else kern) and kern.endswith("bf16_operands"), kern
+    # (64 rows of a [K,N] rhs: the streaming kernels' own rounding form, "|rounded")
+    assert kern == ("fp8_scaled_dot_bf16_operands" if K % 16 else kern) and kern.endswith(("bf16_operands", "|rounded")), kern
     n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
     assert n_floor <= max(8, got.size // 50)
     exact, kern2 = run(w, nk=nk, force=1, **types)
@@ -460,7 +461,7 @@ def test_bf16_typed_multiply_with_any_scale(oracle, M, K, N, nk):
     check_dot(exact, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern2)
     w2 = dict(w, a_scale=np.float32(1 / 64), b_scale=np.float32(1 / 32))
     got2, kern3 = run(w2, nk=nk, **types)
-    assert kern3.endswith("bf16_operands"), kern3
+    assert kern3.endswith(("bf16_operands", "|rounded")), kern3
     if K % 16 == 0:
         plain, _ = run(w2, nk=nk)   # f32-typed: the f8 kernel alone; identical values for power-of-two scales
         assert np.array_equal(got2, plain)
@@ -491,7 +492,7 @@ def test_bf16_typed_multiply_without_scratch_takes_exact_kernel(oracle):
     w["a_scale"] = np.float32(0.3)
     types = dict(dequant_type="bf16")
     got, kern = run(w, scratch=None, **types)
-    assert kern == "fp8_dot_decode_kn_m64", kern   # followed by the exact kernel, which runs for this scale
+    assert kern == "fp8_dot_decode_kn_m64|rounded", kern   # the form that rounds the scaled operands runs for this scale
     n_floor = check_dot(got, reference(oracle, w, **types), floor_for(w, exact_kernel=True), kern)
     assert n_floor <= got.size // 100
 

@@ -236,22 +236,47 @@ def test_bf16_typed_multiply(oracle, M, nk):
     K, N = 1024, 264
     w = dict(workloads.c3_fp8(M, K, N), a_scale=np.float32(1 / 64), b_scale=np.float32(1 / 32))
     types = dict(dequant_type="bf16")
+    # rhs [K,N]: the streaming kernels' own form that rounds the scaled operands to bf16 stands behind the f8
+    # form ("|rounded"); rhs [N,K]: the bf16-operand pre-passes and tiled kernel do
+    tag = "|bf16_operands" if nk else "|rounded"
     out, kern = run(w, nk=nk, force=0, **types)
-    assert kern.startswith("fp8_dot_decode_%s_m" % ("nk" if nk else "kn")) and kern.endswith("|bf16_operands"), kern
+    assert kern.startswith("fp8_dot_decode_%s_m" % ("nk" if nk else "kn")) and kern.endswith(tag), kern
     plain, kern_plain = run(w, nk=nk, force=0)
-    assert kern == kern_plain + "|bf16_operands", (kern, kern_plain)
+    assert kern == kern_plain + tag, (kern, kern_plain)
     assert torch.equal(out, plain)
     w2 = dict(w, a_scale=np.float32(0.3), b_scale=np.float32(0.013))
     ref2 = reference(oracle, w2, **types)
-    out2, kern2 = run(w2, nk=nk, force=0, **types)
-    assert kern2 == kern, kern2
-    n_floor = check_dot(host_bf16(out2), ref2, floor_for(w2, exact_kernel=True), kern2)
-    assert n_floor <= max(8, out2.numel() // 50)
-    out3, kern3 = run(w2, nk=nk, force=0, scratch=None, **types)     # no scratch: one K-slice, then the exact kernel
-    assert kern3 == kern_plain.split(":")[0] or kern3 == kern_plain, kern3
+    for slices in ((0,) if nk else (0, 2)):   # (forced slices size the scratch for the streaming kernels alone)
+        out2, kern2 = run(w2, nk=nk, force=0, slices=slices, **types)
+        assert kern2 == kern, kern2
+        n_floor = check_dot(host_bf16(out2), ref2, floor_for(w2, exact_kernel=True), "%s, %d slices" % (kern2, slices))
+        assert n_floor <= max(8, out2.numel() // 50)
+    out3, kern3 = run(w2, nk=nk, force=0, scratch=None, **types)     # no scratch: one K-slice ([N,K]: then the exact kernel)
+    assert kern3 == kern_plain + ("" if nk else "|rounded"), kern3
     check_dot(host_bf16(out3), ref2, floor_for(w2, exact_kernel=True), kern3)
     out4, _ = run(w, nk=nk, force=0, scratch=None, **types)
     check_dot(host_bf16(out4), reference(oracle, w, **types), floor_for(w), "pow2 scales, no scratch")
+
+
+def test_rounded_operands_read_every_code_back_exactly():
+    """The form that rounds the scaled operands, on one-hot rows: output [m, n] is
+    bf16(bf16(1 * 0.75) * bf16(b[k_m, n] * 0.3125)) for every f8 code at every position of a step -- the
+    hardware widening of each code, the rounding of the product and the k order of both operands."""
+    say("fp8 streaming, rounded operands, one-hot")
+    M, K, N = 32, 384, 256
+    ks = (np.arange(M) * 37 + 5) % K
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), ks] = 1.0
+    b8 = ((np.arange(K)[:, None] * 7 + np.arange(N)[None, :]) % 256).astype(np.uint8)
+    b8[(b8 & 0x7F) == 0x7F] = 0x3A
+    w = dict(a=dtypes.f32_to_f8e4m3fn(a), b=b8, a_scale=np.float32(0.75), b_scale=np.float32(0.3125), bias=None,
+             epilogue="DEFAULT")
+    bs = dtypes.bf16_to_f32(dtypes.f32_to_bf16(dtypes.f8e4m3fn_to_f32(b8[ks]) * np.float32(0.3125)))
+    want = dtypes.f32_to_bf16(np.float32(0.75) * bs)
+    for slices in (0, 2):
+        out, kern = run(w, slices=slices, force=0, dequant_type="bf16")
+        assert kern == "fp8_dot_decode_kn_m32|rounded", kern
+        assert np.array_equal(dtypes.bf16_to_f32(host_bf16(out)), dtypes.bf16_to_f32(want)), slices
 
 
 def test_scales_on_the_sum_option(oracle):

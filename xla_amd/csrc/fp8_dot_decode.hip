@@ -26,6 +26,7 @@
 // Bound: HBM.  Algorithmic bytes: K*N (rhs) + a, scales, bias and out once each.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
 #include <stdio.h>
 
 #include "decode_common.h"
@@ -59,6 +60,10 @@ struct Fp8DecodeParams {
   // nothing and these kernels serve the call; otherwise every workgroup returns at once and the kernels
   // launched behind them, which test the same condition the other way round, do.
   int require_pow2_scales;
+  // The kernels that take over then (rhs [K,N]): every a * a_scale and b * b_scale rounded to bf16 on the way
+  // into the bf16 matrix instruction, the scales therefore no longer on the sum; they return at once
+  // when both scales are powers of two.
+  int rounded_operands;
 };
 
 constexpr int kWaves = 8;
@@ -104,7 +109,8 @@ __device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int li = lane & 15, kb = lane >> 4;
   // (block scales went in with the matrix instructions)
-  const float alpha = p.a_block_scales ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+  const float alpha = p.a_block_scales || p.rounded_operands
+                          ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
   uint32_t amax_bits = 0u;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -139,7 +145,9 @@ __device__ __forceinline__ void reduce_and_store(const Fp8DecodeParams& p, float
 
 // rhs [K,N].  MT: 16-token tiles.  A workgroup owns 128 channels (one 128-byte line per row) and
 // rows_per_slice rows, its waves rows_per_wave consecutive rows each, in steps of 32.
-template <int MT>
+// ROUNDED: the operands are widened, scaled and rounded to bf16 (16 vector instructions per 8 values) and
+// multiplied by v_mfma_f32_16x16x32_bf16, which takes the same 8 consecutive k per lane.
+template <int MT, bool ROUNDED>
 __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, int strip, int slice, int batch) {
   int lane = threadIdx.x & 63;
   // (opaque to the compiler, so that a strip's descriptors and offsets are made anew for every strip of
@@ -176,6 +184,20 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
   const int k_begin = slice * p.rows_per_slice + wave * p.rows_per_wave;
   const int k_stop = min(k_begin + p.rows_per_wave, slice_end);
 
+  float sa_r = 1.0f, sb_r = 1.0f;
+  if constexpr (ROUNDED) {
+    sa_r = round_bf16(*p.a_scale);
+    sb_r = round_bf16(*p.b_scale);
+  }
+  // 8 f8e4m3fn codes (k in byte order) -> bf16(code * s), one rounding each
+  auto scaled_bf16 = [&](uint32_t lo, uint32_t hi, float s) {
+    const floatx2 f0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false), f1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+    const floatx2 f2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false), f3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+    const uintx4 o = {pack_bf16x2(f0[0] * s, f0[1] * s), pack_bf16x2(f1[0] * s, f1[1] * s),
+                      pack_bf16x2(f2[0] * s, f2[1] * s), pack_bf16x2(f3[0] * s, f3[1] * s)};
+    return __builtin_bit_cast(bf16x8, o);
+  };
+
   uintx2 wq[2][8];
   uintx2 aq[2][MT];
   auto load_step = [&](int buf, int k0) {
@@ -195,6 +217,11 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) av[mt] = uintx2{ok ? av[mt][0] : 0u, ok ? av[mt][1] : 0u};
     }
+    bf16x8 ab[MT];
+    if constexpr (ROUNDED) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) ab[mt] = scaled_bf16(av[mt][0], av[mt][1], sa_r);
+    }
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       // 4x4 byte transposes: t[h][e] = byte e of rows 4h .. 4h+3 of dword q
@@ -211,11 +238,18 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const long wop = __builtin_bit_cast(long, uintx2{t[0][e], t[1][e]});
+        if constexpr (ROUNDED) {
+          const bf16x8 wb = scaled_bf16(t[0][e], t[1][e], sb_r);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          acc[4 * q + e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wop, __builtin_bit_cast(long, av[mt]),
-                                                                          acc[4 * q + e][mt], 0, 0, 0);
+          for (int mt = 0; mt < MT; ++mt)
+            acc[4 * q + e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, ab[mt], acc[4 * q + e][mt], 0, 0, 0);
+        } else {
+          const long wop = __builtin_bit_cast(long, uintx2{t[0][e], t[1][e]});
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[4 * q + e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wop, __builtin_bit_cast(long, av[mt]),
+                                                                            acc[4 * q + e][mt], 0, 0, 0);
+        }
       }
     }
   };
@@ -234,18 +268,22 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
 // WALK: a workgroup takes p.cols consecutive strips one after the other (more strips than CUs: one
 // resident workgroup per CU that walks several strips finishes sooner than workgroups queueing for CUs;
 // a kernel of its own, because the loop costs the one-strip form registers).
-template <int MT, bool WALK>
+template <int MT, bool WALK, bool ROUNDED = false>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
-  if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
+  if constexpr (ROUNDED) {
+    if (is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;  // the f8 form has served the call
+  } else {
+    if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
+  }
   const int slice = blockIdx.x % p.slices;
   if constexpr (!WALK) {
-    kn_strip<MT>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
+    kn_strip<MT, ROUNDED>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
   } else {
     const int first = (blockIdx.x / p.slices) * p.cols;
     for (int c = 0; c < p.cols && (first + c) * 128 < p.N; ++c) {
       if (c) __syncthreads();  // the sums of the strip before have left LDS
-      kn_strip<MT>(p, lds, first + c, slice, blockIdx.y);
+      kn_strip<MT, ROUNDED>(p, lds, first + c, slice, blockIdx.y);
     }
   }
 }
@@ -426,7 +464,11 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 
 // Sums the K-slices in slice order and finishes the values.
 __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeParams p) {
-  if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
+  if (p.rounded_operands) {
+    if (is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;
+  } else if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) {
+    return;
+  }
   const size_t total = (size_t)p.M * p.N;
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   const int batch = blockIdx.y;
@@ -435,7 +477,8 @@ __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeP
     const float* ws = p.partial + (size_t)batch * p.slices * total + idx;
     float v = 0.0f;
     for (int s = 0; s < p.slices; ++s) v = v + ws[(size_t)s * total];
-    const float alpha = p.a_block_scales ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
+    const float alpha = p.a_block_scales || p.rounded_operands
+                            ? 1.0f : (p.a_per_row ? 1.0f : *p.a_scale) * (p.b_per_channel ? 1.0f : *p.b_scale);
     finish_value(p, batch, (int)(idx / p.N), (int)(idx % p.N), v, alpha, &amax_bits);
   }
   fold_amax(p, amax_bits);
@@ -510,13 +553,16 @@ size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N
   return bytes;
 }
 
-static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply);
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply, bool* any_scale);
 
 // Returns -1 when the shape is not covered, else the launch status.
-int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply) {
+int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply, bool* any_scale) {
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;
-  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream, bf16_multiply);
+  bool dummy = false;
+  if (!any_scale) any_scale = &dummy;
+  *any_scale = false;
+  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream, bf16_multiply, any_scale);
   if (p.batch > 1) return -1;
   int64_t rows = 0;
   const int passes = Passes(p.M, nk, mx, &rows);
@@ -530,15 +576,20 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf1
     sub.out = (char*)p.out + (size_t)m0 * p.N * out_bytes;
     if (p.a_scale_per_row) sub.a_scale = p.a_scale + m0;
     if (mx) sub.a_block_scales = (const char*)p.a_block_scales + (size_t)m0 * (size_t)(p.K / 32);
-    const int rc = LaunchFp8DotDecodeRows(sub, stream, bf16_multiply);
+    const int rc = LaunchFp8DotDecodeRows(sub, stream, bf16_multiply, any_scale);
     if (rc != 0) return rc;  // (-1 on the first pass: not covered; the passes differ in their row count only)
-    if (!name[0]) snprintf(name, sizeof(name), "%s:x%d", xla_amd_last_kernel(), (int)rows);
+    if (!name[0]) {
+      char base[48];
+      snprintf(base, sizeof(base), "%s", xla_amd_last_kernel());
+      if (char* bar = strchr(base, '|')) *bar = 0;
+      snprintf(name, sizeof(name), "%s:x%d%s", base, (int)rows, *any_scale ? "|rounded" : "");
+    }
   }
   SetLastKernel(name);
   return 0;
 }
 
-static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply) {
+static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply, bool* any_scale) {
   const int64_t batch = p.batch > 1 ? p.batch : 1;
   const bool nk = p.rhs_contracting_dim == 1;
   const bool mx = p.a_block_scales != nullptr;
@@ -630,11 +681,34 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
     rc = CheckLaunch("fp8_dot_decode_finalize");
     if (rc) return rc;
   }
+  // A bf16-typed multiply on a [K,N] rhs: the same launches again in the form that rounds the scaled
+  // operands to bf16, for scales that are no powers of two (one strip per workgroup).
+  if (dp.require_pow2_scales && !nk) {
+    Fp8DecodeParams dr = dp;
+    dr.require_pow2_scales = 0;
+    dr.rounded_operands = 1;
+    dr.cols = 1;
+    const dim3 rgrid((unsigned)(strips * slices), (unsigned)batch);
+    if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<1, false, true>), rgrid, block, 0, stream, dr);
+    else if (mt == 2) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<2, false, true>), rgrid, block, 0, stream, dr);
+    else if (mt == 3) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<3, false, true>), rgrid, block, 0, stream, dr);
+    else hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<4, false, true>), rgrid, block, 0, stream, dr);
+    rc = CheckLaunch("fp8_dot_decode_rounded");
+    if (rc) return rc;
+    if (slices > 1) {
+      dim3 fgrid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)batch);
+      hipLaunchKernelGGL(fp8_dot_decode_finalize_kernel, fgrid, dim3(256), 0, stream, dr);
+      rc = CheckLaunch("fp8_dot_decode_finalize");
+      if (rc) return rc;
+    }
+    *any_scale = true;
+  }
   static const char* names[2][4] = {{"fp8_dot_decode_kn_m16", "fp8_dot_decode_kn_m32", "fp8_dot_decode_kn_m48", "fp8_dot_decode_kn_m64"},
                                     {"fp8_dot_decode_nk_m16", "fp8_dot_decode_nk_m32", "fp8_dot_decode_nk_m48", "fp8_dot_decode_nk_m64"}};
   static const char* mx_names[2] = {"fp8_dot_decode_mx_m16", "fp8_dot_decode_mx_m32"};
-  char name[48];
-  snprintf(name, sizeof(name), "%s%s", mx ? mx_names[mt - 1] : names[nk ? 1 : 0][mt - 1], cols > 1 ? ":walk" : "");
+  char name[56];
+  snprintf(name, sizeof(name), "%s%s%s", mx ? mx_names[mt - 1] : names[nk ? 1 : 0][mt - 1], cols > 1 ? ":walk" : "",
+           *any_scale ? "|rounded" : "");
   SetLastKernel(name);
   return 0;
 }

@@ -32,7 +32,9 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream);
 // K-slices (0: one slice).
 // bf16_multiply: the caller takes care of a bf16-typed dequantise multiply whose per-tensor scales are no
 // powers of two (the kernels here then return at once); without it such calls are not covered.
-int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply = false);
+// *any_scale (if given): the launches also cover scales that are no powers of two (rhs [K,N]).
+int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf16_multiply = false,
+                       bool* any_scale = nullptr);
 size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N, int rhs_contracting_dim);
 
 inline bool IsF32OrBf16(int32_t t) {

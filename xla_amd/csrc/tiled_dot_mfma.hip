@@ -1466,8 +1466,9 @@ int LaunchFp8ScaledDot(const XlaAmdFp8ScaledDot& p, hipStream_t stream) {
   char streamed_name[64] = "";
   if (force == 0 || force == 3) {
     const bool bf16_multiply = p.dequant_type == XLA_FFI_DataType_BF16;
-    const int rc = LaunchFp8DotDecode(p, stream, bf16_multiply);
-    if (rc > 0 || (rc == 0 && !bf16_multiply)) return rc;
+    bool any_scale = false;
+    const int rc = LaunchFp8DotDecode(p, stream, bf16_multiply, &any_scale);
+    if (rc > 0 || (rc == 0 && (!bf16_multiply || any_scale))) return rc;
     if (rc == 0) {
       streamed_if_pow2 = true;
       snprintf(streamed_name, sizeof(streamed_name), "%s", xla_amd_last_kernel());
