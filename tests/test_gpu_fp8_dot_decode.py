@@ -258,6 +258,29 @@ def test_bf16_typed_multiply(oracle, M, nk):
     check_dot(host_bf16(out4), reference(oracle, w, **types), floor_for(w), "pow2 scales, no scratch")
 
 
+@pytest.mark.parametrize("which", ["a", "b", "ab"])
+@pytest.mark.parametrize("M", [20, 64])
+def test_bf16_typed_multiply_with_vector_scales(oracle, which, M):
+    """Per-row and per-channel scales under a bf16-typed multiply (no single test tells whether they round
+    anything): the rounding form of the [K,N] kernel runs alone, each operand scaled by its row's or its
+    channel's scale."""
+    say("fp8 streaming, bf16-typed multiply, vector scales %s, M=%d" % (which, M))
+    K, N = 1024, 200
+    w = workloads.c3_fp8(M, K, N)
+    rng = np.random.default_rng(5)
+    if "a" in which:
+        w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+    if "b" in which:
+        w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+    types = dict(dequant_type="bf16")
+    ref = reference(oracle, w, **types)
+    for slices in (0, 2):
+        out, kern = run(w, force=0, slices=slices, **types)
+        assert kern == tile_name(False, M) + "|rounded", kern
+        n_floor = check_dot(host_bf16(out), ref, floor_for(w, exact_kernel=True), "%s, %d slices" % (kern, slices))
+        assert n_floor <= max(8, out.numel() // 50)
+
+
 def test_rounded_operands_read_every_code_back_exactly():
     """The form that rounds the scaled operands, on one-hot rows: output [m, n] is
     bf16(bf16(1 * 0.75) * bf16(b[k_m, n] * 0.3125)) for every f8 code at every position of a step -- the

@@ -62,7 +62,8 @@ struct Fp8DecodeParams {
   int require_pow2_scales;
   // The kernels that take over then (rhs [K,N]): every a * a_scale and b * b_scale rounded to bf16 on the way
   // into the bf16 matrix instruction, the scales therefore no longer on the sum; they return at once
-  // when both scales are powers of two.
+  // when both scales are powers of two (1), or run whatever the scales are (2: per-row or per-channel
+  // scales, which no single test covers: the f8 form is not launched then).
   int rounded_operands;
 };
 
@@ -73,8 +74,10 @@ constexpr uint32_t kNowhere = 0x80000000u;  // a lane offset no buffer reaches: 
 __device__ __forceinline__ void finish_value(const Fp8DecodeParams& p, int batch, int m, int n, float sum, float alpha,
                                              uint32_t* amax_bits) {
   float v = sum;
-  if (p.a_per_row) v = v * p.a_scale[m];
-  v = v * (p.b_per_channel ? alpha * p.b_scale[n] : alpha);
+  if (!p.rounded_operands) {
+    if (p.a_per_row) v = v * p.a_scale[m];
+    v = v * (p.b_per_channel ? alpha * p.b_scale[n] : alpha);
+  }
   const float bias = p.bias ? load_scale(p.bias, n, p.bias_is_bf16) : 0.0f;
   v = epilogue_dispatch(v, bias, p.epilogue, p.bf16_dot, p.bf16_ops);
   const size_t idx = ((size_t)batch * p.M + m) * p.N + n;
@@ -184,10 +187,13 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
   const int k_begin = slice * p.rows_per_slice + wave * p.rows_per_wave;
   const int k_stop = min(k_begin + p.rows_per_wave, slice_end);
 
-  float sa_r = 1.0f, sb_r = 1.0f;
+  // the lane's operands: token 16 mt + li of a, channels n_lane .. n_lane + 7 of the rhs
+  float sa_r[MT], sb_r[8];
   if constexpr (ROUNDED) {
-    sa_r = round_bf16(*p.a_scale);
-    sb_r = round_bf16(*p.b_scale);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) sa_r[mt] = round_bf16(p.a_per_row ? p.a_scale[min(16 * mt + li, p.M - 1)] : *p.a_scale);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sb_r[j] = round_bf16(p.b_per_channel ? p.b_scale[min(n_lane + j, p.N - 1)] : *p.b_scale);
   }
   // 8 f8e4m3fn codes (k in byte order) -> bf16(code * s), one rounding each
   auto scaled_bf16 = [&](uint32_t lo, uint32_t hi, float s) {
@@ -220,7 +226,7 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
     bf16x8 ab[MT];
     if constexpr (ROUNDED) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) ab[mt] = scaled_bf16(av[mt][0], av[mt][1], sa_r);
+      for (int mt = 0; mt < MT; ++mt) ab[mt] = scaled_bf16(av[mt][0], av[mt][1], sa_r[mt]);
     }
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
@@ -239,7 +245,7 @@ __device__ __forceinline__ void kn_strip(const Fp8DecodeParams& p, float* lds, i
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if constexpr (ROUNDED) {
-          const bf16x8 wb = scaled_bf16(t[0][e], t[1][e], sb_r);
+          const bf16x8 wb = scaled_bf16(t[0][e], t[1][e], sb_r[4 * q + e]);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             acc[4 * q + e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, ab[mt], acc[4 * q + e][mt], 0, 0, 0);
@@ -272,7 +278,7 @@ template <int MT, bool WALK, bool ROUNDED = false>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
   if constexpr (ROUNDED) {
-    if (is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;  // the f8 form has served the call
+    if (p.rounded_operands == 1 && is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;  // the f8 form has served the call
   } else {
     if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
   }
@@ -465,7 +471,7 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8Decod
 // Sums the K-slices in slice order and finishes the values.
 __global__ __launch_bounds__(256) void fp8_dot_decode_finalize_kernel(Fp8DecodeParams p) {
   if (p.rounded_operands) {
-    if (is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;
+    if (p.rounded_operands == 1 && is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;
   } else if (p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) {
     return;
   }
@@ -597,11 +603,14 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
   // (four token tiles of the [N,K] kernel do not fit the registers of two waves per SIMD: 48 rows there,
   // 32 with block scales)
   if (p.M <= 0 || p.M > (mx ? 32 : nk ? 48 : 64) || p.K <= 0 || p.K % align != 0 || p.N % 8 != 0) return -1;
-  // a bf16-typed dequantise multiply: only with per-tensor scales, and only as the caller says (it
-  // launches the kernels that take over when a scale is no power of two)
+  // a bf16-typed dequantise multiply: only as the caller says (for an [N,K] rhs it launches the kernels
+  // that take over when a scale is no power of two); vectors of scales only on a [K,N] rhs, whose
+  // rounding form then runs alone
+  const bool vector_scales = p.a_scale_per_row || p.b_scale_per_channel;
   if (p.dequant_type != XLA_FFI_DataType_F32 &&
-      !(bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16 && !mx && !p.a_scale_per_row && !p.b_scale_per_channel))
+      !(bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16 && !mx && !(nk && vector_scales)))
     return -1;
+  const bool only_rounded = p.dequant_type == XLA_FFI_DataType_BF16 && vector_scales;
   // block scales: a step's four scales of a row move as one dword
   if (mx && (!nk || p.K % 128 != 0 || ((uintptr_t)p.a_block_scales % 4) || ((uintptr_t)p.b_block_scales % 4) ||
              (double)p.N * (p.K / 32) >= 2147483000.0))
@@ -659,7 +668,9 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
     if (cols > 1) hipLaunchKernelGGL((KERNEL<__VA_ARGS__, true>), grid, block, 0, stream, dp);      \
     else hipLaunchKernelGGL((KERNEL<__VA_ARGS__, false>), grid, block, 0, stream, dp);              \
   } while (0)
-  if (nk && mx) {
+  if (only_rounded) {
+    // (the f8 form cannot tell from one value whether a vector of scales rounds anything)
+  } else if (nk && mx) {
     if (mt == 1) XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 1, true);
     else XLA_AMD_LAUNCH_FP8_DECODE(fp8_dot_decode_nk_kernel, 2, true);
   } else if (nk) {
@@ -675,7 +686,7 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
 #undef XLA_AMD_LAUNCH_FP8_DECODE
   int rc = CheckLaunch("fp8_dot_decode");
   if (rc) return rc;
-  if (slices > 1) {
+  if (slices > 1 && !only_rounded) {
     dim3 fgrid((unsigned)(((size_t)p.M * p.N + 255) / 256), (unsigned)batch);
     hipLaunchKernelGGL(fp8_dot_decode_finalize_kernel, fgrid, dim3(256), 0, stream, dp);
     rc = CheckLaunch("fp8_dot_decode_finalize");
@@ -686,7 +697,7 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
   if (dp.require_pow2_scales && !nk) {
     Fp8DecodeParams dr = dp;
     dr.require_pow2_scales = 0;
-    dr.rounded_operands = 1;
+    dr.rounded_operands = only_rounded ? 2 : 1;
     dr.cols = 1;
     const dim3 rgrid((unsigned)(strips * slices), (unsigned)batch);
     if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<1, false, true>), rgrid, block, 0, stream, dr);
