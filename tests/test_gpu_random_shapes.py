@@ -113,6 +113,39 @@ def test_fp8_dot_random_shapes(oracle):
         assert n_floor <= max(8, got.size // 20)
 
 
+def test_fp8_dot_bf16_typed_random_shapes(oracle):
+    """A bf16-typed dequantise multiply over row counts on both sides of what one streaming launch takes,
+    K long enough for passes to be chosen, scales that are powers of two, that are not, and vectors: whichever
+    of the f8 kernels, their rounding form, the bf16-operand kernels and the exact kernel the launcher picks."""
+    rng = np.random.default_rng(78)
+    kernels = set()
+    for case in range(18):
+        M = int(rng.choice([1, 20, 48, 49, 64, 65, 96, 130]))
+        K = 16 * int(rng.choice([8, 33, 64, 128, 200]))
+        N = int(rng.choice([40, 64, 200, 264]))
+        nk = bool(rng.integers(0, 2))
+        w = workloads.c3_fp8(M, K, N)
+        w["epilogue"] = EPILOGUES[int(rng.integers(0, 8))]
+        if "BIAS" not in w["epilogue"]:
+            w["bias"] = None
+        kind = int(rng.integers(0, 4))   # 0: powers of two, 1: any scalar, 2: per-row a, 3: both vectors
+        if kind == 0:
+            w["a_scale"], w["b_scale"] = np.float32(1 / 32), np.float32(1 / 128)
+        elif kind == 1:
+            w["a_scale"], w["b_scale"] = np.float32(0.0234375), np.float32(0.01171875)   # 3/128, 3/256
+        else:
+            w["a_scale"] = rng.uniform(0.004, 0.04, M).astype(np.float32)
+            if kind == 3:
+                w["b_scale"] = rng.uniform(0.004, 0.04, N).astype(np.float32)
+        say("fp8_scaled_dot bf16-typed #%d M=%d K=%d N=%d nk=%s %s scales=%d" % (case, M, K, N, nk, w["epilogue"], kind))
+        got, kern = run(w, nk=nk, dequant_type="bf16")
+        kernels.add("rounded" if "rounded" in kern else "bf16_operands" if "bf16_operands" in kern else kern.split("_m")[0])
+        ref = reference(oracle, w, dequant_type="bf16")
+        n_floor = check_dot(got, ref, floor_for(w, exact_kernel=kind != 0), "#%d %s" % (case, kern))
+        assert n_floor <= max(8, got.size // 20)
+    assert {"rounded", "bf16_operands"} <= kernels, kernels
+
+
 def test_rowwise_quantize_random_shapes(oracle):
     rng = np.random.default_rng(5)
     for case in range(12):
