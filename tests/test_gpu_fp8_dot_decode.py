@@ -233,36 +233,41 @@ def test_bf16_typed_multiply(oracle, M, nk):
     them return at once and the bf16-operand kernels launched behind them (or, without their scratch,
     the exact kernel) produce the result."""
     say("fp8 streaming, bf16-typed multiply, M=%d nk=%s" % (M, nk))
-    K, N = 1024, 264
+    K, N = (8192 if M > 64 else 1024), 264   # (100 rows: K long enough for passes to beat the two tiles)
     w = dict(workloads.c3_fp8(M, K, N), a_scale=np.float32(1 / 64), b_scale=np.float32(1 / 32))
     types = dict(dequant_type="bf16")
-    # rhs [K,N]: the streaming kernels' own form that rounds the scaled operands to bf16 stands behind the f8
-    # form ("|rounded"); rhs [N,K]: the bf16-operand pre-passes and tiled kernel do
-    tag = "|bf16_operands" if nk else "|rounded"
+    # the streaming kernels' own form that rounds the scaled operands to bf16 stands behind the f8 form
+    # ("|rounded"); it takes up to 32 rows of an [N,K] rhs per launch, so 48 rows go through in two passes there
+    tag = "|rounded"
     out, kern = run(w, nk=nk, force=0, **types)
     assert kern.startswith("fp8_dot_decode_%s_m" % ("nk" if nk else "kn")) and kern.endswith(tag), kern
     plain, kern_plain = run(w, nk=nk, force=0)
-    assert kern == kern_plain + tag, (kern, kern_plain)
-    assert torch.equal(out, plain)
+    if nk and M > 32:
+        assert kern == "fp8_dot_decode_nk_m32:x32|rounded", kern
+        check_dot(host_bf16(out), reference(oracle, w), floor_for(w), kern)
+    else:
+        assert kern == kern_plain + tag, (kern, kern_plain)
+        assert torch.equal(out, plain)
     w2 = dict(w, a_scale=np.float32(0.3), b_scale=np.float32(0.013))
     ref2 = reference(oracle, w2, **types)
-    for slices in ((0,) if nk else (0, 2)):   # (forced slices size the scratch for the streaming kernels alone)
+    for slices in (0, 2):
         out2, kern2 = run(w2, nk=nk, force=0, slices=slices, **types)
         assert kern2 == kern, kern2
         n_floor = check_dot(host_bf16(out2), ref2, floor_for(w2, exact_kernel=True), "%s, %d slices" % (kern2, slices))
         assert n_floor <= max(8, out2.numel() // 50)
-    out3, kern3 = run(w2, nk=nk, force=0, scratch=None, **types)     # no scratch: one K-slice ([N,K]: then the exact kernel)
-    assert kern3 == kern_plain + ("" if nk else "|rounded"), kern3
+    out3, kern3 = run(w2, nk=nk, force=0, scratch=None, **types)     # no scratch: one K-slice
+    assert kern3 == kern, kern3
     check_dot(host_bf16(out3), ref2, floor_for(w2, exact_kernel=True), kern3)
     out4, _ = run(w, nk=nk, force=0, scratch=None, **types)
     check_dot(host_bf16(out4), reference(oracle, w, **types), floor_for(w), "pow2 scales, no scratch")
 
 
+@pytest.mark.parametrize("nk", [False, True])
 @pytest.mark.parametrize("which", ["a", "b", "ab"])
 @pytest.mark.parametrize("M", [20, 64])
-def test_bf16_typed_multiply_with_vector_scales(oracle, which, M):
+def test_bf16_typed_multiply_with_vector_scales(oracle, which, M, nk):
     """Per-row and per-channel scales under a bf16-typed multiply (no single test tells whether they round
-    anything): the rounding form of the [K,N] kernel runs alone, each operand scaled by its row's or its
+    anything): the rounding form of the streaming kernels runs alone, each operand scaled by its row's or its
     channel's scale."""
     say("fp8 streaming, bf16-typed multiply, vector scales %s, M=%d" % (which, M))
     K, N = 1024, 200
@@ -275,13 +280,14 @@ def test_bf16_typed_multiply_with_vector_scales(oracle, which, M):
     types = dict(dequant_type="bf16")
     ref = reference(oracle, w, **types)
     for slices in (0, 2):
-        out, kern = run(w, force=0, slices=slices, **types)
-        assert kern == tile_name(False, M) + "|rounded", kern
+        out, kern = run(w, nk=nk, force=0, slices=slices, **types)
+        assert kern == ("fp8_dot_decode_nk_m32:x32|rounded" if nk and M > 32 else tile_name(nk, M) + "|rounded"), kern
         n_floor = check_dot(host_bf16(out), ref, floor_for(w, exact_kernel=True), "%s, %d slices" % (kern, slices))
         assert n_floor <= max(8, out.numel() // 50)
 
 
-def test_rounded_operands_read_every_code_back_exactly():
+@pytest.mark.parametrize("nk", [False, True])
+def test_rounded_operands_read_every_code_back_exactly(nk):
     """The form that rounds the scaled operands, on one-hot rows: output [m, n] is
     bf16(bf16(1 * 0.75) * bf16(b[k_m, n] * 0.3125)) for every f8 code at every position of a step -- the
     hardware widening of each code, the rounding of the product and the k order of both operands."""
@@ -297,8 +303,8 @@ def test_rounded_operands_read_every_code_back_exactly():
     bs = dtypes.bf16_to_f32(dtypes.f32_to_bf16(dtypes.f8e4m3fn_to_f32(b8[ks]) * np.float32(0.3125)))
     want = dtypes.f32_to_bf16(np.float32(0.75) * bs)
     for slices in (0, 2):
-        out, kern = run(w, slices=slices, force=0, dequant_type="bf16")
-        assert kern == "fp8_dot_decode_kn_m32|rounded", kern
+        out, kern = run(w, nk=nk, slices=slices, force=0, dequant_type="bf16")
+        assert kern == "fp8_dot_decode_%s_m32|rounded" % ("nk" if nk else "kn"), kern
         assert np.array_equal(dtypes.bf16_to_f32(host_bf16(out)), dtypes.bf16_to_f32(want)), slices
 
 

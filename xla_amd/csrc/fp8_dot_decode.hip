@@ -303,7 +303,9 @@ __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_kn_kernel(Fp8Decod
 // the second 16 bytes k 64..127).  So with block scales lane (., kb) holds pieces kb and kb + 4 of the
 // line instead of 2 kb and 2 kb + 1; a step's four scales of a channel (or row of a) are one dword,
 // of which lane (., kb) hands in byte kb.
-template <int MT, bool MX>
+// ROUNDED (no block scales, up to two token tiles): as in kn_strip, with four v_mfma_f32_16x16x32_bf16 per
+// 32 bytes of either operand (instruction d takes bytes 8 d .. 8 d + 7 of every lane's 32).
+template <int MT, bool MX, bool ROUNDED = false>
 __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, int strip, int slice, int batch) {
   int lane = threadIdx.x & 63;
   asm volatile("" : "+v"(lane), "+s"(batch));  // as in kn_strip
@@ -354,6 +356,22 @@ __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, i
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[g][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // ROUNDED: the lane's operands are token 16 mt + li of a and channel 16 g + li of the rhs
+  float sa_r[MT], sb_r[8];
+  if constexpr (ROUNDED) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) sa_r[mt] = round_bf16(p.a_per_row ? p.a_scale[min(16 * mt + li, p.M - 1)] : *p.a_scale);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) sb_r[g] = round_bf16(p.b_per_channel ? p.b_scale[min(n_li + 16 * g, p.N - 1)] : *p.b_scale);
+  }
+  auto scaled_bf16 = [&](uint32_t lo, uint32_t hi, float s) {
+    const floatx2 f0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false), f1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+    const floatx2 f2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false), f3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+    const uintx4 o = {pack_bf16x2(f0[0] * s, f0[1] * s), pack_bf16x2(f1[0] * s, f1[1] * s),
+                      pack_bf16x2(f2[0] * s, f2[1] * s), pack_bf16x2(f3[0] * s, f3[1] * s)};
+    return __builtin_bit_cast(bf16x8, o);
+  };
+
   const int slice_end = min((slice + 1) * p.rows_per_slice, p.K);
   const int k_begin = slice * p.rows_per_slice + wave * p.rows_per_wave;
   const int k_stop = min(k_begin + p.rows_per_wave, slice_end);
@@ -402,6 +420,14 @@ __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, i
       wv[g][0] = wq[buf][g][0];
       wv[g][1] = wq[buf][g][1];
     }
+    bf16x8 ab[ROUNDED ? MT : 1][4];
+    if constexpr (ROUNDED) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          ab[mt][d] = scaled_bf16(av[mt][d >> 1][2 * (d & 1)], av[mt][d >> 1][2 * (d & 1) + 1], sa_r[mt]);
+    }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       uint32_t tg[8];
@@ -413,6 +439,17 @@ __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, i
           const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + kSrcStep * x, (int)wv[g][1][d]);
           tg[4 * x + d] = upper ? hi : lo;
         }
+      if constexpr (ROUNDED) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const bf16x8 wb = scaled_bf16(tg[2 * d], tg[2 * d + 1], sb_r[4 * half + g]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[4 * half + g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, ab[mt][d], acc[4 * half + g][mt], 0, 0, 0);
+        }
+        if (g & 1) __builtin_amdgcn_sched_barrier(0);
+        continue;
+      }
       // 32 bytes of k per lane and operand: one v_mfma_f32_16x16x128_f8f6f4 (both formats e4m3, no block scales)
       const intx8 wop = {(int)tg[0], (int)tg[1], (int)tg[2], (int)tg[3], (int)tg[4], (int)tg[5], (int)tg[6], (int)tg[7]};
 #pragma unroll
@@ -452,18 +489,22 @@ __device__ __forceinline__ void nk_strip(const Fp8DecodeParams& p, float* lds, i
   reduce_and_store<MT, true>(p, lds, acc, strip, slice, batch);
 }
 
-template <int MT, bool MX, bool WALK>
+template <int MT, bool MX, bool WALK, bool ROUNDED = false>
 __global__ __launch_bounds__(kWaves * 64) void fp8_dot_decode_nk_kernel(Fp8DecodeParams p) {
   __shared__ float lds[kWaves * 32 * 64];
-  if (!MX && p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
+  if constexpr (ROUNDED) {
+    if (p.rounded_operands == 1 && is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale)) return;  // the f8 form has served the call
+  } else {
+    if (!MX && p.require_pow2_scales && !(is_pow2_f32(*p.a_scale) && is_pow2_f32(*p.b_scale))) return;
+  }
   const int slice = blockIdx.x % p.slices;
   if constexpr (!WALK) {
-    nk_strip<MT, MX>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
+    nk_strip<MT, MX, ROUNDED>(p, lds, blockIdx.x / p.slices, slice, blockIdx.y);
   } else {
     const int first = (blockIdx.x / p.slices) * p.cols;
     for (int c = 0; c < p.cols && (first + c) * 128 < p.N; ++c) {
       if (c) __syncthreads();
-      nk_strip<MT, MX>(p, lds, first + c, slice, blockIdx.y);
+      nk_strip<MT, MX, ROUNDED>(p, lds, first + c, slice, blockIdx.y);
     }
   }
 }
@@ -552,7 +593,7 @@ size_t Fp8DotDecodeWorkspaceBytes(int64_t batch, int64_t M, int64_t K, int64_t N
   if (M <= 0 || K <= 0 || N <= 0 || batch <= 0) return 0;
   const bool nk = rhs_contracting_dim == 1;
   size_t bytes = WorkspaceBytesFor(batch, M, K, N, nk, false);
-  if (nk && K % 128 == 0) {  // the call may come with block scales (not known here): passes of 32 rows
+  if (nk) {  // the call may come with block scales or a bf16-typed multiply (not known here): passes of 32 rows
     const size_t mx = WorkspaceBytesFor(batch, M, K, N, true, true);
     bytes = bytes > mx ? bytes : mx;
   }
@@ -568,10 +609,12 @@ int LaunchFp8DotDecode(const XlaAmdFp8ScaledDot& p, hipStream_t stream, bool bf1
   bool dummy = false;
   if (!any_scale) any_scale = &dummy;
   *any_scale = false;
-  if (p.M <= (mx ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream, bf16_multiply, any_scale);
+  // (the rounding form of the [N,K] kernel takes two token tiles, like the block-scaled one)
+  const bool two_tiles = mx || (nk && bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16);
+  if (p.M <= (two_tiles ? 32 : nk ? 48 : 64)) return LaunchFp8DotDecodeRows(p, stream, bf16_multiply, any_scale);
   if (p.batch > 1) return -1;
   int64_t rows = 0;
-  const int passes = Passes(p.M, nk, mx, &rows);
+  const int passes = Passes(p.M, nk, two_tiles, &rows);
   if (GetOption("fp8_dot_kernel") != 3 && !PassesAreCheaper(p.M, p.K, p.N, nk, passes, rows)) return -1;
   const size_t out_bytes = p.out_dtype == XLA_FFI_DataType_F8E4M3FN ? 1 : 2;
   char name[64] = "";
@@ -608,7 +651,7 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
   // rounding form then runs alone
   const bool vector_scales = p.a_scale_per_row || p.b_scale_per_channel;
   if (p.dequant_type != XLA_FFI_DataType_F32 &&
-      !(bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16 && !mx && !(nk && vector_scales)))
+      !(bf16_multiply && p.dequant_type == XLA_FFI_DataType_BF16 && !mx && !(nk && p.M > 32)))
     return -1;
   const bool only_rounded = p.dequant_type == XLA_FFI_DataType_BF16 && vector_scales;
   // block scales: a step's four scales of a row move as one dword
@@ -692,15 +735,17 @@ static int LaunchFp8DotDecodeRows(const XlaAmdFp8ScaledDot& p, hipStream_t strea
     rc = CheckLaunch("fp8_dot_decode_finalize");
     if (rc) return rc;
   }
-  // A bf16-typed multiply on a [K,N] rhs: the same launches again in the form that rounds the scaled
-  // operands to bf16, for scales that are no powers of two (one strip per workgroup).
-  if (dp.require_pow2_scales && !nk) {
+  // A bf16-typed multiply: the same launches again in the form that rounds the scaled operands to bf16,
+  // for scales that are no powers of two (one strip per workgroup).
+  if (dp.require_pow2_scales) {
     Fp8DecodeParams dr = dp;
     dr.require_pow2_scales = 0;
     dr.rounded_operands = only_rounded ? 2 : 1;
     dr.cols = 1;
     const dim3 rgrid((unsigned)(strips * slices), (unsigned)batch);
-    if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<1, false, true>), rgrid, block, 0, stream, dr);
+    if (nk && mt == 1) hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<1, false, false, true>), rgrid, block, 0, stream, dr);
+    else if (nk) hipLaunchKernelGGL((fp8_dot_decode_nk_kernel<2, false, false, true>), rgrid, block, 0, stream, dr);
+    else if (mt == 1) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<1, false, true>), rgrid, block, 0, stream, dr);
     else if (mt == 2) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<2, false, true>), rgrid, block, 0, stream, dr);
     else if (mt == 3) hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<3, false, true>), rgrid, block, 0, stream, dr);
     else hipLaunchKernelGGL((fp8_dot_decode_kn_kernel<4, false, true>), rgrid, block, 0, stream, dr);
