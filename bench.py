@@ -290,6 +290,12 @@ def main():
         entry("fp8 decode", "fp8 [16,8192]x[8192,28672] + bias + GELU (rhs [K,N])",
               ops.fp8_scaled_dot(a8d, b8d, s64, s64, b3d, epilogue="BIAS_GELU", build_only=True),
               f8d_bytes, 2 * 16 * K2 * N2, "hbm")
+        # every op bf16-typed and scales that are no powers of two: each scaled operand is rounded to bf16
+        s03 = torch.full((), 0.30078125, device=dev)
+        entry("fp8 decode bf16-typed", "fp8 [16,8192]x[8192,28672] + bias + GELU, bf16-typed ops, scales 77/256 (operands rounded to bf16)",
+              ops.fp8_scaled_dot(a8d, b8d, s03, s03, b3d, epilogue="BIAS_GELU", dequant_type="bf16", dot_type="bf16",
+                                 epilogue_type="bf16", build_only=True),
+              f8d_bytes, 2 * 16 * K2 * N2, "hbm")
         b8dt = b8d.view(torch.uint8).t().contiguous()
         del b8d
         entry("fp8 decode nk", "fp8 [16,8192]x[28672,8192] + bias + GELU (rhs [N,K])",
@@ -393,7 +399,7 @@ def main():
             for k in c3_keys:
                 by_key[k]["cpu_baseline"] = base(round(2 * 1024 * 8192 * 2048 / t / 1e12, 4), "TFLOP/s",
                                                  "1024 of 8192 rows x 2048 of 8192 channels (full K), f32-typed ops, %.2f s" % t)
-        f8d_keys = [k for k in ("fp8 decode", "fp8 decode nk") if k in by_key]
+        f8d_keys = [k for k in ("fp8 decode", "fp8 decode nk", "fp8 decode bf16-typed") if k in by_key]
         if f8d_keys:
             w = workloads.c3_fp8(16, K2, 4096)
             t = timed(lambda: oracle.fp8_scaled_dot(w["a"], w["b"], w["a_scale"], w["b_scale"], bias=w["bias"],
