@@ -62,7 +62,7 @@ struct DecodeParams {
   const void* group_sizes;
   int group_sizes_64;
   int ragged_groups;  // number of groups (the kernels that do not carry it in grid.y)
-  int ragged_chunks;  // grid.z of a ragged launch: 64-row chunks any one group may need (1 up to 64 rows)
+  int ragged_chunks;  // (kernels that spread a group's rows over grid.z; the decode kernel walks work items in grid.y)
   // Result and activation layouts beyond bf16 [batch,M,N] / [batch,M,K] (the kernels that honour them
   // store through StoreResult; the launcher keeps every other kernel away from such calls):
   int out_f32;         // out holds f32, not bf16

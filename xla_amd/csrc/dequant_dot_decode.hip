@@ -78,19 +78,65 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
   }
   const int slice = bid % p.slices;
   const int strip = bid / p.slices;
-  const int batch = blockIdx.y;
+  int batch = blockIdx.y;
   // rows of lhs / out this workgroup works on: batch b of an ordinary dot owns rows [b*M, (b+1)*M) of
   // the flattened [batch*M] rows; group b of a ragged dot owns the rows its group sizes say
   int m_begin = batch * p.M, m_rows = p.M, tail_begin = -1;
   if (p.group_sizes) {
-    ragged_rows(p, batch, &m_begin, &m_rows);
-    // the last group also fills the rows no group owns (its first chunk does)
-    if (batch == (int)gridDim.y - 1 && blockIdx.z == 0) tail_begin = m_begin + m_rows;
-    // a group of more than 16 * MT rows is spread over grid.z: chunk c takes rows [c * 16 * MT, + 16 * MT)
-    // of the group; chunks past its end have nothing to do
-    const int skip = min((int)blockIdx.z * 16 * MT, m_rows);
-    m_begin += skip;
-    m_rows = min(m_rows - skip, 16 * MT);
+    // grid.y walks work items: the chunks of 16 * MT rows of every group, in group order (a group of r
+    // rows has ceil(r / (16 MT)) of them: fewer than groups + ceil(M / (16 MT)) in all, which is the
+    // grid); an item past the last chunk has nothing to do, and the last item of the grid -- always one
+    // of those -- fills the rows no group owns.  The sizes are only known here, on the device.
+    const int item = blockIdx.y;
+    // Every wave finds its item by itself, 64 groups at a time: lane l reads the size of group g0 + l, two
+    // scans over the lanes give the rows and the chunks before each group (a serial walk over the sizes,
+    // one scalar load per group, took longer than the dot itself once there were 64 groups and more).
+    constexpr int kRows = 16 * MT;
+    int seen = 0, g_sel = -1, begin_sel = 0, rows_sel = 0, last_end = 0;
+    long long raw_base = 0;  // rows before group g0 as the sizes say (clamped per group like ragged_rows does)
+    for (int g0 = 0; g0 < p.ragged_groups; g0 += 64) {
+      const int g = g0 + lane;
+      const bool valid = g < p.ragged_groups;
+      long long n = !valid ? 0 : p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+      long long incl = n;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int lo = __shfl_up((int)(uint32_t)(unsigned long long)incl, off), hi = __shfl_up((int)(uint32_t)((unsigned long long)incl >> 32), off);
+        if (lane >= off) incl += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
+      }
+      const long long raw = raw_base + incl - n;
+      const long long begin = raw < 0 ? 0 : (raw > p.M ? p.M : raw);
+      n = n < 0 ? 0 : (n > p.M - begin ? p.M - begin : n);
+      const int chunks = valid ? ((int)n + kRows - 1) / kRows : 0;
+      int cincl = chunks;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(cincl, off);
+        if (lane >= off) cincl += t;
+      }
+      const int before = seen + cincl - chunks;
+      const bool mine = item >= before && item < before + chunks;
+      const unsigned long long hit = __ballot(mine);
+      if (hit != 0ull && g_sel < 0) {
+        const int src = __builtin_ctzll(hit);
+        g_sel = g0 + src;
+        begin_sel = __shfl((int)begin + (item - before) * kRows, src);
+        rows_sel = __shfl(min((int)n - (item - before) * kRows, kRows), src);
+      }
+      const int last = min(63, p.ragged_groups - 1 - g0);   // the block's last group
+      last_end = __shfl((int)(begin + n), last);
+      seen += __shfl(cincl, 63);
+      const int lo = __shfl((int)(uint32_t)(unsigned long long)incl, 63), hi = __shfl((int)(uint32_t)((unsigned long long)incl >> 32), 63);
+      raw_base += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
+    }
+    g_sel = __builtin_amdgcn_readfirstlane(g_sel);
+    begin_sel = __builtin_amdgcn_readfirstlane(begin_sel);
+    rows_sel = __builtin_amdgcn_readfirstlane(rows_sel);
+    last_end = __builtin_amdgcn_readfirstlane(last_end);
+    if (item == (int)gridDim.y - 1) tail_begin = last_end;
+    batch = g_sel < 0 ? 0 : g_sel;
+    m_begin = begin_sel;
+    m_rows = rows_sel;
     if (m_rows == 0 && (tail_begin < 0 || tail_begin >= p.M)) return;
   }
 
@@ -498,7 +544,9 @@ int launch_decode(const DecodeParams& dp, int batch, hipStream_t stream, const c
   else
     kern = g32 ? dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, true>
                : dequant_dot_decode_kernel<WBITS, VEC, MT, WAVES, MODE, false, false>;
-  dim3 grid((unsigned)(dp.strips * dp.slices), (unsigned)batch, (unsigned)(dp.ragged_chunks > 1 ? dp.ragged_chunks : 1));
+  // (a ragged dot: one grid row per chunk of 16 * MT rows any group can have, and one for the rows nobody owns)
+  const unsigned rows_y = dp.group_sizes ? (unsigned)(batch + (dp.M + 16 * MT - 1) / (16 * MT)) : (unsigned)batch;
+  dim3 grid((unsigned)(dp.strips * dp.slices), rows_y, 1u);
   hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), 0, stream, dp);
   int rc = CheckLaunch(name);
   if (rc) return rc;
@@ -733,11 +781,9 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
   dp.group_sizes = p.group_sizes;
   dp.group_sizes_64 = p.group_sizes_dtype == XLA_FFI_DataType_S64;
   dp.ragged_groups = ragged ? (int)p.batch : 0;
-  // a ragged dot over more than 64 rows: every group in chunks of 64 rows (grid.z), since any group
-  // may own any number of them; a chunk past its group's end returns at once
-  dp.ragged_chunks = ragged && p.M > 64 ? (int)((p.M + 63) / 64) : 1;
-  if (ragged && (p.M + 63) / 64 > 65535)
-    return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes at most 4194240 rows");
+  dp.ragged_chunks = 1;
+  if (ragged && p.batch + (p.M + 15) / 16 > 65535)
+    return Fail(XLA_FFI_Error_Code_UNIMPLEMENTED, "dequant_dot: a ragged dot takes at most 65535 groups plus 16-row chunks");
   if (p.rhs_contracting_dim != 0 && p.rhs_contracting_dim != 1)
     return Fail(XLA_FFI_Error_Code_INVALID_ARGUMENT, "dequant_dot: rhs_contracting_dim must be 0 or 1");
   if (p.rhs_contracting_dim == 1) {  // weights [N,K]
@@ -831,7 +877,16 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
 
   if (force != 1 && force != 3 && aligned && mode_ok && (p.M <= chunk || ragged) && p.K >= 32 && !dp.lhs_k_major) {
     int mt, vec, nv;
-    const bool shape_ok = decode_shape(p.M > 64 ? 64 : p.M, &mt, &vec, &nv);
+    // A ragged dot works in chunks of 16 * mt rows of one group: sized for twice the average group, so
+    // that few groups need a second chunk (every chunk streams its group's weights) and the many small
+    // ones do not pay for empty token tiles (64 experts, 128 rows: 175 us with 64-row chunks, 37-50 with 16).
+    int64_t tile_rows = p.M > 64 ? 64 : p.M;
+    if (ragged && p.batch > 0) {
+      const int64_t twice = 2 * ((p.M + p.batch - 1) / p.batch);
+      tile_rows = twice < tile_rows ? twice : tile_rows;
+      if (tile_rows < 1) tile_rows = 1;
+    }
+    const bool shape_ok = decode_shape(tile_rows, &mt, &vec, &nv);
     const int64_t row_bytes = p.N * (s4 ? 1 : 2) / 2;
     // s4 with bf16 group scales and a bf16-typed multiply: the kernels that dequantise through the
     // 4x4x4 matrix instruction
