@@ -103,6 +103,59 @@ static __device__ __forceinline__ void ragged_rows(const DecodeParams& p, int g,
   *rows = (int)n;
 }
 
+// Work items of a ragged dot on the streaming kernels: the chunks of ROWS rows of every group, in group
+// order (a group of r rows has ceil(r / ROWS) of them: fewer than groups + ceil(M / ROWS) in all).  Every
+// wave finds item `item` by itself, 64 groups at a time: lane l reads the size of group g0 + l, two scans
+// over the lanes give the rows and the chunks before each group (a serial walk over the sizes, one
+// scalar load per group, took longer than the dot itself once there were 64 groups and more).  All 64
+// lanes must be active.  *group < 0: the item lies past the last chunk; *last_end: where the rows that
+// the groups own end.  Sizes are clamped as in ragged_rows.
+template <int ROWS>
+static __device__ __forceinline__ void ragged_item(const DecodeParams& p, int item, int lane, int* group, int* begin,
+                                                   int* rows, int* last_end_out) {
+  int seen = 0, g_sel = -1, begin_sel = 0, rows_sel = 0, last_end = 0;
+  long long raw_base = 0;  // rows before group g0 as the sizes say
+  for (int g0 = 0; g0 < p.ragged_groups; g0 += 64) {
+    const int g = g0 + lane;
+    const bool valid = g < p.ragged_groups;
+    long long n = !valid ? 0 : p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+    long long incl = n;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int lo = __shfl_up((int)(uint32_t)(unsigned long long)incl, off), hi = __shfl_up((int)(uint32_t)((unsigned long long)incl >> 32), off);
+      if (lane >= off) incl += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
+    }
+    const long long raw = raw_base + incl - n;
+    const long long first = raw < 0 ? 0 : (raw > p.M ? p.M : raw);
+    n = n < 0 ? 0 : (n > p.M - first ? p.M - first : n);
+    const int chunks = valid ? ((int)n + ROWS - 1) / ROWS : 0;
+    int cincl = chunks;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int t = __shfl_up(cincl, off);
+      if (lane >= off) cincl += t;
+    }
+    const int before = seen + cincl - chunks;
+    const bool mine = item >= before && item < before + chunks;
+    const unsigned long long hit = __ballot(mine);
+    if (hit != 0ull && g_sel < 0) {
+      const int src = __builtin_ctzll(hit);
+      g_sel = g0 + src;
+      begin_sel = __shfl((int)first + (item - before) * ROWS, src);
+      rows_sel = __shfl(min((int)n - (item - before) * ROWS, ROWS), src);
+    }
+    const int last = min(63, p.ragged_groups - 1 - g0);   // the block's last group
+    last_end = __shfl((int)(first + n), last);
+    seen += __shfl(cincl, 63);
+    const int lo = __shfl((int)(uint32_t)(unsigned long long)incl, 63), hi = __shfl((int)(uint32_t)((unsigned long long)incl >> 32), 63);
+    raw_base += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
+  }
+  *group = __builtin_amdgcn_readfirstlane(g_sel);
+  *begin = __builtin_amdgcn_readfirstlane(begin_sel);
+  *rows = __builtin_amdgcn_readfirstlane(rows_sel);
+  *last_end_out = __builtin_amdgcn_readfirstlane(last_end);
+}
+
 static __device__ __forceinline__ float load_scale(const void* s, size_t idx, int is_bf16) {
   return is_bf16 ? bf16_to_f32(((const uint16_t*)s)[idx]) : ((const float*)s)[idx];
 }

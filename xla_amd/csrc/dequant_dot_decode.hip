@@ -87,52 +87,9 @@ __global__ __launch_bounds__(WAVES * 64) void dequant_dot_decode_kernel(DecodePa
     // rows has ceil(r / (16 MT)) of them: fewer than groups + ceil(M / (16 MT)) in all, which is the
     // grid); an item past the last chunk has nothing to do, and the last item of the grid -- always one
     // of those -- fills the rows no group owns.  The sizes are only known here, on the device.
+    int g_sel, begin_sel, rows_sel, last_end;
+    ragged_item<16 * MT>(p, (int)blockIdx.y, lane, &g_sel, &begin_sel, &rows_sel, &last_end);
     const int item = blockIdx.y;
-    // Every wave finds its item by itself, 64 groups at a time: lane l reads the size of group g0 + l, two
-    // scans over the lanes give the rows and the chunks before each group (a serial walk over the sizes,
-    // one scalar load per group, took longer than the dot itself once there were 64 groups and more).
-    constexpr int kRows = 16 * MT;
-    int seen = 0, g_sel = -1, begin_sel = 0, rows_sel = 0, last_end = 0;
-    long long raw_base = 0;  // rows before group g0 as the sizes say (clamped per group like ragged_rows does)
-    for (int g0 = 0; g0 < p.ragged_groups; g0 += 64) {
-      const int g = g0 + lane;
-      const bool valid = g < p.ragged_groups;
-      long long n = !valid ? 0 : p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
-      long long incl = n;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int lo = __shfl_up((int)(uint32_t)(unsigned long long)incl, off), hi = __shfl_up((int)(uint32_t)((unsigned long long)incl >> 32), off);
-        if (lane >= off) incl += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
-      }
-      const long long raw = raw_base + incl - n;
-      const long long begin = raw < 0 ? 0 : (raw > p.M ? p.M : raw);
-      n = n < 0 ? 0 : (n > p.M - begin ? p.M - begin : n);
-      const int chunks = valid ? ((int)n + kRows - 1) / kRows : 0;
-      int cincl = chunks;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        const int t = __shfl_up(cincl, off);
-        if (lane >= off) cincl += t;
-      }
-      const int before = seen + cincl - chunks;
-      const bool mine = item >= before && item < before + chunks;
-      const unsigned long long hit = __ballot(mine);
-      if (hit != 0ull && g_sel < 0) {
-        const int src = __builtin_ctzll(hit);
-        g_sel = g0 + src;
-        begin_sel = __shfl((int)begin + (item - before) * kRows, src);
-        rows_sel = __shfl(min((int)n - (item - before) * kRows, kRows), src);
-      }
-      const int last = min(63, p.ragged_groups - 1 - g0);   // the block's last group
-      last_end = __shfl((int)(begin + n), last);
-      seen += __shfl(cincl, 63);
-      const int lo = __shfl((int)(uint32_t)(unsigned long long)incl, 63), hi = __shfl((int)(uint32_t)((unsigned long long)incl >> 32), 63);
-      raw_base += (long long)(((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
-    }
-    g_sel = __builtin_amdgcn_readfirstlane(g_sel);
-    begin_sel = __builtin_amdgcn_readfirstlane(begin_sel);
-    rows_sel = __builtin_amdgcn_readfirstlane(rows_sel);
-    last_end = __builtin_amdgcn_readfirstlane(last_end);
     if (item == (int)gridDim.y - 1) tail_begin = last_end;
     batch = g_sel < 0 ? 0 : g_sel;
     m_begin = begin_sel;

@@ -80,11 +80,21 @@ __global__ __launch_bounds__(kNkWaves * 64) void dequant_dot_nk_kernel(NkParams 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 15, kq = lane >> 4;
   const int strip = blockIdx.x, slice = blockIdx.z;
-  const int batch = blockIdx.y / q.m_chunks, chunk = blockIdx.y % q.m_chunks;
-  // ragged dot: `batch` is the group, whose rows [m_first, m_first + m_rows) of the one [M,K] activation
-  // matrix are read on the device; a chunk past the end of its group has nothing to do
+  int batch = blockIdx.y / q.m_chunks, chunk = blockIdx.y % q.m_chunks;
+  // ragged dot: grid.y walks work items, the chunks of 16 * MT rows of every group in group order
+  // (groups + m_chunks of them at most; the sizes are read on the device); `batch` becomes the item's
+  // group, [m_first, m_first + rows) its rows of the one [M,K] activation matrix; an item past the last
+  // chunk has nothing to do
   int m_first = 0, m_rows = p.M;
-  if (p.group_sizes) ragged_rows(p, batch, &m_first, &m_rows);
+  if (p.group_sizes) {
+    int g_sel, begin_sel, rows_sel, last_end;
+    ragged_item<16 * MT>(p, (int)blockIdx.y, lane, &g_sel, &begin_sel, &rows_sel, &last_end);
+    if (g_sel < 0) return;  // (the whole workgroup, before any barrier)
+    batch = g_sel;
+    chunk = 0;
+    m_first = begin_sel;
+    m_rows = rows_sel;
+  }
   const int a_batch = p.group_sizes ? 0 : batch;
   const int m0 = chunk * 16 * MT;
   const int rows_here = min(16 * MT, m_rows - m0);
@@ -450,7 +460,8 @@ int launch_nk(const NkParams& q, int batch, hipStream_t stream, const char* name
       return Fail(XLA_FFI_Error_Code_INTERNAL, "%s: cannot reserve %zu bytes of LDS: %s", name, kLds, hipGetErrorString(e));
     configured.fetch_or(bit, std::memory_order_release);
   }
-  dim3 grid((unsigned)q.d.strips, (unsigned)(batch * q.m_chunks), (unsigned)q.d.slices);
+  // (a ragged dot: one grid row per chunk any group can have)
+  dim3 grid((unsigned)q.d.strips, (unsigned)(q.d.group_sizes ? batch + q.m_chunks : batch * q.m_chunks), (unsigned)q.d.slices);
   hipLaunchKernelGGL((dequant_dot_nk_kernel<WBITS, MT, CT, MODE, ZP>), grid, dim3(kNkWaves * 64), kLds, stream, q);
   int rc = CheckLaunch(name);
   if (rc) return rc;
