@@ -110,8 +110,9 @@ static __device__ __forceinline__ void ragged_rows(const DecodeParams& p, int g,
 // scalar load per group, took longer than the dot itself once there were 64 groups and more).  All 64
 // lanes must be active.  *group < 0: the item lies past the last chunk; *last_end: where the rows that
 // the groups own end.  Sizes are clamped as in ragged_rows.
-template <int ROWS>
-static __device__ __forceinline__ void ragged_item(const DecodeParams& p, int item, int lane, int* group, int* begin,
+// NONNEG: negative sizes count as zero before the rows are summed (the grouped GEMM of the tiled kernel).
+template <int ROWS, bool NONNEG = false, class Params = DecodeParams>
+static __device__ __forceinline__ void ragged_item(const Params& p, int item, int lane, int* group, int* begin,
                                                    int* rows, int* last_end_out) {
   int seen = 0, g_sel = -1, begin_sel = 0, rows_sel = 0, last_end = 0;
   long long raw_base = 0;  // rows before group g0 as the sizes say
@@ -119,6 +120,7 @@ static __device__ __forceinline__ void ragged_item(const DecodeParams& p, int it
     const int g = g0 + lane;
     const bool valid = g < p.ragged_groups;
     long long n = !valid ? 0 : p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
+    if (NONNEG && n < 0) n = 0;
     long long incl = n;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {

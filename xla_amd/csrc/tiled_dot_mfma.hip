@@ -285,24 +285,17 @@ __global__ __launch_bounds__(512) void tiled_dot_kernel(TiledParams p) {
   const bool ragged = WQ && p.group_sizes != nullptr;
   int m0r = 0, m_limit = p.M;  // ragged: first row of the tile and the end of its group's rows
   if (ragged) {
-    // consecutive ids share a row tile (and with it an activation tile in L2)
-    const int slot0 = bid / p.tiles_n;
-    int slot = slot0;
-    long long start = 0;
-    bool found = false;
-    for (int g = 0; g < p.ragged_groups; ++g) {
-      long long n = p.group_sizes_64 ? ((const long long*)p.group_sizes)[g] : (long long)((const int*)p.group_sizes)[g];
-      n = n < 0 ? 0 : (n > p.M - start ? p.M - start : n);   // sizes that do not add up stay inside [0, M]
-      const int tiles_g = (int)((n + kTM - 1) / kTM);
-      if (slot < tiles_g) {
-        batch = g;
-        m0r = (int)start + slot * kTM;
-        m_limit = (int)(start + n);
-        found = true;
-        break;
-      }
-      slot -= tiles_g;
-      start += n;
+    // consecutive ids share a row tile (and with it an activation tile in L2).  Slot s is the s-th
+    // 256-row tile counted over all groups; every wave finds it with a scan over the lanes, 64 groups
+    // at a time (a serial walk, one scalar load per group, cost a workgroup tens of microseconds at 64
+    // groups and more).
+    int g_sel, begin_sel, rows_sel, last_end;
+    ragged_item<kTM, true>(p, bid / p.tiles_n, lane, &g_sel, &begin_sel, &rows_sel, &last_end);
+    const bool found = g_sel >= 0;
+    if (found) {
+      batch = g_sel;
+      m0r = begin_sel;
+      m_limit = begin_sel + rows_sel;
     }
     if (!found) return;
   }
