@@ -855,6 +855,28 @@ def test_ragged_dot_decode(oracle, M, K, N, G, sizes, sizes_dtype):
     check_dot(got, ref, ragged_floor(w), "ragged %s" % kern)
 
 
+@pytest.mark.parametrize("G,M", [(70, 90), (130, 300), (64, 64), (65, 16)])
+@pytest.mark.parametrize("force", [0, 3])
+def test_ragged_dot_over_many_groups(oracle, G, M, force):
+    """More groups than a wave has lanes: the search for a workgroup's item (its group and chunk of rows)
+    scans the sizes 64 at a time and carries the rows and chunks seen so far into the next block.  Random
+    sizes with empty groups, groups of more rows than a chunk, and rows nobody owns; through the decode
+    kernel's work items and (forced) through the grouped GEMM's tile slots."""
+    if force == 3 and M <= 64:
+        pytest.skip("the grouped GEMM takes more than 64 rows")
+    say("dequant_dot ragged over %d groups, %d rows, force=%d" % (G, M, force))
+    rng = np.random.default_rng(G * 1000 + M)
+    sizes = rng.multinomial(int(M * 0.9), np.ones(G) / G)
+    sizes[rng.integers(0, G, 5)] = 0
+    sizes[int(rng.integers(0, G))] += 20          # one group of more than 16 rows
+    K, N = 256, 136
+    w = workloads.ragged_s8_experts(M=M, K=K, N=N, groups=G, sizes=sizes)
+    got, kern = run_ragged(w, torch.int32, force_kernel=force)
+    assert kern == ("dequant_dot_tiled_s8_factored:ragged" if force == 3 else kern) and ("ragged" in kern or "decode" in kern), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged over %d groups, %s" % (G, kern))
+
+
 def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
     """Every row of the ragged result is bit-identical to an ordinary call on its group's rows with
     that group's weights (the same kernel does both); the one-thread-per-output kernel, which finds

@@ -307,6 +307,23 @@ def test_ragged_dot_over_k_minor_experts(oracle, M, K, N, G, sizes, sizes_dtype)
     check_dot(got_g, ref, ragged_floor(w), "ragged [G,N,K] generic")
 
 
+@pytest.mark.parametrize("G,M", [(70, 90), (130, 300)])
+def test_ragged_dot_k_minor_over_many_groups(oracle, G, M):
+    """More groups than a wave has lanes (the item search scans the sizes 64 at a time), experts [G,N,K]."""
+    from tests.test_gpu_dequant_dot import ragged_floor
+    from tests.gpu_util import check_dot
+    say("dequant_dot ragged [G,N,K] over %d groups, %d rows" % (G, M))
+    rng = np.random.default_rng(G * 1000 + M)
+    sizes = rng.multinomial(int(M * 0.9), np.ones(G) / G)
+    sizes[rng.integers(0, G, 5)] = 0
+    sizes[int(rng.integers(0, G))] += 20
+    w = workloads.ragged_s8_experts(M=M, K=256, N=136, groups=G, sizes=sizes)
+    got, kern = run_ragged_nk(w, torch.int32)
+    assert kern.startswith("dequant_dot_nk_s8_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged [G,N,K] over %d groups, %s" % (G, kern))
+
+
 def test_ragged_dot_k_minor_s4_group_scales(oracle):
     from tests.gpu_util import check_dot, dot_floor
     say("dequant_dot ragged [G,N,K] s4 group scales")
