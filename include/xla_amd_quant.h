@@ -311,7 +311,8 @@ XLA_AMD_EXPORT const char* xla_amd_last_kernel(void);
  * (steps per wave of the single-launch s8 kernel: 1, 2, 4), "dequant_dot_strip" (channels per strip of
  * that kernel: 64 or 128), "handover_test" (1: workgroups that hand partial sums over never raise their
  * flags and the waiting side gives up after 16 polls, so that its own fallback computes the result --
- * for tests of that fallback only), "fp8_dot_kernel" (1 exact, 2 tiled, 3 streaming), "fp8_decode_slices" (K-slices of the streaming kernels),
+ * for tests of that fallback only), "dequant_dot_ragged_tile" (rows per chunk of a ragged dot's groups on the
+ * decode kernels: 16, 32, 48 or 64, at most what the launcher would take), "fp8_dot_kernel" (1 exact, 2 tiled, 3 streaming), "fp8_decode_slices" (K-slices of the streaming kernels),
  * "fp8_scales_on_sum" (1: a bf16-typed dequantise multiply of xla_amd.fp8_scaled_dot is computed as the
  * reference's GPU pipeline computes that HLO -- scales on the f32 sum, gemm_rewriter.cc:1235-1591 -- not
  * op by op: no rounding of a * a_scale and b * b_scale to bf16, so scales that are no powers of two keep

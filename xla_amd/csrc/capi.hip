@@ -20,7 +20,7 @@ struct Option {
   int value;
 };
 thread_local Option g_options[] = {{"dequant_dot_kernel", 0}, {"dequant_dot_vec", 0},
-                      {"dequant_dot_slices", 0}, {"dequant_dot_waves", 0}, {"dequant_dot_skew", 0}, {"dequant_dot_x", 0}, {"dequant_dot_nk_ct", 0}, {"dequant_dot_pair", 0}, {"dequant_dot_share", 0}, {"dequant_dot_depth", 0}, {"dequant_dot_steps", 0}, {"dequant_dot_strip", 0}, {"handover_test", 0},
+                      {"dequant_dot_slices", 0}, {"dequant_dot_waves", 0}, {"dequant_dot_skew", 0}, {"dequant_dot_x", 0}, {"dequant_dot_nk_ct", 0}, {"dequant_dot_pair", 0}, {"dequant_dot_share", 0}, {"dequant_dot_depth", 0}, {"dequant_dot_steps", 0}, {"dequant_dot_strip", 0}, {"handover_test", 0}, {"dequant_dot_ragged_tile", 0},
                       {"fp8_dot_kernel", 0}, {"fp8_decode_slices", 0}, {"fp8_decode_cols", 0}, {"fp8_scales_on_sum", 0},
                       {"quantize_variant", 0}, {"fp8_dot_layout", 0}, {"tiled_epilogue", 0}, {"tiled_tail", 0}};
 }  // namespace
