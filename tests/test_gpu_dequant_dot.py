@@ -877,6 +877,24 @@ def test_ragged_dot_over_many_groups(oracle, G, M, force):
     check_dot(got, ref, ragged_floor(w), "ragged over %d groups, %s" % (G, kern))
 
 
+@pytest.mark.parametrize("force", [0, 3])
+@pytest.mark.parametrize("sizes_dtype", [torch.int32, torch.int64])
+def test_ragged_dot_many_groups_sizes_overrun(oracle, force, sizes_dtype):
+    """Sizes that add up to one and a half times the rows, over 130 groups: the rows run out inside the
+    second block of 64 groups that the item search scans, the group they run out in is cut at M and every
+    later group owns nothing."""
+    G, M = 130, 200
+    say("dequant_dot ragged, sizes overrun the rows, %d groups, %d rows, force=%d" % (G, M, force))
+    rng = np.random.default_rng(77)
+    sizes = rng.multinomial(int(M * 1.5), np.ones(G) / G)
+    assert int(sizes[:64].sum()) < M < int(sizes[:128].sum())
+    w = workloads.ragged_s8_experts(M=M, K=256, N=136, groups=G, sizes=sizes)
+    got, kern = run_ragged(w, sizes_dtype, force_kernel=force)
+    assert kern == "dequant_dot_tiled_s8_factored:ragged" if force == 3 else kern.startswith("dequant_dot_decode_s8_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged, sizes overrun, %s" % kern)
+
+
 def test_ragged_dot_equals_per_group_calls_and_generic_kernel(oracle):
     """Every row of the ragged result is bit-identical to an ordinary call on its group's rows with
     that group's weights (the same kernel does both); the one-thread-per-output kernel, which finds

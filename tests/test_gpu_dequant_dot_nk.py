@@ -324,6 +324,22 @@ def test_ragged_dot_k_minor_over_many_groups(oracle, G, M):
     check_dot(got, ref, ragged_floor(w), "ragged [G,N,K] over %d groups, %s" % (G, kern))
 
 
+def test_ragged_dot_k_minor_many_groups_sizes_overrun(oracle):
+    """Sizes that add up to one and a half times the rows over 130 groups, experts [G,N,K]: the rows run
+    out inside the second block of 64 groups of the item search."""
+    from tests.test_gpu_dequant_dot import ragged_floor
+    from tests.gpu_util import check_dot
+    G, M = 130, 200
+    say("dequant_dot ragged [G,N,K], sizes overrun the rows, %d groups, %d rows" % (G, M))
+    sizes = np.random.default_rng(77).multinomial(int(M * 1.5), np.ones(G) / G)
+    assert int(sizes[:64].sum()) < M < int(sizes[:128].sum())
+    w = workloads.ragged_s8_experts(M=M, K=256, N=136, groups=G, sizes=sizes)
+    got, kern = run_ragged_nk(w, torch.int64)
+    assert kern.startswith("dequant_dot_nk_s8_"), kern
+    ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+    check_dot(got, ref, ragged_floor(w), "ragged [G,N,K], sizes overrun, %s" % kern)
+
+
 def test_ragged_dot_k_minor_s4_group_scales(oracle):
     from tests.gpu_util import check_dot, dot_floor
     say("dequant_dot ragged [G,N,K] s4 group scales")
