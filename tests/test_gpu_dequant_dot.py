@@ -981,11 +981,43 @@ def test_ragged_dot_s4_group_scales(oracle, M, K, N, G, group, sizes):
     check_dot(got, ref, dot_floor(a, wd, K), "ragged s4 %s" % kern)
 
 
+@pytest.mark.parametrize("kind,G,K,N,rows,tiled", [
+    ("s8", 8, 4096, 2048, 512, True), ("s8", 2, 14336, 4096, 96, False), ("s8", 32, 2048, 1536, 96, False),
+    ("s8", 128, 2048, 1536, 96, True), ("s4", 4, 4096, 14336, 96, False), ("s4", 4, 4096, 14336, 192, True),
+    ("s8", 4, 1024, 512, 160, False)])
+def test_ragged_dot_choice_of_kernel(oracle, kind, G, K, N, rows, tiled):
+    """Chunks of the decode kernel or tiles of the grouped GEMM, priced on the average group: few experts
+    of large matrices stay with the chunks well past 96 rows each (fewer than 256 tiles leave the chip
+    partly idle for a whole round), many small experts move to tiles at 96.  Either way the oracle's rows."""
+    say("dequant_dot ragged choice %s G=%d K=%d N=%d rows/expert=%d" % (kind, G, K, N, rows))
+    sizes = [rows] * G
+    if kind == "s8":
+        w = workloads.ragged_s8_experts(M=G * rows, K=K, N=N, groups=G, sizes=sizes)
+    else:
+        w = workloads.ragged_s4_group_experts(M=G * rows, K=K, N=N, groups=G, group=128, sizes=sizes)
+    got, kern = run_ragged(w)
+    assert kern.endswith(":ragged") == tiled and (tiled or kern.startswith("dequant_dot_decode_")), kern
+    other, kern2 = run_ragged(w, force_kernel=2 if tiled else 3)
+    assert kern2.endswith(":ragged") != tiled, kern2
+    if kind == "s8":
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights"], 8, w["scales"], "f32", "f32", w["group_sizes"], bias=w["bias"])
+        floor = ragged_floor(w)
+    else:
+        ref = oracle.ragged_dequant_dot(w["lhs"], w["weights_packed"], 4, w["scales"], "bf16", "bf16", w["group_sizes"],
+                                        bias=w["bias"], group=128)
+        wd = np.max(np.abs(w["weights"].astype(np.float64)) *
+                    np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
+        floor = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
+    check_dot(got, ref, floor, "ragged choice %s" % kern)
+    check_dot(other, ref, floor, "ragged choice, the other kernel %s" % kern2)
+
+
 @pytest.mark.parametrize("kind,M,K,N,G,sizes", [
     ("s8", 640, 1024, 512, 4, None), ("s8", 700, 512, 300, 3, [256, 1, 300]), ("s8", 512, 512, 256, 2, [0, 512]),
     ("s8", 400, 512, 256, 4, [500, 3, 3, 3]), ("s4", 600, 1024, 512, 3, None), ("s4", 300, 2048, 256, 2, [10, 200])])
 def test_ragged_dot_grouped_gemm(oracle, kind, M, K, N, G, sizes):
-    """Groups that average 96 rows or more: the tiled kernel as a grouped GEMM -- 256-row tiles per
+    """The tiled kernel as a grouped GEMM (taken by itself where its tiles are priced below the decode
+    kernel's chunks, see test_ragged_dot_choice_of_kernel) -- 256-row tiles per
     group, found on the device from the group sizes (a group of 257 rows is two tiles, the second with
     one live row; empty groups, one group owning everything, sizes that overrun M, rows nobody owns)."""
     say("dequant_dot ragged grouped GEMM %s M=%d K=%d N=%d G=%d sizes=%s" % (kind, M, K, N, G, sizes))
@@ -1002,7 +1034,7 @@ def test_ragged_dot_grouped_gemm(oracle, kind, M, K, N, G, sizes):
                     np.repeat(dtypes.bf16_to_f32(w["scales"]).astype(np.float64), 128, axis=1), axis=0)
         floor = dot_floor(np.abs(dtypes.bf16_to_f32(w["lhs"]).astype(np.float64)), wd, K)
         want = "dequant_dot_tiled_s4_rounded:ragged"
-    got, kern = run_ragged(w)
+    got, kern = run_ragged(w, force_kernel=3)   # matrices this small are cheaper in chunks: the tiles are asked for
     assert kern == want, kern
     check_dot(got, ref, floor, "ragged grouped GEMM %s" % kind)
     # the decode kernel in 64-row chunks computes the same module

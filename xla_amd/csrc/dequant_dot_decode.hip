@@ -37,6 +37,7 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "decode_common.h"
@@ -759,10 +760,22 @@ static int LaunchDequantDotImpl(const XlaAmdDequantDot& p, hipStream_t stream, b
                        ((uintptr_t)p.weights % 16 == 0);
   const bool mode_ok = mode == kRounded || mode == kGroupFactored || per_channel;
 
-  // A ragged dot takes the tiled kernel (a grouped GEMM: 256-row tiles per group) once the groups
-  // average 96 rows; below that most tiles would be nearly empty and the 64-row chunks of the decode
-  // kernel do less work.  The sizes themselves are only known on the device.
-  const bool ragged_tiles = ragged && (force == 3 || (p.batch > 0 && p.M / p.batch >= 96));
+  // A ragged dot takes the tiled kernel (a grouped GEMM: 256-row tiles per group) where its tiles cost
+  // less than the 64-row chunks of the decode kernel.  The sizes themselves are only known on the
+  // device, so both sides are priced on the average group: a group of r rows has r / 64 + 0.5 chunks
+  // and max(1, r / 256 + 0.5) tiles on average.  A chunk streams one expert matrix (2.4e-7 us per s8
+  // weight, 2.0e-7 per 4-bit one, 0.25-0.3 us per work item); 256 tiles run at a time and take
+  // 25 + 0.025 K us.  Measured on MI355X, 96 rows per expert, chunks against tiles: 8 experts of
+  // 14336 x 4096 s8 218 us / 327, s4 160 / 343; 16 of 4096 x 14336 s8 457 / 471, s4 386 / 503; 128 of
+  // 2048 x 1536 s8 269 / 227.  Below 64 rows per expert most of a tile would be empty.
+  bool ragged_tiles = ragged && force == 3;
+  if (ragged && force == 0 && p.batch > 0 && p.M / p.batch >= 64) {
+    const double rows = (double)p.M / (double)p.batch, kn = (double)p.K * (double)p.N;
+    const double chunks_us = (double)p.batch * (rows / 64.0 + 0.5) * (s4 ? 2.0e-7 * kn + 0.3 : 2.4e-7 * kn + 0.25);
+    const double tiles = (double)p.batch * std::max(1.0, rows / 256.0 + 0.5) * (double)((p.N + 255) / 256);
+    const double tiles_us = std::max(1.0, tiles / 256.0) * (25.0 + 0.025 * (double)p.K) * (s4 ? 1.05 : 1.0);
+    ragged_tiles = tiles_us < chunks_us;
+  }
   if (plain && force != 1 && force != 2 && aligned && mode_ok && p.M > 64 && !weights_shared && (!ragged || ragged_tiles)) {
     int rc = LaunchDequantDotPrefill(p, stream);
     if (rc >= 0) return rc;  // -1: shape not covered by the tiled kernel, fall through
